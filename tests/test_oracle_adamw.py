@@ -1,0 +1,135 @@
+"""The AdamW oracle against the reference's ShardedAdamW outputs (tests/golden/adamw.npz),
+against torch.optim.AdamW(foreach=False) (what the reference itself is tested
+against), and against a float64 evaluation of the textbook formulas."""
+
+import numpy as np
+import torch
+
+from oracle.adamw import AdamW, scalars
+
+from helpers import bits, golden_npz, npz_json
+
+
+def torch_sqrt(v):
+    return torch.from_numpy(v).sqrt().numpy()
+
+
+def run(opt, p0, grads, steps, snaps=()):
+    p = p0.copy()
+    out = {}
+    for s in range(steps):
+        opt.update("k", p, np.ascontiguousarray(grads[s]))
+        if s + 1 in snaps:
+            _, m, v = opt.state["k"]
+            out[s + 1] = (p.copy(), m.copy(), v.copy())
+    return p, out
+
+
+def test_bit_exact_with_reference_when_torch_sqrt_is_substituted():
+    d = golden_npz("adamw.npz")
+    h = npz_json(d, "hyper_json")["main"]
+    opt = AdamW(h["lr"], tuple(h["betas"]), h["eps"], h["weight_decay"], sqrt=torch_sqrt)
+    _, snaps = run(opt, d["p0"], d["grads"], h["steps"], snaps=(1, 2, 20))
+    for s, (p, m, v) in snaps.items():
+        assert np.array_equal(bits(m), bits(d[f"m{s}"])), s
+        assert np.array_equal(bits(v), bits(d[f"v{s}"])), s
+        assert np.array_equal(bits(p), bits(d[f"p{s}"])), s
+    h2 = npz_json(d, "hyper_json")["nowd"]
+    opt2 = AdamW(h2["lr"], tuple(h2["betas"]), h2["eps"], h2["weight_decay"], sqrt=torch_sqrt)
+    p, _ = run(opt2, d["p0"], d["grads"], 3)
+    assert np.array_equal(bits(p), bits(d["nowd_p3"]))
+
+
+def test_correctly_rounded_sqrt_moments_exact_params_within_one_ulp_of_the_update():
+    """torch's vectorised CPU sqrt is 1 ulp off on a fraction of a percent of
+    inputs; with the IEEE sqrtf the moments are still bit-identical and each
+    step's parameter differs by at most 1 ulp of that step's update term."""
+    d = golden_npz("adamw.npz")
+    h = npz_json(d, "hyper_json")["main"]
+    opt = AdamW(h["lr"], tuple(h["betas"]), h["eps"], h["weight_decay"])
+    _, snaps = run(opt, d["p0"], d["grads"], h["steps"], snaps=(1, 20))
+    p1, m1, v1 = snaps[1]
+    assert np.array_equal(bits(m1), bits(d["m1"])) and np.array_equal(bits(v1), bits(d["v1"]))
+    p20, m20, v20 = snaps[20]
+    assert np.array_equal(bits(m20), bits(d["m20"])) and np.array_equal(bits(v20), bits(d["v20"]))
+    # one step: |dp| <= ulp(update) + ulp(p) (the sum is rounded once more)
+    upd = np.abs(d["p1"].astype(np.float64) - d["p0"].astype(np.float64) * (1 - h["lr"] * h["weight_decay"]))
+    tol1 = np.spacing(upd.astype(np.float32)).astype(np.float64) + np.spacing(np.abs(d["p1"])).astype(np.float64)
+    assert np.all(np.abs(p1.astype(np.float64) - d["p1"]) <= tol1)
+    assert (bits(p1) != bits(d["p1"])).mean() < 0.02
+    # twenty steps: the update is ~lr per step
+    assert np.abs(p20.astype(np.float64) - d["p20"]).max() <= 20 * 2 * np.spacing(np.float32(h["lr"]))
+    assert (bits(p20) != bits(d["p20"])).mean() < 0.05
+
+
+def test_matches_torch_adamw_single_tensor_path():
+    n = 4099
+    g = torch.Generator().manual_seed(3)
+    p0 = (torch.randn(n, generator=g) * 0.02)
+    grads = [torch.randn(n, generator=g) * 1e-2 for _ in range(5)]
+    for kw in (dict(lr=3e-3, weight_decay=0.1), dict(lr=1e-3, betas=(0.5, 0.999), weight_decay=0.0),
+               dict(lr=1e-2, betas=(0.3, 0.7), eps=1e-6, weight_decay=0.5)):  # beta1 < 0.5: lerp's other branch
+        pt = torch.nn.Parameter(p0.clone())
+        topt = torch.optim.AdamW([pt], foreach=False, **kw)
+        opt = AdamW(sqrt=torch_sqrt, **{"betas": (0.9, 0.999), "eps": 1e-8, **kw})
+        p = p0.numpy().copy()
+        for gr in grads:
+            pt.grad = gr.clone()
+            topt.step()
+            opt.update(0, p, gr.numpy())
+        st = topt.state[pt]
+        assert np.array_equal(bits(opt.state[0][1]), bits(st["exp_avg"].numpy())), kw
+        assert np.array_equal(bits(opt.state[0][2]), bits(st["exp_avg_sq"].numpy())), kw
+        assert np.array_equal(bits(p), bits(pt.detach().numpy())), kw
+
+
+def test_against_float64_textbook_adamw():
+    """Independent of torch: the textbook recurrences in float64 agree to fp32 rounding."""
+    n, steps = 2048, 10
+    rng = np.random.default_rng(0)
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    grads = (rng.standard_normal((steps, n)) * 1e-3).astype(np.float32)
+    lr, b1, b2, eps, wd = 3e-4, 0.9, 0.95, 1e-8, 0.1
+    opt = AdamW(lr, (b1, b2), eps, wd)
+    p, _ = run(opt, p0, grads, steps)
+    P, M, V = p0.astype(np.float64), np.zeros(n), np.zeros(n)
+    for t in range(1, steps + 1):
+        g = grads[t - 1].astype(np.float64)
+        P = P * (1 - lr * wd)
+        M = b1 * M + (1 - b1) * g
+        V = b2 * V + (1 - b2) * g * g
+        P = P - lr / (1 - b1 ** t) * M / (np.sqrt(V) / np.sqrt(1 - b2 ** t) + eps)
+    assert np.abs(p - P).max() < 5e-8
+    assert np.abs(opt.state["k"][1] - M).max() < 1e-9 and np.abs(opt.state["k"][2] - V).max() < 1e-12
+
+
+def test_scalars_and_empty_shard():
+    s = scalars(1.0, 3e-4, (0.9, 0.95), 1e-8, 0.1)
+    assert s["use_decay"] == 1 and s["decay"] == float(np.float32(1 - 3e-4 * 0.1))
+    assert s["neg_step"] == float(np.float32(-(3e-4 / (1 - 0.9 ** 1.0))))
+    opt = AdamW()
+    opt.update("e", np.zeros(0, np.float32), np.zeros(0, np.float32))
+    assert opt.state["e"][0] == 1.0  # the step still counts (tandem/optim.py:24-27)
+
+
+def test_16bit_conversions_match_numpy_and_torch():
+    import ctypes
+
+    from oracle import lib
+
+    allbits = np.arange(65536, dtype=np.uint16)
+    out = np.empty(65536, np.float32)
+    lib().orc_f16_to_f32(ctypes.c_void_p(allbits.ctypes.data), ctypes.c_void_p(out.ctypes.data), ctypes.c_int64(65536))
+    want = allbits.view(np.float16).astype(np.float32)
+    assert np.array_equal(bits(out), bits(want))
+    rng = np.random.default_rng(1)
+    f = np.concatenate([rng.standard_normal(200000).astype(np.float32) * s for s in (1, 1e-5, 1e-7, 7e4)])
+    f = np.concatenate([f, out[np.isfinite(out)], np.float32([65504, 65519.99, 65520, 65536, 1e9, 2.0 ** -25, 2.0 ** -24 * 1.5, 0.0, -0.0, np.inf, -np.inf])])
+    f = np.ascontiguousarray(f)
+    got = np.empty(f.size, np.uint16)
+    lib().orc_f32_to_f16(ctypes.c_void_p(f.ctypes.data), ctypes.c_void_p(got.ctypes.data), ctypes.c_int64(f.size))
+    with np.errstate(over="ignore"):
+        assert np.array_equal(got, f.astype(np.float16).view(np.uint16))
+    lib().orc_f32_to_bf16(ctypes.c_void_p(f.ctypes.data), ctypes.c_void_p(got.ctypes.data), ctypes.c_int64(f.size))
+    want = torch.from_numpy(f).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, want)
