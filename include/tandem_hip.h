@@ -1,0 +1,157 @@
+/* tandem_hip.h -- C ABI of libtandem_hip.so: tandem's data-parallel reduction
+ * path on one AMD MI355X (gfx950).
+ *
+ * Plain pointers and sizes only; no torch, pybind or CUDA types. Device pointers
+ * are raw HIP device addresses (torch: tensor.data_ptr()); a tdm_stream is a
+ * hipStream_t (torch: torch.cuda.current_stream().cuda_stream; NULL is the
+ * default stream). Every function returns 0 on success and a non-zero code on
+ * failure, with the message available from tdm_last_error() on the same thread.
+ * Launchers enqueue work on the given stream and return without waiting.
+ *
+ * The citations name what each entry point replaces in the reference
+ * (Shakhtar-Sankur/tandem): the Python engine's per-piece torch calls and the
+ * C++ engine's pybind surface (tandem/csrc/engine.cpp:53-123).
+ */
+#ifndef TANDEM_HIP_H
+#define TANDEM_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* tdm_stream;
+
+enum tdm_dtype { TDM_F32 = 0, TDM_F64 = 1, TDM_F16 = 2, TDM_BF16 = 3, TDM_I64 = 4, TDM_I32 = 5 };
+
+enum { TDM_MAX_PAIRS = 16, TDM_MAX_WORLD = 8 };
+
+enum tdm_status {
+  TDM_OK = 0,
+  TDM_EINVAL = 1,   /* bad argument: maps to ValueError / std::invalid_argument (engine.cpp:54) */
+  TDM_ERUNTIME = 2, /* HIP or engine failure: RuntimeError */
+  TDM_ETIMEOUT = 3  /* a peer did not answer in time: TimeoutError (engine.cpp:55) */
+};
+
+/* One (destination, source, element count) stream of a launch. */
+typedef struct tdm_pair {
+  void* dst;
+  const void* src;
+  int64_t count;
+} tdm_pair;
+
+/* ---- library ------------------------------------------------------------ */
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* tdm_last_error(void);
+
+/* Bumped when a signature in this header changes. */
+int tdm_abi_version(void);
+
+/* Name, compute-unit count and memory of HIP device `device`. */
+int tdm_device_info(int device, char* name, int name_len, int* compute_units, int64_t* total_bytes);
+
+/* Launch geometry knob for measurements: workgroups per compute unit used by the
+ * streaming kernels (0 restores the built-in default). Not needed for correctness. */
+int tdm_set_blocks_per_cu(int blocks);
+
+/* ---- K1: one ring step -------------------------------------------------- */
+
+/* The reduce half of a ring reduce-scatter step, for up to TDM_MAX_PAIRS
+ * (receiver chunk, sender chunk) pairs in ONE launch:
+ *
+ *     d = scale_dst ? dst[i] / world : dst[i]
+ *     s = scale_src ? src[i] / world : src[i]
+ *     dst[i] = d + s;      if (writeback_src) src[i] = s
+ *
+ * in the tensor's own precision (16-bit floats: widen to fp32, operate, round to
+ * nearest even after each operation), with a true division and no multiply-add
+ * contraction. world <= 1 means no division. Replaces `flat.div_(size)` +
+ * `into.add_(slot)` per 4 MiB piece (tandem/comm.py:269-285,336-343) and the
+ * C++ engine's take()/add_into (tandem/csrc/collectives.cpp:241-260,
+ * tandem/csrc/reduce.cu:47-58,75-102). scale_src is set on the first step only,
+ * when the sender's chunk is still undivided; writeback_src leaves the sender's
+ * chunk holding x / world, as div_ of the whole tensor does. Integer dtypes
+ * reject scaling. Pointers need only element alignment; 16-byte-aligned pairs
+ * take the dwordx4 path. */
+int tdm_k1_reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, int scale_dst, int scale_src,
+                       int writeback_src, tdm_stream stream);
+
+/* The copy half of a ring step (all-gather, broadcast, flatten): dst[i] = src[i],
+ * or dst[i] = src[i] / world when world > 1. Replaces `into.copy_(slot)`
+ * (tandem/comm.py:282-283) and cudaMemcpyAsync in take()
+ * (tandem/csrc/collectives.cpp:247-250). */
+int tdm_k1_copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, tdm_stream stream);
+
+/* ---- K2: bucket flatten + average + unflatten ---------------------------- */
+
+/* One segment of a bucket: `count` elements that lie in ring chunk `chunk` of the
+ * bucket's flat buffer, held by every rank at src[r]; the averaged value is
+ * written to every non-NULL dst[r] (the rank's gradient itself, or its view in
+ * the bucket). */
+typedef struct tdm_fold_seg {
+  const void* src[TDM_MAX_WORLD];
+  void* dst[TDM_MAX_WORLD];
+  int64_t count;
+  int32_t chunk;
+  int32_t reserved;
+} tdm_fold_seg;
+
+/* Bytes of device memory a table of nseg segments needs. */
+int64_t tdm_k2_table_bytes(int nseg);
+
+/* Writes the device image of the table into host memory `image`
+ * (tdm_k2_table_bytes(nseg) bytes); the caller copies it to the device once. */
+int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype, void* image);
+
+/* For every element of every segment, in one launch:
+ *     y_q = average ? src[q][i] / world : src[q][i]
+ *     acc = y[(chunk+1) % world];  acc = y[(chunk+k) % world] + acc,  k = 2..world
+ *     dst[r][i] = acc  for every rank r
+ * which is bit for bit what DDP's per-parameter `view.copy_(p.grad)` followed by
+ * the bucket's ring all_reduce(op="avg") leaves in every rank's gradient views
+ * (tandem/ddp.py:22-33,89-109; ring order tandem/comm.py:301-311). */
+int tdm_k2_bucket_fold(const void* table_dev, int nseg, int dtype, int world, int average, tdm_stream stream);
+
+/* ---- K3: sharded AdamW --------------------------------------------------- */
+
+/* The step's constants, each already rounded to fp32 from the Python-double
+ * expressions of tandem/optim.py:28-37. */
+typedef struct tdm_adamw_scalars {
+  int32_t use_decay; /* weight_decay != 0 */
+  float decay;       /* 1 - lr * weight_decay */
+  float w1;          /* 1 - beta1 */
+  float beta2;
+  float one_m_b2;    /* 1 - beta2 */
+  float bc2_sqrt;    /* (1 - beta2**t) ** 0.5 */
+  float eps;
+  float neg_step;    /* -(lr / (1 - beta1**t)) */
+} tdm_adamw_scalars;
+
+enum tdm_adamw_order {
+  TDM_ADAMW_HOST_ORDER = 0,  /* p + (neg_step*m)/d : torch's CPU addcdiv_, the reference's CPU engine */
+  TDM_ADAMW_DEVICE_ORDER = 1 /* fma(neg_step, m/d, p): torch's GPU addcdiv_ kernel */
+};
+
+/* One fused AdamW step over a flat fp32 shard, in place (p, m, v); replaces the
+ * seven elementwise torch passes of ShardedAdamW.update (tandem/optim.py:28-37):
+ *     p *= decay;  m = fma(w1, g - m, m);  v = fma(one_m_b2 * g, g, v * beta2);
+ *     d = sqrt(v) / bc2_sqrt + eps;  p += (neg_step * m) / d
+ * with IEEE sqrt and division. */
+int tdm_k3_adamw(float* p, const float* g, float* m, float* v, int64_t n, const tdm_adamw_scalars* s, int order,
+                 tdm_stream stream);
+
+/* ---- K4: ZeRO-3 unit gather ---------------------------------------------- */
+
+/* full[lo_q : lo_q + sizes[q]] = shards[q][0 : sizes[q]] for every rank q, in one
+ * launch (lo_q = sizes[0] + ... + sizes[q-1]); a shard that already is its slice
+ * of `full` is skipped. Replaces `full[lo:hi].copy_(shard)` + the ring all_gather
+ * of FSDP._start_gather (tandem/zero.py:238-245, tandem/comm.py:307-311,371-385). */
+int tdm_k4_unit_gather(void* full, const void* const* shards, const int64_t* sizes, int world, int dtype,
+                       tdm_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TANDEM_HIP_H */

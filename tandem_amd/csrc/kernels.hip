@@ -1,0 +1,858 @@
+// Streaming kernels of tandem's data-parallel reduction path for gfx950 (MI355X):
+// K1 ring-step reduce / copy, K2 bucket fold, K3 sharded AdamW, K4 unit gather.
+//
+// All four are HBM-bound element-wise passes, so they share one shape: a launch
+// covers a small table of streams, the work is cut into tiles of 16 KiB per
+// stream, workgroups walk the tiles grid-stride (consecutive workgroups touch
+// consecutive tiles, so a sweep of the grid is one contiguous multi-MiB slot of
+// every stream), and each lane keeps several independent 16-byte loads in flight
+// before its first use. No LDS. Arithmetic is exact IEEE in the tensor's own
+// precision: built with -ffp-contract=off, true division, correctly rounded
+// sqrt; the only fused multiply-adds are the explicit ones in K3.
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../include/tandem_hip.h"
+#include "common.h"
+
+namespace tandem_hip {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;                      // 16-byte vectors per lane per tile and stream
+constexpr int kTileVecs = kThreads * kUnroll;   // 1024 vectors = 16 KiB of every stream
+constexpr int kDefaultBlocksPerCu = 8;
+
+int g_blocks_per_cu = kDefaultBlocksPerCu;
+
+typedef uint32_t vec16 __attribute__((ext_vector_type(4)));  // one dwordx4 access
+
+// ---------------------------------------------------------------- element types
+struct f16_t { uint16_t bits; };
+struct bf16_t { uint16_t bits; };
+
+template <typename T> struct Elem;
+
+template <> struct Elem<float> {
+  using acc = float;
+  static constexpr bool floating = true;
+  static __device__ __forceinline__ acc widen(float x) { return x; }
+  static __device__ __forceinline__ float narrow(acc x) { return x; }
+};
+template <> struct Elem<double> {
+  using acc = double;
+  static constexpr bool floating = true;
+  static __device__ __forceinline__ acc widen(double x) { return x; }
+  static __device__ __forceinline__ double narrow(acc x) { return x; }
+};
+template <> struct Elem<int64_t> {
+  using acc = int64_t;
+  static constexpr bool floating = false;
+  static __device__ __forceinline__ acc widen(int64_t x) { return x; }
+  static __device__ __forceinline__ int64_t narrow(acc x) { return x; }
+};
+template <> struct Elem<int32_t> {
+  using acc = int32_t;
+  static constexpr bool floating = false;
+  static __device__ __forceinline__ acc widen(int32_t x) { return x; }
+  static __device__ __forceinline__ int32_t narrow(acc x) { return x; }
+};
+template <> struct Elem<f16_t> {
+  using acc = float;
+  static constexpr bool floating = true;
+  static __device__ __forceinline__ acc widen(f16_t x) {
+    _Float16 h;
+    __builtin_memcpy(&h, &x.bits, 2);
+    return static_cast<float>(h);
+  }
+  static __device__ __forceinline__ f16_t narrow(acc x) {
+    _Float16 h = static_cast<_Float16>(x);  // round to nearest even, once
+    f16_t out;
+    __builtin_memcpy(&out.bits, &h, 2);
+    return out;
+  }
+};
+template <> struct Elem<bf16_t> {
+  using acc = float;
+  static constexpr bool floating = true;
+  static __device__ __forceinline__ acc widen(bf16_t x) { return __uint_as_float(static_cast<uint32_t>(x.bits) << 16); }
+  static __device__ __forceinline__ bf16_t narrow(acc x) {
+    uint32_t u = __float_as_uint(x);
+    bf16_t out;
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+      out.bits = 0x7fc0u;  // NaN
+    } else {
+      u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
+      out.bits = static_cast<uint16_t>(u >> 16);
+    }
+    return out;
+  }
+};
+
+// x / world as the element type would store it. kDiv: 0 none, 1 world is a power
+// of two (multiplying by the exact reciprocal gives the same bits as dividing,
+// denormal results included), 2 true division.
+template <typename T, int kDiv>
+__device__ __forceinline__ typename Elem<T>::acc scaled(typename Elem<T>::acc x, typename Elem<T>::acc divisor,
+                                                        typename Elem<T>::acc reciprocal) {
+  using A = typename Elem<T>::acc;
+  if constexpr (kDiv == 0 || !Elem<T>::floating) {
+    return x;
+  } else if constexpr (kDiv == 1) {
+    return Elem<T>::widen(Elem<T>::narrow(static_cast<A>(x * reciprocal)));
+  } else {
+    return Elem<T>::widen(Elem<T>::narrow(static_cast<A>(x / divisor)));
+  }
+}
+
+template <typename T>
+constexpr int lanes() { return 16 / static_cast<int>(sizeof(T)); }
+
+template <typename T>
+struct Lanes {
+  T v[lanes<T>()];
+};
+
+template <typename T>
+__device__ __forceinline__ Lanes<T> unpack(const vec16& raw) {
+  Lanes<T> out;
+  __builtin_memcpy(&out, &raw, 16);
+  return out;
+}
+template <typename T>
+__device__ __forceinline__ vec16 pack(const Lanes<T>& in) {
+  vec16 out;
+  __builtin_memcpy(&out, &in, 16);
+  return out;
+}
+
+// Every byte is touched once per launch: non-temporal accesses keep the streams
+// from evicting each other in L2 / Infinity Cache. -DTDM_TEMPORAL=1 builds the
+// plain variant for comparison.
+#ifndef TDM_TEMPORAL
+#define TDM_TEMPORAL 0
+#endif
+__device__ __forceinline__ vec16 load16(const void* p) {
+#if TDM_TEMPORAL
+  return *static_cast<const vec16*>(p);
+#else
+  return __builtin_nontemporal_load(static_cast<const vec16*>(p));
+#endif
+}
+__device__ __forceinline__ void store16(void* p, const vec16& v) {
+#if TDM_TEMPORAL
+  *static_cast<vec16*>(p) = v;
+#else
+  __builtin_nontemporal_store(v, static_cast<vec16*>(p));
+#endif
+}
+
+// ---------------------------------------------------------------- pair tables
+// Passed by value in the kernel arguments (scalar loads; no device table).
+struct PairTable {
+  int npairs;
+  int flags;  // per launch: bit0 scale_dst, bit1 scale_src, bit2 writeback_src
+  int64_t tile_end[TDM_MAX_PAIRS];  // running tile count
+  char* dst[TDM_MAX_PAIRS];
+  char* src[TDM_MAX_PAIRS];
+  int64_t count[TDM_MAX_PAIRS];
+  int32_t head[TDM_MAX_PAIRS];    // elements before dst reaches a 16-byte boundary
+  int32_t vec_ok[TDM_MAX_PAIRS];  // dst and src share the same phase within 16 bytes
+};
+
+template <typename T>
+struct Divisor {
+  typename Elem<T>::acc divisor, reciprocal;
+};
+
+// dst = (dst[/w]) + (src[/w]) on one element
+template <typename T, int kDiv>
+__device__ __forceinline__ void reduce_elem(T& d, T& s, bool scale_dst, bool scale_src, const Divisor<T>& dv) {
+  using A = typename Elem<T>::acc;
+  A x = Elem<T>::widen(d), y = Elem<T>::widen(s);
+  if (scale_dst) x = scaled<T, kDiv>(x, dv.divisor, dv.reciprocal);
+  if (scale_src) y = scaled<T, kDiv>(y, dv.divisor, dv.reciprocal);
+  s = Elem<T>::narrow(y);
+  d = Elem<T>::narrow(static_cast<A>(x + y));
+}
+
+template <typename T, int kDiv>
+__global__ __launch_bounds__(kThreads) void k1_reduce_kernel(PairTable tab, Divisor<T> dv) {
+  constexpr int L = lanes<T>();
+  constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
+  const bool scale_dst = tab.flags & 1, scale_src = tab.flags & 2, writeback = tab.flags & 4;
+  const int64_t total = tab.tile_end[tab.npairs - 1];
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    int p = 0;
+    while (tile >= tab.tile_end[p]) ++p;
+    const int64_t t = tile - (p ? tab.tile_end[p - 1] : 0);
+    T* __restrict__ dst = reinterpret_cast<T*>(tab.dst[p]);
+    T* __restrict__ src = reinterpret_cast<T*>(tab.src[p]);
+    const int64_t n = tab.count[p];
+    if (tab.vec_ok[p]) {
+      const int64_t head = tab.head[p];
+      const int64_t nv = (n - head) / L;
+      char* dvp = reinterpret_cast<char*>(dst + head);
+      char* svp = reinterpret_cast<char*>(src + head);
+      const int64_t v0 = t * kTileVecs + threadIdx.x;
+      if ((t + 1) * kTileVecs <= nv) {  // a full tile: all loads first, then the arithmetic, then the stores
+        vec16 a[kUnroll], b[kUnroll];
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) a[k] = load16(dvp + (v0 + k * kThreads) * 16);
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) b[k] = load16(svp + (v0 + k * kThreads) * 16);
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+          Lanes<T> x = unpack<T>(a[k]), y = unpack<T>(b[k]);
+#pragma unroll
+          for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
+          store16(dvp + (v0 + k * kThreads) * 16, pack<T>(x));
+          if (writeback) store16(svp + (v0 + k * kThreads) * 16, pack<T>(y));
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+          const int64_t v = v0 + k * kThreads;
+          if (v < nv) {
+            Lanes<T> x = unpack<T>(load16(dvp + v * 16)), y = unpack<T>(load16(svp + v * 16));
+#pragma unroll
+            for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
+            store16(dvp + v * 16, pack<T>(x));
+            if (writeback) store16(svp + v * 16, pack<T>(y));
+          }
+        }
+      }
+      if (t == 0) {  // the few elements before and after the 16-byte body
+        const int64_t tail0 = head + nv * L;
+        int64_t i = -1;
+        if (static_cast<int64_t>(threadIdx.x) < head) i = threadIdx.x;
+        else if (threadIdx.x >= 32 && tail0 + (threadIdx.x - 32) < n && threadIdx.x - 32 < L) i = tail0 + (threadIdx.x - 32);
+        if (i >= 0) {
+          T x = dst[i], y = src[i];
+          reduce_elem<T, kDiv>(x, y, scale_dst, scale_src, dv);
+          dst[i] = x;
+          if (writeback) src[i] = y;
+        }
+      }
+    } else {  // the two pointers disagree within 16 bytes: element-wise, still coalesced
+      const int64_t e0 = t * kTileElems + threadIdx.x;
+#pragma unroll 4
+      for (int k = 0; k < kUnroll * L; ++k) {
+        const int64_t i = e0 + static_cast<int64_t>(k) * kThreads;
+        if (i < n) {
+          T x = dst[i], y = src[i];
+          reduce_elem<T, kDiv>(x, y, scale_dst, scale_src, dv);
+          dst[i] = x;
+          if (writeback) src[i] = y;
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int kDiv>
+__device__ __forceinline__ T copy_elem(T s, const Divisor<T>& dv) {
+  if constexpr (kDiv == 0) {
+    return s;
+  } else {
+    return Elem<T>::narrow(scaled<T, kDiv>(Elem<T>::widen(s), dv.divisor, dv.reciprocal));
+  }
+}
+
+template <typename T, int kDiv>
+__global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Divisor<T> dv) {
+  constexpr int L = lanes<T>();
+  constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
+  const int64_t total = tab.tile_end[tab.npairs - 1];
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    int p = 0;
+    while (tile >= tab.tile_end[p]) ++p;
+    const int64_t t = tile - (p ? tab.tile_end[p - 1] : 0);
+    T* __restrict__ dst = reinterpret_cast<T*>(tab.dst[p]);
+    const T* __restrict__ src = reinterpret_cast<const T*>(tab.src[p]);
+    const int64_t n = tab.count[p];
+    if (tab.vec_ok[p]) {
+      const int64_t head = tab.head[p];
+      const int64_t nv = (n - head) / L;
+      char* dvp = reinterpret_cast<char*>(dst + head);
+      const char* svp = reinterpret_cast<const char*>(src + head);
+      const int64_t v0 = t * kTileVecs + threadIdx.x;
+      if ((t + 1) * kTileVecs <= nv) {
+        vec16 b[kUnroll];
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) b[k] = load16(svp + (v0 + k * kThreads) * 16);
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+          if constexpr (kDiv != 0) {
+            Lanes<T> y = unpack<T>(b[k]);
+#pragma unroll
+            for (int l = 0; l < L; ++l) y.v[l] = copy_elem<T, kDiv>(y.v[l], dv);
+            b[k] = pack<T>(y);
+          }
+          store16(dvp + (v0 + k * kThreads) * 16, b[k]);
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < kUnroll; ++k) {
+          const int64_t v = v0 + k * kThreads;
+          if (v < nv) {
+            Lanes<T> y = unpack<T>(load16(svp + v * 16));
+#pragma unroll
+            for (int l = 0; l < L; ++l) y.v[l] = copy_elem<T, kDiv>(y.v[l], dv);
+            store16(dvp + v * 16, pack<T>(y));
+          }
+        }
+      }
+      if (t == 0) {
+        const int64_t tail0 = head + nv * L;
+        int64_t i = -1;
+        if (static_cast<int64_t>(threadIdx.x) < head) i = threadIdx.x;
+        else if (threadIdx.x >= 32 && tail0 + (threadIdx.x - 32) < n && threadIdx.x - 32 < L) i = tail0 + (threadIdx.x - 32);
+        if (i >= 0) dst[i] = copy_elem<T, kDiv>(src[i], dv);
+      }
+    } else {
+      const int64_t e0 = t * kTileElems + threadIdx.x;
+#pragma unroll 4
+      for (int k = 0; k < kUnroll * L; ++k) {
+        const int64_t i = e0 + static_cast<int64_t>(k) * kThreads;
+        if (i < n) dst[i] = copy_elem<T, kDiv>(src[i], dv);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- K2: bucket fold
+// Device image of a table: a header, the running tile counts, then the segments.
+struct FoldHeader {
+  uint64_t magic;
+  int32_t nseg, world, dtype, reserved;
+  int64_t total_tiles;
+};
+constexpr uint64_t kFoldMagic = 0x74646d4b32746162ull;  // "tdmK2tab"
+
+struct FoldSegDev {
+  const char* src[TDM_MAX_WORLD];
+  char* dst[TDM_MAX_WORLD];
+  int64_t count;
+  int32_t chunk;
+  int32_t vec_ok;  // every pointer of the segment is 16-byte aligned
+};
+
+__host__ __device__ inline int64_t fold_tile_end_offset() { return sizeof(FoldHeader); }
+__host__ __device__ inline int64_t fold_segs_offset(int nseg) {
+  return (sizeof(FoldHeader) + static_cast<int64_t>(nseg) * 8 + 15) / 16 * 16;
+}
+
+template <typename T, int kWorld, int kDiv>
+__global__ __launch_bounds__(kThreads) void k2_fold_kernel(const char* __restrict__ image, Divisor<T> dv) {
+  using A = typename Elem<T>::acc;
+  constexpr int L = lanes<T>();
+  constexpr int kU = kWorld <= 2 ? 4 : 2;  // vectors per lane per tile step, per rank
+  constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
+  const FoldHeader* hd = reinterpret_cast<const FoldHeader*>(image);
+  const int nseg = hd->nseg;
+  const int64_t* tile_end = reinterpret_cast<const int64_t*>(image + fold_tile_end_offset());
+  const FoldSegDev* segs = reinterpret_cast<const FoldSegDev*>(image + fold_segs_offset(nseg));
+  const int64_t total = hd->total_tiles;
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    int lo = 0, hi = nseg - 1;  // first segment whose running tile count exceeds `tile`
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (tile >= tile_end[mid]) lo = mid + 1; else hi = mid;
+    }
+    const FoldSegDev& sg = segs[lo];
+    const int64_t t = tile - (lo ? tile_end[lo - 1] : 0);
+    const int64_t n = sg.count;
+    const int c = sg.chunk;
+    // ring order: the fold starts at rank chunk+1 and ends with the chunk's owner
+    const char* sp[kWorld];
+    char* dp[kWorld];
+#pragma unroll
+    for (int k = 0; k < kWorld; ++k) {
+      sp[k] = sg.src[(c + 1 + k) % kWorld];
+      dp[k] = sg.dst[k];
+    }
+    if (sg.vec_ok) {
+      const int64_t nv = n / L;
+#pragma unroll
+      for (int u0 = 0; u0 < kUnroll; u0 += kU) {
+        const int64_t vbase = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u0) * kThreads;
+        vec16 in[kWorld][kU];
+#pragma unroll
+        for (int k = 0; k < kWorld; ++k)
+#pragma unroll
+          for (int u = 0; u < kU; ++u) {
+            const int64_t v = vbase + u * kThreads;
+            if (v < nv) in[k][u] = load16(sp[k] + v * 16);
+          }
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          const int64_t v = vbase + u * kThreads;
+          if (v < nv) {
+            Lanes<T> out;
+#pragma unroll
+            for (int l = 0; l < L; ++l) {
+              A acc = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[0][u]).v[l]), dv.divisor, dv.reciprocal);
+#pragma unroll
+              for (int k = 1; k < kWorld; ++k) {
+                const A y = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[k][u]).v[l]), dv.divisor, dv.reciprocal);
+                acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+              }
+              out.v[l] = Elem<T>::narrow(acc);
+            }
+            const vec16 packed = pack<T>(out);
+#pragma unroll
+            for (int k = 0; k < kWorld; ++k)
+              if (dp[k]) store16(dp[k] + v * 16, packed);
+          }
+        }
+      }
+      if (t == 0 && threadIdx.x < n - nv * L) {  // tail elements
+        const int64_t i = nv * L + threadIdx.x;
+        A acc = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[0])[i]), dv.divisor, dv.reciprocal);
+#pragma unroll
+        for (int k = 1; k < kWorld; ++k) {
+          const A y = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[k])[i]), dv.divisor, dv.reciprocal);
+          acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+        }
+#pragma unroll
+        for (int k = 0; k < kWorld; ++k)
+          if (dp[k]) reinterpret_cast<T*>(dp[k])[i] = Elem<T>::narrow(acc);
+      }
+    } else {
+      const int64_t e0 = t * kTileElems + threadIdx.x;
+      for (int k2 = 0; k2 < kUnroll * L; ++k2) {
+        const int64_t i = e0 + static_cast<int64_t>(k2) * kThreads;
+        if (i < n) {
+          A acc = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[0])[i]), dv.divisor, dv.reciprocal);
+#pragma unroll
+          for (int k = 1; k < kWorld; ++k) {
+            const A y = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[k])[i]), dv.divisor, dv.reciprocal);
+            acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+          }
+#pragma unroll
+          for (int k = 0; k < kWorld; ++k)
+            if (dp[k]) reinterpret_cast<T*>(dp[k])[i] = Elem<T>::narrow(acc);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- K3: AdamW
+struct AdamwArgs {
+  float* p;
+  const float* g;
+  float* m;
+  float* v;
+  int64_t n;
+  tdm_adamw_scalars s;
+};
+
+template <int kOrder>
+__device__ __forceinline__ void adamw_elem(float& p, float g, float& m, float& v, const tdm_adamw_scalars& s,
+                                           bool small_w) {
+  if (s.use_decay) p = p * s.decay;
+  const float diff = g - m;
+  // lerp_: weight < 0.5 ? fma(w, end-start, start) : fma(w-1, end-start, end)
+  m = small_w ? __builtin_fmaf(s.w1, diff, m) : __builtin_fmaf(s.w1 - 1.0f, diff, g);
+  const float vs = v * s.beta2;
+  v = __builtin_fmaf(s.one_m_b2 * g, g, vs);  // addcmul_: (value*g) rounded, then fused
+  const float d = __builtin_sqrtf(v) / s.bc2_sqrt + s.eps;
+  if constexpr (kOrder == TDM_ADAMW_HOST_ORDER) {
+    p = p + (s.neg_step * m) / d;
+  } else {
+    p = __builtin_fmaf(s.neg_step, m / d, p);
+  }
+}
+
+template <int kOrder, bool kVec>
+__global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
+  const bool small_w = __builtin_fabsf(a.s.w1) < 0.5f;
+  if constexpr (kVec) {
+    constexpr int kU = 2;
+    const int64_t nv = a.n / 4;
+    const int64_t tiles = (nv + kThreads * kU - 1) / (kThreads * kU);
+    for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+      const int64_t v0 = tile * (kThreads * kU) + threadIdx.x;
+      vec16 rp[kU], rg[kU], rm[kU], rv[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int64_t i = v0 + u * kThreads;
+        if (i < nv) {
+          rp[u] = load16(reinterpret_cast<const char*>(a.p) + i * 16);
+          rg[u] = load16(reinterpret_cast<const char*>(a.g) + i * 16);
+          rm[u] = load16(reinterpret_cast<const char*>(a.m) + i * 16);
+          rv[u] = load16(reinterpret_cast<const char*>(a.v) + i * 16);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int64_t i = v0 + u * kThreads;
+        if (i < nv) {
+          Lanes<float> P = unpack<float>(rp[u]), G = unpack<float>(rg[u]), M = unpack<float>(rm[u]),
+                       V = unpack<float>(rv[u]);
+#pragma unroll
+          for (int l = 0; l < 4; ++l) adamw_elem<kOrder>(P.v[l], G.v[l], M.v[l], V.v[l], a.s, small_w);
+          store16(reinterpret_cast<char*>(a.p) + i * 16, pack<float>(P));
+          store16(reinterpret_cast<char*>(a.m) + i * 16, pack<float>(M));
+          store16(reinterpret_cast<char*>(a.v) + i * 16, pack<float>(V));
+        }
+      }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < a.n - nv * 4) {
+      const int64_t i = nv * 4 + threadIdx.x;
+      adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
+    }
+  } else {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < a.n; i += stride) {
+      adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
+    }
+  }
+}
+
+// ---------------------------------------------------------------- host side
+int elem_size(int dtype) {
+  switch (dtype) {
+    case TDM_F32: case TDM_I32: return 4;
+    case TDM_F64: case TDM_I64: return 8;
+    case TDM_F16: case TDM_BF16: return 2;
+    default: return 0;
+  }
+}
+
+bool is_floating(int dtype) { return dtype == TDM_F32 || dtype == TDM_F64 || dtype == TDM_F16 || dtype == TDM_BF16; }
+
+int compute_units() {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
+  }
+  return cus[dev];
+}
+
+int grid_for(int64_t tiles) {
+  const int64_t cap = static_cast<int64_t>(compute_units()) * g_blocks_per_cu;
+  return static_cast<int>(std::max<int64_t>(1, std::min(tiles, cap)));
+}
+
+// Validates the pairs and lays out the by-value table. Returns the tile count (0: nothing to do).
+int64_t build_pairs(const tdm_pair* pairs, int npairs, int esize, bool ranges_must_not_overlap, PairTable* tab) {
+  if (npairs < 0 || npairs > TDM_MAX_PAIRS) throw Invalid("npairs must be in [0, " + std::to_string(TDM_MAX_PAIRS) + "]");
+  if (npairs > 0 && pairs == nullptr) throw Invalid("pairs is NULL");
+  std::memset(tab, 0, sizeof *tab);
+  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / esize);
+  int64_t tiles = 0;
+  int k = 0;
+  for (int i = 0; i < npairs; ++i) {
+    const tdm_pair& p = pairs[i];
+    if (p.count < 0) throw Invalid("pair " + std::to_string(i) + ": negative count");
+    if (p.count == 0) continue;  // an empty chunk exchanges nothing (tandem/comm.py:292-294)
+    if (p.dst == nullptr || p.src == nullptr) throw Invalid("pair " + std::to_string(i) + ": NULL pointer");
+    const uintptr_t d = reinterpret_cast<uintptr_t>(p.dst), s = reinterpret_cast<uintptr_t>(p.src);
+    if (d % esize || s % esize) throw Invalid("pair " + std::to_string(i) + ": pointer not aligned to the element size");
+    const uintptr_t bytes = static_cast<uintptr_t>(p.count) * esize;
+    if (ranges_must_not_overlap && d < s + bytes && s < d + bytes) {
+      throw Invalid("pair " + std::to_string(i) + ": destination and source overlap");
+    }
+    tab->dst[k] = static_cast<char*>(p.dst);
+    tab->src[k] = static_cast<char*>(const_cast<void*>(p.src));
+    tab->count[k] = p.count;
+    tab->vec_ok[k] = (d % 16) == (s % 16);
+    int64_t head = ((16 - d % 16) % 16) / esize;
+    tab->head[k] = static_cast<int32_t>(std::min<int64_t>(head, p.count));
+    tiles += (p.count + tile_elems - 1) / tile_elems;
+    tab->tile_end[k] = tiles;
+    ++k;
+  }
+  tab->npairs = k;
+  return tiles;
+}
+
+template <typename T>
+Divisor<T> make_divisor(int world) {
+  using A = typename Elem<T>::acc;
+  Divisor<T> d;
+  d.divisor = static_cast<A>(world > 0 ? world : 1);
+  if constexpr (Elem<T>::floating) d.reciprocal = static_cast<A>(1) / d.divisor; else d.reciprocal = 1;
+  return d;
+}
+
+// 0: no division, 1: power of two (exact reciprocal), 2: true division
+int div_kind(int world, bool any_scale) {
+  if (world <= 1 || !any_scale) return 0;
+  return (world & (world - 1)) == 0 ? 1 : 2;
+}
+
+template <typename T>
+void launch_reduce(const PairTable& tab, int64_t tiles, int world, bool any_scale, hipStream_t stream) {
+  const Divisor<T> dv = make_divisor<T>(world);
+  const dim3 grid(grid_for(tiles)), block(kThreads);
+  switch (div_kind(world, any_scale)) {
+    case 0: hipLaunchKernelGGL((k1_reduce_kernel<T, 0>), grid, block, 0, stream, tab, dv); break;
+    case 1: hipLaunchKernelGGL((k1_reduce_kernel<T, 1>), grid, block, 0, stream, tab, dv); break;
+    default: hipLaunchKernelGGL((k1_reduce_kernel<T, 2>), grid, block, 0, stream, tab, dv); break;
+  }
+}
+
+template <typename T>
+void launch_copy(const PairTable& tab, int64_t tiles, int world, hipStream_t stream) {
+  const Divisor<T> dv = make_divisor<T>(world);
+  const dim3 grid(grid_for(tiles)), block(kThreads);
+  switch (div_kind(world, true)) {
+    case 0: hipLaunchKernelGGL((k1_copy_kernel<T, 0>), grid, block, 0, stream, tab, dv); break;
+    case 1: hipLaunchKernelGGL((k1_copy_kernel<T, 1>), grid, block, 0, stream, tab, dv); break;
+    default: hipLaunchKernelGGL((k1_copy_kernel<T, 2>), grid, block, 0, stream, tab, dv); break;
+  }
+}
+
+template <typename T, int kWorld>
+void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t stream) {
+  const Divisor<T> dv = make_divisor<T>(kWorld);
+  const dim3 grid(grid_for(tiles)), block(kThreads);
+  const char* img = static_cast<const char*>(image);
+  switch (div_kind(kWorld, average != 0)) {
+    case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0>), grid, block, 0, stream, img, dv); break;
+    case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1>), grid, block, 0, stream, img, dv); break;
+    default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2>), grid, block, 0, stream, img, dv); break;
+  }
+}
+
+template <typename T>
+void launch_fold(const void* image, int64_t tiles, int world, int average, hipStream_t stream) {
+  switch (world) {
+    case 1: launch_fold_w<T, 1>(image, tiles, average, stream); break;
+    case 2: launch_fold_w<T, 2>(image, tiles, average, stream); break;
+    case 3: launch_fold_w<T, 3>(image, tiles, average, stream); break;
+    case 4: launch_fold_w<T, 4>(image, tiles, average, stream); break;
+    case 5: launch_fold_w<T, 5>(image, tiles, average, stream); break;
+    case 6: launch_fold_w<T, 6>(image, tiles, average, stream); break;
+    case 7: launch_fold_w<T, 7>(image, tiles, average, stream); break;
+    case 8: launch_fold_w<T, 8>(image, tiles, average, stream); break;
+    default: throw Invalid("world must be in [1, 8]");
+  }
+}
+
+}  // namespace
+
+// Used by the engine too.
+void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool scale_dst, bool scale_src,
+                 bool writeback_src, hipStream_t stream) {
+  const int es = elem_size(dtype);
+  if (es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
+  const bool any_scale = (scale_dst || scale_src) && world > 1;
+  if (any_scale && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
+  PairTable tab;
+  const int64_t tiles = build_pairs(pairs, npairs, es, true, &tab);
+  if (tiles == 0) return;
+  tab.flags = (any_scale && scale_dst ? 1 : 0) | (any_scale && scale_src ? 2 : 0) | (any_scale && scale_src && writeback_src ? 4 : 0);
+  switch (dtype) {
+    case TDM_F32: launch_reduce<float>(tab, tiles, world, any_scale, stream); break;
+    case TDM_F64: launch_reduce<double>(tab, tiles, world, any_scale, stream); break;
+    case TDM_F16: launch_reduce<f16_t>(tab, tiles, world, any_scale, stream); break;
+    case TDM_BF16: launch_reduce<bf16_t>(tab, tiles, world, any_scale, stream); break;
+    case TDM_I64: launch_reduce<int64_t>(tab, tiles, 1, false, stream); break;
+    default: launch_reduce<int32_t>(tab, tiles, 1, false, stream); break;
+  }
+  check_hip(hipGetLastError(), "k1_reduce launch");
+}
+
+void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream) {
+  const int es = elem_size(dtype);
+  if (es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
+  if (world > 1 && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
+  PairTable tab;
+  // dst == src is allowed when scaling in place (div_ of a chunk); partial overlap never is
+  std::vector<tdm_pair> kept;
+  for (int i = 0; i < npairs && pairs != nullptr; ++i) {
+    if (pairs[i].dst == pairs[i].src && pairs[i].count > 0 && world <= 1) continue;  // copying onto itself
+    kept.push_back(pairs[i]);
+  }
+  if (npairs > 0 && pairs == nullptr) throw Invalid("pairs is NULL");
+  if (npairs < 0 || npairs > TDM_MAX_PAIRS) throw Invalid("npairs must be in [0, " + std::to_string(TDM_MAX_PAIRS) + "]");
+  for (const tdm_pair& p : kept) {
+    if (p.count > 0 && p.dst != p.src && p.dst != nullptr && p.src != nullptr) {
+      const uintptr_t d = reinterpret_cast<uintptr_t>(p.dst), s = reinterpret_cast<uintptr_t>(p.src);
+      const uintptr_t bytes = static_cast<uintptr_t>(p.count) * es;
+      if (d < s + bytes && s < d + bytes) throw Invalid("copy: destination and source overlap");
+    }
+  }
+  const int64_t tiles = build_pairs(kept.data(), static_cast<int>(kept.size()), es, false, &tab);
+  if (tiles == 0) return;
+  switch (dtype) {
+    case TDM_F32: launch_copy<float>(tab, tiles, world, stream); break;
+    case TDM_F64: launch_copy<double>(tab, tiles, world, stream); break;
+    case TDM_F16: launch_copy<f16_t>(tab, tiles, world, stream); break;
+    case TDM_BF16: launch_copy<bf16_t>(tab, tiles, world, stream); break;
+    case TDM_I64: launch_copy<int64_t>(tab, tiles, 1, stream); break;
+    default: launch_copy<int32_t>(tab, tiles, 1, stream); break;
+  }
+  check_hip(hipGetLastError(), "k1_copy launch");
+}
+
+}  // namespace tandem_hip
+
+using namespace tandem_hip;
+
+extern "C" {
+
+int tdm_set_blocks_per_cu(int blocks) {
+  return guard([&] {
+    if (blocks < 0 || blocks > 64) throw Invalid("blocks per compute unit must be in [0, 64]");
+    g_blocks_per_cu = blocks == 0 ? kDefaultBlocksPerCu : blocks;
+  });
+}
+
+int tdm_k1_reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, int scale_dst, int scale_src,
+                       int writeback_src, tdm_stream stream) {
+  return guard([&] {
+    reduce_step(pairs, npairs, dtype, world, scale_dst != 0, scale_src != 0, writeback_src != 0,
+                static_cast<hipStream_t>(stream));
+  });
+}
+
+int tdm_k1_copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, tdm_stream stream) {
+  return guard([&] { copy_step(pairs, npairs, dtype, world, static_cast<hipStream_t>(stream)); });
+}
+
+int64_t tdm_k2_table_bytes(int nseg) {
+  if (nseg < 0) return 0;
+  return fold_segs_offset(nseg) + static_cast<int64_t>(nseg) * static_cast<int64_t>(sizeof(FoldSegDev));
+}
+
+int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype, void* image) {
+  return guard([&] {
+    const int es = elem_size(dtype);
+    if (es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
+    if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
+    if (nseg < 0 || (nseg > 0 && segs == nullptr) || image == nullptr) throw Invalid("bad table arguments");
+    char* img = static_cast<char*>(image);
+    std::memset(img, 0, static_cast<size_t>(tdm_k2_table_bytes(nseg)));
+    FoldHeader* hd = reinterpret_cast<FoldHeader*>(img);
+    int64_t* tile_end = reinterpret_cast<int64_t*>(img + fold_tile_end_offset());
+    FoldSegDev* out = reinterpret_cast<FoldSegDev*>(img + fold_segs_offset(nseg));
+    const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
+    int64_t tiles = 0;
+    for (int i = 0; i < nseg; ++i) {
+      const tdm_fold_seg& s = segs[i];
+      if (s.count < 0) throw Invalid("segment " + std::to_string(i) + ": negative count");
+      if (s.chunk < 0 || s.chunk >= world) throw Invalid("segment " + std::to_string(i) + ": chunk outside [0, world)");
+      bool vec = true;
+      for (int r = 0; r < world; ++r) {
+        if (s.count > 0 && s.src[r] == nullptr) throw Invalid("segment " + std::to_string(i) + ": NULL source");
+        const uintptr_t a = reinterpret_cast<uintptr_t>(s.src[r]), b = reinterpret_cast<uintptr_t>(s.dst[r]);
+        if (a % es || b % es) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to the element size");
+        vec = vec && a % 16 == 0 && b % 16 == 0;
+        out[i].src[r] = static_cast<const char*>(s.src[r]);
+        out[i].dst[r] = static_cast<char*>(s.dst[r]);
+      }
+      out[i].count = s.count;
+      out[i].chunk = s.chunk;
+      out[i].vec_ok = vec;
+      tiles += (s.count + tile_elems - 1) / tile_elems;
+      tile_end[i] = tiles;
+    }
+    hd->magic = kFoldMagic;
+    hd->nseg = nseg;
+    hd->world = world;
+    hd->dtype = dtype;
+    hd->total_tiles = tiles;
+  });
+}
+
+int tdm_k2_bucket_fold(const void* table_dev, int nseg, int dtype, int world, int average, tdm_stream stream) {
+  return guard([&] {
+    if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
+    if (nseg < 0) throw Invalid("nseg is negative");
+    if (nseg == 0) return;
+    if (table_dev == nullptr) throw Invalid("table is NULL");
+    if (average && world > 1 && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
+    // The tile count lives in the device image; reading it back would stall the
+    // stream, so the grid is sized for the device and the kernel strides.
+    const int64_t many = static_cast<int64_t>(compute_units()) * g_blocks_per_cu;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+      case TDM_F32: launch_fold<float>(table_dev, many, world, average, st); break;
+      case TDM_F64: launch_fold<double>(table_dev, many, world, average, st); break;
+      case TDM_F16: launch_fold<f16_t>(table_dev, many, world, average, st); break;
+      case TDM_BF16: launch_fold<bf16_t>(table_dev, many, world, average, st); break;
+      case TDM_I64: launch_fold<int64_t>(table_dev, many, world, 0, st); break;
+      case TDM_I32: launch_fold<int32_t>(table_dev, many, world, 0, st); break;
+      default: throw Invalid("unknown dtype " + std::to_string(dtype));
+    }
+    check_hip(hipGetLastError(), "k2_fold launch");
+  });
+}
+
+int tdm_k3_adamw(float* p, const float* g, float* m, float* v, int64_t n, const tdm_adamw_scalars* s, int order,
+                 tdm_stream stream) {
+  return guard([&] {
+    if (n < 0) throw Invalid("n is negative");
+    if (n == 0) return;
+    if (!p || !g || !m || !v || !s) throw Invalid("NULL argument");
+    if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
+    const uintptr_t ptrs[4] = {reinterpret_cast<uintptr_t>(p), reinterpret_cast<uintptr_t>(g),
+                               reinterpret_cast<uintptr_t>(m), reinterpret_cast<uintptr_t>(v)};
+    bool vec = true;
+    for (uintptr_t a : ptrs) {
+      if (a % 4) throw Invalid("pointer not aligned to 4 bytes");
+      vec = vec && a % 16 == 0;
+    }
+    for (int i = 0; i < 4; ++i)
+      for (int j = i + 1; j < 4; ++j) {
+        const uintptr_t bytes = static_cast<uintptr_t>(n) * 4;
+        if (ptrs[i] < ptrs[j] + bytes && ptrs[j] < ptrs[i] + bytes) throw Invalid("p, g, m, v must not overlap");
+      }
+    AdamwArgs a{p, g, m, v, n, *s};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 block(kThreads);
+    if (vec) {
+      const int64_t tiles = (n / 4 + kThreads * 2 - 1) / (kThreads * 2);
+      const dim3 grid(grid_for(std::max<int64_t>(tiles, 1)));
+      if (order == TDM_ADAMW_HOST_ORDER) hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true>), grid, block, 0, st, a);
+      else hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true>), grid, block, 0, st, a);
+    } else {
+      const dim3 grid(grid_for((n + kThreads - 1) / kThreads));
+      if (order == TDM_ADAMW_HOST_ORDER) hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, false>), grid, block, 0, st, a);
+      else hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, false>), grid, block, 0, st, a);
+    }
+    check_hip(hipGetLastError(), "k3_adamw launch");
+  });
+}
+
+int tdm_k4_unit_gather(void* full, const void* const* shards, const int64_t* sizes, int world, int dtype,
+                       tdm_stream stream) {
+  return guard([&] {
+    const int es = elem_size(dtype);
+    if (es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
+    if (world < 1 || world > TDM_MAX_PAIRS) throw Invalid("world must be in [1, 16]");
+    if (!full || !shards || !sizes) throw Invalid("NULL argument");
+    tdm_pair pairs[TDM_MAX_PAIRS];
+    int np = 0;
+    int64_t lo = 0;
+    for (int q = 0; q < world; ++q) {
+      if (sizes[q] < 0) throw Invalid("negative shard size");
+      char* dst = static_cast<char*>(full) + lo * es;
+      if (sizes[q] > 0) {
+        if (shards[q] == nullptr) throw Invalid("NULL shard");
+        if (shards[q] != dst) pairs[np++] = tdm_pair{dst, shards[q], sizes[q]};
+      }
+      lo += sizes[q];
+    }
+    copy_step(pairs, np, dtype, 0, static_cast<hipStream_t>(stream));
+  });
+}
+
+}  // extern "C"

@@ -1,0 +1,218 @@
+"""A whole group on one GPU, in one process: rank r is a buffer in that GPU's HBM.
+
+`LocalWorld(world)` runs tandem's ring collectives over a list of `world`
+tensors (one per rank) with ONE kernel launch per ring step: the launch carries
+every rank's (receive chunk, neighbour's chunk) pair, so a step that the
+reference runs as `world` processes x pieces x (copy into a slot, add out of
+it) is a single fused pass over HBM. The results, including the partial sums a
+bare reduce_scatter leaves in the other chunks, are bit for bit those of the
+reference's Python engine (tandem/comm.py:301-385 there).
+
+Everything is enqueued on torch's current stream; nothing synchronises.
+"""
+
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import Pair, check, dtype_code, lib, require_device_tensor, stream_ptr
+
+
+def split_sizes(n, world):
+    """Sizes of torch.tensor_split(flat, world): the first n % world chunks get
+    one element more (tandem/comm.py:319-321, tandem/zero.py:29-30)."""
+    base, extra = divmod(int(n), world)
+    return [base + (1 if q < extra else 0) for q in range(world)]
+
+
+def chunk_bounds(numel, world, sizes=None):
+    """[lo, hi) per rank; explicit sizes must partition the tensor, as
+    tandem/comm.py:322-324 demands."""
+    if sizes is None:
+        sizes = split_sizes(numel, world)
+    sizes = [int(s) for s in sizes]
+    if len(sizes) != world or sum(sizes) != numel or any(s < 0 for s in sizes):
+        raise ValueError(f"chunk sizes {sizes} do not partition {numel} elements")
+    out, lo = [], 0
+    for s in sizes:
+        out.append((lo, lo + s))
+        lo += s
+    return out
+
+
+def _pairs(items):
+    arr = (Pair * max(1, len(items)))()
+    for i, (dst, src, count) in enumerate(items):
+        arr[i].dst, arr[i].src, arr[i].count = dst, src, count
+    return arr
+
+
+class LocalWorld:
+    def __init__(self, world):
+        if world < 1:
+            raise ValueError("world must be at least 1")
+        if world > _lib.TDM_MAX_PAIRS:
+            raise ValueError(f"LocalWorld handles up to {_lib.TDM_MAX_PAIRS} ranks per launch")
+        self.world = world
+        lib()  # fail now, not at the first collective, if the HIP library is missing
+
+    # ---- checks
+    def _flat(self, bufs, what):
+        if len(bufs) != self.world:
+            raise ValueError(f"{what}: expected {self.world} rank buffers, got {len(bufs)}")
+        flats = []
+        for t in bufs:
+            require_device_tensor(t, what)
+            flats.append(t.reshape(-1))
+        f0 = flats[0]
+        for f in flats[1:]:
+            if f.numel() != f0.numel() or f.dtype != f0.dtype or f.device != f0.device:
+                raise ValueError(f"{what}: rank buffers differ in size, dtype or device")
+        return flats
+
+    @staticmethod
+    def _op(op):
+        if op not in ("sum", "avg"):
+            raise ValueError(f"unknown op {op}")
+        return op == "avg"
+
+    # ---- ring steps: one launch each
+    def _reduce_scatter(self, flats, bounds, average, keep_sent):
+        n = self.world
+        es = flats[0].element_size()
+        code = dtype_code(flats[0].dtype)
+        base = [f.data_ptr() for f in flats]
+        st = stream_ptr(flats[0].device)
+        for s in range(n - 1):
+            items = []
+            for r in range(n):
+                lo, hi = bounds[(r - s - 2) % n]  # rank r adds what rank r-1 sends (tandem/comm.py:305)
+                if hi > lo:
+                    items.append((base[r] + lo * es, base[(r - 1) % n] + lo * es, hi - lo))
+            if items:
+                # Every receiving chunk is still undivided; the sender's is only on the
+                # first step. keep_sent: the first step also leaves x / n in the sender's
+                # chunk, which div_ of the whole tensor would have (a bare reduce_scatter
+                # shows it; an all_reduce overwrites it anyway).
+                check(lib().tdm_k1_reduce_step(_pairs(items), len(items), code, n if average else 1,
+                                               1, int(s == 0), int(s == 0 and keep_sent), st))
+
+    def _all_gather(self, flats, bounds):
+        n = self.world
+        es = flats[0].element_size()
+        code = dtype_code(flats[0].dtype)
+        base = [f.data_ptr() for f in flats]
+        st = stream_ptr(flats[0].device)
+        for s in range(n - 1):
+            items = []
+            for r in range(n):
+                lo, hi = bounds[(r - s - 1) % n]  # tandem/comm.py:311
+                if hi > lo:
+                    items.append((base[r] + lo * es, base[(r - 1) % n] + lo * es, hi - lo))
+            if items:
+                check(lib().tdm_k1_copy_step(_pairs(items), len(items), code, 0, st))
+
+    # ---- collectives over all ranks at once
+    def reduce_scatter(self, bufs, sizes=None, op="sum"):
+        """In place on every rank's buffer; returns each rank's reduced chunk
+        (a view), as Group.reduce_scatter does per rank (tandem/comm.py:349-369)."""
+        average = self._op(op)
+        flats = self._flat(bufs, "reduce_scatter")
+        bounds = chunk_bounds(flats[0].numel(), self.world, sizes)
+        if self.world > 1:
+            self._reduce_scatter(flats, bounds, average, True)
+        return [flats[r][bounds[r][0]:bounds[r][1]] for r in range(self.world)]
+
+    def all_gather(self, bufs, sizes=None):
+        """Rank r holds chunk r; afterwards every rank holds every chunk
+        (tandem/comm.py:371-385)."""
+        flats = self._flat(bufs, "all_gather")
+        bounds = chunk_bounds(flats[0].numel(), self.world, sizes)
+        if self.world > 1:
+            self._all_gather(flats, bounds)
+        return bufs
+
+    def all_reduce(self, bufs, op="sum"):
+        """Ring all-reduce in place: reduce-scatter then all-gather over the
+        tensor_split chunks (tandem/comm.py:326-347)."""
+        average = self._op(op)
+        flats = self._flat(bufs, "all_reduce")
+        if self.world > 1:
+            bounds = chunk_bounds(flats[0].numel(), self.world, None)
+            self._reduce_scatter(flats, bounds, average, False)
+            self._all_gather(flats, bounds)
+        return bufs
+
+    def unit_gather(self, fulls, shards, sizes):
+        """ZeRO-3's gather of one unit for every rank: fulls[r] receives every
+        rank's shard in one launch per rank (tandem/zero.py:238-245)."""
+        if len(fulls) != self.world or len(shards) != self.world:
+            raise ValueError("unit_gather: one full buffer and one shard per rank")
+        bounds = chunk_bounds(fulls[0].numel(), self.world, sizes)
+        for t in list(fulls) + list(shards):
+            require_device_tensor(t, "unit_gather")
+        for q, (lo, hi) in enumerate(bounds):
+            if shards[q].numel() != hi - lo or shards[q].dtype != fulls[0].dtype:
+                raise ValueError(f"unit_gather: shard {q} has {shards[q].numel()} elements, its chunk {hi - lo}")
+        code = dtype_code(fulls[0].dtype)
+        ptrs = (ctypes.c_void_p * self.world)(*[s.data_ptr() for s in shards])
+        szs = (ctypes.c_int64 * self.world)(*[hi - lo for lo, hi in bounds])
+        st = stream_ptr(fulls[0].device)
+        for full in fulls:
+            check(lib().tdm_k4_unit_gather(ctypes.c_void_p(full.data_ptr()), ptrs, szs, self.world, code, st))
+        return fulls
+
+    def bucket_table(self, tensors_per_rank, buckets, out_per_rank=None):
+        """Prepares the K2 launch for DDP's bucket path with every rank on this
+        GPU. tensors_per_rank[r][i] is rank r's gradient of parameter i;
+        `buckets` lists the parameter positions of each bucket in packing order
+        (tandem/ddp.py:56-68). The table is built and uploaded once; run() then
+        averages every gradient across the ranks in one launch, writing the result
+        to out_per_rank[r][i] (default: in place), bit for bit what flattening into
+        the bucket, ring all_reduce(op="avg") and reading the views back gives."""
+        return FoldTable(self, tensors_per_rank, buckets, out_per_rank)
+
+
+class FoldTable:
+    def __init__(self, lw, tensors_per_rank, buckets, out_per_rank=None):
+        from .buckets import fold_segments
+
+        world = lw.world
+        if world > _lib.TDM_MAX_WORLD:
+            raise ValueError(f"the bucket fold handles up to {_lib.TDM_MAX_WORLD} ranks")
+        if len(tensors_per_rank) != world:
+            raise ValueError("bucket_table: one list of gradients per rank")
+        outs = tensors_per_rank if out_per_rank is None else out_per_rank
+        first = tensors_per_rank[0]
+        for r in range(world):
+            if len(tensors_per_rank[r]) != len(first) or len(outs[r]) != len(first):
+                raise ValueError("bucket_table: ranks differ in their number of tensors")
+            for i, t in enumerate(tensors_per_rank[r]):
+                require_device_tensor(t, "bucket_table")
+                require_device_tensor(outs[r][i], "bucket_table")
+                if t.numel() != first[i].numel() or t.dtype != first[0].dtype or outs[r][i].numel() != t.numel():
+                    raise ValueError("bucket_table: ranks differ in a tensor's size or dtype")
+        self.world, self.dtype, self.device = world, first[0].dtype, first[0].device
+        self._keep = (tensors_per_rank, outs)  # the table holds raw addresses of these
+        es = first[0].element_size()
+        rows = []
+        for members in buckets:
+            for i, off, count, chunk in fold_segments([first[i].numel() for i in members], world):
+                rows.append((members[i], off, count, chunk))
+        self.nseg = len(rows)
+        self.elements = sum(r[2] for r in rows)
+        segs = (_lib.FoldSeg * max(1, self.nseg))()
+        for k, (i, off, count, chunk) in enumerate(rows):
+            for r in range(world):
+                segs[k].src[r] = tensors_per_rank[r][i].data_ptr() + off * es
+                segs[k].dst[r] = outs[r][i].data_ptr() + off * es
+            segs[k].count, segs[k].chunk = count, chunk
+        nbytes = lib().tdm_k2_table_bytes(self.nseg)
+        image = torch.empty(max(16, nbytes), dtype=torch.uint8)
+        check(lib().tdm_k2_table_build(segs, self.nseg, world, dtype_code(self.dtype), ctypes.c_void_p(image.data_ptr())))
+        self.image = image.to(self.device)
+
+    def run(self, average=True):
+        check(lib().tdm_k2_bucket_fold(ctypes.c_void_p(self.image.data_ptr()), self.nseg, dtype_code(self.dtype),
+                                       self.world, int(average), stream_ptr(self.device)))

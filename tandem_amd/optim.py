@@ -1,0 +1,72 @@
+"""AdamW on flat fp32 shards of the parameters, for the ZeRO stages: one fused
+HIP kernel per shard instead of seven elementwise passes.
+
+Same interface as tandem's ShardedAdamW (tandem/optim.py:11-40 there) and the
+same arithmetic, operation for operation: the step's scalars are computed in
+Python doubles by the same expressions and rounded to fp32 once, as torch does
+when it applies a Python scalar to a float tensor; the per-element work is
+tdm_k3_adamw."""
+
+import ctypes
+
+import torch
+
+from ._lib import ADAMW_DEVICE_ORDER, ADAMW_HOST_ORDER, AdamwScalars, check, lib, require_device_tensor, stream_ptr
+
+
+def step_scalars(step, lr, betas, eps, weight_decay):
+    """The constants of step `step` (a float, 1-based), tandem/optim.py:28-37."""
+    beta1, beta2 = betas
+    bias_correction1 = 1 - beta1 ** step
+    bias_correction2 = 1 - beta2 ** step
+    step_size = lr / bias_correction1
+    bias_correction2_sqrt = bias_correction2 ** 0.5
+    s = AdamwScalars()
+    s.use_decay = int(weight_decay != 0)
+    s.decay = 1 - lr * weight_decay  # ctypes rounds a Python float to fp32 (nearest even) on assignment
+    s.w1 = 1 - beta1
+    s.beta2 = beta2
+    s.one_m_b2 = 1 - beta2
+    s.bc2_sqrt = bias_correction2_sqrt
+    s.eps = eps
+    s.neg_step = -step_size
+    return s
+
+
+class ShardedAdamW:
+    """order="host" reproduces torch's CPU addcdiv_ (p + (step*m)/d), which is
+    what the reference's CPU engine computes; order="device" reproduces torch's
+    GPU addcdiv_ kernel (fma(step, m/d, p)), for comparing with
+    torch.optim.AdamW run on the GPU itself."""
+
+    def __init__(self, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, order="host"):
+        if order not in ("host", "device"):
+            raise ValueError(f"unknown update order {order}")
+        self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
+        self.order = ADAMW_HOST_ORDER if order == "host" else ADAMW_DEVICE_ORDER
+        self.state = {}  # key -> [step, exp_avg, exp_avg_sq]
+        lib()
+
+    def update(self, key, param, grad):
+        """One step for one shard: `param` and `grad` are same-shaped fp32
+        tensors in GPU memory; `key` names the shard's optimizer state."""
+        require_device_tensor(param, "ShardedAdamW.update(param)")
+        require_device_tensor(grad, "ShardedAdamW.update(grad)")
+        if param.dtype != torch.float32 or grad.dtype != torch.float32:
+            raise ValueError("ShardedAdamW handles fp32 shards")
+        if param.shape != grad.shape:
+            raise ValueError("param and grad differ in shape")
+        if key not in self.state:
+            self.state[key] = [0.0, torch.zeros_like(param), torch.zeros_like(param)]
+        st = self.state[key]
+        st[0] += 1.0
+        step, exp_avg, exp_avg_sq = st
+        if param.numel() == 0:
+            return
+        s = step_scalars(step, self.lr, self.betas, self.eps, self.weight_decay)
+        check(lib().tdm_k3_adamw(ctypes.c_void_p(param.data_ptr()), ctypes.c_void_p(grad.data_ptr()),
+                                 ctypes.c_void_p(exp_avg.data_ptr()), ctypes.c_void_p(exp_avg_sq.data_ptr()),
+                                 param.numel(), ctypes.byref(s), self.order, stream_ptr(param.device)))
+
+    def state_bytes(self):
+        return sum(t.numel() * t.element_size() for _, a, b in self.state.values() for t in (a, b))

@@ -1,0 +1,79 @@
+"""The C-ABI library loads without a GPU and exports every entry point that
+include/tandem_hip.h declares (no compute calls here)."""
+
+import ctypes
+import os
+import re
+
+from helpers import GOLDEN
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "tandem_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tdm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_entry_point():
+    from tandem_amd import _lib
+
+    L = _lib.lib()
+    names = declared_functions()
+    assert len(names) >= 11
+    for name in names:
+        assert hasattr(L, name), f"{name} is declared in tandem_hip.h but not exported"
+    assert sorted(_lib.exported_symbols()) == names, "the ctypes binding and the header disagree"
+    assert L.tdm_abi_version() == _lib.ABI_VERSION
+    assert L.tdm_last_error() == b""
+
+
+def test_struct_layouts_match_the_header():
+    from tandem_amd import _lib
+
+    assert ctypes.sizeof(_lib.Pair) == 24
+    assert ctypes.sizeof(_lib.FoldSeg) == 8 * 8 * 2 + 16
+    assert ctypes.sizeof(_lib.AdamwScalars) == 32
+
+
+def test_argument_errors_need_no_gpu():
+    from tandem_amd import _lib
+
+    L = _lib.lib()
+    assert L.tdm_k1_reduce_step(None, 17, 0, 2, 1, 1, 0, None) == 1
+    assert b"npairs" in L.tdm_last_error()
+    assert L.tdm_k1_copy_step(None, 0, 99, 0, None) == 1
+    assert L.tdm_k2_table_bytes(0) > 0 and L.tdm_k2_table_bytes(3) > L.tdm_k2_table_bytes(2)
+    assert L.tdm_set_blocks_per_cu(1000) == 1
+    assert L.tdm_set_blocks_per_cu(0) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from tandem_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    try:
+        _lib.lib()
+    except _lib.HipLibraryMissing as e:
+        assert "no CPU" in str(e)
+    else:
+        raise AssertionError("a missing library must raise")
+
+
+def test_cpu_tensors_are_refused():
+    import pytest
+    import torch
+
+    from tandem_amd import LocalWorld, ShardedAdamW
+
+    with pytest.raises(ValueError, match="no CPU path"):
+        LocalWorld(2).all_reduce([torch.zeros(4), torch.zeros(4)])
+    with pytest.raises(ValueError, match="no CPU path"):
+        ShardedAdamW().update("k", torch.zeros(4), torch.zeros(4))
+
+
+def test_fixtures_present():
+    for f in ("ring_w2.npz", "ring_w3.npz", "ring_w4.npz", "ring_dtypes_w3.npz", "adamw.npz", "plans.json", "data.json"):
+        assert os.path.exists(os.path.join(GOLDEN, f))

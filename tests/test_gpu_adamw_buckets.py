@@ -1,0 +1,168 @@
+"""K3 (sharded AdamW) and K2 (bucket fold) on the GPU against the CPU oracle,
+the reference's fixtures and torch's own AdamW. Run with -m gpu on an MI355X."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import bits, golden_json, golden_npz, npz_json, seeded
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return torch.device("cuda", 0)
+
+
+def test_adamw_bit_exact_with_oracle(dev):
+    """Twenty steps with the benchmark's hyper-parameters, on a shard whose length
+    is not a multiple of anything; then the other branches (no decay, beta1 < 0.5)
+    and a shard that starts 4 bytes off a 16-byte boundary."""
+    from oracle.adamw import AdamW as Oracle
+    from tandem_amd import ShardedAdamW
+
+    n = 100_003
+    g = torch.Generator().manual_seed(5)
+    p0 = torch.randn(n, generator=g) * 0.02
+    p0[:6] = torch.tensor([0.0, -0.0, 1e-30, -3e-39, 1e-45, 5.0])
+    for kw, shift in ((dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1), 0),
+                      (dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0), 0),
+                      (dict(lr=1e-2, betas=(0.3, 0.7), eps=1e-6, weight_decay=0.5), 1)):
+        ours, ref = ShardedAdamW(**kw), Oracle(**kw)
+        store = torch.zeros(n + 4, device=dev)
+        p = store[shift:shift + n]
+        p.copy_(p0)
+        pn = p0.numpy().copy()
+        for step in range(20):
+            gr = torch.randn(n, generator=g) * 1e-3
+            gr[:3] = 0.0
+            ours.update("k", p, gr.to(dev))
+            ref.update("k", pn, gr.numpy())
+        _, m, v = ours.state["k"]
+        assert np.array_equal(bits(m.cpu().numpy()), bits(ref.state["k"][1])), kw
+        assert np.array_equal(bits(v.cpu().numpy()), bits(ref.state["k"][2])), kw
+        assert np.array_equal(bits(p.cpu().numpy()), bits(pn)), kw
+        assert ours.state["k"][0] == 20.0 and ours.state_bytes() == 2 * 4 * n
+
+
+def test_adamw_against_reference_fixture(dev):
+    """The reference ran on torch's CPU kernels, whose vectorised sqrt is not
+    correctly rounded: moments must match bit for bit, parameters to 1 ulp of the
+    update term per step."""
+    from tandem_amd import ShardedAdamW
+
+    d = golden_npz("adamw.npz")
+    h = npz_json(d, "hyper_json")["main"]
+    opt = ShardedAdamW(h["lr"], tuple(h["betas"]), h["eps"], h["weight_decay"])
+    p = torch.from_numpy(d["p0"].copy()).to(dev)
+    for s in range(h["steps"]):
+        opt.update("k", p, torch.from_numpy(d["grads"][s].copy()).to(dev))
+        if s == 0:
+            _, m, v = opt.state["k"]
+            assert np.array_equal(bits(m.cpu().numpy()), bits(d["m1"]))
+            assert np.array_equal(bits(v.cpu().numpy()), bits(d["v1"]))
+            upd = np.abs(d["p1"].astype(np.float64) - d["p0"].astype(np.float64) * (1 - h["lr"] * h["weight_decay"]))
+            tol = np.spacing(upd.astype(np.float32)).astype(np.float64) + np.spacing(np.abs(d["p1"])).astype(np.float64)
+            assert np.all(np.abs(p.cpu().numpy().astype(np.float64) - d["p1"]) <= tol)
+    _, m, v = opt.state["k"]
+    assert np.array_equal(bits(m.cpu().numpy()), bits(d["m20"]))
+    assert np.array_equal(bits(v.cpu().numpy()), bits(d["v20"]))
+    got = p.cpu().numpy()
+    assert np.abs(got.astype(np.float64) - d["p20"]).max() <= 20 * 2 * np.spacing(np.float32(h["lr"]))
+    assert (bits(got) != bits(d["p20"])).mean() < 0.05
+
+
+def test_adamw_device_order_matches_torch_on_the_gpu(dev):
+    """torch.optim.AdamW(foreach=False) run on the GPU itself: its addcdiv_ kernel
+    computes fma(step, m/d, p); order="device" reproduces that bit for bit."""
+    from tandem_amd import ShardedAdamW
+
+    n = 250_000
+    g = torch.Generator().manual_seed(8)
+    p0 = torch.randn(n, generator=g) * 0.02
+    kw = dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    pt = torch.nn.Parameter(p0.clone().to(dev))
+    topt = torch.optim.AdamW([pt], foreach=False, fused=False, **kw)
+    ours = ShardedAdamW(order="device", **kw)
+    p = p0.clone().to(dev)
+    for _ in range(20):
+        gr = (torch.randn(n, generator=g) * 1e-3).to(dev)
+        pt.grad = gr.clone()
+        topt.step()
+        ours.update(0, p, gr)
+    st = topt.state[pt]
+    assert torch.equal(ours.state[0][1].view(torch.int32), st["exp_avg"].view(torch.int32))
+    assert torch.equal(ours.state[0][2].view(torch.int32), st["exp_avg_sq"].view(torch.int32))
+    assert torch.equal(p.view(torch.int32), pt.detach().view(torch.int32))
+
+
+def test_adamw_rejects_what_it_cannot_do(dev):
+    from tandem_amd import ShardedAdamW
+
+    opt = ShardedAdamW()
+    with pytest.raises(ValueError):
+        opt.update("cpu", torch.zeros(4), torch.zeros(4))
+    with pytest.raises(ValueError):
+        opt.update("half", torch.zeros(4, device=dev, dtype=torch.float16), torch.zeros(4, device=dev, dtype=torch.float16))
+    opt.update("empty", torch.zeros(0, device=dev), torch.zeros(0, device=dev))
+    assert opt.state["empty"][0] == 1.0
+    p = torch.zeros(8, device=dev)
+    with pytest.raises(ValueError):
+        opt.update("alias", p, p)  # p and g overlap
+
+
+@pytest.mark.parametrize("world", [2, 3, 4])
+def test_bucket_fold_equals_flatten_allreduce_unflatten(dev, world):
+    """K2 against the oracle's ring all-reduce of each flattened bucket, for the
+    small GPT's parameter list with the reference's packing (plans.json)."""
+    from oracle import ring
+    from tandem_amd import LocalWorld
+    from tandem_amd.buckets import pack
+
+    plan = golden_json("plans.json")
+    names = [n for n, _ in plan["small_params"]]
+    numels = [math.prod(s) for _, s in plan["small_params"]]
+    order = list(range(len(numels)))[::-1]
+    groups = pack([numels[i] * 4 for i in order], 4 << 10)
+    buckets = [[order[k] for k in grp] for grp in groups]
+    assert [[names[i] for i in b] for b in buckets] == plan["small_ddp_4KiB"]
+    grads = [[(seeded(r, i, numels[i]) * 1e-3) for i in range(len(numels))] for r in range(world)]
+    dgrads = [[t.to(dev) for t in grads[r]] for r in range(world)]
+    lw = LocalWorld(world)
+    table = lw.bucket_table(dgrads, buckets)
+    assert table.elements == sum(numels)
+    table.run(average=True)
+    for b in buckets:
+        flat = [np.concatenate([grads[r][i].numpy() for i in b]) for r in range(world)]
+        want = ring.expected_all_reduce(flat, True)
+        off = 0
+        for i in b:
+            for r in range(world):
+                assert np.array_equal(bits(dgrads[r][i].cpu().numpy()), bits(want[off:off + numels[i]])), (world, i, r)
+            off += numels[i]
+
+
+def test_bucket_fold_into_other_buffers_and_odd_sizes(dev):
+    from oracle import ring
+    from tandem_amd import LocalWorld
+
+    world = 4
+    numels = [1, 3, 1025, 7, 4096, 10_007, 2]
+    grads = [[seeded(r + 5, i, n) for i, n in enumerate(numels)] for r in range(world)]
+    dgrads = [[t.to(dev) for t in grads[r]] for r in range(world)]
+    outs = [[torch.zeros_like(t) for t in dgrads[r]] for r in range(world)]
+    buckets = [[6, 5, 4], [3, 2], [1, 0]]
+    LocalWorld(world).bucket_table(dgrads, buckets, outs).run(average=False)
+    for b in buckets:
+        flat = [np.concatenate([grads[r][i].numpy() for i in b]) for r in range(world)]
+        want = ring.expected_all_reduce(flat, False)
+        off = 0
+        for i in b:
+            for r in range(world):
+                assert np.array_equal(bits(outs[r][i].cpu().numpy()), bits(want[off:off + numels[i]]))
+                assert torch.equal(dgrads[r][i].cpu(), grads[r][i])  # sources untouched
+            off += numels[i]

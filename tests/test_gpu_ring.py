@@ -1,0 +1,246 @@
+"""K1 / K4 on the GPU, through the C ABI, against the CPU oracle and the fixtures
+written by the reference's Python engine. Bit-exact: every comparison is on bit
+patterns. Run with -m gpu on an MI355X."""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import bits, golden_npz, npz_json, seeded
+
+pytestmark = pytest.mark.gpu
+
+KINDS = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16", torch.int64: "i64"}
+
+
+def to_np(t):
+    t = t.detach().cpu()
+    if t.dtype in (torch.float16, torch.bfloat16):
+        return t.view(torch.int16).numpy().view(np.uint16)
+    return t.numpy()
+
+
+def from_np(a, dtype, dev):
+    if dtype in (torch.float16, torch.bfloat16):
+        return torch.from_numpy(a.view(np.int16).copy()).view(dtype).to(dev)
+    return torch.from_numpy(np.array(a, copy=True)).to(dev)
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return torch.device("cuda", 0)
+
+
+def inputs(world, n, dtype, seed=0):
+    xs = []
+    for r in range(world):
+        if dtype == torch.int64:
+            g = torch.Generator().manual_seed(seed * 1000 + r)
+            xs.append(torch.randint(-1000, 1000, (n,), generator=g))
+        else:
+            xs.append(seeded(seed, r, n).to(dtype))
+    return xs
+
+
+@pytest.mark.parametrize("world", [2, 3, 4])
+def test_fixtures_of_the_reference_engine(dev, world):
+    """Same inputs as the reference run; outputs must equal the reference's, on
+    every rank, for the whole buffer (partial sums included)."""
+    from tandem_amd import LocalWorld
+
+    d = golden_npz(f"ring_w{world}.npz")
+    lw = LocalWorld(world)
+    xs = [d[f"r{r}_in"] for r in range(world)]
+
+    def fresh():
+        return [torch.from_numpy(x.copy()).to(dev) for x in xs]
+
+    for op, key in (("sum", "ar_sum"), ("avg", "ar_avg")):
+        bufs = fresh()
+        lw.all_reduce(bufs, op=op)
+        for r in range(world):
+            assert np.array_equal(bits(to_np(bufs[r])), bits(d[f"r{r}_{key}"])), (key, r)
+    bufs = fresh()
+    lw.reduce_scatter(bufs, None, op="avg")
+    for r in range(world):
+        assert np.array_equal(bits(to_np(bufs[r])), bits(d[f"r{r}_rs_avg_even"]))
+    for name, sizes in npz_json(d, "sizes_json").items():
+        for op in ("avg", "sum"):
+            bufs = fresh()
+            mine = lw.reduce_scatter(bufs, sizes, op=op)
+            lo = 0
+            for r in range(world):
+                want = d[f"r{r}_rs_{op}_{name}"]
+                assert np.array_equal(bits(to_np(bufs[r])), bits(want)), (name, op, r)
+                assert np.array_equal(bits(to_np(mine[r])), bits(want[lo:lo + sizes[r]]))
+                lo += sizes[r]
+        bufs = fresh()
+        lw.all_gather(bufs, sizes)
+        for r in range(world):
+            assert np.array_equal(bits(to_np(bufs[r])), bits(d[f"r{r}_ag_{name}"])), (name, r)
+    bufs = [torch.from_numpy(d[f"r{r}_tiny_in"].copy()).to(dev) for r in range(world)]
+    lw.all_reduce(bufs, op="avg")
+    for r in range(world):
+        assert np.array_equal(bits(to_np(bufs[r])), bits(d[f"r{r}_tiny_ar_avg"]))
+
+
+def test_fixtures_other_dtypes(dev):
+    from tandem_amd import LocalWorld
+
+    d = golden_npz("ring_dtypes_w3.npz")
+    lw = LocalWorld(3)
+    for kind, dtype in (("f64", torch.float64), ("f16", torch.float16), ("bf16", torch.bfloat16)):
+        for op, key in (("sum", "ar_sum"), ("avg", "ar_avg")):
+            bufs = [from_np(d[f"r{r}_{kind}_in"].view(np.uint16) if kind != "f64" else d[f"r{r}_{kind}_in"], dtype, dev)
+                    for r in range(3)]
+            lw.all_reduce(bufs, op=op)
+            for r in range(3):
+                assert np.array_equal(bits(to_np(bufs[r])), bits(d[f"r{r}_{kind}_{key}"])), (kind, key, r)
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16, torch.int64])
+def test_against_oracle(dev, world, dtype):
+    """The sizes the reference tests use (tests/test_comm.py:10, test_engine_cuda.py:34
+    there) plus sizes that cross the kernel's tile and vector boundaries."""
+    from oracle import ring
+    from tandem_amd import LocalWorld
+
+    kind = KINDS[dtype]
+    lw = LocalWorld(world)
+    for n in (0, 1, 5, 64, 1000, 4099, 10_007, 65_536 + 3):
+        xs = inputs(world, n, dtype)
+        xn = [to_np(x) for x in xs]
+        ops = ("sum",) if dtype == torch.int64 else ("sum", "avg")
+        for op in ops:
+            bufs = [x.to(dev) for x in xs]
+            lw.all_reduce(bufs, op=op)
+            want = ring.expected_all_reduce(xn, op == "avg", kind)
+            for r in range(world):
+                assert np.array_equal(bits(to_np(bufs[r])), bits(want)), (world, dtype, n, op, r)
+            sizes = [n // world] * world
+            sizes[-1] += n - sum(sizes)
+            sizes = sizes[1:] + sizes[:1]  # uneven, and empty when n < world
+            bufs = [x.to(dev) for x in xs]
+            lw.reduce_scatter(bufs, sizes, op=op)
+            want = ring.expected_reduce_scatter(xn, sizes, op == "avg", kind)
+            for r in range(world):
+                assert np.array_equal(bits(to_np(bufs[r])), bits(want[r])), (world, dtype, n, op, r)
+        bufs = [x.to(dev) for x in xs]
+        lw.all_gather(bufs, sizes)
+        want = ring.expected_all_gather(xn, sizes)
+        for r in range(world):
+            assert np.array_equal(bits(to_np(bufs[r])), bits(want))
+
+
+def test_unaligned_views_and_special_values(dev):
+    """Views that start 4 bytes into an allocation (no 16-byte alignment, and
+    ranks that disagree on their phase), denormals, signed zeros, infinities."""
+    from oracle import ring
+    from tandem_amd import LocalWorld
+
+    world, n = 4, 9001
+    lw = LocalWorld(world)
+    special = torch.tensor([0.0, -0.0, 1e-45, -1e-45, 1e-39, 3e38, -3e38, float("inf"), float("-inf"), float("nan"),
+                            1.17549435e-38, 2e-38], dtype=torch.float32)
+    xs = []
+    for r in range(world):
+        x = seeded(2, r, n)
+        x[r:r + special.numel()] = special
+        x[100:110] = 1e-40 * (r + 1)
+        xs.append(x)
+    xn = [x.numpy() for x in xs]
+    for shifts in ([1, 1, 1, 1], [0, 1, 2, 3], [3, 0, 0, 1]):
+        for op in ("sum", "avg"):
+            store = [torch.zeros(n + 8, device=dev) for _ in range(world)]
+            bufs = [store[r][shifts[r]:shifts[r] + n] for r in range(world)]
+            for b, x in zip(bufs, xs):
+                b.copy_(x)
+            lw.all_reduce(bufs, op=op)
+            want = ring.expected_all_reduce(xn, op == "avg")
+            for r in range(world):
+                got = to_np(bufs[r])
+                nan = np.isnan(want)
+                assert np.array_equal(np.isnan(got), nan)
+                assert np.array_equal(bits(got)[~nan], bits(want)[~nan]), (shifts, op, r)
+                # nothing outside the view was touched
+                assert float(store[r][:shifts[r]].abs().sum()) == 0 and float(store[r][shifts[r] + n:].abs().sum()) == 0
+
+
+def test_unit_gather(dev):
+    from tandem_amd import LocalWorld
+
+    for world, numel in ((2, 7_087_872), (4, 10_007), (3, 2)):
+        lw = LocalWorld(world)
+        sizes = [numel // world + (1 if q < numel % world else 0) for q in range(world)]
+        shards = [seeded(4, q, sizes[q]).to(dev) for q in range(world)]
+        fulls = [torch.full((numel,), -7.0, device=dev) for _ in range(world)]
+        lw.unit_gather(fulls, shards, sizes)
+        want = torch.cat(shards)
+        for f in fulls:
+            assert torch.equal(f, want)
+    # a shard that already lies in place is left alone
+    lw = LocalWorld(2)
+    full = torch.arange(10, dtype=torch.float32, device=dev)
+    other = torch.full((4,), 5.0, device=dev)
+    lw.unit_gather([full, full.clone()], [full[:6], other], [6, 4])
+    assert torch.equal(full, torch.tensor([0, 1, 2, 3, 4, 5, 5, 5, 5, 5.0], device=dev))
+
+
+def test_bad_arguments_raise(dev):
+    from tandem_amd import LocalWorld, _lib
+
+    lw = LocalWorld(2)
+    a, b = torch.zeros(8, device=dev), torch.zeros(8, device=dev)
+    with pytest.raises(ValueError):
+        lw.reduce_scatter([a, b], [4, 5])
+    with pytest.raises(ValueError):
+        lw.all_reduce([a, b], op="max")
+    with pytest.raises(ValueError):
+        lw.all_reduce([a, torch.zeros(8)])  # a CPU tensor: no CPU path
+    with pytest.raises(ValueError):
+        lw.all_reduce([a, b[::2]])
+    with pytest.raises(ValueError):
+        lw.all_reduce([a.long(), b.long()], op="avg")
+    # overlapping destination and source are refused by the launcher itself
+    pairs = (_lib.Pair * 1)()
+    pairs[0].dst, pairs[0].src, pairs[0].count = a.data_ptr(), a.data_ptr() + 8, 4
+    assert _lib.lib().tdm_k1_reduce_step(pairs, 1, 0, 2, 1, 1, 0, None) == 1
+    assert b"overlap" in _lib.lib().tdm_last_error()
+
+
+def test_full_size_properties(dev):
+    """BASELINE's largest case: four ranks x 64 Mi fp32 (256 MiB each). The
+    oracle is too slow for all of it, so: every rank ends with the same bits,
+    integer-valued inputs sum exactly, a power-of-two scaling of the inputs
+    scales the result exactly, and a strided sample is checked against the
+    oracle."""
+    from oracle import ring
+    from tandem_amd import LocalWorld
+
+    world, n = 4, 64 << 20
+    lw = LocalWorld(world)
+    gens = [torch.Generator(device=dev).manual_seed(10 + r) for r in range(world)]
+    xs = [torch.randn(n, device=dev, generator=g) * 1e-2 for g in gens]
+    bufs = [x.clone() for x in xs]
+    lw.all_reduce(bufs, op="avg")
+    for r in range(1, world):
+        assert torch.equal(bufs[0].view(torch.int32), bufs[r].view(torch.int32))
+    scaled = [x * 16.0 for x in xs]
+    lw.all_reduce(scaled, op="avg")
+    assert torch.equal((bufs[0] * 16.0).view(torch.int32), scaled[0].view(torch.int32))
+    # a sample of 1 Mi elements per chunk against the oracle
+    bounds = ring.chunk_bounds(n, world)
+    for c, (lo, hi) in enumerate(bounds):
+        sl = slice(lo + 12345, lo + 12345 + (1 << 20))
+        sample = [x[sl].cpu().numpy() for x in xs]
+        want = ring.fold(sample, c, 0, 1 << 20, True)
+        assert np.array_equal(bits(to_np(bufs[0][sl])), bits(want)), c
+    del scaled
+    ints = [torch.randint(-100, 100, (n,), device=dev, generator=g).float() for g in gens]
+    exact = sum(i.double() for i in ints)
+    lw.all_reduce(ints, op="sum")
+    assert torch.equal(ints[2].double(), exact)
