@@ -127,11 +127,18 @@ typedef struct tdm_adamw_scalars {
   float bc2_sqrt;    /* (1 - beta2**t) ** 0.5 */
   float eps;
   float neg_step;    /* -(lr / (1 - beta1**t)) */
+  float inv_bc2_sqrt; /* 1 / ((1 - beta2**t) ** 0.5), divided in double: TDM_ADAMW_DEVICE_ORDER only */
 } tdm_adamw_scalars;
 
 enum tdm_adamw_order {
-  TDM_ADAMW_HOST_ORDER = 0,  /* p + (neg_step*m)/d : torch's CPU addcdiv_, the reference's CPU engine */
-  TDM_ADAMW_DEVICE_ORDER = 1 /* fma(neg_step, m/d, p): torch's GPU addcdiv_ kernel */
+  /* torch's CPU kernels, i.e. the reference's CPU engine:
+   *   v = fma((1-beta2)*g, g, v*beta2);  p = p + (neg_step*m)/d */
+  TDM_ADAMW_HOST_ORDER = 0,
+  /* torch's GPU kernels: addcmul_/addcdiv_ compute a + value*(t1 op t2), contracted,
+   * and tensor / scalar multiplies by the scalar's reciprocal:
+   *   v = fma(1-beta2, g*g, v*beta2);  d = sqrt(v) * inv_bc2_sqrt + eps;
+   *   p = fma(neg_step, m/d, p) */
+  TDM_ADAMW_DEVICE_ORDER = 1
 };
 
 /* One fused AdamW step over a flat fp32 shard, in place (p, m, v); replaces the

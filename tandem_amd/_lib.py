@@ -38,7 +38,7 @@ class FoldSeg(ctypes.Structure):
 class AdamwScalars(ctypes.Structure):
     _fields_ = [("use_decay", ctypes.c_int32), ("decay", ctypes.c_float), ("w1", ctypes.c_float),
                 ("beta2", ctypes.c_float), ("one_m_b2", ctypes.c_float), ("bc2_sqrt", ctypes.c_float),
-                ("eps", ctypes.c_float), ("neg_step", ctypes.c_float)]
+                ("eps", ctypes.c_float), ("neg_step", ctypes.c_float), ("inv_bc2_sqrt", ctypes.c_float)]
 
 
 _SIGNATURES = {

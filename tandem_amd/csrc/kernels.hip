@@ -464,12 +464,17 @@ __device__ __forceinline__ void adamw_elem(float& p, float g, float& m, float& v
   // lerp_: weight < 0.5 ? fma(w, end-start, start) : fma(w-1, end-start, end)
   m = small_w ? __builtin_fmaf(s.w1, diff, m) : __builtin_fmaf(s.w1 - 1.0f, diff, g);
   const float vs = v * s.beta2;
-  v = __builtin_fmaf(s.one_m_b2 * g, g, vs);  // addcmul_: (value*g) rounded, then fused
-  const float d = __builtin_sqrtf(v) / s.bc2_sqrt + s.eps;
   if constexpr (kOrder == TDM_ADAMW_HOST_ORDER) {
-    p = p + (s.neg_step * m) / d;
+    v = __builtin_fmaf(s.one_m_b2 * g, g, vs);  // CPU addcmul_: (value*g) rounded, then fused
   } else {
-    p = __builtin_fmaf(s.neg_step, m / d, p);
+    v = __builtin_fmaf(s.one_m_b2, g * g, vs);  // GPU addcmul_: a + value * (g*g), contracted
+  }
+  if constexpr (kOrder == TDM_ADAMW_HOST_ORDER) {
+    const float d = __builtin_sqrtf(v) / s.bc2_sqrt + s.eps;
+    p = p + (s.neg_step * m) / d;  // CPU addcdiv_: (value*m)/d, then add; nothing fused
+  } else {
+    const float d = __builtin_sqrtf(v) * s.inv_bc2_sqrt + s.eps;  // GPU tensor / scalar: times the reciprocal
+    p = __builtin_fmaf(s.neg_step, m / d, p);  // GPU addcdiv_: a + value * (m/d), contracted
   }
 }
 

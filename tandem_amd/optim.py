@@ -30,6 +30,7 @@ def step_scalars(step, lr, betas, eps, weight_decay):
     s.bc2_sqrt = bias_correction2_sqrt
     s.eps = eps
     s.neg_step = -step_size
+    s.inv_bc2_sqrt = 1.0 / bias_correction2_sqrt  # torch's GPU `tensor / scalar` multiplies by this
     return s
 
 

@@ -34,7 +34,7 @@ def test_struct_layouts_match_the_header():
 
     assert ctypes.sizeof(_lib.Pair) == 24
     assert ctypes.sizeof(_lib.FoldSeg) == 8 * 8 * 2 + 16
-    assert ctypes.sizeof(_lib.AdamwScalars) == 32
+    assert ctypes.sizeof(_lib.AdamwScalars) == 36
 
 
 def test_argument_errors_need_no_gpu():
