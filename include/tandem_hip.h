@@ -158,6 +158,67 @@ int tdm_k3_adamw(float* p, const float* g, float* m, float* v, int64_t n, const 
 int tdm_k4_unit_gather(void* full, const void* const* shards, const int64_t* sizes, int world, int dtype,
                        tdm_stream stream);
 
+/* ---- the engine: Group(backend="hip") --------------------------------------- */
+
+/* One rank's half of a group whose ranks are processes sharing one GPU. Mirrors
+ * the object the reference's Group expects from its native plug-in
+ * (tandem/comm.py:149-160; constructor tandem/csrc/collectives.cpp:98-117; pybind
+ * surface tandem/csrc/engine.cpp:103-122): create on every rank, wait until all
+ * ranks have (the launcher's barrier), connect, then collectives. Tensors must be
+ * contiguous and in the engine's GPU memory; results are written in place; the
+ * caller keeps them alive until the Work has been waited for. */
+typedef struct tdm_engine tdm_engine;
+typedef struct tdm_work tdm_work;
+
+/* dtype code for tensors that are only copied (all_gather, broadcast, send/recv): raw bytes */
+enum { TDM_BYTES = 6 };
+
+/* Creates this rank's outgoing slots (`slots` x `slot_bytes` of device memory per
+ * peer, shared through hipIpcGetMemHandle), its interprocess events
+ * (hipIpcGetEventHandle) and its shared-memory region "/tandem-<job>-<rank>-hip",
+ * and starts the progress thread. Replaces Engine::Engine + CudaLinks::CudaLinks
+ * (tandem/csrc/collectives.cpp:98-117, tandem/csrc/cuda_links.cpp:43-84). */
+int tdm_engine_create(const char* job, int rank, int size, int slots, int64_t slot_bytes, double timeout_s, int device,
+                      tdm_engine** out);
+
+/* Opens what the other ranks created (Engine::connect, CudaLinks::connect:
+ * tandem/csrc/collectives.cpp:119-126, tandem/csrc/cuda_links.cpp:86-118). */
+int tdm_engine_connect(tdm_engine* e);
+
+/* Runs what is queued, stops the thread, waits for every rank, then releases
+ * handles, events and slots (tandem/csrc/collectives.cpp:132-149,
+ * tandem/csrc/cuda_links.cpp:162-179). tdm_engine_destroy frees the object. */
+int tdm_engine_close(tdm_engine* e);
+int tdm_engine_destroy(tdm_engine* e);
+
+/* The collectives. Each validates its arguments in the calling thread, records an
+ * event on `caller` (the stream that produced the tensor), queues the work for
+ * the progress thread and returns a Work at once. `average` divides by the group
+ * size before summing, in the ring's rank order; `sizes` (nsizes == 0: as even as
+ * torch.tensor_split) cuts the flat tensor into one chunk per rank. Replace
+ * Engine::all_reduce / reduce_scatter / all_gather / broadcast / send / recv /
+ * sendrecv / barrier (tandem/csrc/collectives.cpp:314-397; the Python engine's
+ * tandem/comm.py:326-460). tdm_sendrecv with dst < 0 is recv, with src < 0 send. */
+int tdm_all_reduce(tdm_engine* e, void* ptr, int64_t numel, int dtype, int average, tdm_stream caller, tdm_work** out);
+int tdm_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
+                       tdm_stream caller, tdm_work** out);
+int tdm_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, tdm_stream caller,
+                   tdm_work** out);
+int tdm_broadcast(tdm_engine* e, void* ptr, int64_t numel, int dtype, int root, tdm_stream caller, tdm_work** out);
+int tdm_sendrecv(tdm_engine* e, const void* send, int64_t send_numel, int dst, void* recv, int64_t recv_numel, int src,
+                 int dtype, tdm_stream caller, tdm_work** out);
+int tdm_barrier(tdm_engine* e, tdm_work** out);
+
+/* Work handle (tandem/csrc/collectives.h:43-66, tandem/csrc/engine.cpp:103-107).
+ * wait: blocks the host until the collective's GPU work has been enqueued, then
+ * makes `caller` wait for it on the GPU; returns the collective's error, if any.
+ * done: 1 once the GPU has finished it. times: when the progress thread started and
+ * finished it, seconds on CLOCK_MONOTONIC (Python's time.perf_counter clock). */
+int tdm_work_wait(tdm_work* w, tdm_stream caller);
+int tdm_work_done(tdm_work* w);
+int tdm_work_times(tdm_work* w, double* started, double* finished);
+int tdm_work_free(tdm_work* w);
+
 #ifdef __cplusplus
 }
 #endif

@@ -63,12 +63,33 @@ _SIGNATURES = {
 _lib = None
 
 
+_VP = ctypes.c_void_p
+_PVP = ctypes.POINTER(ctypes.c_void_p)
+_PI64 = ctypes.POINTER(ctypes.c_int64)
+_ENGINE_SIGNATURES = {
+    "tdm_engine_create": (ctypes.c_int, [ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
+                                         ctypes.c_double, ctypes.c_int, _PVP]),
+    "tdm_engine_connect": (ctypes.c_int, [_VP]),
+    "tdm_engine_close": (ctypes.c_int, [_VP]),
+    "tdm_engine_destroy": (ctypes.c_int, [_VP]),
+    "tdm_all_reduce": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _VP, _PVP]),
+    "tdm_reduce_scatter": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _PI64, ctypes.c_int, ctypes.c_int, _VP, _PVP]),
+    "tdm_all_gather": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _PI64, ctypes.c_int, _VP, _PVP]),
+    "tdm_broadcast": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _VP, _PVP]),
+    "tdm_sendrecv": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _VP, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                    _VP, _PVP]),
+    "tdm_barrier": (ctypes.c_int, [_VP, _PVP]),
+    "tdm_work_wait": (ctypes.c_int, [_VP, _VP]),
+    "tdm_work_done": (ctypes.c_int, [_VP]),
+    "tdm_work_times": (ctypes.c_int, [_VP, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
+    "tdm_work_free": (ctypes.c_int, [_VP]),
+}
+TDM_BYTES = 6
+
+
 def exported_symbols():
     """Every entry point include/tandem_hip.h declares."""
-    return sorted(_SIGNATURES) + sorted(_ENGINE_SIGNATURES)
-
-
-_ENGINE_SIGNATURES = {}
+    return sorted(list(_SIGNATURES) + list(_ENGINE_SIGNATURES))
 
 
 def lib():

@@ -1,0 +1,306 @@
+"""Collectives between processes that share one MI355X: tandem's `Group`,
+`Work`, `CommError` and `launch` with one backend, "hip".
+
+The class is a drop-in for the reference's plug-in point (tandem/comm.py:110-147
+there: `Group(rank, size, device, sync, queues, slot_bytes, slots, timeout,
+transport, priority, backend, job)`), so the DDP / ZeRO / FSDP wrappers and any
+`fn(group, *args)` written for tandem run unchanged with `backend="hip"`. All
+work happens in libtandem_hip.so: an engine per rank with its own progress
+thread and HIP stream, slots shared through HIP IPC memory handles, ordered by
+interprocess events. A collective returns a Work immediately; `wait()` makes the
+caller's current stream wait for it without blocking the host on the GPU.
+
+There is no CPU path and no Python engine here: any other backend, or a CPU
+device, raises CommError.
+"""
+
+import ctypes
+import os
+import time
+
+import torch
+import torch.multiprocessing as mp
+
+from . import _lib
+from ._lib import check, lib
+
+DEFAULT_SLOT_BYTES = 4 << 20
+DEFAULT_SLOTS = 2
+DEFAULT_TIMEOUT = float(os.environ.get("TANDEM_TIMEOUT", "600"))
+DEFAULT_BACKEND = os.environ.get("TANDEM_BACKEND", "hip")
+
+
+class CommError(RuntimeError):
+    pass
+
+
+class Work:
+    """A collective in flight on the engine's thread and stream."""
+
+    def __init__(self, name, group, handle, result, nbytes, keep):
+        self.name, self._group, self._handle, self.result, self._nbytes = name, group, handle, result, nbytes
+        self._keep = keep  # the tensors the engine reads and writes stay alive until waited for
+        self._recorded = False
+        self._waited = False
+
+    def wait(self):
+        g = self._group
+        if self._handle is None:
+            return self.result
+        t0 = time.perf_counter() if g.tracing and not self.is_completed() else None
+        try:
+            check(lib().tdm_work_wait(self._handle, _lib.stream_ptr(g.device)))
+        except Exception as e:
+            raise CommError(f"{self.name} failed") from e
+        if t0 is not None:
+            g.waits.append((self.name, t0, time.perf_counter()))
+        if g.tracing and not self._recorded:
+            a, b = ctypes.c_double(0), ctypes.c_double(0)
+            lib().tdm_work_times(self._handle, ctypes.byref(a), ctypes.byref(b))
+            g.trace.append((self.name, a.value, b.value, self._nbytes))  # steady clock == perf_counter's clock
+        self._recorded = True
+        self._waited = True
+        return self.result
+
+    def is_completed(self):
+        return self._handle is None or bool(lib().tdm_work_done(self._handle))
+
+    def __del__(self):
+        h, self._handle = getattr(self, "_handle", None), None
+        if h is not None:
+            try:
+                lib().tdm_work_free(h)
+            except Exception:
+                pass
+
+
+class Group:
+    """One rank's view of the group."""
+
+    def __init__(self, rank, size, device, sync, queues=None, slot_bytes=DEFAULT_SLOT_BYTES, slots=DEFAULT_SLOTS,
+                 timeout=DEFAULT_TIMEOUT, transport=None, priority=None, backend=None, job=None):
+        self.rank, self.size = rank, size
+        self.device = torch.device(device)
+        self.slot_bytes, self.slots, self.timeout = slot_bytes, slots, timeout
+        self.transport = transport or "device"
+        self.priority = 0  # every stream here runs at the default priority
+        self.backend = backend or DEFAULT_BACKEND
+        self.trace, self.waits, self.tracing = [], [], False
+        self._closed = False
+        self._engine = None
+        if self.backend != "hip":
+            raise CommError(f"unknown backend {self.backend} (tandem_amd provides \"hip\")")
+        if self.transport != "device":
+            raise CommError(f"unknown transport {self.transport} (ranks share one GPU's memory)")
+        if self.device.type != "cuda":
+            raise CommError("the hip backend needs device=\"cuda\": there is no CPU path")
+        if job is None:
+            raise CommError("the hip engine needs a job name (launch() makes one)")
+        self._barrier = sync[2] if isinstance(sync, (tuple, list)) else sync
+        index = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        self.device = torch.device("cuda", index)
+        handle = ctypes.c_void_p()
+        try:
+            check(lib().tdm_engine_create(job.encode(), rank, size, slots, slot_bytes, float(timeout), index,
+                                          ctypes.byref(handle)))
+            self._engine = handle
+            self._barrier.wait(timeout=timeout)  # every rank has published its slots and events
+            check(lib().tdm_engine_connect(self._engine))
+        except CommError:
+            raise
+        except Exception as e:
+            raise CommError(f"could not start the hip engine: {e}") from e
+        self.barrier()
+
+    # ---- plumbing
+    def _start(self, name, call, result, nbytes, async_op, keep=()):
+        if self._closed:
+            raise CommError("group is closed")
+        out = ctypes.c_void_p()
+        try:
+            check(call(ctypes.byref(out)))
+        except (ValueError, RuntimeError, TimeoutError) as e:
+            raise CommError(f"{name}: {e}") from e
+        work = Work(name, self, out, result, nbytes, keep)
+        return work if async_op else work.wait()
+
+    def _flat(self, t, what):
+        if not isinstance(t, torch.Tensor) or t.device != self.device:
+            raise CommError(f"{what}: the tensor is not on {self.device}")
+        if not t.is_contiguous():
+            raise CommError("collectives need contiguous tensors")
+        return t.reshape(-1)
+
+    def _sizes(self, flat, sizes):
+        if sizes is None:
+            return None, (ctypes.c_int64 * 1)(), 0
+        sizes = [int(s) for s in sizes]
+        if len(sizes) != self.size or sum(sizes) != flat.numel() or any(s < 0 for s in sizes):
+            raise CommError(f"chunk sizes {sizes} do not partition {flat.numel()} elements")
+        return sizes, (ctypes.c_int64 * len(sizes))(*sizes), len(sizes)
+
+    def _chunk_of_rank(self, flat, sizes):
+        if sizes is None:
+            return torch.tensor_split(flat, self.size)[self.rank]
+        lo = sum(sizes[:self.rank])
+        return flat[lo:lo + sizes[self.rank]]
+
+    @staticmethod
+    def _code(t, reduce):
+        code = _lib.DTYPES.get(t.dtype)
+        if code is None:
+            if reduce:
+                raise CommError(f"the hip backend cannot reduce {t.dtype}")
+            return _lib.TDM_BYTES
+        return code
+
+    @staticmethod
+    def _count(t, code):
+        return t.numel() * t.element_size() if code == _lib.TDM_BYTES else t.numel()
+
+    def _stream(self):
+        return _lib.stream_ptr(self.device)
+
+    # ---- collectives
+    def all_reduce(self, t, op="sum", async_op=False):
+        """Ring all-reduce in place: reduce-scatter, then all-gather."""
+        if op not in ("sum", "avg"):
+            raise CommError(f"unknown op {op}")
+        flat = self._flat(t, "all_reduce")
+        code = self._code(flat, True)
+        return self._start("all_reduce", lambda out: lib().tdm_all_reduce(
+            self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, int(op == "avg"), self._stream(), out),
+            t, t.numel() * t.element_size(), async_op, keep=(flat,))
+
+    def reduce_scatter(self, t, sizes=None, op="sum", async_op=False):
+        """Sums `t` across ranks, leaving rank r's chunk (chunk r of
+        torch.tensor_split, or of `sizes`) reduced in place; returns that view.
+        The other chunks hold partial sums afterwards."""
+        if op not in ("sum", "avg"):
+            raise CommError(f"unknown op {op}")
+        flat = self._flat(t, "reduce_scatter")
+        code = self._code(flat, True)
+        sizes, arr, n = self._sizes(flat, sizes)
+        mine = self._chunk_of_rank(flat, sizes)
+        return self._start("reduce_scatter", lambda out: lib().tdm_reduce_scatter(
+            self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, arr, n, int(op == "avg"), self._stream(), out),
+            mine, t.numel() * t.element_size(), async_op, keep=(flat,))
+
+    def all_gather(self, t, sizes=None, async_op=False):
+        """Each rank holds its own chunk of `t` (chunk r); fills in the rest."""
+        flat = self._flat(t, "all_gather")
+        code = self._code(flat, False)
+        sizes, arr, n = self._sizes(flat, sizes)
+        if code == _lib.TDM_BYTES and n:
+            arr = (ctypes.c_int64 * n)(*[s * flat.element_size() for s in sizes])
+        return self._start("all_gather", lambda out: lib().tdm_all_gather(
+            self._engine, ctypes.c_void_p(flat.data_ptr()), self._count(flat, code), code, arr, n, self._stream(), out),
+            t, t.numel() * t.element_size(), async_op, keep=(flat,))
+
+    def broadcast(self, t, root=0, async_op=False):
+        """Pipelined along the ring from root."""
+        flat = self._flat(t, "broadcast")
+        code = self._code(flat, False)
+        return self._start("broadcast", lambda out: lib().tdm_broadcast(
+            self._engine, ctypes.c_void_p(flat.data_ptr()), self._count(flat, code), code, root, self._stream(), out),
+            t, t.numel() * t.element_size(), async_op, keep=(flat,))
+
+    def send(self, t, dst, async_op=False):
+        flat = self._flat(t, "send")
+        code = self._code(flat, False)
+        return self._start(f"send->{dst}", lambda out: lib().tdm_sendrecv(
+            self._engine, ctypes.c_void_p(flat.data_ptr()), self._count(flat, code), dst, None, 0, -1, code, self._stream(), out),
+            t, t.numel() * t.element_size(), async_op, keep=(flat,))
+
+    def recv(self, t, src, async_op=False):
+        flat = self._flat(t, "recv")
+        code = self._code(flat, False)
+        return self._start(f"recv<-{src}", lambda out: lib().tdm_sendrecv(
+            self._engine, None, 0, -1, ctypes.c_void_p(flat.data_ptr()), self._count(flat, code), src, code, self._stream(), out),
+            t, t.numel() * t.element_size(), async_op, keep=(flat,))
+
+    def sendrecv(self, send, dst, recv, src, async_op=False):
+        """Sends one tensor while receiving another, piece by piece in lockstep."""
+        sf, rf = self._flat(send, "sendrecv"), self._flat(recv, "sendrecv")
+        if sf.dtype != rf.dtype:
+            raise CommError("sendrecv: the two tensors differ in dtype")
+        code = self._code(sf, False)
+        return self._start(f"sendrecv->{dst}<-{src}", lambda out: lib().tdm_sendrecv(
+            self._engine, ctypes.c_void_p(sf.data_ptr()), self._count(sf, code), dst, ctypes.c_void_p(rf.data_ptr()),
+            self._count(rf, code), src, code, self._stream(), out),
+            recv, (send.numel() + recv.numel()) * send.element_size(), async_op, keep=(sf, rf))
+
+    def barrier(self):
+        return self._start("barrier", lambda out: lib().tdm_barrier(self._engine, out), None, 0, False)
+
+    def close(self):
+        if self._closed:
+            return
+        self.barrier()
+        self._closed = True
+        eng, self._engine = self._engine, None
+        try:
+            check(lib().tdm_engine_close(eng))
+        except Exception as e:
+            raise CommError(f"close: {e}") from e
+        finally:
+            lib().tdm_engine_destroy(eng)
+
+    def abandon(self):
+        """After a failure on this rank: drop the engine without the closing
+        handshake (the other ranks time out or fail on their own)."""
+        self._closed = True
+        eng, self._engine = self._engine, None
+        if eng is not None:
+            lib().tdm_engine_destroy(eng)
+
+
+def _worker(rank, size, fn, args, barrier, device, slot_bytes, slots, backend, job, gpus, timeout, results):
+    if device != "cuda":
+        raise CommError("tandem_amd.launch runs ranks on the GPU only (device=\"cuda\")")
+    index = gpus[rank] if gpus else 0
+    torch.cuda.set_device(index)
+    g = Group(rank, size, torch.device("cuda", index), barrier, None, slot_bytes, slots, timeout=timeout, backend=backend,
+              job=job)
+    try:
+        out = fn(g, *args)
+        torch.cuda.synchronize(index)
+        g.close()
+    except BaseException:
+        try:
+            barrier.abort()  # ranks still starting up fail fast
+        except Exception:
+            pass
+        g.abandon()
+        raise
+    if out is not None:
+        torch.save(out, os.path.join(results, f"rank{rank}.pt"))
+
+
+def launch(fn, size, *args, device="cuda", slot_bytes=DEFAULT_SLOT_BYTES, slots=DEFAULT_SLOTS, transport=None,
+           priority=None, backend=None, gpus=None, timeout=DEFAULT_TIMEOUT):
+    """Runs fn(group, *args) on `size` processes and returns each rank's return
+    value, in rank order (tandem/comm.py:517-547 in the reference). The ranks
+    share GPU 0 unless `gpus` names a device per rank; this build is measured with
+    every rank on one GPU. Return values travel back through files, so keep them
+    small (CPU tensors, numbers, lists)."""
+    import tempfile
+    import uuid
+
+    backend = backend or DEFAULT_BACKEND
+    if backend != "hip":
+        raise CommError(f"unknown backend {backend} (tandem_amd provides \"hip\")")
+    if transport not in (None, "device"):
+        raise CommError(f"unknown transport {transport}")
+    lib()  # load (and fail) here, not in every rank at once
+    job = uuid.uuid4().hex[:12]
+    ctx = mp.get_context("spawn")
+    barrier = ctx.Barrier(size)
+    with tempfile.TemporaryDirectory(prefix="tandem-") as results:
+        mp.spawn(_worker, args=(size, fn, args, barrier, device, slot_bytes, slots, backend, job, gpus, timeout, results),
+                 nprocs=size, join=True)
+        out = []
+        for r in range(size):
+            path = os.path.join(results, f"rank{r}.pt")
+            out.append(torch.load(path, weights_only=False) if os.path.exists(path) else None)
+    return out

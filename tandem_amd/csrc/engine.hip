@@ -1,0 +1,887 @@
+// The engine behind Group(backend="hip"): one rank's half of a group whose ranks
+// are processes sharing one MI355X.
+//
+// Shape of the thing (what the reference's native plug-in also is,
+// tandem/csrc/collectives.h:43-126, tandem/csrc/cuda_links.h:1-22): an Engine per
+// rank, a progress thread that runs queued collectives in submission order and
+// never touches Python, Work handles, and per ordered pair of ranks a ring of
+// `slots` device buffers that the sender owns and the receiver maps through HIP
+// IPC. What differs is what moves through it:
+//   * a put is one launch of the copy kernel into the sender's slot (dividing by
+//     the world size on the way when the collective averages), a take is one
+//     launch of the fused ring-step kernel that reads the peer's slot in place;
+//   * the host never waits for the GPU per piece: slot hand-over is ordered by
+//     interprocess events (full[j] / free[j]) opened from hipIpcEventHandle_t, and
+//     an 8-byte message per piece in a shared-memory ring says which slot and how
+//     long (TANDEM_HIP_SYNC=host replaces the events with stream synchronisation
+//     before each message, for debugging);
+//   * every rank publishes its handles in one POSIX shared-memory region,
+//     "/tandem-<job>-<rank>-hip", which also holds the message rings it sends on.
+//
+// Streams: a collective starts on the engine's stream once the caller's stream
+// has reached the point of submission (an event), and tdm_work_wait makes the
+// caller's stream wait for the collective's last kernel; the host is not blocked
+// on GPU work in either direction (tandem/csrc/collectives.cpp:159-224).
+
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <chrono>
+#include <condition_variable>
+#include <cstdlib>
+#include <cstring>
+#include <deque>
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <new>
+#include <thread>
+#include <vector>
+
+#include "common.h"
+
+namespace tandem_hip {
+
+namespace {
+
+double now_s() {
+  return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+int mod(int a, int n) { return ((a % n) + n) % n; }
+
+constexpr int kBytesDtype = 6;  // TDM_U8 in spirit: copies only
+
+int elem_bytes(int dtype) {
+  switch (dtype) {
+    case TDM_F32: case TDM_I32: return 4;
+    case TDM_F64: case TDM_I64: return 8;
+    case TDM_F16: case TDM_BF16: return 2;
+    case kBytesDtype: return 1;
+    default: throw Invalid("unknown dtype " + std::to_string(dtype));
+  }
+}
+
+// ---------------------------------------------------------------- shared region
+constexpr uint64_t kRegionMagic = 0x74646d4849503031ull;  // "tdmHIP01"
+constexpr size_t kLine = 64;
+constexpr int kMaxSlots = 16;
+
+static_assert(std::atomic<uint64_t>::is_always_lock_free, "atomics shared between processes must be lock-free");
+
+// One direction of one pair, written by the owner of the region (the sender):
+// message k says slot k % slots holds `length[k % slots]` bytes.
+struct alignas(kLine) Ring {
+  alignas(kLine) std::atomic<uint64_t> head;  // messages published, advanced by the sender
+  alignas(kLine) std::atomic<uint64_t> tail;  // messages released, advanced by the receiver
+  alignas(kLine) uint64_t length[kMaxSlots];
+};
+
+struct alignas(kLine) PeerEntry {
+  hipIpcMemHandle_t mem;               // the sender's slots for this peer
+  hipIpcEventHandle_t full[kMaxSlots];  // sender recorded: slot j holds a piece
+  hipIpcEventHandle_t free_[kMaxSlots]; // owner recorded: it finished reading THE PEER's slot j to the owner
+  Ring ring;
+};
+
+struct alignas(kLine) RegionHeader {
+  uint64_t magic;
+  int32_t rank, size, device, slots;
+  uint64_t slot_bytes;
+  int64_t pid;
+  int32_t use_events;
+  int32_t reserved;
+};
+
+class Region {
+ public:
+  Region() = default;
+  ~Region() { reset(); }
+  Region(const Region&) = delete;
+  Region& operator=(const Region&) = delete;
+
+  static size_t bytes_for(int size) { return sizeof(RegionHeader) + static_cast<size_t>(size) * sizeof(PeerEntry); }
+
+  void create(const std::string& name, int size) {
+    reset();
+    name_ = name;
+    bytes_ = bytes_for(size);
+    ::shm_unlink(name.c_str());  // a stale region from a crashed run with the same job name
+    int fd = ::shm_open(name.c_str(), O_CREAT | O_EXCL | O_RDWR, 0600);
+    if (fd < 0) throw std::runtime_error("shm_open(" + name + "): " + std::strerror(errno));
+    if (::ftruncate(fd, static_cast<off_t>(bytes_)) != 0) {
+      ::close(fd);
+      ::shm_unlink(name.c_str());
+      throw std::runtime_error("ftruncate(" + name + "): " + std::strerror(errno));
+    }
+    map(fd);
+    owner_ = true;
+    std::memset(data_, 0, bytes_);
+    for (int p = 0; p < size; ++p) new (&entry(p)->ring) Ring();
+  }
+
+  void open(const std::string& name, int size) {
+    reset();
+    name_ = name;
+    bytes_ = bytes_for(size);
+    int fd = ::shm_open(name.c_str(), O_RDWR, 0600);
+    if (fd < 0) throw std::runtime_error("shm_open(" + name + "): " + std::strerror(errno));
+    struct stat st;
+    if (::fstat(fd, &st) != 0 || static_cast<size_t>(st.st_size) < bytes_) {
+      ::close(fd);
+      throw std::runtime_error("region " + name + " is smaller than expected");
+    }
+    map(fd);
+  }
+
+  RegionHeader* header() const { return static_cast<RegionHeader*>(data_); }
+  PeerEntry* entry(int peer) const {
+    return reinterpret_cast<PeerEntry*>(static_cast<char*>(data_) + sizeof(RegionHeader)) + peer;
+  }
+  bool mapped() const { return data_ != nullptr; }
+
+  void reset() {
+    if (data_) ::munmap(data_, bytes_);
+    if (owner_) ::shm_unlink(name_.c_str());
+    data_ = nullptr;
+    owner_ = false;
+  }
+
+ private:
+  void map(int fd) {
+    void* p = ::mmap(nullptr, bytes_, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+    ::close(fd);
+    if (p == MAP_FAILED) throw std::runtime_error("mmap(" + name_ + "): " + std::strerror(errno));
+    data_ = p;
+  }
+
+  std::string name_;
+  void* data_ = nullptr;
+  size_t bytes_ = 0;
+  bool owner_ = false;
+};
+
+// Spin, then yield, then short sleeps; throws Timeout.
+template <class Ready>
+void wait_until(Ready ready, double timeout_s, const char* what) {
+  using clock = std::chrono::steady_clock;
+  const auto start = clock::now();
+  const auto deadline = start + std::chrono::duration<double>(timeout_s);
+  for (uint64_t i = 0; !ready(); ++i) {
+    if (i < 256) continue;
+    if ((i & 63) != 0) {
+      std::this_thread::yield();
+      continue;
+    }
+    const auto t = clock::now();
+    if (t > deadline) throw Timeout(what);
+    if (t - start > std::chrono::milliseconds(2)) std::this_thread::sleep_for(std::chrono::microseconds(20));
+  }
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------- Work
+struct Work {
+  std::mutex mu;
+  std::condition_variable cv;
+  bool finished = false;   // the job has run (all its GPU work is enqueued)
+  int status = TDM_OK;
+  std::string error;
+  double t0 = 0, t1 = 0;
+  hipEvent_t done_event = nullptr;  // recorded on the engine's stream after the job
+  int device = -1;
+
+  ~Work() {
+    if (done_event) (void)hipEventDestroy(done_event);
+  }
+};
+
+// ---------------------------------------------------------------- Engine
+class Engine {
+ public:
+  Engine(const std::string& job, int rank, int size, int slots, size_t slot_bytes, double timeout_s, int device);
+  ~Engine();
+  void connect();
+  void close();
+
+  struct Buf {
+    char* ptr;
+    int64_t numel;
+    int dtype;
+  };
+
+  std::shared_ptr<Work> all_reduce(Buf t, bool average, hipStream_t caller);
+  std::shared_ptr<Work> reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, hipStream_t caller);
+  std::shared_ptr<Work> all_gather(Buf t, std::vector<int64_t> sizes, hipStream_t caller);
+  std::shared_ptr<Work> broadcast(Buf t, int root, hipStream_t caller);
+  std::shared_ptr<Work> sendrecv(Buf send, int dst, Buf recv, int src, hipStream_t caller);
+  std::shared_ptr<Work> barrier();
+
+  int device() const { return device_; }
+  hipStream_t stream() const { return stream_; }
+  int rank() const { return rank_; }
+  int size() const { return size_; }
+
+ private:
+  struct Chunk {
+    char* ptr;
+    int64_t numel;
+  };
+
+  std::shared_ptr<Work> submit(std::function<void()> job, hipStream_t caller, bool uses_gpu);
+  void loop();
+  void check(const Buf& t, const char* what, bool reduce) const;
+  std::vector<Chunk> chunks(const Buf& t, const std::vector<int64_t>& sizes) const;
+  int64_t piece_elems(int dtype) const { return std::max<int64_t>(1, static_cast<int64_t>(slot_bytes_) / elem_bytes(dtype)); }
+
+  void put(int dst, const char* src, int64_t numel, int dtype, int scale_world);
+  void take(int src, char* into, int64_t numel, int dtype, bool reduce, int scale_world);
+  void exchange(const Chunk* send, int dst, const Chunk* recv, int src, int dtype, bool reduce, int put_scale,
+                int take_scale);
+  void ring_reduce_scatter(const std::vector<Chunk>& c, int dtype, bool average, bool keep_sent);
+  void ring_all_gather(const std::vector<Chunk>& c, int dtype);
+  void signal(int dst, uint64_t length);
+  uint64_t await(int src);
+  void release(int src);
+  void barrier_now();
+
+  std::string region_name(int rank) const { return "/tandem-" + job_ + "-" + std::to_string(rank) + "-hip"; }
+
+  std::string job_;
+  int rank_, size_, slots_;
+  size_t slot_bytes_;
+  double timeout_s_;
+  int device_;
+  bool use_events_;
+  hipStream_t stream_ = nullptr;
+  Region mine_;
+  std::vector<std::unique_ptr<Region>> theirs_;
+  std::vector<void*> out_mem_, peer_mem_;
+  std::vector<std::vector<hipEvent_t>> full_, free_, peer_full_, peer_free_;
+  std::vector<uint64_t> sent_, got_;
+  bool connected_ = false, closed_ = false;
+
+  std::mutex mu_;
+  std::condition_variable cv_;
+  std::deque<std::pair<std::function<void()>, std::shared_ptr<Work>>> jobs_;
+  bool stopping_ = false;
+  std::thread thread_;
+};
+
+Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slot_bytes, double timeout_s, int device)
+    : job_(job), rank_(rank), size_(size), slots_(slots), slot_bytes_(slot_bytes), timeout_s_(timeout_s),
+      device_(device), theirs_(size), out_mem_(size, nullptr), peer_mem_(size, nullptr), full_(size), free_(size),
+      peer_full_(size), peer_free_(size), sent_(size, 0), got_(size, 0) {
+  if (size < 1 || rank < 0 || rank >= size) throw Invalid("rank must be in [0, size)");
+  if (slots < 1 || slots > kMaxSlots) throw Invalid("slots must be in [1, " + std::to_string(kMaxSlots) + "]");
+  if (slot_bytes < 16 || slot_bytes % 16) throw Invalid("slot_bytes must be a positive multiple of 16");
+  if (slot_bytes * static_cast<size_t>(slots) >= (size_t(2) << 30)) {
+    throw Invalid("slots * slot_bytes must stay under 2 GiB per pair (one IPC allocation)");
+  }
+  if (device < 0) throw Invalid("the hip engine needs a GPU: device must be >= 0 (there is no CPU path)");
+  if (job.empty() || job.size() > 64) throw Invalid("job name must have 1..64 characters");
+  const char* mode = std::getenv("TANDEM_HIP_SYNC");
+  use_events_ = !(mode && std::string(mode) == "host");
+
+  check_hip(hipSetDevice(device_), "hipSetDevice");
+  check_hip(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags");  // default priority
+
+  mine_.create(region_name(rank_), size_);
+  RegionHeader* h = mine_.header();
+  h->rank = rank_;
+  h->size = size_;
+  h->device = device_;
+  h->slots = slots_;
+  h->slot_bytes = slot_bytes_;
+  h->pid = static_cast<int64_t>(::getpid());
+  h->use_events = use_events_;
+  constexpr unsigned kFlags = hipEventDisableTiming | hipEventInterprocess;
+  for (int p = 0; p < size_; ++p) {
+    if (p == rank_) continue;
+    PeerEntry* e = mine_.entry(p);
+    check_hip(hipMalloc(&out_mem_[p], static_cast<size_t>(slots_) * slot_bytes_), "hipMalloc (slots)");
+    check_hip(hipIpcGetMemHandle(&e->mem, out_mem_[p]), "hipIpcGetMemHandle");
+    if (use_events_) {
+      full_[p].resize(slots_);
+      free_[p].resize(slots_);
+      for (int j = 0; j < slots_; ++j) {
+        check_hip(hipEventCreateWithFlags(&full_[p][j], kFlags), "hipEventCreateWithFlags (full)");
+        check_hip(hipIpcGetEventHandle(&e->full[j], full_[p][j]), "hipIpcGetEventHandle (full)");
+        check_hip(hipEventCreateWithFlags(&free_[p][j], kFlags), "hipEventCreateWithFlags (free)");
+        check_hip(hipIpcGetEventHandle(&e->free_[j], free_[p][j]), "hipIpcGetEventHandle (free)");
+      }
+    }
+  }
+  std::atomic_thread_fence(std::memory_order_release);
+  h->magic = kRegionMagic;  // published last
+  thread_ = std::thread([this] { loop(); });
+}
+
+void Engine::connect() {
+  if (connected_) return;
+  check_hip(hipSetDevice(device_), "hipSetDevice");
+  for (int p = 0; p < size_; ++p) {
+    if (p == rank_) continue;
+    theirs_[p] = std::make_unique<Region>();
+    theirs_[p]->open(region_name(p), size_);
+    const RegionHeader* h = theirs_[p]->header();
+    if (h->magic != kRegionMagic || h->size != size_ || h->slots != slots_ || h->slot_bytes != slot_bytes_ ||
+        h->rank != p || h->use_events != static_cast<int32_t>(use_events_)) {
+      throw std::runtime_error("rank " + std::to_string(p) + "'s region does not match ours (size, slots, slot_bytes or sync mode)");
+    }
+    if (h->pid == static_cast<int64_t>(::getpid())) {
+      throw std::runtime_error("two ranks of one group in one process: HIP IPC handles cannot be opened by their exporter");
+    }
+    // In p's region, the entry for us: p's slots for sending to us, their full
+    // events, and the free events p records after reading OUR slots.
+    PeerEntry* e = theirs_[p]->entry(rank_);
+    check_hip(hipIpcOpenMemHandle(&peer_mem_[p], e->mem, hipIpcMemLazyEnablePeerAccess), "hipIpcOpenMemHandle");
+    if (use_events_) {
+      peer_full_[p].resize(slots_);
+      peer_free_[p].resize(slots_);
+      for (int j = 0; j < slots_; ++j) {
+        check_hip(hipIpcOpenEventHandle(&peer_full_[p][j], e->full[j]), "hipIpcOpenEventHandle (full)");
+        check_hip(hipIpcOpenEventHandle(&peer_free_[p][j], e->free_[j]), "hipIpcOpenEventHandle (free)");
+      }
+    }
+  }
+  connected_ = true;
+}
+
+void Engine::close() {
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    if (stopping_) return;
+    stopping_ = true;
+  }
+  cv_.notify_all();
+  if (thread_.joinable()) thread_.join();  // runs what was queued first
+  if (closed_) return;
+  closed_ = true;
+  (void)hipSetDevice(device_);
+  // Our GPU work must finish, and every peer's (they read our slots), before any
+  // rank frees its slots and events.
+  hipError_t sync_err = hipStreamSynchronize(stream_);
+  std::string barrier_err;
+  if (connected_) {
+    try {
+      barrier_now();
+    } catch (const std::exception& e) {
+      barrier_err = e.what();
+    }
+  }
+  for (int p = 0; p < size_; ++p) {
+    if (p == rank_) continue;
+    if (peer_mem_[p]) (void)hipIpcCloseMemHandle(peer_mem_[p]);
+    for (hipEvent_t e : peer_full_[p]) (void)hipEventDestroy(e);
+    for (hipEvent_t e : peer_free_[p]) (void)hipEventDestroy(e);
+    for (hipEvent_t e : full_[p]) (void)hipEventDestroy(e);
+    for (hipEvent_t e : free_[p]) (void)hipEventDestroy(e);
+    if (out_mem_[p]) (void)hipFree(out_mem_[p]);
+    peer_mem_[p] = out_mem_[p] = nullptr;
+    peer_full_[p].clear(); peer_free_[p].clear(); full_[p].clear(); free_[p].clear();
+    theirs_[p].reset();
+  }
+  if (stream_) (void)hipStreamDestroy(stream_);
+  stream_ = nullptr;
+  mine_.reset();
+  check_hip(sync_err, "hipStreamSynchronize (close)");
+  if (!barrier_err.empty()) throw std::runtime_error("close: " + barrier_err);
+}
+
+Engine::~Engine() {
+  try {
+    close();
+  } catch (...) {  // a destructor must not throw; call close() to see errors
+  }
+}
+
+// ---------------------------------------------------------------- progress thread
+std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t caller, bool uses_gpu) {
+  auto work = std::make_shared<Work>();
+  work->device = device_;
+  if (uses_gpu) {
+    // Start once the caller's stream has produced the inputs.
+    hipEvent_t ready;
+    check_hip(hipEventCreateWithFlags(&ready, hipEventDisableTiming), "hipEventCreateWithFlags (ready)");
+    hipError_t err = hipEventRecord(ready, caller);
+    if (err != hipSuccess) {
+      (void)hipEventDestroy(ready);
+      check_hip(err, "hipEventRecord (ready)");
+    }
+    job = [this, ready, inner = std::move(job)] {
+      hipError_t e = hipStreamWaitEvent(stream_, ready, 0);
+      (void)hipEventDestroy(ready);  // released once the GPU is past it
+      check_hip(e, "hipStreamWaitEvent (ready)");
+      inner();
+    };
+  }
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    if (stopping_) throw std::runtime_error("the engine is closed");
+    jobs_.emplace_back(std::move(job), work);
+  }
+  cv_.notify_one();
+  return work;
+}
+
+void Engine::loop() {
+  (void)hipSetDevice(device_);
+  for (;;) {
+    std::pair<std::function<void()>, std::shared_ptr<Work>> next;
+    {
+      std::unique_lock<std::mutex> lock(mu_);
+      cv_.wait(lock, [this] { return stopping_ || !jobs_.empty(); });
+      if (jobs_.empty()) return;  // stopping, and everything queued has run
+      next = std::move(jobs_.front());
+      jobs_.pop_front();
+    }
+    Work& w = *next.second;
+    int status = TDM_OK;
+    std::string error;
+    const double t0 = now_s();
+    try {
+      next.first();
+    } catch (const Invalid& e) {
+      status = TDM_EINVAL; error = e.what();
+    } catch (const Timeout& e) {
+      status = TDM_ETIMEOUT; error = e.what();
+    } catch (const std::exception& e) {
+      status = TDM_ERUNTIME; error = e.what();
+    } catch (...) {
+      status = TDM_ERUNTIME; error = "unknown error";
+    }
+    if (status == TDM_OK) {
+      if (hipEventCreateWithFlags(&w.done_event, hipEventDisableTiming) != hipSuccess ||
+          hipEventRecord(w.done_event, stream_) != hipSuccess) {
+        status = TDM_ERUNTIME;
+        error = "could not record the collective's completion event";
+      }
+    }
+    {
+      std::lock_guard<std::mutex> lock(w.mu);
+      w.status = status;
+      w.error = std::move(error);
+      w.t0 = t0;
+      w.t1 = now_s();
+      w.finished = true;
+    }
+    w.cv.notify_all();
+  }
+}
+
+// ---------------------------------------------------------------- messages
+void Engine::signal(int dst, uint64_t length) {
+  Ring& r = mine_.entry(dst)->ring;
+  const uint64_t head = r.head.load(std::memory_order_relaxed);
+  r.length[head % slots_] = length;
+  r.head.store(head + 1, std::memory_order_release);  // the length is visible before the new head
+}
+
+uint64_t Engine::await(int src) {
+  Ring& r = theirs_[src]->entry(rank_)->ring;
+  const uint64_t tail = r.tail.load(std::memory_order_relaxed);
+  wait_until([&] { return r.head.load(std::memory_order_acquire) > tail; }, timeout_s_,
+             "timed out waiting for a message from a peer rank");
+  return r.length[tail % slots_];
+}
+
+void Engine::release(int src) {
+  Ring& r = theirs_[src]->entry(rank_)->ring;
+  r.tail.store(r.tail.load(std::memory_order_relaxed) + 1, std::memory_order_release);
+}
+
+void Engine::barrier_now() {
+  // An empty message to every peer, then one from each. Rings are first in,
+  // first out, so this also orders the barrier after every piece queued before.
+  constexpr uint64_t kEmpty = ~uint64_t(0);
+  for (int p = 0; p < size_; ++p) {
+    if (p == rank_) continue;
+    Ring& r = mine_.entry(p)->ring;
+    const uint64_t head = r.head.load(std::memory_order_relaxed);
+    wait_until([&] { return head - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots_); },
+               timeout_s_, "barrier: a peer rank never drained its messages");
+    signal(p, kEmpty);
+  }
+  for (int p = 0; p < size_; ++p) {
+    if (p == rank_) continue;
+    if (await(p) != kEmpty) throw std::runtime_error("barrier out of step: expected an empty message, got a piece");
+    release(p);
+  }
+}
+
+// ---------------------------------------------------------------- pieces
+void Engine::put(int dst, const char* src, int64_t numel, int dtype, int scale_world) {
+  const size_t nbytes = static_cast<size_t>(numel) * elem_bytes(dtype);
+  if (nbytes > slot_bytes_) throw Invalid("piece larger than a slot");
+  const uint64_t k = sent_[dst];  // pieces so far: picks the slot
+  const int j = static_cast<int>(k % slots_);
+  Ring& r = mine_.entry(dst)->ring;
+  // Room in the message ring means fewer than `slots` messages are unreleased, so
+  // fewer than `slots` pieces are: dst has released slot j's previous piece ...
+  const uint64_t head = r.head.load(std::memory_order_relaxed);
+  wait_until([&] { return head - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots_); }, timeout_s_,
+             "put: the peer never freed a slot");
+  if (use_events_ && k >= static_cast<uint64_t>(slots_)) {
+    // ... and enqueued its reads of it before recording free[j]: wait for those reads.
+    check_hip(hipStreamWaitEvent(stream_, peer_free_[dst][j], 0), "hipStreamWaitEvent (free)");
+  }
+  char* slot = static_cast<char*>(out_mem_[dst]) + static_cast<size_t>(j) * slot_bytes_;
+  if (dtype == kBytesDtype) {
+    check_hip(hipMemcpyAsync(slot, src, nbytes, hipMemcpyDeviceToDevice, stream_), "hipMemcpyAsync (put)");
+  } else {
+    tdm_pair pr{slot, src, numel};
+    copy_step(&pr, 1, dtype, scale_world, stream_);
+  }
+  if (use_events_) {
+    check_hip(hipEventRecord(full_[dst][j], stream_), "hipEventRecord (full)");
+  } else {
+    check_hip(hipStreamSynchronize(stream_), "hipStreamSynchronize (put)");
+  }
+  signal(dst, nbytes);
+  sent_[dst] = k + 1;
+}
+
+void Engine::take(int src, char* into, int64_t numel, int dtype, bool reduce, int scale_world) {
+  const size_t nbytes = static_cast<size_t>(numel) * elem_bytes(dtype);
+  const uint64_t length = await(src);
+  if (length != nbytes) {
+    throw std::runtime_error(length == ~uint64_t(0) ? "collectives out of step: expected a piece, got a barrier"
+                                                    : "a piece arrived with the wrong length");
+  }
+  const int j = static_cast<int>(got_[src] % slots_);
+  if (use_events_) check_hip(hipStreamWaitEvent(stream_, peer_full_[src][j], 0), "hipStreamWaitEvent (full)");
+  const char* slot = static_cast<const char*>(peer_mem_[src]) + static_cast<size_t>(j) * slot_bytes_;
+  if (reduce) {
+    // The kernel reads the peer's slot in place. The slot already holds x / world
+    // when averaging; our own chunk is divided here, as part of the add.
+    tdm_pair pr{into, slot, numel};
+    reduce_step(&pr, 1, dtype, scale_world, scale_world > 1, false, false, stream_);
+  } else if (dtype == kBytesDtype) {
+    check_hip(hipMemcpyAsync(into, slot, nbytes, hipMemcpyDeviceToDevice, stream_), "hipMemcpyAsync (take)");
+  } else {
+    tdm_pair pr{into, slot, numel};
+    copy_step(&pr, 1, dtype, 0, stream_);
+  }
+  if (use_events_) {
+    check_hip(hipEventRecord(free_[src][j], stream_), "hipEventRecord (free)");
+  } else {
+    check_hip(hipStreamSynchronize(stream_), "hipStreamSynchronize (take)");
+  }
+  got_[src] += 1;
+  release(src);
+}
+
+// Sends `send` to dst while receiving `recv` from src, one piece of each at a
+// time, so a ring of ranks all sending at once never waits on itself.
+void Engine::exchange(const Chunk* send, int dst, const Chunk* recv, int src, int dtype, bool reduce, int put_scale,
+                      int take_scale) {
+  const int64_t pe = piece_elems(dtype);
+  const int es = elem_bytes(dtype);
+  const int64_t ns = send ? (send->numel + pe - 1) / pe : 0;
+  const int64_t nr = recv ? (recv->numel + pe - 1) / pe : 0;
+  for (int64_t k = 0; k < std::max(ns, nr); ++k) {
+    if (k < ns) put(dst, send->ptr + k * pe * es, std::min(pe, send->numel - k * pe), dtype, put_scale);
+    if (k < nr) take(src, recv->ptr + k * pe * es, std::min(pe, recv->numel - k * pe), dtype, reduce, take_scale);
+  }
+}
+
+// Step s: send chunk (r-s-1) to r+1, add chunk (r-s-2) from r-1 (tandem/comm.py:301-305).
+// Averaging is fused: the chunk sent on the first step leaves as x / n (and, for a
+// bare reduce_scatter, is divided in place first, because the reference's div_ of
+// the whole tensor is observable there); every receiving chunk is divided as part
+// of its add; later steps send partial sums, already divided.
+void Engine::ring_reduce_scatter(const std::vector<Chunk>& c, int dtype, bool average, bool keep_sent) {
+  const int n = size_, r = rank_;
+  const int w = average ? n : 0;
+  for (int s = 0; s < n - 1; ++s) {
+    const Chunk& out = c[mod(r - s - 1, n)];
+    int put_scale = 0;
+    if (s == 0 && w > 1) {
+      if (keep_sent && out.numel > 0) {
+        tdm_pair pr{out.ptr, out.ptr, out.numel};
+        copy_step(&pr, 1, dtype, w, stream_);  // in place: x / n
+      } else {
+        put_scale = w;
+      }
+    }
+    exchange(&out, mod(r + 1, n), &c[mod(r - s - 2, n)], mod(r - 1, n), dtype, true, put_scale, w);
+  }
+}
+
+void Engine::ring_all_gather(const std::vector<Chunk>& c, int dtype) {
+  const int n = size_, r = rank_;
+  for (int s = 0; s < n - 1; ++s) {
+    exchange(&c[mod(r - s, n)], mod(r + 1, n), &c[mod(r - s - 1, n)], mod(r - 1, n), dtype, false, 0, 0);
+  }
+}
+
+// ---------------------------------------------------------------- collectives
+void Engine::check(const Buf& t, const char* what, bool reduce) const {
+  if (t.numel < 0) throw Invalid(std::string(what) + ": negative element count");
+  if (t.numel > 0 && t.ptr == nullptr) throw Invalid(std::string(what) + ": NULL tensor");
+  const int es = elem_bytes(t.dtype);
+  if (reinterpret_cast<uintptr_t>(t.ptr) % es) throw Invalid(std::string(what) + ": pointer not aligned to the element size");
+  if (reduce && t.dtype == kBytesDtype) throw Invalid(std::string(what) + ": this dtype can be copied but not reduced");
+  if (!connected_) throw std::runtime_error(std::string(what) + ": the engine is not connected");
+  if (t.numel > 0) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, t.ptr) != hipSuccess || attr.type != hipMemoryTypeDevice || attr.device != device_) {
+      (void)hipGetLastError();
+      throw Invalid(std::string(what) + ": the tensor is not in the engine's GPU memory");
+    }
+  }
+}
+
+std::vector<Engine::Chunk> Engine::chunks(const Buf& t, const std::vector<int64_t>& sizes) const {
+  std::vector<Chunk> out(size_);
+  const int es = elem_bytes(t.dtype);
+  if (sizes.empty()) {  // as even as possible, as torch.tensor_split cuts
+    const int64_t base = t.numel / size_, extra = t.numel % size_;
+    int64_t lo = 0;
+    for (int q = 0; q < size_; ++q) {
+      const int64_t n = base + (q < extra ? 1 : 0);
+      out[q] = Chunk{t.ptr + lo * es, n};
+      lo += n;
+    }
+    return out;
+  }
+  int64_t total = 0;
+  for (int64_t s : sizes) {
+    if (s < 0) throw Invalid("chunk sizes do not partition the tensor");
+    total += s;
+  }
+  if (static_cast<int>(sizes.size()) != size_ || total != t.numel) throw Invalid("chunk sizes do not partition the tensor");
+  int64_t lo = 0;
+  for (int q = 0; q < size_; ++q) {
+    out[q] = Chunk{t.ptr + lo * es, sizes[q]};
+    lo += sizes[q];
+  }
+  return out;
+}
+
+std::shared_ptr<Work> Engine::all_reduce(Buf t, bool average, hipStream_t caller) {
+  check(t, "all_reduce", true);
+  if (average && (t.dtype == TDM_I64 || t.dtype == TDM_I32)) throw Invalid("all_reduce: integer tensors cannot be averaged in place");
+  return submit([this, t, average] {
+    if (size_ > 1) {
+      auto c = chunks(t, {});
+      ring_reduce_scatter(c, t.dtype, average, false);
+      ring_all_gather(c, t.dtype);
+    }
+  }, caller, true);
+}
+
+std::shared_ptr<Work> Engine::reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, hipStream_t caller) {
+  check(t, "reduce_scatter", true);
+  if (average && (t.dtype == TDM_I64 || t.dtype == TDM_I32)) throw Invalid("reduce_scatter: integer tensors cannot be averaged in place");
+  chunks(t, sizes);  // validate now, in the caller's thread
+  return submit([this, t, sizes, average] {
+    if (size_ > 1) ring_reduce_scatter(chunks(t, sizes), t.dtype, average, true);
+  }, caller, true);
+}
+
+std::shared_ptr<Work> Engine::all_gather(Buf t, std::vector<int64_t> sizes, hipStream_t caller) {
+  check(t, "all_gather", false);
+  chunks(t, sizes);
+  return submit([this, t, sizes] {
+    if (size_ > 1) ring_all_gather(chunks(t, sizes), t.dtype);
+  }, caller, true);
+}
+
+// Pipelined along the ring from the root: each rank forwards each piece as soon
+// as it has it (tandem/comm.py:387-409).
+std::shared_ptr<Work> Engine::broadcast(Buf t, int root, hipStream_t caller) {
+  check(t, "broadcast", false);
+  if (root < 0 || root >= size_) throw Invalid("broadcast: root outside [0, size)");
+  return submit([this, t, root] {
+    const int n = size_, pos = mod(rank_ - root, n);
+    const int nxt = mod(rank_ + 1, n), prv = mod(rank_ - 1, n);
+    const int64_t pe = piece_elems(t.dtype);
+    const int es = elem_bytes(t.dtype);
+    for (int64_t k = 0; k * pe < t.numel; ++k) {
+      char* piece = t.ptr + k * pe * es;
+      const int64_t m = std::min(pe, t.numel - k * pe);
+      if (pos > 0) take(prv, piece, m, t.dtype, false, 0);
+      if (pos < n - 1) put(nxt, piece, m, t.dtype, 0);
+    }
+  }, caller, true);
+}
+
+std::shared_ptr<Work> Engine::sendrecv(Buf send, int dst, Buf recv, int src, hipStream_t caller) {
+  const bool has_send = dst >= 0, has_recv = src >= 0;
+  if (has_send) check(send, "send", false);
+  if (has_recv) check(recv, "recv", false);
+  if (has_send && (dst >= size_ || dst == rank_)) throw Invalid("send: bad destination rank");
+  if (has_recv && (src >= size_ || src == rank_)) throw Invalid("recv: bad source rank");
+  if (has_send && has_recv && send.dtype != recv.dtype) throw Invalid("sendrecv: the two tensors differ in dtype");
+  return submit([this, send, dst, recv, src, has_send, has_recv] {
+    Chunk s{send.ptr, send.numel}, r{recv.ptr, recv.numel};
+    exchange(has_send ? &s : nullptr, dst, has_recv ? &r : nullptr, src, has_send ? send.dtype : recv.dtype, false, 0, 0);
+  }, caller, true);
+}
+
+std::shared_ptr<Work> Engine::barrier() {
+  if (!connected_) throw std::runtime_error("barrier: the engine is not connected");
+  return submit([this] { barrier_now(); }, nullptr, false);
+}
+
+}  // namespace tandem_hip
+
+// ---------------------------------------------------------------- C ABI
+using namespace tandem_hip;
+
+struct tdm_engine {
+  std::unique_ptr<Engine> impl;
+};
+
+struct tdm_work {
+  std::shared_ptr<Work> impl;
+};
+
+namespace {
+
+int finish_submit(std::shared_ptr<Work> w, tdm_work** out) {
+  auto* handle = new tdm_work{std::move(w)};
+  *out = handle;
+  return TDM_OK;
+}
+
+Engine& engine_of(tdm_engine* e) {
+  if (e == nullptr || !e->impl) throw Invalid("NULL engine");
+  return *e->impl;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tdm_engine_create(const char* job, int rank, int size, int slots, int64_t slot_bytes, double timeout_s, int device,
+                      tdm_engine** out) {
+  return guard([&] {
+    if (job == nullptr || out == nullptr) throw Invalid("NULL argument");
+    if (slot_bytes <= 0) throw Invalid("slot_bytes must be positive");
+    auto e = std::make_unique<Engine>(job, rank, size, slots, static_cast<size_t>(slot_bytes), timeout_s, device);
+    *out = new tdm_engine{std::move(e)};
+  });
+}
+
+int tdm_engine_connect(tdm_engine* e) {
+  return guard([&] { engine_of(e).connect(); });
+}
+
+int tdm_engine_close(tdm_engine* e) {
+  return guard([&] { engine_of(e).close(); });
+}
+
+int tdm_engine_destroy(tdm_engine* e) {
+  return guard([&] { delete e; });
+}
+
+int tdm_all_reduce(tdm_engine* e, void* ptr, int64_t numel, int dtype, int average, tdm_stream caller, tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    finish_submit(engine_of(e).all_reduce(Engine::Buf{static_cast<char*>(ptr), numel, dtype}, average != 0,
+                                          static_cast<hipStream_t>(caller)), out);
+  });
+}
+
+int tdm_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
+                       tdm_stream caller, tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    if (nsizes < 0 || (nsizes > 0 && sizes == nullptr)) throw Invalid("bad sizes");
+    std::vector<int64_t> sz(sizes, sizes + nsizes);
+    finish_submit(engine_of(e).reduce_scatter(Engine::Buf{static_cast<char*>(ptr), numel, dtype}, std::move(sz),
+                                              average != 0, static_cast<hipStream_t>(caller)), out);
+  });
+}
+
+int tdm_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, tdm_stream caller,
+                   tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    if (nsizes < 0 || (nsizes > 0 && sizes == nullptr)) throw Invalid("bad sizes");
+    std::vector<int64_t> sz(sizes, sizes + nsizes);
+    finish_submit(engine_of(e).all_gather(Engine::Buf{static_cast<char*>(ptr), numel, dtype}, std::move(sz),
+                                          static_cast<hipStream_t>(caller)), out);
+  });
+}
+
+int tdm_broadcast(tdm_engine* e, void* ptr, int64_t numel, int dtype, int root, tdm_stream caller, tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    finish_submit(engine_of(e).broadcast(Engine::Buf{static_cast<char*>(ptr), numel, dtype}, root,
+                                         static_cast<hipStream_t>(caller)), out);
+  });
+}
+
+int tdm_sendrecv(tdm_engine* e, const void* send, int64_t send_numel, int dst, void* recv, int64_t recv_numel, int src,
+                 int dtype, tdm_stream caller, tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    finish_submit(engine_of(e).sendrecv(Engine::Buf{static_cast<char*>(const_cast<void*>(send)), send_numel, dtype}, dst,
+                                        Engine::Buf{static_cast<char*>(recv), recv_numel, dtype}, src,
+                                        static_cast<hipStream_t>(caller)), out);
+  });
+}
+
+int tdm_barrier(tdm_engine* e, tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    finish_submit(engine_of(e).barrier(), out);
+  });
+}
+
+int tdm_work_wait(tdm_work* w, tdm_stream caller) {
+  if (w == nullptr || !w->impl) {
+    set_last_error("NULL work");
+    return TDM_EINVAL;
+  }
+  Work& work = *w->impl;
+  {
+    std::unique_lock<std::mutex> lock(work.mu);
+    work.cv.wait(lock, [&] { return work.finished; });
+    if (work.status != TDM_OK) {
+      set_last_error(work.error);
+      return work.status;
+    }
+  }
+  if (work.done_event) {
+    return guard([&] {
+      check_hip(hipStreamWaitEvent(static_cast<hipStream_t>(caller), work.done_event, 0), "hipStreamWaitEvent (wait)");
+    });
+  }
+  return TDM_OK;
+}
+
+int tdm_work_done(tdm_work* w) {
+  if (w == nullptr || !w->impl) return 0;
+  Work& work = *w->impl;
+  std::lock_guard<std::mutex> lock(work.mu);
+  if (!work.finished) return 0;
+  if (work.status == TDM_OK && work.done_event) return hipEventQuery(work.done_event) == hipSuccess ? 1 : 0;
+  return 1;
+}
+
+int tdm_work_times(tdm_work* w, double* started, double* finished) {
+  if (w == nullptr || !w->impl) {
+    set_last_error("NULL work");
+    return TDM_EINVAL;
+  }
+  std::lock_guard<std::mutex> lock(w->impl->mu);
+  if (started) *started = w->impl->t0;
+  if (finished) *finished = w->impl->t1;
+  return TDM_OK;
+}
+
+int tdm_work_free(tdm_work* w) {
+  delete w;
+  return TDM_OK;
+}
+
+}  // extern "C"

@@ -45,7 +45,7 @@ def test_argument_errors_need_no_gpu():
     assert b"npairs" in L.tdm_last_error()
     assert L.tdm_k1_copy_step(None, 0, 99, 0, None) == 1
     assert L.tdm_k2_table_bytes(0) > 0 and L.tdm_k2_table_bytes(3) > L.tdm_k2_table_bytes(2)
-    assert L.tdm_set_blocks_per_cu(1000) == 1
+    assert L.tdm_set_blocks_per_cu(5000) == 1
     assert L.tdm_set_blocks_per_cu(0) == 0
 
 
