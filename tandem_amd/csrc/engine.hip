@@ -10,11 +10,18 @@
 //   * a put is one launch of the copy kernel into the sender's slot (dividing by
 //     the world size on the way when the collective averages), a take is one
 //     launch of the fused ring-step kernel that reads the peer's slot in place;
-//   * the host never waits for the GPU per piece: slot hand-over is ordered by
-//     interprocess events (full[j] / free[j]) opened from hipIpcEventHandle_t, and
-//     an 8-byte message per piece in a shared-memory ring says which slot and how
-//     long (TANDEM_HIP_SYNC=host replaces the events with stream synchronisation
-//     before each message, for debugging);
+//   * an 8-byte message per piece in a shared-memory ring says which slot and how
+//     long. Two ways of ordering a slot's hand-over against the GPU work:
+//       "host"  (default) the progress thread only enqueues; a completion thread
+//               waits on an ordinary event recorded after each kernel and then
+//               publishes the message (piece ready) or the release (slot free), so
+//               a message always means "the bytes have landed" and neither the
+//               progress thread nor the caller ever blocks on the GPU;
+//       "event" (TANDEM_HIP_SYNC=event) interprocess events full[j] / free[j],
+//               exported with hipIpcGetEventHandle and waited for on the stream,
+//               as the reference's CUDA engine does. HIP implements these by
+//               registering a shared host page with the GPU; where the platform
+//               refuses that registration they cannot be recorded, hence the default;
 //   * every rank publishes its handles in one POSIX shared-memory region,
 //     "/tandem-<job>-<rank>-hip", which also holds the message rings it sends on.
 //
@@ -262,8 +269,27 @@ class Engine {
   std::vector<std::unique_ptr<Region>> theirs_;
   std::vector<void*> out_mem_, peer_mem_;
   std::vector<std::vector<hipEvent_t>> full_, free_, peer_full_, peer_free_;
-  std::vector<uint64_t> sent_, got_;
+  std::vector<uint64_t> sent_, got_;     // pieces, per peer: pick the slot
+  std::vector<uint64_t> posted_;         // messages queued or published to each peer (flow control)
+  std::vector<uint64_t> taken_;          // messages consumed from each peer
   bool connected_ = false, closed_ = false;
+
+  // "host" ordering: what to publish once the GPU has passed an event.
+  struct Completion {
+    hipEvent_t after;  // nullptr: publish at once (still in order)
+    bool is_release;
+    int peer;
+    uint64_t length;
+  };
+  void complete_later(bool is_release, int peer, uint64_t length, bool after_stream);
+  void completion_loop();
+  void drain_completions();
+  std::mutex cmu_;
+  std::condition_variable ccv_, cidle_;
+  std::deque<Completion> completions_;
+  bool cstop_ = false, cbusy_ = false;
+  std::string cerror_;
+  std::thread completer_;
 
   std::mutex mu_;
   std::condition_variable cv_;
@@ -275,7 +301,7 @@ class Engine {
 Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slot_bytes, double timeout_s, int device)
     : job_(job), rank_(rank), size_(size), slots_(slots), slot_bytes_(slot_bytes), timeout_s_(timeout_s),
       device_(device), theirs_(size), out_mem_(size, nullptr), peer_mem_(size, nullptr), full_(size), free_(size),
-      peer_full_(size), peer_free_(size), sent_(size, 0), got_(size, 0) {
+      peer_full_(size), peer_free_(size), sent_(size, 0), got_(size, 0), posted_(size, 0), taken_(size, 0) {
   if (size < 1 || rank < 0 || rank >= size) throw Invalid("rank must be in [0, size)");
   if (slots < 1 || slots > kMaxSlots) throw Invalid("slots must be in [1, " + std::to_string(kMaxSlots) + "]");
   if (slot_bytes < 16 || slot_bytes % 16) throw Invalid("slot_bytes must be a positive multiple of 16");
@@ -285,7 +311,7 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
   if (device < 0) throw Invalid("the hip engine needs a GPU: device must be >= 0 (there is no CPU path)");
   if (job.empty() || job.size() > 64) throw Invalid("job name must have 1..64 characters");
   const char* mode = std::getenv("TANDEM_HIP_SYNC");
-  use_events_ = !(mode && std::string(mode) == "host");
+  use_events_ = mode && std::string(mode) == "event";
 
   check_hip(hipSetDevice(device_), "hipSetDevice");
   check_hip(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags");  // default priority
@@ -318,6 +344,7 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
   }
   std::atomic_thread_fence(std::memory_order_release);
   h->magic = kRegionMagic;  // published last
+  if (!use_events_) completer_ = std::thread([this] { completion_loop(); });
   thread_ = std::thread([this] { loop(); });
 }
 
@@ -370,9 +397,18 @@ void Engine::close() {
   if (connected_) {
     try {
       barrier_now();
+      drain_completions();
     } catch (const std::exception& e) {
       barrier_err = e.what();
     }
+  }
+  if (completer_.joinable()) {
+    {
+      std::lock_guard<std::mutex> lock(cmu_);
+      cstop_ = true;
+    }
+    ccv_.notify_all();
+    completer_.join();
   }
   for (int p = 0; p < size_; ++p) {
     if (p == rank_) continue;
@@ -482,17 +518,76 @@ void Engine::signal(int dst, uint64_t length) {
   r.head.store(head + 1, std::memory_order_release);  // the length is visible before the new head
 }
 
+// The next message from src. Messages are consumed in order by the progress
+// thread (taken_), and released, possibly later, in the same order (tail).
 uint64_t Engine::await(int src) {
   Ring& r = theirs_[src]->entry(rank_)->ring;
-  const uint64_t tail = r.tail.load(std::memory_order_relaxed);
-  wait_until([&] { return r.head.load(std::memory_order_acquire) > tail; }, timeout_s_,
+  const uint64_t at = taken_[src];
+  wait_until([&] { return r.head.load(std::memory_order_acquire) > at; }, timeout_s_,
              "timed out waiting for a message from a peer rank");
-  return r.length[tail % slots_];
+  taken_[src] = at + 1;
+  return r.length[at % slots_];
 }
 
 void Engine::release(int src) {
   Ring& r = theirs_[src]->entry(rank_)->ring;
   r.tail.store(r.tail.load(std::memory_order_relaxed) + 1, std::memory_order_release);
+}
+
+// "host" ordering. Completions are published strictly in the order they were
+// queued, which is the order of the kernels on the engine's stream.
+void Engine::complete_later(bool is_release, int peer, uint64_t length, bool after_stream) {
+  Completion c{nullptr, is_release, peer, length};
+  if (after_stream) {
+    check_hip(hipEventCreateWithFlags(&c.after, hipEventDisableTiming), "hipEventCreateWithFlags (completion)");
+    hipError_t err = hipEventRecord(c.after, stream_);
+    if (err != hipSuccess) {
+      (void)hipEventDestroy(c.after);
+      check_hip(err, "hipEventRecord (completion)");
+    }
+  }
+  {
+    std::lock_guard<std::mutex> lock(cmu_);
+    if (!cerror_.empty()) throw std::runtime_error("completion thread failed: " + cerror_);
+    completions_.push_back(c);
+  }
+  ccv_.notify_one();
+}
+
+void Engine::completion_loop() {
+  (void)hipSetDevice(device_);
+  for (;;) {
+    Completion c;
+    {
+      std::unique_lock<std::mutex> lock(cmu_);
+      cbusy_ = false;
+      if (completions_.empty()) cidle_.notify_all();
+      ccv_.wait(lock, [this] { return cstop_ || !completions_.empty(); });
+      if (completions_.empty()) return;
+      c = completions_.front();
+      completions_.pop_front();
+      cbusy_ = true;
+    }
+    if (c.after) {
+      hipError_t err = hipEventSynchronize(c.after);
+      (void)hipEventDestroy(c.after);
+      if (err != hipSuccess) {  // do not publish: the peers time out rather than read bad bytes
+        std::lock_guard<std::mutex> lock(cmu_);
+        if (cerror_.empty()) cerror_ = std::string("hipEventSynchronize: ") + hipGetErrorString(err);
+        continue;
+      }
+    }
+    if (c.is_release) release(c.peer); else signal(c.peer, c.length);
+  }
+}
+
+void Engine::drain_completions() {
+  if (use_events_) return;
+  std::unique_lock<std::mutex> lock(cmu_);
+  if (!cidle_.wait_for(lock, std::chrono::duration<double>(timeout_s_), [this] { return completions_.empty() && !cbusy_; })) {
+    throw Timeout("timed out waiting for the GPU to finish the queued pieces");
+  }
+  if (!cerror_.empty()) throw std::runtime_error("completion thread failed: " + cerror_);
 }
 
 void Engine::barrier_now() {
@@ -502,15 +597,16 @@ void Engine::barrier_now() {
   for (int p = 0; p < size_; ++p) {
     if (p == rank_) continue;
     Ring& r = mine_.entry(p)->ring;
-    const uint64_t head = r.head.load(std::memory_order_relaxed);
-    wait_until([&] { return head - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots_); },
+    const uint64_t posted = posted_[p];
+    wait_until([&] { return posted - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots_); },
                timeout_s_, "barrier: a peer rank never drained its messages");
-    signal(p, kEmpty);
+    posted_[p] = posted + 1;
+    if (use_events_) signal(p, kEmpty); else complete_later(false, p, kEmpty, false);
   }
   for (int p = 0; p < size_; ++p) {
     if (p == rank_) continue;
     if (await(p) != kEmpty) throw std::runtime_error("barrier out of step: expected an empty message, got a piece");
-    release(p);
+    if (use_events_) release(p); else complete_later(true, p, 0, false);
   }
 }
 
@@ -523,8 +619,8 @@ void Engine::put(int dst, const char* src, int64_t numel, int dtype, int scale_w
   Ring& r = mine_.entry(dst)->ring;
   // Room in the message ring means fewer than `slots` messages are unreleased, so
   // fewer than `slots` pieces are: dst has released slot j's previous piece ...
-  const uint64_t head = r.head.load(std::memory_order_relaxed);
-  wait_until([&] { return head - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots_); }, timeout_s_,
+  const uint64_t posted = posted_[dst];
+  wait_until([&] { return posted - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots_); }, timeout_s_,
              "put: the peer never freed a slot");
   if (use_events_ && k >= static_cast<uint64_t>(slots_)) {
     // ... and enqueued its reads of it before recording free[j]: wait for those reads.
@@ -537,13 +633,14 @@ void Engine::put(int dst, const char* src, int64_t numel, int dtype, int scale_w
     tdm_pair pr{slot, src, numel};
     copy_step(&pr, 1, dtype, scale_world, stream_);
   }
+  posted_[dst] = posted + 1;
+  sent_[dst] = k + 1;
   if (use_events_) {
     check_hip(hipEventRecord(full_[dst][j], stream_), "hipEventRecord (full)");
+    signal(dst, nbytes);
   } else {
-    check_hip(hipStreamSynchronize(stream_), "hipStreamSynchronize (put)");
+    complete_later(false, dst, nbytes, true);  // published once the copy has landed
   }
-  signal(dst, nbytes);
-  sent_[dst] = k + 1;
 }
 
 void Engine::take(int src, char* into, int64_t numel, int dtype, bool reduce, int scale_world) {
@@ -567,13 +664,13 @@ void Engine::take(int src, char* into, int64_t numel, int dtype, bool reduce, in
     tdm_pair pr{into, slot, numel};
     copy_step(&pr, 1, dtype, 0, stream_);
   }
+  got_[src] += 1;
   if (use_events_) {
     check_hip(hipEventRecord(free_[src][j], stream_), "hipEventRecord (free)");
+    release(src);
   } else {
-    check_hip(hipStreamSynchronize(stream_), "hipStreamSynchronize (take)");
+    complete_later(true, src, 0, true);  // the slot is free once our kernel has read it
   }
-  got_[src] += 1;
-  release(src);
 }
 
 // Sends `send` to dst while receiving `recv` from src, one piece of each at a

@@ -137,7 +137,8 @@ def async_order(g):
     w2.wait()
     torch.cuda.synchronize()
     assert w2.is_completed() and float(big.sum()) == float(1 << 22)
-    assert len(g.trace) == 1 and g.trace[0][0] == "all_reduce" and g.trace[0][3] == 4 << 22
+    assert len(g.trace) == 6 and g.trace[-1][0] == "all_reduce" and g.trace[-1][3] == 4 << 22
+    assert all(t1 >= t0 for _, t0, t1, _ in g.trace)
     return True
 
 
