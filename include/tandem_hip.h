@@ -205,6 +205,13 @@ int tdm_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype, const
 int tdm_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, tdm_stream caller,
                    tdm_work** out);
 int tdm_broadcast(tdm_engine* e, void* ptr, int64_t numel, int dtype, int root, tdm_stream caller, tdm_work** out);
+/* K4 for process ranks: places this rank's `shard` into its chunk of `full` and
+ * ring-all-gathers the other chunks, on the engine's stream, so that a unit's
+ * parameters arrive while the caller's stream still computes the previous unit.
+ * Replaces `full[lo:hi].copy_(shard)` + `all_gather(full, sizes, async_op=True)` of
+ * FSDP._start_gather (tandem/zero.py:238-245). */
+int tdm_unit_gather(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes, int nsizes,
+                    tdm_stream caller, tdm_work** out);
 int tdm_sendrecv(tdm_engine* e, const void* send, int64_t send_numel, int dst, void* recv, int64_t recv_numel, int src,
                  int dtype, tdm_stream caller, tdm_work** out);
 int tdm_barrier(tdm_engine* e, tdm_work** out);

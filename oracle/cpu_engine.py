@@ -210,6 +210,18 @@ class CpuGroup:
 
         return self._enqueue("all_gather", job, t.numel() * t.element_size(), async_op)
 
+    # ---- the two helpers tandem_amd's wrappers ask of a group, with torch's CPU copy_
+    def pack(self, flat, pieces):
+        dst = self._flat(flat)
+        for off, t in pieces:
+            dst[off:off + t.numel()].copy_(t.reshape(-1))
+        return flat
+
+    def gather_unit(self, full, shard, sizes=None, async_op=False):
+        flat = self._flat(full)
+        self._cut(flat, sizes)[self.rank].copy_(shard.reshape(-1))
+        return self.all_gather(full, sizes, async_op=async_op)
+
     def broadcast(self, t, root=0, async_op=False):
         flat = self._flat(t)
 

@@ -76,6 +76,7 @@ _ENGINE_SIGNATURES = {
     "tdm_reduce_scatter": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _PI64, ctypes.c_int, ctypes.c_int, _VP, _PVP]),
     "tdm_all_gather": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _PI64, ctypes.c_int, _VP, _PVP]),
     "tdm_broadcast": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _VP, _PVP]),
+    "tdm_unit_gather": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _VP, _PI64, ctypes.c_int, _VP, _PVP]),
     "tdm_sendrecv": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _VP, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                     _VP, _PVP]),
     "tdm_barrier": (ctypes.c_int, [_VP, _PVP]),

@@ -197,6 +197,53 @@ class Group:
             self._engine, ctypes.c_void_p(flat.data_ptr()), self._count(flat, code), code, arr, n, self._stream(), out),
             t, t.numel() * t.element_size(), async_op, keep=(flat,))
 
+    def gather_unit(self, full, shard, sizes=None, async_op=False):
+        """ZeRO-3's gather of one unit: `shard` (this rank's chunk) is placed into
+        `full` and the other ranks' chunks are gathered, all on the engine's
+        stream. Same result as `full[lo:hi].copy_(shard); all_gather(full, sizes)`."""
+        flat = self._flat(full, "gather_unit")
+        sh = self._flat(shard, "gather_unit")
+        if sh.dtype != flat.dtype:
+            raise CommError("gather_unit: shard and full buffer differ in dtype")
+        code = self._code(flat, False)
+        sizes, arr, n = self._sizes(flat, sizes)
+        if self._chunk_of_rank(flat, sizes).numel() != sh.numel():
+            raise CommError(f"gather_unit: the shard has {sh.numel()} elements, this rank's chunk another count")
+        if code == _lib.TDM_BYTES and n:
+            arr = (ctypes.c_int64 * n)(*[s * flat.element_size() for s in sizes])
+        return self._start("gather_unit", lambda out: lib().tdm_unit_gather(
+            self._engine, ctypes.c_void_p(flat.data_ptr()), self._count(flat, code), code, ctypes.c_void_p(sh.data_ptr()),
+            arr, n, self._stream(), out), full, full.numel() * full.element_size(), async_op, keep=(flat, sh))
+
+    def pack(self, flat, pieces):
+        """Bucket flatten as one gather: flat[offset : offset + t.numel()] = t for
+        every (offset, t) in `pieces`, in launches of up to 16 streams each on the
+        caller's current stream (the gradients were produced there). Replaces one
+        `view.copy_(p.grad)` per parameter (tandem/ddp.py:92-94, tandem/zero.py:130,297
+        in the reference)."""
+        dst = self._flat(flat, "pack")
+        code = self._code(dst, True)
+        es = dst.element_size()
+        items = []
+        for off, t in pieces:
+            src = self._flat(t, "pack")
+            if src.dtype != dst.dtype:
+                raise CommError("pack: a piece differs in dtype from the flat buffer")
+            if off < 0 or off + src.numel() > dst.numel():
+                raise CommError("pack: a piece does not fit the flat buffer")
+            if src.numel():
+                items.append((dst.data_ptr() + off * es, src.data_ptr(), src.numel()))
+        for k in range(0, len(items), _lib.TDM_MAX_PAIRS):
+            part = items[k:k + _lib.TDM_MAX_PAIRS]
+            arr = (_lib.Pair * len(part))()
+            for i, (d, s, n) in enumerate(part):
+                arr[i].dst, arr[i].src, arr[i].count = d, s, n
+            try:
+                check(lib().tdm_k1_copy_step(arr, len(part), code, 0, self._stream()))
+            except (ValueError, RuntimeError) as e:
+                raise CommError(f"pack: {e}") from e
+        return flat
+
     def broadcast(self, t, root=0, async_op=False):
         """Pipelined along the ring from root."""
         flat = self._flat(t, "broadcast")

@@ -224,6 +224,7 @@ class Engine {
   std::shared_ptr<Work> all_reduce(Buf t, bool average, hipStream_t caller);
   std::shared_ptr<Work> reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, hipStream_t caller);
   std::shared_ptr<Work> all_gather(Buf t, std::vector<int64_t> sizes, hipStream_t caller);
+  std::shared_ptr<Work> unit_gather(Buf full, const char* shard, std::vector<int64_t> sizes, hipStream_t caller);
   std::shared_ptr<Work> broadcast(Buf t, int root, hipStream_t caller);
   std::shared_ptr<Work> sendrecv(Buf send, int dst, Buf recv, int src, hipStream_t caller);
   std::shared_ptr<Work> barrier();
@@ -790,6 +791,33 @@ std::shared_ptr<Work> Engine::all_gather(Buf t, std::vector<int64_t> sizes, hipS
   }, caller, true);
 }
 
+// ZeRO-3's gather of one unit: this rank's shard is placed into its chunk of the
+// (so far uninitialised) full buffer and the ring all-gather fills in the rest, all
+// on the engine's stream, so the unit arrives while the caller's stream computes
+// the previous one (tandem/zero.py:238-245 in the reference).
+std::shared_ptr<Work> Engine::unit_gather(Buf full, const char* shard, std::vector<int64_t> sizes, hipStream_t caller) {
+  check(full, "unit_gather", false);
+  const auto c = chunks(full, sizes);
+  if (c[rank_].numel > 0) {
+    if (shard == nullptr) throw Invalid("unit_gather: NULL shard");
+    check(Buf{const_cast<char*>(shard), c[rank_].numel, full.dtype}, "unit_gather (shard)", false);
+  }
+  return submit([this, full, shard, sizes] {
+    const auto cs = chunks(full, sizes);
+    const Chunk& mine = cs[rank_];
+    if (mine.numel > 0 && shard != mine.ptr) {
+      if (full.dtype == kBytesDtype) {
+        check_hip(hipMemcpyAsync(mine.ptr, shard, static_cast<size_t>(mine.numel), hipMemcpyDeviceToDevice, stream_),
+                  "hipMemcpyAsync (unit_gather)");
+      } else {
+        tdm_pair pr{mine.ptr, shard, mine.numel};
+        copy_step(&pr, 1, full.dtype, 0, stream_);
+      }
+    }
+    if (size_ > 1) ring_all_gather(cs, full.dtype);
+  }, caller, true);
+}
+
 // Pipelined along the ring from the root: each rank forwards each piece as soon
 // as it has it (tandem/comm.py:387-409).
 std::shared_ptr<Work> Engine::broadcast(Buf t, int root, hipStream_t caller) {
@@ -906,6 +934,18 @@ int tdm_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int
     std::vector<int64_t> sz(sizes, sizes + nsizes);
     finish_submit(engine_of(e).all_gather(Engine::Buf{static_cast<char*>(ptr), numel, dtype}, std::move(sz),
                                           static_cast<hipStream_t>(caller)), out);
+  });
+}
+
+int tdm_unit_gather(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes, int nsizes,
+                    tdm_stream caller, tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    if (nsizes < 0 || (nsizes > 0 && sizes == nullptr)) throw Invalid("bad sizes");
+    std::vector<int64_t> sz(sizes, sizes + nsizes);
+    finish_submit(engine_of(e).unit_gather(Engine::Buf{static_cast<char*>(full), numel, dtype},
+                                           static_cast<const char*>(shard), std::move(sz),
+                                           static_cast<hipStream_t>(caller)), out);
   });
 }
 

@@ -1,0 +1,146 @@
+"""Data parallelism over a tandem group: every rank holds the whole model,
+trains on its rows of the batch, and the ranks average gradients before each
+optimizer step.
+
+Drop-in for the reference's wrapper (tandem/ddp.py:36-129 there): same
+constructor, `no_sync()`, bucket packing, launch order and one-time rebuild, so
+the averaged gradients are the reference's bit for bit at any world size (the
+ring's summation order depends on where a gradient sits in its bucket).
+
+What differs is how a bucket is filled. The reference copies each gradient into
+its view of the bucket as it arrives, one small copy per parameter. Here a
+bucket's gradients are gathered by `group.pack`, a single table-driven launch,
+when the bucket's last gradient has arrived, immediately before its all-reduce
+is queued; after that each `p.grad` is its view of the bucket, so the all-reduce
+lands in place and nothing is copied back.
+
+`group` is anything with tandem's Group interface plus `pack(flat, pieces)`;
+tandem_amd.Group(backend="hip") is the one that ships.
+"""
+
+import contextlib
+
+import torch
+from torch.autograd import Variable
+
+
+class Bucket:
+    """Parameters that travel together: one flat buffer, one view per parameter."""
+
+    def __init__(self, params, device, dtype):
+        self.params = list(params)
+        self.flat = torch.zeros(sum(p.numel() for p in self.params), device=device, dtype=dtype)
+        self.views, self.offsets = {}, {}
+        at = 0
+        for p in self.params:
+            self.offsets[p] = at
+            self.views[p] = self.flat[at:at + p.numel()].view_as(p)
+            at += p.numel()
+        self.arrived = 0
+        self.loose = []  # parameters whose gradient still lives outside the bucket
+        self.work = None
+
+
+class DDP(torch.nn.Module):
+    def __init__(self, module, group, bucket_bytes=25 << 20, overlap=True, rebuild=True):
+        super().__init__()
+        if not hasattr(group, "pack"):
+            raise TypeError("tandem_amd.DDP needs a group that provides pack() (tandem_amd.Group does)")
+        self.module, self.g = module, group
+        self.bucket_bytes, self.overlap = bucket_bytes, overlap
+        self._rebuild_pending = rebuild
+        self.params = [p for p in module.parameters() if p.requires_grad]
+        with torch.no_grad():
+            for p in self.params:  # every rank starts from rank 0's weights
+                self.g.broadcast(p.data, root=0)
+        # Before any backward has shown the real order, assume gradients arrive in
+        # reverse registration order.
+        self._build(self.params[::-1])
+        self._reduce_now = True
+        self._arrival = []
+        self._callback_queued = False
+        for p in self.params:
+            p.register_post_accumulate_grad_hook(self._on_grad)
+
+    # ---- buckets
+    def _build(self, order):
+        from .buckets import pack
+
+        groups = pack([p.numel() * p.element_size() for p in order], self.bucket_bytes, [p.dtype for p in order])
+        self.buckets, self.bucket_of = [], {}
+        for members in groups:
+            ps = [order[i] for i in members]
+            b = Bucket(ps, ps[0].device, ps[0].dtype)
+            self.buckets.append(b)
+            for p in ps:
+                self.bucket_of[p] = b
+        self._cursor = 0  # next bucket to launch: every rank launches in the same order
+
+    def _gather(self, bucket):
+        """Moves the bucket's loose gradients into it with one gather, and points
+        each p.grad at its view."""
+        if bucket.loose:
+            self.g.pack(bucket.flat, [(bucket.offsets[p], p.grad) for p in bucket.loose])
+            for p in bucket.loose:
+                p.grad = bucket.views[p]
+            bucket.loose = []
+
+    def forward(self, *args, **kwargs):
+        return self.module(*args, **kwargs)
+
+    @contextlib.contextmanager
+    def no_sync(self):
+        """Gradient accumulation: backward passes inside only accumulate
+        locally; the next one outside reduces the sum."""
+        before, self._reduce_now = self._reduce_now, False
+        try:
+            yield
+        finally:
+            self._reduce_now = before
+
+    # ---- backward
+    def _on_grad(self, p):
+        b = self.bucket_of[p]
+        if p.grad is not b.views[p]:  # first gradient since zero_grad
+            b.loose.append(p)
+        if not self._reduce_now:
+            self._gather(b)  # accumulate inside the bucket from now on
+            return
+        if not self._callback_queued:
+            self._callback_queued = True
+            Variable._execution_engine.queue_callback(self._after_backward)
+        if self._rebuild_pending:
+            self._arrival.append(p)
+        b.arrived += 1
+        while self._cursor < len(self.buckets):
+            nxt = self.buckets[self._cursor]
+            if nxt.arrived != len(nxt.params):
+                break
+            self._gather(nxt)
+            nxt.work = self.g.all_reduce(nxt.flat, op="avg", async_op=True)
+            if not self.overlap:
+                nxt.work.wait()
+            self._cursor += 1
+
+    def _after_backward(self):
+        self._callback_queued = False
+        short = [b for b in self.buckets if b.arrived != len(b.params)]
+        if short:
+            unused = [tuple(p.shape) for b in short for p in b.params if p.grad is None]
+            raise RuntimeError(f"tandem DDP: some parameters received no gradient ({unused[:3]}...); every parameter must be used")
+        for b in self.buckets:
+            b.work.wait()
+            b.arrived, b.work = 0, None
+        self._cursor = 0
+        if self._rebuild_pending and len(self._arrival) == len(self.params):
+            # Once: rebuild the buckets in the order gradients really arrived, so
+            # the first bucket to fill is the first to be sent.
+            order, self._arrival, self._rebuild_pending = self._arrival, [], False
+            old = {p: p.grad for p in self.params}
+            self._build(order)
+            for b in self.buckets:
+                self.g.pack(b.flat, [(b.offsets[p], old[p]) for p in b.params])
+                for p in b.params:
+                    p.grad = b.views[p]
+        else:
+            self._arrival = []

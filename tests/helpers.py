@@ -32,3 +32,28 @@ def bits(a):
     """Bit pattern view for exact comparison (distinguishes -0.0 from 0.0, NaNs)."""
     a = np.ascontiguousarray(a)
     return a.view({2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize])
+
+
+class OracleShardedAdamW:
+    """The oracle's AdamW behind ShardedAdamW's interface, for CPU torch tensors
+    (the wrappers' host logic is tested on the CPU with this and the oracle's
+    CPU-process group; the product's own optimizer and group are GPU only).
+    torch_sqrt=True substitutes torch's CPU sqrt, to compare bit for bit with runs
+    that used torch's CPU kernels."""
+
+    def __init__(self, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, torch_sqrt=True):
+        from oracle.adamw import AdamW
+
+        root = (lambda v: torch.from_numpy(v).sqrt().numpy()) if torch_sqrt else None
+        self.inner = AdamW(lr, betas, eps, weight_decay, sqrt=root)
+
+    def update(self, key, param, grad):
+        assert param.device.type == "cpu" and param.is_contiguous() and grad.is_contiguous()
+        self.inner.update(key, param.detach().numpy(), grad.detach().numpy())
+
+    def state_bytes(self):
+        return self.inner.state_bytes()
+
+    @property
+    def state(self):
+        return self.inner.state
