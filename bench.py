@@ -40,17 +40,18 @@ def ring_pass(lw, bufs, events=None):
     events on the launch stream when asked."""
     import torch
 
-    flats = [b.reshape(-1) for b in bufs]
-    from tandem_amd.local import chunk_bounds
+    from tandem_amd._lib import check, lib, stream_ptr
 
-    bounds = chunk_bounds(flats[0].numel(), lw.world)
+    flats = [b.reshape(-1) for b in bufs]
+    ptrs, n, st = lw._ptrs(flats), flats[0].numel(), stream_ptr(flats[0].device)
+    none = lw._sizes(None, None)[0]
     if events is not None:
         e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
         e[0].record()
-    lw._reduce_scatter(flats, bounds, True, False)
+    check(lib().tdm_local_reduce_scatter(ptrs, lw.world, n, 0, none, 0, 1, 0, st))
     if events is not None:
         e[1].record()
-    lw._all_gather(flats, bounds)
+    check(lib().tdm_local_all_gather(ptrs, lw.world, n, 0, none, 0, st))
     if events is not None:
         e[2].record()
         events.append(e)

@@ -84,6 +84,28 @@ int tdm_k1_reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, 
  * (tandem/csrc/collectives.cpp:247-250). */
 int tdm_k1_copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, tdm_stream stream);
 
+/* ---- a whole group in one process: rank r is bufs[r] in this GPU's HBM ----- */
+
+/* tandem's ring collectives over `world` equally sized, non-overlapping device
+ * buffers, one per rank, with ONE launch of the K1 kernels per ring step carrying
+ * every rank's (receiving chunk, neighbour's chunk) pair. In place; the results,
+ * including the partial sums a bare reduce_scatter leaves in the other chunks
+ * (keep_sent != 0), are bit for bit those of Group.reduce_scatter / all_gather /
+ * all_reduce run as `world` processes (tandem/comm.py:301-385). sizes / nsizes
+ * as for the engine's collectives (nsizes == 0: torch.tensor_split). */
+int tdm_local_reduce_scatter(void* const* bufs, int world, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
+                             int average, int keep_sent, tdm_stream stream);
+int tdm_local_all_gather(void* const* bufs, int world, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
+                         tdm_stream stream);
+
+enum tdm_allreduce_algorithm {
+  TDM_ALLREDUCE_RING = 0, /* reduce-scatter then all-gather: 2 (world - 1) launches */
+  TDM_ALLREDUCE_FOLD = 1  /* one launch: every element read from all ranks, folded in the ring's
+                           * order for its chunk, written to all ranks (world <= 8); same bits */
+};
+int tdm_local_all_reduce(void* const* bufs, int world, int64_t numel, int dtype, int average, int algorithm,
+                         tdm_stream stream);
+
 /* ---- K2: bucket flatten + average + unflatten ---------------------------- */
 
 /* One segment of a bucket: `count` elements that lie in ring chunk `chunk` of the
@@ -98,11 +120,11 @@ typedef struct tdm_fold_seg {
   int32_t reserved;
 } tdm_fold_seg;
 
-/* Bytes of device memory a table of nseg segments needs. */
-int64_t tdm_k2_table_bytes(int nseg);
+/* Bytes of device memory the table of these segments needs (-1: bad arguments). */
+int64_t tdm_k2_table_bytes(const tdm_fold_seg* segs, int nseg, int dtype);
 
 /* Writes the device image of the table into host memory `image`
- * (tdm_k2_table_bytes(nseg) bytes); the caller copies it to the device once. */
+ * (tdm_k2_table_bytes(...) bytes); the caller copies it to the device once. */
 int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype, void* image);
 
 /* For every element of every segment, in one launch:

@@ -18,6 +18,8 @@ ABI_VERSION = 1
 
 DTYPES = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3, torch.int64: 4, torch.int32: 5}
 
+ALLREDUCE_RING = 0
+ALLREDUCE_FOLD = 1
 ADAMW_HOST_ORDER = 0
 ADAMW_DEVICE_ORDER = 1
 
@@ -50,7 +52,14 @@ _SIGNATURES = {
     "tdm_k1_reduce_step": (ctypes.c_int, [ctypes.POINTER(Pair), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                           ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "tdm_k1_copy_step": (ctypes.c_int, [ctypes.POINTER(Pair), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
-    "tdm_k2_table_bytes": (ctypes.c_int64, [ctypes.c_int]),
+    "tdm_local_reduce_scatter": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+                                                ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                ctypes.c_void_p]),
+    "tdm_local_all_gather": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+                                            ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_void_p]),
+    "tdm_local_all_reduce": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+                                            ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
+    "tdm_k2_table_bytes": (ctypes.c_int64, [ctypes.POINTER(FoldSeg), ctypes.c_int, ctypes.c_int]),
     "tdm_k2_table_build": (ctypes.c_int, [ctypes.POINTER(FoldSeg), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "tdm_k2_bucket_fold": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                           ctypes.c_void_p]),

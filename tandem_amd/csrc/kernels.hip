@@ -34,7 +34,11 @@ namespace {
 constexpr int kThreads = TDM_THREADS;
 constexpr int kUnroll = TDM_UNROLL;             // 16-byte vectors per lane per tile and stream
 constexpr int kTileVecs = kThreads * kUnroll;   // 1024 vectors = 16 KiB of every stream
-constexpr int kDefaultBlocksPerCu = 64;  // 16 Ki tiles: one 16 KiB tile per workgroup up to 256 MiB per stream
+// Measured on MI355X: one 16 KiB tile per workgroup beats a persistent grid-stride
+// loop by 5-8% (the hardware dispatcher balances 8 XCDs better than a fixed stride),
+// so the grid covers the tiles one to one up to 256 Ki workgroups (4 GiB per stream)
+// and strides only beyond that.
+constexpr int kDefaultBlocksPerCu = 1024;
 
 int g_blocks_per_cu = kDefaultBlocksPerCu;
 
@@ -361,77 +365,84 @@ struct FoldSegDev {
   int32_t vec_ok;  // every pointer of the segment is 16-byte aligned
 };
 
+// header | tile_end[nseg] (int64) | segments[nseg] | tile_seg[total_tiles] (int32)
 __host__ __device__ inline int64_t fold_tile_end_offset() { return sizeof(FoldHeader); }
 __host__ __device__ inline int64_t fold_segs_offset(int nseg) {
   return (sizeof(FoldHeader) + static_cast<int64_t>(nseg) * 8 + 15) / 16 * 16;
 }
+__host__ __device__ inline int64_t fold_tile_seg_offset(int nseg) {
+  return fold_segs_offset(nseg) + static_cast<int64_t>(nseg) * static_cast<int64_t>(sizeof(FoldSegDev));
+}
 
+// One tile of one segment: W loads per element, the fold in ring order, W stores.
 template <typename T, int kWorld, int kDiv>
-__global__ __launch_bounds__(kThreads) void k2_fold_kernel(const char* __restrict__ image, Divisor<T> dv) {
+__device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const Divisor<T>& dv) {
   using A = typename Elem<T>::acc;
   constexpr int L = lanes<T>();
   constexpr int kU = kWorld <= 2 ? 4 : 2;  // vectors per lane per tile step, per rank
   constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
-  const FoldHeader* hd = reinterpret_cast<const FoldHeader*>(image);
-  const int nseg = hd->nseg;
-  const int64_t* tile_end = reinterpret_cast<const int64_t*>(image + fold_tile_end_offset());
-  const FoldSegDev* segs = reinterpret_cast<const FoldSegDev*>(image + fold_segs_offset(nseg));
-  const int64_t total = hd->total_tiles;
-  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
-    int lo = 0, hi = nseg - 1;  // first segment whose running tile count exceeds `tile`
-    while (lo < hi) {
-      const int mid = (lo + hi) >> 1;
-      if (tile >= tile_end[mid]) lo = mid + 1; else hi = mid;
-    }
-    const FoldSegDev& sg = segs[lo];
-    const int64_t t = tile - (lo ? tile_end[lo - 1] : 0);
-    const int64_t n = sg.count;
-    const int c = sg.chunk;
-    // ring order: the fold starts at rank chunk+1 and ends with the chunk's owner
-    const char* sp[kWorld];
-    char* dp[kWorld];
+  const int64_t n = sg.count;
+  const int c = sg.chunk;
+  // ring order: the fold starts at rank chunk+1 and ends with the chunk's owner
+  const char* sp[kWorld];
+  char* dp[kWorld];
 #pragma unroll
-    for (int k = 0; k < kWorld; ++k) {
-      sp[k] = sg.src[(c + 1 + k) % kWorld];
-      dp[k] = sg.dst[k];
-    }
-    if (sg.vec_ok) {
-      const int64_t nv = n / L;
+  for (int k = 0; k < kWorld; ++k) {
+    sp[k] = sg.src[(c + 1 + k) % kWorld];
+    dp[k] = sg.dst[k];
+  }
+  if (sg.vec_ok) {
+    const int64_t nv = n / L;
 #pragma unroll
-      for (int u0 = 0; u0 < kUnroll; u0 += kU) {
-        const int64_t vbase = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u0) * kThreads;
-        vec16 in[kWorld][kU];
+    for (int u0 = 0; u0 < kUnroll; u0 += kU) {
+      const int64_t vbase = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u0) * kThreads;
+      vec16 in[kWorld][kU];
 #pragma unroll
-        for (int k = 0; k < kWorld; ++k)
-#pragma unroll
-          for (int u = 0; u < kU; ++u) {
-            const int64_t v = vbase + u * kThreads;
-            if (v < nv) in[k][u] = load_rmw(sp[k] + v * 16);
-          }
+      for (int k = 0; k < kWorld; ++k)
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
           const int64_t v = vbase + u * kThreads;
-          if (v < nv) {
-            Lanes<T> out;
+          if (v < nv) in[k][u] = load_stream(sp[k] + v * 16);
+        }
 #pragma unroll
-            for (int l = 0; l < L; ++l) {
-              A acc = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[0][u]).v[l]), dv.divisor, dv.reciprocal);
+      for (int u = 0; u < kU; ++u) {
+        const int64_t v = vbase + u * kThreads;
+        if (v < nv) {
+          Lanes<T> out;
 #pragma unroll
-              for (int k = 1; k < kWorld; ++k) {
-                const A y = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[k][u]).v[l]), dv.divisor, dv.reciprocal);
-                acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
-              }
-              out.v[l] = Elem<T>::narrow(acc);
+          for (int l = 0; l < L; ++l) {
+            A acc = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[0][u]).v[l]), dv.divisor, dv.reciprocal);
+#pragma unroll
+            for (int k = 1; k < kWorld; ++k) {
+              const A y = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[k][u]).v[l]), dv.divisor, dv.reciprocal);
+              acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
             }
-            const vec16 packed = pack<T>(out);
-#pragma unroll
-            for (int k = 0; k < kWorld; ++k)
-              if (dp[k]) store16(dp[k] + v * 16, packed);
+            out.v[l] = Elem<T>::narrow(acc);
           }
+          const vec16 packed = pack<T>(out);
+#pragma unroll
+          for (int k = 0; k < kWorld; ++k)
+            if (dp[k]) store16(dp[k] + v * 16, packed);
         }
       }
-      if (t == 0 && threadIdx.x < n - nv * L) {  // tail elements
-        const int64_t i = nv * L + threadIdx.x;
+    }
+    if (t == 0 && threadIdx.x < n - nv * L) {  // tail elements
+      const int64_t i = nv * L + threadIdx.x;
+      A acc = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[0])[i]), dv.divisor, dv.reciprocal);
+#pragma unroll
+      for (int k = 1; k < kWorld; ++k) {
+        const A y = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[k])[i]), dv.divisor, dv.reciprocal);
+        acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+      }
+#pragma unroll
+      for (int k = 0; k < kWorld; ++k)
+        if (dp[k]) reinterpret_cast<T*>(dp[k])[i] = Elem<T>::narrow(acc);
+    }
+  } else {
+    const int64_t e0 = t * kTileElems + threadIdx.x;
+    for (int k2 = 0; k2 < kUnroll * L; ++k2) {
+      const int64_t i = e0 + static_cast<int64_t>(k2) * kThreads;
+      if (i < n) {
         A acc = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[0])[i]), dv.divisor, dv.reciprocal);
 #pragma unroll
         for (int k = 1; k < kWorld; ++k) {
@@ -442,23 +453,39 @@ __global__ __launch_bounds__(kThreads) void k2_fold_kernel(const char* __restric
         for (int k = 0; k < kWorld; ++k)
           if (dp[k]) reinterpret_cast<T*>(dp[k])[i] = Elem<T>::narrow(acc);
       }
-    } else {
-      const int64_t e0 = t * kTileElems + threadIdx.x;
-      for (int k2 = 0; k2 < kUnroll * L; ++k2) {
-        const int64_t i = e0 + static_cast<int64_t>(k2) * kThreads;
-        if (i < n) {
-          A acc = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[0])[i]), dv.divisor, dv.reciprocal);
-#pragma unroll
-          for (int k = 1; k < kWorld; ++k) {
-            const A y = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[k])[i]), dv.divisor, dv.reciprocal);
-            acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
-          }
-#pragma unroll
-          for (int k = 0; k < kWorld; ++k)
-            if (dp[k]) reinterpret_cast<T*>(dp[k])[i] = Elem<T>::narrow(acc);
-        }
-      }
     }
+  }
+}
+
+// Table in device memory (many segments: DDP's buckets).
+template <typename T, int kWorld, int kDiv>
+__global__ __launch_bounds__(kThreads) void k2_fold_kernel(const char* __restrict__ image, Divisor<T> dv) {
+  const FoldHeader* hd = reinterpret_cast<const FoldHeader*>(image);
+  const int nseg = hd->nseg;
+  const int64_t* tile_end = reinterpret_cast<const int64_t*>(image + fold_tile_end_offset());
+  const FoldSegDev* segs = reinterpret_cast<const FoldSegDev*>(image + fold_segs_offset(nseg));
+  const int32_t* tile_seg = reinterpret_cast<const int32_t*>(image + fold_tile_seg_offset(nseg));
+  const int64_t total = hd->total_tiles;
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    const int lo = tile_seg[tile];  // one lookup, then the loads can go out
+    fold_tile<T, kWorld, kDiv>(segs[lo], tile - (lo ? tile_end[lo - 1] : 0), dv);
+  }
+}
+
+// Table by value (one segment per ring chunk: a whole all-reduce in one launch).
+struct FoldSmall {
+  int nseg;
+  int64_t tile_end[TDM_MAX_WORLD];
+  FoldSegDev seg[TDM_MAX_WORLD];
+};
+
+template <typename T, int kWorld, int kDiv>
+__global__ __launch_bounds__(kThreads) void k2_fold_small_kernel(FoldSmall tab, Divisor<T> dv) {
+  const int64_t total = tab.tile_end[tab.nseg - 1];
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    int lo = 0;
+    while (tile >= tab.tile_end[lo]) ++lo;
+    fold_tile<T, kWorld, kDiv>(tab.seg[lo], tile - (lo ? tab.tile_end[lo - 1] : 0), dv);
   }
 }
 
@@ -651,6 +678,31 @@ void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t st
   }
 }
 
+template <typename T, int kWorld>
+void launch_fold_small_w(const FoldSmall& tab, int average, hipStream_t stream) {
+  const Divisor<T> dv = make_divisor<T>(kWorld);
+  const dim3 grid(grid_for(tab.tile_end[tab.nseg - 1])), block(kThreads);
+  switch (div_kind(kWorld, average != 0)) {
+    case 0: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0>), grid, block, 0, stream, tab, dv); break;
+    case 1: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1>), grid, block, 0, stream, tab, dv); break;
+    default: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2>), grid, block, 0, stream, tab, dv); break;
+  }
+}
+
+template <typename T>
+void launch_fold_small(const FoldSmall& tab, int world, int average, hipStream_t stream) {
+  switch (world) {
+    case 2: launch_fold_small_w<T, 2>(tab, average, stream); break;
+    case 3: launch_fold_small_w<T, 3>(tab, average, stream); break;
+    case 4: launch_fold_small_w<T, 4>(tab, average, stream); break;
+    case 5: launch_fold_small_w<T, 5>(tab, average, stream); break;
+    case 6: launch_fold_small_w<T, 6>(tab, average, stream); break;
+    case 7: launch_fold_small_w<T, 7>(tab, average, stream); break;
+    case 8: launch_fold_small_w<T, 8>(tab, average, stream); break;
+    default: throw Invalid("the direct fold handles world sizes 2..8");
+  }
+}
+
 template <typename T>
 void launch_fold(const void* image, int64_t tiles, int world, int average, hipStream_t stream) {
   switch (world) {
@@ -723,11 +775,172 @@ void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStrea
   check_hip(hipGetLastError(), "k1_copy launch");
 }
 
+// ---------------------------------------------------------------- a whole group in one process
+// Rank r is bufs[r]; a ring step is ONE launch carrying every rank's pair.
+namespace {
+
+struct LocalRanks {
+  std::vector<char*> base;
+  std::vector<int64_t> lo, len;  // chunk bounds, in elements
+  int world, es, dtype;
+};
+
+LocalRanks local_ranks(void* const* bufs, int world, int64_t numel, int dtype, const int64_t* sizes, int nsizes) {
+  LocalRanks lr;
+  lr.es = elem_size(dtype);
+  if (lr.es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
+  if (world < 1 || world > TDM_MAX_PAIRS) throw Invalid("world must be in [1, " + std::to_string(TDM_MAX_PAIRS) + "]");
+  if (numel < 0) throw Invalid("negative element count");
+  if (bufs == nullptr) throw Invalid("NULL rank buffers");
+  lr.world = world;
+  lr.dtype = dtype;
+  for (int r = 0; r < world; ++r) {
+    if (numel > 0 && bufs[r] == nullptr) throw Invalid("rank " + std::to_string(r) + ": NULL buffer");
+    lr.base.push_back(static_cast<char*>(bufs[r]));
+  }
+  for (int a = 0; a < world && numel > 0; ++a)
+    for (int b = a + 1; b < world; ++b) {
+      const uintptr_t x = reinterpret_cast<uintptr_t>(bufs[a]), y = reinterpret_cast<uintptr_t>(bufs[b]);
+      const uintptr_t bytes = static_cast<uintptr_t>(numel) * lr.es;
+      if (x < y + bytes && y < x + bytes) throw Invalid("rank buffers overlap");
+    }
+  lr.lo.resize(world);
+  lr.len.resize(world);
+  if (nsizes == 0) {  // as torch.tensor_split cuts
+    const int64_t base = numel / world, extra = numel % world;
+    int64_t at = 0;
+    for (int q = 0; q < world; ++q) {
+      lr.lo[q] = at;
+      lr.len[q] = base + (q < extra ? 1 : 0);
+      at += lr.len[q];
+    }
+  } else {
+    if (nsizes != world || sizes == nullptr) throw Invalid("chunk sizes do not partition the tensor");
+    int64_t at = 0;
+    for (int q = 0; q < world; ++q) {
+      if (sizes[q] < 0) throw Invalid("chunk sizes do not partition the tensor");
+      lr.lo[q] = at;
+      lr.len[q] = sizes[q];
+      at += sizes[q];
+    }
+    if (at != numel) throw Invalid("chunk sizes do not partition the tensor");
+  }
+  return lr;
+}
+
+int wrap(int a, int n) { return ((a % n) + n) % n; }
+
+// Step s: rank r adds chunk (r-s-2) of rank r-1 into its own (tandem/comm.py:301-305).
+// Every receiving chunk is still undivided; the sender's only on the first step.
+void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hipStream_t stream) {
+  const int n = lr.world;
+  for (int s = 0; s < n - 1; ++s) {
+    tdm_pair pairs[TDM_MAX_PAIRS];
+    int np = 0;
+    for (int r = 0; r < n; ++r) {
+      const int c = wrap(r - s - 2, n);
+      if (lr.len[c] == 0) continue;
+      pairs[np++] = tdm_pair{lr.base[r] + lr.lo[c] * lr.es, lr.base[wrap(r - 1, n)] + lr.lo[c] * lr.es, lr.len[c]};
+    }
+    if (np) reduce_step(pairs, np, lr.dtype, average ? n : 1, true, s == 0, s == 0 && keep_sent, stream);
+  }
+}
+
+// Step s: rank r copies chunk (r-s-1) from rank r-1 (tandem/comm.py:307-311).
+void local_all_gather(const LocalRanks& lr, hipStream_t stream) {
+  const int n = lr.world;
+  for (int s = 0; s < n - 1; ++s) {
+    tdm_pair pairs[TDM_MAX_PAIRS];
+    int np = 0;
+    for (int r = 0; r < n; ++r) {
+      const int c = wrap(r - s - 1, n);
+      if (lr.len[c] == 0) continue;
+      pairs[np++] = tdm_pair{lr.base[r] + lr.lo[c] * lr.es, lr.base[wrap(r - 1, n)] + lr.lo[c] * lr.es, lr.len[c]};
+    }
+    if (np) copy_step(pairs, np, lr.dtype, 0, stream);
+  }
+}
+
+// The whole all-reduce as one launch: every element is read from all ranks,
+// folded in the ring's order for its chunk and written to all ranks.
+void local_all_reduce_fold(const LocalRanks& lr, bool average, hipStream_t stream) {
+  const int n = lr.world;
+  FoldSmall tab;
+  std::memset(&tab, 0, sizeof tab);
+  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / lr.es);
+  int64_t tiles = 0;
+  int k = 0;
+  for (int c = 0; c < n; ++c) {
+    if (lr.len[c] == 0) continue;
+    bool vec = true;
+    for (int r = 0; r < n; ++r) {
+      char* p = lr.base[r] + lr.lo[c] * lr.es;
+      tab.seg[k].src[r] = p;
+      tab.seg[k].dst[r] = p;
+      vec = vec && reinterpret_cast<uintptr_t>(p) % 16 == 0;
+    }
+    tab.seg[k].count = lr.len[c];
+    tab.seg[k].chunk = c;
+    tab.seg[k].vec_ok = vec;
+    tiles += (lr.len[c] + tile_elems - 1) / tile_elems;
+    tab.tile_end[k] = tiles;
+    ++k;
+  }
+  tab.nseg = k;
+  if (k == 0) return;
+  switch (lr.dtype) {
+    case TDM_F32: launch_fold_small<float>(tab, n, average, stream); break;
+    case TDM_F64: launch_fold_small<double>(tab, n, average, stream); break;
+    case TDM_F16: launch_fold_small<f16_t>(tab, n, average, stream); break;
+    case TDM_BF16: launch_fold_small<bf16_t>(tab, n, average, stream); break;
+    case TDM_I64: launch_fold_small<int64_t>(tab, n, 0, stream); break;
+    default: launch_fold_small<int32_t>(tab, n, 0, stream); break;
+  }
+  check_hip(hipGetLastError(), "k2_fold_small launch");
+}
+
+}  // namespace
+
 }  // namespace tandem_hip
 
 using namespace tandem_hip;
 
 extern "C" {
+
+int tdm_local_reduce_scatter(void* const* bufs, int world, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
+                             int average, int keep_sent, tdm_stream stream) {
+  return guard([&] {
+    if (average && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
+    const LocalRanks lr = local_ranks(bufs, world, numel, dtype, sizes, nsizes);
+    if (world > 1) local_reduce_scatter(lr, average != 0, keep_sent != 0, static_cast<hipStream_t>(stream));
+  });
+}
+
+int tdm_local_all_gather(void* const* bufs, int world, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
+                         tdm_stream stream) {
+  return guard([&] {
+    const LocalRanks lr = local_ranks(bufs, world, numel, dtype, sizes, nsizes);
+    if (world > 1) local_all_gather(lr, static_cast<hipStream_t>(stream));
+  });
+}
+
+int tdm_local_all_reduce(void* const* bufs, int world, int64_t numel, int dtype, int average, int algorithm,
+                         tdm_stream stream) {
+  return guard([&] {
+    if (average && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
+    if (algorithm != TDM_ALLREDUCE_RING && algorithm != TDM_ALLREDUCE_FOLD) throw Invalid("unknown all-reduce algorithm");
+    const LocalRanks lr = local_ranks(bufs, world, numel, dtype, nullptr, 0);
+    if (world == 1) return;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (algorithm == TDM_ALLREDUCE_FOLD) {
+      if (world > TDM_MAX_WORLD) throw Invalid("the direct fold handles world sizes up to 8");
+      local_all_reduce_fold(lr, average != 0, st);
+    } else {
+      local_reduce_scatter(lr, average != 0, false, st);
+      local_all_gather(lr, st);
+    }
+  });
+}
 
 int tdm_set_blocks_per_cu(int blocks) {
   return guard([&] {
@@ -748,9 +961,19 @@ int tdm_k1_copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, td
   return guard([&] { copy_step(pairs, npairs, dtype, world, static_cast<hipStream_t>(stream)); });
 }
 
-int64_t tdm_k2_table_bytes(int nseg) {
-  if (nseg < 0) return 0;
-  return fold_segs_offset(nseg) + static_cast<int64_t>(nseg) * static_cast<int64_t>(sizeof(FoldSegDev));
+namespace {
+int64_t fold_tiles(const tdm_fold_seg* segs, int nseg, int es) {
+  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
+  int64_t tiles = 0;
+  for (int i = 0; i < nseg; ++i) tiles += segs[i].count > 0 ? (segs[i].count + tile_elems - 1) / tile_elems : 0;
+  return tiles;
+}
+}  // namespace
+
+int64_t tdm_k2_table_bytes(const tdm_fold_seg* segs, int nseg, int dtype) {
+  const int es = elem_size(dtype);
+  if (nseg < 0 || es == 0 || (nseg > 0 && segs == nullptr)) return -1;
+  return (fold_tile_seg_offset(nseg) + fold_tiles(segs, nseg, es) * 4 + 15) / 16 * 16;
 }
 
 int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype, void* image) {
@@ -760,7 +983,8 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
     if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
     if (nseg < 0 || (nseg > 0 && segs == nullptr) || image == nullptr) throw Invalid("bad table arguments");
     char* img = static_cast<char*>(image);
-    std::memset(img, 0, static_cast<size_t>(tdm_k2_table_bytes(nseg)));
+    std::memset(img, 0, static_cast<size_t>(tdm_k2_table_bytes(segs, nseg, dtype)));
+    int32_t* tile_seg = reinterpret_cast<int32_t*>(img + fold_tile_seg_offset(nseg));
     FoldHeader* hd = reinterpret_cast<FoldHeader*>(img);
     int64_t* tile_end = reinterpret_cast<int64_t*>(img + fold_tile_end_offset());
     FoldSegDev* out = reinterpret_cast<FoldSegDev*>(img + fold_segs_offset(nseg));
@@ -782,7 +1006,9 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
       out[i].count = s.count;
       out[i].chunk = s.chunk;
       out[i].vec_ok = vec;
-      tiles += (s.count + tile_elems - 1) / tile_elems;
+      const int64_t mine = (s.count + tile_elems - 1) / tile_elems;
+      for (int64_t t = 0; t < mine; ++t) tile_seg[tiles + t] = i;
+      tiles += mine;
       tile_end[i] = tiles;
     }
     hd->magic = kFoldMagic;

@@ -4,7 +4,7 @@
 tensors (one per rank) with ONE kernel launch per ring step: the launch carries
 every rank's (receive chunk, neighbour's chunk) pair, so a step that the
 reference runs as `world` processes x pieces x (copy into a slot, add out of
-it) is a single fused pass over HBM. The results, including the partial sums a
+it) is a single fused pass over HBM (an all-reduce can even be one launch). The results, including the partial sums a
 bare reduce_scatter leaves in the other chunks, are bit for bit those of the
 reference's Python engine (tandem/comm.py:301-385 there).
 
@@ -77,71 +77,55 @@ class LocalWorld:
             raise ValueError(f"unknown op {op}")
         return op == "avg"
 
-    # ---- ring steps: one launch each
-    def _reduce_scatter(self, flats, bounds, average, keep_sent):
-        n = self.world
-        es = flats[0].element_size()
-        code = dtype_code(flats[0].dtype)
-        base = [f.data_ptr() for f in flats]
-        st = stream_ptr(flats[0].device)
-        for s in range(n - 1):
-            items = []
-            for r in range(n):
-                lo, hi = bounds[(r - s - 2) % n]  # rank r adds what rank r-1 sends (tandem/comm.py:305)
-                if hi > lo:
-                    items.append((base[r] + lo * es, base[(r - 1) % n] + lo * es, hi - lo))
-            if items:
-                # Every receiving chunk is still undivided; the sender's is only on the
-                # first step. keep_sent: the first step also leaves x / n in the sender's
-                # chunk, which div_ of the whole tensor would have (a bare reduce_scatter
-                # shows it; an all_reduce overwrites it anyway).
-                check(lib().tdm_k1_reduce_step(_pairs(items), len(items), code, n if average else 1,
-                                               1, int(s == 0), int(s == 0 and keep_sent), st))
-
-    def _all_gather(self, flats, bounds):
-        n = self.world
-        es = flats[0].element_size()
-        code = dtype_code(flats[0].dtype)
-        base = [f.data_ptr() for f in flats]
-        st = stream_ptr(flats[0].device)
-        for s in range(n - 1):
-            items = []
-            for r in range(n):
-                lo, hi = bounds[(r - s - 1) % n]  # tandem/comm.py:311
-                if hi > lo:
-                    items.append((base[r] + lo * es, base[(r - 1) % n] + lo * es, hi - lo))
-            if items:
-                check(lib().tdm_k1_copy_step(_pairs(items), len(items), code, 0, st))
-
     # ---- collectives over all ranks at once
+    @staticmethod
+    def _ptrs(flats):
+        return (ctypes.c_void_p * len(flats))(*[f.data_ptr() for f in flats])
+
+    @staticmethod
+    def _sizes(bounds, given):
+        if given is None:
+            return (ctypes.c_int64 * 1)(), 0
+        return (ctypes.c_int64 * len(bounds))(*[hi - lo for lo, hi in bounds]), len(bounds)
+
     def reduce_scatter(self, bufs, sizes=None, op="sum"):
         """In place on every rank's buffer; returns each rank's reduced chunk
-        (a view), as Group.reduce_scatter does per rank (tandem/comm.py:349-369)."""
+        (a view), as Group.reduce_scatter does per rank (tandem/comm.py:349-369).
+        One launch per ring step; the other chunks are left holding the same
+        partial sums as in the reference."""
         average = self._op(op)
         flats = self._flat(bufs, "reduce_scatter")
         bounds = chunk_bounds(flats[0].numel(), self.world, sizes)
-        if self.world > 1:
-            self._reduce_scatter(flats, bounds, average, True)
+        arr, n = self._sizes(bounds, sizes)
+        check(lib().tdm_local_reduce_scatter(self._ptrs(flats), self.world, flats[0].numel(), dtype_code(flats[0].dtype),
+                                             arr, n, int(average), 1, stream_ptr(flats[0].device)))
         return [flats[r][bounds[r][0]:bounds[r][1]] for r in range(self.world)]
 
     def all_gather(self, bufs, sizes=None):
         """Rank r holds chunk r; afterwards every rank holds every chunk
-        (tandem/comm.py:371-385)."""
+        (tandem/comm.py:371-385). One launch per ring step."""
         flats = self._flat(bufs, "all_gather")
         bounds = chunk_bounds(flats[0].numel(), self.world, sizes)
-        if self.world > 1:
-            self._all_gather(flats, bounds)
+        arr, n = self._sizes(bounds, sizes)
+        check(lib().tdm_local_all_gather(self._ptrs(flats), self.world, flats[0].numel(), dtype_code(flats[0].dtype),
+                                         arr, n, stream_ptr(flats[0].device)))
         return bufs
 
-    def all_reduce(self, bufs, op="sum"):
-        """Ring all-reduce in place: reduce-scatter then all-gather over the
-        tensor_split chunks (tandem/comm.py:326-347)."""
+    def all_reduce(self, bufs, op="sum", algorithm=None):
+        """All-reduce in place (tandem/comm.py:326-347). algorithm="ring": the
+        reduce-scatter then the all-gather, one launch per step. algorithm="fold"
+        (the default up to 8 ranks): one launch that reads every rank's element,
+        sums in the ring's order for the element's chunk and writes every rank;
+        the same bits with about half the HBM traffic."""
         average = self._op(op)
         flats = self._flat(bufs, "all_reduce")
-        if self.world > 1:
-            bounds = chunk_bounds(flats[0].numel(), self.world, None)
-            self._reduce_scatter(flats, bounds, average, False)
-            self._all_gather(flats, bounds)
+        if algorithm is None:
+            algorithm = "fold" if self.world <= _lib.TDM_MAX_WORLD else "ring"
+        if algorithm not in ("ring", "fold"):
+            raise ValueError(f"unknown all-reduce algorithm {algorithm}")
+        code = _lib.ALLREDUCE_FOLD if algorithm == "fold" else _lib.ALLREDUCE_RING
+        check(lib().tdm_local_all_reduce(self._ptrs(flats), self.world, flats[0].numel(), dtype_code(flats[0].dtype),
+                                         int(average), code, stream_ptr(flats[0].device)))
         return bufs
 
     def unit_gather(self, fulls, shards, sizes):
@@ -208,7 +192,9 @@ class FoldTable:
                 segs[k].src[r] = tensors_per_rank[r][i].data_ptr() + off * es
                 segs[k].dst[r] = outs[r][i].data_ptr() + off * es
             segs[k].count, segs[k].chunk = count, chunk
-        nbytes = lib().tdm_k2_table_bytes(self.nseg)
+        nbytes = lib().tdm_k2_table_bytes(segs, self.nseg, dtype_code(self.dtype))
+        if nbytes < 0:
+            raise ValueError("bucket_table: bad segment table")
         image = torch.empty(max(16, nbytes), dtype=torch.uint8)
         check(lib().tdm_k2_table_build(segs, self.nseg, world, dtype_code(self.dtype), ctypes.c_void_p(image.data_ptr())))
         self.image = image.to(self.device)
@@ -216,3 +202,71 @@ class FoldTable:
     def run(self, average=True):
         check(lib().tdm_k2_bucket_fold(ctypes.c_void_p(self.image.data_ptr()), self.nseg, dtype_code(self.dtype),
                                        self.world, int(average), stream_ptr(self.device)))
+
+
+class LocalZeRO2:
+    """ZeRO stage 2's communication and optimizer step for a whole group on one
+    GPU: rank r owns bufs[r] (all parameters, flat), staging[r] (its gradients,
+    flat, in registration order), grad_shards[r] and its own optimizer state.
+
+    reduce_grads() is what ZeRO._on_grad/_after_backward do with the buckets
+    (tandem/zero.py:119-156 in the reference): every bucket [a, b) is
+    reduce-scattered (avg) with chunk sizes bucket_sizes(a, b) and each rank adds
+    its chunk into its gradient shard. Buckets are independent, so ring step s of
+    all of them travels in as few launches as the 16-pair limit allows.
+    step() is ZeRO.step (tandem/zero.py:158-163): sharded AdamW on every rank's
+    shard, then the all-gather of the flat parameter buffer."""
+
+    def __init__(self, world, numels, device, bucket_bytes=25 << 20, order="host", **adamw):
+        from .buckets import FlatLayout, zero_buckets
+        from .optim import ShardedAdamW
+
+        self.lw = LocalWorld(world)
+        self.world = world
+        self.layouts = [FlatLayout(numels, world, r) for r in range(world)]
+        n = self.layouts[0].numel
+        self.numel = n
+        self.buckets = zero_buckets(list(numels), 4, bucket_bytes)
+        self.bufs = [torch.zeros(n, device=device) for _ in range(world)]
+        self.staging = [torch.zeros(n, device=device) for _ in range(world)]
+        self.grad_shards = [torch.zeros(l.hi - l.lo, device=device) for l in self.layouts]
+        self.opts = [ShardedAdamW(order=order, **adamw) for _ in range(world)]
+        self.device = torch.device(device)
+        # ring step s of every bucket: (dst, src, count) pairs, and the final adds
+        es = 4
+        self._steps = [[] for _ in range(world - 1)]
+        self._adds = []
+        sb = [t.data_ptr() for t in self.staging]
+        for a, b, _ in self.buckets:
+            sizes = self.layouts[0].bucket_sizes(a, b)
+            lo = a
+            for c, m in enumerate(sizes):
+                if m:
+                    for s in range(world - 1):
+                        r = (c + s + 2) % world  # the rank that receives chunk c on step s
+                        self._steps[s].append((sb[r] + lo * es, sb[(r - 1) % world] + lo * es, m))
+                    shard_at = lo - self.layouts[c].lo
+                    self._adds.append((self.grad_shards[c].data_ptr() + shard_at * es, sb[c] + lo * es, m))
+                lo += m
+
+    def _launch(self, items, scale_dst, scale_src, writeback):
+        st = stream_ptr(self.device)
+        for k in range(0, len(items), _lib.TDM_MAX_PAIRS):
+            part = items[k:k + _lib.TDM_MAX_PAIRS]
+            check(lib().tdm_k1_reduce_step(_pairs(part), len(part), 0, self.world if scale_dst else 1,
+                                           int(scale_dst), int(scale_src), int(writeback), st))
+
+    def reduce_grads(self):
+        for s, items in enumerate(self._steps):
+            self._launch(items, True, s == 0, s == 0)
+        self._launch(self._adds, False, False, False)  # grad_shard += mine (add_, so -0.0 + 0.0 = +0.0 as in the reference)
+
+    def step(self):
+        for r in range(self.world):
+            l = self.layouts[r]
+            self.opts[r].update("flat", self.bufs[r][l.lo:l.hi], self.grad_shards[r])
+        self.lw.all_gather(self.bufs, self.layouts[0].sizes)
+
+    def zero_grad(self):
+        for g in self.grad_shards:
+            g.zero_()

@@ -44,7 +44,10 @@ def test_argument_errors_need_no_gpu():
     assert L.tdm_k1_reduce_step(None, 17, 0, 2, 1, 1, 0, None) == 1
     assert b"npairs" in L.tdm_last_error()
     assert L.tdm_k1_copy_step(None, 0, 99, 0, None) == 1
-    assert L.tdm_k2_table_bytes(0) > 0 and L.tdm_k2_table_bytes(3) > L.tdm_k2_table_bytes(2)
+    segs = (_lib.FoldSeg * 2)()
+    segs[0].count, segs[1].count = 5, 5000
+    assert L.tdm_k2_table_bytes(segs, 0, 0) > 0 and L.tdm_k2_table_bytes(segs, 2, 0) > L.tdm_k2_table_bytes(segs, 1, 0)
+    assert L.tdm_k2_table_bytes(segs, 2, 99) == -1
     assert L.tdm_set_blocks_per_cu(5000) == 1
     assert L.tdm_set_blocks_per_cu(0) == 0
 

@@ -59,10 +59,11 @@ def test_fixtures_of_the_reference_engine(dev, world):
         return [torch.from_numpy(x.copy()).to(dev) for x in xs]
 
     for op, key in (("sum", "ar_sum"), ("avg", "ar_avg")):
-        bufs = fresh()
-        lw.all_reduce(bufs, op=op)
-        for r in range(world):
-            assert np.array_equal(bits(to_np(bufs[r])), bits(d[f"r{r}_{key}"])), (key, r)
+        for algorithm in ("ring", "fold"):
+            bufs = fresh()
+            lw.all_reduce(bufs, op=op, algorithm=algorithm)
+            for r in range(world):
+                assert np.array_equal(bits(to_np(bufs[r])), bits(d[f"r{r}_{key}"])), (key, algorithm, r)
     bufs = fresh()
     lw.reduce_scatter(bufs, None, op="avg")
     for r in range(world):
@@ -116,11 +117,12 @@ def test_against_oracle(dev, world, dtype):
         xn = [to_np(x) for x in xs]
         ops = ("sum",) if dtype == torch.int64 else ("sum", "avg")
         for op in ops:
-            bufs = [x.to(dev) for x in xs]
-            lw.all_reduce(bufs, op=op)
             want = ring.expected_all_reduce(xn, op == "avg", kind)
-            for r in range(world):
-                assert np.array_equal(bits(to_np(bufs[r])), bits(want)), (world, dtype, n, op, r)
+            for algorithm in ("ring", "fold"):
+                bufs = [x.to(dev) for x in xs]
+                lw.all_reduce(bufs, op=op, algorithm=algorithm)
+                for r in range(world):
+                    assert np.array_equal(bits(to_np(bufs[r])), bits(want)), (world, dtype, n, op, algorithm, r)
             sizes = [n // world] * world
             sizes[-1] += n - sum(sizes)
             sizes = sizes[1:] + sizes[:1]  # uneven, and empty when n < world
@@ -159,7 +161,7 @@ def test_unaligned_views_and_special_values(dev):
             bufs = [store[r][shifts[r]:shifts[r] + n] for r in range(world)]
             for b, x in zip(bufs, xs):
                 b.copy_(x)
-            lw.all_reduce(bufs, op=op)
+            lw.all_reduce(bufs, op=op, algorithm="ring" if shifts[0] else "fold")
             want = ring.expected_all_reduce(xn, op == "avg")
             for r in range(world):
                 got = to_np(bufs[r])
@@ -226,7 +228,11 @@ def test_full_size_properties(dev):
     gens = [torch.Generator(device=dev).manual_seed(10 + r) for r in range(world)]
     xs = [torch.randn(n, device=dev, generator=g) * 1e-2 for g in gens]
     bufs = [x.clone() for x in xs]
-    lw.all_reduce(bufs, op="avg")
+    lw.all_reduce(bufs, op="avg", algorithm="ring")
+    folded = [x.clone() for x in xs]
+    lw.all_reduce(folded, op="avg", algorithm="fold")
+    assert torch.equal(bufs[3].view(torch.int32), folded[1].view(torch.int32))  # one launch, same bits
+    del folded
     for r in range(1, world):
         assert torch.equal(bufs[0].view(torch.int32), bufs[r].view(torch.int32))
     scaled = [x * 16.0 for x in xs]
