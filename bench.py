@@ -1,18 +1,30 @@
-"""Benchmark of the data-parallel reduction hot path on one MI355X.
+"""Benchmark of tandem's data-parallel reduction hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mib 256] [--no-sweep] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mib 256] [--quick] [--no-cpu] [--no-fsdp]
 
 A step is one ring reduce-scatter (avg) + all-gather over four rank buffers of
-`--mib` MiB fp32 each, all resident in one GPU's HBM (world size 4 on one GPU,
-4 MiB ring slots as the sweep unit of the kernel's grid). Prints ONE JSON line:
-whole-job algorithmic HBM throughput of the step, the roofline of the dominant
-kernel (the fused ring-step reduce) measured with HIP events inside the timed
-region, a size sweep, the ZeRO-2 step time at 85.8M parameters, and the CPU
-baseline (the oracle's CPU-process engine on this box's host cores).
+`--mib` MiB fp32 each, all resident in one GPU's HBM before the timed region
+starts (world size 4 on one GPU). Prints ONE JSON line:
+
+  value       algorithmic HBM bytes of the step (15 x message bytes) / step time
+  roofline    the dominant kernel, the fused ring-step reduce (K1): 12 bytes per
+              element per launch / the launch's duration, taken from HIP events
+              recorded around the three back-to-back K1 launches of every timed
+              step, against the 8 TB/s HBM peak; `traffic` is the HBM traffic per
+              launch measured with rocprofv3 counters (profiles/)
+  sweep       message sizes 64 KiB .. 256 MiB, ring and single-launch fold
+  bucket_path DDP's bucket flatten+average+unflatten (K2), 85.8M params, world 2
+  zero2_step  reduce-scatter + AdamW + all-gather, 85.8M params, world 4
+  fsdp_gather two processes sharing the GPU through HIP IPC: ZeRO-3 unit gathers
+              of the 85.8M GPT, prefetched on the engine's stream
+  cpu_baseline  the oracle's CPU-process engine (tandem's Python-engine protocol:
+              one process per rank, 1 torch thread each, 2 x 4 MiB shared-memory
+              slots per pair) on this box's host cores, same formula for GB/s
 """
 
 import argparse
 import json
+import math
 import os
 import statistics
 import sys
@@ -23,6 +35,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X, published
 WORLD = 4
+# HBM bytes per K1 launch at the default workload (4 chunk pairs of 64 MiB), from
+# rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads for
+# the plain copy kernel of known size in the same run (profiles/k1_reduce_*.txt).
+K1_TRAFFIC_256MIB = 805_279_000
 
 
 def seeded_grads(world, n, dev, scale):
@@ -35,14 +51,29 @@ def seeded_grads(world, n, dev, scale):
     return out
 
 
-def ring_pass(lw, bufs, events=None):
-    """One step: reduce-scatter (avg) then all-gather, the two halves bracketed by
+def timed(fn, reps, warm=3):
+    """Mean seconds per call, by HIP events on the launch stream."""
+    import torch
+
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / reps
+
+
+def ring_pass(lw, flats, events=None):
+    """One step: reduce-scatter (avg) then all-gather; the two halves bracketed by
     events on the launch stream when asked."""
     import torch
 
     from tandem_amd._lib import check, lib, stream_ptr
 
-    flats = [b.reshape(-1) for b in bufs]
     ptrs, n, st = lw._ptrs(flats), flats[0].numel(), stream_ptr(flats[0].device)
     none = lw._sizes(None, None)[0]
     if events is not None:
@@ -60,13 +91,14 @@ def ring_pass(lw, bufs, events=None):
 def time_ring(lw, bufs, steps, warmup):
     import torch
 
+    flats = [b.reshape(-1) for b in bufs]
     for _ in range(warmup):
-        ring_pass(lw, bufs)
+        ring_pass(lw, flats)
     events = []
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        ring_pass(lw, bufs, events)
+        ring_pass(lw, flats, events)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     rs_ms = sum(e[0].elapsed_time(e[1]) for e in events)
@@ -75,39 +107,187 @@ def time_ring(lw, bufs, steps, warmup):
 
 
 def sweep(lw, dev, steps):
-    """Per-rank message sizes 64 KiB ... 256 MiB; algorithmic bytes 15*B per pass."""
+    """Per-rank message sizes 64 KiB ... 256 MiB. Ring: algorithmic bytes 15 B per
+    pass. Fold: the same all-reduce as one launch, 8 W B = 32 B... per pass."""
     import torch
 
     rows = []
     for kib in (64, 1024, 4096, 16384, 65536, 262144):
         n = kib * 1024 // 4
         bufs = seeded_grads(WORLD, n, dev, 1e-2)
-        reps = max(steps, 20 if kib <= 16384 else steps)
+        reps = steps if kib >= 65536 else max(steps, 30)
         per, rs, ag = time_ring(lw, bufs, reps, 3)
+        fold = timed(lambda: lw.all_reduce(bufs, "avg", algorithm="fold"), reps)
         b = n * 4
-        rows.append({"MiB": kib / 1024, "ms": round(per * 1e3, 4), "GBps": round(15 * b / per / 1e9, 1),
-                     "algbw_GBps": round(b / per / 1e9, 1), "k1_frac_of_hbm": round(12 * n * (WORLD - 1) / (rs * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)})
+        rows.append({"MiB": kib / 1024, "ring_ms": round(per * 1e3, 4), "ring_GBps": round(15 * b / per / 1e9, 1),
+                     "ring_algbw_GBps": round(b / per / 1e9, 1),
+                     "k1_frac_of_hbm": round(12 * n * (WORLD - 1) / (rs * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "fold_ms": round(fold * 1e3, 4), "fold_GBps": round(8 * WORLD * b / fold / 1e9, 1),
+                     "fold_algbw_GBps": round(b / fold / 1e9, 1)})
         del bufs
         torch.cuda.empty_cache()
     return rows
 
 
-def cpu_baseline(n_elems):
-    """The oracle's closed-form ring fold in plain C on one host core, over a
-    bounded sample of the same workload (world 4, N(0, 1e-2))."""
-    import numpy as np
+def gpt_numels():
+    import torch
 
-    from oracle import ring
+    from tandem_amd.model import GPT, Config
 
-    rng = np.random.default_rng(0)
-    xs = [(rng.standard_normal(n_elems) * 1e-2).astype(np.float32) for _ in range(WORLD)]
-    ring.expected_all_reduce([x[:1024] for x in xs], True)  # load the library
+    with torch.device("meta"):
+        m = GPT(Config.preset("medium"))
+    return [p.numel() for p in m.parameters()]
+
+
+def bucket_path(dev, reps):
+    """DDP's bucket path with both ranks on the GPU: 149 gradients per rank, 16
+    buckets of up to 25 MiB in reverse registration order, averaged in place."""
+    import torch
+
+    from tandem_amd import LocalWorld
+    from tandem_amd.buckets import pack
+
+    numels = gpt_numels()
+    n = sum(numels)
+    order = list(range(len(numels)))[::-1]
+    buckets = [[order[k] for k in g] for g in pack([numels[i] * 4 for i in order], 25 << 20)]
+    world = 2
+    grads = []
+    for r in range(world):
+        gen = torch.Generator(device=dev).manual_seed(100 + r)
+        grads.append([torch.randn(m, device=dev, generator=gen) * 1e-3 for m in numels])
+    table = LocalWorld(world).bucket_table(grads, buckets)
+    t = timed(lambda: table.run(True), reps)
+    nbytes = 8 * world * n
+    return {"workload": "149 grads x 2 ranks, 85,842,432 fp32 params, 16 buckets of <= 25 MiB, one launch", "ms": round(t * 1e3, 4),
+            "algorithmic_bytes": nbytes, "GBps": round(nbytes / t / 1e9, 1), "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4),
+            "segments": table.nseg}
+
+
+def zero2_step(dev, reps):
+    """ZeRO-2's reduce-scatter + AdamW + all-gather for the 85.8M GPT, world 4 on
+    one GPU, all four shards stepped."""
+    import torch
+
+    from tandem_amd.local import LocalZeRO2
+
+    numels = gpt_numels()
+    n = sum(numels)
+    z = LocalZeRO2(WORLD, numels, dev, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    gen = torch.Generator(device=dev).manual_seed(7)
+    p0 = torch.randn(n, device=dev, generator=gen) * 0.02
+    grads = [torch.randn(n, device=dev, generator=gen) * 1e-3 for _ in range(WORLD)]
+    for b in z.bufs:
+        b.copy_(p0)
+
+    def refill():
+        for r in range(WORLD):
+            z.staging[r].copy_(grads[r])
+        z.zero_grad()
+
+    def whole():
+        z.reduce_grads()
+        z.step()
+
+    # the refill (fresh gradients) is outside the timed region: time it alone and subtract
+    t_refill = timed(refill, reps)
+    t_all = timed(lambda: (refill(), whole()), reps)
+    t_rs = timed(lambda: (refill(), z.reduce_grads()), reps) - t_refill
+    step = t_all - t_refill
+    opt = timed(lambda: [z.opts[r].update("bench", z.bufs[r][z.layouts[r].lo:z.layouts[r].hi], z.grad_shards[r]) for r in range(WORLD)], reps)
+    shard = z.layouts[0].hi - z.layouts[0].lo
+    nbytes = 12 * (WORLD - 1) * n + 12 * n + 28 * n + 8 * (WORLD - 1) * n
+    return {"workload": "85,842,432 fp32 params, world 4 on one GPU, 16 buckets, AdamW(3e-4, (0.9, 0.95), 1e-8, 0.1) on all 4 shards",
+            "ms": round(step * 1e3, 4), "reduce_scatter_ms": round(t_rs * 1e3, 4), "adamw_4_shards_ms": round(opt * 1e3, 4),
+            "adamw_GBps": round(28 * shard * WORLD / opt / 1e9, 1), "adamw_frac_of_hbm_peak": round(28 * shard * WORLD / opt / 1e9 / HBM_PEAK_GBPS, 4),
+            "algorithmic_bytes": nbytes, "GBps": round(nbytes / step / 1e9, 1), "roofline_floor_ms": round(nbytes / (HBM_PEAK_GBPS * 1e9) * 1e3, 4)}
+
+
+# ---------------------------------------------------------------- two processes, HIP IPC
+def fsdp_rank(g, steps, prefetch):
+    import torch
+
+    from tandem_amd import ShardedAdamW
+    from tandem_amd.data import synthetic
+    from tandem_amd.model import GPT, Config
+    from tandem_amd.zero import FSDP
+
+    cfg = Config.preset("medium")
+    torch.manual_seed(0)
+    text = synthetic(100_000)
+    model = GPT(cfg).to(g.device)
+    f = FSDP(model, g, ShardedAdamW(lr=3e-4, betas=(0.9, 0.95), weight_decay=0.1), prefetch=prefetch)
+    times, waits = [], []
+    for step in range(steps + 2):
+        x, y = text.batch(step, 8, cfg.seq, rank=g.rank, world=g.size, device=g.device)
+        g.barrier()
+        torch.cuda.synchronize()
+        g.tracing = True
+        g.waits.clear()
+        g.trace.clear()
+        t0 = time.perf_counter()
+        loss = f(x, y)
+        loss.backward()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        f.step()
+        f.zero_grad()
+        torch.cuda.synchronize()
+        if step >= 2:
+            times.append(t1 - t0)
+            waits.append(sum(b - a for name, a, b in g.waits if name == "gather_unit"))
+    n_gathers = sum(1 for name, *_ in g.trace if name == "gather_unit")
+    return {"fwd_bwd_ms": statistics.median(times) * 1e3, "host_blocked_on_gathers_ms": statistics.median(waits) * 1e3,
+            "gathers_per_step": n_gathers, "max_live": f.max_live, "live": f.live, "loss": float(loss)}
+
+
+def fsdp_gather(steps):
+    from tandem_amd import launch
+
+    out = {}
+    for prefetch in (True, False):
+        res = launch(fsdp_rank, 2, steps, prefetch, slot_bytes=32 << 20, gpus=[0, 0], timeout=120.0)
+        out["prefetch" if prefetch else "no_prefetch"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in res[0].items()}
+    out["workload"] = "2 processes sharing the GPU (HIP IPC memory handles), 85.8M GPT = 14 units (12 blocks of 7,087,872), batch 8x512 split over 2 ranks, 32 MiB slots"
+    return out
+
+
+# ---------------------------------------------------------------- CPU baseline
+def cpu_rank(g, n, reps):
+    import torch
+
+    x = torch.randn(n, generator=torch.Generator().manual_seed(g.rank)) * 1e-2
+    g.all_reduce(x, op="avg")
+    ts = []
+    for _ in range(reps):
+        g.barrier()
+        t = time.perf_counter()
+        g.all_reduce(x, op="avg")
+        ts.append(time.perf_counter() - t)
+    return statistics.median(ts)
+
+
+def cpu_baseline(mib, reps):
+    from oracle.cpu_engine import cpu_launch
+
+    n = mib * (1 << 20) // 4
     t0 = time.perf_counter()
-    ring.expected_all_reduce(xs, True)
-    dt = time.perf_counter() - t0
-    return {"value": round(15 * n_elems * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"world 4 ring all-reduce (avg) of {n_elems * 4 >> 20} MiB fp32 per rank, closed-form fold in C, one pass, {dt:.2f} s",
-            "host_cores": os.cpu_count()}
+    t = max(cpu_launch(cpu_rank, WORLD, n, reps))
+    total = time.perf_counter() - t0
+    return {"value": round(15 * n * 4 / t / 1e9, 3), "unit": "GB/s", "cores": WORLD, "kind": "port",
+            "sample": f"oracle CPU-process engine (tandem's Python-engine protocol): ring all-reduce(avg), world 4 x 1 torch thread, "
+                      f"{mib} MiB fp32 per rank, 2 x 4 MiB shared-memory slots per pair, median of {reps}; {t * 1e3:.1f} ms per all-reduce, "
+                      f"{total:.1f} s including process start",
+            "algbw_GBps": round(n * 4 / t / 1e9, 3), "host_cores": os.cpu_count()}
+
+
+def device_name(_lib):
+    import ctypes
+
+    buf = ctypes.create_string_buffer(128)
+    cus, mem = ctypes.c_int(0), ctypes.c_int64(0)
+    _lib.check(_lib.lib().tdm_device_info(0, buf, 128, ctypes.byref(cus), ctypes.byref(mem)))
+    return f"{buf.value.decode()} ({cus.value} CUs, {mem.value >> 30} GiB)"
 
 
 def main():
@@ -116,18 +296,30 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--mib", type=int, default=256)
-    ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--quick", action="store_true", help="only the main workload (for profiling runs)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-fsdp", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: every rank of the group is a buffer in that GPU's HBM; run with --gpus 1")
+        sys.exit("bench.py measures one GPU: every rank of the group is a buffer in that GPU's HBM, or a process sharing it; "
+                 "run with --gpus 1")
+
+    # The two multi-process figures first, while this process has not touched the GPU.
+    cpu = fsdp = None
+    if not args.quick and not args.no_cpu:
+        cpu = cpu_baseline(64, 7)
+    if not args.quick and not args.no_fsdp:
+        try:
+            fsdp = fsdp_gather(3)
+        except Exception as e:  # a secondary figure must not lose the line
+            fsdp = {"error": repr(e)[:300]}
 
     import torch
 
     from tandem_amd import LocalWorld, _lib
 
     if not torch.cuda.is_available():
-        sys.exit("bench.py needs the MI355X (no CPU path exists)")
+        sys.exit("bench.py needs the MI355X (tandem_amd has no CPU path)")
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     lw = LocalWorld(WORLD)
@@ -136,7 +328,7 @@ def main():
     per, rs_ms, ag_ms = time_ring(lw, bufs, args.steps, args.warmup)
     b = n * 4
     k1_launch_s = rs_ms * 1e-3 / (WORLD - 1)
-    k1_bytes = 12 * n  # one launch: W chunks of n/W elements, two loads and one store each
+    k1_bytes = 12 * n  # one launch: 4 chunk pairs of n/4 elements; two loads and one store of 4 bytes per element
     achieved = k1_bytes / k1_launch_s / 1e9
     line = {
         "metric": "fused-reduce GB/s (ring reduce-scatter+all-gather, world 4 on one GPU)",
@@ -151,32 +343,31 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": f"ring reduce-scatter(avg)+all-gather, world 4 simulated on one MI355X, {args.mib} MiB fp32 per rank, N(0,1e-2) seeded per rank",
+        "config": {"workload": f"ring reduce-scatter(avg)+all-gather, world 4 simulated on one MI355X, {args.mib} MiB fp32 per rank, "
+                               "N(0,1e-2) seeded per rank, inputs resident in HBM",
                    "algorithmic_bytes_per_step": 15 * b, "algbw_GBps": round(b / per / 1e9, 1),
                    "frac_of_hbm_peak": round(15 * b / per / 1e9 / HBM_PEAK_GBPS, 4)},
-        "roofline": {"bound": "hbm", "kernel": "k1_reduce_kernel<float>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+        "roofline": {"bound": "hbm", "kernel": "k1_reduce_kernel<float> (ring-step fused reduce)", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": K1_TRAFFIC_256MIB if args.mib == 256 else None,
                      "bytes_per_launch": k1_bytes, "launch_us": round(k1_launch_s * 1e6, 2),
                      "copy_step_GBps": round(8 * n / (ag_ms * 1e-3 / (WORLD - 1)) / 1e9, 1)},
     }
     del bufs
     torch.cuda.empty_cache()
-    if not args.no_sweep:
+    if not args.quick:
         line["sweep"] = sweep(lw, dev, max(5, args.steps // 2))
-    if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(16 << 20)
-    name = ctypes_device_name(_lib)
-    line["device"] = name
+        line["bucket_path"] = bucket_path(dev, args.steps)
+        torch.cuda.empty_cache()
+        line["zero2_step"] = zero2_step(dev, max(5, args.steps // 2))
+        torch.cuda.empty_cache()
+        if fsdp is not None:
+            line["fsdp_gather"] = fsdp
+        if cpu is not None:
+            cpu["gpu_over_cpu"] = round(line["value"] / cpu["value"], 1)
+            line["cpu_baseline"] = cpu
+    line["device"] = device_name(_lib)
     print(json.dumps(line), flush=True)
-
-
-def ctypes_device_name(_lib):
-    import ctypes
-
-    buf = ctypes.create_string_buffer(128)
-    cus, mem = ctypes.c_int(0), ctypes.c_int64(0)
-    _lib.check(_lib.lib().tdm_device_info(0, buf, 128, ctypes.byref(cus), ctypes.byref(mem)))
-    return f"{buf.value.decode()} ({cus.value} CUs, {mem.value >> 30} GiB)"
 
 
 if __name__ == "__main__":
