@@ -130,11 +130,14 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
 /* For every element of every segment, in one launch:
  *     y_q = average ? src[q][i] / world : src[q][i]
  *     acc = y[(chunk+1) % world];  acc = y[(chunk+k) % world] + acc,  k = 2..world
- *     dst[r][i] = acc  for every rank r
+ *     dst[r][i] = acc  for every rank r with a non-NULL dst   (accumulate: dst[r][i] = dst[r][i] + acc)
  * which is bit for bit what DDP's per-parameter `view.copy_(p.grad)` followed by
  * the bucket's ring all_reduce(op="avg") leaves in every rank's gradient views
- * (tandem/ddp.py:22-33,89-109; ring order tandem/comm.py:301-311). */
-int tdm_k2_bucket_fold(const void* table_dev, int nseg, int dtype, int world, int average, tdm_stream stream);
+ * (tandem/ddp.py:22-33,89-109; ring order tandem/comm.py:301-311). With a dst only for
+ * the chunk's owner and accumulate set, a segment is ZeRO-2's reduce_scatter of that chunk
+ * followed by `grad_shard[...].add_(mine)` (tandem/zero.py:141,150-153). */
+int tdm_k2_bucket_fold(const void* table_dev, int nseg, int dtype, int world, int average, int accumulate,
+                       tdm_stream stream);
 
 /* ---- K3: sharded AdamW --------------------------------------------------- */
 

@@ -62,7 +62,7 @@ _SIGNATURES = {
     "tdm_k2_table_bytes": (ctypes.c_int64, [ctypes.POINTER(FoldSeg), ctypes.c_int, ctypes.c_int]),
     "tdm_k2_table_build": (ctypes.c_int, [ctypes.POINTER(FoldSeg), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "tdm_k2_bucket_fold": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                          ctypes.c_void_p]),
+                                          ctypes.c_int, ctypes.c_void_p]),
     "tdm_k3_adamw": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                     ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
     "tdm_k4_unit_gather": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_int64),

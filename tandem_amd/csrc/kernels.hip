@@ -375,7 +375,8 @@ __host__ __device__ inline int64_t fold_tile_seg_offset(int nseg) {
 }
 
 // One tile of one segment: W loads per element, the fold in ring order, W stores.
-template <typename T, int kWorld, int kDiv>
+// kAcc: the result is added into each destination (dst = dst + sum) instead of replacing it.
+template <typename T, int kWorld, int kDiv, bool kAcc>
 __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const Divisor<T>& dv) {
   using A = typename Elem<T>::acc;
   constexpr int L = lanes<T>();
@@ -422,7 +423,17 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
           const vec16 packed = pack<T>(out);
 #pragma unroll
           for (int k = 0; k < kWorld; ++k)
-            if (dp[k]) store16(dp[k] + v * 16, packed);
+            if (dp[k]) {
+              if constexpr (kAcc) {
+                Lanes<T> cur = unpack<T>(load_rmw(dp[k] + v * 16));
+#pragma unroll
+                for (int l = 0; l < L; ++l)
+                  cur.v[l] = Elem<T>::narrow(static_cast<A>(Elem<T>::widen(cur.v[l]) + Elem<T>::widen(out.v[l])));
+                store16(dp[k] + v * 16, pack<T>(cur));
+              } else {
+                store16(dp[k] + v * 16, packed);
+              }
+            }
         }
       }
     }
@@ -436,7 +447,10 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
       }
 #pragma unroll
       for (int k = 0; k < kWorld; ++k)
-        if (dp[k]) reinterpret_cast<T*>(dp[k])[i] = Elem<T>::narrow(acc);
+        if (dp[k]) {
+          T* out1 = reinterpret_cast<T*>(dp[k]) + i;
+          *out1 = kAcc ? Elem<T>::narrow(static_cast<A>(Elem<T>::widen(*out1) + Elem<T>::widen(Elem<T>::narrow(acc)))) : Elem<T>::narrow(acc);
+        }
     }
   } else {
     const int64_t e0 = t * kTileElems + threadIdx.x;
@@ -451,14 +465,17 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
         }
 #pragma unroll
         for (int k = 0; k < kWorld; ++k)
-          if (dp[k]) reinterpret_cast<T*>(dp[k])[i] = Elem<T>::narrow(acc);
+          if (dp[k]) {
+            T* out1 = reinterpret_cast<T*>(dp[k]) + i;
+            *out1 = kAcc ? Elem<T>::narrow(static_cast<A>(Elem<T>::widen(*out1) + Elem<T>::widen(Elem<T>::narrow(acc)))) : Elem<T>::narrow(acc);
+          }
       }
     }
   }
 }
 
 // Table in device memory (many segments: DDP's buckets).
-template <typename T, int kWorld, int kDiv>
+template <typename T, int kWorld, int kDiv, bool kAcc>
 __global__ __launch_bounds__(kThreads) void k2_fold_kernel(const char* __restrict__ image, Divisor<T> dv) {
   const FoldHeader* hd = reinterpret_cast<const FoldHeader*>(image);
   const int nseg = hd->nseg;
@@ -468,7 +485,7 @@ __global__ __launch_bounds__(kThreads) void k2_fold_kernel(const char* __restric
   const int64_t total = hd->total_tiles;
   for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
     const int lo = tile_seg[tile];  // one lookup, then the loads can go out
-    fold_tile<T, kWorld, kDiv>(segs[lo], tile - (lo ? tile_end[lo - 1] : 0), dv);
+    fold_tile<T, kWorld, kDiv, kAcc>(segs[lo], tile - (lo ? tile_end[lo - 1] : 0), dv);
   }
 }
 
@@ -485,7 +502,7 @@ __global__ __launch_bounds__(kThreads) void k2_fold_small_kernel(FoldSmall tab, 
   for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
     int lo = 0;
     while (tile >= tab.tile_end[lo]) ++lo;
-    fold_tile<T, kWorld, kDiv>(tab.seg[lo], tile - (lo ? tab.tile_end[lo - 1] : 0), dv);
+    fold_tile<T, kWorld, kDiv, false>(tab.seg[lo], tile - (lo ? tab.tile_end[lo - 1] : 0), dv);
   }
 }
 
@@ -666,15 +683,15 @@ void launch_copy(const PairTable& tab, int64_t tiles, int world, hipStream_t str
   }
 }
 
-template <typename T, int kWorld>
+template <typename T, int kWorld, bool kAcc>
 void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(kWorld);
   const dim3 grid(grid_for(tiles)), block(kThreads);
   const char* img = static_cast<const char*>(image);
   switch (div_kind(kWorld, average != 0)) {
-    case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0>), grid, block, 0, stream, img, dv); break;
-    case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1>), grid, block, 0, stream, img, dv); break;
-    default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2>), grid, block, 0, stream, img, dv); break;
+    case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, 0, stream, img, dv); break;
+    case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1, kAcc>), grid, block, 0, stream, img, dv); break;
+    default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2, kAcc>), grid, block, 0, stream, img, dv); break;
   }
 }
 
@@ -703,19 +720,25 @@ void launch_fold_small(const FoldSmall& tab, int world, int average, hipStream_t
   }
 }
 
-template <typename T>
-void launch_fold(const void* image, int64_t tiles, int world, int average, hipStream_t stream) {
+template <typename T, bool kAcc>
+void launch_fold_a(const void* image, int64_t tiles, int world, int average, hipStream_t stream) {
   switch (world) {
-    case 1: launch_fold_w<T, 1>(image, tiles, average, stream); break;
-    case 2: launch_fold_w<T, 2>(image, tiles, average, stream); break;
-    case 3: launch_fold_w<T, 3>(image, tiles, average, stream); break;
-    case 4: launch_fold_w<T, 4>(image, tiles, average, stream); break;
-    case 5: launch_fold_w<T, 5>(image, tiles, average, stream); break;
-    case 6: launch_fold_w<T, 6>(image, tiles, average, stream); break;
-    case 7: launch_fold_w<T, 7>(image, tiles, average, stream); break;
-    case 8: launch_fold_w<T, 8>(image, tiles, average, stream); break;
+    case 1: launch_fold_w<T, 1, kAcc>(image, tiles, average, stream); break;
+    case 2: launch_fold_w<T, 2, kAcc>(image, tiles, average, stream); break;
+    case 3: launch_fold_w<T, 3, kAcc>(image, tiles, average, stream); break;
+    case 4: launch_fold_w<T, 4, kAcc>(image, tiles, average, stream); break;
+    case 5: launch_fold_w<T, 5, kAcc>(image, tiles, average, stream); break;
+    case 6: launch_fold_w<T, 6, kAcc>(image, tiles, average, stream); break;
+    case 7: launch_fold_w<T, 7, kAcc>(image, tiles, average, stream); break;
+    case 8: launch_fold_w<T, 8, kAcc>(image, tiles, average, stream); break;
     default: throw Invalid("world must be in [1, 8]");
   }
+}
+
+template <typename T>
+void launch_fold(const void* image, int64_t tiles, int world, int average, bool accumulate, hipStream_t stream) {
+  if (accumulate) launch_fold_a<T, true>(image, tiles, world, average, stream);
+  else launch_fold_a<T, false>(image, tiles, world, average, stream);
 }
 
 }  // namespace
@@ -1019,7 +1042,8 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
   });
 }
 
-int tdm_k2_bucket_fold(const void* table_dev, int nseg, int dtype, int world, int average, tdm_stream stream) {
+int tdm_k2_bucket_fold(const void* table_dev, int nseg, int dtype, int world, int average, int accumulate,
+                       tdm_stream stream) {
   return guard([&] {
     if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
     if (nseg < 0) throw Invalid("nseg is negative");
@@ -1031,12 +1055,12 @@ int tdm_k2_bucket_fold(const void* table_dev, int nseg, int dtype, int world, in
     const int64_t many = static_cast<int64_t>(compute_units()) * g_blocks_per_cu;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (dtype) {
-      case TDM_F32: launch_fold<float>(table_dev, many, world, average, st); break;
-      case TDM_F64: launch_fold<double>(table_dev, many, world, average, st); break;
-      case TDM_F16: launch_fold<f16_t>(table_dev, many, world, average, st); break;
-      case TDM_BF16: launch_fold<bf16_t>(table_dev, many, world, average, st); break;
-      case TDM_I64: launch_fold<int64_t>(table_dev, many, world, 0, st); break;
-      case TDM_I32: launch_fold<int32_t>(table_dev, many, world, 0, st); break;
+      case TDM_F32: launch_fold<float>(table_dev, many, world, average, accumulate != 0, st); break;
+      case TDM_F64: launch_fold<double>(table_dev, many, world, average, accumulate != 0, st); break;
+      case TDM_F16: launch_fold<f16_t>(table_dev, many, world, average, accumulate != 0, st); break;
+      case TDM_BF16: launch_fold<bf16_t>(table_dev, many, world, average, accumulate != 0, st); break;
+      case TDM_I64: launch_fold<int64_t>(table_dev, many, world, 0, accumulate != 0, st); break;
+      case TDM_I32: launch_fold<int32_t>(table_dev, many, world, 0, accumulate != 0, st); break;
       default: throw Invalid("unknown dtype " + std::to_string(dtype));
     }
     check_hip(hipGetLastError(), "k2_fold launch");

@@ -184,24 +184,41 @@ class FoldTable:
         for members in buckets:
             for i, off, count, chunk in fold_segments([first[i].numel() for i in members], world):
                 rows.append((members[i], off, count, chunk))
-        self.nseg = len(rows)
-        self.elements = sum(r[2] for r in rows)
-        segs = (_lib.FoldSeg * max(1, self.nseg))()
+        segs = (_lib.FoldSeg * max(1, len(rows)))()
         for k, (i, off, count, chunk) in enumerate(rows):
             for r in range(world):
                 segs[k].src[r] = tensors_per_rank[r][i].data_ptr() + off * es
                 segs[k].dst[r] = outs[r][i].data_ptr() + off * es
             segs[k].count, segs[k].chunk = count, chunk
+        self._upload(segs, len(rows))
+
+    @classmethod
+    def from_segments(cls, world, dtype, device, rows, keep=()):
+        """rows: (src addresses per rank, dst addresses per rank (0 = none), count, chunk)."""
+        self = cls.__new__(cls)
+        self.world, self.dtype, self.device, self._keep = world, dtype, torch.device(device), keep
+        segs = (_lib.FoldSeg * max(1, len(rows)))()
+        for k, (srcs, dsts, count, chunk) in enumerate(rows):
+            for r in range(world):
+                segs[k].src[r] = srcs[r]
+                segs[k].dst[r] = dsts[r] or None
+            segs[k].count, segs[k].chunk = count, chunk
+        self._upload(segs, len(rows))
+        return self
+
+    def _upload(self, segs, nseg):
+        self.nseg = nseg
+        self.elements = sum(segs[k].count for k in range(nseg))
         nbytes = lib().tdm_k2_table_bytes(segs, self.nseg, dtype_code(self.dtype))
         if nbytes < 0:
             raise ValueError("bucket_table: bad segment table")
         image = torch.empty(max(16, nbytes), dtype=torch.uint8)
-        check(lib().tdm_k2_table_build(segs, self.nseg, world, dtype_code(self.dtype), ctypes.c_void_p(image.data_ptr())))
+        check(lib().tdm_k2_table_build(segs, self.nseg, self.world, dtype_code(self.dtype), ctypes.c_void_p(image.data_ptr())))
         self.image = image.to(self.device)
 
-    def run(self, average=True):
+    def run(self, average=True, accumulate=False):
         check(lib().tdm_k2_bucket_fold(ctypes.c_void_p(self.image.data_ptr()), self.nseg, dtype_code(self.dtype),
-                                       self.world, int(average), stream_ptr(self.device)))
+                                       self.world, int(average), int(accumulate), stream_ptr(self.device)))
 
 
 class LocalZeRO2:
@@ -236,6 +253,7 @@ class LocalZeRO2:
         es = 4
         self._steps = [[] for _ in range(world - 1)]
         self._adds = []
+        rows = []
         sb = [t.data_ptr() for t in self.staging]
         for a, b, _ in self.buckets:
             sizes = self.layouts[0].bucket_sizes(a, b)
@@ -247,7 +265,12 @@ class LocalZeRO2:
                         self._steps[s].append((sb[r] + lo * es, sb[(r - 1) % world] + lo * es, m))
                     shard_at = lo - self.layouts[c].lo
                     self._adds.append((self.grad_shards[c].data_ptr() + shard_at * es, sb[c] + lo * es, m))
+                    dsts = [0] * world
+                    dsts[c] = self.grad_shards[c].data_ptr() + shard_at * es
+                    rows.append(([p + lo * es for p in sb], dsts, m, c))
                 lo += m
+        self._fold = (FoldTable.from_segments(world, torch.float32, device, rows, keep=(self.staging, self.grad_shards))
+                      if world <= _lib.TDM_MAX_WORLD else None)
 
     def _launch(self, items, scale_dst, scale_src, writeback):
         st = stream_ptr(self.device)
@@ -256,10 +279,19 @@ class LocalZeRO2:
             check(lib().tdm_k1_reduce_step(_pairs(part), len(part), 0, self.world if scale_dst else 1,
                                            int(scale_dst), int(scale_src), int(writeback), st))
 
-    def reduce_grads(self):
+    def reduce_grads(self, algorithm="fold"):
+        """algorithm="ring": the reduce-scatter's ring steps (all buckets of a step
+        together), then grad_shard += mine. algorithm="fold" (default, up to 8
+        ranks): one launch that reads every rank's gradient, sums in the ring's
+        order for the chunk, and adds into the owner's gradient shard; the same bits
+        (including -0.0 + 0.0 = +0.0 from the add) with half the HBM traffic. The
+        staging buffers are left untouched by the fold."""
+        if algorithm == "fold" and self._fold is not None:
+            self._fold.run(average=True, accumulate=True)
+            return
         for s, items in enumerate(self._steps):
             self._launch(items, True, s == 0, s == 0)
-        self._launch(self._adds, False, False, False)  # grad_shard += mine (add_, so -0.0 + 0.0 = +0.0 as in the reference)
+        self._launch(self._adds, False, False, False)  # grad_shard += mine
 
     def step(self):
         for r in range(self.world):

@@ -43,8 +43,9 @@ def oracle_zero2(world, numels, bucket_bytes, params0, grads_per_step):
     return bufs, opts
 
 
+@pytest.mark.parametrize("algorithm", ["fold", "ring"])
 @pytest.mark.parametrize("world", [2, 4, 3])
-def test_small_model_bit_exact_with_oracle(world):
+def test_small_model_bit_exact_with_oracle(world, algorithm):
     from tandem_amd.local import LocalZeRO2
 
     dev = torch.device("cuda", 0)
@@ -62,7 +63,7 @@ def test_small_model_bit_exact_with_oracle(world):
     for s in range(steps):
         for r in range(world):
             z.staging[r].copy_(torch.from_numpy(grads[s][r]))
-        z.reduce_grads()
+        z.reduce_grads(algorithm)
         z.step()
         z.zero_grad()
     want, opts = oracle_zero2(world, numels, 4 << 10, p0, grads)
@@ -97,7 +98,15 @@ def test_full_size_step():
         g = torch.randn(n, device=dev, generator=gen) * 1e-3
         z.staging[r].copy_(g)
         grads.append(g)
-    z.reduce_grads()
+    z.reduce_grads("ring")
+    ring_shards = [g.clone() for g in z.grad_shards]
+    z.zero_grad()
+    for r in range(world):
+        z.staging[r].copy_(grads[r])
+    z.reduce_grads("fold")
+    for r in range(world):  # one launch, same bits as the ring steps
+        assert torch.equal(ring_shards[r].view(torch.int32), z.grad_shards[r].view(torch.int32))
+    del ring_shards
     # the averaged gradient in ring order, sampled per bucket chunk
     lay = z.layouts
     for a, b, _ in z.buckets[::5]:
