@@ -120,14 +120,16 @@ typedef struct tdm_fold_seg {
   int32_t reserved;
 } tdm_fold_seg;
 
-/* Bytes of device memory the table of these segments needs (-1: bad arguments). */
+/* The device table holds one record per 16 KiB tile of every segment. Number of tiles
+ * and bytes of device memory the table of these segments needs (-1: bad arguments). */
+int64_t tdm_k2_table_tiles(const tdm_fold_seg* segs, int nseg, int dtype);
 int64_t tdm_k2_table_bytes(const tdm_fold_seg* segs, int nseg, int dtype);
 
 /* Writes the device image of the table into host memory `image`
  * (tdm_k2_table_bytes(...) bytes); the caller copies it to the device once. */
 int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype, void* image);
 
-/* For every element of every segment, in one launch:
+/* For every element of every segment, in one launch over `ntiles` tiles:
  *     y_q = average ? src[q][i] / world : src[q][i]
  *     acc = y[(chunk+1) % world];  acc = y[(chunk+k) % world] + acc,  k = 2..world
  *     dst[r][i] = acc  for every rank r with a non-NULL dst   (accumulate: dst[r][i] = dst[r][i] + acc)
@@ -136,7 +138,7 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
  * (tandem/ddp.py:22-33,89-109; ring order tandem/comm.py:301-311). With a dst only for
  * the chunk's owner and accumulate set, a segment is ZeRO-2's reduce_scatter of that chunk
  * followed by `grad_shard[...].add_(mine)` (tandem/zero.py:141,150-153). */
-int tdm_k2_bucket_fold(const void* table_dev, int nseg, int dtype, int world, int average, int accumulate,
+int tdm_k2_bucket_fold(const void* table_dev, int64_t ntiles, int dtype, int world, int average, int accumulate,
                        tdm_stream stream);
 
 /* ---- K3: sharded AdamW --------------------------------------------------- */

@@ -61,7 +61,8 @@ _SIGNATURES = {
                                             ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "tdm_k2_table_bytes": (ctypes.c_int64, [ctypes.POINTER(FoldSeg), ctypes.c_int, ctypes.c_int]),
     "tdm_k2_table_build": (ctypes.c_int, [ctypes.POINTER(FoldSeg), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
-    "tdm_k2_bucket_fold": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+    "tdm_k2_table_tiles": (ctypes.c_int64, [ctypes.POINTER(FoldSeg), ctypes.c_int, ctypes.c_int]),
+    "tdm_k2_bucket_fold": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                           ctypes.c_int, ctypes.c_void_p]),
     "tdm_k3_adamw": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                     ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),

@@ -349,14 +349,10 @@ __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Diviso
 }
 
 // ---------------------------------------------------------------- K2: bucket fold
-// Device image of a table: a header, the running tile counts, then the segments.
-struct FoldHeader {
-  uint64_t magic;
-  int32_t nseg, world, dtype, reserved;
-  int64_t total_tiles;
-};
-constexpr uint64_t kFoldMagic = 0x74646d4b32746162ull;  // "tdmK2tab"
-
+// A segment as the kernels see it. The device table of K2 is an array of these, ONE
+// PER TILE: the pointers already advanced to the tile's first element and `count`
+// the tile's elements, so a workgroup needs a single lookup before its loads go out
+// (a tile -> segment -> pointers chain cost 20% of the kernel's throughput).
 struct FoldSegDev {
   const char* src[TDM_MAX_WORLD];
   char* dst[TDM_MAX_WORLD];
@@ -364,15 +360,6 @@ struct FoldSegDev {
   int32_t chunk;
   int32_t vec_ok;  // every pointer of the segment is 16-byte aligned
 };
-
-// header | tile_end[nseg] (int64) | segments[nseg] | tile_seg[total_tiles] (int32)
-__host__ __device__ inline int64_t fold_tile_end_offset() { return sizeof(FoldHeader); }
-__host__ __device__ inline int64_t fold_segs_offset(int nseg) {
-  return (sizeof(FoldHeader) + static_cast<int64_t>(nseg) * 8 + 15) / 16 * 16;
-}
-__host__ __device__ inline int64_t fold_tile_seg_offset(int nseg) {
-  return fold_segs_offset(nseg) + static_cast<int64_t>(nseg) * static_cast<int64_t>(sizeof(FoldSegDev));
-}
 
 // One tile of one segment: W loads per element, the fold in ring order, W stores.
 // kAcc: the result is added into each destination (dst = dst + sum) instead of replacing it.
@@ -474,18 +461,12 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
   }
 }
 
-// Table in device memory (many segments: DDP's buckets).
+// Table in device memory, one record per tile (many segments: DDP's buckets).
 template <typename T, int kWorld, int kDiv, bool kAcc>
-__global__ __launch_bounds__(kThreads) void k2_fold_kernel(const char* __restrict__ image, Divisor<T> dv) {
-  const FoldHeader* hd = reinterpret_cast<const FoldHeader*>(image);
-  const int nseg = hd->nseg;
-  const int64_t* tile_end = reinterpret_cast<const int64_t*>(image + fold_tile_end_offset());
-  const FoldSegDev* segs = reinterpret_cast<const FoldSegDev*>(image + fold_segs_offset(nseg));
-  const int32_t* tile_seg = reinterpret_cast<const int32_t*>(image + fold_tile_seg_offset(nseg));
-  const int64_t total = hd->total_tiles;
+__global__ __launch_bounds__(kThreads) void k2_fold_kernel(const FoldSegDev* __restrict__ tiles, int64_t total,
+                                                           Divisor<T> dv) {
   for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
-    const int lo = tile_seg[tile];  // one lookup, then the loads can go out
-    fold_tile<T, kWorld, kDiv, kAcc>(segs[lo], tile - (lo ? tile_end[lo - 1] : 0), dv);
+    fold_tile<T, kWorld, kDiv, kAcc>(tiles[tile], 0, dv);
   }
 }
 
@@ -687,11 +668,11 @@ template <typename T, int kWorld, bool kAcc>
 void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(kWorld);
   const dim3 grid(grid_for(tiles)), block(kThreads);
-  const char* img = static_cast<const char*>(image);
+  const FoldSegDev* img = static_cast<const FoldSegDev*>(image);
   switch (div_kind(kWorld, average != 0)) {
-    case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, 0, stream, img, dv); break;
-    case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1, kAcc>), grid, block, 0, stream, img, dv); break;
-    default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2, kAcc>), grid, block, 0, stream, img, dv); break;
+    case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, 0, stream, img, tiles, dv); break;
+    case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1, kAcc>), grid, block, 0, stream, img, tiles, dv); break;
+    default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2, kAcc>), grid, block, 0, stream, img, tiles, dv); break;
   }
 }
 
@@ -993,10 +974,16 @@ int64_t fold_tiles(const tdm_fold_seg* segs, int nseg, int es) {
 }
 }  // namespace
 
-int64_t tdm_k2_table_bytes(const tdm_fold_seg* segs, int nseg, int dtype) {
+int64_t tdm_k2_table_tiles(const tdm_fold_seg* segs, int nseg, int dtype) {
   const int es = elem_size(dtype);
   if (nseg < 0 || es == 0 || (nseg > 0 && segs == nullptr)) return -1;
-  return (fold_tile_seg_offset(nseg) + fold_tiles(segs, nseg, es) * 4 + 15) / 16 * 16;
+  return fold_tiles(segs, nseg, es);
+}
+
+int64_t tdm_k2_table_bytes(const tdm_fold_seg* segs, int nseg, int dtype) {
+  const int64_t tiles = tdm_k2_table_tiles(segs, nseg, dtype);
+  if (tiles < 0) return -1;
+  return std::max<int64_t>(16, tiles * static_cast<int64_t>(sizeof(FoldSegDev)));
 }
 
 int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype, void* image) {
@@ -1005,12 +992,8 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
     if (es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
     if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
     if (nseg < 0 || (nseg > 0 && segs == nullptr) || image == nullptr) throw Invalid("bad table arguments");
-    char* img = static_cast<char*>(image);
-    std::memset(img, 0, static_cast<size_t>(tdm_k2_table_bytes(segs, nseg, dtype)));
-    int32_t* tile_seg = reinterpret_cast<int32_t*>(img + fold_tile_seg_offset(nseg));
-    FoldHeader* hd = reinterpret_cast<FoldHeader*>(img);
-    int64_t* tile_end = reinterpret_cast<int64_t*>(img + fold_tile_end_offset());
-    FoldSegDev* out = reinterpret_cast<FoldSegDev*>(img + fold_segs_offset(nseg));
+    std::memset(image, 0, static_cast<size_t>(tdm_k2_table_bytes(segs, nseg, dtype)));
+    FoldSegDev* out = static_cast<FoldSegDev*>(image);
     const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
     int64_t tiles = 0;
     for (int i = 0; i < nseg; ++i) {
@@ -1023,44 +1006,37 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
         const uintptr_t a = reinterpret_cast<uintptr_t>(s.src[r]), b = reinterpret_cast<uintptr_t>(s.dst[r]);
         if (a % es || b % es) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to the element size");
         vec = vec && a % 16 == 0 && b % 16 == 0;
-        out[i].src[r] = static_cast<const char*>(s.src[r]);
-        out[i].dst[r] = static_cast<char*>(s.dst[r]);
       }
-      out[i].count = s.count;
-      out[i].chunk = s.chunk;
-      out[i].vec_ok = vec;
-      const int64_t mine = (s.count + tile_elems - 1) / tile_elems;
-      for (int64_t t = 0; t < mine; ++t) tile_seg[tiles + t] = i;
-      tiles += mine;
-      tile_end[i] = tiles;
+      for (int64_t at = 0; at < s.count; at += tile_elems) {  // a tile's byte offset is a multiple of 16 KiB
+        FoldSegDev& rec = out[tiles++];
+        for (int r = 0; r < world; ++r) {
+          rec.src[r] = static_cast<const char*>(s.src[r]) + at * es;
+          rec.dst[r] = s.dst[r] ? static_cast<char*>(s.dst[r]) + at * es : nullptr;
+        }
+        rec.count = std::min<int64_t>(tile_elems, s.count - at);
+        rec.chunk = s.chunk;
+        rec.vec_ok = vec;
+      }
     }
-    hd->magic = kFoldMagic;
-    hd->nseg = nseg;
-    hd->world = world;
-    hd->dtype = dtype;
-    hd->total_tiles = tiles;
   });
 }
 
-int tdm_k2_bucket_fold(const void* table_dev, int nseg, int dtype, int world, int average, int accumulate,
+int tdm_k2_bucket_fold(const void* table_dev, int64_t ntiles, int dtype, int world, int average, int accumulate,
                        tdm_stream stream) {
   return guard([&] {
     if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
-    if (nseg < 0) throw Invalid("nseg is negative");
-    if (nseg == 0) return;
+    if (ntiles < 0) throw Invalid("ntiles is negative");
+    if (ntiles == 0) return;
     if (table_dev == nullptr) throw Invalid("table is NULL");
     if (average && world > 1 && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
-    // The tile count lives in the device image; reading it back would stall the
-    // stream, so the grid is sized for the device and the kernel strides.
-    const int64_t many = static_cast<int64_t>(compute_units()) * g_blocks_per_cu;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (dtype) {
-      case TDM_F32: launch_fold<float>(table_dev, many, world, average, accumulate != 0, st); break;
-      case TDM_F64: launch_fold<double>(table_dev, many, world, average, accumulate != 0, st); break;
-      case TDM_F16: launch_fold<f16_t>(table_dev, many, world, average, accumulate != 0, st); break;
-      case TDM_BF16: launch_fold<bf16_t>(table_dev, many, world, average, accumulate != 0, st); break;
-      case TDM_I64: launch_fold<int64_t>(table_dev, many, world, 0, accumulate != 0, st); break;
-      case TDM_I32: launch_fold<int32_t>(table_dev, many, world, 0, accumulate != 0, st); break;
+      case TDM_F32: launch_fold<float>(table_dev, ntiles, world, average, accumulate != 0, st); break;
+      case TDM_F64: launch_fold<double>(table_dev, ntiles, world, average, accumulate != 0, st); break;
+      case TDM_F16: launch_fold<f16_t>(table_dev, ntiles, world, average, accumulate != 0, st); break;
+      case TDM_BF16: launch_fold<bf16_t>(table_dev, ntiles, world, average, accumulate != 0, st); break;
+      case TDM_I64: launch_fold<int64_t>(table_dev, ntiles, world, 0, accumulate != 0, st); break;
+      case TDM_I32: launch_fold<int32_t>(table_dev, ntiles, world, 0, accumulate != 0, st); break;
       default: throw Invalid("unknown dtype " + std::to_string(dtype));
     }
     check_hip(hipGetLastError(), "k2_fold launch");

@@ -210,6 +210,7 @@ class FoldTable:
         self.nseg = nseg
         self.elements = sum(segs[k].count for k in range(nseg))
         nbytes = lib().tdm_k2_table_bytes(segs, self.nseg, dtype_code(self.dtype))
+        self.ntiles = lib().tdm_k2_table_tiles(segs, self.nseg, dtype_code(self.dtype))
         if nbytes < 0:
             raise ValueError("bucket_table: bad segment table")
         image = torch.empty(max(16, nbytes), dtype=torch.uint8)
@@ -217,7 +218,7 @@ class FoldTable:
         self.image = image.to(self.device)
 
     def run(self, average=True, accumulate=False):
-        check(lib().tdm_k2_bucket_fold(ctypes.c_void_p(self.image.data_ptr()), self.nseg, dtype_code(self.dtype),
+        check(lib().tdm_k2_bucket_fold(ctypes.c_void_p(self.image.data_ptr()), self.ntiles, dtype_code(self.dtype),
                                        self.world, int(average), int(accumulate), stream_ptr(self.device)))
 
 
