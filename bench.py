@@ -256,8 +256,14 @@ def fsdp_gather(steps):
 
 
 # ---------------------------------------------------------------- CPU baseline
-def cpu_rank(g, n, reps):
+def cpu_rank(g, n, reps, numels):
+    """Timed on the host: (i) the ring all-reduce(avg) of the GPU's main workload,
+    (ii) the ZeRO-2 step (16 bucket reduce-scatters, shard add, AdamW, all-gather)."""
+    import numpy as np
     import torch
+
+    from oracle.adamw import AdamW
+    from tandem_amd.buckets import FlatLayout, zero_buckets
 
     x = torch.randn(n, generator=torch.Generator().manual_seed(g.rank)) * 1e-2
     g.all_reduce(x, op="avg")
@@ -267,7 +273,32 @@ def cpu_rank(g, n, reps):
         t = time.perf_counter()
         g.all_reduce(x, op="avg")
         ts.append(time.perf_counter() - t)
-    return statistics.median(ts)
+    out = {"all_reduce_s": statistics.median(ts)}
+    del x
+    lay = FlatLayout(numels, g.size, g.rank)
+    buckets = zero_buckets(numels, 4, 25 << 20)
+    buf = torch.randn(lay.numel, generator=torch.Generator().manual_seed(5)) * 0.02
+    grads = torch.randn(lay.numel, generator=torch.Generator().manual_seed(10 + g.rank)) * 1e-3
+    staging = torch.empty_like(grads)
+    shard = torch.zeros(lay.hi - lay.lo)
+    opt = AdamW(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    ts = []
+    for _ in range(3):
+        staging.copy_(grads)
+        shard.zero_()
+        g.barrier()
+        t = time.perf_counter()
+        works = [g.reduce_scatter(staging[a:b], lay.bucket_sizes(a, b), op="avg", async_op=True) for a, b, _ in buckets]
+        for (a, b, _), w in zip(buckets, works):
+            mine = w.wait()
+            if mine.numel():
+                at = max(a, lay.lo) - lay.lo
+                shard[at:at + mine.numel()].add_(mine)
+        opt.update("flat", buf[lay.lo:lay.hi].numpy(), shard.numpy())
+        g.all_gather(buf, lay.sizes)
+        ts.append(time.perf_counter() - t)
+    out["zero2_step_s"] = statistics.median(ts)
+    return out
 
 
 def cpu_baseline(mib, reps):
@@ -275,13 +306,15 @@ def cpu_baseline(mib, reps):
 
     n = mib * (1 << 20) // 4
     t0 = time.perf_counter()
-    t = max(cpu_launch(cpu_rank, WORLD, n, reps))
+    res = cpu_launch(cpu_rank, WORLD, n, reps, gpt_numels())
     total = time.perf_counter() - t0
+    t = max(r["all_reduce_s"] for r in res)
+    z = max(r["zero2_step_s"] for r in res)
     return {"value": round(15 * n * 4 / t / 1e9, 3), "unit": "GB/s", "cores": WORLD, "kind": "port",
             "sample": f"oracle CPU-process engine (tandem's Python-engine protocol): ring all-reduce(avg), world 4 x 1 torch thread, "
-                      f"{mib} MiB fp32 per rank, 2 x 4 MiB shared-memory slots per pair, median of {reps}; {t * 1e3:.1f} ms per all-reduce, "
-                      f"{total:.1f} s including process start",
-            "algbw_GBps": round(n * 4 / t / 1e9, 3), "host_cores": os.cpu_count()}
+                      f"{mib} MiB fp32 per rank (the GPU workload), 2 x 4 MiB shared-memory slots per pair, median of {reps}: "
+                      f"{t * 1e3:.1f} ms per all-reduce; then 3 ZeRO-2 steps at 85,842,432 params; {total:.1f} s in all, {total * WORLD:.0f} core-seconds",
+            "algbw_GBps": round(n * 4 / t / 1e9, 3), "zero2_step_ms": round(z * 1e3, 1), "host_cores": os.cpu_count()}
 
 
 def device_name(_lib):
@@ -310,7 +343,7 @@ def main():
     # The two multi-process figures first, while this process has not touched the GPU.
     cpu = fsdp = None
     if not args.quick and not args.no_cpu:
-        cpu = cpu_baseline(64, 7)
+        cpu = cpu_baseline(args.mib, 15)
     if not args.quick and not args.no_fsdp:
         try:
             fsdp = fsdp_gather(3)
@@ -368,6 +401,7 @@ def main():
             line["fsdp_gather"] = fsdp
         if cpu is not None:
             cpu["gpu_over_cpu"] = round(line["value"] / cpu["value"], 1)
+            cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["ms"], 1)
             line["cpu_baseline"] = cpu
     line["device"] = device_name(_lib)
     print(json.dumps(line), flush=True)

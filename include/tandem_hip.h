@@ -239,6 +239,19 @@ int tdm_broadcast(tdm_engine* e, void* ptr, int64_t numel, int dtype, int root, 
  * FSDP._start_gather (tandem/zero.py:238-245). */
 int tdm_unit_gather(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes, int nsizes,
                     tdm_stream caller, tdm_work** out);
+/* Shared arena + direct gather (no counterpart in the reference, which stages every
+ * gather through its slots): tdm_engine_share allocates `bytes` (< 2 GiB) of device
+ * memory on this rank and publishes its hipIpcMemHandle_t; peers map it on first use.
+ * tdm_unit_gather_direct then fills `full` with W-1 copy kernels that read chunk q
+ * straight from rank q's arena at byte offset peer_offsets[q] (own chunk: from `shard`),
+ * on the engine's stream, without any message. The caller must bracket every change of
+ * arena contents with tdm_fence, a barrier that is also ordered against the GPU: it
+ * starts once `caller` has finished what it held, and a rank's arrival is announced
+ * only when its engine stream has finished as well. */
+int tdm_engine_share(tdm_engine* e, int64_t bytes, void** ptr);
+int tdm_unit_gather_direct(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes,
+                           int nsizes, const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out);
+int tdm_fence(tdm_engine* e, tdm_stream caller, tdm_work** out);
 int tdm_sendrecv(tdm_engine* e, const void* send, int64_t send_numel, int dst, void* recv, int64_t recv_numel, int src,
                  int dtype, tdm_stream caller, tdm_work** out);
 int tdm_barrier(tdm_engine* e, tdm_work** out);

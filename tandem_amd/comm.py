@@ -88,6 +88,7 @@ class Group:
         self.trace, self.waits, self.tracing = [], [], False
         self._closed = False
         self._engine = None
+        self._arena = None
         if self.backend != "hip":
             raise CommError(f"unknown backend {self.backend} (tandem_amd provides \"hip\")")
         if self.transport != "device":
@@ -197,7 +198,43 @@ class Group:
             self._engine, ctypes.c_void_p(flat.data_ptr()), self._count(flat, code), code, arr, n, self._stream(), out),
             t, t.numel() * t.element_size(), async_op, keep=(flat,))
 
-    def gather_unit(self, full, shard, sizes=None, async_op=False):
+    # ---- shared arena: long-lived data that peers read directly
+    def shared_empty(self, numel, dtype=torch.float32):
+        """A tensor of `numel` elements in this rank's shared arena: device memory
+        owned by the engine (freed by close()), exported once through HIP IPC, that
+        the other ranks read directly in gather_unit(..., peer_offsets=...). One
+        arena per group, under 2 GiB. Every change of its contents must sit between
+        two fence() calls."""
+        if self._arena is not None:
+            raise CommError("this group already has a shared arena")
+        es = torch.empty(0, dtype=dtype).element_size()
+        nbytes = max(16, numel * es)
+        ptr = ctypes.c_void_p()
+        try:
+            check(lib().tdm_engine_share(self._engine, nbytes, ctypes.byref(ptr)))
+        except (ValueError, RuntimeError) as e:
+            raise CommError(f"shared_empty: {e}") from e
+
+        class _Raw:  # what torch needs to wrap foreign device memory
+            __cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (ptr.value, False), "version": 3}
+
+        raw = torch.as_tensor(_Raw(), device=self.device)
+        self._arena = raw
+        return raw[:numel * es].view(dtype)
+
+    def arena_offset(self, t):
+        """Byte offset of tensor `t` inside this rank's arena (None if it is not there)."""
+        if self._arena is None:
+            return None
+        off = t.data_ptr() - self._arena.data_ptr()
+        return off if 0 <= off and off + t.numel() * t.element_size() <= self._arena.numel() else None
+
+    def fence(self):
+        """A barrier ordered against the GPU: returns (on the caller's stream) once
+        every rank's work queued before its fence() has finished on its GPU streams."""
+        return self._start("fence", lambda out: lib().tdm_fence(self._engine, self._stream(), out), None, 0, False)
+
+    def gather_unit(self, full, shard, sizes=None, async_op=False, peer_offsets=None):
         """ZeRO-3's gather of one unit: `shard` (this rank's chunk) is placed into
         `full` and the other ranks' chunks are gathered, all on the engine's
         stream. Same result as `full[lo:hi].copy_(shard); all_gather(full, sizes)`."""
@@ -209,6 +246,14 @@ class Group:
         sizes, arr, n = self._sizes(flat, sizes)
         if self._chunk_of_rank(flat, sizes).numel() != sh.numel():
             raise CommError(f"gather_unit: the shard has {sh.numel()} elements, this rank's chunk another count")
+        if peer_offsets is not None:
+            # every rank's chunk is read straight from that rank's arena: no staging, no handshake
+            if len(peer_offsets) != self.size:
+                raise CommError("gather_unit: one arena offset per rank")
+            offs = (ctypes.c_int64 * self.size)(*[int(o) for o in peer_offsets])
+            return self._start("gather_unit", lambda out: lib().tdm_unit_gather_direct(
+                self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, ctypes.c_void_p(sh.data_ptr()), arr, n,
+                offs, self.size, self._stream(), out), full, full.numel() * full.element_size(), async_op, keep=(flat, sh))
         if code == _lib.TDM_BYTES and n:
             arr = (ctypes.c_int64 * n)(*[s * flat.element_size() for s in sizes])
         return self._start("gather_unit", lambda out: lib().tdm_unit_gather(
@@ -286,6 +331,7 @@ class Group:
         self.barrier()
         self._closed = True
         eng, self._engine = self._engine, None
+        self._arena = None  # the engine frees it; tensors carved from it must not be used after close()
         try:
             check(lib().tdm_engine_close(eng))
         except Exception as e:

@@ -101,6 +101,9 @@ struct alignas(kLine) RegionHeader {
   int64_t pid;
   int32_t use_events;
   int32_t reserved;
+  // A rank's shared arena (tdm_engine_share): device memory its peers may read directly.
+  std::atomic<uint64_t> arena_bytes;  // 0 until published
+  hipIpcMemHandle_t arena_mem;
 };
 
 class Region {
@@ -228,6 +231,10 @@ class Engine {
   std::shared_ptr<Work> broadcast(Buf t, int root, hipStream_t caller);
   std::shared_ptr<Work> sendrecv(Buf send, int dst, Buf recv, int src, hipStream_t caller);
   std::shared_ptr<Work> barrier();
+  std::shared_ptr<Work> fence(hipStream_t caller);
+  void* share(size_t bytes);
+  std::shared_ptr<Work> unit_gather_direct(Buf full, const char* shard, std::vector<int64_t> sizes,
+                                           std::vector<int64_t> peer_offsets, hipStream_t caller);
 
   int device() const { return device_; }
   hipStream_t stream() const { return stream_; }
@@ -255,7 +262,8 @@ class Engine {
   void signal(int dst, uint64_t length);
   uint64_t await(int src);
   void release(int src);
-  void barrier_now();
+  void barrier_now(bool after_gpu = false);
+  const char* peer_arena(int peer, size_t need_bytes);
 
   std::string region_name(int rank) const { return "/tandem-" + job_ + "-" + std::to_string(rank) + "-hip"; }
 
@@ -269,6 +277,10 @@ class Engine {
   Region mine_;
   std::vector<std::unique_ptr<Region>> theirs_;
   std::vector<void*> out_mem_, peer_mem_;
+  void* arena_ = nullptr;
+  size_t arena_bytes_ = 0;
+  std::vector<void*> peer_arena_;
+  std::vector<size_t> peer_arena_bytes_;
   std::vector<std::vector<hipEvent_t>> full_, free_, peer_full_, peer_free_;
   std::vector<uint64_t> sent_, got_;     // pieces, per peer: pick the slot
   std::vector<uint64_t> posted_;         // messages queued or published to each peer (flow control)
@@ -303,6 +315,8 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
     : job_(job), rank_(rank), size_(size), slots_(slots), slot_bytes_(slot_bytes), timeout_s_(timeout_s),
       device_(device), theirs_(size), out_mem_(size, nullptr), peer_mem_(size, nullptr), full_(size), free_(size),
       peer_full_(size), peer_free_(size), sent_(size, 0), got_(size, 0), posted_(size, 0), taken_(size, 0) {
+  peer_arena_.assign(size, nullptr);
+  peer_arena_bytes_.assign(size, 0);
   if (size < 1 || rank < 0 || rank >= size) throw Invalid("rank must be in [0, size)");
   if (slots < 1 || slots > kMaxSlots) throw Invalid("slots must be in [1, " + std::to_string(kMaxSlots) + "]");
   if (slot_bytes < 16 || slot_bytes % 16) throw Invalid("slot_bytes must be a positive multiple of 16");
@@ -419,12 +433,16 @@ void Engine::close() {
     for (hipEvent_t e : full_[p]) (void)hipEventDestroy(e);
     for (hipEvent_t e : free_[p]) (void)hipEventDestroy(e);
     if (out_mem_[p]) (void)hipFree(out_mem_[p]);
+    if (peer_arena_[p]) (void)hipIpcCloseMemHandle(peer_arena_[p]);
+    peer_arena_[p] = nullptr;
     peer_mem_[p] = out_mem_[p] = nullptr;
     peer_full_[p].clear(); peer_free_[p].clear(); full_[p].clear(); free_[p].clear();
     theirs_[p].reset();
   }
   if (stream_) (void)hipStreamDestroy(stream_);
   stream_ = nullptr;
+  if (arena_) (void)hipFree(arena_);  // after the closing barrier: no peer reads it any more
+  arena_ = nullptr;
   mine_.reset();
   check_hip(sync_err, "hipStreamSynchronize (close)");
   if (!barrier_err.empty()) throw std::runtime_error("close: " + barrier_err);
@@ -591,7 +609,10 @@ void Engine::drain_completions() {
   if (!cerror_.empty()) throw std::runtime_error("completion thread failed: " + cerror_);
 }
 
-void Engine::barrier_now() {
+// after_gpu: the empty messages are published only once the GPU has finished what
+// the engine's stream holds so far (a fence), not merely when it has been enqueued.
+void Engine::barrier_now(bool after_gpu) {
+  if (after_gpu && use_events_) check_hip(hipStreamSynchronize(stream_), "hipStreamSynchronize (fence)");
   // An empty message to every peer, then one from each. Rings are first in,
   // first out, so this also orders the barrier after every piece queued before.
   constexpr uint64_t kEmpty = ~uint64_t(0);
@@ -602,7 +623,7 @@ void Engine::barrier_now() {
     wait_until([&] { return posted - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots_); },
                timeout_s_, "barrier: a peer rank never drained its messages");
     posted_[p] = posted + 1;
-    if (use_events_) signal(p, kEmpty); else complete_later(false, p, kEmpty, false);
+    if (use_events_) signal(p, kEmpty); else complete_later(false, p, kEmpty, after_gpu);
   }
   for (int p = 0; p < size_; ++p) {
     if (p == rank_) continue;
@@ -850,6 +871,83 @@ std::shared_ptr<Work> Engine::sendrecv(Buf send, int dst, Buf recv, int src, hip
   }, caller, true);
 }
 
+// ---------------------------------------------------------------- shared arena, direct gather
+// A rank may keep long-lived data (ZeRO-3's parameter shards) in an arena that its
+// peers map once and then read directly: a unit gather is then W-1 copy kernels from
+// the peers' arenas on this rank's engine stream, with no staging copy and no
+// handshake per gather. The caller brackets every modification of the arena with
+// fence(): before (every peer has finished reading) and after (the new contents are
+// complete) -- ZeRO-3 changes its shards once per step, and gathers them 27 times.
+void* Engine::share(size_t bytes) {
+  if (arena_) throw std::runtime_error("share: this engine already has an arena");
+  if (bytes == 0 || bytes >= (size_t(2) << 30)) throw Invalid("share: the arena must be between 1 byte and 2 GiB (one IPC allocation)");
+  check_hip(hipSetDevice(device_), "hipSetDevice");
+  check_hip(hipMalloc(&arena_, bytes), "hipMalloc (arena)");
+  RegionHeader* h = mine_.header();
+  hipError_t err = hipIpcGetMemHandle(&h->arena_mem, arena_);
+  if (err != hipSuccess) {
+    (void)hipFree(arena_);
+    arena_ = nullptr;
+    check_hip(err, "hipIpcGetMemHandle (arena)");
+  }
+  arena_bytes_ = bytes;
+  h->arena_bytes.store(bytes, std::memory_order_release);  // the handle is visible before the size
+  return arena_;
+}
+
+const char* Engine::peer_arena(int peer, size_t need_bytes) {
+  if (!peer_arena_[peer]) {
+    RegionHeader* h = theirs_[peer]->header();
+    const uint64_t bytes = h->arena_bytes.load(std::memory_order_acquire);
+    if (bytes == 0) throw std::runtime_error("direct gather: rank " + std::to_string(peer) + " has not shared an arena");
+    check_hip(hipIpcOpenMemHandle(&peer_arena_[peer], h->arena_mem, hipIpcMemLazyEnablePeerAccess), "hipIpcOpenMemHandle (arena)");
+    peer_arena_bytes_[peer] = bytes;
+  }
+  if (need_bytes > peer_arena_bytes_[peer]) throw Invalid("direct gather: the range lies outside rank " + std::to_string(peer) + "'s arena");
+  return static_cast<const char*>(peer_arena_[peer]);
+}
+
+std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, std::vector<int64_t> sizes,
+                                                 std::vector<int64_t> peer_offsets, hipStream_t caller) {
+  check(full, "unit_gather", false);
+  if (full.dtype == kBytesDtype) throw Invalid("unit_gather: direct gathers need a typed tensor");
+  const auto c = chunks(full, sizes);
+  if (static_cast<int>(peer_offsets.size()) != size_) throw Invalid("unit_gather: one arena offset per rank");
+  if (c[rank_].numel > 0 && shard == nullptr) throw Invalid("unit_gather: NULL shard");
+  return submit([this, full, shard, sizes, peer_offsets] {
+    const auto cs = chunks(full, sizes);
+    const int es = elem_bytes(full.dtype);
+    tdm_pair pairs[TDM_MAX_PAIRS];
+    int np = 0;
+    auto flush = [&] {
+      if (np) copy_step(pairs, np, full.dtype, 0, stream_);
+      np = 0;
+    };
+    for (int q = 0; q < size_; ++q) {
+      if (cs[q].numel == 0) continue;
+      const char* from;
+      if (q == rank_) {
+        if (shard == cs[q].ptr) continue;
+        from = shard;
+      } else {
+        if (peer_offsets[q] < 0 || peer_offsets[q] % es) throw Invalid("unit_gather: bad arena offset");
+        from = peer_arena(q, static_cast<size_t>(peer_offsets[q]) + static_cast<size_t>(cs[q].numel) * es) + peer_offsets[q];
+      }
+      pairs[np++] = tdm_pair{cs[q].ptr, from, cs[q].numel};
+      if (np == TDM_MAX_PAIRS) flush();
+    }
+    flush();
+  }, caller, true);
+}
+
+// A barrier that is also ordered against the GPU: it starts after the caller's
+// stream has finished what it held at the call, and a rank's arrival is only
+// announced once its engine stream has finished too.
+std::shared_ptr<Work> Engine::fence(hipStream_t caller) {
+  if (!connected_) throw std::runtime_error("fence: the engine is not connected");
+  return submit([this] { barrier_now(true); }, caller, true);
+}
+
 std::shared_ptr<Work> Engine::barrier() {
   if (!connected_) throw std::runtime_error("barrier: the engine is not connected");
   return submit([this] { barrier_now(); }, nullptr, false);
@@ -964,6 +1062,34 @@ int tdm_sendrecv(tdm_engine* e, const void* send, int64_t send_numel, int dst, v
     finish_submit(engine_of(e).sendrecv(Engine::Buf{static_cast<char*>(const_cast<void*>(send)), send_numel, dtype}, dst,
                                         Engine::Buf{static_cast<char*>(recv), recv_numel, dtype}, src,
                                         static_cast<hipStream_t>(caller)), out);
+  });
+}
+
+int tdm_engine_share(tdm_engine* e, int64_t bytes, void** ptr) {
+  return guard([&] {
+    if (ptr == nullptr || bytes <= 0) throw Invalid("share: bad arguments");
+    *ptr = engine_of(e).share(static_cast<size_t>(bytes));
+  });
+}
+
+int tdm_unit_gather_direct(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes,
+                           int nsizes, const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    if (nsizes < 0 || (nsizes > 0 && sizes == nullptr) || noffsets < 0 || (noffsets > 0 && peer_offsets == nullptr)) {
+      throw Invalid("bad sizes or offsets");
+    }
+    std::vector<int64_t> sz(sizes, sizes + nsizes), off(peer_offsets, peer_offsets + noffsets);
+    finish_submit(engine_of(e).unit_gather_direct(Engine::Buf{static_cast<char*>(full), numel, dtype},
+                                                  static_cast<const char*>(shard), std::move(sz), std::move(off),
+                                                  static_cast<hipStream_t>(caller)), out);
+  });
+}
+
+int tdm_fence(tdm_engine* e, tdm_stream caller, tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    finish_submit(engine_of(e).fence(static_cast<hipStream_t>(caller)), out);
   });
 }
 

@@ -156,6 +156,11 @@ class ZeRO(torch.nn.Module):
             self.grad_shard.zero_()
 
 
+def _pad(n):
+    """Shards start on 16-byte boundaries inside the arena (fp32: multiples of 4 elements)."""
+    return (n + 3) // 4 * 4
+
+
 class _Unit:
     def __init__(self, index, module, params, world, rank, device, dtype):
         self.index, self.module, self.params = index, module, params
@@ -170,12 +175,13 @@ class _Unit:
         self.arrived = 0
         self.rs = None  # reduce-scatter in flight
         self.staging = None
+        self.peer_offsets = None
 
 
 class FSDP(torch.nn.Module):
     """ZeRO stage 3 over model.units()."""
 
-    def __init__(self, model, group, optimizer=None, prefetch=True):
+    def __init__(self, model, group, optimizer=None, prefetch=True, direct=None):
         super().__init__()
         _need(group, "pack", "gather_unit")
         self.module, self.g = model, group
@@ -188,6 +194,26 @@ class FSDP(torch.nn.Module):
         self.max_live = 0
         self.units, self.unit_of = [], {}
         claimed = set()
+        # Where the group offers it, all shards live in one arena that the other ranks
+        # map once and read directly: a gather is then copies only, with a fence()
+        # around the optimizer step instead of a handshake per gather.
+        self._direct = direct if direct is not None else hasattr(group, "shared_empty")
+        arena, arena_at, self._peer_at = None, 0, [0] * group.size
+        if self._direct:
+            from .buckets import FlatLayout as _L
+
+            mods = model.units()
+            seen, total = set(), [0] * group.size
+            for m in mods:
+                ps = [p for p in m.parameters() if p.requires_grad and id(p) not in seen]
+                seen.update(id(p) for p in ps)
+                sizes = _L([p.numel() for p in ps], group.size, 0).sizes
+                total = [t + _pad(s) for t, s in zip(total, sizes)]
+            p0 = next(model.parameters())
+            try:
+                arena = group.shared_empty(max(total), p0.dtype)
+            except Exception:
+                self._direct, arena = False, None  # too large for one IPC allocation: stage through the slots
         for i, m in enumerate(model.units()):
             ps = [p for p in m.parameters() if p.requires_grad and id(p) not in claimed]
             claimed.update(id(p) for p in ps)
@@ -198,7 +224,14 @@ class FSDP(torch.nn.Module):
                 for p in ps:
                     o = u.offset[p]
                     p.data = u.full[o:o + p.numel()].view_as(p)
-                u.shard = u.full[u.flat.lo:u.flat.hi].clone()
+                if arena is not None:
+                    es = u.full.element_size()
+                    u.shard = arena[self._peer_at[group.rank]:self._peer_at[group.rank] + (u.flat.hi - u.flat.lo)]
+                    u.shard.copy_(u.full[u.flat.lo:u.flat.hi])
+                    u.peer_offsets = [at * es for at in self._peer_at]  # this unit's shard in every rank's arena, bytes
+                    self._peer_at = [at + _pad(s) for at, s in zip(self._peer_at, u.flat.sizes)]
+                else:
+                    u.shard = u.full[u.flat.lo:u.flat.hi].clone()
             for p in ps:
                 self.unit_of[p] = u
                 p.register_post_accumulate_grad_hook(self._on_grad)
@@ -212,6 +245,8 @@ class FSDP(torch.nn.Module):
             raise ValueError("every parameter must belong to one of model.units()")
         self._callback_queued = False
         self.max_live = 0
+        if self._direct:
+            self.g.fence()  # every rank's shards are in place before anyone gathers
 
     def forward(self, *args, **kwargs):
         return self.module(*args, **kwargs)
@@ -223,7 +258,10 @@ class FSDP(torch.nn.Module):
         u.full.untyped_storage().resize_(u.nbytes)
         self.live += 1
         self.max_live = max(self.max_live, self.live)
-        u.pending = self.g.gather_unit(u.full, u.shard, u.flat.sizes, async_op=True)
+        if self._direct:
+            u.pending = self.g.gather_unit(u.full, u.shard, u.flat.sizes, async_op=True, peer_offsets=u.peer_offsets)
+        else:
+            u.pending = self.g.gather_unit(u.full, u.shard, u.flat.sizes, async_op=True)
 
     def _ensure(self, u):
         self._start(u)
@@ -298,8 +336,12 @@ class FSDP(torch.nn.Module):
 
     @torch.no_grad()
     def step(self):
+        if self._direct:
+            self.g.fence()  # no rank still reads the shards this step rewrites
         for u in self.units:
             self.opt.update(u.index, u.shard, u.grad_shard)
+        if self._direct:
+            self.g.fence()  # the new shards are complete before any rank gathers them
 
     def zero_grad(self):
         for u in self.units:
@@ -311,6 +353,9 @@ class FSDP(torch.nn.Module):
         out = []
         for u in self.units:
             full = torch.empty(u.flat.numel, device=u.shard.device, dtype=u.shard.dtype)
-            self.g.gather_unit(full, u.shard, u.flat.sizes)
+            if self._direct:
+                self.g.gather_unit(full, u.shard, u.flat.sizes, peer_offsets=u.peer_offsets)
+            else:
+                self.g.gather_unit(full, u.shard, u.flat.sizes)
             out.append(full)
         return torch.cat(out)

@@ -123,6 +123,46 @@ def test_reference_fixtures(world):
             assert np.array_equal(bits(got), bits(d[f"r{r}_{key}"])), (world, r, key)
 
 
+def direct_gather(g, numel):
+    """Shards in the shared arena, read directly by the peers; fences around every rewrite."""
+    w, r = g.size, g.rank
+    sizes = [numel // w + (1 if q < numel % w else 0) for q in range(w)]
+    pad = lambda n: (n + 3) // 4 * 4
+    arena = g.shared_empty(2 * max(pad(s) for s in sizes) + 8)
+    offs = [0] * w                               # unit 0 sits at the start of every arena
+    offs2 = [pad(s) * 4 for s in sizes]          # unit 1 right behind it (bytes)
+    mine, mine2 = arena[:sizes[r]], arena[pad(sizes[r]):pad(sizes[r]) + sizes[r]]
+    out = []
+    for round_ in range(3):
+        g.fence()
+        mine.copy_(values(r + 10 * round_, sizes[r], torch.float32).to(g.device))
+        mine2.copy_(values(r + 10 * round_ + 5, sizes[r], torch.float32).to(g.device))
+        g.fence()
+        full = torch.full((numel,), -7.0, device=g.device)
+        full2 = torch.full((numel,), -7.0, device=g.device)
+        wk = g.gather_unit(full, mine, sizes, async_op=True, peer_offsets=offs)
+        g.gather_unit(full2, mine2, sizes, peer_offsets=offs2)
+        wk.wait()
+        out.append((full.cpu(), full2.cpu()))
+    assert g.arena_offset(mine2) == pad(sizes[r]) * 4 and g.arena_offset(torch.zeros(4, device=g.device)) is None
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("world", [2, 3])
+def test_direct_gather_from_shared_arenas(world):
+    from tandem_amd import launch
+
+    numel = 100_003
+    sizes = [numel // world + (1 if q < numel % world else 0) for q in range(world)]
+    res = launch(direct_gather, world, numel, gpus=[0] * world, timeout=TIMEOUT)
+    for out in res:
+        for round_, (full, full2) in enumerate(out):
+            want = torch.cat([values(q + 10 * round_, sizes[q], torch.float32) for q in range(world)])
+            want2 = torch.cat([values(q + 10 * round_ + 5, sizes[q], torch.float32) for q in range(world)])
+            assert torch.equal(full, want) and torch.equal(full2, want2), round_
+
+
 def async_order(g):
     # several collectives in flight complete in submission order with the right values
     xs = [torch.full((3000 + k,), float(g.rank + k), device=g.device) for k in range(5)]

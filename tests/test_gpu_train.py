@@ -45,8 +45,12 @@ def train_rank(g, strategy, bucket_bytes, steps, batch):
         opt = torch.optim.AdamW(model.parameters(), lr=LR, weight_decay=WD, foreach=False, fused=False)
     else:
         sopt = ShardedAdamW(lr=LR, weight_decay=WD, order="device")  # torch's GPU op order, to compare with torch.optim.AdamW
-        stage = int(strategy[-1])
-        z = ZeRO(model, g, stage, sopt, bucket_bytes) if stage < 3 else FSDP(model, g, sopt)
+        stage = int(strategy[4])
+        if stage < 3:
+            z = ZeRO(model, g, stage, sopt, bucket_bytes)
+        else:  # "zero3": shards in the shared arena, gathered directly; "zero3s": staged through the slots
+            z = FSDP(model, g, sopt, direct=not strategy.endswith("s"))
+            assert z._direct == (not strategy.endswith("s"))
     losses = []
     for step in range(steps):
         x, y = text.batch(step, batch, c.seq, rank=g.rank, world=g.size, device=g.device)
@@ -59,7 +63,7 @@ def train_rank(g, strategy, bucket_bytes, steps, batch):
         else:
             z.step()
             z.zero_grad()
-    if strategy == "zero3":
+    if strategy.startswith("zero3"):
         w = z.full_parameters()
         extra = {"max_live": z.max_live, "live": z.live}
     else:
@@ -102,14 +106,15 @@ def test_two_ranks_all_strategies_agree_bit_for_bit():
     from tandem_amd import launch
 
     runs = {s: launch(train_rank, 2, s, 4 << 10, STEPS, BATCH, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT)
-            for s in ("ddp", "zero1", "zero2", "zero3")}
+            for s in ("ddp", "zero1", "zero2", "zero3", "zero3s")}
     ref_losses, ref_w = one_process(2)
     for s, res in runs.items():
         assert torch.equal(res[0]["weights"], res[1]["weights"]), f"{s}: the ranks drifted apart"
         for r in range(2):
             assert res[r]["losses"] == ref_losses[r], (s, r)
             assert torch.equal(res[r]["weights"], ref_w), (s, r)
-    assert runs["zero3"][0]["max_live"] <= 3 and runs["zero3"][0]["live"] == 0
+    for s in ("zero3", "zero3s"):
+        assert runs[s][0]["max_live"] <= 3 and runs[s][0]["live"] == 0
 
 
 def test_four_ranks_stay_in_step():
@@ -119,12 +124,12 @@ def test_four_ranks_stay_in_step():
     more than three units whole."""
     from tandem_amd import launch
 
-    for s in ("ddp", "zero2", "zero3"):
+    for s in ("ddp", "zero2", "zero3", "zero3s"):
         res = launch(train_rank, 4, s, 4 << 10, 6, 8, slot_bytes=1024, gpus=[0] * 4, timeout=TIMEOUT)
         for r in range(1, 4):
             assert torch.equal(res[0]["weights"], res[r]["weights"]), (s, r)
         mean_first = sum(res[r]["losses"][0] for r in range(4)) / 4
         mean_last = sum(res[r]["losses"][-1] for r in range(4)) / 4
         assert mean_last < mean_first, s
-        if s == "zero3":
+        if s.startswith("zero3"):
             assert all(x["max_live"] <= 3 and x["live"] == 0 for x in res)
