@@ -226,6 +226,28 @@ def test_error_propagates_from_a_rank():
         launch(failing, 2, gpus=[0, 0], timeout=10.0)
 
 
+def out_of_step(g):
+    from tandem_amd import CommError
+
+    x = torch.ones(1000, device=g.device)
+    if g.rank == 0:
+        try:
+            g.all_reduce(x)  # rank 1 never joins: the wait for its piece must time out, on the host
+        except CommError as e:
+            return "timed out" in str(e.__cause__)
+        return False
+    return True
+
+
+def test_a_missing_peer_times_out_on_the_host():
+    """Forced from the host: every kernel that was launched still finishes; the
+    progress thread gives up waiting for a message after the group's timeout."""
+    from tandem_amd import launch
+
+    with pytest.raises(Exception, match="timed out|barrier|drained"):
+        launch(out_of_step, 2, gpus=[0, 0], timeout=3.0)
+
+
 def test_unknown_backend_and_cpu_device_are_refused():
     from tandem_amd import CommError, Group, launch
 
