@@ -11,7 +11,7 @@ starts (world size 4 on one GPU). Prints ONE JSON line:
               element per launch / the launch's duration, taken from HIP events
               recorded around the three back-to-back K1 launches of every timed
               step, against the 8 TB/s HBM peak; `traffic` is the HBM traffic per
-              launch measured with rocprofv3 counters (profiles/)
+              launch measured with rocprofv3 counters
   sweep       message sizes 64 KiB .. 256 MiB, ring and single-launch fold
   bucket_path DDP's bucket flatten+average+unflatten (K2), 85.8M params, world 2
   zero2_step  reduce-scatter + AdamW + all-gather, 85.8M params, world 4
@@ -37,7 +37,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X, published
 WORLD = 4
 # HBM bytes per K1 launch at the default workload (4 chunk pairs of 64 MiB), from
 # rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads for
-# the plain copy kernel of known size in the same run (profiles/k1_reduce_*.txt).
+# the plain copy kernel of known size in the same run: FETCH_SIZE x 1.99965 + WRITE_SIZE x 1.0.
 K1_TRAFFIC_256MIB = 805_279_000
 
 

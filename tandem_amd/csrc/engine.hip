@@ -351,7 +351,11 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
       free_[p].resize(slots_);
       for (int j = 0; j < slots_; ++j) {
         check_hip(hipEventCreateWithFlags(&full_[p][j], kFlags), "hipEventCreateWithFlags (full)");
-        check_hip(hipIpcGetEventHandle(&e->full[j], full_[p][j]), "hipIpcGetEventHandle (full)");
+        if (hipIpcGetEventHandle(&e->full[j], full_[p][j]) != hipSuccess) {
+          (void)hipGetLastError();
+          throw std::runtime_error("TANDEM_HIP_SYNC=event: this platform cannot export interprocess events "
+                                   "(hipIpcGetEventHandle failed); use the default host ordering");
+        }
         check_hip(hipEventCreateWithFlags(&free_[p][j], kFlags), "hipEventCreateWithFlags (free)");
         check_hip(hipIpcGetEventHandle(&e->free_[j], free_[p][j]), "hipIpcGetEventHandle (free)");
       }

@@ -215,7 +215,7 @@ def test_bad_arguments_raise(dev):
 
 
 def test_full_size_properties(dev):
-    """BASELINE's largest case: four ranks x 64 Mi fp32 (256 MiB each). The
+    """The benchmark's largest case: four ranks x 64 Mi fp32 (256 MiB each). The
     oracle is too slow for all of it, so: every rank ends with the same bits,
     integer-valued inputs sum exactly, a power-of-two scaling of the inputs
     scales the result exactly, and a strided sample is checked against the
