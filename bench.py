@@ -17,6 +17,8 @@ starts (world size 4 on one GPU). Prints ONE JSON line:
   zero2_step  reduce-scatter + AdamW + all-gather, 85.8M params, world 4
   fsdp_gather two processes sharing the GPU through HIP IPC: ZeRO-3 unit gathers
               of the 85.8M GPT, prefetched on the engine's stream
+  ipc_allreduce_2_processes  Group(backend="hip") all_reduce between two processes
+              sharing the GPU, the reference's one-GPU engine protocol and sizes
   cpu_baseline  the oracle's CPU-process engine (tandem's Python-engine protocol:
               one process per rank, 1 torch thread each, 2 x 4 MiB shared-memory
               slots per pair) on this box's host cores, same formula for GB/s
@@ -255,6 +257,40 @@ def fsdp_gather(steps):
     return out
 
 
+def ipc_rank(g, sizes_kib, reps):
+    """The reference's one-GPU engine benchmark (bench/engine_one_gpu.py there):
+    barrier, then time all_reduce + device sync; median."""
+    import torch
+
+    out = {}
+    for kib in sizes_kib:
+        x = torch.ones(kib * 1024 // 4, device=g.device)
+        g.all_reduce(x)
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(reps):
+            g.barrier()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            g.all_reduce(x)
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t)
+        out[kib] = statistics.median(ts)
+    return out
+
+
+def ipc_allreduce():
+    from tandem_amd import launch
+
+    sizes = [64, 256, 1024, 4096, 16384, 65536]
+    out = {"workload": "all_reduce(sum) fp32 between 2 processes sharing the GPU through HIP IPC, barrier + all_reduce + device sync, median of 20",
+           "reference_T4_cpp_engine_ms": {"64": 0.64, "256": 0.80, "1024": 0.83, "4096": 0.75, "16384": 1.72, "65536": 6.24}}
+    for label, slot in (("slots_2x4MiB_ms", 4 << 20), ("slots_2x64MiB_ms", 64 << 20)):
+        res = launch(ipc_rank, 2, sizes, 20, slot_bytes=slot, gpus=[0, 0], timeout=120.0)[0]
+        out[label] = {str(k): round(v * 1e3, 3) for k, v in res.items()}
+    return out
+
+
 # ---------------------------------------------------------------- CPU baseline
 def cpu_rank(g, n, reps, numels):
     """Timed on the host: (i) the ring all-reduce(avg) of the GPU's main workload,
@@ -344,11 +380,16 @@ def main():
     cpu = fsdp = None
     if not args.quick and not args.no_cpu:
         cpu = cpu_baseline(args.mib, 15)
+    ipc = None
     if not args.quick and not args.no_fsdp:
         try:
             fsdp = fsdp_gather(3)
         except Exception as e:  # a secondary figure must not lose the line
             fsdp = {"error": repr(e)[:300]}
+        try:
+            ipc = ipc_allreduce()
+        except Exception as e:
+            ipc = {"error": repr(e)[:300]}
 
     import torch
 
@@ -399,6 +440,8 @@ def main():
         torch.cuda.empty_cache()
         if fsdp is not None:
             line["fsdp_gather"] = fsdp
+        if ipc is not None:
+            line["ipc_allreduce_2_processes"] = ipc
         if cpu is not None:
             cpu["gpu_over_cpu"] = round(line["value"] / cpu["value"], 1)
             cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["ms"], 1)

@@ -592,7 +592,15 @@ void Engine::completion_loop() {
       cbusy_ = true;
     }
     if (c.after) {
-      hipError_t err = hipEventSynchronize(c.after);
+      // Short kernels finish within microseconds: poll first, then block.
+      hipError_t err = hipErrorNotReady;
+      const auto spin_until = std::chrono::steady_clock::now() + std::chrono::microseconds(200);
+      while ((err = hipEventQuery(c.after)) == hipErrorNotReady && std::chrono::steady_clock::now() < spin_until) {
+      }
+      if (err == hipErrorNotReady) {
+        (void)hipGetLastError();
+        err = hipEventSynchronize(c.after);
+      }
       (void)hipEventDestroy(c.after);
       if (err != hipSuccess) {  // do not publish: the peers time out rather than read bad bytes
         std::lock_guard<std::mutex> lock(cmu_);
