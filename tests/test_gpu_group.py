@@ -99,6 +99,52 @@ def test_collectives_bit_exact(dtype, world):
         assert out["bool_bcast_ok"]
 
 
+def tiny_slots(g, sizes_list):
+    """The reference's tests/test_comm.py shape: integer-valued data, 64-byte slots,
+    so that every message travels in many pieces and every slot is reused."""
+    r, w = g.rank, g.size
+    ok = True
+    for dtype in (torch.float32, torch.int64, torch.bfloat16):
+        hi = 30 if dtype == torch.bfloat16 else 100
+        for n in sizes_list:
+            def data(q, seed=0):
+                gen = torch.Generator().manual_seed(seed * 1000 + q)
+                return torch.randint(-hi, hi, (n,), generator=gen).to(dtype)
+            want = sum(data(q).double() for q in range(w)) if n else torch.zeros(0, dtype=torch.float64)
+            x = data(r).to(g.device)
+            g.all_reduce(x)
+            ok &= torch.equal(x.cpu().double(), want)
+            sizes = [n // w] * w
+            sizes[-1] += n - sum(sizes)
+            sizes = sizes[1:] + sizes[:1]  # uneven chunks, one of them empty when n < w
+            x = data(r).to(g.device)
+            mine = g.reduce_scatter(x, sizes)
+            lo = sum(sizes[:r])
+            ok &= torch.equal(mine.cpu().double(), want[lo:lo + sizes[r]])
+            full = want.to(dtype)
+            x = torch.full((n,), -7, dtype=dtype)
+            x[lo:lo + sizes[r]] = full[lo:lo + sizes[r]]
+            x = x.to(g.device)
+            g.all_gather(x, sizes)
+            ok &= torch.equal(x.cpu(), full)
+            x = data(r, seed=1).to(g.device)
+            g.broadcast(x, root=w - 1)
+            ok &= torch.equal(x.cpu(), data(w - 1, seed=1))
+    x = torch.arange(37, dtype=torch.float32, device=g.device) * (r + 1)
+    g.all_reduce(x, op="avg")
+    want = sum(torch.arange(37, dtype=torch.float64) * (q + 1) for q in range(w)) / w
+    ok &= torch.allclose(x.cpu().double(), want, rtol=0, atol=1e-5)
+    torch.cuda.synchronize()
+    return bool(ok)
+
+
+@pytest.mark.parametrize("world", [2, 3])
+def test_many_pieces_through_64_byte_slots(world):
+    from tandem_amd import launch
+
+    assert launch(tiny_slots, world, [0, 1, 5, 64, 1000], slot_bytes=64, gpus=[0] * world, timeout=TIMEOUT) == [True] * world
+
+
 def replay_fixture(g, inputs, cases):
     x = torch.from_numpy(inputs[g.rank].copy()).to(g.device)
     out = {}
