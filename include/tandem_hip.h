@@ -260,11 +260,20 @@ int tdm_barrier(tdm_engine* e, tdm_work** out);
  * wait: blocks the host until the collective's GPU work has been enqueued, then
  * makes `caller` wait for it on the GPU; returns the collective's error, if any.
  * done: 1 once the GPU has finished it. times: when the progress thread started and
- * finished it, seconds on CLOCK_MONOTONIC (Python's time.perf_counter clock). */
+ * finished it, seconds on CLOCK_MONOTONIC (Python's time.perf_counter clock); for a
+ * collective submitted while tdm_engine_set_timing was on, when the GPU started it
+ * (inputs ready, first kernel not yet begun) and finished its last kernel instead, on
+ * the same clock: this form blocks the host until the GPU has finished it. */
 int tdm_work_wait(tdm_work* w, tdm_stream caller);
 int tdm_work_done(tdm_work* w);
 int tdm_work_times(tdm_work* w, double* started, double* finished);
 int tdm_work_free(tdm_work* w);
+
+/* Device time stamps for the collectives submitted from now on (on != 0) or host
+ * time stamps as the reference's engine keeps them (tandem/csrc/collectives.cpp:203-223;
+ * the default). Feeds Group.trace (tandem/comm.py:101-102) so that tandem/profile.py's
+ * summarize and chrome_trace see the GPU's span of each collective. */
+int tdm_engine_set_timing(tdm_engine* e, int on);
 
 #ifdef __cplusplus
 }

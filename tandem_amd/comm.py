@@ -55,9 +55,7 @@ class Work:
         if t0 is not None:
             g.waits.append((self.name, t0, time.perf_counter()))
         if g.tracing and not self._recorded:
-            a, b = ctypes.c_double(0), ctypes.c_double(0)
-            lib().tdm_work_times(self._handle, ctypes.byref(a), ctypes.byref(b))
-            g.trace.append((self.name, a.value, b.value, self._nbytes))  # steady clock == perf_counter's clock
+            g._untimed.append(self)  # its span is read when Group.trace is next looked at
         self._recorded = True
         self._waited = True
         return self.result
@@ -85,7 +83,7 @@ class Group:
         self.transport = transport or "device"
         self.priority = 0  # every stream here runs at the default priority
         self.backend = backend or DEFAULT_BACKEND
-        self.trace, self.waits, self.tracing = [], [], False
+        self._trace, self._untimed, self.waits, self._tracing = [], [], [], False
         self._closed = False
         self._engine = None
         self._arena = None
@@ -112,6 +110,43 @@ class Group:
         except Exception as e:
             raise CommError(f"could not start the hip engine: {e}") from e
         self.barrier()
+
+    # ---- tracing (tandem/comm.py:132-134 there: trace, waits, tracing)
+    @property
+    def tracing(self):
+        return self._tracing
+
+    @tracing.setter
+    def tracing(self, on):
+        """While on, every collective waited for leaves (name, start, end, bytes) in
+        `trace` and the time its caller was blocked in `waits`, on time.perf_counter's
+        clock. start and end are the GPU's: from the moment the inputs were ready on
+        the engine's stream to the end of the collective's last kernel (device time
+        stamps placed on the host clock), unless TANDEM_HIP_TRACE=host asks for the
+        progress thread's own start and end as the reference's engine records them
+        (tandem/csrc/collectives.cpp:203-223)."""
+        self._tracing = bool(on)
+        if self._engine is not None and os.environ.get("TANDEM_HIP_TRACE", "device") != "host":
+            check(lib().tdm_engine_set_timing(self._engine, 1 if on else 0))
+
+    @property
+    def trace(self):
+        # Reading a device time stamp waits for that collective's last kernel, so the
+        # spans are filled in here, when somebody looks, and not inside wait().
+        pending, self._untimed = self._untimed, []
+        for w in pending:
+            a, b = ctypes.c_double(0), ctypes.c_double(0)
+            try:
+                check(lib().tdm_work_times(w._handle, ctypes.byref(a), ctypes.byref(b)))
+            except Exception as e:
+                raise CommError(f"{w.name}: could not read its time stamps") from e
+            self._trace.append((w.name, a.value, b.value, w._nbytes))  # steady clock == perf_counter's clock
+        return self._trace
+
+    @trace.setter
+    def trace(self, spans):
+        self._untimed = []
+        self._trace = spans
 
     # ---- plumbing
     def _start(self, name, call, result, nbytes, async_op, keep=()):
@@ -328,6 +363,7 @@ class Group:
     def close(self):
         if self._closed:
             return
+        self.trace  # spans still owed are read while the engine is alive
         self.barrier()
         self._closed = True
         eng, self._engine = self._engine, None
@@ -343,6 +379,7 @@ class Group:
         """After a failure on this rank: drop the engine without the closing
         handshake (the other ranks time out or fail on their own)."""
         self._closed = True
+        self._untimed = []
         eng, self._engine = self._engine, None
         if eng is not None:
             lib().tdm_engine_destroy(eng)

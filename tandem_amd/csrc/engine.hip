@@ -195,6 +195,16 @@ void wait_until(Ready ready, double timeout_s, const char* what) {
 }  // namespace
 
 // ---------------------------------------------------------------- Work
+// A point that is known on both clocks: the event was recorded on the engine's
+// stream and waited for, and `host` was read right after.
+struct Anchor {
+  hipEvent_t event = nullptr;
+  double host = 0;
+  ~Anchor() {
+    if (event) (void)hipEventDestroy(event);
+  }
+};
+
 struct Work {
   std::mutex mu;
   std::condition_variable cv;
@@ -204,11 +214,18 @@ struct Work {
   double t0 = 0, t1 = 0;
   hipEvent_t done_event = nullptr;  // recorded on the engine's stream after the job
   int device = -1;
+  // Device timing (only while the engine's timing switch is on): start_event is
+  // recorded on the engine's stream once the inputs are ready; both events carry
+  // time stamps, placed on the host clock through the engine's anchor.
+  hipEvent_t start_event = nullptr;
+  std::shared_ptr<Anchor> anchor;
 
   ~Work() {
     if (done_event) (void)hipEventDestroy(done_event);
+    if (start_event) (void)hipEventDestroy(start_event);
   }
 };
+
 
 // ---------------------------------------------------------------- Engine
 class Engine {
@@ -217,6 +234,7 @@ class Engine {
   ~Engine();
   void connect();
   void close();
+  void set_timing(bool on) { timing_.store(on ? 1 : 0, std::memory_order_release); }
 
   struct Buf {
     char* ptr;
@@ -248,6 +266,7 @@ class Engine {
   };
 
   std::shared_ptr<Work> submit(std::function<void()> job, hipStream_t caller, bool uses_gpu);
+  void stamp_start(Work& w);
   void loop();
   void check(const Buf& t, const char* what, bool reduce) const;
   std::vector<Chunk> chunks(const Buf& t, const std::vector<int64_t>& sizes) const;
@@ -286,6 +305,9 @@ class Engine {
   std::vector<uint64_t> posted_;         // messages queued or published to each peer (flow control)
   std::vector<uint64_t> taken_;          // messages consumed from each peer
   bool connected_ = false, closed_ = false;
+  std::atomic<int> timing_{0};
+  bool timing_seen_ = false;           // progress thread only
+  std::shared_ptr<Anchor> anchor_;     // progress thread only
 
   // "host" ordering: what to publish once the GPU has passed an event.
   struct Completion {
@@ -472,10 +494,11 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
       (void)hipEventDestroy(ready);
       check_hip(err, "hipEventRecord (ready)");
     }
-    job = [this, ready, inner = std::move(job)] {
+    job = [this, ready, w = work.get(), inner = std::move(job)] {
       hipError_t e = hipStreamWaitEvent(stream_, ready, 0);
       (void)hipEventDestroy(ready);  // released once the GPU is past it
       check_hip(e, "hipStreamWaitEvent (ready)");
+      stamp_start(*w);
       inner();
     };
   }
@@ -486,6 +509,29 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
   }
   cv_.notify_one();
   return work;
+}
+
+// With timing on: a time-stamped event on the engine's stream, after the wait for
+// the inputs and before the collective's first kernel. A fresh anchor is taken
+// each time the switch goes on, so the two clocks cannot drift far apart.
+void Engine::stamp_start(Work& w) {
+  const bool on = timing_.load(std::memory_order_acquire) != 0;
+  if (!on) {
+    timing_seen_ = false;
+    return;
+  }
+  if (!timing_seen_ || !anchor_) {
+    auto a = std::make_shared<Anchor>();
+    check_hip(hipEventCreateWithFlags(&a->event, hipEventDefault), "hipEventCreate (anchor)");
+    check_hip(hipEventRecord(a->event, stream_), "hipEventRecord (anchor)");
+    check_hip(hipEventSynchronize(a->event), "hipEventSynchronize (anchor)");
+    a->host = now_s();
+    anchor_ = std::move(a);
+    timing_seen_ = true;
+  }
+  check_hip(hipEventCreateWithFlags(&w.start_event, hipEventDefault), "hipEventCreate (start)");
+  check_hip(hipEventRecord(w.start_event, stream_), "hipEventRecord (start)");
+  w.anchor = anchor_;
 }
 
 void Engine::loop() {
@@ -515,7 +561,7 @@ void Engine::loop() {
       status = TDM_ERUNTIME; error = "unknown error";
     }
     if (status == TDM_OK) {
-      if (hipEventCreateWithFlags(&w.done_event, hipEventDisableTiming) != hipSuccess ||
+      if (hipEventCreateWithFlags(&w.done_event, w.start_event ? hipEventDefault : hipEventDisableTiming) != hipSuccess ||
           hipEventRecord(w.done_event, stream_) != hipSuccess) {
         status = TDM_ERUNTIME;
         error = "could not record the collective's completion event";
@@ -1148,9 +1194,31 @@ int tdm_work_times(tdm_work* w, double* started, double* finished) {
     set_last_error("NULL work");
     return TDM_EINVAL;
   }
-  std::lock_guard<std::mutex> lock(w->impl->mu);
-  if (started) *started = w->impl->t0;
-  if (finished) *finished = w->impl->t1;
+  Work& work = *w->impl;
+  {
+    std::unique_lock<std::mutex> lock(work.mu);
+    work.cv.wait(lock, [&] { return work.finished; });
+    if (started) *started = work.t0;
+    if (finished) *finished = work.t1;
+    if (work.status != TDM_OK || !work.start_event || !work.done_event || !work.anchor) return TDM_OK;
+  }
+  // Timed on the device: wait for its last kernel, then place both stamps on the host clock.
+  return guard([&] {
+    check_hip(hipEventSynchronize(work.done_event), "hipEventSynchronize (times)");
+    float ms0 = 0, ms1 = 0;
+    check_hip(hipEventElapsedTime(&ms0, work.anchor->event, work.start_event), "hipEventElapsedTime (start)");
+    check_hip(hipEventElapsedTime(&ms1, work.anchor->event, work.done_event), "hipEventElapsedTime (done)");
+    if (started) *started = work.anchor->host + static_cast<double>(ms0) * 1e-3;
+    if (finished) *finished = work.anchor->host + static_cast<double>(ms1) * 1e-3;
+  });
+}
+
+int tdm_engine_set_timing(tdm_engine* e, int on) {
+  if (e == nullptr || !e->impl) {
+    set_last_error("NULL engine");
+    return TDM_EINVAL;
+  }
+  e->impl->set_timing(on != 0);
   return TDM_OK;
 }
 

@@ -148,26 +148,26 @@ __device__ __forceinline__ vec16 pack(const Lanes<T>& in) {
 // L2 / Infinity Cache), a stream that is read, modified and written back does best
 // with plain loads and plain stores (the store hits the line the load brought in).
 // Both non-temporal: 6.4 TB/s; both plain: 5.4; this split: 7.0.
-// -DTDM_TEMPORAL=1 builds the all-plain variant, =0 the all-non-temporal one.
-#ifndef TDM_TEMPORAL
-#define TDM_TEMPORAL 4
+// -DTDM_NT_MASK=<0..7> builds the other combinations for measurement.
+#ifndef TDM_NT_MASK
+#define TDM_NT_MASK 2  // bit0: read-modify-write loads, bit1: read-once loads, bit2: stores are non-temporal
 #endif
 __device__ __forceinline__ vec16 load_stream(const void* p) {  // read once, never written here
-#if TDM_TEMPORAL == 1
-  return *static_cast<const vec16*>(p);
-#else
+#if TDM_NT_MASK & 2
   return __builtin_nontemporal_load(static_cast<const vec16*>(p));
+#else
+  return *static_cast<const vec16*>(p);
 #endif
 }
 __device__ __forceinline__ vec16 load_rmw(const void* p) {  // about to be overwritten by this lane
-#if TDM_TEMPORAL == 0
+#if TDM_NT_MASK & 1
   return __builtin_nontemporal_load(static_cast<const vec16*>(p));
 #else
   return *static_cast<const vec16*>(p);
 #endif
 }
 __device__ __forceinline__ void store16(void* p, const vec16& v) {
-#if TDM_TEMPORAL == 0
+#if TDM_NT_MASK & 4
   __builtin_nontemporal_store(v, static_cast<vec16*>(p));
 #else
   *static_cast<vec16*>(p) = v;

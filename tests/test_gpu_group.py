@@ -234,6 +234,67 @@ def test_async_and_large_message_default_slots():
     assert launch(async_order, 3, gpus=[0, 0, 0], timeout=TIMEOUT) == [True, True, True]
 
 
+def traced(g, mib, gemms):
+    """The reference's protocol for a collective's own time (bench/engine_one_gpu.py
+    there: the span from Group.trace while the default stream is idle, then while
+    it runs matmuls the collective does not depend on)."""
+    import time
+
+    from tandem_amd.profile import summarize
+
+    n = mib * (1 << 20) // 4
+    x = torch.ones(n, device=g.device)
+    a = torch.randn(2048, 2048, device=g.device)
+    g.all_reduce(x)
+    a @ a
+    torch.cuda.synchronize()
+    chunk = 4 * n / g.size
+    floor = (g.size - 1) * (8 + 12 + 8 + 8) * chunk / 8e12  # this rank's own copies and reduces at HBM peak
+    out = {}
+    for mode in ("idle", "busy", "host"):
+        os.environ["TANDEM_HIP_TRACE"] = "host" if mode == "host" else "device"
+        g.barrier()
+        x.fill_(1.0)
+        torch.cuda.synchronize()
+        g.trace.clear()
+        g.waits.clear()
+        g.tracing = True
+        t = time.perf_counter()
+        w = g.all_reduce(x, async_op=True)
+        for _ in range(gemms if mode == "busy" else 0):
+            a @ a
+        w.wait()
+        waited = time.perf_counter()
+        torch.cuda.synchronize()
+        end = time.perf_counter()
+        g.tracing = False
+        assert len(g.trace) == 1
+        name, s, e, nbytes = g.trace[-1]
+        assert name == "all_reduce" and nbytes == 4 * n
+        assert torch.equal(x, torch.full_like(x, float(g.size)))
+        if mode == "host":  # the progress thread's own clock readings
+            assert t <= s <= e <= end
+        else:  # the GPU's span, on the host's clock: inside the bracket, no shorter than the traffic allows
+            assert t - 1e-3 <= s <= e <= end + 1e-3, (mode, s - t, e - t, end - t)
+            assert e - s >= floor, (mode, e - s, floor)
+        summary = summarize([], g.trace, list(g.waits), end - t)
+        assert summary["comm_bytes"] == 4 * n and abs(summary["comm_s"] - (e - s)) < 1e-12
+        assert summary["exposed_comm_s"] <= summary["comm_s"] + 1e-12 and 0.0 <= summary["overlap"] <= 1.0
+        out[mode] = {"span_ms": (e - s) * 1e3, "wait_returned_ms": (waited - t) * 1e3, "total_ms": (end - t) * 1e3}
+    os.environ.pop("TANDEM_HIP_TRACE", None)
+    return out
+
+
+def test_trace_holds_the_gpu_span_of_a_collective():
+    from tandem_amd import launch
+
+    res = launch(traced, 2, 64, 40, gpus=[0, 0], timeout=TIMEOUT)
+    print("\ntrace of a 64 MiB all_reduce, 2 ranks:", res[0])
+    for r in res:
+        # behind 40 matmuls the collective still finishes long before they do
+        assert r["busy"]["span_ms"] < r["busy"]["total_ms"]
+
+
 def errors(g):
     from tandem_amd import CommError
 
