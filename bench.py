@@ -257,22 +257,26 @@ def fsdp_gather(steps):
     return out
 
 
-def ipc_rank(g, sizes_kib, reps):
+def ipc_rank(g, sizes_kib, reps, direct=False):
     """The reference's one-GPU engine benchmark (bench/engine_one_gpu.py there):
-    barrier, then time all_reduce + device sync; median."""
+    barrier, then time all_reduce + device sync; median. direct: the tensor lives in
+    the ranks' shared arenas and is reduced arena to arena, without slots."""
     import torch
 
     out = {}
+    if direct:
+        g.share_arena(max(sizes_kib) * 1024 + 4096)
+        pool = g.shared_empty(max(sizes_kib) * 1024 // 4)
     for kib in sizes_kib:
-        x = torch.ones(kib * 1024 // 4, device=g.device)
-        g.all_reduce(x)
+        x = pool[:kib * 1024 // 4].fill_(1.0) if direct else torch.ones(kib * 1024 // 4, device=g.device)
+        g.all_reduce(x, direct=direct)
         torch.cuda.synchronize()
         ts = []
         for _ in range(reps):
             g.barrier()
             torch.cuda.synchronize()
             t = time.perf_counter()
-            g.all_reduce(x)
+            g.all_reduce(x, direct=direct)
             torch.cuda.synchronize()
             ts.append(time.perf_counter() - t)
         out[kib] = statistics.median(ts)
@@ -288,6 +292,8 @@ def ipc_allreduce():
     for label, slot in (("slots_2x4MiB_ms", 4 << 20), ("slots_2x64MiB_ms", 64 << 20)):
         res = launch(ipc_rank, 2, sizes, 20, slot_bytes=slot, gpus=[0, 0], timeout=120.0)[0]
         out[label] = {str(k): round(v * 1e3, 3) for k, v in res.items()}
+    res = launch(ipc_rank, 2, sizes, 20, True, gpus=[0, 0], timeout=120.0)[0]
+    out["direct_arena_ms"] = {str(k): round(v * 1e3, 3) for k, v in res.items()}
     return out
 
 

@@ -252,6 +252,26 @@ int tdm_engine_share(tdm_engine* e, int64_t bytes, void** ptr);
 int tdm_unit_gather_direct(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes,
                            int nsizes, const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out);
 int tdm_fence(tdm_engine* e, tdm_stream caller, tdm_work** out);
+
+/* The three collectives for tensors that lie in the ranks' shared arenas (this rank's
+ * at `ptr`, rank q's at byte offset peer_offsets[q] of its arena), with the results of
+ * tdm_all_reduce / tdm_reduce_scatter / tdm_all_gather (tandem/comm.py:326-385) bit
+ * for bit, by reading the peers' tensors where they lie instead of passing pieces
+ * through slots:
+ *   all_reduce      fence; this rank folds its own ring chunk out of all W tensors in
+ *                   the ring's order for that chunk (the sum order of tandem/comm.py:301-305),
+ *                   in place; fence; it copies every other chunk from its owner; fence.
+ *   reduce_scatter  fence; the same fold; fence. Unlike the ring (tandem/comm.py:350-352),
+ *                   the chunks this rank does not own are left as they were.
+ *   all_gather      fence; the same copies; fence.
+ * World sizes up to 8 for the two that reduce. The tensors must not change between
+ * the call and the end of the Work on any rank. */
+int tdm_direct_all_reduce(tdm_engine* e, void* ptr, int64_t numel, int dtype, int average, const int64_t* peer_offsets,
+                          int noffsets, tdm_stream caller, tdm_work** out);
+int tdm_direct_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
+                              int average, const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out);
+int tdm_direct_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
+                          const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out);
 int tdm_sendrecv(tdm_engine* e, const void* send, int64_t send_numel, int dst, void* recv, int64_t recv_numel, int src,
                  int dtype, tdm_stream caller, tdm_work** out);
 int tdm_barrier(tdm_engine* e, tdm_work** out);

@@ -92,6 +92,12 @@ _ENGINE_SIGNATURES = {
                                     _VP, _PVP]),
     "tdm_barrier": (ctypes.c_int, [_VP, _PVP]),
     "tdm_fence": (ctypes.c_int, [_VP, _VP, _PVP]),
+    "tdm_direct_all_reduce": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _PI64, ctypes.c_int, _VP,
+                                             _PVP]),
+    "tdm_direct_reduce_scatter": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _PI64, ctypes.c_int, ctypes.c_int,
+                                                 _PI64, ctypes.c_int, _VP, _PVP]),
+    "tdm_direct_all_gather": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _PI64, ctypes.c_int, _PI64, ctypes.c_int,
+                                             _VP, _PVP]),
     "tdm_engine_share": (ctypes.c_int, [_VP, ctypes.c_int64, _PVP]),
     "tdm_unit_gather_direct": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _VP, _PI64, ctypes.c_int, _PI64,
                                               ctypes.c_int, _VP, _PVP]),

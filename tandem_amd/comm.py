@@ -198,35 +198,71 @@ class Group:
         return _lib.stream_ptr(self.device)
 
     # ---- collectives
-    def all_reduce(self, t, op="sum", async_op=False):
-        """Ring all-reduce in place: reduce-scatter, then all-gather."""
+    def _direct_offsets(self, flat, direct, what):
+        """Arena byte offsets of every rank's tensor for a direct collective:
+        `direct=True` says every rank holds it at the same offset of its arena (ranks
+        that allocate the same things in the same order do), a list gives them."""
+        if flat.numel() == 0:  # nothing to read, but the ranks still meet
+            return (ctypes.c_int64 * self.size)()
+        mine = self.arena_offset(flat)
+        if mine is None:
+            raise CommError(f"{what}: direct collectives need a tensor from shared_empty()")
+        offs = [mine] * self.size if direct is True else [int(o) for o in direct]
+        if len(offs) != self.size or offs[self.rank] != mine:
+            raise CommError(f"{what}: one arena offset per rank, this rank's own among them")
+        return (ctypes.c_int64 * self.size)(*offs)
+
+    def all_reduce(self, t, op="sum", async_op=False, direct=False):
+        """Ring all-reduce in place: reduce-scatter, then all-gather. With `direct`
+        (tensors in the ranks' shared arenas) each rank folds its own chunk straight
+        out of its peers' tensors, in the ring's order, and copies the other chunks
+        from their owners: the same bits, without slots."""
         if op not in ("sum", "avg"):
             raise CommError(f"unknown op {op}")
         flat = self._flat(t, "all_reduce")
         code = self._code(flat, True)
+        if direct:
+            offs = self._direct_offsets(flat, direct, "all_reduce")
+            return self._start("all_reduce", lambda out: lib().tdm_direct_all_reduce(
+                self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, int(op == "avg"), offs, self.size,
+                self._stream(), out), t, t.numel() * t.element_size(), async_op, keep=(flat,))
         return self._start("all_reduce", lambda out: lib().tdm_all_reduce(
             self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, int(op == "avg"), self._stream(), out),
             t, t.numel() * t.element_size(), async_op, keep=(flat,))
 
-    def reduce_scatter(self, t, sizes=None, op="sum", async_op=False):
+    def reduce_scatter(self, t, sizes=None, op="sum", async_op=False, direct=False):
         """Sums `t` across ranks, leaving rank r's chunk (chunk r of
         torch.tensor_split, or of `sizes`) reduced in place; returns that view.
-        The other chunks hold partial sums afterwards."""
+        The other chunks hold partial sums afterwards; with `direct` (tensors in
+        the shared arenas) they are left untouched instead."""
         if op not in ("sum", "avg"):
             raise CommError(f"unknown op {op}")
         flat = self._flat(t, "reduce_scatter")
         code = self._code(flat, True)
         sizes, arr, n = self._sizes(flat, sizes)
         mine = self._chunk_of_rank(flat, sizes)
+        if direct:
+            offs = self._direct_offsets(flat, direct, "reduce_scatter")
+            return self._start("reduce_scatter", lambda out: lib().tdm_direct_reduce_scatter(
+                self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, arr, n, int(op == "avg"), offs,
+                self.size, self._stream(), out), mine, t.numel() * t.element_size(), async_op, keep=(flat,))
         return self._start("reduce_scatter", lambda out: lib().tdm_reduce_scatter(
             self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, arr, n, int(op == "avg"), self._stream(), out),
             mine, t.numel() * t.element_size(), async_op, keep=(flat,))
 
-    def all_gather(self, t, sizes=None, async_op=False):
-        """Each rank holds its own chunk of `t` (chunk r); fills in the rest."""
+    def all_gather(self, t, sizes=None, async_op=False, direct=False):
+        """Each rank holds its own chunk of `t` (chunk r); fills in the rest (with
+        `direct`, by copying every chunk straight from its owner's arena)."""
         flat = self._flat(t, "all_gather")
         code = self._code(flat, False)
         sizes, arr, n = self._sizes(flat, sizes)
+        if direct:
+            if code == _lib.TDM_BYTES:
+                raise CommError(f"all_gather: direct gathers need one of {sorted(str(d) for d in _lib.DTYPES)}")
+            offs = self._direct_offsets(flat, direct, "all_gather")
+            return self._start("all_gather", lambda out: lib().tdm_direct_all_gather(
+                self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, arr, n, offs, self.size,
+                self._stream(), out), t, t.numel() * t.element_size(), async_op, keep=(flat,))
         if code == _lib.TDM_BYTES and n:
             arr = (ctypes.c_int64 * n)(*[s * flat.element_size() for s in sizes])
         return self._start("all_gather", lambda out: lib().tdm_all_gather(
@@ -234,28 +270,41 @@ class Group:
             t, t.numel() * t.element_size(), async_op, keep=(flat,))
 
     # ---- shared arena: long-lived data that peers read directly
-    def shared_empty(self, numel, dtype=torch.float32):
-        """A tensor of `numel` elements in this rank's shared arena: device memory
-        owned by the engine (freed by close()), exported once through HIP IPC, that
-        the other ranks read directly in gather_unit(..., peer_offsets=...). One
-        arena per group, under 2 GiB. Every change of its contents must sit between
-        two fence() calls."""
+    def share_arena(self, nbytes):
+        """Creates this rank's shared arena: `nbytes` (under 2 GiB) of device memory
+        owned by the engine (freed by close()) and exported once through HIP IPC, so
+        that the other ranks can read it directly. One arena per group."""
         if self._arena is not None:
             raise CommError("this group already has a shared arena")
-        es = torch.empty(0, dtype=dtype).element_size()
-        nbytes = max(16, numel * es)
+        nbytes = max(16, int(nbytes))
         ptr = ctypes.c_void_p()
         try:
             check(lib().tdm_engine_share(self._engine, nbytes, ctypes.byref(ptr)))
         except (ValueError, RuntimeError) as e:
-            raise CommError(f"shared_empty: {e}") from e
+            raise CommError(f"share_arena: {e}") from e
 
         class _Raw:  # what torch needs to wrap foreign device memory
             __cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (ptr.value, False), "version": 3}
 
-        raw = torch.as_tensor(_Raw(), device=self.device)
-        self._arena = raw
-        return raw[:numel * es].view(dtype)
+        self._arena = torch.as_tensor(_Raw(), device=self.device)
+        self._arena_used = 0
+
+    def shared_empty(self, numel, dtype=torch.float32):
+        """A tensor of `numel` elements in this rank's shared arena, for
+        gather_unit(..., peer_offsets=...) and the `direct` collectives. Without an
+        arena, one of exactly this size is created; otherwise the tensor is carved
+        from what share_arena() reserved (256-byte aligned, never given back). Every
+        change of an arena tensor that peers read on their own (gather_unit) must sit
+        between two fence() calls; the direct collectives fence by themselves."""
+        es = torch.empty(0, dtype=dtype).element_size()
+        if self._arena is None:
+            self.share_arena(numel * es)
+        at = -(-self._arena_used // 256) * 256
+        if at + numel * es > self._arena.numel():
+            raise CommError(f"shared_empty: {numel * es} bytes do not fit in the arena "
+                            f"({self._arena.numel() - at} of {self._arena.numel()} left)")
+        self._arena_used = at + numel * es
+        return self._arena[at:at + numel * es].view(dtype)
 
     def arena_offset(self, t):
         """Byte offset of tensor `t` inside this rank's arena (None if it is not there)."""

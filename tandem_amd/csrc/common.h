@@ -49,5 +49,6 @@ int guard(F&& body) {
 void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool scale_dst, bool scale_src,
                  bool writeback_src, hipStream_t stream);
 void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream);
+void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream);
 
 }  // namespace tandem_hip

@@ -174,6 +174,20 @@ class Region {
   bool owner_ = false;
 };
 
+// A wake-up through a condition variable costs 10-20 us; whoever expects news within
+// that time polls for it first.
+constexpr auto kSpinBeforeSleep = std::chrono::microseconds(100);
+
+template <class Ready>
+bool spin_for(Ready ready, std::chrono::microseconds limit = kSpinBeforeSleep) {
+  const auto until = std::chrono::steady_clock::now() + limit;
+  for (int i = 0;; ++i) {
+    if (ready()) return true;
+    if ((i & 15) == 15 && std::chrono::steady_clock::now() > until) return false;
+    __builtin_ia32_pause();
+  }
+}
+
 // Spin, then yield, then short sleeps; throws Timeout.
 template <class Ready>
 void wait_until(Ready ready, double timeout_s, const char* what) {
@@ -209,10 +223,13 @@ struct Work {
   std::mutex mu;
   std::condition_variable cv;
   bool finished = false;   // the job has run (all its GPU work is enqueued)
+  std::atomic<bool> finished_hint{false};  // set after `finished`: lets a waiter poll before it sleeps
   int status = TDM_OK;
   std::string error;
   double t0 = 0, t1 = 0;
-  hipEvent_t done_event = nullptr;  // recorded on the engine's stream after the job
+  hipEvent_t done_event = nullptr;  // recorded on the engine's stream after the job (jobs with GPU work)
+  bool uses_gpu = false;
+  bool drained = false;  // the job ends with a fence: the engine's stream is idle when it has run
   int device = -1;
   // Device timing (only while the engine's timing switch is on): start_event is
   // recorded on the engine's stream once the inputs are ready; both events carry
@@ -253,6 +270,9 @@ class Engine {
   void* share(size_t bytes);
   std::shared_ptr<Work> unit_gather_direct(Buf full, const char* shard, std::vector<int64_t> sizes,
                                            std::vector<int64_t> peer_offsets, hipStream_t caller);
+  // kind 0: all_reduce, 1: reduce_scatter (the owner's chunk only), 2: all_gather
+  std::shared_ptr<Work> direct(int kind, Buf t, std::vector<int64_t> sizes, bool average, std::vector<int64_t> peer_offsets,
+                               hipStream_t caller);
 
   int device() const { return device_; }
   hipStream_t stream() const { return stream_; }
@@ -265,8 +285,13 @@ class Engine {
     int64_t numel;
   };
 
-  std::shared_ptr<Work> submit(std::function<void()> job, hipStream_t caller, bool uses_gpu);
+  std::shared_ptr<Work> submit(std::function<void()> job, hipStream_t caller, bool uses_gpu, bool host_ready = false);
   void stamp_start(Work& w);
+  void direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets, const char** base);
+  void direct_fold(const Buf& t, const std::vector<Chunk>& cs, const char* const* base, bool average);
+  void direct_copies(const Buf& t, const std::vector<Chunk>& cs, const char* const* base);
+  void start();
+  void release_device();
   void loop();
   void check(const Buf& t, const char* what, bool reduce) const;
   std::vector<Chunk> chunks(const Buf& t, const std::vector<int64_t>& sizes) const;
@@ -323,12 +348,16 @@ class Engine {
   std::condition_variable ccv_, cidle_;
   std::deque<Completion> completions_;
   bool cstop_ = false, cbusy_ = false;
+  std::atomic<uint64_t> cqueued_{0};  // completions ever queued
+  uint64_t cdone_ = 0;                // completions ever taken (completion thread, under cmu_)
   std::string cerror_;
   std::thread completer_;
 
   std::mutex mu_;
   std::condition_variable cv_;
   std::deque<std::pair<std::function<void()>, std::shared_ptr<Work>>> jobs_;
+  std::atomic<uint64_t> submitted_{0};  // jobs ever queued
+  uint64_t started_ = 0;                // jobs ever taken (progress thread only)
   bool stopping_ = false;
   std::thread thread_;
 };
@@ -351,6 +380,15 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
   use_events_ = mode && std::string(mode) == "event";
 
   check_hip(hipSetDevice(device_), "hipSetDevice");
+  try {
+    start();
+  } catch (...) {  // no destructor runs for a constructor that throws
+    release_device();
+    throw;
+  }
+}
+
+void Engine::start() {
   check_hip(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags");  // default priority
 
   mine_.create(region_name(rank_), size_);
@@ -451,6 +489,13 @@ void Engine::close() {
     ccv_.notify_all();
     completer_.join();
   }
+  release_device();  // after the closing barrier: no peer reads our slots or arena any more
+  check_hip(sync_err, "hipStreamSynchronize (close)");
+  if (!barrier_err.empty()) throw std::runtime_error("close: " + barrier_err);
+}
+
+// Mappings of the peers' memory, our slots, events, stream, arena and region.
+void Engine::release_device() {
   for (int p = 0; p < size_; ++p) {
     if (p == rank_) continue;
     if (peer_mem_[p]) (void)hipIpcCloseMemHandle(peer_mem_[p]);
@@ -467,11 +512,9 @@ void Engine::close() {
   }
   if (stream_) (void)hipStreamDestroy(stream_);
   stream_ = nullptr;
-  if (arena_) (void)hipFree(arena_);  // after the closing barrier: no peer reads it any more
+  if (arena_) (void)hipFree(arena_);
   arena_ = nullptr;
   mine_.reset();
-  check_hip(sync_err, "hipStreamSynchronize (close)");
-  if (!barrier_err.empty()) throw std::runtime_error("close: " + barrier_err);
 }
 
 Engine::~Engine() {
@@ -482,30 +525,47 @@ Engine::~Engine() {
 }
 
 // ---------------------------------------------------------------- progress thread
-std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t caller, bool uses_gpu) {
+// host_ready: the job begins with a handshake that needs the inputs complete, not
+// merely ordered on the GPU, so the progress thread itself waits for them (polling:
+// an idle stream passes the event within microseconds) and the engine's stream
+// is spared a wait packet.
+std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t caller, bool uses_gpu, bool host_ready) {
   auto work = std::make_shared<Work>();
   work->device = device_;
+  work->uses_gpu = uses_gpu;
+  work->drained = host_ready;
+  hipEvent_t ready = nullptr;
   if (uses_gpu) {
     // Start once the caller's stream has produced the inputs.
-    hipEvent_t ready;
     check_hip(hipEventCreateWithFlags(&ready, hipEventDisableTiming), "hipEventCreateWithFlags (ready)");
     hipError_t err = hipEventRecord(ready, caller);
     if (err != hipSuccess) {
       (void)hipEventDestroy(ready);
       check_hip(err, "hipEventRecord (ready)");
     }
-    job = [this, ready, w = work.get(), inner = std::move(job)] {
-      hipError_t e = hipStreamWaitEvent(stream_, ready, 0);
+    job = [this, ready, host_ready, w = work.get(), inner = std::move(job)] {
+      hipError_t e;
+      if (host_ready) {
+        const bool passed = spin_for([&] { return hipEventQuery(ready) != hipErrorNotReady; }, std::chrono::microseconds(300));
+        e = passed ? hipEventQuery(ready) : hipEventSynchronize(ready);
+        if (!passed) (void)hipGetLastError();  // the "not ready" left by the last poll
+      } else {
+        e = hipStreamWaitEvent(stream_, ready, 0);
+      }
       (void)hipEventDestroy(ready);  // released once the GPU is past it
-      check_hip(e, "hipStreamWaitEvent (ready)");
+      check_hip(e, "waiting for the caller's stream (ready)");
       stamp_start(*w);
       inner();
     };
   }
   {
     std::lock_guard<std::mutex> lock(mu_);
-    if (stopping_) throw std::runtime_error("the engine is closed");
+    if (stopping_) {
+      if (ready) (void)hipEventDestroy(ready);  // the job that would have released it never runs
+      throw std::runtime_error("the engine is closed");
+    }
     jobs_.emplace_back(std::move(job), work);
+    submitted_.fetch_add(1, std::memory_order_release);
   }
   cv_.notify_one();
   return work;
@@ -538,10 +598,12 @@ void Engine::loop() {
   (void)hipSetDevice(device_);
   for (;;) {
     std::pair<std::function<void()>, std::shared_ptr<Work>> next;
+    spin_for([this] { return submitted_.load(std::memory_order_acquire) != started_; });
     {
       std::unique_lock<std::mutex> lock(mu_);
       cv_.wait(lock, [this] { return stopping_ || !jobs_.empty(); });
       if (jobs_.empty()) return;  // stopping, and everything queued has run
+      ++started_;
       next = std::move(jobs_.front());
       jobs_.pop_front();
     }
@@ -560,7 +622,7 @@ void Engine::loop() {
     } catch (...) {
       status = TDM_ERUNTIME; error = "unknown error";
     }
-    if (status == TDM_OK) {
+    if (status == TDM_OK && w.uses_gpu && !(w.drained && !w.start_event)) {
       if (hipEventCreateWithFlags(&w.done_event, w.start_event ? hipEventDefault : hipEventDisableTiming) != hipSuccess ||
           hipEventRecord(w.done_event, stream_) != hipSuccess) {
         status = TDM_ERUNTIME;
@@ -575,6 +637,7 @@ void Engine::loop() {
       w.t1 = now_s();
       w.finished = true;
     }
+    w.finished_hint.store(true, std::memory_order_release);
     w.cv.notify_all();
   }
 }
@@ -619,6 +682,7 @@ void Engine::complete_later(bool is_release, int peer, uint64_t length, bool aft
     std::lock_guard<std::mutex> lock(cmu_);
     if (!cerror_.empty()) throw std::runtime_error("completion thread failed: " + cerror_);
     completions_.push_back(c);
+    cqueued_.fetch_add(1, std::memory_order_release);
   }
   ccv_.notify_one();
 }
@@ -630,11 +694,17 @@ void Engine::completion_loop() {
     {
       std::unique_lock<std::mutex> lock(cmu_);
       cbusy_ = false;
-      if (completions_.empty()) cidle_.notify_all();
+      if (completions_.empty()) {
+        cidle_.notify_all();
+        lock.unlock();
+        spin_for([this] { return cqueued_.load(std::memory_order_acquire) != cdone_; });
+        lock.lock();
+      }
       ccv_.wait(lock, [this] { return cstop_ || !completions_.empty(); });
       if (completions_.empty()) return;
       c = completions_.front();
       completions_.pop_front();
+      ++cdone_;
       cbusy_ = true;
     }
     if (c.after) {
@@ -648,11 +718,16 @@ void Engine::completion_loop() {
         err = hipEventSynchronize(c.after);
       }
       (void)hipEventDestroy(c.after);
-      if (err != hipSuccess) {  // do not publish: the peers time out rather than read bad bytes
+      if (err != hipSuccess) {
         std::lock_guard<std::mutex> lock(cmu_);
         if (cerror_.empty()) cerror_ = std::string("hipEventSynchronize: ") + hipGetErrorString(err);
-        continue;
       }
+    }
+    {
+      // After a failure nothing more is published, this message or any later one:
+      // the peers time out rather than read bad bytes or reuse a slot still in use.
+      std::lock_guard<std::mutex> lock(cmu_);
+      if (!cerror_.empty()) continue;
     }
     if (c.is_release) release(c.peer); else signal(c.peer, c.length);
   }
@@ -670,7 +745,22 @@ void Engine::drain_completions() {
 // after_gpu: the empty messages are published only once the GPU has finished what
 // the engine's stream holds so far (a fence), not merely when it has been enqueued.
 void Engine::barrier_now(bool after_gpu) {
-  if (after_gpu && use_events_) check_hip(hipStreamSynchronize(stream_), "hipStreamSynchronize (fence)");
+  // Messages are published in order: everything queued for the completion thread
+  // goes first. After that this thread publishes by itself; it has to wait for the
+  // peers anyway, and handing over to the completion thread would cost two wake-ups.
+  drain_completions();
+  if (after_gpu) {
+    const auto done = [this] {
+      const hipError_t err = hipStreamQuery(stream_);
+      if (err == hipErrorNotReady) {
+        (void)hipGetLastError();
+        return false;
+      }
+      check_hip(err, "hipStreamQuery (fence)");
+      return true;
+    };
+    if (!spin_for(done, std::chrono::microseconds(300))) check_hip(hipStreamSynchronize(stream_), "hipStreamSynchronize (fence)");
+  }
   // An empty message to every peer, then one from each. Rings are first in,
   // first out, so this also orders the barrier after every piece queued before.
   constexpr uint64_t kEmpty = ~uint64_t(0);
@@ -681,12 +771,12 @@ void Engine::barrier_now(bool after_gpu) {
     wait_until([&] { return posted - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots_); },
                timeout_s_, "barrier: a peer rank never drained its messages");
     posted_[p] = posted + 1;
-    if (use_events_) signal(p, kEmpty); else complete_later(false, p, kEmpty, after_gpu);
+    signal(p, kEmpty);
   }
   for (int p = 0; p < size_; ++p) {
     if (p == rank_) continue;
     if (await(p) != kEmpty) throw std::runtime_error("barrier out of step: expected an empty message, got a piece");
-    if (use_events_) release(p); else complete_later(true, p, 0, false);
+    release(p);
   }
 }
 
@@ -998,12 +1088,97 @@ std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, st
   }, caller, true);
 }
 
+// ---------------------------------------------------------------- direct collectives
+// For tensors that live in the ranks' shared arenas. No slots and no per-piece
+// messages: a rank reads its peers' tensors where they lie.
+//   all_reduce      fence; fold my chunk out of all ranks' tensors, in the ring's order
+//                   for that chunk, into my tensor; fence; copy every other chunk from
+//                   its owner's tensor; fence.
+//   reduce_scatter  fence; the same fold; fence. Only the owner's chunk is produced.
+//   all_gather      fence; the same copies; fence.
+// Per rank and element of the tensor that is (W+1)/W + 2(W-1)/W accesses for an
+// all-reduce where the slot ring makes 9(W-1)/W, and three handshakes in all instead
+// of two per piece. The first fence says every rank's input is complete, the last
+// that nobody reads a tensor any more, so the caller may change it again.
+void Engine::direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets, const char** base) {
+  const int es = elem_bytes(t.dtype);
+  const size_t bytes = static_cast<size_t>(t.numel) * es;
+  const char* a = static_cast<const char*>(arena_);
+  if (!arena_ || t.ptr < a || t.ptr + bytes > a + arena_bytes_) {
+    throw Invalid("direct collective: the tensor does not lie in this rank's shared arena");
+  }
+  for (int q = 0; q < size_; ++q) {
+    if (q == rank_) {
+      base[q] = t.ptr;
+      continue;
+    }
+    if (peer_offsets[q] < 0 || peer_offsets[q] % es) throw Invalid("direct collective: bad arena offset");
+    base[q] = peer_arena(q, static_cast<size_t>(peer_offsets[q]) + bytes) + peer_offsets[q];
+  }
+}
+
+void Engine::direct_fold(const Buf& t, const std::vector<Chunk>& cs, const char* const* base, bool average) {
+  const Chunk& mine = cs[rank_];
+  if (mine.numel == 0) return;
+  tdm_fold_seg seg;
+  std::memset(&seg, 0, sizeof seg);
+  const size_t lo = static_cast<size_t>(mine.ptr - t.ptr);
+  for (int q = 0; q < size_; ++q) seg.src[q] = base[q] + lo;
+  seg.dst[rank_] = mine.ptr;
+  seg.count = mine.numel;
+  seg.chunk = rank_;
+  fold_step(&seg, 1, size_, t.dtype, average, stream_);
+}
+
+void Engine::direct_copies(const Buf& t, const std::vector<Chunk>& cs, const char* const* base) {
+  tdm_pair pairs[TDM_MAX_PAIRS];
+  int np = 0;
+  for (int q = 0; q < size_; ++q) {
+    if (q == rank_ || cs[q].numel == 0) continue;
+    pairs[np++] = tdm_pair{cs[q].ptr, base[q] + (cs[q].ptr - t.ptr), cs[q].numel};
+    if (np == TDM_MAX_PAIRS) {
+      copy_step(pairs, np, t.dtype, 0, stream_);
+      np = 0;
+    }
+  }
+  if (np) copy_step(pairs, np, t.dtype, 0, stream_);
+}
+
+std::shared_ptr<Work> Engine::direct(int kind, Buf t, std::vector<int64_t> sizes, bool average,
+                                     std::vector<int64_t> peer_offsets, hipStream_t caller) {
+  const char* what = kind == 0 ? "all_reduce (direct)" : kind == 1 ? "reduce_scatter (direct)" : "all_gather (direct)";
+  check(t, what, kind != 2);
+  if (t.dtype == kBytesDtype) throw Invalid(std::string(what) + ": needs a typed tensor");
+  if (kind != 2 && average && (t.dtype == TDM_I64 || t.dtype == TDM_I32)) {
+    throw Invalid(std::string(what) + ": integer tensors cannot be averaged in place");
+  }
+  if (kind != 2 && size_ > TDM_MAX_WORLD) throw Invalid(std::string(what) + ": the direct fold handles world sizes up to 8");
+  if (static_cast<int>(peer_offsets.size()) != size_) throw Invalid(std::string(what) + ": one arena offset per rank");
+  chunks(t, sizes);  // validate now, in the caller's thread
+  return submit([this, kind, t, sizes, average, peer_offsets] {
+    if (size_ == 1) return;
+    const auto cs = chunks(t, sizes);
+    const char* base[TDM_MAX_PAIRS > TDM_MAX_WORLD ? TDM_MAX_PAIRS : TDM_MAX_WORLD];
+    if (size_ > static_cast<int>(sizeof base / sizeof base[0])) throw Invalid("direct collective: too many ranks");
+    if (t.numel > 0) direct_bases(t, peer_offsets, base);  // an empty tensor still takes part in the fences
+    barrier_now(true);  // every rank's input is complete
+    if (kind != 2) {
+      direct_fold(t, cs, base, average);
+      barrier_now(true);  // every chunk is folded (or, for reduce_scatter: nobody reads our tensor any more)
+    }
+    if (kind != 1) {
+      direct_copies(t, cs, base);
+      barrier_now(true);  // nobody reads our tensor any more
+    }
+  }, caller, true, true);
+}
+
 // A barrier that is also ordered against the GPU: it starts after the caller's
 // stream has finished what it held at the call, and a rank's arrival is only
 // announced once its engine stream has finished too.
 std::shared_ptr<Work> Engine::fence(hipStream_t caller) {
   if (!connected_) throw std::runtime_error("fence: the engine is not connected");
-  return submit([this] { barrier_now(true); }, caller, true);
+  return submit([this] { barrier_now(true); }, caller, true, true);
 }
 
 std::shared_ptr<Work> Engine::barrier() {
@@ -1144,6 +1319,36 @@ int tdm_unit_gather_direct(tdm_engine* e, void* full, int64_t numel, int dtype, 
   });
 }
 
+namespace {
+int direct_call(tdm_engine* e, int kind, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
+                const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    if (nsizes < 0 || (nsizes > 0 && sizes == nullptr) || noffsets < 0 || (noffsets > 0 && peer_offsets == nullptr)) {
+      throw Invalid("bad sizes or offsets");
+    }
+    std::vector<int64_t> sz(sizes, sizes + nsizes), off(peer_offsets, peer_offsets + noffsets);
+    finish_submit(engine_of(e).direct(kind, Engine::Buf{static_cast<char*>(ptr), numel, dtype}, std::move(sz), average != 0,
+                                      std::move(off), static_cast<hipStream_t>(caller)), out);
+  });
+}
+}  // namespace
+
+int tdm_direct_all_reduce(tdm_engine* e, void* ptr, int64_t numel, int dtype, int average, const int64_t* peer_offsets,
+                          int noffsets, tdm_stream caller, tdm_work** out) {
+  return direct_call(e, 0, ptr, numel, dtype, nullptr, 0, average, peer_offsets, noffsets, caller, out);
+}
+
+int tdm_direct_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
+                              int average, const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out) {
+  return direct_call(e, 1, ptr, numel, dtype, sizes, nsizes, average, peer_offsets, noffsets, caller, out);
+}
+
+int tdm_direct_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
+                          const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out) {
+  return direct_call(e, 2, ptr, numel, dtype, sizes, nsizes, 0, peer_offsets, noffsets, caller, out);
+}
+
 int tdm_fence(tdm_engine* e, tdm_stream caller, tdm_work** out) {
   return guard([&] {
     if (out == nullptr) throw Invalid("NULL work pointer");
@@ -1164,6 +1369,7 @@ int tdm_work_wait(tdm_work* w, tdm_stream caller) {
     return TDM_EINVAL;
   }
   Work& work = *w->impl;
+  spin_for([&] { return work.finished_hint.load(std::memory_order_acquire); });
   {
     std::unique_lock<std::mutex> lock(work.mu);
     work.cv.wait(lock, [&] { return work.finished; });
@@ -1174,6 +1380,9 @@ int tdm_work_wait(tdm_work* w, tdm_stream caller) {
   }
   if (work.done_event) {
     return guard([&] {
+      const hipError_t q = hipEventQuery(work.done_event);
+      if (q == hipSuccess) return;  // the GPU is past it already: nothing to order
+      if (q == hipErrorNotReady) (void)hipGetLastError();
       check_hip(hipStreamWaitEvent(static_cast<hipStream_t>(caller), work.done_event, 0), "hipStreamWaitEvent (wait)");
     });
   }

@@ -869,41 +869,68 @@ void local_all_gather(const LocalRanks& lr, hipStream_t stream) {
 // folded in the ring's order for its chunk and written to all ranks.
 void local_all_reduce_fold(const LocalRanks& lr, bool average, hipStream_t stream) {
   const int n = lr.world;
-  FoldSmall tab;
-  std::memset(&tab, 0, sizeof tab);
-  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / lr.es);
-  int64_t tiles = 0;
-  int k = 0;
+  tdm_fold_seg segs[TDM_MAX_WORLD];
+  std::memset(segs, 0, sizeof segs);
   for (int c = 0; c < n; ++c) {
-    if (lr.len[c] == 0) continue;
-    bool vec = true;
     for (int r = 0; r < n; ++r) {
       char* p = lr.base[r] + lr.lo[c] * lr.es;
-      tab.seg[k].src[r] = p;
-      tab.seg[k].dst[r] = p;
-      vec = vec && reinterpret_cast<uintptr_t>(p) % 16 == 0;
+      segs[c].src[r] = p;
+      segs[c].dst[r] = p;
     }
-    tab.seg[k].count = lr.len[c];
-    tab.seg[k].chunk = c;
+    segs[c].count = lr.len[c];
+    segs[c].chunk = c;
+  }
+  fold_step(segs, n, n, lr.dtype, average, stream);
+}
+
+}  // namespace
+
+// Up to 8 segments folded in one launch, the table passed by value. Used by the
+// engine too (a rank folding its own chunk out of its peers' shared arenas).
+void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream) {
+  const int es = elem_size(dtype);
+  if (es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
+  if (world < 2 || world > TDM_MAX_WORLD) throw Invalid("the direct fold handles world sizes 2..8");
+  if (nseg < 0 || nseg > TDM_MAX_WORLD || (nseg > 0 && segs == nullptr)) throw Invalid("the direct fold takes up to 8 segments");
+  if (average && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
+  FoldSmall tab;
+  std::memset(&tab, 0, sizeof tab);
+  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
+  int64_t tiles = 0;
+  int k = 0;
+  for (int i = 0; i < nseg; ++i) {
+    const tdm_fold_seg& s = segs[i];
+    if (s.count < 0) throw Invalid("fold: negative count");
+    if (s.count == 0) continue;
+    if (s.chunk < 0 || s.chunk >= world) throw Invalid("fold: chunk outside [0, world)");
+    bool vec = true;
+    for (int r = 0; r < world; ++r) {
+      if (s.src[r] == nullptr) throw Invalid("fold: NULL source");
+      const uintptr_t a = reinterpret_cast<uintptr_t>(s.src[r]), b = reinterpret_cast<uintptr_t>(s.dst[r]);
+      if (a % es || b % es) throw Invalid("fold: pointer not aligned to the element size");
+      vec = vec && a % 16 == 0 && b % 16 == 0;
+      tab.seg[k].src[r] = static_cast<const char*>(s.src[r]);
+      tab.seg[k].dst[r] = static_cast<char*>(s.dst[r]);
+    }
+    tab.seg[k].count = s.count;
+    tab.seg[k].chunk = s.chunk;
     tab.seg[k].vec_ok = vec;
-    tiles += (lr.len[c] + tile_elems - 1) / tile_elems;
+    tiles += (s.count + tile_elems - 1) / tile_elems;
     tab.tile_end[k] = tiles;
     ++k;
   }
   tab.nseg = k;
   if (k == 0) return;
-  switch (lr.dtype) {
-    case TDM_F32: launch_fold_small<float>(tab, n, average, stream); break;
-    case TDM_F64: launch_fold_small<double>(tab, n, average, stream); break;
-    case TDM_F16: launch_fold_small<f16_t>(tab, n, average, stream); break;
-    case TDM_BF16: launch_fold_small<bf16_t>(tab, n, average, stream); break;
-    case TDM_I64: launch_fold_small<int64_t>(tab, n, 0, stream); break;
-    default: launch_fold_small<int32_t>(tab, n, 0, stream); break;
+  switch (dtype) {
+    case TDM_F32: launch_fold_small<float>(tab, world, average, stream); break;
+    case TDM_F64: launch_fold_small<double>(tab, world, average, stream); break;
+    case TDM_F16: launch_fold_small<f16_t>(tab, world, average, stream); break;
+    case TDM_BF16: launch_fold_small<bf16_t>(tab, world, average, stream); break;
+    case TDM_I64: launch_fold_small<int64_t>(tab, world, 0, stream); break;
+    default: launch_fold_small<int32_t>(tab, world, 0, stream); break;
   }
   check_hip(hipGetLastError(), "k2_fold_small launch");
 }
-
-}  // namespace
 
 }  // namespace tandem_hip
 

@@ -53,19 +53,34 @@ class _Range:
 class ZeRO(torch.nn.Module):
     """Stages 1 and 2."""
 
-    def __init__(self, module, group, stage=1, optimizer=None, bucket_bytes=25 << 20):
+    def __init__(self, module, group, stage=1, optimizer=None, bucket_bytes=25 << 20, direct=False):
+        """direct: the flat parameter buffer and the gradient buffer (stage 2: one
+        staging buffer the size of the model, kept, instead of one per bucket that is
+        dropped) live in the group's shared arena (created here if the group has none:
+        twice the model, under 2 GiB), and every collective runs arena to arena
+        (`direct=True` of tandem_amd.Group): same bits, fewer passes over memory, no
+        slots."""
         super().__init__()
         if stage not in (1, 2):
             raise ValueError("ZeRO handles stages 1 and 2; stage 3 is FSDP")
         _need(group, "pack")
+        if direct:
+            _need(group, "shared_empty", "share_arena")
         self.module, self.g, self.stage = module, group, stage
+        self.direct = bool(direct)
         self.opt = optimizer if optimizer is not None else ShardedAdamW()
         params = [p for p in module.parameters() if p.requires_grad]
         self.params = params
         dev, dtype = params[0].device, params[0].dtype
         self.flat = FlatLayout([p.numel() for p in params], group.size, group.rank)
         self.offset = dict(zip(params, self.flat.offsets))
-        self.buf = torch.empty(self.flat.numel, device=dev, dtype=dtype)
+        if self.direct:
+            if getattr(group, "_arena", None) is None:
+                group.share_arena(2 * (self.flat.numel * params[0].element_size() + 4096))
+            self.buf = group.shared_empty(self.flat.numel, dtype)
+            self._pool = group.shared_empty(self.flat.numel, dtype).zero_()  # stage 1: gradients; stage 2: staging
+        else:
+            self.buf = torch.empty(self.flat.numel, device=dev, dtype=dtype)
         with torch.no_grad():
             self.g.pack(self.buf, [(self.offset[p], p.data) for p in params])
             self.g.broadcast(self.buf, root=0)  # every rank starts from rank 0's weights
@@ -73,7 +88,7 @@ class ZeRO(torch.nn.Module):
                 o = self.offset[p]
                 p.data = self.buf[o:o + p.numel()].view_as(p)
         if stage == 1:
-            self.grad = torch.zeros_like(self.buf)
+            self.grad = self._pool if self.direct else torch.zeros_like(self.buf)
         else:
             self.grad_shard = torch.zeros(self.flat.hi - self.flat.lo, device=dev, dtype=dtype)
         # Buckets are contiguous ranges of the flat buffer taken from its end: the
@@ -103,14 +118,16 @@ class ZeRO(torch.nn.Module):
                 for p in rng.loose:
                     p.grad = self._grad_view(p)
                 rng.loose = []
-            rng.work = self.g.all_reduce(self.grad[rng.a:rng.b], op="avg", async_op=True)
+            rng.work = self.g.all_reduce(self.grad[rng.a:rng.b], op="avg", async_op=True, **self._how)
         else:
             p0 = rng.params[0]
-            rng.staging = torch.empty(rng.b - rng.a, device=p0.device, dtype=p0.dtype)
+            rng.staging = (self._pool[rng.a:rng.b] if self.direct
+                           else torch.empty(rng.b - rng.a, device=p0.device, dtype=p0.dtype))
             self.g.pack(rng.staging, [(self.offset[p] - rng.a, p.grad) for p in rng.params])
             for p in rng.params:
                 p.grad = None  # the full-size gradient is not kept
-            rng.work = self.g.reduce_scatter(rng.staging, self.flat.bucket_sizes(rng.a, rng.b), op="avg", async_op=True)
+            rng.work = self.g.reduce_scatter(rng.staging, self.flat.bucket_sizes(rng.a, rng.b), op="avg", async_op=True,
+                                             **self._how)
 
     def _on_grad(self, p):
         rng = self.bucket_of[p]
@@ -146,7 +163,11 @@ class ZeRO(torch.nn.Module):
         lo, hi = self.flat.lo, self.flat.hi
         grad = self.grad[lo:hi] if self.stage == 1 else self.grad_shard
         self.opt.update("flat", self.buf[lo:hi], grad)
-        self.g.all_gather(self.buf, self.flat.sizes)
+        self.g.all_gather(self.buf, self.flat.sizes, **self._how)
+
+    @property
+    def _how(self):
+        return {"direct": True} if self.direct else {}
 
     def zero_grad(self):
         if self.stage == 1:

@@ -40,14 +40,16 @@ def train_rank(g, strategy, bucket_bytes, steps, batch):
     text = synthetic(20_000)
     model = GPT(c).to(g.device)
     extra = {}
-    if strategy == "ddp":
-        z = DDP(model, g, bucket_bytes=bucket_bytes)
+    # a trailing "d": buckets and flat buffers in the shared arenas, collectives arena to arena
+    if strategy.startswith("ddp"):
+        z = DDP(model, g, bucket_bytes=bucket_bytes, direct=strategy.endswith("d"))
         opt = torch.optim.AdamW(model.parameters(), lr=LR, weight_decay=WD, foreach=False, fused=False)
     else:
         sopt = ShardedAdamW(lr=LR, weight_decay=WD, order="device")  # torch's GPU op order, to compare with torch.optim.AdamW
         stage = int(strategy[4])
         if stage < 3:
-            z = ZeRO(model, g, stage, sopt, bucket_bytes)
+            z = ZeRO(model, g, stage, sopt, bucket_bytes, direct=strategy.endswith("d"))
+            assert z.direct == strategy.endswith("d")
         else:  # "zero3": shards in the shared arena, gathered directly; "zero3s": staged through the slots
             z = FSDP(model, g, sopt, direct=not strategy.endswith("s"))
             assert z._direct == (not strategy.endswith("s"))
@@ -57,7 +59,7 @@ def train_rank(g, strategy, bucket_bytes, steps, batch):
         loss = z(x, y)
         loss.backward()
         losses.append(loss.item())
-        if strategy == "ddp":
+        if strategy.startswith("ddp"):
             opt.step()
             opt.zero_grad()
         else:
@@ -106,7 +108,7 @@ def test_two_ranks_all_strategies_agree_bit_for_bit():
     from tandem_amd import launch
 
     runs = {s: launch(train_rank, 2, s, 4 << 10, STEPS, BATCH, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT)
-            for s in ("ddp", "zero1", "zero2", "zero3", "zero3s")}
+            for s in ("ddp", "ddpd", "zero1", "zero1d", "zero2", "zero2d", "zero3", "zero3s")}
     ref_losses, ref_w = one_process(2)
     for s, res in runs.items():
         assert torch.equal(res[0]["weights"], res[1]["weights"]), f"{s}: the ranks drifted apart"
@@ -124,8 +126,10 @@ def test_four_ranks_stay_in_step():
     more than three units whole."""
     from tandem_amd import launch
 
-    for s in ("ddp", "zero2", "zero3", "zero3s"):
+    kept = {}
+    for s in ("ddp", "ddpd", "zero1", "zero1d", "zero2", "zero2d", "zero3", "zero3s"):
         res = launch(train_rank, 4, s, 4 << 10, 6, 8, slot_bytes=1024, gpus=[0] * 4, timeout=TIMEOUT)
+        kept[s] = res[0]
         for r in range(1, 4):
             assert torch.equal(res[0]["weights"], res[r]["weights"]), (s, r)
         mean_first = sum(res[r]["losses"][0] for r in range(4)) / 4
@@ -133,3 +137,7 @@ def test_four_ranks_stay_in_step():
         assert mean_last < mean_first, s
         if s.startswith("zero3"):
             assert all(x["max_live"] <= 3 and x["live"] == 0 for x in res)
+    # arena to arena or through the slots: the same sums in the same order, so the same bits
+    for direct, ring in (("ddpd", "ddp"), ("zero2d", "zero2"), ("zero1d", "zero1")):
+        assert kept[direct]["losses"] == kept[ring]["losses"], direct
+        assert torch.equal(kept[direct]["weights"], kept[ring]["weights"]), direct
