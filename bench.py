@@ -257,6 +257,81 @@ def fsdp_gather(steps):
     return out
 
 
+def train_rank(g, strategy, steps):
+    """One training step (forward, backward, optimizer) of the 85.8M GPT on this
+    rank's rows of a batch of 8 x 512 tokens, as the reference's bench/run.py times
+    its strategies; "alone" runs the same rows without any communication."""
+    import torch
+
+    from tandem_amd import ShardedAdamW
+    from tandem_amd.data import synthetic
+    from tandem_amd.ddp import DDP
+    from tandem_amd.model import GPT, Config
+    from tandem_amd.zero import FSDP, ZeRO
+
+    cfg = Config.preset("medium")
+    torch.manual_seed(0)
+    text = synthetic(100_000)
+    model = GPT(cfg).to(g.device)
+    adamw = dict(lr=3e-4, betas=(0.9, 0.95), weight_decay=0.1)
+    direct = strategy.endswith("+direct")
+    kind = strategy.split("+")[0]
+    opt = None
+    if kind == "alone":
+        z, opt = model, torch.optim.AdamW(model.parameters(), foreach=False, **adamw)
+    elif kind == "ddp":
+        z, opt = DDP(model, g, direct=direct), torch.optim.AdamW(model.parameters(), foreach=False, **adamw)
+    elif kind in ("zero1", "zero2"):
+        z = ZeRO(model, g, int(kind[-1]), ShardedAdamW(**adamw), direct=direct)
+    else:
+        z = FSDP(model, g, ShardedAdamW(**adamw))
+    from tandem_amd.profile import Timeline, summarize
+
+    times = []
+    tl = Timeline(enabled=False, device=g.device)
+    for step in range(steps + 3):
+        x, y = text.batch(step, 8, cfg.seq, rank=g.rank, world=g.size, device=g.device)
+        g.barrier()
+        torch.cuda.synchronize()
+        if step == steps + 2:  # one more step, profiled as the reference's bench/run.py profiles its last one
+            g.trace.clear()
+            g.waits.clear()
+            g.tracing = tl.enabled = True
+        t0 = time.perf_counter()
+        with tl.span("forward"):
+            loss = z(x, y)
+        with tl.span("backward"):
+            loss.backward()
+        with tl.span("optimizer"):
+            if opt is not None:
+                opt.step()
+                opt.zero_grad()
+            else:
+                z.step()
+                z.zero_grad()
+        torch.cuda.synchronize()
+        if 2 <= step < steps + 2:
+            times.append(time.perf_counter() - t0)
+    g.tracing = False
+    prof = summarize(tl.spans, [s for s in g.trace if s[0] != "barrier"], list(g.waits), time.perf_counter() - t0)
+    prof.update({name + "_ms": round((e - s) * 1e3, 3) for name, s, e in tl.spans})
+    return {"step_ms": statistics.median(times) * 1e3, "loss": loss.item(),
+            "profile": {k: (round(v, 5) if isinstance(v, float) else v) for k, v in prof.items()}}
+
+
+def train_steps(steps):
+    from tandem_amd import launch
+
+    out = {"workload": "2 processes sharing the GPU, 85.8M GPT, batch 8x512 split over the ranks, fp32, full step "
+                       "(forward, backward, optimizer); 'alone' = the same rows with no communication and torch AdamW; "
+                       "'+direct' = buckets / flat buffers in the shared arenas, collectives arena to arena"}
+    for s in ("alone", "ddp", "ddp+direct", "zero1", "zero1+direct", "zero2", "zero2+direct", "zero3"):
+        res = launch(train_rank, 2, s, steps, gpus=[0, 0], timeout=120.0)
+        out[s] = {"step_ms": round(max(r["step_ms"] for r in res), 3), "loss": round(res[0]["loss"], 4),
+                  "profile_rank0": res[0]["profile"]}
+    return out
+
+
 def ipc_rank(g, sizes_kib, reps, direct=False):
     """The reference's one-GPU engine benchmark (bench/engine_one_gpu.py there):
     barrier, then time all_reduce + device sync; median. direct: the tensor lives in
@@ -386,7 +461,7 @@ def main():
     cpu = fsdp = None
     if not args.quick and not args.no_cpu:
         cpu = cpu_baseline(args.mib, 15)
-    ipc = None
+    ipc = train = None
     if not args.quick and not args.no_fsdp:
         try:
             fsdp = fsdp_gather(3)
@@ -396,6 +471,10 @@ def main():
             ipc = ipc_allreduce()
         except Exception as e:
             ipc = {"error": repr(e)[:300]}
+        try:
+            train = train_steps(5)
+        except Exception as e:
+            train = {"error": repr(e)[:300]}
 
     import torch
 
@@ -448,6 +527,8 @@ def main():
             line["fsdp_gather"] = fsdp
         if ipc is not None:
             line["ipc_allreduce_2_processes"] = ipc
+        if train is not None:
+            line["train_step_2_processes"] = train
         if cpu is not None:
             cpu["gpu_over_cpu"] = round(line["value"] / cpu["value"], 1)
             cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["ms"], 1)
