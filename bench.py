@@ -124,7 +124,7 @@ def sweep(lw, dev, steps):
         rows.append({"MiB": kib / 1024, "ring_ms": round(per * 1e3, 4), "ring_GBps": round(15 * b / per / 1e9, 1),
                      "ring_algbw_GBps": round(b / per / 1e9, 1),
                      "k1_frac_of_hbm": round(12 * n * (WORLD - 1) / (rs * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-                     "fold_ms": round(fold * 1e3, 4), "fold_GBps": round(8 * WORLD * b / fold / 1e9, 1),
+                     "fold_ms": round(fold * 1e3, 4), "fold_GBps": round(2 * WORLD * b / fold / 1e9, 1),  # every rank's b bytes read once, written once
                      "fold_algbw_GBps": round(b / fold / 1e9, 1)})
         del bufs
         torch.cuda.empty_cache()

@@ -143,35 +143,39 @@ __device__ __forceinline__ vec16 pack(const Lanes<T>& in) {
   return out;
 }
 
-// Cache policy, measured on MI355X with 4 x 64 MiB chunk pairs per launch: a
+// Cache policy, measured on MI355X. K1 with 4 x 64 MiB chunk pairs per launch: a
 // stream that is only read does best with non-temporal loads (it is not kept in
 // L2 / Infinity Cache), a stream that is read, modified and written back does best
 // with plain loads and plain stores (the store hits the line the load brought in).
-// Both non-temporal: 6.4 TB/s; both plain: 5.4; this split: 7.0.
-// -DTDM_NT_MASK=<0..7> builds the other combinations for measurement.
+// Both non-temporal: 6.4 TB/s; both plain: 5.4; this split: 7.0. The bucket fold
+// and AdamW run once per training step over data that nothing has touched since
+// the last step: there non-temporal stores pay as well (fold 0.260 -> 0.240 ms,
+// AdamW on four shards 0.448 -> 0.415 ms), and for AdamW non-temporal loads of
+// the streams it rewrites.
+// -DTDM_NT_MASK=<0..7> (and _K2, _K3) build the other combinations for measurement.
 #ifndef TDM_NT_MASK
 #define TDM_NT_MASK 2  // bit0: read-modify-write loads, bit1: read-once loads, bit2: stores are non-temporal
 #endif
+#ifndef TDM_NT_MASK_K2
+#define TDM_NT_MASK_K2 6  // the bucket fold over a device table (the by-value fold of one collective keeps TDM_NT_MASK)
+#endif
+#ifndef TDM_NT_MASK_K3
+#define TDM_NT_MASK_K3 7  // AdamW
+#endif
+template <int kMask = TDM_NT_MASK>
 __device__ __forceinline__ vec16 load_stream(const void* p) {  // read once, never written here
-#if TDM_NT_MASK & 2
-  return __builtin_nontemporal_load(static_cast<const vec16*>(p));
-#else
-  return *static_cast<const vec16*>(p);
-#endif
+  if constexpr (kMask & 2) return __builtin_nontemporal_load(static_cast<const vec16*>(p));
+  else return *static_cast<const vec16*>(p);
 }
+template <int kMask = TDM_NT_MASK>
 __device__ __forceinline__ vec16 load_rmw(const void* p) {  // about to be overwritten by this lane
-#if TDM_NT_MASK & 1
-  return __builtin_nontemporal_load(static_cast<const vec16*>(p));
-#else
-  return *static_cast<const vec16*>(p);
-#endif
+  if constexpr (kMask & 1) return __builtin_nontemporal_load(static_cast<const vec16*>(p));
+  else return *static_cast<const vec16*>(p);
 }
+template <int kMask = TDM_NT_MASK>
 __device__ __forceinline__ void store16(void* p, const vec16& v) {
-#if TDM_NT_MASK & 4
-  __builtin_nontemporal_store(v, static_cast<vec16*>(p));
-#else
-  *static_cast<vec16*>(p) = v;
-#endif
+  if constexpr (kMask & 4) __builtin_nontemporal_store(v, static_cast<vec16*>(p));
+  else *static_cast<vec16*>(p) = v;
 }
 
 // ---------------------------------------------------------------- pair tables
@@ -363,7 +367,7 @@ struct FoldSegDev {
 
 // One tile of one segment: W loads per element, the fold in ring order, W stores.
 // kAcc: the result is added into each destination (dst = dst + sum) instead of replacing it.
-template <typename T, int kWorld, int kDiv, bool kAcc>
+template <typename T, int kWorld, int kDiv, bool kAcc, int kMask>
 __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const Divisor<T>& dv) {
   using A = typename Elem<T>::acc;
   constexpr int L = lanes<T>();
@@ -390,7 +394,7 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
           const int64_t v = vbase + u * kThreads;
-          if (v < nv) in[k][u] = load_stream(sp[k] + v * 16);
+          if (v < nv) in[k][u] = load_stream<kMask>(sp[k] + v * 16);
         }
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
@@ -412,13 +416,13 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
           for (int k = 0; k < kWorld; ++k)
             if (dp[k]) {
               if constexpr (kAcc) {
-                Lanes<T> cur = unpack<T>(load_rmw(dp[k] + v * 16));
+                Lanes<T> cur = unpack<T>(load_rmw<kMask>(dp[k] + v * 16));
 #pragma unroll
                 for (int l = 0; l < L; ++l)
                   cur.v[l] = Elem<T>::narrow(static_cast<A>(Elem<T>::widen(cur.v[l]) + Elem<T>::widen(out.v[l])));
-                store16(dp[k] + v * 16, pack<T>(cur));
+                store16<kMask>(dp[k] + v * 16, pack<T>(cur));
               } else {
-                store16(dp[k] + v * 16, packed);
+                store16<kMask>(dp[k] + v * 16, packed);
               }
             }
         }
@@ -466,7 +470,7 @@ template <typename T, int kWorld, int kDiv, bool kAcc>
 __global__ __launch_bounds__(kThreads) void k2_fold_kernel(const FoldSegDev* __restrict__ tiles, int64_t total,
                                                            Divisor<T> dv) {
   for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
-    fold_tile<T, kWorld, kDiv, kAcc>(tiles[tile], 0, dv);
+    fold_tile<T, kWorld, kDiv, kAcc, TDM_NT_MASK_K2>(tiles[tile], 0, dv);
   }
 }
 
@@ -483,7 +487,7 @@ __global__ __launch_bounds__(kThreads) void k2_fold_small_kernel(FoldSmall tab, 
   for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
     int lo = 0;
     while (tile >= tab.tile_end[lo]) ++lo;
-    fold_tile<T, kWorld, kDiv, false>(tab.seg[lo], tile - (lo ? tab.tile_end[lo - 1] : 0), dv);
+    fold_tile<T, kWorld, kDiv, false, TDM_NT_MASK>(tab.seg[lo], tile - (lo ? tab.tile_end[lo - 1] : 0), dv);
   }
 }
 
@@ -533,10 +537,10 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
       for (int u = 0; u < kU; ++u) {
         const int64_t i = v0 + u * kThreads;
         if (i < nv) {
-          rp[u] = load_rmw(reinterpret_cast<const char*>(a.p) + i * 16);
-          rg[u] = load_stream(reinterpret_cast<const char*>(a.g) + i * 16);
-          rm[u] = load_rmw(reinterpret_cast<const char*>(a.m) + i * 16);
-          rv[u] = load_rmw(reinterpret_cast<const char*>(a.v) + i * 16);
+          rp[u] = load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.p) + i * 16);
+          rg[u] = load_stream<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.g) + i * 16);
+          rm[u] = load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.m) + i * 16);
+          rv[u] = load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.v) + i * 16);
         }
       }
 #pragma unroll
@@ -547,9 +551,9 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
                        V = unpack<float>(rv[u]);
 #pragma unroll
           for (int l = 0; l < 4; ++l) adamw_elem<kOrder>(P.v[l], G.v[l], M.v[l], V.v[l], a.s, small_w);
-          store16(reinterpret_cast<char*>(a.p) + i * 16, pack<float>(P));
-          store16(reinterpret_cast<char*>(a.m) + i * 16, pack<float>(M));
-          store16(reinterpret_cast<char*>(a.v) + i * 16, pack<float>(V));
+          store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.p) + i * 16, pack<float>(P));
+          store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.m) + i * 16, pack<float>(M));
+          store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.v) + i * 16, pack<float>(V));
         }
       }
     }
