@@ -229,6 +229,11 @@ int tdm_engine_destroy(tdm_engine* e);
 int tdm_all_reduce(tdm_engine* e, void* ptr, int64_t numel, int dtype, int average, tdm_stream caller, tdm_work** out);
 int tdm_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
                        tdm_stream caller, tdm_work** out);
+/* The same, when the caller only wants its own chunk (ZeRO's use, tandem/zero.py:141-153):
+ * the chunks this rank does not own are left as they were instead of holding the ring's
+ * partial sums, which lets the engine take one handshake per pass instead of two per piece. */
+int tdm_reduce_scatter_owner(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
+                             tdm_stream caller, tdm_work** out);
 int tdm_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, tdm_stream caller,
                    tdm_work** out);
 int tdm_broadcast(tdm_engine* e, void* ptr, int64_t numel, int dtype, int root, tdm_stream caller, tdm_work** out);

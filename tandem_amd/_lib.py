@@ -86,6 +86,7 @@ _ENGINE_SIGNATURES = {
     "tdm_all_reduce": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _VP, _PVP]),
     "tdm_reduce_scatter": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _PI64, ctypes.c_int, ctypes.c_int, _VP, _PVP]),
     "tdm_all_gather": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _PI64, ctypes.c_int, _VP, _PVP]),
+    "tdm_reduce_scatter_owner": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _PI64, ctypes.c_int, ctypes.c_int, _VP, _PVP]),
     "tdm_broadcast": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _VP, _PVP]),
     "tdm_unit_gather": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _VP, _PI64, ctypes.c_int, _VP, _PVP]),
     "tdm_sendrecv": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _VP, ctypes.c_int64, ctypes.c_int, ctypes.c_int,

@@ -230,11 +230,16 @@ class Group:
             self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, int(op == "avg"), self._stream(), out),
             t, t.numel() * t.element_size(), async_op, keep=(flat,))
 
-    def reduce_scatter(self, t, sizes=None, op="sum", async_op=False, direct=False):
+    partial_sums_optional = True  # reduce_scatter(partial_sums=False) exists: wrappers that drop the rest may ask for it
+
+    def reduce_scatter(self, t, sizes=None, op="sum", async_op=False, direct=False, partial_sums=True):
         """Sums `t` across ranks, leaving rank r's chunk (chunk r of
         torch.tensor_split, or of `sizes`) reduced in place; returns that view.
-        The other chunks hold partial sums afterwards; with `direct` (tensors in
-        the shared arenas) they are left untouched instead."""
+        The other chunks hold the ring's partial sums afterwards, as in the
+        reference (tandem/comm.py:350-352). A caller that only wants its chunk says
+        `partial_sums=False`: the rest of `t` is then left as it was, and the engine
+        needs one handshake per pass instead of two per piece. `direct` (tensors
+        in the shared arenas) implies it."""
         if op not in ("sum", "avg"):
             raise CommError(f"unknown op {op}")
         flat = self._flat(t, "reduce_scatter")
@@ -246,7 +251,8 @@ class Group:
             return self._start("reduce_scatter", lambda out: lib().tdm_direct_reduce_scatter(
                 self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, arr, n, int(op == "avg"), offs,
                 self.size, self._stream(), out), mine, t.numel() * t.element_size(), async_op, keep=(flat,))
-        return self._start("reduce_scatter", lambda out: lib().tdm_reduce_scatter(
+        call = lib().tdm_reduce_scatter if partial_sums else lib().tdm_reduce_scatter_owner
+        return self._start("reduce_scatter", lambda out: call(
             self._engine, ctypes.c_void_p(flat.data_ptr()), flat.numel(), code, arr, n, int(op == "avg"), self._stream(), out),
             mine, t.numel() * t.element_size(), async_op, keep=(flat,))
 

@@ -104,6 +104,9 @@ struct alignas(kLine) RegionHeader {
   // A rank's shared arena (tdm_engine_share): device memory its peers may read directly.
   std::atomic<uint64_t> arena_bytes;  // 0 until published
   hipIpcMemHandle_t arena_mem;
+  // The engine's own staging memory for the staged collectives (two halves, used in turn).
+  std::atomic<uint64_t> staging_bytes;  // 0 until published
+  hipIpcMemHandle_t staging_mem;
 };
 
 class Region {
@@ -260,7 +263,7 @@ class Engine {
   };
 
   std::shared_ptr<Work> all_reduce(Buf t, bool average, hipStream_t caller);
-  std::shared_ptr<Work> reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, hipStream_t caller);
+  std::shared_ptr<Work> reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, bool owner_only, hipStream_t caller);
   std::shared_ptr<Work> all_gather(Buf t, std::vector<int64_t> sizes, hipStream_t caller);
   std::shared_ptr<Work> unit_gather(Buf full, const char* shard, std::vector<int64_t> sizes, hipStream_t caller);
   std::shared_ptr<Work> broadcast(Buf t, int root, hipStream_t caller);
@@ -287,6 +290,12 @@ class Engine {
 
   std::shared_ptr<Work> submit(std::function<void()> job, hipStream_t caller, bool uses_gpu, bool host_ready = false);
   void stamp_start(Work& w);
+  char* staging_half();
+  const char* peer_staging(int peer, int half);
+  void copy_pairs(const tdm_pair* pairs, int np, int dtype);
+  void staged_all_reduce(const Buf& t, bool average);
+  void staged_all_gather(const Buf& t, const std::vector<Chunk>& cs, const char* own);
+  void staged_reduce_scatter_owner(const Buf& t, const std::vector<Chunk>& cs, bool average);
   void direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets, const char** base);
   void direct_fold(const Buf& t, const std::vector<Chunk>& cs, const char* const* base, bool average);
   void direct_copies(const Buf& t, const std::vector<Chunk>& cs, const char* const* base);
@@ -330,6 +339,12 @@ class Engine {
   std::vector<uint64_t> posted_;         // messages queued or published to each peer (flow control)
   std::vector<uint64_t> taken_;          // messages consumed from each peer
   bool connected_ = false, closed_ = false;
+  // staged collectives
+  bool staged_ = true;               // TANDEM_HIP_ALGO=ring switches them off
+  size_t staging_half_ = 32u << 20;  // bytes per half (TANDEM_HIP_STAGING_BYTES)
+  void* staging_ = nullptr;
+  std::vector<void*> peer_staging_;
+  uint64_t staged_ops_ = 0;          // picks the half; the same count on every rank
   std::atomic<int> timing_{0};
   bool timing_seen_ = false;           // progress thread only
   std::shared_ptr<Anchor> anchor_;     // progress thread only
@@ -378,6 +393,15 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
   if (job.empty() || job.size() > 64) throw Invalid("job name must have 1..64 characters");
   const char* mode = std::getenv("TANDEM_HIP_SYNC");
   use_events_ = mode && std::string(mode) == "event";
+  const char* algo = std::getenv("TANDEM_HIP_ALGO");
+  if (algo && std::string(algo) == "ring") staged_ = false;
+  else if (algo && *algo && std::string(algo) != "staged") throw Invalid("TANDEM_HIP_ALGO must be \"staged\" or \"ring\"");
+  if (const char* sb = std::getenv("TANDEM_HIP_STAGING_BYTES")) {
+    const long long v = std::atoll(sb);
+    if (v < 4096 || v >= (1ll << 30) || v % 4096) throw Invalid("TANDEM_HIP_STAGING_BYTES must be a multiple of 4096 in [4096, 1 GiB)");
+    staging_half_ = static_cast<size_t>(v);
+  }
+  peer_staging_.assign(size, nullptr);
 
   check_hip(hipSetDevice(device_), "hipSetDevice");
   try {
@@ -506,6 +530,8 @@ void Engine::release_device() {
     if (out_mem_[p]) (void)hipFree(out_mem_[p]);
     if (peer_arena_[p]) (void)hipIpcCloseMemHandle(peer_arena_[p]);
     peer_arena_[p] = nullptr;
+    if (peer_staging_[p]) (void)hipIpcCloseMemHandle(peer_staging_[p]);
+    peer_staging_[p] = nullptr;
     peer_mem_[p] = out_mem_[p] = nullptr;
     peer_full_[p].clear(); peer_free_[p].clear(); full_[p].clear(); free_[p].clear();
     theirs_[p].reset();
@@ -514,6 +540,8 @@ void Engine::release_device() {
   stream_ = nullptr;
   if (arena_) (void)hipFree(arena_);
   arena_ = nullptr;
+  if (staging_) (void)hipFree(staging_);
+  staging_ = nullptr;
   mine_.reset();
 }
 
@@ -887,6 +915,168 @@ void Engine::ring_all_gather(const std::vector<Chunk>& c, int dtype) {
   }
 }
 
+// ---------------------------------------------------------------- staged collectives
+// all_reduce and all_gather of any tensor without the slots' piece-by-piece
+// handshakes. Every rank owns staging memory that its peers map once: two halves,
+// used in turn by successive staged operations.
+//   all_reduce, per pass over at most half/W bytes of every ring chunk:
+//     copy my tensor's part of every chunk I do not own into my staging; fence;
+//     fold my own chunk's part out of my tensor and the peers' stagings, in the
+//     ring's order for that chunk, into my tensor AND my staging; fence; copy the
+//     other chunks' parts from their owners' stagings.
+//   all_gather, per pass over at most half bytes of every chunk:
+//     copy my chunk's part into my staging; fence; copy the others' from theirs.
+// Two handshakes (one) per pass where the slot ring makes 2(W-1) per 4 MiB piece, and
+// the bits are the ring's: the fold adds in the ring's order.
+// Why two halves are enough without a closing fence: an operation writes a half that
+// the peers last read two staged operations ago; every staged operation contains a
+// fence that a rank enters only when its engine stream has drained, so when this rank
+// has passed the fence of the operation in between, those reads are over.
+char* Engine::staging_half() {
+  if (!staging_) {
+    check_hip(hipMalloc(&staging_, 2 * staging_half_), "hipMalloc (staging)");
+    RegionHeader* h = mine_.header();
+    check_hip(hipIpcGetMemHandle(&h->staging_mem, staging_), "hipIpcGetMemHandle (staging)");
+    h->staging_bytes.store(2 * staging_half_, std::memory_order_release);  // the handle is visible before the size
+  }
+  return static_cast<char*>(staging_) + (staged_ops_++ % 2) * staging_half_;
+}
+
+// Only after a fence of the same operation: every rank publishes before it enters one.
+const char* Engine::peer_staging(int peer, int half) {
+  if (!peer_staging_[peer]) {
+    RegionHeader* h = theirs_[peer]->header();
+    if (h->staging_bytes.load(std::memory_order_acquire) != 2 * staging_half_) {
+      throw std::runtime_error("rank " + std::to_string(peer) + " has no staging memory of our size (TANDEM_HIP_STAGING_BYTES, TANDEM_HIP_ALGO differ?)");
+    }
+    check_hip(hipIpcOpenMemHandle(&peer_staging_[peer], h->staging_mem, hipIpcMemLazyEnablePeerAccess), "hipIpcOpenMemHandle (staging)");
+  }
+  return static_cast<const char*>(peer_staging_[peer]) + static_cast<size_t>(half) * staging_half_;
+}
+
+void Engine::copy_pairs(const tdm_pair* pairs, int np, int dtype) {
+  if (np == 0) return;
+  if (dtype != kBytesDtype) {
+    copy_step(pairs, np, dtype, 0, stream_);
+    return;
+  }
+  for (int i = 0; i < np; ++i) {
+    check_hip(hipMemcpyAsync(pairs[i].dst, pairs[i].src, static_cast<size_t>(pairs[i].count), hipMemcpyDeviceToDevice, stream_),
+              "hipMemcpyAsync (staged copy)");
+  }
+}
+
+void Engine::staged_all_reduce(const Buf& t, bool average) {
+  const auto cs = chunks(t, {});
+  const int es = elem_bytes(t.dtype), n = size_, r = rank_;
+  const size_t sub_bytes = staging_half_ / n / 256 * 256;  // one sub-slab per ring chunk
+  const int64_t sub = static_cast<int64_t>(sub_bytes) / es;
+  if (sub == 0) throw Invalid("all_reduce: the staging memory is too small for this world size");
+  int64_t longest = 0;
+  for (const Chunk& c : cs) longest = std::max(longest, c.numel);
+  for (int64_t at = 0; at < longest; at += sub) {
+    char* mine = staging_half();
+    const int half = static_cast<int>((staged_ops_ - 1) % 2);
+    auto part = [&](int c) { return std::max<int64_t>(0, std::min(sub, cs[c].numel - at)); };
+    tdm_pair pairs[TDM_MAX_PAIRS];
+    int np = 0;
+    for (int c = 0; c < n; ++c) {
+      if (c == r || part(c) == 0) continue;
+      pairs[np++] = tdm_pair{mine + c * sub_bytes, cs[c].ptr + at * es, part(c)};
+    }
+    copy_pairs(pairs, np, t.dtype);
+    barrier_now(true);  // every rank's parts are in its staging
+    if (part(r) > 0) {
+      tdm_fold_seg seg;
+      std::memset(&seg, 0, sizeof seg);
+      char* own = cs[r].ptr + at * es;
+      for (int q = 0; q < n; ++q) seg.src[q] = q == r ? own : peer_staging(q, half) + r * sub_bytes;
+      seg.dst[r] = own;
+      seg.dst[(r + 1) % n] = mine + r * sub_bytes;  // a second copy of the result, for the peers to fetch
+      seg.count = part(r);
+      seg.chunk = r;
+      fold_step(&seg, 1, n, t.dtype, average, stream_);
+    }
+    barrier_now(true);  // every chunk's part is folded
+    np = 0;
+    for (int c = 0; c < n; ++c) {
+      if (c == r || part(c) == 0) continue;
+      pairs[np++] = tdm_pair{cs[c].ptr + at * es, peer_staging(c, half) + c * sub_bytes, part(c)};
+    }
+    copy_pairs(pairs, np, t.dtype);
+  }
+}
+
+// reduce_scatter when only the owner's chunk is wanted (the ring also leaves partial
+// sums in the other chunks; ZeRO drops them). Per pass over a window of `half` bytes of
+// the tensor: copy the window's parts of the chunks I do not own into my staging, at
+// the same offsets; fence; fold my chunk's part out of my tensor and the peers' stagings.
+void Engine::staged_reduce_scatter_owner(const Buf& t, const std::vector<Chunk>& cs, bool average) {
+  const int es = elem_bytes(t.dtype), n = size_, r = rank_;
+  const int64_t cap = static_cast<int64_t>(staging_half_) / es;
+  for (int64_t at = 0; at < t.numel; at += cap) {
+    char* mine = staging_half();
+    const int half = static_cast<int>((staged_ops_ - 1) % 2);
+    const int64_t end = std::min(t.numel, at + cap);
+    // chunk c within the window, as element offsets of the tensor
+    auto lo = [&](int c) { return std::max<int64_t>(at, (cs[c].ptr - t.ptr) / es); };
+    auto hi = [&](int c) { return std::min<int64_t>(end, (cs[c].ptr - t.ptr) / es + cs[c].numel); };
+    tdm_pair pairs[TDM_MAX_PAIRS];
+    int np = 0;
+    for (int c = 0; c < n; ++c) {
+      if (c == r || hi(c) <= lo(c)) continue;
+      pairs[np++] = tdm_pair{mine + (lo(c) - at) * es, t.ptr + lo(c) * es, hi(c) - lo(c)};
+      if (np == TDM_MAX_PAIRS) {
+        copy_pairs(pairs, np, t.dtype);
+        np = 0;
+      }
+    }
+    copy_pairs(pairs, np, t.dtype);
+    barrier_now(true);  // every rank's parts are in its staging
+    if (hi(r) > lo(r)) {
+      tdm_fold_seg seg;
+      std::memset(&seg, 0, sizeof seg);
+      char* own = t.ptr + lo(r) * es;
+      for (int q = 0; q < n; ++q) seg.src[q] = q == r ? own : peer_staging(q, half) + (lo(r) - at) * es;
+      seg.dst[r] = own;
+      seg.count = hi(r) - lo(r);
+      seg.chunk = r;
+      fold_step(&seg, 1, n, t.dtype, average, stream_);
+    }
+  }
+}
+
+// `own`: where this rank's chunk is read from (the chunk itself, or ZeRO-3's shard).
+void Engine::staged_all_gather(const Buf& t, const std::vector<Chunk>& cs, const char* own) {
+  const int es = elem_bytes(t.dtype), n = size_, r = rank_;
+  const int64_t cap = static_cast<int64_t>(staging_half_) / es;
+  int64_t longest = 0;
+  for (const Chunk& c : cs) longest = std::max(longest, c.numel);
+  for (int64_t at = 0; at < longest; at += cap) {
+    char* mine = staging_half();
+    const int half = static_cast<int>((staged_ops_ - 1) % 2);
+    auto part = [&](int c) { return std::max<int64_t>(0, std::min(cap, cs[c].numel - at)); };
+    tdm_pair pairs[TDM_MAX_PAIRS];
+    int np = 0;
+    if (part(r) > 0) {
+      pairs[np++] = tdm_pair{mine, own + at * es, part(r)};
+      if (own != cs[r].ptr) pairs[np++] = tdm_pair{cs[r].ptr + at * es, own + at * es, part(r)};
+    }
+    copy_pairs(pairs, np, t.dtype);
+    barrier_now(true);  // every rank's part is in its staging
+    np = 0;
+    for (int c = 0; c < n; ++c) {
+      if (c == r || part(c) == 0) continue;
+      pairs[np++] = tdm_pair{cs[c].ptr + at * es, peer_staging(c, half), part(c)};
+      if (np == TDM_MAX_PAIRS) {
+        copy_pairs(pairs, np, t.dtype);
+        np = 0;
+      }
+    }
+    copy_pairs(pairs, np, t.dtype);
+  }
+}
+
 // ---------------------------------------------------------------- collectives
 void Engine::check(const Buf& t, const char* what, bool reduce) const {
   if (t.numel < 0) throw Invalid(std::string(what) + ": negative element count");
@@ -935,20 +1125,27 @@ std::shared_ptr<Work> Engine::all_reduce(Buf t, bool average, hipStream_t caller
   check(t, "all_reduce", true);
   if (average && (t.dtype == TDM_I64 || t.dtype == TDM_I32)) throw Invalid("all_reduce: integer tensors cannot be averaged in place");
   return submit([this, t, average] {
-    if (size_ > 1) {
-      auto c = chunks(t, {});
-      ring_reduce_scatter(c, t.dtype, average, false);
-      ring_all_gather(c, t.dtype);
+    if (size_ == 1) return;
+    if (staged_ && size_ <= TDM_MAX_WORLD) {
+      staged_all_reduce(t, average);
+      return;
     }
+    auto c = chunks(t, {});
+    ring_reduce_scatter(c, t.dtype, average, false);
+    ring_all_gather(c, t.dtype);
   }, caller, true);
 }
 
-std::shared_ptr<Work> Engine::reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, hipStream_t caller) {
+std::shared_ptr<Work> Engine::reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, bool owner_only,
+                                             hipStream_t caller) {
   check(t, "reduce_scatter", true);
   if (average && (t.dtype == TDM_I64 || t.dtype == TDM_I32)) throw Invalid("reduce_scatter: integer tensors cannot be averaged in place");
   chunks(t, sizes);  // validate now, in the caller's thread
-  return submit([this, t, sizes, average] {
-    if (size_ > 1) ring_reduce_scatter(chunks(t, sizes), t.dtype, average, true);
+  return submit([this, t, sizes, average, owner_only] {
+    if (size_ == 1) return;
+    const auto cs = chunks(t, sizes);
+    if (owner_only && staged_ && size_ <= TDM_MAX_WORLD) staged_reduce_scatter_owner(t, cs, average);
+    else ring_reduce_scatter(cs, t.dtype, average, true);
   }, caller, true);
 }
 
@@ -956,7 +1153,10 @@ std::shared_ptr<Work> Engine::all_gather(Buf t, std::vector<int64_t> sizes, hipS
   check(t, "all_gather", false);
   chunks(t, sizes);
   return submit([this, t, sizes] {
-    if (size_ > 1) ring_all_gather(chunks(t, sizes), t.dtype);
+    if (size_ == 1) return;
+    const auto cs = chunks(t, sizes);
+    if (staged_ && size_ < TDM_MAX_PAIRS) staged_all_gather(t, cs, cs[rank_].ptr);
+    else ring_all_gather(cs, t.dtype);
   }, caller, true);
 }
 
@@ -974,6 +1174,10 @@ std::shared_ptr<Work> Engine::unit_gather(Buf full, const char* shard, std::vect
   return submit([this, full, shard, sizes] {
     const auto cs = chunks(full, sizes);
     const Chunk& mine = cs[rank_];
+    if (size_ > 1 && staged_ && size_ < TDM_MAX_PAIRS) {
+      staged_all_gather(full, cs, mine.numel > 0 ? shard : mine.ptr);
+      return;
+    }
     if (mine.numel > 0 && shard != mine.ptr) {
       if (full.dtype == kBytesDtype) {
         check_hip(hipMemcpyAsync(mine.ptr, shard, static_cast<size_t>(mine.numel), hipMemcpyDeviceToDevice, stream_),
@@ -1246,15 +1450,27 @@ int tdm_all_reduce(tdm_engine* e, void* ptr, int64_t numel, int dtype, int avera
   });
 }
 
-int tdm_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
-                       tdm_stream caller, tdm_work** out) {
+namespace {
+int reduce_scatter_call(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
+                        bool owner_only, tdm_stream caller, tdm_work** out) {
   return guard([&] {
     if (out == nullptr) throw Invalid("NULL work pointer");
     if (nsizes < 0 || (nsizes > 0 && sizes == nullptr)) throw Invalid("bad sizes");
     std::vector<int64_t> sz(sizes, sizes + nsizes);
     finish_submit(engine_of(e).reduce_scatter(Engine::Buf{static_cast<char*>(ptr), numel, dtype}, std::move(sz),
-                                              average != 0, static_cast<hipStream_t>(caller)), out);
+                                              average != 0, owner_only, static_cast<hipStream_t>(caller)), out);
   });
+}
+}  // namespace
+
+int tdm_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
+                       tdm_stream caller, tdm_work** out) {
+  return reduce_scatter_call(e, ptr, numel, dtype, sizes, nsizes, average, false, caller, out);
+}
+
+int tdm_reduce_scatter_owner(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
+                             tdm_stream caller, tdm_work** out) {
+  return reduce_scatter_call(e, ptr, numel, dtype, sizes, nsizes, average, true, caller, out);
 }
 
 int tdm_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, tdm_stream caller,

@@ -127,7 +127,7 @@ class ZeRO(torch.nn.Module):
             for p in rng.params:
                 p.grad = None  # the full-size gradient is not kept
             rng.work = self.g.reduce_scatter(rng.staging, self.flat.bucket_sizes(rng.a, rng.b), op="avg", async_op=True,
-                                             **self._how)
+                                             **self._how, **self._mine_only)
 
     def _on_grad(self, p):
         rng = self.bucket_of[p]
@@ -168,6 +168,12 @@ class ZeRO(torch.nn.Module):
     @property
     def _how(self):
         return {"direct": True} if self.direct else {}
+
+    @property
+    def _mine_only(self):
+        """Stage 2 keeps only `mine` of a bucket's reduce_scatter and drops the staging
+        buffer: a group that can skip the other chunks' partial sums is told so."""
+        return {"partial_sums": False} if getattr(self.g, "partial_sums_optional", False) and not self.direct else {}
 
     def zero_grad(self):
         if self.stage == 1:
@@ -341,7 +347,9 @@ class FSDP(torch.nn.Module):
             for q in u.params:
                 q.grad = None
             self._release(u)
-            u.rs = self.g.reduce_scatter(u.staging, u.flat.sizes, op="avg", async_op=True)
+            # only `mine` is kept of the staging buffer: the other chunks' partial sums are not needed
+            how = {"partial_sums": False} if getattr(self.g, "partial_sums_optional", False) else {}
+            u.rs = self.g.reduce_scatter(u.staging, u.flat.sizes, op="avg", async_op=True, **how)
 
     def _after_backward(self):
         self._callback_queued = False

@@ -52,6 +52,10 @@ def collectives(g, dtype, n):
         mine = g.reduce_scatter(t, sizes, op=op)
         assert mine.data_ptr() == t.data_ptr() + lo * t.element_size() and mine.numel() == sizes[r]
         out[f"rs_{op}"] = t.cpu()
+        t = x.clone()
+        mine = g.reduce_scatter(t, sizes, op=op, partial_sums=False)  # the rest of t stays as it was
+        assert mine.data_ptr() == t.data_ptr() + lo * t.element_size() and mine.numel() == sizes[r]
+        out[f"rso_{op}"] = t.cpu()
     t = torch.zeros(n, dtype=dtype, device=dev)
     t[lo:lo + sizes[r]] = x[lo:lo + sizes[r]]
     g.all_gather(t, sizes)
@@ -70,9 +74,21 @@ def collectives(g, dtype, n):
     return out
 
 
+def choose(monkeypatch, algo):
+    """The engine's two ways through all_reduce / all_gather: staged through memory the
+    peers map (default; "small": 4 KiB halves, so n = 10,007 takes several passes and
+    both halves are reused), or the reference's ring through the slots."""
+    monkeypatch.setenv("TANDEM_HIP_ALGO", "ring" if algo == "ring" else "staged")
+    if algo == "small":
+        monkeypatch.setenv("TANDEM_HIP_STAGING_BYTES", "4096")
+    else:
+        monkeypatch.delenv("TANDEM_HIP_STAGING_BYTES", raising=False)
+
+
+@pytest.mark.parametrize("algo", ["staged", "small", "ring"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.int64, torch.float64])
 @pytest.mark.parametrize("world", [2, 3, 4])
-def test_collectives_bit_exact(dtype, world):
+def test_collectives_bit_exact(dtype, world, algo, monkeypatch):
     """4 KiB slots and n = 10,007: every collective runs through several pieces,
     reuses each slot, and ends on a short piece (tests/test_engine_cuda.py:84-96 in
     the reference, which only asks for a tolerance at world 3)."""
@@ -81,6 +97,9 @@ def test_collectives_bit_exact(dtype, world):
 
     if world == 4 and dtype in (torch.float16, torch.float64):
         pytest.skip("covered at world 2 and 3")
+    if algo != "small" and dtype in (torch.float16, torch.float64, torch.int64) and world == 3:
+        pytest.skip("these dtypes at world 3: the several-pass case only")
+    choose(monkeypatch, algo)
     n, kind = 10_007, KINDS[dtype]
     res = launch(collectives, world, dtype, n, slot_bytes=4096, gpus=[0] * world, timeout=TIMEOUT)
     xs = [to_np(values(q, n, dtype)) for q in range(world)]
@@ -92,6 +111,15 @@ def test_collectives_bit_exact(dtype, world):
             assert np.array_equal(bits(to_np(out["ar_avg"])), bits(ring.expected_all_reduce(xs, True, kind))), (r, "ar_avg")
             assert np.array_equal(bits(to_np(out["rs_avg"])), bits(ring.expected_reduce_scatter(xs, sizes, True, kind)[r])), (r, "rs_avg")
         assert np.array_equal(bits(to_np(out["rs_sum"])), bits(ring.expected_reduce_scatter(xs, sizes, False, kind)[r])), (r, "rs_sum")
+        lo = sum(sizes[:r])
+        for op in (("sum", "avg") if dtype.is_floating_point else ("sum",)):
+            got = to_np(out[f"rso_{op}"])
+            own = ring.expected_reduce_scatter(xs, sizes, op == "avg", kind)[r][lo:lo + sizes[r]]
+            assert np.array_equal(bits(got[lo:lo + sizes[r]]), bits(own)), (r, op, "owner's chunk")
+            if algo != "ring":  # (the ring leaves its partial sums there in any case)
+                rest = np.ones(n, bool)
+                rest[lo:lo + sizes[r]] = False
+                assert np.array_equal(bits(got[rest]), bits(xs[r][rest])), (r, op, "rest untouched")
         assert np.array_equal(bits(to_np(out["ag"])), bits(ring.expected_all_gather(xs, sizes))), (r, "ag")
         assert np.array_equal(bits(to_np(out["bcast"])), bits(xs[world - 1])), (r, "bcast")
         if world == 2:
@@ -156,11 +184,13 @@ def replay_fixture(g, inputs, cases):
     return out
 
 
+@pytest.mark.parametrize("algo", ["staged", "small", "ring"])
 @pytest.mark.parametrize("world", [2, 3, 4])
-def test_reference_fixtures(world):
+def test_reference_fixtures(world, algo, monkeypatch):
     """The same inputs and slot size as the reference engine's run."""
     from tandem_amd import launch
 
+    choose(monkeypatch, algo)
     d = golden_npz(f"ring_w{world}.npz")
     inputs = [d[f"r{r}_in"] for r in range(world)]
     res = launch(replay_fixture, world, inputs, npz_json(d, "sizes_json"), slot_bytes=256, gpus=[0] * world, timeout=TIMEOUT)
