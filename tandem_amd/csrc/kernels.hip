@@ -371,7 +371,13 @@ template <typename T, int kWorld, int kDiv, bool kAcc, int kMask>
 __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const Divisor<T>& dv) {
   using A = typename Elem<T>::acc;
   constexpr int L = lanes<T>();
-  constexpr int kU = kWorld <= 2 ? 4 : 2;  // vectors per lane per tile step, per rank
+#ifndef TDM_K2_UNROLL_W2
+#define TDM_K2_UNROLL_W2 4
+#endif
+#ifndef TDM_K2_UNROLL
+#define TDM_K2_UNROLL 2
+#endif
+  constexpr int kU = kWorld <= 2 ? TDM_K2_UNROLL_W2 : TDM_K2_UNROLL;  // vectors per lane per tile step, per rank
   constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
   const int64_t n = sg.count;
   const int c = sg.chunk;
@@ -523,11 +529,16 @@ __device__ __forceinline__ void adamw_elem(float& p, float g, float& m, float& v
   }
 }
 
+#ifndef TDM_K3_UNROLL
+#define TDM_K3_UNROLL 1
+#endif
+constexpr int kAdamwUnroll = TDM_K3_UNROLL;  // vectors per lane and stream in flight
+
 template <int kOrder, bool kVec>
 __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
   const bool small_w = __builtin_fabsf(a.s.w1) < 0.5f;
   if constexpr (kVec) {
-    constexpr int kU = 2;
+    constexpr int kU = kAdamwUnroll;
     const int64_t nv = a.n / 4;
     const int64_t tiles = (nv + kThreads * kU - 1) / (kThreads * kU);
     for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
@@ -1097,7 +1108,7 @@ int tdm_k3_adamw(float* p, const float* g, float* m, float* v, int64_t n, const 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 block(kThreads);
     if (vec) {
-      const int64_t tiles = (n / 4 + kThreads * 2 - 1) / (kThreads * 2);
+      const int64_t tiles = (n / 4 + kThreads * kAdamwUnroll - 1) / (kThreads * kAdamwUnroll);
       const dim3 grid(grid_for(std::max<int64_t>(tiles, 1)));
       if (order == TDM_ADAMW_HOST_ORDER) hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true>), grid, block, 0, st, a);
       else hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true>), grid, block, 0, st, a);
