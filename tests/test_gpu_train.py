@@ -27,7 +27,7 @@ def deterministic():
     torch.backends.cuda.matmul.allow_tf32 = False
 
 
-def train_rank(g, strategy, bucket_bytes, steps, batch):
+def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1):
     from tandem_amd import ShardedAdamW
     from tandem_amd.data import synthetic
     from tandem_amd.ddp import DDP
@@ -55,9 +55,15 @@ def train_rank(g, strategy, bucket_bytes, steps, batch):
             assert z._direct == (not strategy.endswith("s"))
     losses = []
     for step in range(steps):
-        x, y = text.batch(step, batch, c.seq, rank=g.rank, world=g.size, device=g.device)
-        loss = z(x, y)
-        loss.backward()
+        for micro in range(accumulate):
+            x, y = text.batch(step * accumulate + micro, batch, c.seq, rank=g.rank, world=g.size, device=g.device)
+            if micro < accumulate - 1:  # DDP only: accumulate locally, reduce with the last micro-batch
+                with z.no_sync():
+                    loss = z(x, y)
+                    (loss / accumulate).backward()
+            else:
+                loss = z(x, y)
+                (loss / accumulate).backward() if accumulate > 1 else loss.backward()
         losses.append(loss.item())
         if strategy.startswith("ddp"):
             opt.step()
@@ -74,7 +80,7 @@ def train_rank(g, strategy, bucket_bytes, steps, batch):
     return {"losses": losses, "weights": w.cpu(), **extra}
 
 
-def one_process(world):
+def one_process(world, accumulate=1):
     """Both ranks' gradients computed in this process, averaged as (a/2) + (b/2),
     torch AdamW on the GPU."""
     from tandem_amd.data import synthetic
@@ -91,9 +97,10 @@ def one_process(world):
     for step in range(STEPS):
         grads = []
         for r in range(world):
-            x, y = text.batch(step, BATCH, c.seq, rank=r, world=world, device=dev)
-            loss = model(x, y)
-            loss.backward()
+            for micro in range(accumulate):
+                x, y = text.batch(step * accumulate + micro, BATCH, c.seq, rank=r, world=world, device=dev)
+                loss = model(x, y)
+                (loss / accumulate).backward() if accumulate > 1 else loss.backward()
             losses[r].append(loss.item())
             grads.append([p.grad.clone() for p in model.parameters()])
             opt.zero_grad()
@@ -141,3 +148,16 @@ def test_four_ranks_stay_in_step():
     for direct, ring in (("ddpd", "ddp"), ("zero2d", "zero2"), ("zero1d", "zero1")):
         assert kept[direct]["losses"] == kept[ring]["losses"], direct
         assert torch.equal(kept[direct]["weights"], kept[ring]["weights"]), direct
+
+
+def test_gradient_accumulation_matches_one_process():
+    """DDP.no_sync (tests/test_ddp.py:115-119 in the reference): two micro-batches, the
+    first accumulated locally inside the buckets, the sum reduced with the second."""
+    from tandem_amd import launch
+
+    ref_losses, ref_w = one_process(2, accumulate=2)
+    for s in ("ddp", "ddpd"):
+        res = launch(train_rank, 2, s, 4 << 10, STEPS, BATCH, 2, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT)
+        for r in range(2):
+            assert res[r]["losses"] == ref_losses[r], (s, r)
+            assert torch.equal(res[r]["weights"], ref_w), (s, r)
