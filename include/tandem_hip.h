@@ -284,6 +284,9 @@ int tdm_barrier(tdm_engine* e, tdm_work** out);
 /* Work handle (tandem/csrc/collectives.h:43-66, tandem/csrc/engine.cpp:103-107).
  * wait: blocks the host until the collective's GPU work has been enqueued, then
  * makes `caller` wait for it on the GPU; returns the collective's error, if any.
+ * (With the default host ordering between ranks, a collective's last launch is
+ * enqueued only when the GPU has finished the hand-over before it, so wait returns
+ * about when that last kernel starts, not right after submission.)
  * done: 1 once the GPU has finished it. times: when the progress thread started and
  * finished it, seconds on CLOCK_MONOTONIC (Python's time.perf_counter clock); for a
  * collective submitted while tdm_engine_set_timing was on, when the GPU started it

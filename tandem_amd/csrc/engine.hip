@@ -27,8 +27,12 @@
 //
 // Streams: a collective starts on the engine's stream once the caller's stream
 // has reached the point of submission (an event), and tdm_work_wait makes the
-// caller's stream wait for the collective's last kernel; the host is not blocked
-// on GPU work in either direction (tandem/csrc/collectives.cpp:159-224).
+// caller's stream wait for the collective's last kernel, as in the reference
+// (tandem/csrc/collectives.cpp:159-224). Submission never blocks the caller. With
+// host ordering, however, the progress thread hands every piece (and every fence)
+// over only once the GPU has produced it, so a job is not fully enqueued before its
+// last hand-over has happened on the GPU, and tdm_work_wait, which waits for the
+// job to be enqueued, returns about when the collective's last kernel starts.
 
 #include <fcntl.h>
 #include <sys/mman.h>

@@ -6,10 +6,11 @@ Compute spans are taken on the training thread between device synchronisations
 (`Timeline.span`), communication spans come from `Group.trace`, which here holds
 the GPU's own start and end of every collective (device time stamps placed on
 time.perf_counter's clock), and `Group.waits` holds the time the training thread
-was blocked in `Work.wait()`. On this backend `wait()` blocks the host only until
-the collective has been enqueued, so `exposed_comm_s` is the host's share; what
-the GPU's default stream waited for shows in the Chrome trace, where compute and
-communication rows share one clock.
+was blocked in `Work.wait()`. On this backend `wait()` returns once the collective's
+last kernel has been enqueued, which (hand-over between ranks being ordered on the
+host) is about when that kernel starts on the GPU; what the GPU's default stream
+then still waits for shows in the Chrome trace, where compute and communication
+rows share one clock.
 """
 
 import contextlib
