@@ -364,11 +364,22 @@ def ipc_allreduce():
     sizes = [64, 256, 1024, 4096, 16384, 65536]
     out = {"workload": "all_reduce(sum) fp32 between 2 processes sharing the GPU through HIP IPC, barrier + all_reduce + device sync, median of 20",
            "reference_T4_cpp_engine_ms": {"64": 0.64, "256": 0.80, "1024": 0.83, "4096": 0.75, "16384": 1.72, "65536": 6.24}}
-    for label, slot in (("slots_2x4MiB_ms", 4 << 20), ("slots_2x64MiB_ms", 64 << 20)):
-        res = launch(ipc_rank, 2, sizes, 20, slot_bytes=slot, gpus=[0, 0], timeout=120.0)[0]
-        out[label] = {str(k): round(v * 1e3, 3) for k, v in res.items()}
-    res = launch(ipc_rank, 2, sizes, 20, True, gpus=[0, 0], timeout=120.0)[0]
-    out["direct_arena_ms"] = {str(k): round(v * 1e3, 3) for k, v in res.items()}
+
+    def run(direct=False):
+        res = launch(ipc_rank, 2, sizes, 20, direct, gpus=[0, 0], timeout=120.0)[0]
+        return {str(k): round(v * 1e3, 3) for k, v in res.items()}
+
+    out["staged_ms"] = run()  # the default: through peer-mapped staging memory
+    out["direct_arena_ms"] = run(True)  # tensors in the shared arenas
+    before = os.environ.get("TANDEM_HIP_ALGO")
+    os.environ["TANDEM_HIP_ALGO"] = "ring"  # the reference's protocol: pieces through 2 x 4 MiB slots per pair
+    try:
+        out["slot_ring_2x4MiB_ms"] = run()
+    finally:
+        if before is None:
+            del os.environ["TANDEM_HIP_ALGO"]
+        else:
+            os.environ["TANDEM_HIP_ALGO"] = before
     return out
 
 

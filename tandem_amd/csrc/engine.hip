@@ -195,6 +195,22 @@ bool spin_for(Ready ready, std::chrono::microseconds limit = kSpinBeforeSleep) {
   }
 }
 
+// Waiting for the GPU from a helper thread: poll (a query is cheap and takes no lock for
+// long), first tightly, then every 50 us. The runtime's own blocking waits are avoided on
+// purpose: while one thread sat in them for milliseconds, the training thread's kernel
+// launches were seen to stall. `query` returns hipErrorNotReady until the work is done.
+template <class Query>
+hipError_t poll_gpu(Query query, double timeout_s) {
+  hipError_t err = hipErrorNotReady;
+  if (spin_for([&] { return (err = query()) != hipErrorNotReady; }, std::chrono::microseconds(300))) return err;
+  const auto deadline = std::chrono::steady_clock::now() + std::chrono::duration<double>(timeout_s);
+  for (;;) {
+    std::this_thread::sleep_for(std::chrono::microseconds(50));
+    if ((err = query()) != hipErrorNotReady) return err;
+    if (std::chrono::steady_clock::now() > deadline) throw Timeout("timed out waiting for the GPU");
+  }
+}
+
 // Spin, then yield, then short sleeps; throws Timeout.
 template <class Ready>
 void wait_until(Ready ready, double timeout_s, const char* what) {
@@ -236,6 +252,7 @@ struct Work {
   double t0 = 0, t1 = 0;
   hipEvent_t done_event = nullptr;  // recorded on the engine's stream after the job (jobs with GPU work)
   bool uses_gpu = false;
+  bool same_stream = false;  // its kernels were launched on the caller's own stream: wait() has nothing to order
   bool drained = false;  // the job ends with a fence: the engine's stream is idle when it has run
   int device = -1;
   // Device timing (only while the engine's timing switch is on): start_event is
@@ -292,8 +309,9 @@ class Engine {
     int64_t numel;
   };
 
-  std::shared_ptr<Work> submit(std::function<void()> job, hipStream_t caller, bool uses_gpu, bool host_ready = false);
-  void stamp_start(Work& w);
+  std::shared_ptr<Work> submit(std::function<void()> job, hipStream_t caller, bool uses_gpu, bool host_ready = false,
+                               bool drained = false);
+  void stamp_start(Work& w, hipStream_t on);
   char* staging_half();
   const char* peer_staging(int peer, int half);
   void copy_pairs(const tdm_pair* pairs, int np, int dtype);
@@ -331,6 +349,9 @@ class Engine {
   int device_;
   bool use_events_;
   hipStream_t stream_ = nullptr;
+  hipStream_t gather_stream_ = nullptr;  // direct unit gathers, launched by the caller's thread
+  hipStream_t anchor_stream_ = nullptr;  // carries nothing but the timing anchors: always idle
+  std::mutex anchor_mu_, arena_mu_;      // both threads time their work and map peers' arenas
   Region mine_;
   std::vector<std::unique_ptr<Region>> theirs_;
   std::vector<void*> out_mem_, peer_mem_;
@@ -345,13 +366,15 @@ class Engine {
   bool connected_ = false, closed_ = false;
   // staged collectives
   bool staged_ = true;               // TANDEM_HIP_ALGO=ring switches them off
-  size_t staging_half_ = 32u << 20;  // bytes per half (TANDEM_HIP_STAGING_BYTES)
+  bool gathers_on_side_stream_ = false;  // TANDEM_HIP_GATHER=stream
+  bool ready_on_host_ = true;        // TANDEM_HIP_READY=gpu: wait for the caller's stream on the GPU instead
+  size_t staging_half_ = 64u << 20;  // bytes per half (TANDEM_HIP_STAGING_BYTES)
   void* staging_ = nullptr;
   std::vector<void*> peer_staging_;
   uint64_t staged_ops_ = 0;          // picks the half; the same count on every rank
   std::atomic<int> timing_{0};
-  bool timing_seen_ = false;           // progress thread only
-  std::shared_ptr<Anchor> anchor_;     // progress thread only
+  bool timing_seen_ = false;           // under anchor_mu_
+  std::shared_ptr<Anchor> anchor_;     // under anchor_mu_
 
   // "host" ordering: what to publish once the GPU has passed an event.
   struct Completion {
@@ -405,6 +428,8 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
     if (v < 4096 || v >= (1ll << 30) || v % 4096) throw Invalid("TANDEM_HIP_STAGING_BYTES must be a multiple of 4096 in [4096, 1 GiB)");
     staging_half_ = static_cast<size_t>(v);
   }
+  if (const char* gm = std::getenv("TANDEM_HIP_GATHER")) gathers_on_side_stream_ = std::string(gm) == "stream";
+  if (const char* rd = std::getenv("TANDEM_HIP_READY")) ready_on_host_ = std::string(rd) != "gpu";
   peer_staging_.assign(size, nullptr);
 
   check_hip(hipSetDevice(device_), "hipSetDevice");
@@ -417,7 +442,9 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
 }
 
 void Engine::start() {
-  check_hip(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags");  // default priority
+  check_hip(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags");  // default priority, all three
+  check_hip(hipStreamCreateWithFlags(&gather_stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags (gathers)");
+  check_hip(hipStreamCreateWithFlags(&anchor_stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags (anchors)");
 
   mine_.create(region_name(rank_), size_);
   RegionHeader* h = mine_.header();
@@ -500,6 +527,7 @@ void Engine::close() {
   // Our GPU work must finish, and every peer's (they read our slots), before any
   // rank frees its slots and events.
   hipError_t sync_err = hipStreamSynchronize(stream_);
+  if (sync_err == hipSuccess && gather_stream_) sync_err = hipStreamSynchronize(gather_stream_);
   std::string barrier_err;
   if (connected_) {
     try {
@@ -540,8 +568,10 @@ void Engine::release_device() {
     peer_full_[p].clear(); peer_free_[p].clear(); full_[p].clear(); free_[p].clear();
     theirs_[p].reset();
   }
-  if (stream_) (void)hipStreamDestroy(stream_);
-  stream_ = nullptr;
+  for (hipStream_t* st : {&stream_, &gather_stream_, &anchor_stream_}) {
+    if (*st) (void)hipStreamDestroy(*st);
+    *st = nullptr;
+  }
   if (arena_) (void)hipFree(arena_);
   arena_ = nullptr;
   if (staging_) (void)hipFree(staging_);
@@ -561,11 +591,11 @@ Engine::~Engine() {
 // merely ordered on the GPU, so the progress thread itself waits for them (polling:
 // an idle stream passes the event within microseconds) and the engine's stream
 // is spared a wait packet.
-std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t caller, bool uses_gpu, bool host_ready) {
+std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t caller, bool uses_gpu, bool host_ready, bool drained) {
   auto work = std::make_shared<Work>();
   work->device = device_;
   work->uses_gpu = uses_gpu;
-  work->drained = host_ready;
+  work->drained = drained;
   hipEvent_t ready = nullptr;
   if (uses_gpu) {
     // Start once the caller's stream has produced the inputs.
@@ -578,15 +608,14 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
     job = [this, ready, host_ready, w = work.get(), inner = std::move(job)] {
       hipError_t e;
       if (host_ready) {
-        const bool passed = spin_for([&] { return hipEventQuery(ready) != hipErrorNotReady; }, std::chrono::microseconds(300));
-        e = passed ? hipEventQuery(ready) : hipEventSynchronize(ready);
-        if (!passed) (void)hipGetLastError();  // the "not ready" left by the last poll
+        e = poll_gpu([&] { return hipEventQuery(ready); }, timeout_s_);
+        (void)hipGetLastError();  // the "not ready" left by the polls
       } else {
         e = hipStreamWaitEvent(stream_, ready, 0);
       }
       (void)hipEventDestroy(ready);  // released once the GPU is past it
       check_hip(e, "waiting for the caller's stream (ready)");
-      stamp_start(*w);
+      stamp_start(*w, stream_);
       inner();
     };
   }
@@ -606,23 +635,23 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
 // With timing on: a time-stamped event on the engine's stream, after the wait for
 // the inputs and before the collective's first kernel. A fresh anchor is taken
 // each time the switch goes on, so the two clocks cannot drift far apart.
-void Engine::stamp_start(Work& w) {
-  const bool on = timing_.load(std::memory_order_acquire) != 0;
-  if (!on) {
+void Engine::stamp_start(Work& w, hipStream_t on) {
+  std::lock_guard<std::mutex> lock(anchor_mu_);
+  if (timing_.load(std::memory_order_acquire) == 0) {
     timing_seen_ = false;
     return;
   }
   if (!timing_seen_ || !anchor_) {
     auto a = std::make_shared<Anchor>();
     check_hip(hipEventCreateWithFlags(&a->event, hipEventDefault), "hipEventCreate (anchor)");
-    check_hip(hipEventRecord(a->event, stream_), "hipEventRecord (anchor)");
+    check_hip(hipEventRecord(a->event, anchor_stream_), "hipEventRecord (anchor)");
     check_hip(hipEventSynchronize(a->event), "hipEventSynchronize (anchor)");
     a->host = now_s();
     anchor_ = std::move(a);
     timing_seen_ = true;
   }
   check_hip(hipEventCreateWithFlags(&w.start_event, hipEventDefault), "hipEventCreate (start)");
-  check_hip(hipEventRecord(w.start_event, stream_), "hipEventRecord (start)");
+  check_hip(hipEventRecord(w.start_event, on), "hipEventRecord (start)");
   w.anchor = anchor_;
 }
 
@@ -740,19 +769,17 @@ void Engine::completion_loop() {
       cbusy_ = true;
     }
     if (c.after) {
-      // Short kernels finish within microseconds: poll first, then block.
-      hipError_t err = hipErrorNotReady;
-      const auto spin_until = std::chrono::steady_clock::now() + std::chrono::microseconds(200);
-      while ((err = hipEventQuery(c.after)) == hipErrorNotReady && std::chrono::steady_clock::now() < spin_until) {
+      hipError_t err;
+      try {
+        err = poll_gpu([&] { return hipEventQuery(c.after); }, timeout_s_);
+      } catch (const Timeout&) {
+        err = hipErrorNotReady;
       }
-      if (err == hipErrorNotReady) {
-        (void)hipGetLastError();
-        err = hipEventSynchronize(c.after);
-      }
+      (void)hipGetLastError();
       (void)hipEventDestroy(c.after);
       if (err != hipSuccess) {
         std::lock_guard<std::mutex> lock(cmu_);
-        if (cerror_.empty()) cerror_ = std::string("hipEventSynchronize: ") + hipGetErrorString(err);
+        if (cerror_.empty()) cerror_ = std::string("waiting for a piece's kernel: ") + hipGetErrorString(err);
       }
     }
     {
@@ -782,16 +809,11 @@ void Engine::barrier_now(bool after_gpu) {
   // peers anyway, and handing over to the completion thread would cost two wake-ups.
   drain_completions();
   if (after_gpu) {
-    const auto done = [this] {
-      const hipError_t err = hipStreamQuery(stream_);
-      if (err == hipErrorNotReady) {
-        (void)hipGetLastError();
-        return false;
-      }
+    for (hipStream_t st : {stream_, gather_stream_}) {
+      const hipError_t err = poll_gpu([st] { return hipStreamQuery(st); }, timeout_s_);
+      (void)hipGetLastError();
       check_hip(err, "hipStreamQuery (fence)");
-      return true;
-    };
-    if (!spin_for(done, std::chrono::microseconds(300))) check_hip(hipStreamSynchronize(stream_), "hipStreamSynchronize (fence)");
+    }
   }
   // An empty message to every peer, then one from each. Rings are first in,
   // first out, so this also orders the barrier after every piece queued before.
@@ -1137,7 +1159,7 @@ std::shared_ptr<Work> Engine::all_reduce(Buf t, bool average, hipStream_t caller
     auto c = chunks(t, {});
     ring_reduce_scatter(c, t.dtype, average, false);
     ring_all_gather(c, t.dtype);
-  }, caller, true);
+  }, caller, true, ready_on_host_);
 }
 
 std::shared_ptr<Work> Engine::reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, bool owner_only,
@@ -1150,7 +1172,7 @@ std::shared_ptr<Work> Engine::reduce_scatter(Buf t, std::vector<int64_t> sizes, 
     const auto cs = chunks(t, sizes);
     if (owner_only && staged_ && size_ <= TDM_MAX_WORLD) staged_reduce_scatter_owner(t, cs, average);
     else ring_reduce_scatter(cs, t.dtype, average, true);
-  }, caller, true);
+  }, caller, true, ready_on_host_);
 }
 
 std::shared_ptr<Work> Engine::all_gather(Buf t, std::vector<int64_t> sizes, hipStream_t caller) {
@@ -1161,7 +1183,7 @@ std::shared_ptr<Work> Engine::all_gather(Buf t, std::vector<int64_t> sizes, hipS
     const auto cs = chunks(t, sizes);
     if (staged_ && size_ < TDM_MAX_PAIRS) staged_all_gather(t, cs, cs[rank_].ptr);
     else ring_all_gather(cs, t.dtype);
-  }, caller, true);
+  }, caller, true, ready_on_host_);
 }
 
 // ZeRO-3's gather of one unit: this rank's shard is placed into its chunk of the
@@ -1192,7 +1214,7 @@ std::shared_ptr<Work> Engine::unit_gather(Buf full, const char* shard, std::vect
       }
     }
     if (size_ > 1) ring_all_gather(cs, full.dtype);
-  }, caller, true);
+  }, caller, true, ready_on_host_);
 }
 
 // Pipelined along the ring from the root: each rank forwards each piece as soon
@@ -1211,7 +1233,7 @@ std::shared_ptr<Work> Engine::broadcast(Buf t, int root, hipStream_t caller) {
       if (pos > 0) take(prv, piece, m, t.dtype, false, 0);
       if (pos < n - 1) put(nxt, piece, m, t.dtype, 0);
     }
-  }, caller, true);
+  }, caller, true, ready_on_host_);
 }
 
 std::shared_ptr<Work> Engine::sendrecv(Buf send, int dst, Buf recv, int src, hipStream_t caller) {
@@ -1224,7 +1246,7 @@ std::shared_ptr<Work> Engine::sendrecv(Buf send, int dst, Buf recv, int src, hip
   return submit([this, send, dst, recv, src, has_send, has_recv] {
     Chunk s{send.ptr, send.numel}, r{recv.ptr, recv.numel};
     exchange(has_send ? &s : nullptr, dst, has_recv ? &r : nullptr, src, has_send ? send.dtype : recv.dtype, false, 0, 0);
-  }, caller, true);
+  }, caller, true, ready_on_host_);
 }
 
 // ---------------------------------------------------------------- shared arena, direct gather
@@ -1252,6 +1274,7 @@ void* Engine::share(size_t bytes) {
 }
 
 const char* Engine::peer_arena(int peer, size_t need_bytes) {
+  std::lock_guard<std::mutex> lock(arena_mu_);
   if (!peer_arena_[peer]) {
     RegionHeader* h = theirs_[peer]->header();
     const uint64_t bytes = h->arena_bytes.load(std::memory_order_acquire);
@@ -1263,37 +1286,71 @@ const char* Engine::peer_arena(int peer, size_t need_bytes) {
   return static_cast<const char*>(peer_arena_[peer]);
 }
 
+// Launched by the caller's thread: a direct gather exchanges no message with any
+// rank, so it need not take its turn behind collectives whose hand-overs the progress
+// thread is waiting for, and the caller never blocks on it. By default the copies go
+// onto the caller's own stream, in order with its kernels: the copy of a 28 MB unit
+// takes tens of microseconds at HBM speed, while running it on a side stream (the
+// reference's design, TANDEM_HIP_GATHER=stream) costs two cross-queue waits per gather,
+// which on a GPU shared by several processes were measured to cost more than they hide
+// (85.8M GPT, 2 ranks: 26.7 ms per step in order, 29-34 ms on the side stream).
 std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, std::vector<int64_t> sizes,
                                                  std::vector<int64_t> peer_offsets, hipStream_t caller) {
   check(full, "unit_gather", false);
   if (full.dtype == kBytesDtype) throw Invalid("unit_gather: direct gathers need a typed tensor");
-  const auto c = chunks(full, sizes);
+  const auto cs = chunks(full, sizes);
   if (static_cast<int>(peer_offsets.size()) != size_) throw Invalid("unit_gather: one arena offset per rank");
-  if (c[rank_].numel > 0 && shard == nullptr) throw Invalid("unit_gather: NULL shard");
-  return submit([this, full, shard, sizes, peer_offsets] {
-    const auto cs = chunks(full, sizes);
-    const int es = elem_bytes(full.dtype);
-    tdm_pair pairs[TDM_MAX_PAIRS];
-    int np = 0;
-    auto flush = [&] {
-      if (np) copy_step(pairs, np, full.dtype, 0, stream_);
-      np = 0;
-    };
-    for (int q = 0; q < size_; ++q) {
-      if (cs[q].numel == 0) continue;
-      const char* from;
-      if (q == rank_) {
-        if (shard == cs[q].ptr) continue;
-        from = shard;
-      } else {
-        if (peer_offsets[q] < 0 || peer_offsets[q] % es) throw Invalid("unit_gather: bad arena offset");
-        from = peer_arena(q, static_cast<size_t>(peer_offsets[q]) + static_cast<size_t>(cs[q].numel) * es) + peer_offsets[q];
-      }
-      pairs[np++] = tdm_pair{cs[q].ptr, from, cs[q].numel};
-      if (np == TDM_MAX_PAIRS) flush();
+  if (cs[rank_].numel > 0 && shard == nullptr) throw Invalid("unit_gather: NULL shard");
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    if (stopping_) throw std::runtime_error("the engine is closed");
+  }
+  const int es = elem_bytes(full.dtype);
+  tdm_pair pairs[TDM_MAX_PAIRS * 2];
+  int np = 0;
+  for (int q = 0; q < size_; ++q) {
+    if (cs[q].numel == 0) continue;
+    const char* from;
+    if (q == rank_) {
+      if (shard == cs[q].ptr) continue;
+      from = shard;
+    } else {
+      if (peer_offsets[q] < 0 || peer_offsets[q] % es) throw Invalid("unit_gather: bad arena offset");
+      from = peer_arena(q, static_cast<size_t>(peer_offsets[q]) + static_cast<size_t>(cs[q].numel) * es) + peer_offsets[q];
     }
-    flush();
-  }, caller, true);
+    if (np == TDM_MAX_PAIRS * 2) throw Invalid("unit_gather: too many ranks");
+    pairs[np++] = tdm_pair{cs[q].ptr, from, cs[q].numel};
+  }
+  auto work = std::make_shared<Work>();
+  work->device = device_;
+  work->uses_gpu = true;
+  work->t0 = now_s();
+  check_hip(hipSetDevice(device_), "hipSetDevice");
+  hipStream_t on = caller;
+  if (gathers_on_side_stream_) {
+    // Start once the caller's stream has produced the buffer (and finished with its last use).
+    on = gather_stream_;
+    hipEvent_t ready;
+    check_hip(hipEventCreateWithFlags(&ready, hipEventDisableTiming), "hipEventCreateWithFlags (ready)");
+    hipError_t err = hipEventRecord(ready, caller);
+    if (err == hipSuccess) err = hipStreamWaitEvent(gather_stream_, ready, 0);
+    (void)hipEventDestroy(ready);
+    check_hip(err, "ordering a gather after the caller's stream");
+  }
+  stamp_start(*work, on);
+  for (int at = 0; at < np; at += TDM_MAX_PAIRS) {
+    copy_step(pairs + at, std::min<int>(TDM_MAX_PAIRS, np - at), full.dtype, 0, on);
+  }
+  // On the caller's own stream nothing needs ordering afterwards: the done event only
+  // serves done() and the time stamps, and wait() finds it on the stream it would wait on.
+  check_hip(hipEventCreateWithFlags(&work->done_event, work->start_event ? hipEventDefault : hipEventDisableTiming),
+            "hipEventCreateWithFlags (done)");
+  check_hip(hipEventRecord(work->done_event, on), "hipEventRecord (done)");
+  work->same_stream = !gathers_on_side_stream_;
+  work->t1 = now_s();
+  work->finished = true;
+  work->finished_hint.store(true, std::memory_order_release);
+  return work;
 }
 
 // ---------------------------------------------------------------- direct collectives
@@ -1378,7 +1435,7 @@ std::shared_ptr<Work> Engine::direct(int kind, Buf t, std::vector<int64_t> sizes
       direct_copies(t, cs, base);
       barrier_now(true);  // nobody reads our tensor any more
     }
-  }, caller, true, true);
+  }, caller, true, true, true);
 }
 
 // A barrier that is also ordered against the GPU: it starts after the caller's
@@ -1386,7 +1443,7 @@ std::shared_ptr<Work> Engine::direct(int kind, Buf t, std::vector<int64_t> sizes
 // announced once its engine stream has finished too.
 std::shared_ptr<Work> Engine::fence(hipStream_t caller) {
   if (!connected_) throw std::runtime_error("fence: the engine is not connected");
-  return submit([this] { barrier_now(true); }, caller, true, true);
+  return submit([this] { barrier_now(true); }, caller, true, true, true);
 }
 
 std::shared_ptr<Work> Engine::barrier() {
@@ -1598,7 +1655,7 @@ int tdm_work_wait(tdm_work* w, tdm_stream caller) {
       return work.status;
     }
   }
-  if (work.done_event) {
+  if (work.done_event && !work.same_stream) {
     return guard([&] {
       const hipError_t q = hipEventQuery(work.done_event);
       if (q == hipSuccess) return;  // the GPU is past it already: nothing to order

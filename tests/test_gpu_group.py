@@ -225,9 +225,13 @@ def direct_gather(g, numel):
     return out
 
 
+@pytest.mark.parametrize("where", ["caller", "stream"])
 @pytest.mark.parametrize("world", [2, 3])
-def test_direct_gather_from_shared_arenas(world):
+def test_direct_gather_from_shared_arenas(world, where, monkeypatch):
+    """The copies run on the caller's own stream (default) or on a side stream of the engine."""
     from tandem_amd import launch
+
+    monkeypatch.setenv("TANDEM_HIP_GATHER", where)
 
     numel = 100_003
     sizes = [numel // world + (1 if q < numel % world else 0) for q in range(world)]
@@ -369,8 +373,10 @@ def traced(g, mib, gemms):
     g.all_reduce(x)
     a @ a
     torch.cuda.synchronize()
+    # Whatever the algorithm, a rank reads W chunks and writes one to fold its own, and
+    # reads and writes the W-1 others: that much traffic at HBM peak bounds the span.
     chunk = 4 * n / g.size
-    floor = (g.size - 1) * (8 + 12 + 8 + 8) * chunk / 8e12  # this rank's own copies and reduces at HBM peak
+    floor = ((g.size + 1) + 2 * (g.size - 1)) * chunk / 8e12
     out = {}
     for mode in ("idle", "busy", "host"):
         os.environ["TANDEM_HIP_TRACE"] = "host" if mode == "host" else "device"
