@@ -247,13 +247,25 @@ def fsdp_rank(g, steps, prefetch):
 
 
 def fsdp_gather(steps):
+    """ZeRO-3's unit gathers: copies launched in order on the training stream (the
+    default), or on the engine's side stream with and without prefetch."""
     from tandem_amd import launch
 
     out = {}
-    for prefetch in (True, False):
-        res = launch(fsdp_rank, 2, steps, prefetch, slot_bytes=32 << 20, gpus=[0, 0], timeout=120.0)
-        out["prefetch" if prefetch else "no_prefetch"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in res[0].items()}
-    out["workload"] = "2 processes sharing the GPU (HIP IPC memory handles), 85.8M GPT = 14 units (12 blocks of 7,087,872), batch 8x512 split over 2 ranks, 32 MiB slots"
+    before = os.environ.get("TANDEM_HIP_GATHER")
+    try:
+        for label, where, prefetch in (("in_order", "caller", True), ("side_stream_prefetch", "stream", True),
+                                       ("side_stream_no_prefetch", "stream", False)):
+            os.environ["TANDEM_HIP_GATHER"] = where
+            res = launch(fsdp_rank, 2, steps, prefetch, gpus=[0, 0], timeout=120.0)
+            out[label] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in res[0].items()}
+    finally:
+        if before is None:
+            os.environ.pop("TANDEM_HIP_GATHER", None)
+        else:
+            os.environ["TANDEM_HIP_GATHER"] = before
+    out["workload"] = ("2 processes sharing the GPU (HIP IPC memory handles), 85.8M GPT = 14 units (12 blocks of 7,087,872), "
+                       "batch 8x512 split over 2 ranks, shards read directly from the peers' arenas")
     return out
 
 
