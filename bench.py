@@ -331,14 +331,14 @@ def train_rank(g, strategy, steps):
             "profile": {k: (round(v, 5) if isinstance(v, float) else v) for k, v in prof.items()}}
 
 
-def train_steps(steps):
+def train_steps(steps, world=2, strategies=("alone", "ddp", "ddp+direct", "zero1", "zero1+direct", "zero2", "zero2+direct", "zero3")):
     from tandem_amd import launch
 
-    out = {"workload": "2 processes sharing the GPU, 85.8M GPT, batch 8x512 split over the ranks, fp32, full step "
+    out = {"workload": f"{world} processes sharing the GPU, 85.8M GPT, batch 8x512 split over the ranks, fp32, full step "
                        "(forward, backward, optimizer); 'alone' = the same rows with no communication and torch AdamW; "
                        "'+direct' = buckets / flat buffers in the shared arenas, collectives arena to arena"}
-    for s in ("alone", "ddp", "ddp+direct", "zero1", "zero1+direct", "zero2", "zero2+direct", "zero3"):
-        res = launch(train_rank, 2, s, steps, gpus=[0, 0], timeout=120.0)
+    for s in strategies:
+        res = launch(train_rank, world, s, steps, gpus=[0] * world, timeout=120.0)
         out[s] = {"step_ms": round(max(r["step_ms"] for r in res), 3), "loss": round(res[0]["loss"], 4),
                   "profile_rank0": res[0]["profile"]}
     return out
@@ -484,7 +484,7 @@ def main():
     cpu = fsdp = None
     if not args.quick and not args.no_cpu:
         cpu = cpu_baseline(args.mib, 15)
-    ipc = train = None
+    ipc = train = train4 = None
     if not args.quick and not args.no_fsdp:
         try:
             fsdp = fsdp_gather(3)
@@ -498,6 +498,10 @@ def main():
             train = train_steps(5)
         except Exception as e:
             train = {"error": repr(e)[:300]}
+        try:
+            train4 = train_steps(5, 4, ("alone", "ddp", "zero2", "zero2+direct", "zero3"))
+        except Exception as e:
+            train4 = {"error": repr(e)[:300]}
 
     import torch
 
@@ -552,6 +556,8 @@ def main():
             line["ipc_allreduce_2_processes"] = ipc
         if train is not None:
             line["train_step_2_processes"] = train
+        if train4 is not None:
+            line["train_step_4_processes"] = train4
         if cpu is not None:
             cpu["gpu_over_cpu"] = round(line["value"] / cpu["value"], 1)
             cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["ms"], 1)
