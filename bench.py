@@ -193,10 +193,15 @@ def zero2_step(dev, reps):
     shard = z.layouts[0].hi - z.layouts[0].lo
     opt = timed(lambda: [z.opts[r].update("bench", z.bufs[r][z.layouts[r].lo:z.layouts[r].hi], z.grad_shards[r]) for r in range(WORLD)], reps)
     ag = timed(lambda: z.lw.all_gather(z.bufs, z.layouts[0].sizes), reps)
+    fused = timed(lambda: [z.opts[r].update("bench", z.bufs[r][z.layouts[r].lo:z.layouts[r].hi], z.grad_shards[r],
+                                            [z.bufs[q][z.layouts[r].lo:z.layouts[r].hi] for q in range(WORLD) if q != r])
+                           for r in range(WORLD)], reps)
     for algorithm, rs_bytes in (("fold", (WORLD + 2) * 4 * n), ("ring", 12 * (WORLD - 1) * n + 12 * n)):
-        step = timed(lambda: (refill(), z.reduce_grads(algorithm), z.step()), reps) - t_refill
+        # default: fold + the update that also writes the other ranks' copies; ring: three ring steps, update, ring all-gather
+        is_fold = algorithm == "fold"
+        step = timed(lambda: (refill(), z.reduce_grads(algorithm), z.step(fused_gather=is_fold)), reps) - t_refill
         rs = timed(lambda: (refill(), z.reduce_grads(algorithm)), reps) - t_refill
-        nbytes = rs_bytes + 28 * n + 8 * (WORLD - 1) * n
+        nbytes = rs_bytes + ((28 + 4 * (WORLD - 1)) * n if is_fold else 28 * n + 8 * (WORLD - 1) * n)
         key = "" if algorithm == "fold" else "ring_"
         out.update({f"{key}ms": round(step * 1e3, 4), f"{key}reduce_scatter_ms": round(rs * 1e3, 4),
                     f"{key}algorithmic_bytes": nbytes, f"{key}GBps": round(nbytes / step / 1e9, 1),
@@ -204,7 +209,11 @@ def zero2_step(dev, reps):
     out.update({"adamw_4_shards_ms": round(opt * 1e3, 4), "adamw_GBps": round(28 * shard * WORLD / opt / 1e9, 1),
                 "adamw_frac_of_hbm_peak": round(28 * shard * WORLD / opt / 1e9 / HBM_PEAK_GBPS, 4),
                 "all_gather_ms": round(ag * 1e3, 4), "all_gather_GBps": round(8 * (WORLD - 1) * n / ag / 1e9, 1),
-                "note": "ms: gradients reduced by the single-launch ring-order fold (default); ring_ms: by the ring's three steps"})
+                "adamw_gather_4_shards_ms": round(fused * 1e3, 4),
+                "adamw_gather_GBps": round((28 + 4 * (WORLD - 1)) * shard * WORLD / fused / 1e9, 1),
+                "note": "ms: gradients reduced by the single-launch ring-order fold, then AdamW writing the new parameters to all "
+                        "four ranks' buffers in the same pass (default); ring_ms: the ring's three reduce steps, AdamW, the ring's "
+                        "three gather steps"})
     return out
 
 

@@ -176,6 +176,13 @@ enum tdm_adamw_order {
 int tdm_k3_adamw(float* p, const float* g, float* m, float* v, int64_t n, const tdm_adamw_scalars* s, int order,
                  tdm_stream stream);
 
+/* The same step, and the all-gather that follows it in ZeRO's step (tandem/zero.py:160-164),
+ * in one pass: the updated parameters are also written to `ncopies` (<= 7) further buffers,
+ * the other ranks' copies of this shard. For ranks that are buffers in one memory; saves
+ * the gather's read of p and one launch per ring step. */
+int tdm_k3_adamw_gather(float* p, const float* g, float* m, float* v, int64_t n, const tdm_adamw_scalars* s, int order,
+                        float* const* copies, int ncopies, tdm_stream stream);
+
 /* ---- K4: ZeRO-3 unit gather ---------------------------------------------- */
 
 /* full[lo_q : lo_q + sizes[q]] = shards[q][0 : sizes[q]] for every rank q, in one

@@ -67,6 +67,9 @@ _SIGNATURES = {
                                           ctypes.c_int, ctypes.c_void_p]),
     "tdm_k3_adamw": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                     ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
+    "tdm_k3_adamw_gather": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+                                           ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.POINTER(ctypes.c_void_p),
+                                           ctypes.c_int, ctypes.c_void_p]),
     "tdm_k4_unit_gather": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_int64),
                                           ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
 }

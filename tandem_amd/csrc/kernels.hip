@@ -505,6 +505,10 @@ struct AdamwArgs {
   float* v;
   int64_t n;
   tdm_adamw_scalars s;
+  // Further copies of the updated parameters (the other ranks' flat buffers): the
+  // update and the all-gather of the result in one pass.
+  int ncopies;
+  float* copy[TDM_MAX_WORLD - 1];
 };
 
 template <int kOrder>
@@ -562,7 +566,9 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
                        V = unpack<float>(rv[u]);
 #pragma unroll
           for (int l = 0; l < 4; ++l) adamw_elem<kOrder>(P.v[l], G.v[l], M.v[l], V.v[l], a.s, small_w);
-          store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.p) + i * 16, pack<float>(P));
+          const vec16 packed = pack<float>(P);
+          store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.p) + i * 16, packed);
+          for (int c = 0; c < a.ncopies; ++c) store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.copy[c]) + i * 16, packed);
           store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.m) + i * 16, pack<float>(M));
           store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.v) + i * 16, pack<float>(V));
         }
@@ -571,11 +577,13 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
     if (blockIdx.x == 0 && threadIdx.x < a.n - nv * 4) {
       const int64_t i = nv * 4 + threadIdx.x;
       adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
+      for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
     }
   } else {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < a.n; i += stride) {
       adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
+      for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
     }
   }
 }
@@ -1085,40 +1093,55 @@ int tdm_k2_bucket_fold(const void* table_dev, int64_t ntiles, int dtype, int wor
   });
 }
 
+namespace {
+void adamw_launch(float* p, const float* g, float* m, float* v, int64_t n, const tdm_adamw_scalars* s, int order,
+                  float* const* copies, int ncopies, hipStream_t st) {
+  if (n < 0) throw Invalid("n is negative");
+  if (ncopies < 0 || ncopies > TDM_MAX_WORLD - 1) throw Invalid("at most 7 further copies of the parameters");
+  if (n == 0) return;
+  if (!p || !g || !m || !v || !s || (ncopies > 0 && !copies)) throw Invalid("NULL argument");
+  if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
+  uintptr_t ptrs[4 + TDM_MAX_WORLD - 1] = {reinterpret_cast<uintptr_t>(p), reinterpret_cast<uintptr_t>(g),
+                                           reinterpret_cast<uintptr_t>(m), reinterpret_cast<uintptr_t>(v)};
+  AdamwArgs a{p, g, m, v, n, *s, ncopies, {}};
+  for (int c = 0; c < ncopies; ++c) {
+    if (!copies[c]) throw Invalid("NULL copy of the parameters");
+    a.copy[c] = copies[c];
+    ptrs[4 + c] = reinterpret_cast<uintptr_t>(copies[c]);
+  }
+  bool vec = true;
+  for (int i = 0; i < 4 + ncopies; ++i) {
+    if (ptrs[i] % 4) throw Invalid("pointer not aligned to 4 bytes");
+    vec = vec && ptrs[i] % 16 == 0;
+  }
+  for (int i = 0; i < 4 + ncopies; ++i)
+    for (int j = i + 1; j < 4 + ncopies; ++j) {
+      const uintptr_t bytes = static_cast<uintptr_t>(n) * 4;
+      if (ptrs[i] < ptrs[j] + bytes && ptrs[j] < ptrs[i] + bytes) throw Invalid("p, g, m, v and the copies must not overlap");
+    }
+  const dim3 block(kThreads);
+  if (vec) {
+    const int64_t tiles = (n / 4 + kThreads * kAdamwUnroll - 1) / (kThreads * kAdamwUnroll);
+    const dim3 grid(grid_for(std::max<int64_t>(tiles, 1)));
+    if (order == TDM_ADAMW_HOST_ORDER) hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true>), grid, block, 0, st, a);
+  } else {
+    const dim3 grid(grid_for((n + kThreads - 1) / kThreads));
+    if (order == TDM_ADAMW_HOST_ORDER) hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, false>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, false>), grid, block, 0, st, a);
+  }
+  check_hip(hipGetLastError(), "k3_adamw launch");
+}
+}  // namespace
+
 int tdm_k3_adamw(float* p, const float* g, float* m, float* v, int64_t n, const tdm_adamw_scalars* s, int order,
                  tdm_stream stream) {
-  return guard([&] {
-    if (n < 0) throw Invalid("n is negative");
-    if (n == 0) return;
-    if (!p || !g || !m || !v || !s) throw Invalid("NULL argument");
-    if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
-    const uintptr_t ptrs[4] = {reinterpret_cast<uintptr_t>(p), reinterpret_cast<uintptr_t>(g),
-                               reinterpret_cast<uintptr_t>(m), reinterpret_cast<uintptr_t>(v)};
-    bool vec = true;
-    for (uintptr_t a : ptrs) {
-      if (a % 4) throw Invalid("pointer not aligned to 4 bytes");
-      vec = vec && a % 16 == 0;
-    }
-    for (int i = 0; i < 4; ++i)
-      for (int j = i + 1; j < 4; ++j) {
-        const uintptr_t bytes = static_cast<uintptr_t>(n) * 4;
-        if (ptrs[i] < ptrs[j] + bytes && ptrs[j] < ptrs[i] + bytes) throw Invalid("p, g, m, v must not overlap");
-      }
-    AdamwArgs a{p, g, m, v, n, *s};
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    const dim3 block(kThreads);
-    if (vec) {
-      const int64_t tiles = (n / 4 + kThreads * kAdamwUnroll - 1) / (kThreads * kAdamwUnroll);
-      const dim3 grid(grid_for(std::max<int64_t>(tiles, 1)));
-      if (order == TDM_ADAMW_HOST_ORDER) hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true>), grid, block, 0, st, a);
-      else hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true>), grid, block, 0, st, a);
-    } else {
-      const dim3 grid(grid_for((n + kThreads - 1) / kThreads));
-      if (order == TDM_ADAMW_HOST_ORDER) hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, false>), grid, block, 0, st, a);
-      else hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, false>), grid, block, 0, st, a);
-    }
-    check_hip(hipGetLastError(), "k3_adamw launch");
-  });
+  return guard([&] { adamw_launch(p, g, m, v, n, s, order, nullptr, 0, static_cast<hipStream_t>(stream)); });
+}
+
+int tdm_k3_adamw_gather(float* p, const float* g, float* m, float* v, int64_t n, const tdm_adamw_scalars* s, int order,
+                        float* const* copies, int ncopies, tdm_stream stream) {
+  return guard([&] { adamw_launch(p, g, m, v, n, s, order, copies, ncopies, static_cast<hipStream_t>(stream)); });
 }
 
 int tdm_k4_unit_gather(void* full, const void* const* shards, const int64_t* sizes, int world, int dtype,

@@ -48,11 +48,18 @@ class ShardedAdamW:
         self.state = {}  # key -> [step, exp_avg, exp_avg_sq]
         lib()
 
-    def update(self, key, param, grad):
+    def update(self, key, param, grad, copies=()):
         """One step for one shard: `param` and `grad` are same-shaped fp32
-        tensors in GPU memory; `key` names the shard's optimizer state."""
+        tensors in GPU memory; `key` names the shard's optimizer state. `copies`:
+        further tensors of the same shape (the other ranks' copies of this shard, when
+        the ranks are buffers in one memory) that receive the updated parameters in the
+        same pass, which makes the all-gather after the step unnecessary."""
         require_device_tensor(param, "ShardedAdamW.update(param)")
         require_device_tensor(grad, "ShardedAdamW.update(grad)")
+        for c in copies:
+            require_device_tensor(c, "ShardedAdamW.update(copies)")
+            if c.dtype != torch.float32 or c.shape != param.shape:
+                raise ValueError("a copy differs from param in dtype or shape")
         if param.dtype != torch.float32 or grad.dtype != torch.float32:
             raise ValueError("ShardedAdamW handles fp32 shards")
         if param.shape != grad.shape:
@@ -65,6 +72,13 @@ class ShardedAdamW:
         if param.numel() == 0:
             return
         s = step_scalars(step, self.lr, self.betas, self.eps, self.weight_decay)
+        if copies:
+            arr = (ctypes.c_void_p * len(copies))(*[c.data_ptr() for c in copies])
+            check(lib().tdm_k3_adamw_gather(ctypes.c_void_p(param.data_ptr()), ctypes.c_void_p(grad.data_ptr()),
+                                            ctypes.c_void_p(exp_avg.data_ptr()), ctypes.c_void_p(exp_avg_sq.data_ptr()),
+                                            param.numel(), ctypes.byref(s), self.order, arr, len(copies),
+                                            stream_ptr(param.device)))
+            return
         check(lib().tdm_k3_adamw(ctypes.c_void_p(param.data_ptr()), ctypes.c_void_p(grad.data_ptr()),
                                  ctypes.c_void_p(exp_avg.data_ptr()), ctypes.c_void_p(exp_avg_sq.data_ptr()),
                                  param.numel(), ctypes.byref(s), self.order, stream_ptr(param.device)))
