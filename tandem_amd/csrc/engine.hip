@@ -252,7 +252,8 @@ struct Work {
   double t0 = 0, t1 = 0;
   hipEvent_t done_event = nullptr;  // recorded on the engine's stream after the job (jobs with GPU work)
   bool uses_gpu = false;
-  bool same_stream = false;  // its kernels were launched on the caller's own stream: wait() has nothing to order
+  bool on_callers_stream = false;  // its kernels were launched on the submitting stream itself:
+  hipStream_t launched_on = nullptr;  // wait() from that stream has nothing to order
   bool drained = false;  // the job ends with a fence: the engine's stream is idle when it has run
   int device = -1;
   // Device timing (only while the engine's timing switch is on): start_event is
@@ -1346,7 +1347,8 @@ std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, st
   check_hip(hipEventCreateWithFlags(&work->done_event, work->start_event ? hipEventDefault : hipEventDisableTiming),
             "hipEventCreateWithFlags (done)");
   check_hip(hipEventRecord(work->done_event, on), "hipEventRecord (done)");
-  work->same_stream = !gathers_on_side_stream_;
+  work->on_callers_stream = !gathers_on_side_stream_;
+  work->launched_on = on;
   work->t1 = now_s();
   work->finished = true;
   work->finished_hint.store(true, std::memory_order_release);
@@ -1655,7 +1657,7 @@ int tdm_work_wait(tdm_work* w, tdm_stream caller) {
       return work.status;
     }
   }
-  if (work.done_event && !work.same_stream) {
+  if (work.done_event && !(work.on_callers_stream && work.launched_on == static_cast<hipStream_t>(caller))) {
     return guard([&] {
       const hipError_t q = hipEventQuery(work.done_event);
       if (q == hipSuccess) return;  // the GPU is past it already: nothing to order
