@@ -162,6 +162,9 @@ __device__ __forceinline__ vec16 pack(const Lanes<T>& in) {
 #ifndef TDM_NT_MASK_K3
 #define TDM_NT_MASK_K3 7  // AdamW
 #endif
+#ifndef TDM_NT_MASK_K3C
+#define TDM_NT_MASK_K3C TDM_NT_MASK_K3  // AdamW's further copies of the parameters
+#endif
 template <int kMask = TDM_NT_MASK>
 __device__ __forceinline__ vec16 load_stream(const void* p) {  // read once, never written here
   if constexpr (kMask & 2) return __builtin_nontemporal_load(static_cast<const vec16*>(p));
@@ -568,7 +571,7 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
           for (int l = 0; l < 4; ++l) adamw_elem<kOrder>(P.v[l], G.v[l], M.v[l], V.v[l], a.s, small_w);
           const vec16 packed = pack<float>(P);
           store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.p) + i * 16, packed);
-          for (int c = 0; c < a.ncopies; ++c) store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.copy[c]) + i * 16, packed);
+          for (int c = 0; c < a.ncopies; ++c) store16<TDM_NT_MASK_K3C>(reinterpret_cast<char*>(a.copy[c]) + i * 16, packed);
           store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.m) + i * 16, pack<float>(M));
           store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.v) + i * 16, pack<float>(V));
         }
