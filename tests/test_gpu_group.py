@@ -74,6 +74,19 @@ def collectives(g, dtype, n):
     return out
 
 
+def test_a_group_of_one():
+    """World 1 (tests/test_comm.py:55 in the reference runs its collectives at world 1 too):
+    every collective leaves the tensor as it is, averaging included."""
+    from tandem_amd import launch
+
+    n = 1000
+    (out,) = launch(collectives, 1, torch.float32, n, gpus=[0], timeout=TIMEOUT)
+    x = values(0, n, torch.float32)
+    for key in ("ar_sum", "ar_avg", "rs_sum", "rs_avg", "rso_sum", "rso_avg", "ag", "bcast"):
+        assert torch.equal(out[key], x), key
+    assert out["bool_bcast_ok"]
+
+
 def choose(monkeypatch, algo):
     """The engine's two ways through all_reduce / all_gather: staged through memory the
     peers map (default; "small": 4 KiB halves, so n = 10,007 takes several passes and
