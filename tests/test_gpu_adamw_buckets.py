@@ -100,6 +100,43 @@ def test_adamw_device_order_matches_torch_on_the_gpu(dev):
     assert torch.equal(p.view(torch.int32), pt.detach().view(torch.int32))
 
 
+def test_adamw_writing_further_copies(dev):
+    """The update that also writes the other ranks' copies of the shard (update and
+    all-gather in one pass): the same bits as the plain update in p, m, v, and the new
+    p in every copy; aligned and unaligned, one and seven copies; overlap refused."""
+    from tandem_amd import ShardedAdamW
+
+    kw = dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    g = torch.Generator().manual_seed(9)
+    for n, ncopies, shift in ((100_003, 1, 0), (4099, 7, 0), (65_536, 3, 0), (10_007, 3, 1)):
+        p0 = torch.randn(n, generator=g) * 0.02
+        plain, fused = ShardedAdamW(**kw), ShardedAdamW(**kw)
+        p = p0.clone().to(dev)
+        q_store = torch.zeros(n + 4, device=dev)
+        q = q_store[shift:shift + n]
+        q.copy_(p0)
+        stores = [torch.full((n + 8,), -7.0, device=dev) for _ in range(ncopies)]
+        copies = [st[shift + 1:shift + 1 + n] if shift else st[4:4 + n] for st in stores]
+        for step in range(3):
+            gr = (torch.randn(n, generator=g) * 1e-3).to(dev)
+            plain.update("k", p, gr)
+            fused.update("k", q, gr, copies)
+            for c in copies:
+                assert torch.equal(c.view(torch.int32), p.view(torch.int32)), (n, ncopies, step)
+        assert torch.equal(q.view(torch.int32), p.view(torch.int32))
+        for i in (1, 2):
+            assert torch.equal(fused.state["k"][i].view(torch.int32), plain.state["k"][i].view(torch.int32))
+        for st in stores:  # nothing outside the copies was written
+            lo = shift + 1 if shift else 4
+            assert float((st[:lo] + 7.0).abs().sum()) == 0 and float((st[lo + n:] + 7.0).abs().sum()) == 0
+    with pytest.raises(ValueError, match="overlap"):
+        fused.update("k", q, gr, [q])
+    with pytest.raises(ValueError, match="shape"):
+        fused.update("k", q, gr, [torch.zeros(n + 1, device=dev)])
+    with pytest.raises(ValueError, match="at most 7"):
+        fused.update("k", q, gr, [torch.zeros(n, device=dev) for _ in range(8)])
+
+
 def test_adamw_rejects_what_it_cannot_do(dev):
     from tandem_amd import ShardedAdamW
 
