@@ -541,7 +541,7 @@ __device__ __forceinline__ void adamw_elem(float& p, float g, float& m, float& v
 #endif
 constexpr int kAdamwUnroll = TDM_K3_UNROLL;  // vectors per lane and stream in flight
 
-template <int kOrder, bool kVec>
+template <int kOrder, bool kVec, bool kCopies>
 __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
   const bool small_w = __builtin_fabsf(a.s.w1) < 0.5f;
   if constexpr (kVec) {
@@ -571,7 +571,8 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
           for (int l = 0; l < 4; ++l) adamw_elem<kOrder>(P.v[l], G.v[l], M.v[l], V.v[l], a.s, small_w);
           const vec16 packed = pack<float>(P);
           store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.p) + i * 16, packed);
-          for (int c = 0; c < a.ncopies; ++c) store16<TDM_NT_MASK_K3C>(reinterpret_cast<char*>(a.copy[c]) + i * 16, packed);
+          if constexpr (kCopies)
+            for (int c = 0; c < a.ncopies; ++c) store16<TDM_NT_MASK_K3C>(reinterpret_cast<char*>(a.copy[c]) + i * 16, packed);
           store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.m) + i * 16, pack<float>(M));
           store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.v) + i * 16, pack<float>(V));
         }
@@ -580,13 +581,15 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
     if (blockIdx.x == 0 && threadIdx.x < a.n - nv * 4) {
       const int64_t i = nv * 4 + threadIdx.x;
       adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
-      for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
+      if constexpr (kCopies)
+        for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
     }
   } else {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < a.n; i += stride) {
       adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
-      for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
+      if constexpr (kCopies)
+        for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
     }
   }
 }
@@ -1123,15 +1126,18 @@ void adamw_launch(float* p, const float* g, float* m, float* v, int64_t n, const
       if (ptrs[i] < ptrs[j] + bytes && ptrs[j] < ptrs[i] + bytes) throw Invalid("p, g, m, v and the copies must not overlap");
     }
   const dim3 block(kThreads);
-  if (vec) {
-    const int64_t tiles = (n / 4 + kThreads * kAdamwUnroll - 1) / (kThreads * kAdamwUnroll);
-    const dim3 grid(grid_for(std::max<int64_t>(tiles, 1)));
-    if (order == TDM_ADAMW_HOST_ORDER) hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true>), grid, block, 0, st, a);
-  } else {
-    const dim3 grid(grid_for((n + kThreads - 1) / kThreads));
-    if (order == TDM_ADAMW_HOST_ORDER) hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, false>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, false>), grid, block, 0, st, a);
+  const int64_t tiles = vec ? (n / 4 + kThreads * kAdamwUnroll - 1) / (kThreads * kAdamwUnroll) : (n + kThreads - 1) / kThreads;
+  const dim3 grid(grid_for(std::max<int64_t>(tiles, 1)));
+  const int which = (order == TDM_ADAMW_HOST_ORDER ? 0 : 4) + (vec ? 2 : 0) + (ncopies > 0 ? 1 : 0);
+  switch (which) {
+    case 0: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, false, false>), grid, block, 0, st, a); break;
+    case 1: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, false, true>), grid, block, 0, st, a); break;
+    case 2: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true, false>), grid, block, 0, st, a); break;
+    case 3: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true, true>), grid, block, 0, st, a); break;
+    case 4: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, false, false>), grid, block, 0, st, a); break;
+    case 5: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, false, true>), grid, block, 0, st, a); break;
+    case 6: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true, false>), grid, block, 0, st, a); break;
+    default: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true, true>), grid, block, 0, st, a); break;
   }
   check_hip(hipGetLastError(), "k3_adamw launch");
 }
