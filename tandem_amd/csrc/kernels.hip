@@ -41,6 +41,7 @@ constexpr int kTileVecs = kThreads * kUnroll;   // 1024 vectors = 16 KiB of ever
 constexpr int kDefaultBlocksPerCu = 1024;
 
 int g_blocks_per_cu = kDefaultBlocksPerCu;
+constexpr int64_t kColdFootprint = int64_t(512) << 20;  // twice the Infinity Cache
 
 typedef uint32_t vec16 __attribute__((ext_vector_type(4)));  // one dwordx4 access
 
@@ -490,13 +491,15 @@ struct FoldSmall {
   FoldSegDev seg[TDM_MAX_WORLD];
 };
 
-template <typename T, int kWorld, int kDiv>
+// kCold: the launch's footprint is far beyond the 256 MB Infinity Cache, so nothing it
+// writes will be read from there: the cache policy of the once-per-step bucket fold.
+template <typename T, int kWorld, int kDiv, bool kCold>
 __global__ __launch_bounds__(kThreads) void k2_fold_small_kernel(FoldSmall tab, Divisor<T> dv) {
   const int64_t total = tab.tile_end[tab.nseg - 1];
   for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
     int lo = 0;
     while (tile >= tab.tile_end[lo]) ++lo;
-    fold_tile<T, kWorld, kDiv, false, TDM_NT_MASK>(tab.seg[lo], tile - (lo ? tab.tile_end[lo - 1] : 0), dv);
+    fold_tile<T, kWorld, kDiv, false, kCold ? TDM_NT_MASK_K2 : TDM_NT_MASK>(tab.seg[lo], tile - (lo ? tab.tile_end[lo - 1] : 0), dv);
   }
 }
 
@@ -709,10 +712,15 @@ template <typename T, int kWorld>
 void launch_fold_small_w(const FoldSmall& tab, int average, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(kWorld);
   const dim3 grid(grid_for(tab.tile_end[tab.nseg - 1])), block(kThreads);
-  switch (div_kind(kWorld, average != 0)) {
-    case 0: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0>), grid, block, 0, stream, tab, dv); break;
-    case 1: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1>), grid, block, 0, stream, tab, dv); break;
-    default: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2>), grid, block, 0, stream, tab, dv); break;
+  // bytes touched: every tile is read from kWorld ranks (and written back to most of them)
+  const bool cold = tab.tile_end[tab.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld > kColdFootprint;
+  switch (div_kind(kWorld, average != 0) * 2 + (cold ? 1 : 0)) {
+    case 0: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, 0, stream, tab, dv); break;
+    case 1: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, 0, stream, tab, dv); break;
+    case 2: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, false>), grid, block, 0, stream, tab, dv); break;
+    case 3: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, true>), grid, block, 0, stream, tab, dv); break;
+    case 4: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2, false>), grid, block, 0, stream, tab, dv); break;
+    default: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2, true>), grid, block, 0, stream, tab, dv); break;
   }
 }
 
