@@ -46,9 +46,10 @@ int guard(F&& body) {
 }
 
 // kernels.hip
+// policy: which accesses are non-temporal (2, 5 or 7; see kernels.hip); 2 suits a launch on its own
 void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool scale_dst, bool scale_src,
-                 bool writeback_src, hipStream_t stream);
-void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream);
+                 bool writeback_src, hipStream_t stream, int policy = 2);
+void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream, int policy = 2);
 void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream);
 
 }  // namespace tandem_hip

@@ -14,6 +14,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -211,7 +212,7 @@ __device__ __forceinline__ void reduce_elem(T& d, T& s, bool scale_dst, bool sca
   d = Elem<T>::narrow(static_cast<A>(x + y));
 }
 
-template <typename T, int kDiv>
+template <typename T, int kDiv, int kMask>
 __global__ __launch_bounds__(kThreads) void k1_reduce_kernel(PairTable tab, Divisor<T> dv) {
   constexpr int L = lanes<T>();
   constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
@@ -233,27 +234,27 @@ __global__ __launch_bounds__(kThreads) void k1_reduce_kernel(PairTable tab, Divi
       if ((t + 1) * kTileVecs <= nv) {  // a full tile: all loads first, then the arithmetic, then the stores
         vec16 a[kUnroll], b[kUnroll];
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) a[k] = load_rmw(dvp + (v0 + k * kThreads) * 16);
+        for (int k = 0; k < kUnroll; ++k) a[k] = load_rmw<kMask>(dvp + (v0 + k * kThreads) * 16);
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) b[k] = load_stream(svp + (v0 + k * kThreads) * 16);
+        for (int k = 0; k < kUnroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kThreads) * 16);
 #pragma unroll
         for (int k = 0; k < kUnroll; ++k) {
           Lanes<T> x = unpack<T>(a[k]), y = unpack<T>(b[k]);
 #pragma unroll
           for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
-          store16(dvp + (v0 + k * kThreads) * 16, pack<T>(x));
-          if (writeback) store16(svp + (v0 + k * kThreads) * 16, pack<T>(y));
+          store16<kMask>(dvp + (v0 + k * kThreads) * 16, pack<T>(x));
+          if (writeback) store16<kMask>(svp + (v0 + k * kThreads) * 16, pack<T>(y));
         }
       } else {
 #pragma unroll
         for (int k = 0; k < kUnroll; ++k) {
           const int64_t v = v0 + k * kThreads;
           if (v < nv) {
-            Lanes<T> x = unpack<T>(load_rmw(dvp + v * 16)), y = unpack<T>(load_stream(svp + v * 16));
+            Lanes<T> x = unpack<T>(load_rmw<kMask>(dvp + v * 16)), y = unpack<T>(load_stream<kMask>(svp + v * 16));
 #pragma unroll
             for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
-            store16(dvp + v * 16, pack<T>(x));
-            if (writeback) store16(svp + v * 16, pack<T>(y));
+            store16<kMask>(dvp + v * 16, pack<T>(x));
+            if (writeback) store16<kMask>(svp + v * 16, pack<T>(y));
           }
         }
       }
@@ -294,7 +295,7 @@ __device__ __forceinline__ T copy_elem(T s, const Divisor<T>& dv) {
   }
 }
 
-template <typename T, int kDiv>
+template <typename T, int kDiv, int kMask>
 __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Divisor<T> dv) {
   constexpr int L = lanes<T>();
   constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
@@ -315,7 +316,7 @@ __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Diviso
       if ((t + 1) * kTileVecs <= nv) {
         vec16 b[kUnroll];
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) b[k] = load_stream(svp + (v0 + k * kThreads) * 16);
+        for (int k = 0; k < kUnroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kThreads) * 16);
 #pragma unroll
         for (int k = 0; k < kUnroll; ++k) {
           if constexpr (kDiv != 0) {
@@ -324,17 +325,17 @@ __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Diviso
             for (int l = 0; l < L; ++l) y.v[l] = copy_elem<T, kDiv>(y.v[l], dv);
             b[k] = pack<T>(y);
           }
-          store16(dvp + (v0 + k * kThreads) * 16, b[k]);
+          store16<kMask>(dvp + (v0 + k * kThreads) * 16, b[k]);
         }
       } else {
 #pragma unroll
         for (int k = 0; k < kUnroll; ++k) {
           const int64_t v = v0 + k * kThreads;
           if (v < nv) {
-            Lanes<T> y = unpack<T>(load_stream(svp + v * 16));
+            Lanes<T> y = unpack<T>(load_stream<kMask>(svp + v * 16));
 #pragma unroll
             for (int l = 0; l < L; ++l) y.v[l] = copy_elem<T, kDiv>(y.v[l], dv);
-            store16(dvp + v * 16, pack<T>(y));
+            store16<kMask>(dvp + v * 16, pack<T>(y));
           }
         }
       }
@@ -674,25 +675,46 @@ int div_kind(int world, bool any_scale) {
   return (world & (world - 1)) == 0 ? 1 : 2;
 }
 
-template <typename T>
-void launch_reduce(const PairTable& tab, int64_t tiles, int world, bool any_scale, hipStream_t stream) {
+// The three cache policies K1 is built with (bit 0: loads of the stream that is read,
+// modified and written back; bit 1: loads of the read-once stream; bit 2: stores are
+// non-temporal): 2 for a launch on its own, 7 and 5 for the first and last steps of a ring.
+template <typename T, int kMask>
+void launch_reduce_m(const PairTable& tab, int64_t tiles, int world, bool any_scale, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(world);
   const dim3 grid(grid_for(tiles)), block(kThreads);
   switch (div_kind(world, any_scale)) {
-    case 0: hipLaunchKernelGGL((k1_reduce_kernel<T, 0>), grid, block, 0, stream, tab, dv); break;
-    case 1: hipLaunchKernelGGL((k1_reduce_kernel<T, 1>), grid, block, 0, stream, tab, dv); break;
-    default: hipLaunchKernelGGL((k1_reduce_kernel<T, 2>), grid, block, 0, stream, tab, dv); break;
+    case 0: hipLaunchKernelGGL((k1_reduce_kernel<T, 0, kMask>), grid, block, 0, stream, tab, dv); break;
+    case 1: hipLaunchKernelGGL((k1_reduce_kernel<T, 1, kMask>), grid, block, 0, stream, tab, dv); break;
+    default: hipLaunchKernelGGL((k1_reduce_kernel<T, 2, kMask>), grid, block, 0, stream, tab, dv); break;
   }
 }
 
 template <typename T>
-void launch_copy(const PairTable& tab, int64_t tiles, int world, hipStream_t stream) {
+void launch_reduce(const PairTable& tab, int64_t tiles, int world, bool any_scale, int policy, hipStream_t stream) {
+  switch (policy) {
+    case 7: launch_reduce_m<T, 7>(tab, tiles, world, any_scale, stream); break;
+    case 5: launch_reduce_m<T, 5>(tab, tiles, world, any_scale, stream); break;
+    default: launch_reduce_m<T, TDM_NT_MASK>(tab, tiles, world, any_scale, stream); break;
+  }
+}
+
+template <typename T, int kMask>
+void launch_copy_m(const PairTable& tab, int64_t tiles, int world, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(world);
   const dim3 grid(grid_for(tiles)), block(kThreads);
   switch (div_kind(world, true)) {
-    case 0: hipLaunchKernelGGL((k1_copy_kernel<T, 0>), grid, block, 0, stream, tab, dv); break;
-    case 1: hipLaunchKernelGGL((k1_copy_kernel<T, 1>), grid, block, 0, stream, tab, dv); break;
-    default: hipLaunchKernelGGL((k1_copy_kernel<T, 2>), grid, block, 0, stream, tab, dv); break;
+    case 0: hipLaunchKernelGGL((k1_copy_kernel<T, 0, kMask>), grid, block, 0, stream, tab, dv); break;
+    case 1: hipLaunchKernelGGL((k1_copy_kernel<T, 1, kMask>), grid, block, 0, stream, tab, dv); break;
+    default: hipLaunchKernelGGL((k1_copy_kernel<T, 2, kMask>), grid, block, 0, stream, tab, dv); break;
+  }
+}
+
+template <typename T>
+void launch_copy(const PairTable& tab, int64_t tiles, int world, int policy, hipStream_t stream) {
+  switch (policy) {
+    case 7: launch_copy_m<T, 7>(tab, tiles, world, stream); break;
+    case 5: launch_copy_m<T, 5>(tab, tiles, world, stream); break;
+    default: launch_copy_m<T, TDM_NT_MASK>(tab, tiles, world, stream); break;
   }
 }
 
@@ -763,7 +785,7 @@ void launch_fold(const void* image, int64_t tiles, int world, int average, bool 
 
 // Used by the engine too.
 void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool scale_dst, bool scale_src,
-                 bool writeback_src, hipStream_t stream) {
+                 bool writeback_src, hipStream_t stream, int policy) {
   const int es = elem_size(dtype);
   if (es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
   const bool any_scale = (scale_dst || scale_src) && world > 1;
@@ -773,17 +795,17 @@ void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool s
   if (tiles == 0) return;
   tab.flags = (any_scale && scale_dst ? 1 : 0) | (any_scale && scale_src ? 2 : 0) | (any_scale && scale_src && writeback_src ? 4 : 0);
   switch (dtype) {
-    case TDM_F32: launch_reduce<float>(tab, tiles, world, any_scale, stream); break;
-    case TDM_F64: launch_reduce<double>(tab, tiles, world, any_scale, stream); break;
-    case TDM_F16: launch_reduce<f16_t>(tab, tiles, world, any_scale, stream); break;
-    case TDM_BF16: launch_reduce<bf16_t>(tab, tiles, world, any_scale, stream); break;
-    case TDM_I64: launch_reduce<int64_t>(tab, tiles, 1, false, stream); break;
-    default: launch_reduce<int32_t>(tab, tiles, 1, false, stream); break;
+    case TDM_F32: launch_reduce<float>(tab, tiles, world, any_scale, policy, stream); break;
+    case TDM_F64: launch_reduce<double>(tab, tiles, world, any_scale, policy, stream); break;
+    case TDM_F16: launch_reduce<f16_t>(tab, tiles, world, any_scale, policy, stream); break;
+    case TDM_BF16: launch_reduce<bf16_t>(tab, tiles, world, any_scale, policy, stream); break;
+    case TDM_I64: launch_reduce<int64_t>(tab, tiles, 1, false, policy, stream); break;
+    default: launch_reduce<int32_t>(tab, tiles, 1, false, policy, stream); break;
   }
   check_hip(hipGetLastError(), "k1_reduce launch");
 }
 
-void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream) {
+void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream, int policy) {
   const int es = elem_size(dtype);
   if (es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
   if (world > 1 && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
@@ -806,12 +828,12 @@ void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStrea
   const int64_t tiles = build_pairs(kept.data(), static_cast<int>(kept.size()), es, false, &tab);
   if (tiles == 0) return;
   switch (dtype) {
-    case TDM_F32: launch_copy<float>(tab, tiles, world, stream); break;
-    case TDM_F64: launch_copy<double>(tab, tiles, world, stream); break;
-    case TDM_F16: launch_copy<f16_t>(tab, tiles, world, stream); break;
-    case TDM_BF16: launch_copy<bf16_t>(tab, tiles, world, stream); break;
-    case TDM_I64: launch_copy<int64_t>(tab, tiles, 1, stream); break;
-    default: launch_copy<int32_t>(tab, tiles, 1, stream); break;
+    case TDM_F32: launch_copy<float>(tab, tiles, world, policy, stream); break;
+    case TDM_F64: launch_copy<double>(tab, tiles, world, policy, stream); break;
+    case TDM_F16: launch_copy<f16_t>(tab, tiles, world, policy, stream); break;
+    case TDM_BF16: launch_copy<bf16_t>(tab, tiles, world, policy, stream); break;
+    case TDM_I64: launch_copy<int64_t>(tab, tiles, 1, policy, stream); break;
+    default: launch_copy<int32_t>(tab, tiles, 1, policy, stream); break;
   }
   check_hip(hipGetLastError(), "k1_copy launch");
 }
@@ -873,6 +895,29 @@ int wrap(int a, int n) { return ((a % n) + n) % n; }
 
 // Step s: rank r adds chunk (r-s-2) of rank r-1 into its own (tandem/comm.py:301-305).
 // Every receiving chunk is still undivided; the sender's only on the first step.
+// Cache policy of each step of a ring on one GPU: the best of all combinations of 2, 5
+// and 7 over the steps, searched at 64 and 256 MiB per rank (TB/s over the whole
+// reduce-scatter + all-gather at 256 MiB, against policy 2 throughout): W=2: 7.07 vs 6.90
+// (64 MiB: 6.77 vs 6.33); W=3: 6.85 vs 6.47; W=4: 7.06 vs 6.58; W=8: nothing gained.
+// What the winners at W=4 share: the first reduce step, which touches everything for the
+// first time, loads and stores non-temporally; the last step of either phase stores
+// non-temporally and loads plainly what the step before it has just written.
+int ring_policy(int world, int step, bool gather) {
+  // Measurement knob: TDM_RING_POLICY="r0,r1,...,g0,g1,..." (digits 2, 5 or 7; reduce steps, then gather steps).
+  if (const char* env = std::getenv("TDM_RING_POLICY")) {
+    const size_t at = static_cast<size_t>(2 * ((gather ? world - 1 : 0) + step));
+    if (std::strlen(env) > at && (env[at] == '5' || env[at] == '7')) return env[at] - '0';
+    return TDM_NT_MASK;
+  }
+  const bool first = step == 0, last = step == world - 2;
+  switch (world) {
+    case 2: return gather ? 7 : TDM_NT_MASK;
+    case 3: return last ? 5 : TDM_NT_MASK;
+    case 4: return gather ? (last ? 5 : TDM_NT_MASK) : (first ? 7 : last ? 5 : TDM_NT_MASK);
+    default: return TDM_NT_MASK;
+  }
+}
+
 void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hipStream_t stream) {
   const int n = lr.world;
   for (int s = 0; s < n - 1; ++s) {
@@ -883,7 +928,7 @@ void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hi
       if (lr.len[c] == 0) continue;
       pairs[np++] = tdm_pair{lr.base[r] + lr.lo[c] * lr.es, lr.base[wrap(r - 1, n)] + lr.lo[c] * lr.es, lr.len[c]};
     }
-    if (np) reduce_step(pairs, np, lr.dtype, average ? n : 1, true, s == 0, s == 0 && keep_sent, stream);
+    if (np) reduce_step(pairs, np, lr.dtype, average ? n : 1, true, s == 0, s == 0 && keep_sent, stream, ring_policy(n, s, false));
   }
 }
 
@@ -898,7 +943,7 @@ void local_all_gather(const LocalRanks& lr, hipStream_t stream) {
       if (lr.len[c] == 0) continue;
       pairs[np++] = tdm_pair{lr.base[r] + lr.lo[c] * lr.es, lr.base[wrap(r - 1, n)] + lr.lo[c] * lr.es, lr.len[c]};
     }
-    if (np) copy_step(pairs, np, lr.dtype, 0, stream);
+    if (np) copy_step(pairs, np, lr.dtype, 0, stream, ring_policy(n, s, true));
   }
 }
 
