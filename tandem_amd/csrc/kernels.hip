@@ -17,6 +17,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "../../include/tandem_hip.h"
@@ -675,9 +676,9 @@ int div_kind(int world, bool any_scale) {
   return (world & (world - 1)) == 0 ? 1 : 2;
 }
 
-// The three cache policies K1 is built with (bit 0: loads of the stream that is read,
+// The four cache policies K1 is built with (bit 0: loads of the stream that is read,
 // modified and written back; bit 1: loads of the read-once stream; bit 2: stores are
-// non-temporal): 2 for a launch on its own, 7 and 5 for the first and last steps of a ring.
+// non-temporal): 2 for a launch on its own; 7, 5 and 0 for particular steps of a ring.
 template <typename T, int kMask>
 void launch_reduce_m(const PairTable& tab, int64_t tiles, int world, bool any_scale, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(world);
@@ -691,9 +692,21 @@ void launch_reduce_m(const PairTable& tab, int64_t tiles, int world, bool any_sc
 
 template <typename T>
 void launch_reduce(const PairTable& tab, int64_t tiles, int world, bool any_scale, int policy, hipStream_t stream) {
+#ifdef TDM_ALL_POLICIES  // search builds: every policy, fp32 only
+  if constexpr (std::is_same<T, float>::value) {
+    switch (policy) {
+      case 1: launch_reduce_m<T, 1>(tab, tiles, world, any_scale, stream); return;
+      case 3: launch_reduce_m<T, 3>(tab, tiles, world, any_scale, stream); return;
+      case 4: launch_reduce_m<T, 4>(tab, tiles, world, any_scale, stream); return;
+      case 6: launch_reduce_m<T, 6>(tab, tiles, world, any_scale, stream); return;
+      default: break;
+    }
+  }
+#endif
   switch (policy) {
     case 7: launch_reduce_m<T, 7>(tab, tiles, world, any_scale, stream); break;
     case 5: launch_reduce_m<T, 5>(tab, tiles, world, any_scale, stream); break;
+    case 0: launch_reduce_m<T, 0>(tab, tiles, world, any_scale, stream); break;
     default: launch_reduce_m<T, TDM_NT_MASK>(tab, tiles, world, any_scale, stream); break;
   }
 }
@@ -711,9 +724,19 @@ void launch_copy_m(const PairTable& tab, int64_t tiles, int world, hipStream_t s
 
 template <typename T>
 void launch_copy(const PairTable& tab, int64_t tiles, int world, int policy, hipStream_t stream) {
+#ifdef TDM_ALL_POLICIES
+  if constexpr (std::is_same<T, float>::value) {
+    switch (policy) {
+      case 4: launch_copy_m<T, 4>(tab, tiles, world, stream); return;
+      case 6: launch_copy_m<T, 6>(tab, tiles, world, stream); return;
+      default: break;
+    }
+  }
+#endif
   switch (policy) {
     case 7: launch_copy_m<T, 7>(tab, tiles, world, stream); break;
-    case 5: launch_copy_m<T, 5>(tab, tiles, world, stream); break;
+    case 5: launch_copy_m<T, 5>(tab, tiles, world, stream); break;  // (a copy has no read-modify-write stream: 5 is 4)
+    case 0: launch_copy_m<T, 0>(tab, tiles, world, stream); break;
     default: launch_copy_m<T, TDM_NT_MASK>(tab, tiles, world, stream); break;
   }
 }
@@ -895,27 +918,42 @@ int wrap(int a, int n) { return ((a % n) + n) % n; }
 
 // Step s: rank r adds chunk (r-s-2) of rank r-1 into its own (tandem/comm.py:301-305).
 // Every receiving chunk is still undivided; the sender's only on the first step.
-// Cache policy of each step of a ring on one GPU: the best of all combinations of 2, 5
-// and 7 over the steps, searched at 64 and 256 MiB per rank (TB/s over the whole
-// reduce-scatter + all-gather at 256 MiB, against policy 2 throughout): W=2: 7.07 vs 6.90
-// (64 MiB: 6.77 vs 6.33); W=3: 6.85 vs 6.47; W=4: 7.06 vs 6.58; W=8: nothing gained.
-// What the winners at W=4 share: the first reduce step, which touches everything for the
-// first time, loads and stores non-temporally; the last step of either phase stores
-// non-temporally and loads plainly what the step before it has just written.
-int ring_policy(int world, int step, bool gather) {
-  // Measurement knob: TDM_RING_POLICY="r0,r1,...,g0,g1,..." (digits 2, 5 or 7; reduce steps, then gather steps).
+// Cache policy of each step of a ring on one GPU, from searches over the policies of
+// every step at 8 MiB - 1 GiB per rank (TB/s over the whole reduce-scatter + all-gather
+// at 256 MiB per rank, against policy 2 throughout): W=2: 7.07 vs 6.90 (64 MiB: 6.77 vs
+// 6.33); W=3: 6.85 vs 6.47; W=4: 7.04 vs 6.59; W=8: nothing gained.
+// What the winners at W=4 share. Footprint beyond the 256 MB Infinity Cache: the first
+// reduce step, which touches everything for the first time, loads and stores non-
+// temporally; the last step of either phase stores non-temporally and loads plainly
+// what the step before it has just written. Footprint that fits (up to 80 MiB per rank;
+// 64 MiB: 6.76 vs 6.57, 16 MiB: 5.99 vs 5.75): after the first touch everything stays
+// cached, only the very last stores are non-temporal.
+int ring_policy(int world, int step, bool gather, int64_t footprint_bytes) {
+  // Measurement knob: TDM_RING_POLICY="r0,r1,...,g0,g1,..." (one digit per step; reduce steps, then gather steps).
   if (const char* env = std::getenv("TDM_RING_POLICY")) {
     const size_t at = static_cast<size_t>(2 * ((gather ? world - 1 : 0) + step));
-    if (std::strlen(env) > at && (env[at] == '5' || env[at] == '7')) return env[at] - '0';
+#ifdef TDM_ALL_POLICIES
+    if (std::strlen(env) > at && env[at] >= '0' && env[at] <= '7') return env[at] - '0';
+#else
+    if (std::strlen(env) > at && (env[at] == '0' || env[at] == '5' || env[at] == '7')) return env[at] - '0';
+#endif
     return TDM_NT_MASK;
   }
   const bool first = step == 0, last = step == world - 2;
   switch (world) {
     case 2: return gather ? 7 : TDM_NT_MASK;
     case 3: return last ? 5 : TDM_NT_MASK;
-    case 4: return gather ? (last ? 5 : TDM_NT_MASK) : (first ? 7 : last ? 5 : TDM_NT_MASK);
+    case 4:
+      if (footprint_bytes <= (int64_t(352) << 20)) return gather ? (last ? 5 : 0) : (first ? 7 : last ? TDM_NT_MASK : 0);
+      return gather ? (last ? 5 : TDM_NT_MASK) : (first ? 7 : last ? 5 : TDM_NT_MASK);
     default: return TDM_NT_MASK;
   }
+}
+
+int64_t footprint(const LocalRanks& lr) {  // bytes of all ranks' tensors together
+  int64_t elems = 0;
+  for (int64_t l : lr.len) elems += l;
+  return elems * lr.es * lr.world;
 }
 
 void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hipStream_t stream) {
@@ -928,7 +966,7 @@ void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hi
       if (lr.len[c] == 0) continue;
       pairs[np++] = tdm_pair{lr.base[r] + lr.lo[c] * lr.es, lr.base[wrap(r - 1, n)] + lr.lo[c] * lr.es, lr.len[c]};
     }
-    if (np) reduce_step(pairs, np, lr.dtype, average ? n : 1, true, s == 0, s == 0 && keep_sent, stream, ring_policy(n, s, false));
+    if (np) reduce_step(pairs, np, lr.dtype, average ? n : 1, true, s == 0, s == 0 && keep_sent, stream, ring_policy(n, s, false, footprint(lr)));
   }
 }
 
@@ -943,7 +981,7 @@ void local_all_gather(const LocalRanks& lr, hipStream_t stream) {
       if (lr.len[c] == 0) continue;
       pairs[np++] = tdm_pair{lr.base[r] + lr.lo[c] * lr.es, lr.base[wrap(r - 1, n)] + lr.lo[c] * lr.es, lr.len[c]};
     }
-    if (np) copy_step(pairs, np, lr.dtype, 0, stream, ring_policy(n, s, true));
+    if (np) copy_step(pairs, np, lr.dtype, 0, stream, ring_policy(n, s, true, footprint(lr)));
   }
 }
 
