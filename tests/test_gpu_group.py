@@ -88,17 +88,22 @@ def test_a_group_of_one():
 
 
 def choose(monkeypatch, algo):
-    """The engine's two ways through all_reduce / all_gather: staged through memory the
-    peers map (default; "small": 4 KiB halves, so n = 10,007 takes several passes and
-    both halves are reused), or the reference's ring through the slots."""
+    """The engine's ways through all_reduce / all_gather: staged through memory the
+    peers map (default: tensors up to 1 MiB with one handshake; "two": the two-handshake
+    passes also for small tensors; "small": 4 KiB halves, so n = 10,007 takes several
+    passes and both halves are reused), or the reference's ring through the slots."""
     monkeypatch.setenv("TANDEM_HIP_ALGO", "ring" if algo == "ring" else "staged")
     if algo == "small":
         monkeypatch.setenv("TANDEM_HIP_STAGING_BYTES", "4096")
     else:
         monkeypatch.delenv("TANDEM_HIP_STAGING_BYTES", raising=False)
+    if algo == "two":  # no one-handshake form for small tensors: the two-handshake passes at every size
+        monkeypatch.setenv("TANDEM_HIP_SMALL_BYTES", "0")
+    else:
+        monkeypatch.delenv("TANDEM_HIP_SMALL_BYTES", raising=False)
 
 
-@pytest.mark.parametrize("algo", ["staged", "small", "ring"])
+@pytest.mark.parametrize("algo", ["staged", "two", "small", "ring"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.int64, torch.float64])
 @pytest.mark.parametrize("world", [2, 3, 4])
 def test_collectives_bit_exact(dtype, world, algo, monkeypatch):
@@ -110,7 +115,7 @@ def test_collectives_bit_exact(dtype, world, algo, monkeypatch):
 
     if world == 4 and dtype in (torch.float16, torch.float64):
         pytest.skip("covered at world 2 and 3")
-    if algo != "small" and dtype in (torch.float16, torch.float64, torch.int64) and world == 3:
+    if algo not in ("small", "staged") and dtype in (torch.float16, torch.float64, torch.int64) and world == 3:
         pytest.skip("these dtypes at world 3: the several-pass case only")
     choose(monkeypatch, algo)
     n, kind = 10_007, KINDS[dtype]
@@ -197,7 +202,7 @@ def replay_fixture(g, inputs, cases):
     return out
 
 
-@pytest.mark.parametrize("algo", ["staged", "small", "ring"])
+@pytest.mark.parametrize("algo", ["staged", "two", "small", "ring"])
 @pytest.mark.parametrize("world", [2, 3, 4])
 def test_reference_fixtures(world, algo, monkeypatch):
     """The same inputs and slot size as the reference engine's run."""
