@@ -89,7 +89,7 @@ def test_a_group_of_one():
 
 def choose(monkeypatch, algo):
     """The engine's ways through all_reduce / all_gather: staged through memory the
-    peers map (default: tensors up to 1 MiB with one handshake; "two": the two-handshake
+    peers map (default: tensors up to 32 MiB with one handshake; "two": the two-handshake
     passes also for small tensors; "small": 4 KiB halves, so n = 10,007 takes several
     passes and both halves are reused), or the reference's ring through the slots."""
     monkeypatch.setenv("TANDEM_HIP_ALGO", "ring" if algo == "ring" else "staged")
