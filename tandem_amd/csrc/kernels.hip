@@ -381,9 +381,10 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
 #define TDM_K2_UNROLL_W2 4
 #endif
 #ifndef TDM_K2_UNROLL
-#define TDM_K2_UNROLL 2
+#define TDM_K2_UNROLL 4
 #endif
-  constexpr int kU = kWorld <= 2 ? TDM_K2_UNROLL_W2 : TDM_K2_UNROLL;  // vectors per lane per tile step, per rank
+  // vectors per lane per tile step, per rank (worlds 3-4: 4 beats 2 by 2-3 %; beyond that the registers run out)
+  constexpr int kU = kWorld <= 2 ? TDM_K2_UNROLL_W2 : kWorld <= 4 ? TDM_K2_UNROLL : 2;
   constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
   const int64_t n = sg.count;
   const int c = sg.chunk;
