@@ -66,6 +66,12 @@ int mod(int a, int n) { return ((a % n) + n) % n; }
 
 constexpr int kBytesDtype = 6;  // TDM_U8 in spirit: copies only
 
+// Messages: a piece's length in bytes, or (top bit set) a barrier with a tag in the low bits.
+constexpr uint64_t kNoPiece = uint64_t(1) << 63;
+constexpr uint64_t fence_tag(int kind, int dtype, int64_t numel) {
+  return (static_cast<uint64_t>(kind) << 56) | (static_cast<uint64_t>(dtype) << 48) | (static_cast<uint64_t>(numel) & ((uint64_t(1) << 48) - 1));
+}
+
 int elem_bytes(int dtype) {
   switch (dtype) {
     case TDM_F32: case TDM_I32: return 4;
@@ -339,7 +345,7 @@ class Engine {
   void signal(int dst, uint64_t length);
   uint64_t await(int src);
   void release(int src);
-  void barrier_now(bool after_gpu = false);
+  void barrier_now(bool after_gpu = false, uint64_t tag = 0);
   const char* peer_arena(int peer, size_t need_bytes);
 
   std::string region_name(int rank) const { return "/tandem-" + job_ + "-" + std::to_string(rank) + "-hip"; }
@@ -811,7 +817,11 @@ void Engine::drain_completions() {
 
 // after_gpu: the empty messages are published only once the GPU has finished what
 // the engine's stream holds so far (a fence), not merely when it has been enqueued.
-void Engine::barrier_now(bool after_gpu) {
+// tag: what the ranks must agree on at this point (0 for a plain barrier; the staged and
+// direct collectives send the kind of operation and the tensor's size). A rank that is
+// somewhere else in its program, or has a tensor of another size, is found out here
+// instead of reading stale bytes: the slot ring finds such a rank by its piece lengths.
+void Engine::barrier_now(bool after_gpu, uint64_t tag) {
   // Messages are published in order: everything queued for the completion thread
   // goes first. After that this thread publishes by itself; it has to wait for the
   // peers anyway, and handing over to the completion thread would cost two wake-ups.
@@ -825,7 +835,7 @@ void Engine::barrier_now(bool after_gpu) {
   }
   // An empty message to every peer, then one from each. Rings are first in,
   // first out, so this also orders the barrier after every piece queued before.
-  constexpr uint64_t kEmpty = ~uint64_t(0);
+  const uint64_t kEmpty = kNoPiece | (tag & ~kNoPiece);
   for (int p = 0; p < size_; ++p) {
     if (p == rank_) continue;
     Ring& r = mine_.entry(p)->ring;
@@ -837,7 +847,12 @@ void Engine::barrier_now(bool after_gpu) {
   }
   for (int p = 0; p < size_; ++p) {
     if (p == rank_) continue;
-    if (await(p) != kEmpty) throw std::runtime_error("barrier out of step: expected an empty message, got a piece");
+    const uint64_t got = await(p);
+    if (!(got & kNoPiece)) throw std::runtime_error("barrier out of step: expected an empty message, got a piece");
+    if (got != kEmpty) {
+      throw std::runtime_error("collectives out of step: rank " + std::to_string(p) + " is in another collective, or in the same "
+                               "one with a tensor of another size");
+    }
     release(p);
   }
 }
@@ -879,7 +894,7 @@ void Engine::take(int src, char* into, int64_t numel, int dtype, bool reduce, in
   const size_t nbytes = static_cast<size_t>(numel) * elem_bytes(dtype);
   const uint64_t length = await(src);
   if (length != nbytes) {
-    throw std::runtime_error(length == ~uint64_t(0) ? "collectives out of step: expected a piece, got a barrier"
+    throw std::runtime_error((length & kNoPiece) ? "collectives out of step: expected a piece, got a barrier"
                                                     : "a piece arrived with the wrong length");
   }
   const int j = static_cast<int>(got_[src] % slots_);
@@ -1014,7 +1029,7 @@ void Engine::staged_all_reduce_small(const Buf& t, bool average) {
   const int half = static_cast<int>((staged_ops_ - 1) % 2);
   tdm_pair whole{mine, t.ptr, t.numel};
   copy_pairs(&whole, 1, t.dtype);
-  barrier_now(true);  // every rank's tensor is in its staging
+  barrier_now(true, fence_tag(1, t.dtype, t.numel));  // every rank's tensor is in its staging
   tdm_fold_seg segs[TDM_MAX_WORLD];
   std::memset(segs, 0, sizeof segs);
   int ns = 0;
@@ -1053,7 +1068,7 @@ void Engine::staged_all_reduce(const Buf& t, bool average) {
       pairs[np++] = tdm_pair{mine + c * sub_bytes, cs[c].ptr + at * es, part(c)};
     }
     copy_pairs(pairs, np, t.dtype);
-    barrier_now(true);  // every rank's parts are in its staging
+    barrier_now(true, fence_tag(2, t.dtype, t.numel));  // every rank's parts are in its staging
     if (part(r) > 0) {
       tdm_fold_seg seg;
       std::memset(&seg, 0, sizeof seg);
@@ -1100,7 +1115,7 @@ void Engine::staged_reduce_scatter_owner(const Buf& t, const std::vector<Chunk>&
       }
     }
     copy_pairs(pairs, np, t.dtype);
-    barrier_now(true);  // every rank's parts are in its staging
+    barrier_now(true, fence_tag(3, t.dtype, t.numel));  // every rank's parts are in its staging
     if (hi(r) > lo(r)) {
       tdm_fold_seg seg;
       std::memset(&seg, 0, sizeof seg);
@@ -1131,7 +1146,7 @@ void Engine::staged_all_gather(const Buf& t, const std::vector<Chunk>& cs, const
       if (own != cs[r].ptr) pairs[np++] = tdm_pair{cs[r].ptr + at * es, own + at * es, part(r)};
     }
     copy_pairs(pairs, np, t.dtype);
-    barrier_now(true);  // every rank's part is in its staging
+    barrier_now(true, fence_tag(4, t.dtype, t.numel));  // every rank's part is in its staging
     np = 0;
     for (int c = 0; c < n; ++c) {
       if (c == r || part(c) == 0) continue;
@@ -1469,7 +1484,7 @@ std::shared_ptr<Work> Engine::direct(int kind, Buf t, std::vector<int64_t> sizes
     const char* base[TDM_MAX_PAIRS > TDM_MAX_WORLD ? TDM_MAX_PAIRS : TDM_MAX_WORLD];
     if (size_ > static_cast<int>(sizeof base / sizeof base[0])) throw Invalid("direct collective: too many ranks");
     if (t.numel > 0) direct_bases(t, peer_offsets, base);  // an empty tensor still takes part in the fences
-    barrier_now(true);  // every rank's input is complete
+    barrier_now(true, fence_tag(5 + kind, t.dtype, t.numel));  // every rank's input is complete
     if (kind != 2) {
       direct_fold(t, cs, base, average);
       barrier_now(true);  // every chunk is folded (or, for reduce_scatter: nobody reads our tensor any more)

@@ -500,6 +500,30 @@ def test_a_missing_peer_times_out_on_the_host():
         launch(out_of_step, 2, gpus=[0, 0], timeout=3.0)
 
 
+def disagree(g, what):
+    """Ranks that call different collectives, or the same one on tensors of different
+    sizes: found out at the first handshake, on every rank, not by reading stale bytes."""
+    from tandem_amd import CommError
+
+    x = torch.ones(1000 + (g.rank if what == "size" else 0), device=g.device)
+    try:
+        if what == "kind" and g.rank == 1:
+            g.all_gather(x)
+        else:
+            g.all_reduce(x)
+    except CommError as e:
+        g.abandon()
+        return "out of step" in str(e.__cause__)
+    return False
+
+
+@pytest.mark.parametrize("what", ["size", "kind"])
+def test_ranks_that_disagree_are_found_out(what):
+    from tandem_amd import launch
+
+    assert launch(disagree, 2, what, gpus=[0, 0], timeout=TIMEOUT) == [True, True]
+
+
 def test_unknown_backend_and_cpu_device_are_refused():
     from tandem_amd import CommError, Group, launch
 
