@@ -1314,6 +1314,7 @@ std::shared_ptr<Work> Engine::sendrecv(Buf send, int dst, Buf recv, int src, hip
 // fence(): before (every peer has finished reading) and after (the new contents are
 // complete) -- ZeRO-3 changes its shards once per step, and gathers them 27 times.
 void* Engine::share(size_t bytes) {
+  std::lock_guard<std::mutex> lock(arena_mu_);
   if (arena_) throw std::runtime_error("share: this engine already has an arena");
   if (bytes == 0 || bytes >= (size_t(2) << 30)) throw Invalid("share: the arena must be between 1 byte and 2 GiB (one IPC allocation)");
   check_hip(hipSetDevice(device_), "hipSetDevice");
@@ -1426,8 +1427,14 @@ std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, st
 void Engine::direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets, const char** base) {
   const int es = elem_bytes(t.dtype);
   const size_t bytes = static_cast<size_t>(t.numel) * es;
-  const char* a = static_cast<const char*>(arena_);
-  if (!arena_ || t.ptr < a || t.ptr + bytes > a + arena_bytes_) {
+  const char* a;
+  size_t arena_bytes;
+  {
+    std::lock_guard<std::mutex> lock(arena_mu_);
+    a = static_cast<const char*>(arena_);
+    arena_bytes = arena_bytes_;
+  }
+  if (!a || t.ptr < a || t.ptr + bytes > a + arena_bytes) {
     throw Invalid("direct collective: the tensor does not lie in this rank's shared arena");
   }
   for (int q = 0; q < size_; ++q) {

@@ -35,6 +35,19 @@ namespace {
 #endif
 constexpr int kThreads = TDM_THREADS;
 constexpr int kUnroll = TDM_UNROLL;             // 16-byte vectors per lane per tile and stream
+#ifndef TDM_K1_UNROLL
+#define TDM_K1_UNROLL 2
+#endif
+// K1 and the copy kernel cut their pairs into tiles of their own, 8 KiB per stream: against 16 KiB the
+// ring (reduce-scatter + all-gather, world 4) runs 3 % faster at 64 MiB per rank (6.95 vs 6.74 TB/s), 2 %
+// at 16 MiB and equally fast at 256 MiB; different tile sizes for the two kernels are worse than either.
+constexpr int kK1Unroll = TDM_K1_UNROLL;
+constexpr int kK1TileVecs = kThreads * kK1Unroll;
+#ifndef TDM_COPY_UNROLL
+#define TDM_COPY_UNROLL TDM_K1_UNROLL
+#endif
+constexpr int kCopyUnroll = TDM_COPY_UNROLL;
+constexpr int kCopyTileVecs = kThreads * kCopyUnroll;
 constexpr int kTileVecs = kThreads * kUnroll;   // 1024 vectors = 16 KiB of every stream
 // Measured on MI355X: one 16 KiB tile per workgroup beats a persistent grid-stride
 // loop by 5-8% (the hardware dispatcher balances 8 XCDs better than a fixed stride),
@@ -216,7 +229,7 @@ __device__ __forceinline__ void reduce_elem(T& d, T& s, bool scale_dst, bool sca
 template <typename T, int kDiv, int kMask>
 __global__ __launch_bounds__(kThreads) void k1_reduce_kernel(PairTable tab, Divisor<T> dv) {
   constexpr int L = lanes<T>();
-  constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
+  constexpr int64_t kTileElems = static_cast<int64_t>(kK1TileVecs) * L;
   const bool scale_dst = tab.flags & 1, scale_src = tab.flags & 2, writeback = tab.flags & 4;
   const int64_t total = tab.tile_end[tab.npairs - 1];
   for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
@@ -231,15 +244,15 @@ __global__ __launch_bounds__(kThreads) void k1_reduce_kernel(PairTable tab, Divi
       const int64_t nv = (n - head) / L;
       char* dvp = reinterpret_cast<char*>(dst + head);
       char* svp = reinterpret_cast<char*>(src + head);
-      const int64_t v0 = t * kTileVecs + threadIdx.x;
-      if ((t + 1) * kTileVecs <= nv) {  // a full tile: all loads first, then the arithmetic, then the stores
-        vec16 a[kUnroll], b[kUnroll];
+      const int64_t v0 = t * kK1TileVecs + threadIdx.x;
+      if ((t + 1) * kK1TileVecs <= nv) {  // a full tile: all loads first, then the arithmetic, then the stores
+        vec16 a[kK1Unroll], b[kK1Unroll];
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) a[k] = load_rmw<kMask>(dvp + (v0 + k * kThreads) * 16);
+        for (int k = 0; k < kK1Unroll; ++k) a[k] = load_rmw<kMask>(dvp + (v0 + k * kThreads) * 16);
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kThreads) * 16);
+        for (int k = 0; k < kK1Unroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kThreads) * 16);
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
+        for (int k = 0; k < kK1Unroll; ++k) {
           Lanes<T> x = unpack<T>(a[k]), y = unpack<T>(b[k]);
 #pragma unroll
           for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
@@ -248,7 +261,7 @@ __global__ __launch_bounds__(kThreads) void k1_reduce_kernel(PairTable tab, Divi
         }
       } else {
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
+        for (int k = 0; k < kK1Unroll; ++k) {
           const int64_t v = v0 + k * kThreads;
           if (v < nv) {
             Lanes<T> x = unpack<T>(load_rmw<kMask>(dvp + v * 16)), y = unpack<T>(load_stream<kMask>(svp + v * 16));
@@ -274,7 +287,7 @@ __global__ __launch_bounds__(kThreads) void k1_reduce_kernel(PairTable tab, Divi
     } else {  // the two pointers disagree within 16 bytes: element-wise, still coalesced
       const int64_t e0 = t * kTileElems + threadIdx.x;
 #pragma unroll 4
-      for (int k = 0; k < kUnroll * L; ++k) {
+      for (int k = 0; k < kK1Unroll * L; ++k) {
         const int64_t i = e0 + static_cast<int64_t>(k) * kThreads;
         if (i < n) {
           T x = dst[i], y = src[i];
@@ -299,7 +312,7 @@ __device__ __forceinline__ T copy_elem(T s, const Divisor<T>& dv) {
 template <typename T, int kDiv, int kMask>
 __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Divisor<T> dv) {
   constexpr int L = lanes<T>();
-  constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
+  constexpr int64_t kTileElems = static_cast<int64_t>(kCopyTileVecs) * L;
   const int64_t total = tab.tile_end[tab.npairs - 1];
   for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
     int p = 0;
@@ -313,13 +326,13 @@ __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Diviso
       const int64_t nv = (n - head) / L;
       char* dvp = reinterpret_cast<char*>(dst + head);
       const char* svp = reinterpret_cast<const char*>(src + head);
-      const int64_t v0 = t * kTileVecs + threadIdx.x;
-      if ((t + 1) * kTileVecs <= nv) {
-        vec16 b[kUnroll];
+      const int64_t v0 = t * kCopyTileVecs + threadIdx.x;
+      if ((t + 1) * kCopyTileVecs <= nv) {
+        vec16 b[kCopyUnroll];
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kThreads) * 16);
+        for (int k = 0; k < kCopyUnroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kThreads) * 16);
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
+        for (int k = 0; k < kCopyUnroll; ++k) {
           if constexpr (kDiv != 0) {
             Lanes<T> y = unpack<T>(b[k]);
 #pragma unroll
@@ -330,7 +343,7 @@ __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Diviso
         }
       } else {
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
+        for (int k = 0; k < kCopyUnroll; ++k) {
           const int64_t v = v0 + k * kThreads;
           if (v < nv) {
             Lanes<T> y = unpack<T>(load_stream<kMask>(svp + v * 16));
@@ -350,7 +363,7 @@ __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Diviso
     } else {
       const int64_t e0 = t * kTileElems + threadIdx.x;
 #pragma unroll 4
-      for (int k = 0; k < kUnroll * L; ++k) {
+      for (int k = 0; k < kCopyUnroll * L; ++k) {
         const int64_t i = e0 + static_cast<int64_t>(k) * kThreads;
         if (i < n) dst[i] = copy_elem<T, kDiv>(src[i], dv);
       }
@@ -630,11 +643,11 @@ int grid_for(int64_t tiles) {
 }
 
 // Validates the pairs and lays out the by-value table. Returns the tile count (0: nothing to do).
-int64_t build_pairs(const tdm_pair* pairs, int npairs, int esize, bool ranges_must_not_overlap, PairTable* tab) {
+int64_t build_pairs(const tdm_pair* pairs, int npairs, int esize, bool ranges_must_not_overlap, int tile_vecs, PairTable* tab) {
   if (npairs < 0 || npairs > TDM_MAX_PAIRS) throw Invalid("npairs must be in [0, " + std::to_string(TDM_MAX_PAIRS) + "]");
   if (npairs > 0 && pairs == nullptr) throw Invalid("pairs is NULL");
   std::memset(tab, 0, sizeof *tab);
-  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / esize);
+  const int64_t tile_elems = static_cast<int64_t>(tile_vecs) * (16 / esize);
   int64_t tiles = 0;
   int k = 0;
   for (int i = 0; i < npairs; ++i) {
@@ -815,7 +828,7 @@ void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool s
   const bool any_scale = (scale_dst || scale_src) && world > 1;
   if (any_scale && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
   PairTable tab;
-  const int64_t tiles = build_pairs(pairs, npairs, es, true, &tab);
+  const int64_t tiles = build_pairs(pairs, npairs, es, true, kK1TileVecs, &tab);
   if (tiles == 0) return;
   tab.flags = (any_scale && scale_dst ? 1 : 0) | (any_scale && scale_src ? 2 : 0) | (any_scale && scale_src && writeback_src ? 4 : 0);
   switch (dtype) {
@@ -849,7 +862,7 @@ void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStrea
       if (d < s + bytes && s < d + bytes) throw Invalid("copy: destination and source overlap");
     }
   }
-  const int64_t tiles = build_pairs(kept.data(), static_cast<int>(kept.size()), es, false, &tab);
+  const int64_t tiles = build_pairs(kept.data(), static_cast<int>(kept.size()), es, false, kCopyTileVecs, &tab);
   if (tiles == 0) return;
   switch (dtype) {
     case TDM_F32: launch_copy<float>(tab, tiles, world, policy, stream); break;
