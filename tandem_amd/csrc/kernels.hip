@@ -941,7 +941,8 @@ int wrap(int a, int n) { return ((a % n) + n) % n; }
 // temporally; the last step of either phase stores non-temporally and loads plainly
 // what the step before it has just written. Footprint that fits (up to 80 MiB per rank;
 // 64 MiB: 6.76 vs 6.57, 16 MiB: 5.99 vs 5.75): after the first touch everything stays
-// cached, only the very last stores are non-temporal.
+// cached, only the very last stores are non-temporal. At W=2 and W=3 a footprint that
+// fits with room to spare does best with everything cached.
 int ring_policy(int world, int step, bool gather, int64_t footprint_bytes) {
   // Measurement knob: TDM_RING_POLICY="r0,r1,...,g0,g1,..." (one digit per step; reduce steps, then gather steps).
   if (const char* env = std::getenv("TDM_RING_POLICY")) {
@@ -955,8 +956,12 @@ int ring_policy(int world, int step, bool gather, int64_t footprint_bytes) {
   }
   const bool first = step == 0, last = step == world - 2;
   switch (world) {
-    case 2: return gather ? 7 : TDM_NT_MASK;
-    case 3: return last ? 5 : TDM_NT_MASK;
+    case 2:
+      if (footprint_bytes <= (int64_t(80) << 20)) return 0;  // 32 MiB per rank: 6.94 vs 6.56
+      return gather ? 7 : TDM_NT_MASK;
+    case 3:
+      if (footprint_bytes <= (int64_t(224) << 20)) return 0;  // 64 MiB per rank: 6.54 vs 6.11; 16 MiB: 5.20 vs 4.03
+      return last ? 5 : TDM_NT_MASK;
     case 4:
       if (footprint_bytes <= (int64_t(352) << 20)) return gather ? (last ? 5 : 0) : (first ? 7 : last ? TDM_NT_MASK : 0);
       return gather ? (last ? 5 : TDM_NT_MASK) : (first ? 7 : last ? 5 : TDM_NT_MASK);
