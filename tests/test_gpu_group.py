@@ -65,6 +65,10 @@ def collectives(g, dtype, n):
         got = torch.empty(n, dtype=dtype, device=dev)
         g.sendrecv(x, 1 - r, got, 1 - r)
         out["sendrecv"] = got.cpu()
+    codes = torch.zeros(n, dtype=torch.uint8, device=dev)  # a dtype the kernels do not know: gathered as bytes
+    codes[lo:lo + sizes[r]] = r + 1
+    g.all_gather(codes, sizes)
+    out["bytes_ag_ok"] = bool(torch.equal(codes.cpu(), torch.cat([torch.full((sizes[q],), q + 1, dtype=torch.uint8) for q in range(w)])))
     flags = torch.arange(n, device=dev) % 2 == 0  # bool: copied as bytes
     if r != 0:
         flags = torch.zeros_like(flags)
@@ -84,7 +88,7 @@ def test_a_group_of_one():
     x = values(0, n, torch.float32)
     for key in ("ar_sum", "ar_avg", "rs_sum", "rs_avg", "rso_sum", "rso_avg", "ag", "bcast"):
         assert torch.equal(out[key], x), key
-    assert out["bool_bcast_ok"]
+    assert out["bool_bcast_ok"] and out["bytes_ag_ok"]
 
 
 def choose(monkeypatch, algo):
@@ -142,7 +146,7 @@ def test_collectives_bit_exact(dtype, world, algo, monkeypatch):
         assert np.array_equal(bits(to_np(out["bcast"])), bits(xs[world - 1])), (r, "bcast")
         if world == 2:
             assert np.array_equal(bits(to_np(out["sendrecv"])), bits(xs[1 - r]))
-        assert out["bool_bcast_ok"]
+        assert out["bool_bcast_ok"] and out["bytes_ag_ok"]
 
 
 def tiny_slots(g, sizes_list):
