@@ -504,6 +504,75 @@ def test_a_missing_peer_times_out_on_the_host():
         launch(out_of_step, 2, gpus=[0, 0], timeout=3.0)
 
 
+def mixed_sequence(g, seed, count):
+    """The same seeded sequence of collectives on every rank, sizes and kinds mixed, some
+    waited for at once and some later, in submission order."""
+    import random
+
+    rng = random.Random(seed)
+    w, r, dev = g.size, g.rank, g.device
+    results, pending = [], []
+    for k in range(count):
+        kind = rng.choice(["ar_sum", "ar_avg", "ag", "rs", "rso", "bcast", "barrier"])
+        n = rng.choice([0, 1, 7, 300, 1023, 4096, 10_007, 40_000])
+        cut = sorted(rng.randint(0, n) for _ in range(w - 1))
+        sizes = [b - a for a, b in zip([0] + cut, cut + [n])]
+        later = rng.random() < 0.5
+        x = (torch.randn(n, generator=torch.Generator().manual_seed(seed * 7919 + k * 31 + r)) * 0.5).to(dev)
+        if kind == "barrier":
+            g.barrier()
+            continue
+        if kind.startswith("ar"):
+            work = g.all_reduce(x, op=kind[3:], async_op=True)
+        elif kind == "ag":
+            work = g.all_gather(x, sizes, async_op=True)
+        elif kind == "bcast":
+            work = g.broadcast(x, root=k % w, async_op=True)
+        else:
+            work = g.reduce_scatter(x, sizes, op="avg", async_op=True, partial_sums=kind == "rs")
+        pending.append((k, kind, sizes, x, work))
+        if not later:
+            while pending:  # waits happen in submission order
+                k2, kind2, sizes2, x2, w2 = pending.pop(0)
+                w2.wait()
+                results.append((k2, kind2, sizes2, x2.cpu().numpy()))
+    for k2, kind2, sizes2, x2, w2 in pending:
+        w2.wait()
+        results.append((k2, kind2, sizes2, x2.cpu().numpy()))
+    torch.cuda.synchronize()
+    return results
+
+
+@pytest.mark.parametrize("algo", ["staged", "small"])
+@pytest.mark.parametrize("world", [2, 3])
+def test_a_long_mixed_sequence_stays_bit_exact(world, algo, monkeypatch):
+    """Forty collectives of mixed kinds and sizes in flight behind one another: the
+    staging halves, slots and handshakes are reused in every order the mix produces."""
+    from oracle import ring
+    from tandem_amd import launch
+
+    choose(monkeypatch, algo)
+    seed, count = 11 + world, 40
+    res = launch(mixed_sequence, world, seed, count, slot_bytes=4096, gpus=[0] * world, timeout=TIMEOUT)
+    for r, results in enumerate(res):
+        for k, kind, sizes, got in results:
+            n = sum(sizes)
+            xs = [(torch.randn(n, generator=torch.Generator().manual_seed(seed * 7919 + k * 31 + q)) * 0.5).numpy() for q in range(world)]
+            lo = sum(sizes[:r])
+            if kind.startswith("ar"):
+                want = ring.expected_all_reduce(xs, kind == "ar_avg")
+            elif kind == "ag":
+                want = ring.expected_all_gather(xs, sizes)
+            elif kind == "bcast":
+                want = xs[k % world]
+            elif kind == "rs":
+                want = ring.expected_reduce_scatter(xs, sizes, True)[r]
+            else:  # only the owner's chunk is specified
+                want = ring.expected_reduce_scatter(xs, sizes, True)[r][lo:lo + sizes[r]]
+                got = got[lo:lo + sizes[r]]
+            assert np.array_equal(bits(got), bits(want)), (world, algo, r, k, kind, sizes)
+
+
 def disagree(g, what):
     """Ranks that call different collectives, or the same one on tensors of different
     sizes: found out at the first handshake, on every rank, not by reading stale bytes."""
