@@ -529,6 +529,14 @@ def main():
             train4 = train_steps(5, 4, ("alone", "ddp", "zero2", "zero2+direct", "zero3"))
         except Exception as e:
             train4 = {"error": repr(e)[:300]}
+        os.environ["TANDEM_HIP_WAIT"] = "stream"  # wait() parks the training stream instead of blocking the host
+        try:
+            train["stream_ordered_wait"] = {k: v["step_ms"] for k, v in train_steps(5, 2, ("ddp", "ddp+direct", "zero2")).items()
+                                            if k != "workload"}
+        except Exception as e:
+            train["stream_ordered_wait"] = {"error": repr(e)[:300]}
+        finally:
+            del os.environ["TANDEM_HIP_WAIT"]
 
     import torch
 

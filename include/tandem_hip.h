@@ -293,7 +293,10 @@ int tdm_barrier(tdm_engine* e, tdm_work** out);
  * makes `caller` wait for it on the GPU; returns the collective's error, if any.
  * (With the default host ordering between ranks, a collective's last launch is
  * enqueued only when the GPU has finished the hand-over before it, so wait returns
- * about when that last kernel starts, not right after submission.)
+ * about when that last kernel starts, not right after submission. With TANDEM_HIP_WAIT=stream
+ * in the environment at tdm_engine_create, wait on a collective that has not run yet makes
+ * `caller` wait for a word the engine sets behind the collective's last kernel and returns at
+ * once; a failure of that collective is then returned by the next call on the engine.)
  * done: 1 once the GPU has finished it. times: when the progress thread started and
  * finished it, seconds on CLOCK_MONOTONIC (Python's time.perf_counter clock); for a
  * collective submitted while tdm_engine_set_timing was on, when the GPU started it

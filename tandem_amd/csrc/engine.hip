@@ -248,6 +248,48 @@ struct Anchor {
   }
 };
 
+// Words in pinned host memory that a GPU stream can wait on (hipStreamWaitValue32) and
+// that either the engine's stream (hipStreamWriteValue32) or the host sets: how
+// wait() can order the caller's stream behind a collective whose launches the progress
+// thread has not even made yet. Shared by the engine and its Works, freed by the last.
+struct FlagPool {
+  static constexpr int kFlags = 1024;
+  uint32_t* base = nullptr;
+  std::mutex mu;
+  std::vector<int> free_list;
+  std::vector<uint32_t> generation;  // a word only ever grows: a stream still parked on an earlier
+                                     // generation of it is let go by every later one as well
+
+  static std::shared_ptr<FlagPool> make() {
+    auto p = std::make_shared<FlagPool>();
+    check_hip(hipHostMalloc(reinterpret_cast<void**>(&p->base), kFlags * sizeof(uint32_t), hipHostMallocDefault), "hipHostMalloc (flags)");
+    std::memset(p->base, 0, kFlags * sizeof(uint32_t));
+    p->generation.assign(kFlags, 0);
+    for (int i = kFlags - 1; i >= 0; --i) p->free_list.push_back(i);
+    return p;
+  }
+  ~FlagPool() {
+    if (base) (void)hipHostFree(base);
+  }
+  // A word and the value its owner will wait for; -1: none left (the Work then waits on the host as usual).
+  int acquire(uint32_t* value) {
+    std::lock_guard<std::mutex> lock(mu);
+    if (free_list.empty()) return -1;
+    const int i = free_list.back();
+    free_list.pop_back();
+    *value = ++generation[i];
+    return i;
+  }
+  void release(int i) {
+    std::lock_guard<std::mutex> lock(mu);
+    free_list.push_back(i);
+  }
+  void set(int i, uint32_t value) {
+    reinterpret_cast<volatile uint32_t*>(base)[i] = value;
+    std::atomic_thread_fence(std::memory_order_seq_cst);
+  }
+};
+
 struct Work {
   std::mutex mu;
   std::condition_variable cv;
@@ -267,10 +309,18 @@ struct Work {
   // time stamps, placed on the host clock through the engine's anchor.
   hipEvent_t start_event = nullptr;
   std::shared_ptr<Anchor> anchor;
+  // Stream-ordered waiting (TANDEM_HIP_WAIT=stream): the word the caller's stream waits for.
+  std::shared_ptr<FlagPool> flags;
+  int flag = -1;
+  uint32_t flag_value = 0;  // the word reaches this value when the collective is over
 
   ~Work() {
     if (done_event) (void)hipEventDestroy(done_event);
     if (start_event) (void)hipEventDestroy(start_event);
+    if (flags && flag >= 0) {
+      if (!finished) flags->set(flag, flag_value);  // the job never ran: nobody may stay parked on the word
+      flags->release(flag);
+    }
   }
 };
 
@@ -375,6 +425,9 @@ class Engine {
   // staged collectives
   bool staged_ = true;               // TANDEM_HIP_ALGO=ring switches them off
   bool gathers_on_side_stream_ = false;  // TANDEM_HIP_GATHER=stream
+  std::shared_ptr<FlagPool> flags_;      // TANDEM_HIP_WAIT=stream
+  bool want_flags_ = false;
+  std::string sticky_error_;             // under mu_: a collective failed after its wait() had already returned
   bool ready_on_host_ = true;        // TANDEM_HIP_READY=gpu: wait for the caller's stream on the GPU instead
   size_t staging_half_ = 64u << 20;  // bytes per half (TANDEM_HIP_STAGING_BYTES)
   size_t small_bytes_ = 32u << 20;   // all_reduce up to this size takes the one-handshake form (TANDEM_HIP_SMALL_BYTES)
@@ -442,6 +495,16 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
     if (v < 0) throw Invalid("TANDEM_HIP_SMALL_BYTES must not be negative");
     small_bytes_ = static_cast<size_t>(v);
   }
+  if (const char* wm = std::getenv("TANDEM_HIP_WAIT")) {
+    if (std::string(wm) == "stream") {
+      int can = 0;
+      (void)hipDeviceGetAttribute(&can, hipDeviceAttributeCanUseStreamWaitValue, device);
+      if (can != 1) throw Invalid("TANDEM_HIP_WAIT=stream: this device cannot make a stream wait for a value");
+      want_flags_ = true;
+    } else if (std::string(wm) != "host") {
+      throw Invalid("TANDEM_HIP_WAIT must be \"host\" or \"stream\"");
+    }
+  }
   if (const char* gm = std::getenv("TANDEM_HIP_GATHER")) gathers_on_side_stream_ = std::string(gm) == "stream";
   if (const char* rd = std::getenv("TANDEM_HIP_READY")) ready_on_host_ = std::string(rd) != "gpu";
   peer_staging_.assign(size, nullptr);
@@ -457,6 +520,7 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
 
 void Engine::start() {
   check_hip(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags");  // default priority, all three
+  if (want_flags_) flags_ = FlagPool::make();
   check_hip(hipStreamCreateWithFlags(&gather_stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags (gathers)");
   check_hip(hipStreamCreateWithFlags(&anchor_stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags (anchors)");
 
@@ -610,6 +674,10 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
   work->device = device_;
   work->uses_gpu = uses_gpu;
   work->drained = drained;
+  if (flags_ && uses_gpu) {
+    work->flag = flags_->acquire(&work->flag_value);
+    if (work->flag >= 0) work->flags = flags_;
+  }
   hipEvent_t ready = nullptr;
   if (uses_gpu) {
     // Start once the caller's stream has produced the inputs.
@@ -635,9 +703,9 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
   }
   {
     std::lock_guard<std::mutex> lock(mu_);
-    if (stopping_) {
+    if (stopping_ || !sticky_error_.empty()) {
       if (ready) (void)hipEventDestroy(ready);  // the job that would have released it never runs
-      throw std::runtime_error("the engine is closed");
+      throw std::runtime_error(stopping_ ? "the engine is closed" : "an earlier collective failed: " + sticky_error_);
     }
     jobs_.emplace_back(std::move(job), work);
     submitted_.fetch_add(1, std::memory_order_release);
@@ -702,6 +770,18 @@ void Engine::loop() {
           hipEventRecord(w.done_event, stream_) != hipSuccess) {
         status = TDM_ERUNTIME;
         error = "could not record the collective's completion event";
+      }
+    }
+    if (w.flag >= 0) {
+      // Whoever waits for the word on the GPU is let go behind the job's last kernel, by the
+      // engine's own stream; after a failure (or with that stream idle anyway) at once, by the host.
+      uint32_t* word = w.flags->base + w.flag;
+      if (status != TDM_OK || w.drained || hipStreamWriteValue32(stream_, word, w.flag_value, 0) != hipSuccess) {
+        w.flags->set(w.flag, w.flag_value);
+      }
+      if (status != TDM_OK) {  // its wait() may have returned long ago: the next call reports it
+        std::lock_guard<std::mutex> lock(mu_);
+        if (sticky_error_.empty()) sticky_error_ = error;
       }
     }
     {
@@ -1711,6 +1791,15 @@ int tdm_work_wait(tdm_work* w, tdm_stream caller) {
     return TDM_EINVAL;
   }
   Work& work = *w->impl;
+  if (work.flag >= 0 && !work.finished_hint.load(std::memory_order_acquire)) {
+    // The job has not run yet: park the caller's stream on its word and return. The host
+    // goes on queueing work behind the collective; a failure shows at the next call.
+    return guard([&] {
+      check_hip(hipStreamWaitValue32(static_cast<hipStream_t>(caller), work.flags->base + work.flag, work.flag_value,
+                                     hipStreamWaitValueGte, 0xffffffffu),
+                "hipStreamWaitValue32 (wait)");
+    });
+  }
   spin_for([&] { return work.finished_hint.load(std::memory_order_acquire); });
   {
     std::unique_lock<std::mutex> lock(work.mu);

@@ -543,7 +543,7 @@ def mixed_sequence(g, seed, count):
     return results
 
 
-@pytest.mark.parametrize("algo", ["staged", "small"])
+@pytest.mark.parametrize("algo", ["staged", "small", "stream"])
 @pytest.mark.parametrize("world", [2, 3])
 def test_a_long_mixed_sequence_stays_bit_exact(world, algo, monkeypatch):
     """Forty collectives of mixed kinds and sizes in flight behind one another: the
@@ -551,7 +551,9 @@ def test_a_long_mixed_sequence_stays_bit_exact(world, algo, monkeypatch):
     from oracle import ring
     from tandem_amd import launch
 
-    choose(monkeypatch, algo)
+    choose(monkeypatch, "staged" if algo == "stream" else algo)
+    if algo == "stream":  # wait() parks the caller's stream on a word instead of blocking the host
+        monkeypatch.setenv("TANDEM_HIP_WAIT", "stream")
     seed, count = 11 + world, 40
     res = launch(mixed_sequence, world, seed, count, slot_bytes=4096, gpus=[0] * world, timeout=TIMEOUT)
     for r, results in enumerate(res):
@@ -595,6 +597,36 @@ def test_ranks_that_disagree_are_found_out(what):
     from tandem_amd import launch
 
     assert launch(disagree, 2, what, gpus=[0, 0], timeout=TIMEOUT) == [True, True]
+
+
+def late_failure(g):
+    """With stream-ordered waiting a collective's wait() can return before the collective
+    has run; when it then fails (here: the peer never joins), the caller's stream is let
+    go, and the next call on the group reports the failure."""
+    import time
+
+    from tandem_amd import CommError
+
+    x = torch.ones(1000, device=g.device)
+    if g.rank == 1:
+        time.sleep(5.0)  # never joins; leaves after rank 0 has given up
+        g.abandon()
+        return True
+    g.all_reduce(x)  # returns at once: the stream is parked behind the collective
+    torch.cuda.synchronize()  # ... and released when the collective gives up
+    try:
+        g.all_reduce(x)
+    except CommError as e:
+        g.abandon()
+        return "an earlier collective failed" in str(e) and "timed out" in str(e)
+    return False
+
+
+def test_stream_ordered_wait_reports_a_failure_at_the_next_call(monkeypatch):
+    from tandem_amd import launch
+
+    monkeypatch.setenv("TANDEM_HIP_WAIT", "stream")
+    assert launch(late_failure, 2, gpus=[0, 0], timeout=2.0) == [True, True]
 
 
 def test_unknown_backend_and_cpu_device_are_refused():

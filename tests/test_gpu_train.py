@@ -161,3 +161,18 @@ def test_gradient_accumulation_matches_one_process():
         for r in range(2):
             assert res[r]["losses"] == ref_losses[r], (s, r)
             assert torch.equal(res[r]["weights"], ref_w), (s, r)
+
+
+
+def test_stream_ordered_wait_gives_the_same_weights(monkeypatch):
+    """TANDEM_HIP_WAIT=stream: wait() parks the training stream on a word the engine sets
+    behind the collective's last kernel, and the host runs ahead. Same bits."""
+    from tandem_amd import launch
+
+    monkeypatch.setenv("TANDEM_HIP_WAIT", "stream")
+    ref_losses, ref_w = one_process(2)
+    for s in ("ddp", "ddpd", "zero2", "zero3"):
+        res = launch(train_rank, 2, s, 4 << 10, STEPS, BATCH, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT)
+        for r in range(2):
+            assert res[r]["losses"] == ref_losses[r], (s, r)
+            assert torch.equal(res[r]["weights"], ref_w), (s, r)
