@@ -196,6 +196,16 @@ def zero2_step(dev, reps):
     fused = timed(lambda: [z.opts[r].update("bench", z.bufs[r][z.layouts[r].lo:z.layouts[r].hi], z.grad_shards[r],
                                             [z.bufs[q][z.layouts[r].lo:z.layouts[r].hi] for q in range(WORLD) if q != r])
                            for r in range(WORLD)], reps)
+    def refill_grads():
+        for r in range(WORLD):
+            z.staging[r].copy_(grads[r])
+
+    t_refill_grads = timed(refill_grads, reps)
+    one = timed(lambda: (refill_grads(), z.reduce_and_step()), reps) - t_refill_grads
+    one_bytes = (8 * WORLD + 20) * n
+    out.update({"one_launch_ms": round(one * 1e3, 4), "one_launch_algorithmic_bytes": one_bytes,
+                "one_launch_GBps": round(one_bytes / one / 1e9, 1),
+                "one_launch_roofline_floor_ms": round(one_bytes / (HBM_PEAK_GBPS * 1e9) * 1e3, 4)})
     for algorithm, rs_bytes in (("fold", (WORLD + 2) * 4 * n), ("ring", 12 * (WORLD - 1) * n + 12 * n)):
         # default: fold + the update that also writes the other ranks' copies; ring: three ring steps, update, ring all-gather
         is_fold = algorithm == "fold"
@@ -211,7 +221,8 @@ def zero2_step(dev, reps):
                 "all_gather_ms": round(ag * 1e3, 4), "all_gather_GBps": round(8 * (WORLD - 1) * n / ag / 1e9, 1),
                 "adamw_gather_4_shards_ms": round(fused * 1e3, 4),
                 "adamw_gather_GBps": round((28 + 4 * (WORLD - 1)) * shard * WORLD / fused / 1e9, 1),
-                "note": "ms: gradients reduced by the single-launch ring-order fold, then AdamW writing the new parameters to all "
+                "note": "one_launch_ms: reduce-scatter, gradient add, AdamW and all-gather fused into one kernel (LocalZeRO2.reduce_and_step); "
+                        "ms: gradients reduced by the single-launch ring-order fold, then AdamW writing the new parameters to all "
                         "four ranks' buffers in the same pass (default); ring_ms: the ring's three reduce steps, AdamW, the ring's "
                         "three gather steps"})
     return out

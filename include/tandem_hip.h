@@ -183,6 +183,38 @@ int tdm_k3_adamw(float* p, const float* g, float* m, float* v, int64_t n, const 
 int tdm_k3_adamw_gather(float* p, const float* g, float* m, float* v, int64_t n, const tdm_adamw_scalars* s, int order,
                         float* const* copies, int ncopies, tdm_stream stream);
 
+/* ---- K2 + K3: ZeRO-2's reduce-scatter, gradient add, AdamW and all-gather in one launch ---- */
+
+/* One segment: `count` elements that lie in ring chunk `chunk` (= the rank that owns
+ * them) of a ZeRO bucket. grad[r]: rank r's gradient (its staging buffer); param[r]: rank
+ * r's copy of the parameters; exp_avg, exp_avg_sq: the owner's optimizer state. fp32. */
+typedef struct tdm_step_seg {
+  const void* grad[TDM_MAX_WORLD];
+  void* param[TDM_MAX_WORLD];
+  void* exp_avg;
+  void* exp_avg_sq;
+  int64_t count;
+  int32_t chunk;
+  int32_t reserved;
+} tdm_step_seg;
+
+/* The device table, as for K2: tiles and bytes it needs (-1: bad arguments), its image
+ * in host memory (the caller copies it to the device once). */
+int64_t tdm_k23_table_tiles(const tdm_step_seg* segs, int nseg);
+int64_t tdm_k23_table_bytes(const tdm_step_seg* segs, int nseg);
+int tdm_k23_table_build(const tdm_step_seg* segs, int nseg, int world, void* image);
+
+/* For every element of every segment:
+ *     mine = the ring-order fold of grad[0..W) (average: each divided by W first), as tdm_k2_bucket_fold
+ *     g    = 0 + mine                      (grad_shard.add_(mine) onto a zeroed shard, tandem/zero.py:150-153)
+ *     p, exp_avg, exp_avg_sq updated as tdm_k3_adamw does, on the owner's copy
+ *     param[r] = p for every rank r        (the all-gather of tandem/zero.py:163)
+ * i.e. ZeRO stage 2's communication and optimizer step (tandem/zero.py:141-163) for ranks
+ * that are buffers of one process, provided the gradient shards were zero (no accumulation
+ * over several backward passes); the same bits, (8W + 20) instead of (12W + 28) bytes per element. */
+int tdm_k23_zero2_step(const void* table_dev, int64_t ntiles, int world, int average, const tdm_adamw_scalars* s, int order,
+                       tdm_stream stream);
+
 /* ---- K4: ZeRO-3 unit gather ---------------------------------------------- */
 
 /* full[lo_q : lo_q + sizes[q]] = shards[q][0 : sizes[q]] for every rank q, in one

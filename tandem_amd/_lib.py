@@ -37,6 +37,12 @@ class FoldSeg(ctypes.Structure):
                 ("count", ctypes.c_int64), ("chunk", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
 
+class StepSeg(ctypes.Structure):
+    _fields_ = [("grad", ctypes.c_void_p * TDM_MAX_WORLD), ("param", ctypes.c_void_p * TDM_MAX_WORLD),
+                ("exp_avg", ctypes.c_void_p), ("exp_avg_sq", ctypes.c_void_p), ("count", ctypes.c_int64),
+                ("chunk", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+
 class AdamwScalars(ctypes.Structure):
     _fields_ = [("use_decay", ctypes.c_int32), ("decay", ctypes.c_float), ("w1", ctypes.c_float),
                 ("beta2", ctypes.c_float), ("one_m_b2", ctypes.c_float), ("bc2_sqrt", ctypes.c_float),
@@ -70,6 +76,11 @@ _SIGNATURES = {
     "tdm_k3_adamw_gather": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                            ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.POINTER(ctypes.c_void_p),
                                            ctypes.c_int, ctypes.c_void_p]),
+    "tdm_k23_table_tiles": (ctypes.c_int64, [ctypes.POINTER(StepSeg), ctypes.c_int]),
+    "tdm_k23_table_bytes": (ctypes.c_int64, [ctypes.POINTER(StepSeg), ctypes.c_int]),
+    "tdm_k23_table_build": (ctypes.c_int, [ctypes.POINTER(StepSeg), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
+    "tdm_k23_zero2_step": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                          ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
     "tdm_k4_unit_gather": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_int64),
                                           ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
 }

@@ -613,6 +613,114 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
   }
 }
 
+// ---------------------------------------------------------------- K2 + K3: ZeRO-2's whole step
+// For every element of every bucket segment, in one launch: the gradients of all ranks
+// are folded in the ring's order for the segment's chunk (K2), the sum is added to a zero
+// gradient shard as ZeRO's grad_shard.add_(mine) would (0.0f + mine: a -0.0 becomes +0.0),
+// the chunk's owner takes its AdamW step (K3), and the new parameter is written into every
+// rank's flat buffer (the all-gather). 4W + 12 bytes read and 4W + 8 written per element,
+// where reduce-scatter, add, AdamW and all-gather apart move 4(W+2) + 28 + 8(W-1).
+struct StepSegDev {
+  const char* g[TDM_MAX_WORLD];  // every rank's gradient for this tile
+  char* p[TDM_MAX_WORLD];        // every rank's copy of the parameters for this tile
+  char* m;                       // the owner's exp_avg
+  char* v;                       // the owner's exp_avg_sq
+  int64_t count;
+  int32_t chunk;                 // the owner
+  int32_t vec_ok;
+};
+
+template <int kWorld, int kDiv, int kOrder>
+__global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegDev* __restrict__ tiles, int64_t total,
+                                                                  Divisor<float> dv, tdm_adamw_scalars s) {
+#ifndef TDM_K23_UNROLL
+#define TDM_K23_UNROLL 4
+#endif
+#ifndef TDM_NT_MASK_K23
+#define TDM_NT_MASK_K23 TDM_NT_MASK_K3
+#endif
+  constexpr int kU = kWorld <= 4 ? TDM_K23_UNROLL : 1;  // vectors per lane in flight, per stream
+  constexpr int kM = TDM_NT_MASK_K23;
+  const bool small_w = __builtin_fabsf(s.w1) < 0.5f;
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    const StepSegDev& sg = tiles[tile];
+    const int c = sg.chunk;
+    const int64_t n = sg.count;
+    const char* gp[kWorld];
+#pragma unroll
+    for (int k = 0; k < kWorld; ++k) gp[k] = sg.g[(c + 1 + k) % kWorld];  // the fold ends with the owner's own term
+    char* own = sg.p[c];
+    auto one = [&](float grads_in_order[kWorld], float& P, float& M, float& V) {
+      float acc = scaled<float, kDiv>(grads_in_order[0], dv.divisor, dv.reciprocal);
+#pragma unroll
+      for (int k = 1; k < kWorld; ++k) acc = scaled<float, kDiv>(grads_in_order[k], dv.divisor, dv.reciprocal) + acc;
+      const float g = 0.0f + acc;  // grad_shard (zero) += mine
+      adamw_elem<kOrder>(P, g, M, V, s, small_w);
+    };
+    if (sg.vec_ok) {
+      const int64_t nv = n / 4;
+#pragma unroll
+      for (int u0 = 0; u0 < kUnroll; u0 += kU) {
+        vec16 in[kWorld][kU], rp[kU], rm[kU], rv[kU];
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          const int64_t v = threadIdx.x + static_cast<int64_t>(u0 + u) * kThreads;
+          if (v < nv) {
+#pragma unroll
+            for (int k = 0; k < kWorld; ++k) in[k][u] = load_stream<kM>(gp[k] + v * 16);
+            rp[u] = load_rmw<kM>(own + v * 16);
+            rm[u] = load_rmw<kM>(sg.m + v * 16);
+            rv[u] = load_rmw<kM>(sg.v + v * 16);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          const int64_t v = threadIdx.x + static_cast<int64_t>(u0 + u) * kThreads;
+          if (v < nv) {
+            Lanes<float> P = unpack<float>(rp[u]), M = unpack<float>(rm[u]), V = unpack<float>(rv[u]);
+#pragma unroll
+            for (int l = 0; l < 4; ++l) {
+              float gs[kWorld];
+#pragma unroll
+              for (int k = 0; k < kWorld; ++k) gs[k] = unpack<float>(in[k][u]).v[l];
+              one(gs, P.v[l], M.v[l], V.v[l]);
+            }
+            const vec16 packed = pack<float>(P);
+#pragma unroll
+            for (int q = 0; q < kWorld; ++q) store16<kM>(sg.p[q] + v * 16, packed);
+            store16<kM>(sg.m + v * 16, pack<float>(M));
+            store16<kM>(sg.v + v * 16, pack<float>(V));
+          }
+        }
+      }
+      if (threadIdx.x < n - nv * 4) {  // the tile's last few elements
+        const int64_t i = nv * 4 + threadIdx.x;
+        float gs[kWorld];
+#pragma unroll
+        for (int k = 0; k < kWorld; ++k) gs[k] = reinterpret_cast<const float*>(gp[k])[i];
+        float P = reinterpret_cast<float*>(own)[i], M = reinterpret_cast<float*>(sg.m)[i], V = reinterpret_cast<float*>(sg.v)[i];
+        one(gs, P, M, V);
+#pragma unroll
+        for (int q = 0; q < kWorld; ++q) reinterpret_cast<float*>(sg.p[q])[i] = P;
+        reinterpret_cast<float*>(sg.m)[i] = M;
+        reinterpret_cast<float*>(sg.v)[i] = V;
+      }
+    } else {
+      for (int64_t i = threadIdx.x; i < n; i += kThreads) {
+        float gs[kWorld];
+#pragma unroll
+        for (int k = 0; k < kWorld; ++k) gs[k] = reinterpret_cast<const float*>(gp[k])[i];
+        float P = reinterpret_cast<float*>(own)[i], M = reinterpret_cast<float*>(sg.m)[i], V = reinterpret_cast<float*>(sg.v)[i];
+        one(gs, P, M, V);
+#pragma unroll
+        for (int q = 0; q < kWorld; ++q) reinterpret_cast<float*>(sg.p[q])[i] = P;
+        reinterpret_cast<float*>(sg.m)[i] = M;
+        reinterpret_cast<float*>(sg.v)[i] = V;
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- host side
 int elem_size(int dtype) {
   switch (dtype) {
@@ -816,6 +924,31 @@ template <typename T>
 void launch_fold(const void* image, int64_t tiles, int world, int average, bool accumulate, hipStream_t stream) {
   if (accumulate) launch_fold_a<T, true>(image, tiles, world, average, stream);
   else launch_fold_a<T, false>(image, tiles, world, average, stream);
+}
+
+template <int kWorld, int kOrder>
+void launch_step_o(const void* image, int64_t tiles, int average, const tdm_adamw_scalars& s, hipStream_t stream) {
+  const Divisor<float> dv = make_divisor<float>(kWorld);
+  const StepSegDev* t = static_cast<const StepSegDev*>(image);
+  const dim3 grid(grid_for(tiles)), block(kThreads);
+  switch (div_kind(kWorld, average != 0)) {
+    case 0: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 0, kOrder>), grid, block, 0, stream, t, tiles, dv, s); break;
+    case 1: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 1, kOrder>), grid, block, 0, stream, t, tiles, dv, s); break;
+    default: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 2, kOrder>), grid, block, 0, stream, t, tiles, dv, s); break;
+  }
+}
+
+template <int kWorld>
+void launch_step_w(const void* image, int64_t tiles, int average, const tdm_adamw_scalars& s, int order, hipStream_t stream) {
+  if (order == TDM_ADAMW_HOST_ORDER) launch_step_o<kWorld, TDM_ADAMW_HOST_ORDER>(image, tiles, average, s, stream);
+  else launch_step_o<kWorld, TDM_ADAMW_DEVICE_ORDER>(image, tiles, average, s, stream);
+}
+
+int64_t step_tiles(const tdm_step_seg* segs, int nseg) {
+  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * 4;
+  int64_t tiles = 0;
+  for (int i = 0; i < nseg; ++i) tiles += segs[i].count > 0 ? (segs[i].count + tile_elems - 1) / tile_elems : 0;
+  return tiles;
 }
 
 }  // namespace
@@ -1261,6 +1394,80 @@ int tdm_k3_adamw(float* p, const float* g, float* m, float* v, int64_t n, const 
 int tdm_k3_adamw_gather(float* p, const float* g, float* m, float* v, int64_t n, const tdm_adamw_scalars* s, int order,
                         float* const* copies, int ncopies, tdm_stream stream) {
   return guard([&] { adamw_launch(p, g, m, v, n, s, order, copies, ncopies, static_cast<hipStream_t>(stream)); });
+}
+
+int64_t tdm_k23_table_tiles(const tdm_step_seg* segs, int nseg) {
+  if (nseg < 0 || (nseg > 0 && segs == nullptr)) return -1;
+  return step_tiles(segs, nseg);
+}
+
+int64_t tdm_k23_table_bytes(const tdm_step_seg* segs, int nseg) {
+  const int64_t tiles = tdm_k23_table_tiles(segs, nseg);
+  if (tiles < 0) return -1;
+  return std::max<int64_t>(16, tiles * static_cast<int64_t>(sizeof(StepSegDev)));
+}
+
+int tdm_k23_table_build(const tdm_step_seg* segs, int nseg, int world, void* image) {
+  return guard([&] {
+    if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
+    if (nseg < 0 || (nseg > 0 && segs == nullptr) || image == nullptr) throw Invalid("bad table arguments");
+    std::memset(image, 0, static_cast<size_t>(tdm_k23_table_bytes(segs, nseg)));
+    StepSegDev* out = static_cast<StepSegDev*>(image);
+    const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * 4;
+    int64_t tiles = 0;
+    for (int i = 0; i < nseg; ++i) {
+      const tdm_step_seg& sg = segs[i];
+      if (sg.count < 0) throw Invalid("segment " + std::to_string(i) + ": negative count");
+      if (sg.count == 0) continue;
+      if (sg.chunk < 0 || sg.chunk >= world) throw Invalid("segment " + std::to_string(i) + ": chunk outside [0, world)");
+      if (!sg.exp_avg || !sg.exp_avg_sq) throw Invalid("segment " + std::to_string(i) + ": NULL optimizer state");
+      bool vec = reinterpret_cast<uintptr_t>(sg.exp_avg) % 16 == 0 && reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % 16 == 0;
+      if (reinterpret_cast<uintptr_t>(sg.exp_avg) % 4 || reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % 4) {
+        throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to 4 bytes");
+      }
+      for (int r = 0; r < world; ++r) {
+        if (!sg.grad[r] || !sg.param[r]) throw Invalid("segment " + std::to_string(i) + ": NULL gradient or parameter");
+        const uintptr_t a = reinterpret_cast<uintptr_t>(sg.grad[r]), b = reinterpret_cast<uintptr_t>(sg.param[r]);
+        if (a % 4 || b % 4) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to 4 bytes");
+        vec = vec && a % 16 == 0 && b % 16 == 0;
+      }
+      for (int64_t at = 0; at < sg.count; at += tile_elems) {
+        StepSegDev& rec = out[tiles++];
+        for (int r = 0; r < world; ++r) {
+          rec.g[r] = static_cast<const char*>(sg.grad[r]) + at * 4;
+          rec.p[r] = static_cast<char*>(sg.param[r]) + at * 4;
+        }
+        rec.m = static_cast<char*>(sg.exp_avg) + at * 4;
+        rec.v = static_cast<char*>(sg.exp_avg_sq) + at * 4;
+        rec.count = std::min<int64_t>(tile_elems, sg.count - at);
+        rec.chunk = sg.chunk;
+        rec.vec_ok = vec;
+      }
+    }
+  });
+}
+
+int tdm_k23_zero2_step(const void* table_dev, int64_t ntiles, int world, int average, const tdm_adamw_scalars* s, int order,
+                       tdm_stream stream) {
+  return guard([&] {
+    if (ntiles < 0) throw Invalid("ntiles is negative");
+    if (ntiles == 0) return;
+    if (table_dev == nullptr || s == nullptr) throw Invalid("NULL argument");
+    if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (world) {
+      case 1: launch_step_w<1>(table_dev, ntiles, average, *s, order, st); break;
+      case 2: launch_step_w<2>(table_dev, ntiles, average, *s, order, st); break;
+      case 3: launch_step_w<3>(table_dev, ntiles, average, *s, order, st); break;
+      case 4: launch_step_w<4>(table_dev, ntiles, average, *s, order, st); break;
+      case 5: launch_step_w<5>(table_dev, ntiles, average, *s, order, st); break;
+      case 6: launch_step_w<6>(table_dev, ntiles, average, *s, order, st); break;
+      case 7: launch_step_w<7>(table_dev, ntiles, average, *s, order, st); break;
+      case 8: launch_step_w<8>(table_dev, ntiles, average, *s, order, st); break;
+      default: throw Invalid("world must be in [1, 8]");
+    }
+    check_hip(hipGetLastError(), "k23_zero2_step launch");
+  });
 }
 
 int tdm_k4_unit_gather(void* full, const void* const* shards, const int64_t* sizes, int world, int dtype,

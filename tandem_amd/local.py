@@ -272,6 +272,28 @@ class LocalZeRO2:
                 lo += m
         self._fold = (FoldTable.from_segments(world, torch.float32, device, rows, keep=(self.staging, self.grad_shards))
                       if world <= _lib.TDM_MAX_WORLD else None)
+        # The whole step as one launch (reduce_and_step): the optimizer state must exist, at fixed addresses.
+        self._shards_zero = True
+        self._step_table = None
+        if world <= _lib.TDM_MAX_WORLD:
+            for r in range(world):
+                self.opts[r].state["flat"] = [0.0, torch.zeros_like(self.grad_shards[r]), torch.zeros_like(self.grad_shards[r])]
+            segs = (_lib.StepSeg * max(1, len(rows)))()
+            bb = [t.data_ptr() for t in self.bufs]
+            for k, (srcs, _dsts, m, c) in enumerate(rows):
+                lo = (srcs[0] - sb[0]) // es  # the segment's offset in the flat buffers
+                at = lo - self.layouts[c].lo
+                _, exp_avg, exp_avg_sq = self.opts[c].state["flat"]
+                for r in range(world):
+                    segs[k].grad[r] = srcs[r]
+                    segs[k].param[r] = bb[r] + lo * es
+                segs[k].exp_avg = exp_avg.data_ptr() + at * es
+                segs[k].exp_avg_sq = exp_avg_sq.data_ptr() + at * es
+                segs[k].count, segs[k].chunk = m, c
+            ntiles = lib().tdm_k23_table_tiles(segs, len(rows))
+            image = torch.empty(max(16, lib().tdm_k23_table_bytes(segs, len(rows))), dtype=torch.uint8)
+            check(lib().tdm_k23_table_build(segs, len(rows), world, ctypes.c_void_p(image.data_ptr())))
+            self._step_table = (image.to(device), ntiles)
 
     def _launch(self, items, scale_dst, scale_src, writeback):
         st = stream_ptr(self.device)
@@ -287,12 +309,35 @@ class LocalZeRO2:
         order for the chunk, and adds into the owner's gradient shard; the same bits
         (including -0.0 + 0.0 = +0.0 from the add) with half the HBM traffic. The
         staging buffers are left untouched by the fold."""
+        self._shards_zero = False
         if algorithm == "fold" and self._fold is not None:
             self._fold.run(average=True, accumulate=True)
             return
         for s, items in enumerate(self._steps):
             self._launch(items, True, s == 0, s == 0)
         self._launch(self._adds, False, False, False)  # grad_shard += mine
+
+    def reduce_and_step(self):
+        """reduce_grads() and step() as ONE launch: for every element the ranks' gradients
+        are folded in the ring's order, added to the (zero) gradient shard as
+        grad_shard.add_(mine) would, the owner takes its AdamW step and the new
+        parameter goes into every rank's buffer. The same bits as reduce_grads(); step()
+        with 8W + 20 instead of 12W + 28 bytes of HBM traffic per element. Needs the
+        gradient shards at zero (no accumulation since zero_grad()) and at most 8 ranks;
+        the shards stay zero."""
+        from .optim import step_scalars
+
+        if self._step_table is None or not self._shards_zero:
+            self.reduce_grads()
+            self.step()
+            return
+        for opt in self.opts:
+            opt.state["flat"][0] += 1.0
+        o = self.opts[0]
+        scalars = step_scalars(o.state["flat"][0], o.lr, o.betas, o.eps, o.weight_decay)
+        image, ntiles = self._step_table
+        check(lib().tdm_k23_zero2_step(ctypes.c_void_p(image.data_ptr()), ntiles, self.world, 1, ctypes.byref(scalars),
+                                       o.order, stream_ptr(self.device)))
 
     def step(self, fused_gather=True):
         """Every rank's AdamW step on its shard, then the all-gather of the flat
@@ -309,5 +354,7 @@ class LocalZeRO2:
             self.lw.all_gather(self.bufs, self.layouts[0].sizes)
 
     def zero_grad(self):
-        for g in self.grad_shards:
-            g.zero_()
+        if not self._shards_zero:
+            for g in self.grad_shards:
+                g.zero_()
+        self._shards_zero = True

@@ -43,7 +43,7 @@ def oracle_zero2(world, numels, bucket_bytes, params0, grads_per_step):
     return bufs, opts
 
 
-@pytest.mark.parametrize("algorithm", ["fold", "ring"])
+@pytest.mark.parametrize("algorithm", ["fold", "ring", "fused"])
 @pytest.mark.parametrize("world", [2, 4, 3])
 def test_small_model_bit_exact_with_oracle(world, algorithm):
     from tandem_amd.local import LocalZeRO2
@@ -63,8 +63,12 @@ def test_small_model_bit_exact_with_oracle(world, algorithm):
     for s in range(steps):
         for r in range(world):
             z.staging[r].copy_(torch.from_numpy(grads[s][r]))
-        z.reduce_grads(algorithm)
-        z.step(fused_gather=algorithm == "fold")  # the update writes every rank's copy, or a ring all-gather follows
+        if algorithm == "fused":  # reduce-scatter, add, AdamW and all-gather as one launch
+            assert z._step_table is not None and z._shards_zero
+            z.reduce_and_step()
+        else:
+            z.reduce_grads(algorithm)
+            z.step(fused_gather=algorithm == "fold")  # the update writes every rank's copy, or a ring all-gather follows
         z.zero_grad()
     want, opts = oracle_zero2(world, numels, 4 << 10, p0, grads)
     for r in range(world):
@@ -130,3 +134,40 @@ def test_full_size_step():
     pn = p0[lay[r].lo:lay[r].hi].cpu().numpy().copy()
     AdamW(**KW).update("k", pn, shards_before[r].cpu().numpy())
     assert np.array_equal(bits(z.bufs[0][lay[r].lo:lay[r].hi].cpu().numpy()), bits(pn))
+
+
+def test_full_size_step_in_one_launch():
+    """The same 85,842,432-parameter step as reduce_and_step(): one launch must leave
+    every rank's parameters and every rank's optimizer state with the bits that
+    reduce_grads() + step() leave, over three steps."""
+    from tandem_amd.local import LocalZeRO2
+
+    dev = torch.device("cuda", 0)
+    plan = golden_json("plans.json")
+    numels = [math.prod(s) for _, s in plan["medium_params"]]
+    world, n = 4, sum(numels)
+    apart, fused = LocalZeRO2(world, numels, dev, **KW), LocalZeRO2(world, numels, dev, **KW)
+    gen = torch.Generator(device=dev).manual_seed(3)
+    p0 = torch.randn(n, device=dev, generator=gen) * 0.02
+    for z in (apart, fused):
+        for b in z.bufs:
+            b.copy_(p0)
+    del p0
+    for step in range(3):
+        for r in range(world):
+            g = torch.randn(n, device=dev, generator=gen) * 1e-3
+            g[:4] = torch.tensor([0.0, -0.0, 1e-45, -1e-45], device=dev)
+            apart.staging[r].copy_(g)
+            fused.staging[r].copy_(g)
+        del g
+        apart.reduce_grads()
+        apart.step()
+        apart.zero_grad()
+        fused.reduce_and_step()
+        fused.zero_grad()
+    for r in range(world):
+        assert torch.equal(apart.bufs[r].view(torch.int32), fused.bufs[r].view(torch.int32)), r
+        for i in (1, 2):
+            assert torch.equal(apart.opts[r].state["flat"][i].view(torch.int32), fused.opts[r].state["flat"][i].view(torch.int32)), (r, i)
+        assert apart.opts[r].state["flat"][0] == fused.opts[r].state["flat"][0] == 3.0
+        assert float(fused.grad_shards[r].abs().sum()) == 0.0
