@@ -606,7 +606,7 @@ def main():
             line["train_step_4_processes"] = train4
         if cpu is not None:
             cpu["gpu_over_cpu"] = round(line["value"] / cpu["value"], 1)
-            cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["ms"], 1)
+            cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["one_launch_ms"], 1)
             line["cpu_baseline"] = cpu
     line["device"] = device_name(_lib)
     print(json.dumps(line), flush=True)
