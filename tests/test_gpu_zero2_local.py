@@ -171,3 +171,81 @@ def test_full_size_step_in_one_launch():
             assert torch.equal(apart.opts[r].state["flat"][i].view(torch.int32), fused.opts[r].state["flat"][i].view(torch.int32)), (r, i)
         assert apart.opts[r].state["flat"][0] == fused.opts[r].state["flat"][0] == 3.0
         assert float(fused.grad_shards[r].abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("average", [1, 0])
+@pytest.mark.parametrize("world", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_one_launch_step_through_the_c_abi(world, average):
+    """tdm_k23_zero2_step on its own, at every world size it is built for: segments of
+    odd lengths (one element, a tile and a bit, several tiles), each owned by a different
+    chunk, once 16-byte aligned and once 4 bytes off (the scalar path), two steps. Host
+    order against the oracle's fold + AdamW; device order against the oracle's fold fed
+    to the separate AdamW kernel in device order."""
+    import ctypes
+
+    from oracle import ring
+    from oracle.adamw import AdamW
+    from tandem_amd import _lib
+    from tandem_amd._lib import check, lib, stream_ptr
+    from tandem_amd.optim import ShardedAdamW, step_scalars
+
+    dev = torch.device("cuda", 0)
+    counts = [1, 3, 4099, 10007, 0, 4 * 4096 + 4, 2048]
+    for shift in (0, 1):
+        for order in ("host", "device"):
+            nseg = len(counts)
+            total = sum(counts) + 8 * nseg + 8
+            grads_h = [(seeded(40 + shift, r, total) * 1e-3).numpy() for r in range(world)]
+            for g in grads_h:
+                g[shift:shift + 4] = [0.0, -0.0, 1e-45, -1e-45]
+            p_h = (seeded(50, 0, total) * 0.02).numpy()
+            grads = [torch.from_numpy(g).to(dev) for g in grads_h]
+            params = [torch.from_numpy(p_h).to(dev) for _ in range(world)]
+            m, v = torch.zeros(total, device=dev), torch.zeros(total, device=dev)
+            segs = (_lib.StepSeg * nseg)()
+            spans, at = [], shift
+            for k, n in enumerate(counts):
+                spans.append((at, at + n, k % world))
+                for r in range(world):
+                    segs[k].grad[r] = grads[r].data_ptr() + at * 4
+                    segs[k].param[r] = params[r].data_ptr() + at * 4
+                segs[k].exp_avg, segs[k].exp_avg_sq = m.data_ptr() + at * 4, v.data_ptr() + at * 4
+                segs[k].count, segs[k].chunk = n, k % world
+                at += -(-n // 4) * 4 + 4  # keeps every segment's start at the same offset from 16-byte alignment
+            ntiles = lib().tdm_k23_table_tiles(segs, nseg)
+            assert ntiles == sum(-(-n // 4096) for n in counts)  # 16 KiB of every stream per tile
+            image = torch.empty(lib().tdm_k23_table_bytes(segs, nseg), dtype=torch.uint8)
+            check(lib().tdm_k23_table_build(segs, nseg, world, ctypes.c_void_p(image.data_ptr())))
+            table = image.to(dev)
+            # expectation
+            want_p, want_m, want_v = p_h.copy(), np.zeros(total, np.float32), np.zeros(total, np.float32)
+            oracle_opts = {k: AdamW(**KW) for k in range(nseg)}
+            device_opt = ShardedAdamW(order="device", **KW)
+            dp = torch.from_numpy(p_h).to(dev)
+            for step in (1.0, 2.0):
+                s = step_scalars(step, KW["lr"], KW["betas"], KW["eps"], KW["weight_decay"])
+                check(lib().tdm_k23_zero2_step(ctypes.c_void_p(table.data_ptr()), ntiles, world, average, ctypes.byref(s),
+                                               _lib.ADAMW_HOST_ORDER if order == "host" else _lib.ADAMW_DEVICE_ORDER,
+                                               stream_ptr(dev)))
+                for k, (lo, hi, c) in enumerate(spans):
+                    if hi == lo:
+                        continue
+                    mine = np.float32(0.0) + ring.fold(grads_h, c, lo, hi, bool(average))
+                    if order == "host":
+                        o = oracle_opts[k]
+                        o.update("s", want_p[lo:hi], mine)
+                        want_m[lo:hi], want_v[lo:hi] = o.state["s"][1], o.state["s"][2]
+                    else:
+                        device_opt.update(k, dp[lo:hi], torch.from_numpy(mine).to(dev))
+            torch.cuda.synchronize(dev)
+            if order == "device":
+                want_p = dp.cpu().numpy()
+                for k, (lo, hi, _) in enumerate(spans):
+                    if hi > lo:
+                        want_m[lo:hi] = device_opt.state[k][1].cpu().numpy()
+                        want_v[lo:hi] = device_opt.state[k][2].cpu().numpy()
+            what = (world, average, shift, order)
+            for r in range(world):  # every rank's copy, and nothing outside the segments touched
+                assert np.array_equal(bits(params[r].cpu().numpy()), bits(want_p)), what + (r,)
+            assert np.array_equal(bits(m.cpu().numpy()), bits(want_m)), what
+            assert np.array_equal(bits(v.cpu().numpy()), bits(want_v)), what
