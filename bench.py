@@ -121,11 +121,21 @@ def sweep(lw, dev, steps):
         per, rs, ag = time_ring(lw, bufs, reps, 3)
         fold = timed(lambda: lw.all_reduce(bufs, "avg", algorithm="fold"), reps)
         b = n * 4
+        graph_ms = None
+        if kib <= 16384:  # launch-bound sizes: the same ring pass replayed from a HIP graph
+            flats = [x.reshape(-1) for x in bufs]
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                ring_pass(lw, flats)
+            graph_ms = round(timed(graph.replay, reps) * 1e3, 4)
+            del graph
         rows.append({"MiB": kib / 1024, "ring_ms": round(per * 1e3, 4), "ring_GBps": round(15 * b / per / 1e9, 1),
                      "ring_algbw_GBps": round(b / per / 1e9, 1),
                      "k1_frac_of_hbm": round(12 * n * (WORLD - 1) / (rs * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                      "fold_ms": round(fold * 1e3, 4), "fold_GBps": round(2 * WORLD * b / fold / 1e9, 1),  # every rank's b bytes read once, written once
                      "fold_algbw_GBps": round(b / fold / 1e9, 1)})
+        if graph_ms is not None:
+            rows[-1]["ring_hip_graph_ms"] = graph_ms
         del bufs
         torch.cuda.empty_cache()
     return rows

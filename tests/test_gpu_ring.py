@@ -250,3 +250,46 @@ def test_full_size_properties(dev):
     exact = sum(i.double() for i in ints)
     lw.all_reduce(ints, op="sum")
     assert torch.equal(ints[2].double(), exact)
+
+
+@pytest.mark.parametrize("world", [2, 4])
+def test_collectives_replayed_from_a_hip_graph(dev, world):
+    """The single-process collectives make no allocation, copy or host wait, so a caller
+    may capture them into a HIP graph (a ring pass at a small size is six launches of a
+    few microseconds each). Every replay, with eager work and a host wait between the
+    replays, must give the eager result's bits."""
+    from oracle import ring
+    from tandem_amd import LocalWorld
+
+    lw = LocalWorld(world)
+    n = 16 * 1024 + 37
+    ins = [[seeded(60 + k, r, n) * 1e-2 for r in range(world)] for k in range(4)]
+    bufs = [torch.empty(n, device=dev) for _ in range(world)]
+    other = [torch.empty(n, device=dev) for _ in range(world)]
+
+    def ring_pass(b):
+        lw.reduce_scatter(b, op="avg")
+        lw.all_gather(b)
+
+    def fold(b):
+        lw.all_reduce(b, "avg", algorithm="fold")
+
+    for run in (ring_pass, fold):
+        for b, x in zip(bufs, ins[0]):
+            b.copy_(x)
+        run(bufs)  # warm-up outside the capture
+        torch.cuda.synchronize(dev)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run(bufs)
+        for k in range(1, 4):
+            want = ring.expected_all_reduce([x.numpy() for x in ins[k]], True)
+            for b, o, x in zip(bufs, other, ins[k]):
+                b.copy_(x)
+                o.copy_(x)
+            graph.replay()
+            run(other)  # the same call made eagerly, behind the replay on the same stream
+            torch.cuda.synchronize(dev)
+            for r in range(world):
+                assert np.array_equal(bits(bufs[r].cpu().numpy()), bits(want)), (run.__name__, k, r)
+                assert torch.equal(bufs[r].view(torch.int32), other[r].view(torch.int32)), (run.__name__, k, r)
