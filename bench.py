@@ -316,7 +316,8 @@ def train_rank(g, strategy, steps):
     text = synthetic(100_000)
     model = GPT(cfg).to(g.device)
     adamw = dict(lr=3e-4, betas=(0.9, 0.95), weight_decay=0.1)
-    direct = strategy.endswith("+direct")
+    fused = strategy.endswith("+fused")
+    direct = strategy.endswith("+direct") or fused
     kind = strategy.split("+")[0]
     opt = None
     if kind == "alone":
@@ -324,7 +325,7 @@ def train_rank(g, strategy, steps):
     elif kind == "ddp":
         z, opt = DDP(model, g, direct=direct), torch.optim.AdamW(model.parameters(), foreach=False, **adamw)
     elif kind in ("zero1", "zero2"):
-        z = ZeRO(model, g, int(kind[-1]), ShardedAdamW(**adamw), direct=direct)
+        z = ZeRO(model, g, int(kind[-1]), ShardedAdamW(**adamw), direct=direct, fused_step=fused)
     else:
         z = FSDP(model, g, ShardedAdamW(**adamw))
     from tandem_amd.profile import Timeline, summarize
@@ -361,12 +362,13 @@ def train_rank(g, strategy, steps):
             "profile": {k: (round(v, 5) if isinstance(v, float) else v) for k, v in prof.items()}}
 
 
-def train_steps(steps, world=2, strategies=("alone", "ddp", "ddp+direct", "zero1", "zero1+direct", "zero2", "zero2+direct", "zero3")):
+def train_steps(steps, world=2, strategies=("alone", "ddp", "ddp+direct", "zero1", "zero1+direct", "zero2", "zero2+direct", "zero2+fused", "zero3")):
     from tandem_amd import launch
 
     out = {"workload": f"{world} processes sharing the GPU, 85.8M GPT, batch 8x512 split over the ranks, fp32, full step "
                        "(forward, backward, optimizer); 'alone' = the same rows with no communication and torch AdamW; "
-                       "'+direct' = buckets / flat buffers in the shared arenas, collectives arena to arena"}
+                       "'+direct' = buckets / flat buffers in the shared arenas, collectives arena to arena; '+fused' = that, and ZeRO-2's "
+                       "reduce-scatters, AdamW and all-gather as one launch per rank"}
     for s in strategies:
         res = launch(train_rank, world, s, steps, gpus=[0] * world, timeout=120.0)
         out[s] = {"step_ms": round(max(r["step_ms"] for r in res), 3), "loss": round(res[0]["loss"], 4),
@@ -547,7 +549,7 @@ def main():
         except Exception as e:
             train = {"error": repr(e)[:300]}
         try:
-            train4 = train_steps(5, 4, ("alone", "ddp", "zero2", "zero2+direct", "zero3"))
+            train4 = train_steps(5, 4, ("alone", "ddp", "zero2", "zero2+direct", "zero2+fused", "zero3"))
         except Exception as e:
             train4 = {"error": repr(e)[:300]}
         os.environ["TANDEM_HIP_WAIT"] = "stream"  # wait() parks the training stream instead of blocking the host

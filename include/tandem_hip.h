@@ -215,6 +215,11 @@ int tdm_k23_table_build(const tdm_step_seg* segs, int nseg, int world, void* ima
 int tdm_k23_zero2_step(const void* table_dev, int64_t ntiles, int world, int average, const tdm_adamw_scalars* s, int order,
                        tdm_stream stream);
 
+/* The same step for ONE segment, passed in the launch itself (no table in device memory):
+ * what a rank that is a process of its own runs over its shard, chunk = its rank. */
+int tdm_k23_zero2_step_segment(const tdm_step_seg* seg, int world, int average, const tdm_adamw_scalars* s, int order,
+                               tdm_stream stream);
+
 /* ---- K4: ZeRO-3 unit gather ---------------------------------------------- */
 
 /* full[lo_q : lo_q + sizes[q]] = shards[q][0 : sizes[q]] for every rank q, in one
@@ -316,6 +321,22 @@ int tdm_direct_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype
                               int average, const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out);
 int tdm_direct_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
                           const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out);
+
+/* ZeRO stage 2's reduce_scatter (every bucket), grad_shard.add_, AdamW and all_gather
+ * (tandem/zero.py:141-163) as one launch per rank, for ranks whose flat parameter buffer and
+ * flat gradient buffer lie in their shared arenas. `param` and `grad` are THIS rank's shard
+ * of its own two buffers (`count` fp32 elements, the rank's slice of the flat layout);
+ * param_offsets[q] / grad_offsets[q] are the byte offsets of the same slice inside rank q's
+ * arena; exp_avg / exp_avg_sq are this rank's optimizer state for the shard (ordinary device
+ * memory). The Work: fence (every rank's gradients are complete and nobody computes with
+ * the old parameters any more); tdm_k23_zero2_step_segment with chunk = this rank over
+ * all ranks' gradients, writing the new parameters into every rank's buffer; fence.
+ * `total` (the flat buffer's length) only serves to find ranks that disagree. The same
+ * bits as the separate calls provided the gradient shard was zero before (no accumulation
+ * over several backward passes). World sizes up to 8. */
+int tdm_direct_zero2_step(tdm_engine* e, void* param, const int64_t* param_offsets, const void* grad, const int64_t* grad_offsets,
+                          int noffsets, void* exp_avg, void* exp_avg_sq, int64_t count, int64_t total, int average,
+                          const tdm_adamw_scalars* s, int order, tdm_stream caller, tdm_work** out);
 int tdm_sendrecv(tdm_engine* e, const void* send, int64_t send_numel, int dst, void* recv, int64_t recv_numel, int src,
                  int dtype, tdm_stream caller, tdm_work** out);
 int tdm_barrier(tdm_engine* e, tdm_work** out);

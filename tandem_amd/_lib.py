@@ -81,6 +81,8 @@ _SIGNATURES = {
     "tdm_k23_table_build": (ctypes.c_int, [ctypes.POINTER(StepSeg), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "tdm_k23_zero2_step": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                           ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
+    "tdm_k23_zero2_step_segment": (ctypes.c_int, [ctypes.POINTER(StepSeg), ctypes.c_int, ctypes.c_int,
+                                                  ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
     "tdm_k4_unit_gather": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_int64),
                                           ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
 }
@@ -113,6 +115,8 @@ _ENGINE_SIGNATURES = {
                                                  _PI64, ctypes.c_int, _VP, _PVP]),
     "tdm_direct_all_gather": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _PI64, ctypes.c_int, _PI64, ctypes.c_int,
                                              _VP, _PVP]),
+    "tdm_direct_zero2_step": (ctypes.c_int, [_VP, _VP, _PI64, _VP, _PI64, ctypes.c_int, _VP, _VP, ctypes.c_int64, ctypes.c_int64,
+                                             ctypes.c_int, ctypes.POINTER(AdamwScalars), ctypes.c_int, _VP, _PVP]),
     "tdm_engine_share": (ctypes.c_int, [_VP, ctypes.c_int64, _PVP]),
     "tdm_unit_gather_direct": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _VP, _PI64, ctypes.c_int, _PI64,
                                               ctypes.c_int, _VP, _PVP]),

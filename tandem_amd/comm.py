@@ -275,6 +275,38 @@ class Group:
             self._engine, ctypes.c_void_p(flat.data_ptr()), self._count(flat, code), code, arr, n, self._stream(), out),
             t, t.numel() * t.element_size(), async_op, keep=(flat,))
 
+    def zero2_step(self, params, grads, sizes, exp_avg, exp_avg_sq, scalars, order, op="avg", async_op=False):
+        """ZeRO stage 2's reduce_scatter, gradient add, AdamW and all_gather as one
+        launch per rank (tandem/zero.py:141-163 in the reference, which makes a
+        reduce_scatter per bucket, `grad_shard.add_`, seven elementwise passes and an
+        all_gather of it). `params` and `grads` are the flat parameter and gradient
+        buffers, from shared_empty() at the same arena offsets on every rank; `sizes`
+        the shard sizes; `exp_avg`/`exp_avg_sq` this rank's state for its shard;
+        `scalars` from optim.step_scalars. The same bits as the separate calls when the
+        gradient shard was zero before."""
+        if op not in ("sum", "avg"):
+            raise CommError(f"unknown op {op}")
+        p, g = self._flat(params, "zero2_step"), self._flat(grads, "zero2_step")
+        if p.dtype != torch.float32 or g.dtype != torch.float32 or p.numel() != g.numel():
+            raise CommError("zero2_step: two fp32 buffers of one length")
+        sizes, _, _ = self._sizes(p, sizes if sizes is not None else [c.numel() for c in torch.tensor_split(p, self.size)])
+        lo, n = sum(sizes[:self.rank]), sizes[self.rank]
+        for name, t in (("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq)):
+            if t.device != self.device or t.dtype != torch.float32 or t.numel() != n or not t.is_contiguous():
+                raise CommError(f"zero2_step: {name} must be this rank's shard ({n} fp32 elements on {self.device})")
+        bases = []
+        for t in (p, g):
+            off = self.arena_offset(t)
+            if off is None:
+                raise CommError("zero2_step: the buffers must come from shared_empty()")
+            bases.append((ctypes.c_int64 * self.size)(*[off + lo * 4] * self.size))
+        mine_p, mine_g = p[lo:lo + n], g[lo:lo + n]
+        return self._start("zero2_step", lambda out: lib().tdm_direct_zero2_step(
+            self._engine, ctypes.c_void_p(mine_p.data_ptr()), bases[0], ctypes.c_void_p(mine_g.data_ptr()), bases[1], self.size,
+            ctypes.c_void_p(exp_avg.data_ptr()), ctypes.c_void_p(exp_avg_sq.data_ptr()), n, p.numel(), int(op == "avg"),
+            ctypes.byref(scalars), order, self._stream(), out),
+            params, (2 * self.size + 5) * 4 * n, async_op, keep=(p, g, exp_avg, exp_avg_sq, scalars))
+
     # ---- shared arena: long-lived data that peers read directly
     def share_arena(self, nbytes):
         """Creates this rank's shared arena: `nbytes` (under 2 GiB) of device memory

@@ -51,5 +51,6 @@ void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool s
                  bool writeback_src, hipStream_t stream, int policy = 2);
 void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream, int policy = 2);
 void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream);
+void zero2_step_segment(const tdm_step_seg& seg, int world, bool average, const tdm_adamw_scalars& s, int order, hipStream_t stream);
 
 }  // namespace tandem_hip

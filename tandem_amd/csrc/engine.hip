@@ -355,6 +355,10 @@ class Engine {
   std::shared_ptr<Work> direct(int kind, Buf t, std::vector<int64_t> sizes, bool average, std::vector<int64_t> peer_offsets,
                                hipStream_t caller);
 
+  std::shared_ptr<Work> zero2_step_direct(Buf param, Buf grad, std::vector<int64_t> param_offsets, std::vector<int64_t> grad_offsets,
+                                          char* exp_avg, char* exp_avg_sq, int64_t total, bool average, tdm_adamw_scalars s,
+                                          int order, hipStream_t caller);
+
   int device() const { return device_; }
   hipStream_t stream() const { return stream_; }
   int rank() const { return rank_; }
@@ -690,7 +694,13 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
     job = [this, ready, host_ready, w = work.get(), inner = std::move(job)] {
       hipError_t e;
       if (host_ready) {
-        e = poll_gpu([&] { return hipEventQuery(ready); }, timeout_s_);
+        try {
+          e = poll_gpu([&] { return hipEventQuery(ready); }, timeout_s_);
+        } catch (...) {
+          (void)hipGetLastError();
+          (void)hipEventDestroy(ready);
+          throw;
+        }
         (void)hipGetLastError();  // the "not ready" left by the polls
       } else {
         e = hipStreamWaitEvent(stream_, ready, 0);
@@ -1583,6 +1593,51 @@ std::shared_ptr<Work> Engine::direct(int kind, Buf t, std::vector<int64_t> sizes
   }, caller, true, true, true);
 }
 
+// ZeRO stage 2's communication and optimizer step in one launch per rank, for gradient
+// and parameter buffers that live in the arenas: fence (every rank's gradients are
+// complete, and no rank still computes with the old parameters); this rank folds its
+// shard's gradients out of all ranks' buffers in the ring's order, takes the AdamW step
+// and writes the new parameters into every rank's buffer; fence (every rank's writes have
+// landed). Replaces a reduce_scatter per bucket, grad_shard.add_, the update and the
+// all_gather (tandem/zero.py:141-163) with (8W + 20) bytes per element of the shard.
+std::shared_ptr<Work> Engine::zero2_step_direct(Buf param, Buf grad, std::vector<int64_t> param_offsets,
+                                                std::vector<int64_t> grad_offsets, char* exp_avg, char* exp_avg_sq,
+                                                int64_t total, bool average, tdm_adamw_scalars s, int order, hipStream_t caller) {
+  const char* what = "zero2_step (direct)";
+  check(param, what, true);
+  check(grad, what, true);
+  if (param.dtype != TDM_F32 || grad.dtype != TDM_F32) throw Invalid(std::string(what) + ": fp32 only");
+  if (param.numel != grad.numel) throw Invalid(std::string(what) + ": parameters and gradients differ in length");
+  if (size_ > TDM_MAX_WORLD) throw Invalid(std::string(what) + ": world sizes up to 8");
+  if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid(std::string(what) + ": unknown update order");
+  if (static_cast<int>(param_offsets.size()) != size_ || static_cast<int>(grad_offsets.size()) != size_) {
+    throw Invalid(std::string(what) + ": one arena offset per rank");
+  }
+  if (param.numel > 0) {
+    if (!exp_avg || !exp_avg_sq) throw Invalid(std::string(what) + ": NULL optimizer state");
+    check(Buf{exp_avg, param.numel, TDM_F32}, what, false);
+    check(Buf{exp_avg_sq, param.numel, TDM_F32}, what, false);
+  }
+  return submit([this, param, grad, param_offsets, grad_offsets, exp_avg, exp_avg_sq, total, average, s, order] {
+    tdm_step_seg seg;
+    std::memset(&seg, 0, sizeof seg);
+    if (param.numel > 0) {  // a rank with an empty shard still takes part in the fences
+      const char* base[TDM_MAX_WORLD];
+      direct_bases(grad, grad_offsets, base);
+      for (int q = 0; q < size_; ++q) seg.grad[q] = base[q];
+      direct_bases(param, param_offsets, base);
+      for (int q = 0; q < size_; ++q) seg.param[q] = const_cast<char*>(base[q]);  // the peers' arenas are mapped writable
+      seg.exp_avg = exp_avg;
+      seg.exp_avg_sq = exp_avg_sq;
+      seg.count = param.numel;
+      seg.chunk = rank_;
+    }
+    if (size_ > 1) barrier_now(true, fence_tag(9, TDM_F32, total));
+    zero2_step_segment(seg, size_, average, s, order, stream_);
+    if (size_ > 1) barrier_now(true);
+  }, caller, true, true, true);
+}
+
 // A barrier that is also ordered against the GPU: it starts after the caller's
 // stream has finished what it held at the call, and a rank's arrival is only
 // announced once its engine stream has finished too.
@@ -1769,6 +1824,23 @@ int tdm_direct_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype
 int tdm_direct_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
                           const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out) {
   return direct_call(e, 2, ptr, numel, dtype, sizes, nsizes, 0, peer_offsets, noffsets, caller, out);
+}
+
+int tdm_direct_zero2_step(tdm_engine* e, void* param, const int64_t* param_offsets, const void* grad, const int64_t* grad_offsets,
+                          int noffsets, void* exp_avg, void* exp_avg_sq, int64_t count, int64_t total, int average,
+                          const tdm_adamw_scalars* s, int order, tdm_stream caller, tdm_work** out) {
+  return guard([&] {
+    if (out == nullptr) throw Invalid("NULL work pointer");
+    if (s == nullptr) throw Invalid("NULL scalars");
+    if (noffsets < 0 || (noffsets > 0 && (param_offsets == nullptr || grad_offsets == nullptr))) throw Invalid("bad offsets argument");
+    std::vector<int64_t> po(param_offsets, param_offsets + noffsets), go(grad_offsets, grad_offsets + noffsets);
+    finish_submit(engine_of(e).zero2_step_direct(Engine::Buf{static_cast<char*>(param), count, TDM_F32},
+                                                 Engine::Buf{static_cast<char*>(const_cast<void*>(grad)), count, TDM_F32},
+                                                 std::move(po), std::move(go), static_cast<char*>(exp_avg),
+                                                 static_cast<char*>(exp_avg_sq), total, average != 0, *s, order,
+                                                 static_cast<hipStream_t>(caller)),
+                  out);
+  });
 }
 
 int tdm_fence(tdm_engine* e, tdm_stream caller, tdm_work** out) {

@@ -630,26 +630,31 @@ struct StepSegDev {
   int32_t vec_ok;
 };
 
-template <int kWorld, int kDiv, int kOrder>
-__global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegDev* __restrict__ tiles, int64_t total,
-                                                                  Divisor<float> dv, tdm_adamw_scalars s) {
 #ifndef TDM_K23_UNROLL
 #define TDM_K23_UNROLL 4
 #endif
 #ifndef TDM_NT_MASK_K23
 #define TDM_NT_MASK_K23 TDM_NT_MASK_K3
 #endif
+
+// One tile (at most 16 KiB of every stream) of the step.
+template <int kWorld, int kDiv, int kOrder>
+__device__ __forceinline__ void step_tile(const StepSegDev& sg, int64_t at, int64_t n, const Divisor<float>& dv,
+                                          const tdm_adamw_scalars& s, bool small_w) {
   constexpr int kU = kWorld <= 4 ? TDM_K23_UNROLL : 1;  // vectors per lane in flight, per stream
   constexpr int kM = TDM_NT_MASK_K23;
-  const bool small_w = __builtin_fabsf(s.w1) < 0.5f;
-  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
-    const StepSegDev& sg = tiles[tile];
-    const int c = sg.chunk;
-    const int64_t n = sg.count;
+  {
+    const int c = sg.chunk;  // `at`: the tile's offset in bytes from the record's pointers; n: its elements
     const char* gp[kWorld];
+    char* pp[kWorld];
 #pragma unroll
-    for (int k = 0; k < kWorld; ++k) gp[k] = sg.g[(c + 1 + k) % kWorld];  // the fold ends with the owner's own term
-    char* own = sg.p[c];
+    for (int k = 0; k < kWorld; ++k) {
+      gp[k] = sg.g[(c + 1 + k) % kWorld] + at;  // the fold ends with the owner's own term
+      pp[k] = sg.p[k] + at;
+    }
+    char* own = sg.p[c] + at;
+    char* const mm = sg.m + at;
+    char* const vv = sg.v + at;
     auto one = [&](float grads_in_order[kWorld], float& P, float& M, float& V) {
       float acc = scaled<float, kDiv>(grads_in_order[0], dv.divisor, dv.reciprocal);
 #pragma unroll
@@ -669,8 +674,8 @@ __global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegD
 #pragma unroll
             for (int k = 0; k < kWorld; ++k) in[k][u] = load_stream<kM>(gp[k] + v * 16);
             rp[u] = load_rmw<kM>(own + v * 16);
-            rm[u] = load_rmw<kM>(sg.m + v * 16);
-            rv[u] = load_rmw<kM>(sg.v + v * 16);
+            rm[u] = load_rmw<kM>(mm + v * 16);
+            rv[u] = load_rmw<kM>(vv + v * 16);
           }
         }
 #pragma unroll
@@ -687,9 +692,9 @@ __global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegD
             }
             const vec16 packed = pack<float>(P);
 #pragma unroll
-            for (int q = 0; q < kWorld; ++q) store16<kM>(sg.p[q] + v * 16, packed);
-            store16<kM>(sg.m + v * 16, pack<float>(M));
-            store16<kM>(sg.v + v * 16, pack<float>(V));
+            for (int q = 0; q < kWorld; ++q) store16<kM>(pp[q] + v * 16, packed);
+            store16<kM>(mm + v * 16, pack<float>(M));
+            store16<kM>(vv + v * 16, pack<float>(V));
           }
         }
       }
@@ -698,26 +703,49 @@ __global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegD
         float gs[kWorld];
 #pragma unroll
         for (int k = 0; k < kWorld; ++k) gs[k] = reinterpret_cast<const float*>(gp[k])[i];
-        float P = reinterpret_cast<float*>(own)[i], M = reinterpret_cast<float*>(sg.m)[i], V = reinterpret_cast<float*>(sg.v)[i];
+        float P = reinterpret_cast<float*>(own)[i], M = reinterpret_cast<float*>(mm)[i], V = reinterpret_cast<float*>(vv)[i];
         one(gs, P, M, V);
 #pragma unroll
-        for (int q = 0; q < kWorld; ++q) reinterpret_cast<float*>(sg.p[q])[i] = P;
-        reinterpret_cast<float*>(sg.m)[i] = M;
-        reinterpret_cast<float*>(sg.v)[i] = V;
+        for (int q = 0; q < kWorld; ++q) reinterpret_cast<float*>(pp[q])[i] = P;
+        reinterpret_cast<float*>(mm)[i] = M;
+        reinterpret_cast<float*>(vv)[i] = V;
       }
     } else {
       for (int64_t i = threadIdx.x; i < n; i += kThreads) {
         float gs[kWorld];
 #pragma unroll
         for (int k = 0; k < kWorld; ++k) gs[k] = reinterpret_cast<const float*>(gp[k])[i];
-        float P = reinterpret_cast<float*>(own)[i], M = reinterpret_cast<float*>(sg.m)[i], V = reinterpret_cast<float*>(sg.v)[i];
+        float P = reinterpret_cast<float*>(own)[i], M = reinterpret_cast<float*>(mm)[i], V = reinterpret_cast<float*>(vv)[i];
         one(gs, P, M, V);
 #pragma unroll
-        for (int q = 0; q < kWorld; ++q) reinterpret_cast<float*>(sg.p[q])[i] = P;
-        reinterpret_cast<float*>(sg.m)[i] = M;
-        reinterpret_cast<float*>(sg.v)[i] = V;
+        for (int q = 0; q < kWorld; ++q) reinterpret_cast<float*>(pp[q])[i] = P;
+        reinterpret_cast<float*>(mm)[i] = M;
+        reinterpret_cast<float*>(vv)[i] = V;
       }
     }
+  }
+}
+
+template <int kWorld, int kDiv, int kOrder>
+__global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegDev* __restrict__ tiles, int64_t total,
+                                                                  Divisor<float> dv, tdm_adamw_scalars s) {
+  const bool small_w = __builtin_fabsf(s.w1) < 0.5f;
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    step_tile<kWorld, kDiv, kOrder>(tiles[tile], 0, tiles[tile].count, dv, s, small_w);
+  }
+}
+
+// The same for ONE segment, described in the kernel's arguments: no table to keep in
+// device memory. A rank that is a process of its own steps exactly one segment, its
+// shard, out of its peers' gradient buffers and into their parameter buffers.
+template <int kWorld, int kDiv, int kOrder>
+__global__ __launch_bounds__(kThreads) void k23_zero2_step_one_kernel(StepSegDev whole, int64_t total, Divisor<float> dv,
+                                                                      tdm_adamw_scalars s) {
+  const bool small_w = __builtin_fabsf(s.w1) < 0.5f;
+  constexpr int64_t kTileBytes = static_cast<int64_t>(kTileVecs) * 16;
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    const int64_t n = min(static_cast<int64_t>(kTileVecs) * 4, whole.count - tile * kTileVecs * 4);
+    step_tile<kWorld, kDiv, kOrder>(whole, tile * kTileBytes, n, dv, s, small_w);
   }
 }
 
@@ -944,6 +972,23 @@ void launch_step_w(const void* image, int64_t tiles, int average, const tdm_adam
   else launch_step_o<kWorld, TDM_ADAMW_DEVICE_ORDER>(image, tiles, average, s, stream);
 }
 
+template <int kWorld, int kOrder>
+void launch_step_one_o(const StepSegDev& whole, int64_t tiles, int average, const tdm_adamw_scalars& s, hipStream_t stream) {
+  const Divisor<float> dv = make_divisor<float>(kWorld);
+  const dim3 grid(grid_for(tiles)), block(kThreads);
+  switch (div_kind(kWorld, average != 0)) {
+    case 0: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 0, kOrder>), grid, block, 0, stream, whole, tiles, dv, s); break;
+    case 1: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 1, kOrder>), grid, block, 0, stream, whole, tiles, dv, s); break;
+    default: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 2, kOrder>), grid, block, 0, stream, whole, tiles, dv, s); break;
+  }
+}
+
+template <int kWorld>
+void launch_step_one_w(const StepSegDev& whole, int64_t tiles, int average, const tdm_adamw_scalars& s, int order, hipStream_t stream) {
+  if (order == TDM_ADAMW_HOST_ORDER) launch_step_one_o<kWorld, TDM_ADAMW_HOST_ORDER>(whole, tiles, average, s, stream);
+  else launch_step_one_o<kWorld, TDM_ADAMW_DEVICE_ORDER>(whole, tiles, average, s, stream);
+}
+
 int64_t step_tiles(const tdm_step_seg* segs, int nseg) {
   const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * 4;
   int64_t tiles = 0;
@@ -952,6 +997,45 @@ int64_t step_tiles(const tdm_step_seg* segs, int nseg) {
 }
 
 }  // namespace
+
+// Used by the engine too: ZeRO-2's step over one segment (a rank's shard), see tdm_k23_zero2_step_segment.
+void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const tdm_adamw_scalars& s, int order, hipStream_t stream) {
+  if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
+  if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
+  if (sg.count < 0) throw Invalid("negative count");
+  if (sg.count == 0) return;
+  if (sg.chunk < 0 || sg.chunk >= world) throw Invalid("chunk outside [0, world)");
+  if (!sg.exp_avg || !sg.exp_avg_sq) throw Invalid("NULL optimizer state");
+  StepSegDev whole;
+  std::memset(&whole, 0, sizeof whole);
+  bool vec = reinterpret_cast<uintptr_t>(sg.exp_avg) % 16 == 0 && reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % 16 == 0;
+  if (reinterpret_cast<uintptr_t>(sg.exp_avg) % 4 || reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % 4) throw Invalid("pointer not aligned to 4 bytes");
+  for (int r = 0; r < world; ++r) {
+    if (!sg.grad[r] || !sg.param[r]) throw Invalid("NULL gradient or parameter");
+    const uintptr_t a = reinterpret_cast<uintptr_t>(sg.grad[r]), b = reinterpret_cast<uintptr_t>(sg.param[r]);
+    if (a % 4 || b % 4) throw Invalid("pointer not aligned to 4 bytes");
+    vec = vec && a % 16 == 0 && b % 16 == 0;
+    whole.g[r] = static_cast<const char*>(sg.grad[r]);
+    whole.p[r] = static_cast<char*>(sg.param[r]);
+  }
+  whole.m = static_cast<char*>(sg.exp_avg);
+  whole.v = static_cast<char*>(sg.exp_avg_sq);
+  whole.count = sg.count;
+  whole.chunk = sg.chunk;
+  whole.vec_ok = vec;
+  const int64_t tiles = step_tiles(&sg, 1);
+  switch (world) {
+    case 1: launch_step_one_w<1>(whole, tiles, average, s, order, stream); break;
+    case 2: launch_step_one_w<2>(whole, tiles, average, s, order, stream); break;
+    case 3: launch_step_one_w<3>(whole, tiles, average, s, order, stream); break;
+    case 4: launch_step_one_w<4>(whole, tiles, average, s, order, stream); break;
+    case 5: launch_step_one_w<5>(whole, tiles, average, s, order, stream); break;
+    case 6: launch_step_one_w<6>(whole, tiles, average, s, order, stream); break;
+    case 7: launch_step_one_w<7>(whole, tiles, average, s, order, stream); break;
+    default: launch_step_one_w<8>(whole, tiles, average, s, order, stream); break;
+  }
+  check_hip(hipGetLastError(), "k23_zero2_step_one launch");
+}
 
 // Used by the engine too.
 void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool scale_dst, bool scale_src,
@@ -1467,6 +1551,14 @@ int tdm_k23_zero2_step(const void* table_dev, int64_t ntiles, int world, int ave
       default: throw Invalid("world must be in [1, 8]");
     }
     check_hip(hipGetLastError(), "k23_zero2_step launch");
+  });
+}
+
+int tdm_k23_zero2_step_segment(const tdm_step_seg* seg, int world, int average, const tdm_adamw_scalars* s, int order,
+                               tdm_stream stream) {
+  return guard([&] {
+    if (seg == nullptr || s == nullptr) throw Invalid("NULL argument");
+    zero2_step_segment(*seg, world, average != 0, *s, order, static_cast<hipStream_t>(stream));
   });
 }
 

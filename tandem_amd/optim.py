@@ -83,5 +83,18 @@ class ShardedAdamW:
                                  ctypes.c_void_p(exp_avg.data_ptr()), ctypes.c_void_p(exp_avg_sq.data_ptr()),
                                  param.numel(), ctypes.byref(s), self.order, stream_ptr(param.device)))
 
+    def begin_step(self, key, param):
+        """For a caller that runs the update inside a fused launch of its own
+        (Group.zero2_step): creates the shard's state if need be, counts the step, and
+        returns (scalars, exp_avg, exp_avg_sq, order) for it."""
+        require_device_tensor(param, "ShardedAdamW.begin_step(param)")
+        if param.dtype != torch.float32:
+            raise ValueError("ShardedAdamW handles fp32 shards")
+        if key not in self.state:
+            self.state[key] = [0.0, torch.zeros_like(param), torch.zeros_like(param)]
+        st = self.state[key]
+        st[0] += 1.0
+        return step_scalars(st[0], self.lr, self.betas, self.eps, self.weight_decay), st[1], st[2], self.order
+
     def state_bytes(self):
         return sum(t.numel() * t.element_size() for _, a, b in self.state.values() for t in (a, b))

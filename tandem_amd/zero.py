@@ -53,13 +53,22 @@ class _Range:
 class ZeRO(torch.nn.Module):
     """Stages 1 and 2."""
 
-    def __init__(self, module, group, stage=1, optimizer=None, bucket_bytes=25 << 20, direct=False):
+    def __init__(self, module, group, stage=1, optimizer=None, bucket_bytes=25 << 20, direct=False, fused_step=False):
         """direct: the flat parameter buffer and the gradient buffer (stage 2: one
         staging buffer the size of the model, kept, instead of one per bucket that is
         dropped) live in the group's shared arena (created here if the group has none:
         twice the model, under 2 GiB), and every collective runs arena to arena
         (`direct=True` of tandem_amd.Group): same bits, fewer passes over memory, no
-        slots."""
+        slots.
+
+        fused_step (stage 2 with direct): backward only packs the gradients; step()
+        is then ONE launch per rank (`group.zero2_step`) that folds this rank's shard
+        out of every rank's gradients in the ring's order, takes the AdamW step and
+        writes the new parameters into every rank's buffer: the reduce_scatters,
+        `grad_shard.add_`, the update and the all_gather in one pass, same bits.
+        `grad_shard` is then only filled when a second backward comes before step()
+        (accumulation): that backward first reduces the packed gradients the ordinary
+        way, and the step after it is the ordinary one."""
         super().__init__()
         if stage not in (1, 2):
             raise ValueError("ZeRO handles stages 1 and 2; stage 3 is FSDP")
@@ -69,6 +78,15 @@ class ZeRO(torch.nn.Module):
         self.module, self.g, self.stage = module, group, stage
         self.direct = bool(direct)
         self.opt = optimizer if optimizer is not None else ShardedAdamW()
+        self.fused_step = bool(fused_step)
+        if self.fused_step:
+            if stage != 2 or not direct:
+                raise ValueError("fused_step needs stage=2 and direct=True")
+            _need(group, "zero2_step")
+            if not hasattr(self.opt, "begin_step"):
+                raise TypeError("fused_step needs an optimizer with begin_step() (tandem_amd.ShardedAdamW has it)")
+        self._packed = False      # fused_step: a whole backward's gradients lie packed in the pool, not yet reduced
+        self._shard_zero = True   # nothing has been added to grad_shard since zero_grad()
         params = [p for p in module.parameters() if p.requires_grad]
         self.params = params
         dev, dtype = params[0].device, params[0].dtype
@@ -120,12 +138,16 @@ class ZeRO(torch.nn.Module):
                 rng.loose = []
             rng.work = self.g.all_reduce(self.grad[rng.a:rng.b], op="avg", async_op=True, **self._how)
         else:
+            if self._packed:
+                self._reduce_packed()  # accumulation: the previous backward's gradients, before they are overwritten
             p0 = rng.params[0]
             rng.staging = (self._pool[rng.a:rng.b] if self.direct
                            else torch.empty(rng.b - rng.a, device=p0.device, dtype=p0.dtype))
             self.g.pack(rng.staging, [(self.offset[p] - rng.a, p.grad) for p in rng.params])
             for p in rng.params:
                 p.grad = None  # the full-size gradient is not kept
+            if self.fused_step and self._shard_zero:
+                return  # step() reduces, updates and gathers in one launch
             rng.work = self.g.reduce_scatter(rng.staging, self.flat.bucket_sizes(rng.a, rng.b), op="avg", async_op=True,
                                              **self._how, **self._mine_only)
 
@@ -148,19 +170,43 @@ class ZeRO(torch.nn.Module):
         self._callback_queued = False
         if any(r.arrived != len(r.params) for r in self.buckets):
             raise RuntimeError("tandem ZeRO: every parameter must receive a gradient")
+        if self.fused_step and self._shard_zero:
+            for rng in self.buckets:
+                rng.arrived, rng.staging = 0, None
+            self._cursor, self._packed = 0, True
+            return
         for rng in self.buckets:
             mine = rng.work.wait()
             if self.stage == 2:
-                if mine.numel():
-                    at = max(rng.a, self.flat.lo) - self.flat.lo
-                    self.grad_shard[at:at + mine.numel()].add_(mine)
+                self._add_mine(rng, mine)
                 rng.staging = None
             rng.arrived, rng.work = 0, None
         self._cursor = 0
 
+    def _add_mine(self, rng, mine):
+        if mine.numel():
+            at = max(rng.a, self.flat.lo) - self.flat.lo
+            self.grad_shard[at:at + mine.numel()].add_(mine)
+        self._shard_zero = False
+
+    @torch.no_grad()
+    def _reduce_packed(self):
+        """fused_step: what backward would have done bucket by bucket, for gradients
+        that were only packed."""
+        works = [self.g.reduce_scatter(self._pool[r.a:r.b], self.flat.bucket_sizes(r.a, r.b), op="avg", async_op=True, direct=True)
+                 for r in self.buckets]
+        for rng, work in zip(self.buckets, works):
+            self._add_mine(rng, work.wait())
+        self._packed = False
+
     @torch.no_grad()
     def step(self):
         lo, hi = self.flat.lo, self.flat.hi
+        if self._packed:
+            scalars, exp_avg, exp_avg_sq, order = self.opt.begin_step("flat", self.buf[lo:hi])
+            self.g.zero2_step(self.buf, self._pool, self.flat.sizes, exp_avg, exp_avg_sq, scalars, order, op="avg")
+            self._packed = False
+            return
         grad = self.grad[lo:hi] if self.stage == 1 else self.grad_shard
         self.opt.update("flat", self.buf[lo:hi], grad)
         self.g.all_gather(self.buf, self.flat.sizes, **self._how)
@@ -180,7 +226,10 @@ class ZeRO(torch.nn.Module):
             for p in self.params:
                 p.grad = None
         else:
-            self.grad_shard.zero_()
+            self._packed = False  # packed gradients not yet reduced are dropped with the rest
+            if not self._shard_zero:
+                self.grad_shard.zero_()
+            self._shard_zero = True
 
 
 def _pad(n):

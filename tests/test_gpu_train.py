@@ -40,7 +40,8 @@ def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1):
     text = synthetic(20_000)
     model = GPT(c).to(g.device)
     extra = {}
-    # a trailing "d": buckets and flat buffers in the shared arenas, collectives arena to arena
+    # a trailing "d": buckets and flat buffers in the shared arenas, collectives arena to arena;
+    # "f": that, and ZeRO-2's reduce-scatters, update and all-gather as one launch per rank
     if strategy.startswith("ddp"):
         z = DDP(model, g, bucket_bytes=bucket_bytes, direct=strategy.endswith("d"))
         opt = torch.optim.AdamW(model.parameters(), lr=LR, weight_decay=WD, foreach=False, fused=False)
@@ -48,8 +49,8 @@ def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1):
         sopt = ShardedAdamW(lr=LR, weight_decay=WD, order="device")  # torch's GPU op order, to compare with torch.optim.AdamW
         stage = int(strategy[4])
         if stage < 3:
-            z = ZeRO(model, g, stage, sopt, bucket_bytes, direct=strategy.endswith("d"))
-            assert z.direct == strategy.endswith("d")
+            z = ZeRO(model, g, stage, sopt, bucket_bytes, direct=strategy[-1] in "df", fused_step=strategy.endswith("f"))
+            assert z.direct == (strategy[-1] in "df") and z.fused_step == strategy.endswith("f")
         else:  # "zero3": shards in the shared arena, gathered directly; "zero3s": staged through the slots
             z = FSDP(model, g, sopt, direct=not strategy.endswith("s"))
             assert z._direct == (not strategy.endswith("s"))
@@ -57,7 +58,7 @@ def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1):
     for step in range(steps):
         for micro in range(accumulate):
             x, y = text.batch(step * accumulate + micro, batch, c.seq, rank=g.rank, world=g.size, device=g.device)
-            if micro < accumulate - 1:  # DDP only: accumulate locally, reduce with the last micro-batch
+            if micro < accumulate - 1 and strategy.startswith("ddp"):  # accumulate locally, reduce with the last micro-batch
                 with z.no_sync():
                     loss = z(x, y)
                     (loss / accumulate).backward()
@@ -115,7 +116,7 @@ def test_two_ranks_all_strategies_agree_bit_for_bit():
     from tandem_amd import launch
 
     runs = {s: launch(train_rank, 2, s, 4 << 10, STEPS, BATCH, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT)
-            for s in ("ddp", "ddpd", "zero1", "zero1d", "zero2", "zero2d", "zero3", "zero3s")}
+            for s in ("ddp", "ddpd", "zero1", "zero1d", "zero2", "zero2d", "zero2f", "zero3", "zero3s")}
     ref_losses, ref_w = one_process(2)
     for s, res in runs.items():
         assert torch.equal(res[0]["weights"], res[1]["weights"]), f"{s}: the ranks drifted apart"
@@ -134,7 +135,7 @@ def test_four_ranks_stay_in_step():
     from tandem_amd import launch
 
     kept = {}
-    for s in ("ddp", "ddpd", "zero1", "zero1d", "zero2", "zero2d", "zero3", "zero3s"):
+    for s in ("ddp", "ddpd", "zero1", "zero1d", "zero2", "zero2d", "zero2f", "zero3", "zero3s"):
         res = launch(train_rank, 4, s, 4 << 10, 6, 8, slot_bytes=1024, gpus=[0] * 4, timeout=TIMEOUT)
         kept[s] = res[0]
         for r in range(1, 4):
@@ -145,7 +146,7 @@ def test_four_ranks_stay_in_step():
         if s.startswith("zero3"):
             assert all(x["max_live"] <= 3 and x["live"] == 0 for x in res)
     # arena to arena or through the slots: the same sums in the same order, so the same bits
-    for direct, ring in (("ddpd", "ddp"), ("zero2d", "zero2"), ("zero1d", "zero1")):
+    for direct, ring in (("ddpd", "ddp"), ("zero2d", "zero2"), ("zero2f", "zero2"), ("zero1d", "zero1")):
         assert kept[direct]["losses"] == kept[ring]["losses"], direct
         assert torch.equal(kept[direct]["weights"], kept[ring]["weights"]), direct
 
@@ -163,6 +164,21 @@ def test_gradient_accumulation_matches_one_process():
             assert torch.equal(res[r]["weights"], ref_w), (s, r)
 
 
+def test_zero2_accumulation_with_and_without_the_fused_step():
+    """ZeRO-2 accumulates by reducing every backward into the gradient shard. With
+    fused_step the first backward is only packed; the second one must first reduce it
+    the ordinary way, and the step after is the ordinary one: the same bits as without,
+    at two ranks and (where the ring's order matters) at four."""
+    from tandem_amd import launch
+
+    for world, slot in ((2, 4096), (4, 1024)):
+        runs = {s: launch(train_rank, world, s, 4 << 10, 4, 8, 2, slot_bytes=slot, gpus=[0] * world, timeout=TIMEOUT)
+                for s in ("zero2", "zero2d", "zero2f")}
+        for s in ("zero2d", "zero2f"):
+            for r in range(world):
+                assert runs[s][r]["losses"] == runs["zero2"][r]["losses"], (world, s, r)
+                assert torch.equal(runs[s][r]["weights"], runs["zero2"][0]["weights"]), (world, s, r)
+
 
 def test_stream_ordered_wait_gives_the_same_weights(monkeypatch):
     """TANDEM_HIP_WAIT=stream: wait() parks the training stream on a word the engine sets
@@ -171,7 +187,7 @@ def test_stream_ordered_wait_gives_the_same_weights(monkeypatch):
 
     monkeypatch.setenv("TANDEM_HIP_WAIT", "stream")
     ref_losses, ref_w = one_process(2)
-    for s in ("ddp", "ddpd", "zero2", "zero3"):
+    for s in ("ddp", "ddpd", "zero2", "zero2f", "zero3"):
         res = launch(train_rank, 2, s, 4 << 10, STEPS, BATCH, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT)
         for r in range(2):
             assert res[r]["losses"] == ref_losses[r], (s, r)

@@ -249,3 +249,50 @@ def test_one_launch_step_through_the_c_abi(world, average):
                 assert np.array_equal(bits(params[r].cpu().numpy()), bits(want_p)), what + (r,)
             assert np.array_equal(bits(m.cpu().numpy()), bits(want_m)), what
             assert np.array_equal(bits(v.cpu().numpy()), bits(want_v)), what
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_one_segment_in_the_launch_equals_the_table(world):
+    """tdm_k23_zero2_step_segment (the segment travels in the kernel's arguments: what a
+    process rank runs over its shard) against tdm_k23_zero2_step over a one-row table,
+    which the test above pins to the oracle: same bits in every buffer, aligned and not,
+    sum and average, both orders."""
+    import ctypes
+
+    from tandem_amd import _lib
+    from tandem_amd._lib import check, lib, stream_ptr
+    from tandem_amd.optim import step_scalars
+
+    dev = torch.device("cuda", 0)
+    n = 3 * 4096 + 1031
+    for shift, average, order, chunk in ((0, 1, _lib.ADAMW_HOST_ORDER, world - 1), (1, 0, _lib.ADAMW_DEVICE_ORDER, 0),
+                                         (0, 0, _lib.ADAMW_HOST_ORDER, world // 2), (3, 1, _lib.ADAMW_DEVICE_ORDER, world // 3)):
+        grads = [(seeded(70 + shift, r, n + 8) * 1e-3).to(dev) for r in range(world)]
+        p0 = (seeded(71, 0, n + 8) * 0.02).to(dev)
+        results = []
+        for entry in ("table", "segment"):
+            params = [p0.clone() for _ in range(world)]
+            m, v = torch.zeros(n + 8, device=dev), torch.zeros(n + 8, device=dev)
+            seg = (_lib.StepSeg * 1)()
+            for r in range(world):
+                seg[0].grad[r] = grads[r].data_ptr() + shift * 4
+                seg[0].param[r] = params[r].data_ptr() + shift * 4
+            seg[0].exp_avg, seg[0].exp_avg_sq = m.data_ptr() + shift * 4, v.data_ptr() + shift * 4
+            seg[0].count, seg[0].chunk = n, chunk
+            if entry == "table":
+                ntiles = lib().tdm_k23_table_tiles(seg, 1)
+                image = torch.empty(lib().tdm_k23_table_bytes(seg, 1), dtype=torch.uint8)
+                check(lib().tdm_k23_table_build(seg, 1, world, ctypes.c_void_p(image.data_ptr())))
+                table = image.to(dev)
+            for step in (1.0, 2.0):
+                s = step_scalars(step, KW["lr"], KW["betas"], KW["eps"], KW["weight_decay"])
+                if entry == "table":
+                    check(lib().tdm_k23_zero2_step(ctypes.c_void_p(table.data_ptr()), ntiles, world, average, ctypes.byref(s), order,
+                                                   stream_ptr(dev)))
+                else:
+                    check(lib().tdm_k23_zero2_step_segment(seg, world, average, ctypes.byref(s), order, stream_ptr(dev)))
+            torch.cuda.synchronize(dev)
+            results.append([t.cpu() for t in params + [m, v]])
+        for a, b in zip(*results):
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (world, shift, average, order)
+        assert not torch.equal(results[0][0], p0.cpu())  # the step did happen
