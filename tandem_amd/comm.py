@@ -296,7 +296,7 @@ class Group:
                 raise CommError(f"zero2_step: {name} must be this rank's shard ({n} fp32 elements on {self.device})")
         bases = []
         for t in (p, g):
-            off = self.arena_offset(t)
+            off = self.arena_offset(t) if t.numel() else 0  # empty buffers: nothing to read, but the ranks still meet
             if off is None:
                 raise CommError("zero2_step: the buffers must come from shared_empty()")
             bases.append((ctypes.c_int64 * self.size)(*[off + lo * 4] * self.size))

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import bits, golden_npz, npz_json
+from helpers import bits, golden_npz, npz_json, seeded
 
 pytestmark = pytest.mark.gpu
 
@@ -354,6 +354,73 @@ def test_direct_collectives_bit_exact(dtype, world):
     xs = [to_np(values(q, 1000, dtype)) for q in range(world)]
     for out in res:
         assert np.array_equal(bits(to_np(out["ar_same"])), bits(ring.expected_all_reduce(xs, False, kind)))
+
+
+def zero2_steps(g, ns, steps):
+    """Group.zero2_step on flat buffers in the arenas: gradients differ per rank and step,
+    parameters start equal; returns this rank's parameter buffer and optimizer state."""
+    from tandem_amd import CommError, ShardedAdamW
+    from tandem_amd.optim import step_scalars
+
+    dev, w, r = g.device, g.size, g.rank
+    g.share_arena(8 << 20)
+    out = {}
+    for n in ns:
+        sizes = [n // w + (1 if q < n % w else 0) for q in range(w)]
+        lo = sum(sizes[:r])
+        params, grads = g.shared_empty(n), g.shared_empty(n)
+        params.copy_(seeded(3, 0, n) * 0.02)
+        opt = ShardedAdamW(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+        for step in range(steps):
+            grads.copy_(seeded(100 + step, r, n) * 1e-3)
+            scalars, m, v, order = opt.begin_step("flat", params[lo:lo + sizes[r]])
+            got = g.zero2_step(params, grads, sizes, m, v, scalars, order)
+            assert got is params
+        out[n] = (params.cpu(), m.cpu(), v.cpu())
+    # what it refuses
+    n = 1000
+    sizes = [n // w + (1 if q < n % w else 0) for q in range(w)]
+    arena, plain = g.shared_empty(n), torch.zeros(n, device=dev)
+    state = torch.zeros(sizes[r], device=dev)
+    s = step_scalars(1.0, 3e-4, (0.9, 0.95), 1e-8, 0.1)
+    refused = 0
+    for p_, g_, m_, sz in ((plain, arena, state, sizes), (arena, plain, state, sizes), (arena, arena, torch.zeros(sizes[r] + 1, device=dev), sizes),
+                           (arena, arena, state, sizes[:-1]), (arena.double(), arena, state, sizes)):
+        try:
+            g.zero2_step(p_, g_, sz, m_, m_.clone(), s, 0)
+        except CommError:
+            refused += 1
+    out["refused"] = refused
+    return out
+
+
+@pytest.mark.parametrize("world", [2, 3, 4])
+def test_zero2_step_in_one_launch_per_rank(world):
+    """Every rank's parameters after the fused step equal the oracle's reduce-scatter,
+    `0 + mine`, AdamW per shard and all-gather; each rank's state equals its shard's."""
+    from oracle import ring
+    from oracle.adamw import AdamW
+    from tandem_amd import launch
+
+    ns, steps = (0, 3, 1001, 40_007), 3
+    res = launch(zero2_steps, world, ns, steps, gpus=[0] * world, timeout=TIMEOUT)
+    for n in ns:
+        sizes = [n // world + (1 if q < n % world else 0) for q in range(world)]
+        want = (seeded(3, 0, n) * 0.02).numpy()
+        opts = [AdamW(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1) for _ in range(world)]
+        for step in range(steps):
+            xs = [(seeded(100 + step, q, n) * 1e-3).numpy() for q in range(world)]
+            outs = ring.expected_reduce_scatter(xs, sizes, True)
+            for q in range(world):
+                lo = sum(sizes[:q])
+                opts[q].update("flat", want[lo:lo + sizes[q]], np.float32(0.0) + outs[q][lo:lo + sizes[q]])
+        for r, out in enumerate(res):
+            p, m, v = out[n]
+            assert np.array_equal(bits(p.numpy()), bits(want)), (world, n, r)
+            if sizes[r]:
+                assert np.array_equal(bits(m.numpy()), bits(opts[r].state["flat"][1])), (world, n, r)
+                assert np.array_equal(bits(v.numpy()), bits(opts[r].state["flat"][2])), (world, n, r)
+    assert all(out["refused"] == 5 for out in res)
 
 
 def async_order(g):
