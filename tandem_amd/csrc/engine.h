@@ -1,0 +1,241 @@
+// The process-rank engine's types: Work handles and the Engine itself (see engine.hip).
+#pragma once
+
+#include "engine_shm.h"
+
+namespace tandem_hip {
+
+// ---------------------------------------------------------------- Work
+// A point that is known on both clocks: the event was recorded on the engine's
+// stream and waited for, and `host` was read right after.
+struct Anchor {
+  hipEvent_t event = nullptr;
+  double host = 0;
+  ~Anchor() {
+    if (event) (void)hipEventDestroy(event);
+  }
+};
+
+// Words in pinned host memory that a GPU stream can wait on (hipStreamWaitValue32) and
+// that either the engine's stream (hipStreamWriteValue32) or the host sets: how
+// wait() can order the caller's stream behind a collective whose launches the progress
+// thread has not even made yet. Shared by the engine and its Works, freed by the last.
+struct FlagPool {
+  static constexpr int kFlags = 1024;
+  uint32_t* base = nullptr;
+  std::mutex mu;
+  std::vector<int> free_list;
+  std::vector<uint32_t> generation;  // a word only ever grows: a stream still parked on an earlier
+                                     // generation of it is let go by every later one as well
+
+  static std::shared_ptr<FlagPool> make() {
+    auto p = std::make_shared<FlagPool>();
+    check_hip(hipHostMalloc(reinterpret_cast<void**>(&p->base), kFlags * sizeof(uint32_t), hipHostMallocDefault), "hipHostMalloc (flags)");
+    std::memset(p->base, 0, kFlags * sizeof(uint32_t));
+    p->generation.assign(kFlags, 0);
+    for (int i = kFlags - 1; i >= 0; --i) p->free_list.push_back(i);
+    return p;
+  }
+  ~FlagPool() {
+    if (base) (void)hipHostFree(base);
+  }
+  // A word and the value its owner will wait for; -1: none left (the Work then waits on the host as usual).
+  int acquire(uint32_t* value) {
+    std::lock_guard<std::mutex> lock(mu);
+    if (free_list.empty()) return -1;
+    const int i = free_list.back();
+    free_list.pop_back();
+    *value = ++generation[i];
+    return i;
+  }
+  void release(int i) {
+    std::lock_guard<std::mutex> lock(mu);
+    free_list.push_back(i);
+  }
+  void set(int i, uint32_t value) {
+    reinterpret_cast<volatile uint32_t*>(base)[i] = value;
+    std::atomic_thread_fence(std::memory_order_seq_cst);
+  }
+};
+
+struct Work {
+  std::mutex mu;
+  std::condition_variable cv;
+  bool finished = false;   // the job has run (all its GPU work is enqueued)
+  std::atomic<bool> finished_hint{false};  // set after `finished`: lets a waiter poll before it sleeps
+  int status = TDM_OK;
+  std::string error;
+  double t0 = 0, t1 = 0;
+  hipEvent_t done_event = nullptr;  // recorded on the engine's stream after the job (jobs with GPU work)
+  bool uses_gpu = false;
+  bool on_callers_stream = false;  // its kernels were launched on the submitting stream itself:
+  hipStream_t launched_on = nullptr;  // wait() from that stream has nothing to order
+  bool drained = false;  // the job ends with a fence: the engine's stream is idle when it has run
+  int device = -1;
+  // Device timing (only while the engine's timing switch is on): start_event is
+  // recorded on the engine's stream once the inputs are ready; both events carry
+  // time stamps, placed on the host clock through the engine's anchor.
+  hipEvent_t start_event = nullptr;
+  std::shared_ptr<Anchor> anchor;
+  // Stream-ordered waiting (TANDEM_HIP_WAIT=stream): the word the caller's stream waits for.
+  std::shared_ptr<FlagPool> flags;
+  int flag = -1;
+  uint32_t flag_value = 0;  // the word reaches this value when the collective is over
+
+  ~Work() {
+    if (done_event) (void)hipEventDestroy(done_event);
+    if (start_event) (void)hipEventDestroy(start_event);
+    if (flags && flag >= 0) {
+      if (!finished) flags->set(flag, flag_value);  // the job never ran: nobody may stay parked on the word
+      flags->release(flag);
+    }
+  }
+};
+
+
+// ---------------------------------------------------------------- Engine
+class Engine {
+ public:
+  Engine(const std::string& job, int rank, int size, int slots, size_t slot_bytes, double timeout_s, int device);
+  ~Engine();
+  void connect();
+  void close();
+  void set_timing(bool on) { timing_.store(on ? 1 : 0, std::memory_order_release); }
+
+  struct Buf {
+    char* ptr;
+    int64_t numel;
+    int dtype;
+  };
+
+  std::shared_ptr<Work> all_reduce(Buf t, bool average, hipStream_t caller);
+  std::shared_ptr<Work> reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, bool owner_only, hipStream_t caller);
+  std::shared_ptr<Work> all_gather(Buf t, std::vector<int64_t> sizes, hipStream_t caller);
+  std::shared_ptr<Work> unit_gather(Buf full, const char* shard, std::vector<int64_t> sizes, hipStream_t caller);
+  std::shared_ptr<Work> broadcast(Buf t, int root, hipStream_t caller);
+  std::shared_ptr<Work> sendrecv(Buf send, int dst, Buf recv, int src, hipStream_t caller);
+  std::shared_ptr<Work> barrier();
+  std::shared_ptr<Work> fence(hipStream_t caller);
+  void* share(size_t bytes);
+  std::shared_ptr<Work> unit_gather_direct(Buf full, const char* shard, std::vector<int64_t> sizes,
+                                           std::vector<int64_t> peer_offsets, hipStream_t caller);
+  // kind 0: all_reduce, 1: reduce_scatter (the owner's chunk only), 2: all_gather
+  std::shared_ptr<Work> direct(int kind, Buf t, std::vector<int64_t> sizes, bool average, std::vector<int64_t> peer_offsets,
+                               hipStream_t caller);
+
+  std::shared_ptr<Work> zero2_step_direct(Buf param, Buf grad, std::vector<int64_t> param_offsets, std::vector<int64_t> grad_offsets,
+                                          char* exp_avg, char* exp_avg_sq, int64_t total, bool average, tdm_adamw_scalars s,
+                                          int order, hipStream_t caller);
+
+  int device() const { return device_; }
+  hipStream_t stream() const { return stream_; }
+  int rank() const { return rank_; }
+  int size() const { return size_; }
+
+ private:
+  struct Chunk {
+    char* ptr;
+    int64_t numel;
+  };
+
+  std::shared_ptr<Work> submit(std::function<void()> job, hipStream_t caller, bool uses_gpu, bool host_ready = false,
+                               bool drained = false);
+  void stamp_start(Work& w, hipStream_t on);
+  char* staging_half();
+  const char* peer_staging(int peer, int half);
+  void copy_pairs(const tdm_pair* pairs, int np, int dtype);
+  void staged_all_reduce(const Buf& t, bool average);
+  void staged_all_reduce_small(const Buf& t, bool average);
+  void staged_all_gather(const Buf& t, const std::vector<Chunk>& cs, const char* own);
+  void staged_reduce_scatter_owner(const Buf& t, const std::vector<Chunk>& cs, bool average);
+  void direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets, const char** base);
+  void direct_fold(const Buf& t, const std::vector<Chunk>& cs, const char* const* base, bool average);
+  void direct_copies(const Buf& t, const std::vector<Chunk>& cs, const char* const* base);
+  void start();
+  void release_device();
+  void loop();
+  void check(const Buf& t, const char* what, bool reduce) const;
+  std::vector<Chunk> chunks(const Buf& t, const std::vector<int64_t>& sizes) const;
+  int64_t piece_elems(int dtype) const { return std::max<int64_t>(1, static_cast<int64_t>(slot_bytes_) / elem_bytes(dtype)); }
+
+  void put(int dst, const char* src, int64_t numel, int dtype, int scale_world);
+  void take(int src, char* into, int64_t numel, int dtype, bool reduce, int scale_world);
+  void exchange(const Chunk* send, int dst, const Chunk* recv, int src, int dtype, bool reduce, int put_scale,
+                int take_scale);
+  void ring_reduce_scatter(const std::vector<Chunk>& c, int dtype, bool average, bool keep_sent);
+  void ring_all_gather(const std::vector<Chunk>& c, int dtype);
+  void signal(int dst, uint64_t length);
+  uint64_t await(int src);
+  void release(int src);
+  void barrier_now(bool after_gpu = false, uint64_t tag = 0);
+  const char* peer_arena(int peer, size_t need_bytes);
+
+  std::string region_name(int rank) const { return "/tandem-" + job_ + "-" + std::to_string(rank) + "-hip"; }
+
+  std::string job_;
+  int rank_, size_, slots_;
+  size_t slot_bytes_;
+  double timeout_s_;
+  int device_;
+  bool use_events_;
+  hipStream_t stream_ = nullptr;
+  hipStream_t gather_stream_ = nullptr;  // direct unit gathers, launched by the caller's thread
+  hipStream_t anchor_stream_ = nullptr;  // carries nothing but the timing anchors: always idle
+  std::mutex anchor_mu_, arena_mu_;      // both threads time their work and map peers' arenas
+  Region mine_;
+  std::vector<std::unique_ptr<Region>> theirs_;
+  std::vector<void*> out_mem_, peer_mem_;
+  void* arena_ = nullptr;
+  size_t arena_bytes_ = 0;
+  std::vector<void*> peer_arena_;
+  std::vector<size_t> peer_arena_bytes_;
+  std::vector<std::vector<hipEvent_t>> full_, free_, peer_full_, peer_free_;
+  std::vector<uint64_t> sent_, got_;     // pieces, per peer: pick the slot
+  std::vector<uint64_t> posted_;         // messages queued or published to each peer (flow control)
+  std::vector<uint64_t> taken_;          // messages consumed from each peer
+  bool connected_ = false, closed_ = false;
+  // staged collectives
+  bool staged_ = true;               // TANDEM_HIP_ALGO=ring switches them off
+  bool gathers_on_side_stream_ = false;  // TANDEM_HIP_GATHER=stream
+  std::shared_ptr<FlagPool> flags_;      // TANDEM_HIP_WAIT=stream
+  bool want_flags_ = false;
+  std::string sticky_error_;             // under mu_: a collective failed after its wait() had already returned
+  bool ready_on_host_ = true;        // TANDEM_HIP_READY=gpu: wait for the caller's stream on the GPU instead
+  size_t staging_half_ = 64u << 20;  // bytes per half (TANDEM_HIP_STAGING_BYTES)
+  size_t small_bytes_ = 32u << 20;   // all_reduce up to this size takes the one-handshake form (TANDEM_HIP_SMALL_BYTES)
+  void* staging_ = nullptr;
+  std::vector<void*> peer_staging_;
+  uint64_t staged_ops_ = 0;          // picks the half; the same count on every rank
+  std::atomic<int> timing_{0};
+  bool timing_seen_ = false;           // under anchor_mu_
+  std::shared_ptr<Anchor> anchor_;     // under anchor_mu_
+
+  // "host" ordering: what to publish once the GPU has passed an event.
+  struct Completion {
+    hipEvent_t after;  // nullptr: publish at once (still in order)
+    bool is_release;
+    int peer;
+    uint64_t length;
+  };
+  void complete_later(bool is_release, int peer, uint64_t length, bool after_stream);
+  void completion_loop();
+  void drain_completions();
+  std::mutex cmu_;
+  std::condition_variable ccv_, cidle_;
+  std::deque<Completion> completions_;
+  bool cstop_ = false, cbusy_ = false;
+  std::atomic<uint64_t> cqueued_{0};  // completions ever queued
+  uint64_t cdone_ = 0;                // completions ever taken (completion thread, under cmu_)
+  std::string cerror_;
+  std::thread completer_;
+
+  std::mutex mu_;
+  std::condition_variable cv_;
+  std::deque<std::pair<std::function<void()>, std::shared_ptr<Work>>> jobs_;
+  std::atomic<uint64_t> submitted_{0};  // jobs ever queued
+  uint64_t started_ = 0;                // jobs ever taken (progress thread only)
+  bool stopping_ = false;
+  std::thread thread_;
+};
+
+}  // namespace tandem_hip

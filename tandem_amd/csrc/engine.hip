@@ -34,441 +34,9 @@
 // last hand-over has happened on the GPU, and tdm_work_wait, which waits for the
 // job to be enqueued, returns about when the collective's last kernel starts.
 
-#include <fcntl.h>
-#include <sys/mman.h>
-#include <sys/stat.h>
-#include <unistd.h>
-
-#include <atomic>
-#include <chrono>
-#include <condition_variable>
-#include <cstdlib>
-#include <cstring>
-#include <deque>
-#include <functional>
-#include <memory>
-#include <mutex>
-#include <new>
-#include <thread>
-#include <vector>
-
-#include "common.h"
+#include "engine.h"
 
 namespace tandem_hip {
-
-namespace {
-
-double now_s() {
-  return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
-}
-
-int mod(int a, int n) { return ((a % n) + n) % n; }
-
-constexpr int kBytesDtype = 6;  // TDM_U8 in spirit: copies only
-
-// Messages: a piece's length in bytes, or (top bit set) a barrier with a tag in the low bits.
-constexpr uint64_t kNoPiece = uint64_t(1) << 63;
-constexpr uint64_t fence_tag(int kind, int dtype, int64_t numel) {
-  return (static_cast<uint64_t>(kind) << 56) | (static_cast<uint64_t>(dtype) << 48) | (static_cast<uint64_t>(numel) & ((uint64_t(1) << 48) - 1));
-}
-
-int elem_bytes(int dtype) {
-  switch (dtype) {
-    case TDM_F32: case TDM_I32: return 4;
-    case TDM_F64: case TDM_I64: return 8;
-    case TDM_F16: case TDM_BF16: return 2;
-    case kBytesDtype: return 1;
-    default: throw Invalid("unknown dtype " + std::to_string(dtype));
-  }
-}
-
-// ---------------------------------------------------------------- shared region
-constexpr uint64_t kRegionMagic = 0x74646d4849503031ull;  // "tdmHIP01"
-constexpr size_t kLine = 64;
-constexpr int kMaxSlots = 16;
-
-static_assert(std::atomic<uint64_t>::is_always_lock_free, "atomics shared between processes must be lock-free");
-
-// One direction of one pair, written by the owner of the region (the sender):
-// message k says slot k % slots holds `length[k % slots]` bytes.
-struct alignas(kLine) Ring {
-  alignas(kLine) std::atomic<uint64_t> head;  // messages published, advanced by the sender
-  alignas(kLine) std::atomic<uint64_t> tail;  // messages released, advanced by the receiver
-  alignas(kLine) uint64_t length[kMaxSlots];
-};
-
-struct alignas(kLine) PeerEntry {
-  hipIpcMemHandle_t mem;               // the sender's slots for this peer
-  hipIpcEventHandle_t full[kMaxSlots];  // sender recorded: slot j holds a piece
-  hipIpcEventHandle_t free_[kMaxSlots]; // owner recorded: it finished reading THE PEER's slot j to the owner
-  Ring ring;
-};
-
-struct alignas(kLine) RegionHeader {
-  uint64_t magic;
-  int32_t rank, size, device, slots;
-  uint64_t slot_bytes;
-  int64_t pid;
-  int32_t use_events;
-  int32_t reserved;
-  // A rank's shared arena (tdm_engine_share): device memory its peers may read directly.
-  std::atomic<uint64_t> arena_bytes;  // 0 until published
-  hipIpcMemHandle_t arena_mem;
-  // The engine's own staging memory for the staged collectives (two halves, used in turn).
-  std::atomic<uint64_t> staging_bytes;  // 0 until published
-  hipIpcMemHandle_t staging_mem;
-};
-
-class Region {
- public:
-  Region() = default;
-  ~Region() { reset(); }
-  Region(const Region&) = delete;
-  Region& operator=(const Region&) = delete;
-
-  static size_t bytes_for(int size) { return sizeof(RegionHeader) + static_cast<size_t>(size) * sizeof(PeerEntry); }
-
-  void create(const std::string& name, int size) {
-    reset();
-    name_ = name;
-    bytes_ = bytes_for(size);
-    ::shm_unlink(name.c_str());  // a stale region from a crashed run with the same job name
-    int fd = ::shm_open(name.c_str(), O_CREAT | O_EXCL | O_RDWR, 0600);
-    if (fd < 0) throw std::runtime_error("shm_open(" + name + "): " + std::strerror(errno));
-    if (::ftruncate(fd, static_cast<off_t>(bytes_)) != 0) {
-      ::close(fd);
-      ::shm_unlink(name.c_str());
-      throw std::runtime_error("ftruncate(" + name + "): " + std::strerror(errno));
-    }
-    map(fd);
-    owner_ = true;
-    std::memset(data_, 0, bytes_);
-    for (int p = 0; p < size; ++p) new (&entry(p)->ring) Ring();
-  }
-
-  void open(const std::string& name, int size) {
-    reset();
-    name_ = name;
-    bytes_ = bytes_for(size);
-    int fd = ::shm_open(name.c_str(), O_RDWR, 0600);
-    if (fd < 0) throw std::runtime_error("shm_open(" + name + "): " + std::strerror(errno));
-    struct stat st;
-    if (::fstat(fd, &st) != 0 || static_cast<size_t>(st.st_size) < bytes_) {
-      ::close(fd);
-      throw std::runtime_error("region " + name + " is smaller than expected");
-    }
-    map(fd);
-  }
-
-  RegionHeader* header() const { return static_cast<RegionHeader*>(data_); }
-  PeerEntry* entry(int peer) const {
-    return reinterpret_cast<PeerEntry*>(static_cast<char*>(data_) + sizeof(RegionHeader)) + peer;
-  }
-  bool mapped() const { return data_ != nullptr; }
-
-  void reset() {
-    if (data_) ::munmap(data_, bytes_);
-    if (owner_) ::shm_unlink(name_.c_str());
-    data_ = nullptr;
-    owner_ = false;
-  }
-
- private:
-  void map(int fd) {
-    void* p = ::mmap(nullptr, bytes_, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
-    ::close(fd);
-    if (p == MAP_FAILED) throw std::runtime_error("mmap(" + name_ + "): " + std::strerror(errno));
-    data_ = p;
-  }
-
-  std::string name_;
-  void* data_ = nullptr;
-  size_t bytes_ = 0;
-  bool owner_ = false;
-};
-
-// A wake-up through a condition variable costs 10-20 us; whoever expects news within
-// that time polls for it first.
-constexpr auto kSpinBeforeSleep = std::chrono::microseconds(100);
-
-template <class Ready>
-bool spin_for(Ready ready, std::chrono::microseconds limit = kSpinBeforeSleep) {
-  const auto until = std::chrono::steady_clock::now() + limit;
-  for (int i = 0;; ++i) {
-    if (ready()) return true;
-    if ((i & 15) == 15 && std::chrono::steady_clock::now() > until) return false;
-    __builtin_ia32_pause();
-  }
-}
-
-// Waiting for the GPU from a helper thread: poll (a query is cheap and takes no lock for
-// long), first tightly, then every 50 us. The runtime's own blocking waits are avoided on
-// purpose: while one thread sat in them for milliseconds, the training thread's kernel
-// launches were seen to stall. `query` returns hipErrorNotReady until the work is done.
-template <class Query>
-hipError_t poll_gpu(Query query, double timeout_s) {
-  hipError_t err = hipErrorNotReady;
-  if (spin_for([&] { return (err = query()) != hipErrorNotReady; }, std::chrono::microseconds(300))) return err;
-  const auto deadline = std::chrono::steady_clock::now() + std::chrono::duration<double>(timeout_s);
-  for (;;) {
-    std::this_thread::sleep_for(std::chrono::microseconds(50));
-    if ((err = query()) != hipErrorNotReady) return err;
-    if (std::chrono::steady_clock::now() > deadline) throw Timeout("timed out waiting for the GPU");
-  }
-}
-
-// Spin, then yield, then short sleeps; throws Timeout.
-template <class Ready>
-void wait_until(Ready ready, double timeout_s, const char* what) {
-  using clock = std::chrono::steady_clock;
-  const auto start = clock::now();
-  const auto deadline = start + std::chrono::duration<double>(timeout_s);
-  for (uint64_t i = 0; !ready(); ++i) {
-    if (i < 256) continue;
-    if ((i & 63) != 0) {
-      std::this_thread::yield();
-      continue;
-    }
-    const auto t = clock::now();
-    if (t > deadline) throw Timeout(what);
-    if (t - start > std::chrono::milliseconds(2)) std::this_thread::sleep_for(std::chrono::microseconds(20));
-  }
-}
-
-}  // namespace
-
-// ---------------------------------------------------------------- Work
-// A point that is known on both clocks: the event was recorded on the engine's
-// stream and waited for, and `host` was read right after.
-struct Anchor {
-  hipEvent_t event = nullptr;
-  double host = 0;
-  ~Anchor() {
-    if (event) (void)hipEventDestroy(event);
-  }
-};
-
-// Words in pinned host memory that a GPU stream can wait on (hipStreamWaitValue32) and
-// that either the engine's stream (hipStreamWriteValue32) or the host sets: how
-// wait() can order the caller's stream behind a collective whose launches the progress
-// thread has not even made yet. Shared by the engine and its Works, freed by the last.
-struct FlagPool {
-  static constexpr int kFlags = 1024;
-  uint32_t* base = nullptr;
-  std::mutex mu;
-  std::vector<int> free_list;
-  std::vector<uint32_t> generation;  // a word only ever grows: a stream still parked on an earlier
-                                     // generation of it is let go by every later one as well
-
-  static std::shared_ptr<FlagPool> make() {
-    auto p = std::make_shared<FlagPool>();
-    check_hip(hipHostMalloc(reinterpret_cast<void**>(&p->base), kFlags * sizeof(uint32_t), hipHostMallocDefault), "hipHostMalloc (flags)");
-    std::memset(p->base, 0, kFlags * sizeof(uint32_t));
-    p->generation.assign(kFlags, 0);
-    for (int i = kFlags - 1; i >= 0; --i) p->free_list.push_back(i);
-    return p;
-  }
-  ~FlagPool() {
-    if (base) (void)hipHostFree(base);
-  }
-  // A word and the value its owner will wait for; -1: none left (the Work then waits on the host as usual).
-  int acquire(uint32_t* value) {
-    std::lock_guard<std::mutex> lock(mu);
-    if (free_list.empty()) return -1;
-    const int i = free_list.back();
-    free_list.pop_back();
-    *value = ++generation[i];
-    return i;
-  }
-  void release(int i) {
-    std::lock_guard<std::mutex> lock(mu);
-    free_list.push_back(i);
-  }
-  void set(int i, uint32_t value) {
-    reinterpret_cast<volatile uint32_t*>(base)[i] = value;
-    std::atomic_thread_fence(std::memory_order_seq_cst);
-  }
-};
-
-struct Work {
-  std::mutex mu;
-  std::condition_variable cv;
-  bool finished = false;   // the job has run (all its GPU work is enqueued)
-  std::atomic<bool> finished_hint{false};  // set after `finished`: lets a waiter poll before it sleeps
-  int status = TDM_OK;
-  std::string error;
-  double t0 = 0, t1 = 0;
-  hipEvent_t done_event = nullptr;  // recorded on the engine's stream after the job (jobs with GPU work)
-  bool uses_gpu = false;
-  bool on_callers_stream = false;  // its kernels were launched on the submitting stream itself:
-  hipStream_t launched_on = nullptr;  // wait() from that stream has nothing to order
-  bool drained = false;  // the job ends with a fence: the engine's stream is idle when it has run
-  int device = -1;
-  // Device timing (only while the engine's timing switch is on): start_event is
-  // recorded on the engine's stream once the inputs are ready; both events carry
-  // time stamps, placed on the host clock through the engine's anchor.
-  hipEvent_t start_event = nullptr;
-  std::shared_ptr<Anchor> anchor;
-  // Stream-ordered waiting (TANDEM_HIP_WAIT=stream): the word the caller's stream waits for.
-  std::shared_ptr<FlagPool> flags;
-  int flag = -1;
-  uint32_t flag_value = 0;  // the word reaches this value when the collective is over
-
-  ~Work() {
-    if (done_event) (void)hipEventDestroy(done_event);
-    if (start_event) (void)hipEventDestroy(start_event);
-    if (flags && flag >= 0) {
-      if (!finished) flags->set(flag, flag_value);  // the job never ran: nobody may stay parked on the word
-      flags->release(flag);
-    }
-  }
-};
-
-
-// ---------------------------------------------------------------- Engine
-class Engine {
- public:
-  Engine(const std::string& job, int rank, int size, int slots, size_t slot_bytes, double timeout_s, int device);
-  ~Engine();
-  void connect();
-  void close();
-  void set_timing(bool on) { timing_.store(on ? 1 : 0, std::memory_order_release); }
-
-  struct Buf {
-    char* ptr;
-    int64_t numel;
-    int dtype;
-  };
-
-  std::shared_ptr<Work> all_reduce(Buf t, bool average, hipStream_t caller);
-  std::shared_ptr<Work> reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, bool owner_only, hipStream_t caller);
-  std::shared_ptr<Work> all_gather(Buf t, std::vector<int64_t> sizes, hipStream_t caller);
-  std::shared_ptr<Work> unit_gather(Buf full, const char* shard, std::vector<int64_t> sizes, hipStream_t caller);
-  std::shared_ptr<Work> broadcast(Buf t, int root, hipStream_t caller);
-  std::shared_ptr<Work> sendrecv(Buf send, int dst, Buf recv, int src, hipStream_t caller);
-  std::shared_ptr<Work> barrier();
-  std::shared_ptr<Work> fence(hipStream_t caller);
-  void* share(size_t bytes);
-  std::shared_ptr<Work> unit_gather_direct(Buf full, const char* shard, std::vector<int64_t> sizes,
-                                           std::vector<int64_t> peer_offsets, hipStream_t caller);
-  // kind 0: all_reduce, 1: reduce_scatter (the owner's chunk only), 2: all_gather
-  std::shared_ptr<Work> direct(int kind, Buf t, std::vector<int64_t> sizes, bool average, std::vector<int64_t> peer_offsets,
-                               hipStream_t caller);
-
-  std::shared_ptr<Work> zero2_step_direct(Buf param, Buf grad, std::vector<int64_t> param_offsets, std::vector<int64_t> grad_offsets,
-                                          char* exp_avg, char* exp_avg_sq, int64_t total, bool average, tdm_adamw_scalars s,
-                                          int order, hipStream_t caller);
-
-  int device() const { return device_; }
-  hipStream_t stream() const { return stream_; }
-  int rank() const { return rank_; }
-  int size() const { return size_; }
-
- private:
-  struct Chunk {
-    char* ptr;
-    int64_t numel;
-  };
-
-  std::shared_ptr<Work> submit(std::function<void()> job, hipStream_t caller, bool uses_gpu, bool host_ready = false,
-                               bool drained = false);
-  void stamp_start(Work& w, hipStream_t on);
-  char* staging_half();
-  const char* peer_staging(int peer, int half);
-  void copy_pairs(const tdm_pair* pairs, int np, int dtype);
-  void staged_all_reduce(const Buf& t, bool average);
-  void staged_all_reduce_small(const Buf& t, bool average);
-  void staged_all_gather(const Buf& t, const std::vector<Chunk>& cs, const char* own);
-  void staged_reduce_scatter_owner(const Buf& t, const std::vector<Chunk>& cs, bool average);
-  void direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets, const char** base);
-  void direct_fold(const Buf& t, const std::vector<Chunk>& cs, const char* const* base, bool average);
-  void direct_copies(const Buf& t, const std::vector<Chunk>& cs, const char* const* base);
-  void start();
-  void release_device();
-  void loop();
-  void check(const Buf& t, const char* what, bool reduce) const;
-  std::vector<Chunk> chunks(const Buf& t, const std::vector<int64_t>& sizes) const;
-  int64_t piece_elems(int dtype) const { return std::max<int64_t>(1, static_cast<int64_t>(slot_bytes_) / elem_bytes(dtype)); }
-
-  void put(int dst, const char* src, int64_t numel, int dtype, int scale_world);
-  void take(int src, char* into, int64_t numel, int dtype, bool reduce, int scale_world);
-  void exchange(const Chunk* send, int dst, const Chunk* recv, int src, int dtype, bool reduce, int put_scale,
-                int take_scale);
-  void ring_reduce_scatter(const std::vector<Chunk>& c, int dtype, bool average, bool keep_sent);
-  void ring_all_gather(const std::vector<Chunk>& c, int dtype);
-  void signal(int dst, uint64_t length);
-  uint64_t await(int src);
-  void release(int src);
-  void barrier_now(bool after_gpu = false, uint64_t tag = 0);
-  const char* peer_arena(int peer, size_t need_bytes);
-
-  std::string region_name(int rank) const { return "/tandem-" + job_ + "-" + std::to_string(rank) + "-hip"; }
-
-  std::string job_;
-  int rank_, size_, slots_;
-  size_t slot_bytes_;
-  double timeout_s_;
-  int device_;
-  bool use_events_;
-  hipStream_t stream_ = nullptr;
-  hipStream_t gather_stream_ = nullptr;  // direct unit gathers, launched by the caller's thread
-  hipStream_t anchor_stream_ = nullptr;  // carries nothing but the timing anchors: always idle
-  std::mutex anchor_mu_, arena_mu_;      // both threads time their work and map peers' arenas
-  Region mine_;
-  std::vector<std::unique_ptr<Region>> theirs_;
-  std::vector<void*> out_mem_, peer_mem_;
-  void* arena_ = nullptr;
-  size_t arena_bytes_ = 0;
-  std::vector<void*> peer_arena_;
-  std::vector<size_t> peer_arena_bytes_;
-  std::vector<std::vector<hipEvent_t>> full_, free_, peer_full_, peer_free_;
-  std::vector<uint64_t> sent_, got_;     // pieces, per peer: pick the slot
-  std::vector<uint64_t> posted_;         // messages queued or published to each peer (flow control)
-  std::vector<uint64_t> taken_;          // messages consumed from each peer
-  bool connected_ = false, closed_ = false;
-  // staged collectives
-  bool staged_ = true;               // TANDEM_HIP_ALGO=ring switches them off
-  bool gathers_on_side_stream_ = false;  // TANDEM_HIP_GATHER=stream
-  std::shared_ptr<FlagPool> flags_;      // TANDEM_HIP_WAIT=stream
-  bool want_flags_ = false;
-  std::string sticky_error_;             // under mu_: a collective failed after its wait() had already returned
-  bool ready_on_host_ = true;        // TANDEM_HIP_READY=gpu: wait for the caller's stream on the GPU instead
-  size_t staging_half_ = 64u << 20;  // bytes per half (TANDEM_HIP_STAGING_BYTES)
-  size_t small_bytes_ = 32u << 20;   // all_reduce up to this size takes the one-handshake form (TANDEM_HIP_SMALL_BYTES)
-  void* staging_ = nullptr;
-  std::vector<void*> peer_staging_;
-  uint64_t staged_ops_ = 0;          // picks the half; the same count on every rank
-  std::atomic<int> timing_{0};
-  bool timing_seen_ = false;           // under anchor_mu_
-  std::shared_ptr<Anchor> anchor_;     // under anchor_mu_
-
-  // "host" ordering: what to publish once the GPU has passed an event.
-  struct Completion {
-    hipEvent_t after;  // nullptr: publish at once (still in order)
-    bool is_release;
-    int peer;
-    uint64_t length;
-  };
-  void complete_later(bool is_release, int peer, uint64_t length, bool after_stream);
-  void completion_loop();
-  void drain_completions();
-  std::mutex cmu_;
-  std::condition_variable ccv_, cidle_;
-  std::deque<Completion> completions_;
-  bool cstop_ = false, cbusy_ = false;
-  std::atomic<uint64_t> cqueued_{0};  // completions ever queued
-  uint64_t cdone_ = 0;                // completions ever taken (completion thread, under cmu_)
-  std::string cerror_;
-  std::thread completer_;
-
-  std::mutex mu_;
-  std::condition_variable cv_;
-  std::deque<std::pair<std::function<void()>, std::shared_ptr<Work>>> jobs_;
-  std::atomic<uint64_t> submitted_{0};  // jobs ever queued
-  uint64_t started_ = 0;                // jobs ever taken (progress thread only)
-  bool stopping_ = false;
-  std::thread thread_;
-};
 
 Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slot_bytes, double timeout_s, int device)
     : job_(job), rank_(rank), size_(size), slots_(slots), slot_bytes_(slot_bytes), timeout_s_(timeout_s),
@@ -1652,291 +1220,3 @@ std::shared_ptr<Work> Engine::barrier() {
 }
 
 }  // namespace tandem_hip
-
-// ---------------------------------------------------------------- C ABI
-using namespace tandem_hip;
-
-struct tdm_engine {
-  std::unique_ptr<Engine> impl;
-};
-
-struct tdm_work {
-  std::shared_ptr<Work> impl;
-};
-
-namespace {
-
-int finish_submit(std::shared_ptr<Work> w, tdm_work** out) {
-  auto* handle = new tdm_work{std::move(w)};
-  *out = handle;
-  return TDM_OK;
-}
-
-Engine& engine_of(tdm_engine* e) {
-  if (e == nullptr || !e->impl) throw Invalid("NULL engine");
-  return *e->impl;
-}
-
-}  // namespace
-
-extern "C" {
-
-int tdm_engine_create(const char* job, int rank, int size, int slots, int64_t slot_bytes, double timeout_s, int device,
-                      tdm_engine** out) {
-  return guard([&] {
-    if (job == nullptr || out == nullptr) throw Invalid("NULL argument");
-    if (slot_bytes <= 0) throw Invalid("slot_bytes must be positive");
-    auto e = std::make_unique<Engine>(job, rank, size, slots, static_cast<size_t>(slot_bytes), timeout_s, device);
-    *out = new tdm_engine{std::move(e)};
-  });
-}
-
-int tdm_engine_connect(tdm_engine* e) {
-  return guard([&] { engine_of(e).connect(); });
-}
-
-int tdm_engine_close(tdm_engine* e) {
-  return guard([&] { engine_of(e).close(); });
-}
-
-int tdm_engine_destroy(tdm_engine* e) {
-  return guard([&] { delete e; });
-}
-
-int tdm_all_reduce(tdm_engine* e, void* ptr, int64_t numel, int dtype, int average, tdm_stream caller, tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    finish_submit(engine_of(e).all_reduce(Engine::Buf{static_cast<char*>(ptr), numel, dtype}, average != 0,
-                                          static_cast<hipStream_t>(caller)), out);
-  });
-}
-
-namespace {
-int reduce_scatter_call(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
-                        bool owner_only, tdm_stream caller, tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    if (nsizes < 0 || (nsizes > 0 && sizes == nullptr)) throw Invalid("bad sizes");
-    std::vector<int64_t> sz(sizes, sizes + nsizes);
-    finish_submit(engine_of(e).reduce_scatter(Engine::Buf{static_cast<char*>(ptr), numel, dtype}, std::move(sz),
-                                              average != 0, owner_only, static_cast<hipStream_t>(caller)), out);
-  });
-}
-}  // namespace
-
-int tdm_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
-                       tdm_stream caller, tdm_work** out) {
-  return reduce_scatter_call(e, ptr, numel, dtype, sizes, nsizes, average, false, caller, out);
-}
-
-int tdm_reduce_scatter_owner(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
-                             tdm_stream caller, tdm_work** out) {
-  return reduce_scatter_call(e, ptr, numel, dtype, sizes, nsizes, average, true, caller, out);
-}
-
-int tdm_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, tdm_stream caller,
-                   tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    if (nsizes < 0 || (nsizes > 0 && sizes == nullptr)) throw Invalid("bad sizes");
-    std::vector<int64_t> sz(sizes, sizes + nsizes);
-    finish_submit(engine_of(e).all_gather(Engine::Buf{static_cast<char*>(ptr), numel, dtype}, std::move(sz),
-                                          static_cast<hipStream_t>(caller)), out);
-  });
-}
-
-int tdm_unit_gather(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes, int nsizes,
-                    tdm_stream caller, tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    if (nsizes < 0 || (nsizes > 0 && sizes == nullptr)) throw Invalid("bad sizes");
-    std::vector<int64_t> sz(sizes, sizes + nsizes);
-    finish_submit(engine_of(e).unit_gather(Engine::Buf{static_cast<char*>(full), numel, dtype},
-                                           static_cast<const char*>(shard), std::move(sz),
-                                           static_cast<hipStream_t>(caller)), out);
-  });
-}
-
-int tdm_broadcast(tdm_engine* e, void* ptr, int64_t numel, int dtype, int root, tdm_stream caller, tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    finish_submit(engine_of(e).broadcast(Engine::Buf{static_cast<char*>(ptr), numel, dtype}, root,
-                                         static_cast<hipStream_t>(caller)), out);
-  });
-}
-
-int tdm_sendrecv(tdm_engine* e, const void* send, int64_t send_numel, int dst, void* recv, int64_t recv_numel, int src,
-                 int dtype, tdm_stream caller, tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    finish_submit(engine_of(e).sendrecv(Engine::Buf{static_cast<char*>(const_cast<void*>(send)), send_numel, dtype}, dst,
-                                        Engine::Buf{static_cast<char*>(recv), recv_numel, dtype}, src,
-                                        static_cast<hipStream_t>(caller)), out);
-  });
-}
-
-int tdm_engine_share(tdm_engine* e, int64_t bytes, void** ptr) {
-  return guard([&] {
-    if (ptr == nullptr || bytes <= 0) throw Invalid("share: bad arguments");
-    *ptr = engine_of(e).share(static_cast<size_t>(bytes));
-  });
-}
-
-int tdm_unit_gather_direct(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes,
-                           int nsizes, const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    if (nsizes < 0 || (nsizes > 0 && sizes == nullptr) || noffsets < 0 || (noffsets > 0 && peer_offsets == nullptr)) {
-      throw Invalid("bad sizes or offsets");
-    }
-    std::vector<int64_t> sz(sizes, sizes + nsizes), off(peer_offsets, peer_offsets + noffsets);
-    finish_submit(engine_of(e).unit_gather_direct(Engine::Buf{static_cast<char*>(full), numel, dtype},
-                                                  static_cast<const char*>(shard), std::move(sz), std::move(off),
-                                                  static_cast<hipStream_t>(caller)), out);
-  });
-}
-
-namespace {
-int direct_call(tdm_engine* e, int kind, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes, int average,
-                const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    if (nsizes < 0 || (nsizes > 0 && sizes == nullptr) || noffsets < 0 || (noffsets > 0 && peer_offsets == nullptr)) {
-      throw Invalid("bad sizes or offsets");
-    }
-    std::vector<int64_t> sz(sizes, sizes + nsizes), off(peer_offsets, peer_offsets + noffsets);
-    finish_submit(engine_of(e).direct(kind, Engine::Buf{static_cast<char*>(ptr), numel, dtype}, std::move(sz), average != 0,
-                                      std::move(off), static_cast<hipStream_t>(caller)), out);
-  });
-}
-}  // namespace
-
-int tdm_direct_all_reduce(tdm_engine* e, void* ptr, int64_t numel, int dtype, int average, const int64_t* peer_offsets,
-                          int noffsets, tdm_stream caller, tdm_work** out) {
-  return direct_call(e, 0, ptr, numel, dtype, nullptr, 0, average, peer_offsets, noffsets, caller, out);
-}
-
-int tdm_direct_reduce_scatter(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
-                              int average, const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out) {
-  return direct_call(e, 1, ptr, numel, dtype, sizes, nsizes, average, peer_offsets, noffsets, caller, out);
-}
-
-int tdm_direct_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
-                          const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out) {
-  return direct_call(e, 2, ptr, numel, dtype, sizes, nsizes, 0, peer_offsets, noffsets, caller, out);
-}
-
-int tdm_direct_zero2_step(tdm_engine* e, void* param, const int64_t* param_offsets, const void* grad, const int64_t* grad_offsets,
-                          int noffsets, void* exp_avg, void* exp_avg_sq, int64_t count, int64_t total, int average,
-                          const tdm_adamw_scalars* s, int order, tdm_stream caller, tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    if (s == nullptr) throw Invalid("NULL scalars");
-    if (noffsets < 0 || (noffsets > 0 && (param_offsets == nullptr || grad_offsets == nullptr))) throw Invalid("bad offsets argument");
-    std::vector<int64_t> po(param_offsets, param_offsets + noffsets), go(grad_offsets, grad_offsets + noffsets);
-    finish_submit(engine_of(e).zero2_step_direct(Engine::Buf{static_cast<char*>(param), count, TDM_F32},
-                                                 Engine::Buf{static_cast<char*>(const_cast<void*>(grad)), count, TDM_F32},
-                                                 std::move(po), std::move(go), static_cast<char*>(exp_avg),
-                                                 static_cast<char*>(exp_avg_sq), total, average != 0, *s, order,
-                                                 static_cast<hipStream_t>(caller)),
-                  out);
-  });
-}
-
-int tdm_fence(tdm_engine* e, tdm_stream caller, tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    finish_submit(engine_of(e).fence(static_cast<hipStream_t>(caller)), out);
-  });
-}
-
-int tdm_barrier(tdm_engine* e, tdm_work** out) {
-  return guard([&] {
-    if (out == nullptr) throw Invalid("NULL work pointer");
-    finish_submit(engine_of(e).barrier(), out);
-  });
-}
-
-int tdm_work_wait(tdm_work* w, tdm_stream caller) {
-  if (w == nullptr || !w->impl) {
-    set_last_error("NULL work");
-    return TDM_EINVAL;
-  }
-  Work& work = *w->impl;
-  if (work.flag >= 0 && !work.finished_hint.load(std::memory_order_acquire)) {
-    // The job has not run yet: park the caller's stream on its word and return. The host
-    // goes on queueing work behind the collective; a failure shows at the next call.
-    return guard([&] {
-      check_hip(hipStreamWaitValue32(static_cast<hipStream_t>(caller), work.flags->base + work.flag, work.flag_value,
-                                     hipStreamWaitValueGte, 0xffffffffu),
-                "hipStreamWaitValue32 (wait)");
-    });
-  }
-  spin_for([&] { return work.finished_hint.load(std::memory_order_acquire); });
-  {
-    std::unique_lock<std::mutex> lock(work.mu);
-    work.cv.wait(lock, [&] { return work.finished; });
-    if (work.status != TDM_OK) {
-      set_last_error(work.error);
-      return work.status;
-    }
-  }
-  if (work.done_event && !(work.on_callers_stream && work.launched_on == static_cast<hipStream_t>(caller))) {
-    return guard([&] {
-      const hipError_t q = hipEventQuery(work.done_event);
-      if (q == hipSuccess) return;  // the GPU is past it already: nothing to order
-      if (q == hipErrorNotReady) (void)hipGetLastError();
-      check_hip(hipStreamWaitEvent(static_cast<hipStream_t>(caller), work.done_event, 0), "hipStreamWaitEvent (wait)");
-    });
-  }
-  return TDM_OK;
-}
-
-int tdm_work_done(tdm_work* w) {
-  if (w == nullptr || !w->impl) return 0;
-  Work& work = *w->impl;
-  std::lock_guard<std::mutex> lock(work.mu);
-  if (!work.finished) return 0;
-  if (work.status == TDM_OK && work.done_event) return hipEventQuery(work.done_event) == hipSuccess ? 1 : 0;
-  return 1;
-}
-
-int tdm_work_times(tdm_work* w, double* started, double* finished) {
-  if (w == nullptr || !w->impl) {
-    set_last_error("NULL work");
-    return TDM_EINVAL;
-  }
-  Work& work = *w->impl;
-  {
-    std::unique_lock<std::mutex> lock(work.mu);
-    work.cv.wait(lock, [&] { return work.finished; });
-    if (started) *started = work.t0;
-    if (finished) *finished = work.t1;
-    if (work.status != TDM_OK || !work.start_event || !work.done_event || !work.anchor) return TDM_OK;
-  }
-  // Timed on the device: wait for its last kernel, then place both stamps on the host clock.
-  return guard([&] {
-    check_hip(hipEventSynchronize(work.done_event), "hipEventSynchronize (times)");
-    float ms0 = 0, ms1 = 0;
-    check_hip(hipEventElapsedTime(&ms0, work.anchor->event, work.start_event), "hipEventElapsedTime (start)");
-    check_hip(hipEventElapsedTime(&ms1, work.anchor->event, work.done_event), "hipEventElapsedTime (done)");
-    if (started) *started = work.anchor->host + static_cast<double>(ms0) * 1e-3;
-    if (finished) *finished = work.anchor->host + static_cast<double>(ms1) * 1e-3;
-  });
-}
-
-int tdm_engine_set_timing(tdm_engine* e, int on) {
-  if (e == nullptr || !e->impl) {
-    set_last_error("NULL engine");
-    return TDM_EINVAL;
-  }
-  e->impl->set_timing(on != 0);
-  return TDM_OK;
-}
-
-int tdm_work_free(tdm_work* w) {
-  delete w;
-  return TDM_OK;
-}
-
-}  // extern "C"
