@@ -1,0 +1,744 @@
+// The device side of libtandem_hip: element types, load/store helpers with their cache
+// policies, and the kernels K1 (ring-step reduce, copy), K2 (bucket fold), K3 (AdamW),
+// K2+K3 (ZeRO-2's step) and K4's copies. Included by kernels.hip only: everything here
+// has internal linkage.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <type_traits>
+
+#include "../../include/tandem_hip.h"
+#include "common.h"
+
+namespace tandem_hip {
+
+namespace {
+
+
+#ifndef TDM_THREADS
+#define TDM_THREADS 256
+#endif
+#ifndef TDM_UNROLL
+#define TDM_UNROLL 4
+#endif
+constexpr int kThreads = TDM_THREADS;
+constexpr int kUnroll = TDM_UNROLL;             // 16-byte vectors per lane per tile and stream
+#ifndef TDM_K1_UNROLL
+#define TDM_K1_UNROLL 2
+#endif
+// K1 and the copy kernel cut their pairs into tiles of their own, 8 KiB per stream: against 16 KiB the
+// ring (reduce-scatter + all-gather, world 4) runs 3 % faster at 64 MiB per rank (6.95 vs 6.74 TB/s), 2 %
+// at 16 MiB and equally fast at 256 MiB; different tile sizes for the two kernels are worse than either.
+constexpr int kK1Unroll = TDM_K1_UNROLL;
+constexpr int kK1TileVecs = kThreads * kK1Unroll;
+#ifndef TDM_COPY_UNROLL
+#define TDM_COPY_UNROLL TDM_K1_UNROLL
+#endif
+constexpr int kCopyUnroll = TDM_COPY_UNROLL;
+constexpr int kCopyTileVecs = kThreads * kCopyUnroll;
+constexpr int kTileVecs = kThreads * kUnroll;   // 1024 vectors = 16 KiB of every stream
+// Measured on MI355X: one 16 KiB tile per workgroup beats a persistent grid-stride
+// loop by 5-8% (the hardware dispatcher balances 8 XCDs better than a fixed stride),
+// so the grid covers the tiles one to one up to 256 Ki workgroups (4 GiB per stream)
+// and strides only beyond that.
+constexpr int kDefaultBlocksPerCu = 1024;
+
+int g_blocks_per_cu = kDefaultBlocksPerCu;
+constexpr int64_t kColdFootprint = int64_t(512) << 20;  // twice the Infinity Cache
+
+typedef uint32_t vec16 __attribute__((ext_vector_type(4)));  // one dwordx4 access
+
+// ---------------------------------------------------------------- element types
+struct f16_t { uint16_t bits; };
+struct bf16_t { uint16_t bits; };
+
+template <typename T> struct Elem;
+
+template <> struct Elem<float> {
+  using acc = float;
+  static constexpr bool floating = true;
+  static __device__ __forceinline__ acc widen(float x) { return x; }
+  static __device__ __forceinline__ float narrow(acc x) { return x; }
+};
+template <> struct Elem<double> {
+  using acc = double;
+  static constexpr bool floating = true;
+  static __device__ __forceinline__ acc widen(double x) { return x; }
+  static __device__ __forceinline__ double narrow(acc x) { return x; }
+};
+template <> struct Elem<int64_t> {
+  using acc = int64_t;
+  static constexpr bool floating = false;
+  static __device__ __forceinline__ acc widen(int64_t x) { return x; }
+  static __device__ __forceinline__ int64_t narrow(acc x) { return x; }
+};
+template <> struct Elem<int32_t> {
+  using acc = int32_t;
+  static constexpr bool floating = false;
+  static __device__ __forceinline__ acc widen(int32_t x) { return x; }
+  static __device__ __forceinline__ int32_t narrow(acc x) { return x; }
+};
+template <> struct Elem<f16_t> {
+  using acc = float;
+  static constexpr bool floating = true;
+  static __device__ __forceinline__ acc widen(f16_t x) {
+    _Float16 h;
+    __builtin_memcpy(&h, &x.bits, 2);
+    return static_cast<float>(h);
+  }
+  static __device__ __forceinline__ f16_t narrow(acc x) {
+    _Float16 h = static_cast<_Float16>(x);  // round to nearest even, once
+    f16_t out;
+    __builtin_memcpy(&out.bits, &h, 2);
+    return out;
+  }
+};
+template <> struct Elem<bf16_t> {
+  using acc = float;
+  static constexpr bool floating = true;
+  static __device__ __forceinline__ acc widen(bf16_t x) { return __uint_as_float(static_cast<uint32_t>(x.bits) << 16); }
+  static __device__ __forceinline__ bf16_t narrow(acc x) {
+    uint32_t u = __float_as_uint(x);
+    bf16_t out;
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+      out.bits = 0x7fc0u;  // NaN
+    } else {
+      u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
+      out.bits = static_cast<uint16_t>(u >> 16);
+    }
+    return out;
+  }
+};
+
+// x / world as the element type would store it. kDiv: 0 none, 1 world is a power
+// of two (multiplying by the exact reciprocal gives the same bits as dividing,
+// denormal results included), 2 true division.
+template <typename T, int kDiv>
+__device__ __forceinline__ typename Elem<T>::acc scaled(typename Elem<T>::acc x, typename Elem<T>::acc divisor,
+                                                        typename Elem<T>::acc reciprocal) {
+  using A = typename Elem<T>::acc;
+  if constexpr (kDiv == 0 || !Elem<T>::floating) {
+    return x;
+  } else if constexpr (kDiv == 1) {
+    return Elem<T>::widen(Elem<T>::narrow(static_cast<A>(x * reciprocal)));
+  } else {
+    return Elem<T>::widen(Elem<T>::narrow(static_cast<A>(x / divisor)));
+  }
+}
+
+template <typename T>
+constexpr int lanes() { return 16 / static_cast<int>(sizeof(T)); }
+
+template <typename T>
+struct Lanes {
+  T v[lanes<T>()];
+};
+
+template <typename T>
+__device__ __forceinline__ Lanes<T> unpack(const vec16& raw) {
+  Lanes<T> out;
+  __builtin_memcpy(&out, &raw, 16);
+  return out;
+}
+template <typename T>
+__device__ __forceinline__ vec16 pack(const Lanes<T>& in) {
+  vec16 out;
+  __builtin_memcpy(&out, &in, 16);
+  return out;
+}
+
+// Cache policy, measured on MI355X. K1 with 4 x 64 MiB chunk pairs per launch: a
+// stream that is only read does best with non-temporal loads (it is not kept in
+// L2 / Infinity Cache), a stream that is read, modified and written back does best
+// with plain loads and plain stores (the store hits the line the load brought in).
+// Both non-temporal: 6.4 TB/s; both plain: 5.4; this split: 7.0. The bucket fold
+// and AdamW run once per training step over data that nothing has touched since
+// the last step: there non-temporal stores pay as well (fold 0.260 -> 0.240 ms,
+// AdamW on four shards 0.448 -> 0.415 ms), and for AdamW non-temporal loads of
+// the streams it rewrites.
+// -DTDM_NT_MASK=<0..7> (and _K2, _K3) build the other combinations for measurement.
+#ifndef TDM_NT_MASK
+#define TDM_NT_MASK 2  // bit0: read-modify-write loads, bit1: read-once loads, bit2: stores are non-temporal
+#endif
+#ifndef TDM_NT_MASK_K2
+#define TDM_NT_MASK_K2 6  // the bucket fold over a device table (the by-value fold of one collective keeps TDM_NT_MASK)
+#endif
+#ifndef TDM_NT_MASK_K3
+#define TDM_NT_MASK_K3 7  // AdamW
+#endif
+#ifndef TDM_NT_MASK_K3C
+#define TDM_NT_MASK_K3C TDM_NT_MASK_K3  // AdamW's further copies of the parameters
+#endif
+template <int kMask = TDM_NT_MASK>
+__device__ __forceinline__ vec16 load_stream(const void* p) {  // read once, never written here
+  if constexpr (kMask & 2) return __builtin_nontemporal_load(static_cast<const vec16*>(p));
+  else return *static_cast<const vec16*>(p);
+}
+template <int kMask = TDM_NT_MASK>
+__device__ __forceinline__ vec16 load_rmw(const void* p) {  // about to be overwritten by this lane
+  if constexpr (kMask & 1) return __builtin_nontemporal_load(static_cast<const vec16*>(p));
+  else return *static_cast<const vec16*>(p);
+}
+template <int kMask = TDM_NT_MASK>
+__device__ __forceinline__ void store16(void* p, const vec16& v) {
+  if constexpr (kMask & 4) __builtin_nontemporal_store(v, static_cast<vec16*>(p));
+  else *static_cast<vec16*>(p) = v;
+}
+
+// ---------------------------------------------------------------- pair tables
+// Passed by value in the kernel arguments (scalar loads; no device table).
+struct PairTable {
+  int npairs;
+  int flags;  // per launch: bit0 scale_dst, bit1 scale_src, bit2 writeback_src
+  int64_t tile_end[TDM_MAX_PAIRS];  // running tile count
+  char* dst[TDM_MAX_PAIRS];
+  char* src[TDM_MAX_PAIRS];
+  int64_t count[TDM_MAX_PAIRS];
+  int32_t head[TDM_MAX_PAIRS];    // elements before dst reaches a 16-byte boundary
+  int32_t vec_ok[TDM_MAX_PAIRS];  // dst and src share the same phase within 16 bytes
+};
+
+template <typename T>
+struct Divisor {
+  typename Elem<T>::acc divisor, reciprocal;
+};
+
+// dst = (dst[/w]) + (src[/w]) on one element
+template <typename T, int kDiv>
+__device__ __forceinline__ void reduce_elem(T& d, T& s, bool scale_dst, bool scale_src, const Divisor<T>& dv) {
+  using A = typename Elem<T>::acc;
+  A x = Elem<T>::widen(d), y = Elem<T>::widen(s);
+  if (scale_dst) x = scaled<T, kDiv>(x, dv.divisor, dv.reciprocal);
+  if (scale_src) y = scaled<T, kDiv>(y, dv.divisor, dv.reciprocal);
+  s = Elem<T>::narrow(y);
+  d = Elem<T>::narrow(static_cast<A>(x + y));
+}
+
+template <typename T, int kDiv, int kMask>
+__global__ __launch_bounds__(kThreads) void k1_reduce_kernel(PairTable tab, Divisor<T> dv) {
+  constexpr int L = lanes<T>();
+  constexpr int64_t kTileElems = static_cast<int64_t>(kK1TileVecs) * L;
+  const bool scale_dst = tab.flags & 1, scale_src = tab.flags & 2, writeback = tab.flags & 4;
+  const int64_t total = tab.tile_end[tab.npairs - 1];
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    int p = 0;
+    while (tile >= tab.tile_end[p]) ++p;
+    const int64_t t = tile - (p ? tab.tile_end[p - 1] : 0);
+    T* __restrict__ dst = reinterpret_cast<T*>(tab.dst[p]);
+    T* __restrict__ src = reinterpret_cast<T*>(tab.src[p]);
+    const int64_t n = tab.count[p];
+    if (tab.vec_ok[p]) {
+      const int64_t head = tab.head[p];
+      const int64_t nv = (n - head) / L;
+      char* dvp = reinterpret_cast<char*>(dst + head);
+      char* svp = reinterpret_cast<char*>(src + head);
+      const int64_t v0 = t * kK1TileVecs + threadIdx.x;
+      if ((t + 1) * kK1TileVecs <= nv) {  // a full tile: all loads first, then the arithmetic, then the stores
+        vec16 a[kK1Unroll], b[kK1Unroll];
+#pragma unroll
+        for (int k = 0; k < kK1Unroll; ++k) a[k] = load_rmw<kMask>(dvp + (v0 + k * kThreads) * 16);
+#pragma unroll
+        for (int k = 0; k < kK1Unroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kThreads) * 16);
+#pragma unroll
+        for (int k = 0; k < kK1Unroll; ++k) {
+          Lanes<T> x = unpack<T>(a[k]), y = unpack<T>(b[k]);
+#pragma unroll
+          for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
+          store16<kMask>(dvp + (v0 + k * kThreads) * 16, pack<T>(x));
+          if (writeback) store16<kMask>(svp + (v0 + k * kThreads) * 16, pack<T>(y));
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < kK1Unroll; ++k) {
+          const int64_t v = v0 + k * kThreads;
+          if (v < nv) {
+            Lanes<T> x = unpack<T>(load_rmw<kMask>(dvp + v * 16)), y = unpack<T>(load_stream<kMask>(svp + v * 16));
+#pragma unroll
+            for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
+            store16<kMask>(dvp + v * 16, pack<T>(x));
+            if (writeback) store16<kMask>(svp + v * 16, pack<T>(y));
+          }
+        }
+      }
+      if (t == 0) {  // the few elements before and after the 16-byte body
+        const int64_t tail0 = head + nv * L;
+        int64_t i = -1;
+        if (static_cast<int64_t>(threadIdx.x) < head) i = threadIdx.x;
+        else if (threadIdx.x >= 32 && tail0 + (threadIdx.x - 32) < n && threadIdx.x - 32 < L) i = tail0 + (threadIdx.x - 32);
+        if (i >= 0) {
+          T x = dst[i], y = src[i];
+          reduce_elem<T, kDiv>(x, y, scale_dst, scale_src, dv);
+          dst[i] = x;
+          if (writeback) src[i] = y;
+        }
+      }
+    } else {  // the two pointers disagree within 16 bytes: element-wise, still coalesced
+      const int64_t e0 = t * kTileElems + threadIdx.x;
+#pragma unroll 4
+      for (int k = 0; k < kK1Unroll * L; ++k) {
+        const int64_t i = e0 + static_cast<int64_t>(k) * kThreads;
+        if (i < n) {
+          T x = dst[i], y = src[i];
+          reduce_elem<T, kDiv>(x, y, scale_dst, scale_src, dv);
+          dst[i] = x;
+          if (writeback) src[i] = y;
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int kDiv>
+__device__ __forceinline__ T copy_elem(T s, const Divisor<T>& dv) {
+  if constexpr (kDiv == 0) {
+    return s;
+  } else {
+    return Elem<T>::narrow(scaled<T, kDiv>(Elem<T>::widen(s), dv.divisor, dv.reciprocal));
+  }
+}
+
+template <typename T, int kDiv, int kMask>
+__global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Divisor<T> dv) {
+  constexpr int L = lanes<T>();
+  constexpr int64_t kTileElems = static_cast<int64_t>(kCopyTileVecs) * L;
+  const int64_t total = tab.tile_end[tab.npairs - 1];
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    int p = 0;
+    while (tile >= tab.tile_end[p]) ++p;
+    const int64_t t = tile - (p ? tab.tile_end[p - 1] : 0);
+    T* __restrict__ dst = reinterpret_cast<T*>(tab.dst[p]);
+    const T* __restrict__ src = reinterpret_cast<const T*>(tab.src[p]);
+    const int64_t n = tab.count[p];
+    if (tab.vec_ok[p]) {
+      const int64_t head = tab.head[p];
+      const int64_t nv = (n - head) / L;
+      char* dvp = reinterpret_cast<char*>(dst + head);
+      const char* svp = reinterpret_cast<const char*>(src + head);
+      const int64_t v0 = t * kCopyTileVecs + threadIdx.x;
+      if ((t + 1) * kCopyTileVecs <= nv) {
+        vec16 b[kCopyUnroll];
+#pragma unroll
+        for (int k = 0; k < kCopyUnroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kThreads) * 16);
+#pragma unroll
+        for (int k = 0; k < kCopyUnroll; ++k) {
+          if constexpr (kDiv != 0) {
+            Lanes<T> y = unpack<T>(b[k]);
+#pragma unroll
+            for (int l = 0; l < L; ++l) y.v[l] = copy_elem<T, kDiv>(y.v[l], dv);
+            b[k] = pack<T>(y);
+          }
+          store16<kMask>(dvp + (v0 + k * kThreads) * 16, b[k]);
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < kCopyUnroll; ++k) {
+          const int64_t v = v0 + k * kThreads;
+          if (v < nv) {
+            Lanes<T> y = unpack<T>(load_stream<kMask>(svp + v * 16));
+#pragma unroll
+            for (int l = 0; l < L; ++l) y.v[l] = copy_elem<T, kDiv>(y.v[l], dv);
+            store16<kMask>(dvp + v * 16, pack<T>(y));
+          }
+        }
+      }
+      if (t == 0) {
+        const int64_t tail0 = head + nv * L;
+        int64_t i = -1;
+        if (static_cast<int64_t>(threadIdx.x) < head) i = threadIdx.x;
+        else if (threadIdx.x >= 32 && tail0 + (threadIdx.x - 32) < n && threadIdx.x - 32 < L) i = tail0 + (threadIdx.x - 32);
+        if (i >= 0) dst[i] = copy_elem<T, kDiv>(src[i], dv);
+      }
+    } else {
+      const int64_t e0 = t * kTileElems + threadIdx.x;
+#pragma unroll 4
+      for (int k = 0; k < kCopyUnroll * L; ++k) {
+        const int64_t i = e0 + static_cast<int64_t>(k) * kThreads;
+        if (i < n) dst[i] = copy_elem<T, kDiv>(src[i], dv);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- K2: bucket fold
+// A segment as the kernels see it. The device table of K2 is an array of these, ONE
+// PER TILE: the pointers already advanced to the tile's first element and `count`
+// the tile's elements, so a workgroup needs a single lookup before its loads go out
+// (a tile -> segment -> pointers chain cost 20% of the kernel's throughput).
+struct FoldSegDev {
+  const char* src[TDM_MAX_WORLD];
+  char* dst[TDM_MAX_WORLD];
+  int64_t count;
+  int32_t chunk;
+  int32_t vec_ok;  // every pointer of the segment is 16-byte aligned
+};
+
+// One tile of one segment: W loads per element, the fold in ring order, W stores.
+// kAcc: the result is added into each destination (dst = dst + sum) instead of replacing it.
+template <typename T, int kWorld, int kDiv, bool kAcc, int kMask>
+__device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const Divisor<T>& dv) {
+  using A = typename Elem<T>::acc;
+  constexpr int L = lanes<T>();
+#ifndef TDM_K2_UNROLL_W2
+#define TDM_K2_UNROLL_W2 4
+#endif
+#ifndef TDM_K2_UNROLL
+#define TDM_K2_UNROLL 4
+#endif
+  // vectors per lane per tile step, per rank (worlds 3-4: 4 beats 2 by 2-3 %; beyond that the registers run out)
+  constexpr int kU = kWorld <= 2 ? TDM_K2_UNROLL_W2 : kWorld <= 4 ? TDM_K2_UNROLL : 2;
+  constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
+  const int64_t n = sg.count;
+  const int c = sg.chunk;
+  // ring order: the fold starts at rank chunk+1 and ends with the chunk's owner
+  const char* sp[kWorld];
+  char* dp[kWorld];
+#pragma unroll
+  for (int k = 0; k < kWorld; ++k) {
+    sp[k] = sg.src[(c + 1 + k) % kWorld];
+    dp[k] = sg.dst[k];
+  }
+  if (sg.vec_ok) {
+    const int64_t nv = n / L;
+#pragma unroll
+    for (int u0 = 0; u0 < kUnroll; u0 += kU) {
+      const int64_t vbase = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u0) * kThreads;
+      vec16 in[kWorld][kU];
+#pragma unroll
+      for (int k = 0; k < kWorld; ++k)
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          const int64_t v = vbase + u * kThreads;
+          if (v < nv) in[k][u] = load_stream<kMask>(sp[k] + v * 16);
+        }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int64_t v = vbase + u * kThreads;
+        if (v < nv) {
+          Lanes<T> out;
+#pragma unroll
+          for (int l = 0; l < L; ++l) {
+            A acc = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[0][u]).v[l]), dv.divisor, dv.reciprocal);
+#pragma unroll
+            for (int k = 1; k < kWorld; ++k) {
+              const A y = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[k][u]).v[l]), dv.divisor, dv.reciprocal);
+              acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+            }
+            out.v[l] = Elem<T>::narrow(acc);
+          }
+          const vec16 packed = pack<T>(out);
+#pragma unroll
+          for (int k = 0; k < kWorld; ++k)
+            if (dp[k]) {
+              if constexpr (kAcc) {
+                Lanes<T> cur = unpack<T>(load_rmw<kMask>(dp[k] + v * 16));
+#pragma unroll
+                for (int l = 0; l < L; ++l)
+                  cur.v[l] = Elem<T>::narrow(static_cast<A>(Elem<T>::widen(cur.v[l]) + Elem<T>::widen(out.v[l])));
+                store16<kMask>(dp[k] + v * 16, pack<T>(cur));
+              } else {
+                store16<kMask>(dp[k] + v * 16, packed);
+              }
+            }
+        }
+      }
+    }
+    if (t == 0 && threadIdx.x < n - nv * L) {  // tail elements
+      const int64_t i = nv * L + threadIdx.x;
+      A acc = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[0])[i]), dv.divisor, dv.reciprocal);
+#pragma unroll
+      for (int k = 1; k < kWorld; ++k) {
+        const A y = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[k])[i]), dv.divisor, dv.reciprocal);
+        acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+      }
+#pragma unroll
+      for (int k = 0; k < kWorld; ++k)
+        if (dp[k]) {
+          T* out1 = reinterpret_cast<T*>(dp[k]) + i;
+          *out1 = kAcc ? Elem<T>::narrow(static_cast<A>(Elem<T>::widen(*out1) + Elem<T>::widen(Elem<T>::narrow(acc)))) : Elem<T>::narrow(acc);
+        }
+    }
+  } else {
+    const int64_t e0 = t * kTileElems + threadIdx.x;
+    for (int k2 = 0; k2 < kUnroll * L; ++k2) {
+      const int64_t i = e0 + static_cast<int64_t>(k2) * kThreads;
+      if (i < n) {
+        A acc = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[0])[i]), dv.divisor, dv.reciprocal);
+#pragma unroll
+        for (int k = 1; k < kWorld; ++k) {
+          const A y = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[k])[i]), dv.divisor, dv.reciprocal);
+          acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+        }
+#pragma unroll
+        for (int k = 0; k < kWorld; ++k)
+          if (dp[k]) {
+            T* out1 = reinterpret_cast<T*>(dp[k]) + i;
+            *out1 = kAcc ? Elem<T>::narrow(static_cast<A>(Elem<T>::widen(*out1) + Elem<T>::widen(Elem<T>::narrow(acc)))) : Elem<T>::narrow(acc);
+          }
+      }
+    }
+  }
+}
+
+// Table in device memory, one record per tile (many segments: DDP's buckets).
+template <typename T, int kWorld, int kDiv, bool kAcc>
+__global__ __launch_bounds__(kThreads) void k2_fold_kernel(const FoldSegDev* __restrict__ tiles, int64_t total,
+                                                           Divisor<T> dv) {
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    fold_tile<T, kWorld, kDiv, kAcc, TDM_NT_MASK_K2>(tiles[tile], 0, dv);
+  }
+}
+
+// Table by value (one segment per ring chunk: a whole all-reduce in one launch).
+struct FoldSmall {
+  int nseg;
+  int64_t tile_end[TDM_MAX_WORLD];
+  FoldSegDev seg[TDM_MAX_WORLD];
+};
+
+// kCold: the launch's footprint is far beyond the 256 MB Infinity Cache, so nothing it
+// writes will be read from there: the cache policy of the once-per-step bucket fold.
+template <typename T, int kWorld, int kDiv, bool kCold>
+__global__ __launch_bounds__(kThreads) void k2_fold_small_kernel(FoldSmall tab, Divisor<T> dv) {
+  const int64_t total = tab.tile_end[tab.nseg - 1];
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    int lo = 0;
+    while (tile >= tab.tile_end[lo]) ++lo;
+    fold_tile<T, kWorld, kDiv, false, kCold ? TDM_NT_MASK_K2 : TDM_NT_MASK>(tab.seg[lo], tile - (lo ? tab.tile_end[lo - 1] : 0), dv);
+  }
+}
+
+// ---------------------------------------------------------------- K3: AdamW
+struct AdamwArgs {
+  float* p;
+  const float* g;
+  float* m;
+  float* v;
+  int64_t n;
+  tdm_adamw_scalars s;
+  // Further copies of the updated parameters (the other ranks' flat buffers): the
+  // update and the all-gather of the result in one pass.
+  int ncopies;
+  float* copy[TDM_MAX_WORLD - 1];
+};
+
+template <int kOrder>
+__device__ __forceinline__ void adamw_elem(float& p, float g, float& m, float& v, const tdm_adamw_scalars& s,
+                                           bool small_w) {
+  if (s.use_decay) p = p * s.decay;
+  const float diff = g - m;
+  // lerp_: weight < 0.5 ? fma(w, end-start, start) : fma(w-1, end-start, end)
+  m = small_w ? __builtin_fmaf(s.w1, diff, m) : __builtin_fmaf(s.w1 - 1.0f, diff, g);
+  const float vs = v * s.beta2;
+  if constexpr (kOrder == TDM_ADAMW_HOST_ORDER) {
+    v = __builtin_fmaf(s.one_m_b2 * g, g, vs);  // CPU addcmul_: (value*g) rounded, then fused
+  } else {
+    v = __builtin_fmaf(s.one_m_b2, g * g, vs);  // GPU addcmul_: a + value * (g*g), contracted
+  }
+  if constexpr (kOrder == TDM_ADAMW_HOST_ORDER) {
+    const float d = __builtin_sqrtf(v) / s.bc2_sqrt + s.eps;
+    p = p + (s.neg_step * m) / d;  // CPU addcdiv_: (value*m)/d, then add; nothing fused
+  } else {
+    const float d = __builtin_sqrtf(v) * s.inv_bc2_sqrt + s.eps;  // GPU tensor / scalar: times the reciprocal
+    p = __builtin_fmaf(s.neg_step, m / d, p);  // GPU addcdiv_: a + value * (m/d), contracted
+  }
+}
+
+#ifndef TDM_K3_UNROLL
+#define TDM_K3_UNROLL 1
+#endif
+constexpr int kAdamwUnroll = TDM_K3_UNROLL;  // vectors per lane and stream in flight
+
+template <int kOrder, bool kVec, bool kCopies>
+__global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
+  const bool small_w = __builtin_fabsf(a.s.w1) < 0.5f;
+  if constexpr (kVec) {
+    constexpr int kU = kAdamwUnroll;
+    const int64_t nv = a.n / 4;
+    const int64_t tiles = (nv + kThreads * kU - 1) / (kThreads * kU);
+    for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+      const int64_t v0 = tile * (kThreads * kU) + threadIdx.x;
+      vec16 rp[kU], rg[kU], rm[kU], rv[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int64_t i = v0 + u * kThreads;
+        if (i < nv) {
+          rp[u] = load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.p) + i * 16);
+          rg[u] = load_stream<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.g) + i * 16);
+          rm[u] = load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.m) + i * 16);
+          rv[u] = load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.v) + i * 16);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int64_t i = v0 + u * kThreads;
+        if (i < nv) {
+          Lanes<float> P = unpack<float>(rp[u]), G = unpack<float>(rg[u]), M = unpack<float>(rm[u]),
+                       V = unpack<float>(rv[u]);
+#pragma unroll
+          for (int l = 0; l < 4; ++l) adamw_elem<kOrder>(P.v[l], G.v[l], M.v[l], V.v[l], a.s, small_w);
+          const vec16 packed = pack<float>(P);
+          store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.p) + i * 16, packed);
+          if constexpr (kCopies)
+            for (int c = 0; c < a.ncopies; ++c) store16<TDM_NT_MASK_K3C>(reinterpret_cast<char*>(a.copy[c]) + i * 16, packed);
+          store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.m) + i * 16, pack<float>(M));
+          store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.v) + i * 16, pack<float>(V));
+        }
+      }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < a.n - nv * 4) {
+      const int64_t i = nv * 4 + threadIdx.x;
+      adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
+      if constexpr (kCopies)
+        for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
+    }
+  } else {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < a.n; i += stride) {
+      adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
+      if constexpr (kCopies)
+        for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
+    }
+  }
+}
+
+// ---------------------------------------------------------------- K2 + K3: ZeRO-2's whole step
+// For every element of every bucket segment, in one launch: the gradients of all ranks
+// are folded in the ring's order for the segment's chunk (K2), the sum is added to a zero
+// gradient shard as ZeRO's grad_shard.add_(mine) would (0.0f + mine: a -0.0 becomes +0.0),
+// the chunk's owner takes its AdamW step (K3), and the new parameter is written into every
+// rank's flat buffer (the all-gather). 4W + 12 bytes read and 4W + 8 written per element,
+// where reduce-scatter, add, AdamW and all-gather apart move 4(W+2) + 28 + 8(W-1).
+struct StepSegDev {
+  const char* g[TDM_MAX_WORLD];  // every rank's gradient for this tile
+  char* p[TDM_MAX_WORLD];        // every rank's copy of the parameters for this tile
+  char* m;                       // the owner's exp_avg
+  char* v;                       // the owner's exp_avg_sq
+  int64_t count;
+  int32_t chunk;                 // the owner
+  int32_t vec_ok;
+};
+
+#ifndef TDM_K23_UNROLL
+#define TDM_K23_UNROLL 4
+#endif
+#ifndef TDM_NT_MASK_K23
+#define TDM_NT_MASK_K23 TDM_NT_MASK_K3
+#endif
+
+// One tile (at most 16 KiB of every stream) of the step.
+template <int kWorld, int kDiv, int kOrder>
+__device__ __forceinline__ void step_tile(const StepSegDev& sg, int64_t at, int64_t n, const Divisor<float>& dv,
+                                          const tdm_adamw_scalars& s, bool small_w) {
+  constexpr int kU = kWorld <= 4 ? TDM_K23_UNROLL : 1;  // vectors per lane in flight, per stream
+  constexpr int kM = TDM_NT_MASK_K23;
+  {
+    const int c = sg.chunk;  // `at`: the tile's offset in bytes from the record's pointers; n: its elements
+    const char* gp[kWorld];
+    char* pp[kWorld];
+#pragma unroll
+    for (int k = 0; k < kWorld; ++k) {
+      gp[k] = sg.g[(c + 1 + k) % kWorld] + at;  // the fold ends with the owner's own term
+      pp[k] = sg.p[k] + at;
+    }
+    char* own = sg.p[c] + at;
+    char* const mm = sg.m + at;
+    char* const vv = sg.v + at;
+    auto one = [&](float grads_in_order[kWorld], float& P, float& M, float& V) {
+      float acc = scaled<float, kDiv>(grads_in_order[0], dv.divisor, dv.reciprocal);
+#pragma unroll
+      for (int k = 1; k < kWorld; ++k) acc = scaled<float, kDiv>(grads_in_order[k], dv.divisor, dv.reciprocal) + acc;
+      const float g = 0.0f + acc;  // grad_shard (zero) += mine
+      adamw_elem<kOrder>(P, g, M, V, s, small_w);
+    };
+    if (sg.vec_ok) {
+      const int64_t nv = n / 4;
+#pragma unroll
+      for (int u0 = 0; u0 < kUnroll; u0 += kU) {
+        vec16 in[kWorld][kU], rp[kU], rm[kU], rv[kU];
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          const int64_t v = threadIdx.x + static_cast<int64_t>(u0 + u) * kThreads;
+          if (v < nv) {
+#pragma unroll
+            for (int k = 0; k < kWorld; ++k) in[k][u] = load_stream<kM>(gp[k] + v * 16);
+            rp[u] = load_rmw<kM>(own + v * 16);
+            rm[u] = load_rmw<kM>(mm + v * 16);
+            rv[u] = load_rmw<kM>(vv + v * 16);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kU; ++u) {
+          const int64_t v = threadIdx.x + static_cast<int64_t>(u0 + u) * kThreads;
+          if (v < nv) {
+            Lanes<float> P = unpack<float>(rp[u]), M = unpack<float>(rm[u]), V = unpack<float>(rv[u]);
+#pragma unroll
+            for (int l = 0; l < 4; ++l) {
+              float gs[kWorld];
+#pragma unroll
+              for (int k = 0; k < kWorld; ++k) gs[k] = unpack<float>(in[k][u]).v[l];
+              one(gs, P.v[l], M.v[l], V.v[l]);
+            }
+            const vec16 packed = pack<float>(P);
+#pragma unroll
+            for (int q = 0; q < kWorld; ++q) store16<kM>(pp[q] + v * 16, packed);
+            store16<kM>(mm + v * 16, pack<float>(M));
+            store16<kM>(vv + v * 16, pack<float>(V));
+          }
+        }
+      }
+      if (threadIdx.x < n - nv * 4) {  // the tile's last few elements
+        const int64_t i = nv * 4 + threadIdx.x;
+        float gs[kWorld];
+#pragma unroll
+        for (int k = 0; k < kWorld; ++k) gs[k] = reinterpret_cast<const float*>(gp[k])[i];
+        float P = reinterpret_cast<float*>(own)[i], M = reinterpret_cast<float*>(mm)[i], V = reinterpret_cast<float*>(vv)[i];
+        one(gs, P, M, V);
+#pragma unroll
+        for (int q = 0; q < kWorld; ++q) reinterpret_cast<float*>(pp[q])[i] = P;
+        reinterpret_cast<float*>(mm)[i] = M;
+        reinterpret_cast<float*>(vv)[i] = V;
+      }
+    } else {
+      for (int64_t i = threadIdx.x; i < n; i += kThreads) {
+        float gs[kWorld];
+#pragma unroll
+        for (int k = 0; k < kWorld; ++k) gs[k] = reinterpret_cast<const float*>(gp[k])[i];
+        float P = reinterpret_cast<float*>(own)[i], M = reinterpret_cast<float*>(mm)[i], V = reinterpret_cast<float*>(vv)[i];
+        one(gs, P, M, V);
+#pragma unroll
+        for (int q = 0; q < kWorld; ++q) reinterpret_cast<float*>(pp[q])[i] = P;
+        reinterpret_cast<float*>(mm)[i] = M;
+        reinterpret_cast<float*>(vv)[i] = V;
+      }
+    }
+  }
+}
+
+template <int kWorld, int kDiv, int kOrder>
+__global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegDev* __restrict__ tiles, int64_t total,
+                                                                  Divisor<float> dv, tdm_adamw_scalars s) {
+  const bool small_w = __builtin_fabsf(s.w1) < 0.5f;
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    step_tile<kWorld, kDiv, kOrder>(tiles[tile], 0, tiles[tile].count, dv, s, small_w);
+  }
+}
+
+// The same for ONE segment, described in the kernel's arguments: no table to keep in
+// device memory. A rank that is a process of its own steps exactly one segment, its
+// shard, out of its peers' gradient buffers and into their parameter buffers.
+template <int kWorld, int kDiv, int kOrder>
+__global__ __launch_bounds__(kThreads) void k23_zero2_step_one_kernel(StepSegDev whole, int64_t total, Divisor<float> dv,
+                                                                      tdm_adamw_scalars s) {
+  const bool small_w = __builtin_fabsf(s.w1) < 0.5f;
+  constexpr int64_t kTileBytes = static_cast<int64_t>(kTileVecs) * 16;
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    const int64_t n = min(static_cast<int64_t>(kTileVecs) * 4, whole.count - tile * kTileVecs * 4);
+    step_tile<kWorld, kDiv, kOrder>(whole, tile * kTileBytes, n, dv, s, small_w);
+  }
+}
+
+}  // namespace
+
+}  // namespace tandem_hip
