@@ -377,26 +377,21 @@ void Engine::loop() {
 
 // ---------------------------------------------------------------- messages
 void Engine::signal(int dst, uint64_t length) {
-  Ring& r = mine_.entry(dst)->ring;
-  const uint64_t head = r.head.load(std::memory_order_relaxed);
-  r.length[head % slots_] = length;
-  r.head.store(head + 1, std::memory_order_release);  // the length is visible before the new head
+  ring_publish(mine_.entry(dst)->ring, slots_, length);
 }
 
 // The next message from src. Messages are consumed in order by the progress
 // thread (taken_), and released, possibly later, in the same order (tail).
 uint64_t Engine::await(int src) {
-  Ring& r = theirs_[src]->entry(rank_)->ring;
   const uint64_t at = taken_[src];
-  wait_until([&] { return r.head.load(std::memory_order_acquire) > at; }, timeout_s_,
-             "timed out waiting for a message from a peer rank");
+  const uint64_t length = ring_read(theirs_[src]->entry(rank_)->ring, at, slots_, timeout_s_,
+                                    "timed out waiting for a message from a peer rank");
   taken_[src] = at + 1;
-  return r.length[at % slots_];
+  return length;
 }
 
 void Engine::release(int src) {
-  Ring& r = theirs_[src]->entry(rank_)->ring;
-  r.tail.store(r.tail.load(std::memory_order_relaxed) + 1, std::memory_order_release);
+  ring_release(theirs_[src]->entry(rank_)->ring);
 }
 
 // "host" ordering. Completions are published strictly in the order they were
@@ -498,8 +493,7 @@ void Engine::barrier_now(bool after_gpu, uint64_t tag) {
     if (p == rank_) continue;
     Ring& r = mine_.entry(p)->ring;
     const uint64_t posted = posted_[p];
-    wait_until([&] { return posted - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots_); },
-               timeout_s_, "barrier: a peer rank never drained its messages");
+    ring_wait_for_room(r, posted, slots_, timeout_s_, "barrier: a peer rank never drained its messages");
     posted_[p] = posted + 1;
     signal(p, kEmpty);
   }
@@ -525,8 +519,7 @@ void Engine::put(int dst, const char* src, int64_t numel, int dtype, int scale_w
   // Room in the message ring means fewer than `slots` messages are unreleased, so
   // fewer than `slots` pieces are: dst has released slot j's previous piece ...
   const uint64_t posted = posted_[dst];
-  wait_until([&] { return posted - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots_); }, timeout_s_,
-             "put: the peer never freed a slot");
+  ring_wait_for_room(r, posted, slots_, timeout_s_, "put: the peer never freed a slot");
   if (use_events_ && k >= static_cast<uint64_t>(slots_)) {
     // ... and enqueued its reads of it before recording free[j]: wait for those reads.
     check_hip(hipStreamWaitEvent(stream_, peer_free_[dst][j], 0), "hipStreamWaitEvent (free)");

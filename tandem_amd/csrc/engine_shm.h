@@ -201,4 +201,32 @@ void wait_until(Ready ready, double timeout_s, const char* what) {
   }
 }
 
+// ---------------------------------------------------------------- ring operations
+// The sender publishes message k into length[k % slots] and advances head; the receiver
+// reads messages in order and advances tail when it is done with one (possibly later,
+// in the same order). Room for a new message: fewer than `slots` unreleased ones.
+inline void ring_publish(Ring& r, int slots, uint64_t length) {
+  const uint64_t head = r.head.load(std::memory_order_relaxed);
+  r.length[head % slots] = length;
+  r.head.store(head + 1, std::memory_order_release);  // the length is visible before the new head
+}
+
+inline bool ring_has_room(const Ring& r, uint64_t posted, int slots) {
+  return posted - r.tail.load(std::memory_order_acquire) < static_cast<uint64_t>(slots);
+}
+
+inline void ring_wait_for_room(const Ring& r, uint64_t posted, int slots, double timeout_s, const char* what) {
+  wait_until([&] { return ring_has_room(r, posted, slots); }, timeout_s, what);
+}
+
+// Message number `at` (0-based, the count of messages the receiver has read so far).
+inline uint64_t ring_read(const Ring& r, uint64_t at, int slots, double timeout_s, const char* what) {
+  wait_until([&] { return r.head.load(std::memory_order_acquire) > at; }, timeout_s, what);
+  return r.length[at % slots];
+}
+
+inline void ring_release(Ring& r) {
+  r.tail.store(r.tail.load(std::memory_order_relaxed) + 1, std::memory_order_release);
+}
+
 }  // namespace tandem_hip
