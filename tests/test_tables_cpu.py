@@ -1,0 +1,146 @@
+"""The host half of K2 and K2+K3: tdm_k2_table_* and tdm_k23_table_* cut segments into
+tiles of 16 KiB per stream and write the records the kernels walk. They build an image in
+host memory and launch nothing, so they are checked here without a GPU: tile counts,
+every record's pointers, counts, owner and alignment flag, and what they refuse."""
+
+import ctypes
+
+import numpy as np
+import pytest
+
+from tandem_amd import _lib
+from tandem_amd._lib import lib
+
+W = _lib.TDM_MAX_WORLD
+F32, F64, BF16, EINVAL = 0, 1, 3, 1  # enum tdm_dtype and TDM_EINVAL of include/tandem_hip.h
+FOLD_REC = np.dtype([("src", np.uint64, W), ("dst", np.uint64, W), ("count", np.int64), ("chunk", np.int32), ("vec_ok", np.int32)])
+STEP_REC = np.dtype([("g", np.uint64, W), ("p", np.uint64, W), ("m", np.uint64), ("v", np.uint64), ("count", np.int64),
+                     ("chunk", np.int32), ("vec_ok", np.int32)])
+TILE_BYTES = 16384
+
+
+def fold_segs(world, es, rows):
+    """rows: (count, chunk, byte offset added to every pointer)."""
+    segs = (_lib.FoldSeg * len(rows))()
+    for k, (count, chunk, off) in enumerate(rows):
+        for r in range(world):
+            segs[k].src[r] = (1 << 32) * (r + 1) + (k << 24) + off
+            segs[k].dst[r] = (1 << 40) * (r + 1) + (k << 24) + off if r != 1 or world == 1 else 0  # rank 1 receives nothing
+        segs[k].count, segs[k].chunk = count, chunk
+    return segs
+
+
+@pytest.mark.parametrize("dtype,es", [(F32, 4), (F64, 8), (BF16, 2)])
+@pytest.mark.parametrize("world", [1, 2, 3, 8])
+def test_fold_table_records(world, dtype, es):
+    tile = TILE_BYTES // es
+    rows = [(1, 0, 0), (tile, world - 1, 0), (tile + 1, world // 2, es), (0, 0, 0), (5 * tile - 3, 0, 16), (17, world - 1, 32 + es)]
+    segs = fold_segs(world, es, rows)
+    ntiles = lib().tdm_k2_table_tiles(segs, len(rows), dtype)
+    assert ntiles == sum(-(-c // tile) for c, _, _ in rows)
+    nbytes = lib().tdm_k2_table_bytes(segs, len(rows), dtype)
+    assert nbytes == ntiles * FOLD_REC.itemsize
+    image = np.full(nbytes, 0xAB, np.uint8)
+    assert lib().tdm_k2_table_build(segs, len(rows), world, dtype, ctypes.c_void_p(image.ctypes.data)) == 0
+    recs = image.view(FOLD_REC)
+    at = 0
+    for k, (count, chunk, off) in enumerate(rows):
+        done = 0
+        while done < count:
+            rec = recs[at]
+            assert rec["count"] == min(tile, count - done) and rec["chunk"] == chunk
+            assert rec["vec_ok"] == int(off % 16 == 0)
+            for r in range(world):
+                assert rec["src"][r] == segs[k].src[r] + done * es
+                assert rec["dst"][r] == (segs[k].dst[r] + done * es if segs[k].dst[r] else 0)
+            assert not rec["src"][world:].any() and not rec["dst"][world:].any()  # unused ranks stay zero
+            done += int(rec["count"])
+            at += 1
+    assert at == ntiles
+
+
+def step_segs(world, rows):
+    segs = (_lib.StepSeg * len(rows))()
+    for k, (count, chunk, off) in enumerate(rows):
+        for r in range(world):
+            segs[k].grad[r] = (1 << 32) * (r + 1) + (k << 24) + off
+            segs[k].param[r] = (1 << 40) * (r + 1) + (k << 24) + off
+        segs[k].exp_avg, segs[k].exp_avg_sq = (1 << 50) + (k << 24) + off, (1 << 51) + (k << 24) + off
+        segs[k].count, segs[k].chunk = count, chunk
+    return segs
+
+
+@pytest.mark.parametrize("world", [1, 2, 4, 7])
+def test_step_table_records(world):
+    tile = TILE_BYTES // 4
+    rows = [(3, 0, 0), (2 * tile, world - 1, 0), (0, 0, 0), (tile + 9, world // 2, 4), (4 * tile - 1, 0, 48)]
+    segs = step_segs(world, rows)
+    ntiles = lib().tdm_k23_table_tiles(segs, len(rows))
+    assert ntiles == sum(-(-c // tile) for c, _, _ in rows)
+    nbytes = lib().tdm_k23_table_bytes(segs, len(rows))
+    assert nbytes == ntiles * STEP_REC.itemsize
+    image = np.full(nbytes, 0xCD, np.uint8)
+    assert lib().tdm_k23_table_build(segs, len(rows), world, ctypes.c_void_p(image.ctypes.data)) == 0
+    recs = image.view(STEP_REC)
+    at = 0
+    for k, (count, chunk, off) in enumerate(rows):
+        done = 0
+        while done < count:
+            rec = recs[at]
+            assert rec["count"] == min(tile, count - done) and rec["chunk"] == chunk and rec["vec_ok"] == int(off % 16 == 0)
+            for r in range(world):
+                assert rec["g"][r] == segs[k].grad[r] + done * 4 and rec["p"][r] == segs[k].param[r] + done * 4
+            assert rec["m"] == segs[k].exp_avg + done * 4 and rec["v"] == segs[k].exp_avg_sq + done * 4
+            assert not rec["g"][world:].any() and not rec["p"][world:].any()
+            done += int(rec["count"])
+            at += 1
+    assert at == ntiles
+
+
+def test_empty_tables_and_refusals():
+    L = lib()
+    none = (_lib.FoldSeg * 1)()
+    assert L.tdm_k2_table_tiles(none, 0, F32) == 0 and L.tdm_k2_table_bytes(none, 0, F32) == 16
+    assert L.tdm_k2_table_tiles(none, -1, F32) == -1 and L.tdm_k2_table_tiles(none, 1, 99) == -1
+    assert L.tdm_k2_table_tiles(None, 1, F32) == -1
+    image = np.zeros(1 << 16, np.uint8)
+    ptr = ctypes.c_void_p(image.ctypes.data)
+
+    def refused(call, needle):
+        assert call() == EINVAL
+        assert needle in L.tdm_last_error().decode(), L.tdm_last_error().decode()
+
+    good = fold_segs(2, 4, [(10, 1, 0)])
+    assert L.tdm_k2_table_build(good, 1, 2, F32, ptr) == 0
+    refused(lambda: L.tdm_k2_table_build(good, 1, 0, F32, ptr), "world")
+    refused(lambda: L.tdm_k2_table_build(good, 1, 9, F32, ptr), "world")
+    refused(lambda: L.tdm_k2_table_build(good, 1, 2, 99, ptr), "dtype")
+    refused(lambda: L.tdm_k2_table_build(good, 1, 2, F32, None), "bad table arguments")
+    refused(lambda: L.tdm_k2_table_build(good, 1, 1, F32, ptr), "chunk")  # chunk 1 of a world of one
+    bad = fold_segs(2, 4, [(10, 0, 0)])
+    bad[0].count = -1
+    refused(lambda: L.tdm_k2_table_build(bad, 1, 2, F32, ptr), "negative count")
+    bad = fold_segs(2, 4, [(10, 0, 2)])
+    refused(lambda: L.tdm_k2_table_build(bad, 1, 2, F32, ptr), "aligned")
+    bad = fold_segs(2, 4, [(10, 0, 0)])
+    bad[0].src[1] = 0
+    refused(lambda: L.tdm_k2_table_build(bad, 1, 2, F32, ptr), "NULL source")
+
+    step = step_segs(2, [(10, 1, 0)])
+    assert L.tdm_k23_table_build(step, 1, 2, ptr) == 0
+    assert L.tdm_k23_table_tiles(step, -1) == -1 and L.tdm_k23_table_bytes(None, 2) == -1
+    refused(lambda: L.tdm_k23_table_build(step, 1, 9, ptr), "world")
+    refused(lambda: L.tdm_k23_table_build(step, 1, 1, ptr), "chunk")
+    refused(lambda: L.tdm_k23_table_build(step, 1, 2, None), "bad table arguments")
+    for field, needle in (("exp_avg", "NULL optimizer state"), ("exp_avg_sq", "NULL optimizer state")):
+        bad = step_segs(2, [(10, 0, 0)])
+        setattr(bad[0], field, 0)
+        refused(lambda: L.tdm_k23_table_build(bad, 1, 2, ptr), needle)
+    bad = step_segs(2, [(10, 0, 0)])
+    bad[0].param[1] = 0
+    refused(lambda: L.tdm_k23_table_build(bad, 1, 2, ptr), "NULL gradient or parameter")
+    bad = step_segs(2, [(10, 0, 2)])
+    refused(lambda: L.tdm_k23_table_build(bad, 1, 2, ptr), "aligned")
+    bad = step_segs(2, [(10, 0, 0)])
+    bad[0].count = -5
+    refused(lambda: L.tdm_k23_table_build(bad, 1, 2, ptr), "negative count")
