@@ -533,7 +533,10 @@ def main():
     # The two multi-process figures first, while this process has not touched the GPU.
     cpu = fsdp = None
     if not args.quick and not args.no_cpu:
-        cpu = cpu_baseline(args.mib, 15)
+        try:
+            cpu = cpu_baseline(args.mib, 15)
+        except Exception as e:  # reported, not measured by: the GPU figures must still come out
+            cpu = {"error": repr(e)[:300]}
     ipc = train = train4 = None
     if not args.quick and not args.no_fsdp:
         try:
@@ -616,9 +619,10 @@ def main():
             line["train_step_2_processes"] = train
         if train4 is not None:
             line["train_step_4_processes"] = train4
-        if cpu is not None:
+        if cpu is not None and "error" not in cpu:
             cpu["gpu_over_cpu"] = round(line["value"] / cpu["value"], 1)
             cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["one_launch_ms"], 1)
+        if cpu is not None:
             line["cpu_baseline"] = cpu
     line["device"] = device_name(_lib)
     print(json.dumps(line), flush=True)
