@@ -120,7 +120,7 @@ typedef struct tdm_fold_seg {
   int32_t reserved;
 } tdm_fold_seg;
 
-/* The device table holds one record per 16 KiB tile of every segment. Number of tiles
+/* The device table holds one record per 8 KiB tile of every segment. Number of tiles
  * and bytes of device memory the table of these segments needs (-1: bad arguments). */
 int64_t tdm_k2_table_tiles(const tdm_fold_seg* segs, int nseg, int dtype);
 int64_t tdm_k2_table_bytes(const tdm_fold_seg* segs, int nseg, int dtype);

@@ -2,7 +2,7 @@
 // K1 ring-step reduce / copy, K2 bucket fold, K3 sharded AdamW, K4 unit gather.
 //
 // All four are HBM-bound element-wise passes, so they share one shape: a launch
-// covers a small table of streams, the work is cut into tiles of 16 KiB per
+// covers a small table of streams, the work is cut into tiles of 4 to 8 KiB per
 // stream, workgroups walk the tiles grid-stride (consecutive workgroups touch
 // consecutive tiles, so a sweep of the grid is one contiguous multi-MiB slot of
 // every stream), and each lane keeps several independent 16-byte loads in flight
@@ -174,7 +174,7 @@ void launch_copy(const PairTable& tab, int64_t tiles, int world, int policy, hip
 template <typename T, int kWorld, bool kAcc>
 void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(kWorld);
-  const dim3 grid(grid_for(tiles)), block(kThreads);
+  const dim3 grid(grid_for(tiles * (kWorld <= 2 ? 2 : 1))), block(kThreads);  // up to two ranks: half a record per workgroup
   const FoldSegDev* img = static_cast<const FoldSegDev*>(image);
   switch (div_kind(kWorld, average != 0)) {
     case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, 0, stream, img, tiles, dv); break;
@@ -670,7 +670,7 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
         if (a % es || b % es) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to the element size");
         vec = vec && a % 16 == 0 && b % 16 == 0;
       }
-      for (int64_t at = 0; at < s.count; at += tile_elems) {  // a tile's byte offset is a multiple of 16 KiB
+      for (int64_t at = 0; at < s.count; at += tile_elems) {  // a tile's byte offset is a multiple of 8 KiB
         FoldSegDev& rec = out[tiles++];
         for (int r = 0; r < world; ++r) {
           rec.src[r] = static_cast<const char*>(s.src[r]) + at * es;

@@ -21,7 +21,7 @@ namespace {
 #define TDM_THREADS 256
 #endif
 #ifndef TDM_UNROLL
-#define TDM_UNROLL 4
+#define TDM_UNROLL 2
 #endif
 constexpr int kThreads = TDM_THREADS;
 constexpr int kUnroll = TDM_UNROLL;             // 16-byte vectors per lane per tile and stream
@@ -38,8 +38,8 @@ constexpr int kK1TileVecs = kThreads * kK1Unroll;
 #endif
 constexpr int kCopyUnroll = TDM_COPY_UNROLL;
 constexpr int kCopyTileVecs = kThreads * kCopyUnroll;
-constexpr int kTileVecs = kThreads * kUnroll;   // 1024 vectors = 16 KiB of every stream
-// Measured on MI355X: one 16 KiB tile per workgroup beats a persistent grid-stride
+constexpr int kTileVecs = kThreads * kUnroll;   // 512 vectors = 8 KiB of every stream
+// Measured on MI355X: one tile per workgroup beats a persistent grid-stride
 // loop by 5-8% (the hardware dispatcher balances 8 XCDs better than a fixed stride),
 // so the grid covers the tiles one to one up to 256 Ki workgroups (4 GiB per stream)
 // and strides only beyond that.
@@ -376,19 +376,27 @@ struct FoldSegDev {
 
 // One tile of one segment: W loads per element, the fold in ring order, W stores.
 // kAcc: the result is added into each destination (dst = dst + sum) instead of replacing it.
-template <typename T, int kWorld, int kDiv, bool kAcc, int kMask>
+// kRounds: the part of the segment one call covers, in rounds of one vector per lane
+// (kThreads vectors = 4 KiB of every stream); `t` counts such parts from the segment's start.
+// How much one workgroup takes in one go matters more than how many loads a lane keeps in
+// flight: the fewer streams a launch has, the smaller the part that serves it best (a
+// two-rank bucket fold: 4 KiB, -4 %; worlds 3 and more, and the whole ZeRO-2 step: 8 KiB,
+// -2.5 to -6.5 %, all against 16 KiB).
+template <typename T, int kWorld, int kDiv, bool kAcc, int kMask, int kRounds = kUnroll>
 __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const Divisor<T>& dv) {
   using A = typename Elem<T>::acc;
   constexpr int L = lanes<T>();
 #ifndef TDM_K2_UNROLL_W2
-#define TDM_K2_UNROLL_W2 4
+#define TDM_K2_UNROLL_W2 2
 #endif
 #ifndef TDM_K2_UNROLL
-#define TDM_K2_UNROLL 4
+#define TDM_K2_UNROLL 2
 #endif
-  // vectors per lane per tile step, per rank (worlds 3-4: 4 beats 2 by 2-3 %; beyond that the registers run out)
-  constexpr int kU = kWorld <= 2 ? TDM_K2_UNROLL_W2 : kWorld <= 4 ? TDM_K2_UNROLL : 2;
-  constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
+  // vectors per lane in flight, per rank
+  constexpr int kWant = kWorld <= 2 ? TDM_K2_UNROLL_W2 : kWorld <= 4 ? TDM_K2_UNROLL : 2;
+  constexpr int kU = kWant < kRounds ? kWant : kRounds;
+  constexpr int kPartVecs = kThreads * kRounds;
+  constexpr int64_t kTileElems = static_cast<int64_t>(kPartVecs) * L;
   const int64_t n = sg.count;
   const int c = sg.chunk;
   // ring order: the fold starts at rank chunk+1 and ends with the chunk's owner
@@ -402,8 +410,8 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
   if (sg.vec_ok) {
     const int64_t nv = n / L;
 #pragma unroll
-    for (int u0 = 0; u0 < kUnroll; u0 += kU) {
-      const int64_t vbase = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u0) * kThreads;
+    for (int u0 = 0; u0 < kRounds; u0 += kU) {
+      const int64_t vbase = t * kPartVecs + threadIdx.x + static_cast<int64_t>(u0) * kThreads;
       vec16 in[kWorld][kU];
 #pragma unroll
       for (int k = 0; k < kWorld; ++k)
@@ -461,7 +469,7 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
     }
   } else {
     const int64_t e0 = t * kTileElems + threadIdx.x;
-    for (int k2 = 0; k2 < kUnroll * L; ++k2) {
+    for (int k2 = 0; k2 < kRounds * L; ++k2) {
       const int64_t i = e0 + static_cast<int64_t>(k2) * kThreads;
       if (i < n) {
         A acc = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[0])[i]), dv.divisor, dv.reciprocal);
@@ -485,8 +493,10 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
 template <typename T, int kWorld, int kDiv, bool kAcc>
 __global__ __launch_bounds__(kThreads) void k2_fold_kernel(const FoldSegDev* __restrict__ tiles, int64_t total,
                                                            Divisor<T> dv) {
-  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
-    fold_tile<T, kWorld, kDiv, kAcc, TDM_NT_MASK_K2>(tiles[tile], 0, dv);
+  // a record describes 8 KiB of every stream; up to two ranks a workgroup takes half of one at a time
+  constexpr int kParts = kWorld <= 2 && kUnroll % 2 == 0 ? 2 : 1;
+  for (int64_t part = blockIdx.x; part < total * kParts; part += gridDim.x) {
+    fold_tile<T, kWorld, kDiv, kAcc, TDM_NT_MASK_K2, kUnroll / kParts>(tiles[part / kParts], part % kParts, dv);
   }
 }
 
@@ -621,13 +631,13 @@ struct StepSegDev {
 };
 
 #ifndef TDM_K23_UNROLL
-#define TDM_K23_UNROLL 4
+#define TDM_K23_UNROLL 2
 #endif
 #ifndef TDM_NT_MASK_K23
 #define TDM_NT_MASK_K23 TDM_NT_MASK_K3
 #endif
 
-// One tile (at most 16 KiB of every stream) of the step.
+// One tile (at most 8 KiB of every stream) of the step.
 template <int kWorld, int kDiv, int kOrder>
 __device__ __forceinline__ void step_tile(const StepSegDev& sg, int64_t at, int64_t n, const Divisor<float>& dv,
                                           const tdm_adamw_scalars& s, bool small_w) {
