@@ -56,6 +56,9 @@ int tdm_device_info(int device, char* name, int name_len, int* compute_units, in
  * streaming kernels (0 restores the built-in default). Not needed for correctness. */
 int tdm_set_blocks_per_cu(int blocks);
 
+/* Bytes of every stream that one record of the K2 and K2+K3 device tables covers (a build constant). */
+int tdm_table_tile_bytes(void);
+
 /* ---- K1: one ring step -------------------------------------------------- */
 
 /* The reduce half of a ring reduce-scatter step, for up to TDM_MAX_PAIRS
@@ -120,7 +123,7 @@ typedef struct tdm_fold_seg {
   int32_t reserved;
 } tdm_fold_seg;
 
-/* The device table holds one record per 8 KiB tile of every segment. Number of tiles
+/* The device table holds one record per tile (tdm_table_tile_bytes() of every stream) of every segment. Number of tiles
  * and bytes of device memory the table of these segments needs (-1: bad arguments). */
 int64_t tdm_k2_table_tiles(const tdm_fold_seg* segs, int nseg, int dtype);
 int64_t tdm_k2_table_bytes(const tdm_fold_seg* segs, int nseg, int dtype);

@@ -2,7 +2,7 @@
 // K1 ring-step reduce / copy, K2 bucket fold, K3 sharded AdamW, K4 unit gather.
 //
 // All four are HBM-bound element-wise passes, so they share one shape: a launch
-// covers a small table of streams, the work is cut into tiles of 4 to 8 KiB per
+// covers a small table of streams, the work is cut into tiles of 2 to 4 KiB per
 // stream, workgroups walk the tiles grid-stride (consecutive workgroups touch
 // consecutive tiles, so a sweep of the grid is one contiguous multi-MiB slot of
 // every stream), and each lane keeps several independent 16-byte loads in flight
@@ -144,7 +144,7 @@ void launch_reduce(const PairTable& tab, int64_t tiles, int world, bool any_scal
 template <typename T, int kMask>
 void launch_copy_m(const PairTable& tab, int64_t tiles, int world, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(world);
-  const dim3 grid(grid_for(tiles)), block(kThreads);
+  const dim3 grid(grid_for(tiles)), block(kCopyThreads);
   switch (div_kind(world, true)) {
     case 0: hipLaunchKernelGGL((k1_copy_kernel<T, 0, kMask>), grid, block, 0, stream, tab, dv); break;
     case 1: hipLaunchKernelGGL((k1_copy_kernel<T, 1, kMask>), grid, block, 0, stream, tab, dv); break;
@@ -174,7 +174,7 @@ void launch_copy(const PairTable& tab, int64_t tiles, int world, int policy, hip
 template <typename T, int kWorld, bool kAcc>
 void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(kWorld);
-  const dim3 grid(grid_for(tiles * (kWorld <= 2 ? 2 : 1))), block(kThreads);  // up to two ranks: half a record per workgroup
+  const dim3 grid(grid_for(tiles * FoldShape<kWorld>::kParts)), block(FoldShape<kWorld>::kT);
   const FoldSegDev* img = static_cast<const FoldSegDev*>(image);
   switch (div_kind(kWorld, average != 0)) {
     case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, 0, stream, img, tiles, dv); break;
@@ -609,6 +609,8 @@ int tdm_local_all_reduce(void* const* bufs, int world, int64_t numel, int dtype,
   });
 }
 
+int tdm_table_tile_bytes(void) { return kTileVecs * 16; }
+
 int tdm_set_blocks_per_cu(int blocks) {
   return guard([&] {
     if (blocks < 0 || blocks > 1024) throw Invalid("blocks per compute unit must be in [0, 1024]");
@@ -670,7 +672,7 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
         if (a % es || b % es) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to the element size");
         vec = vec && a % 16 == 0 && b % 16 == 0;
       }
-      for (int64_t at = 0; at < s.count; at += tile_elems) {  // a tile's byte offset is a multiple of 8 KiB
+      for (int64_t at = 0; at < s.count; at += tile_elems) {  // a tile's byte offset is a multiple of 4 KiB
         FoldSegDev& rec = out[tiles++];
         for (int r = 0; r < world; ++r) {
           rec.src[r] = static_cast<const char*>(s.src[r]) + at * es;

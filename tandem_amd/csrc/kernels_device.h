@@ -18,30 +18,43 @@ namespace {
 
 
 #ifndef TDM_THREADS
-#define TDM_THREADS 256
+#define TDM_THREADS 128
 #endif
 #ifndef TDM_UNROLL
 #define TDM_UNROLL 2
 #endif
+// Workgroups of two waves, two 16-byte vectors per lane and stream: 4 KiB of every stream per
+// workgroup. How much one workgroup takes matters more than how many loads a lane keeps in flight,
+// and it is the writes that are sensitive to it (a write-only probe over 2 GiB: 6.9 TB/s at 4 KiB
+// per workgroup, 6.0 at 8-16 KiB, 5.7 at 32 KiB, 4.9 from a persistent grid, 5.5 at 2 KiB; read-only
+// 7.0-7.1 at any of these). Against four waves and 8 KiB, in A/B runs inside one process on several
+// machines: the ring's copy step 2.4-3.9 % faster, the two-rank bucket fold 3-7 %, the single-launch
+// all-reduce at 256 MiB between 2.5 % faster and 1.8 % slower, K1's reduce step and AdamW equal, the
+// one-launch ZeRO-2 step equal to 1.5 % slower. One wave per workgroup is slower throughout (too
+// many workgroups to dispatch), and so is 16 KiB.
 constexpr int kThreads = TDM_THREADS;
 constexpr int kUnroll = TDM_UNROLL;             // 16-byte vectors per lane per tile and stream
 #ifndef TDM_K1_UNROLL
 #define TDM_K1_UNROLL 2
 #endif
-// K1 and the copy kernel cut their pairs into tiles of their own, 8 KiB per stream: against 16 KiB the
-// ring (reduce-scatter + all-gather, world 4) runs 3 % faster at 64 MiB per rank (6.95 vs 6.74 TB/s), 2 %
-// at 16 MiB and equally fast at 256 MiB; different tile sizes for the two kernels are worse than either.
+// K1 and the copy kernel cut their pairs into tiles of their own. Both must use the same tile: a ring
+// whose reduce steps and gather steps differ in tile size or workgroup size is up to 5 % slower at
+// 64 MiB per rank than with either size for both (what one kernel leaves in the caches, the other finds).
 constexpr int kK1Unroll = TDM_K1_UNROLL;
 constexpr int kK1TileVecs = kThreads * kK1Unroll;
+#ifndef TDM_COPY_THREADS
+#define TDM_COPY_THREADS TDM_THREADS
+#endif
 #ifndef TDM_COPY_UNROLL
 #define TDM_COPY_UNROLL TDM_K1_UNROLL
 #endif
+constexpr int kCopyThreads = TDM_COPY_THREADS;
 constexpr int kCopyUnroll = TDM_COPY_UNROLL;
-constexpr int kCopyTileVecs = kThreads * kCopyUnroll;
-constexpr int kTileVecs = kThreads * kUnroll;   // 512 vectors = 8 KiB of every stream
+constexpr int kCopyTileVecs = kCopyThreads * kCopyUnroll;
+constexpr int kTileVecs = kThreads * kUnroll;   // 256 vectors = 4 KiB of every stream
 // Measured on MI355X: one tile per workgroup beats a persistent grid-stride
 // loop by 5-8% (the hardware dispatcher balances 8 XCDs better than a fixed stride),
-// so the grid covers the tiles one to one up to 256 Ki workgroups (4 GiB per stream)
+// so the grid covers the tiles one to one up to 256 Ki workgroups (1-2 GiB per stream)
 // and strides only beyond that.
 constexpr int kDefaultBlocksPerCu = 1024;
 
@@ -300,7 +313,7 @@ __device__ __forceinline__ T copy_elem(T s, const Divisor<T>& dv) {
 }
 
 template <typename T, int kDiv, int kMask>
-__global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Divisor<T> dv) {
+__global__ __launch_bounds__(kCopyThreads) void k1_copy_kernel(PairTable tab, Divisor<T> dv) {
   constexpr int L = lanes<T>();
   constexpr int64_t kTileElems = static_cast<int64_t>(kCopyTileVecs) * L;
   const int64_t total = tab.tile_end[tab.npairs - 1];
@@ -320,7 +333,7 @@ __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Diviso
       if ((t + 1) * kCopyTileVecs <= nv) {
         vec16 b[kCopyUnroll];
 #pragma unroll
-        for (int k = 0; k < kCopyUnroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kThreads) * 16);
+        for (int k = 0; k < kCopyUnroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kCopyThreads) * 16);
 #pragma unroll
         for (int k = 0; k < kCopyUnroll; ++k) {
           if constexpr (kDiv != 0) {
@@ -329,12 +342,12 @@ __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Diviso
             for (int l = 0; l < L; ++l) y.v[l] = copy_elem<T, kDiv>(y.v[l], dv);
             b[k] = pack<T>(y);
           }
-          store16<kMask>(dvp + (v0 + k * kThreads) * 16, b[k]);
+          store16<kMask>(dvp + (v0 + k * kCopyThreads) * 16, b[k]);
         }
       } else {
 #pragma unroll
         for (int k = 0; k < kCopyUnroll; ++k) {
-          const int64_t v = v0 + k * kThreads;
+          const int64_t v = v0 + k * kCopyThreads;
           if (v < nv) {
             Lanes<T> y = unpack<T>(load_stream<kMask>(svp + v * 16));
 #pragma unroll
@@ -354,7 +367,7 @@ __global__ __launch_bounds__(kThreads) void k1_copy_kernel(PairTable tab, Diviso
       const int64_t e0 = t * kTileElems + threadIdx.x;
 #pragma unroll 4
       for (int k = 0; k < kCopyUnroll * L; ++k) {
-        const int64_t i = e0 + static_cast<int64_t>(k) * kThreads;
+        const int64_t i = e0 + static_cast<int64_t>(k) * kCopyThreads;
         if (i < n) dst[i] = copy_elem<T, kDiv>(src[i], dv);
       }
     }
@@ -377,12 +390,8 @@ struct FoldSegDev {
 // One tile of one segment: W loads per element, the fold in ring order, W stores.
 // kAcc: the result is added into each destination (dst = dst + sum) instead of replacing it.
 // kRounds: the part of the segment one call covers, in rounds of one vector per lane
-// (kThreads vectors = 4 KiB of every stream); `t` counts such parts from the segment's start.
-// How much one workgroup takes in one go matters more than how many loads a lane keeps in
-// flight: the fewer streams a launch has, the smaller the part that serves it best (a
-// two-rank bucket fold: 4 KiB, -4 %; worlds 3 and more, and the whole ZeRO-2 step: 8 KiB,
-// -2.5 to -6.5 %, all against 16 KiB).
-template <typename T, int kWorld, int kDiv, bool kAcc, int kMask, int kRounds = kUnroll>
+// (kT vectors, kT = the workgroup's lanes); `t` counts such parts from the segment's start.
+template <typename T, int kWorld, int kDiv, bool kAcc, int kMask, int kRounds = kUnroll, int kT = kThreads>
 __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const Divisor<T>& dv) {
   using A = typename Elem<T>::acc;
   constexpr int L = lanes<T>();
@@ -395,7 +404,7 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
   // vectors per lane in flight, per rank
   constexpr int kWant = kWorld <= 2 ? TDM_K2_UNROLL_W2 : kWorld <= 4 ? TDM_K2_UNROLL : 2;
   constexpr int kU = kWant < kRounds ? kWant : kRounds;
-  constexpr int kPartVecs = kThreads * kRounds;
+  constexpr int kPartVecs = kT * kRounds;
   constexpr int64_t kTileElems = static_cast<int64_t>(kPartVecs) * L;
   const int64_t n = sg.count;
   const int c = sg.chunk;
@@ -411,18 +420,18 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
     const int64_t nv = n / L;
 #pragma unroll
     for (int u0 = 0; u0 < kRounds; u0 += kU) {
-      const int64_t vbase = t * kPartVecs + threadIdx.x + static_cast<int64_t>(u0) * kThreads;
+      const int64_t vbase = t * kPartVecs + threadIdx.x + static_cast<int64_t>(u0) * kT;
       vec16 in[kWorld][kU];
 #pragma unroll
       for (int k = 0; k < kWorld; ++k)
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
-          const int64_t v = vbase + u * kThreads;
+          const int64_t v = vbase + u * kT;
           if (v < nv) in[k][u] = load_stream<kMask>(sp[k] + v * 16);
         }
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
-        const int64_t v = vbase + u * kThreads;
+        const int64_t v = vbase + u * kT;
         if (v < nv) {
           Lanes<T> out;
 #pragma unroll
@@ -470,7 +479,7 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
   } else {
     const int64_t e0 = t * kTileElems + threadIdx.x;
     for (int k2 = 0; k2 < kRounds * L; ++k2) {
-      const int64_t i = e0 + static_cast<int64_t>(k2) * kThreads;
+      const int64_t i = e0 + static_cast<int64_t>(k2) * kT;
       if (i < n) {
         A acc = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[0])[i]), dv.divisor, dv.reciprocal);
 #pragma unroll
@@ -489,14 +498,23 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
   }
 }
 
-// Table in device memory, one record per tile (many segments: DDP's buckets).
+// Table in device memory, one record per tile (many segments: DDP's buckets). A record
+// describes 4 KiB of every stream; up to two ranks it is taken in two parts of 2 KiB, by one
+// workgroup each (the fewer streams a launch has, the smaller the part that serves it best).
+template <int kWorld>
+struct FoldShape {
+  static constexpr bool kSmall = kWorld <= 2 && kThreads >= 128 && kTileVecs % 128 == 0;
+  static constexpr int kT = kSmall ? 128 : kThreads;
+  static constexpr int kRounds = kSmall ? 1 : kUnroll;
+  static constexpr int kParts = kTileVecs / (kT * kRounds);
+};
+
 template <typename T, int kWorld, int kDiv, bool kAcc>
 __global__ __launch_bounds__(kThreads) void k2_fold_kernel(const FoldSegDev* __restrict__ tiles, int64_t total,
                                                            Divisor<T> dv) {
-  // a record describes 8 KiB of every stream; up to two ranks a workgroup takes half of one at a time
-  constexpr int kParts = kWorld <= 2 && kUnroll % 2 == 0 ? 2 : 1;
-  for (int64_t part = blockIdx.x; part < total * kParts; part += gridDim.x) {
-    fold_tile<T, kWorld, kDiv, kAcc, TDM_NT_MASK_K2, kUnroll / kParts>(tiles[part / kParts], part % kParts, dv);
+  using S = FoldShape<kWorld>;
+  for (int64_t part = blockIdx.x; part < total * S::kParts; part += gridDim.x) {
+    fold_tile<T, kWorld, kDiv, kAcc, TDM_NT_MASK_K2, S::kRounds, S::kT>(tiles[part / S::kParts], part % S::kParts, dv);
   }
 }
 
@@ -637,7 +655,7 @@ struct StepSegDev {
 #define TDM_NT_MASK_K23 TDM_NT_MASK_K3
 #endif
 
-// One tile (at most 8 KiB of every stream) of the step.
+// One tile (at most 4 KiB of every stream) of the step.
 template <int kWorld, int kDiv, int kOrder>
 __device__ __forceinline__ void step_tile(const StepSegDev& sg, int64_t at, int64_t n, const Divisor<float>& dv,
                                           const tdm_adamw_scalars& s, bool small_w) {

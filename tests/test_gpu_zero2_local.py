@@ -213,7 +213,8 @@ def test_one_launch_step_through_the_c_abi(world, average):
                 segs[k].count, segs[k].chunk = n, k % world
                 at += -(-n // 4) * 4 + 4  # keeps every segment's start at the same offset from 16-byte alignment
             ntiles = lib().tdm_k23_table_tiles(segs, nseg)
-            assert ntiles == sum(-(-n // 2048) for n in counts)  # 8 KiB of every stream per tile
+            tile = lib().tdm_table_tile_bytes() // 4
+            assert ntiles == sum(-(-n // tile) for n in counts)
             image = torch.empty(lib().tdm_k23_table_bytes(segs, nseg), dtype=torch.uint8)
             check(lib().tdm_k23_table_build(segs, nseg, world, ctypes.c_void_p(image.data_ptr())))
             table = image.to(dev)

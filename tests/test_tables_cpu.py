@@ -1,5 +1,5 @@
 """The host half of K2 and K2+K3: tdm_k2_table_* and tdm_k23_table_* cut segments into
-tiles of 8 KiB per stream and write the records the kernels walk. They build an image in
+tiles (tdm_table_tile_bytes() of every stream) and write the records the kernels walk. They build an image in
 host memory and launch nothing, so they are checked here without a GPU: tile counts,
 every record's pointers, counts, owner and alignment flag, and what they refuse."""
 
@@ -16,7 +16,7 @@ F32, F64, BF16, EINVAL = 0, 1, 3, 1  # enum tdm_dtype and TDM_EINVAL of include/
 FOLD_REC = np.dtype([("src", np.uint64, W), ("dst", np.uint64, W), ("count", np.int64), ("chunk", np.int32), ("vec_ok", np.int32)])
 STEP_REC = np.dtype([("g", np.uint64, W), ("p", np.uint64, W), ("m", np.uint64), ("v", np.uint64), ("count", np.int64),
                      ("chunk", np.int32), ("vec_ok", np.int32)])
-TILE_BYTES = 8192
+TILE_BYTES = lib().tdm_table_tile_bytes()
 
 
 def fold_segs(world, es, rows):
