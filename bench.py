@@ -40,7 +40,7 @@ WORLD = 4
 # HBM bytes per K1 launch at the default workload (4 chunk pairs of 64 MiB), from
 # rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads for
 # the plain copy kernel of known size in the same run: FETCH_SIZE x 1.9997 + WRITE_SIZE x 1.0.
-K1_TRAFFIC_256MIB = 805_291_000
+K1_TRAFFIC_256MIB = 805_273_000
 
 
 def seeded_grads(world, n, dev, scale):
