@@ -96,6 +96,32 @@ def test_a_group_of_one():
     assert out["bool_bcast_ok"] and out["bytes_ag_ok"]
 
 
+@pytest.mark.parametrize("world", [8, 9])
+def test_eight_and_nine_ranks(world):
+    """Eight ranks are the most the single-launch folds take (the staged forms); a group
+    of nine goes through the slots' ring for everything. The ring's order for every
+    chunk, whichever way it was summed."""
+    from oracle import ring
+    from tandem_amd import launch
+
+    n, dtype = 10_007, torch.float32
+    res = launch(collectives_of, world, [dtype], n, slot_bytes=4096, gpus=[0] * world, timeout=TIMEOUT)
+    xs = [to_np(values(q, n, dtype)) for q in range(world)]
+    sizes = [n // world + (1 if q < n % world else 0) for q in range(world)]
+    sizes = sizes[1:] + sizes[:1]
+    for r, per_dtype in enumerate(res):
+        out = per_dtype[str(dtype)]
+        assert np.array_equal(bits(to_np(out["ar_sum"])), bits(ring.expected_all_reduce(xs, False, "f32"))), r
+        assert np.array_equal(bits(to_np(out["ar_avg"])), bits(ring.expected_all_reduce(xs, True, "f32"))), r
+        assert np.array_equal(bits(to_np(out["rs_avg"])), bits(ring.expected_reduce_scatter(xs, sizes, True, "f32")[r])), r
+        lo = sum(sizes[:r])
+        own = ring.expected_reduce_scatter(xs, sizes, True, "f32")[r][lo:lo + sizes[r]]
+        assert np.array_equal(bits(to_np(out["rso_avg"])[lo:lo + sizes[r]]), bits(own)), r
+        assert np.array_equal(bits(to_np(out["ag"])), bits(ring.expected_all_gather(xs, sizes))), r
+        assert np.array_equal(bits(to_np(out["bcast"])), bits(xs[world - 1])), r
+        assert out["bool_bcast_ok"] and out["bytes_ag_ok"]
+
+
 def choose(monkeypatch, algo):
     """The engine's ways through all_reduce / all_gather: staged through memory the
     peers map (default: tensors up to 32 MiB with one handshake; "two": the two-handshake
