@@ -56,6 +56,19 @@ int tdm_device_info(int device, char* name, int name_len, int* compute_units, in
  * streaming kernels (0 restores the built-in default). Not needed for correctness. */
 int tdm_set_blocks_per_cu(int blocks);
 
+/* Launch geometry knob for measurements: which tile a workgroup takes. Consecutive workgroups
+ * go to the GPU's 8 XCDs in turn; with shift s each XCD takes (1 << s) consecutive tiles out of
+ * every group of (8 << s), so its L2 sees runs of (tile << s) bytes per stream. `kind` names the
+ * kernel family (TDM_XCD_*, -1: all), `shift` is 0..12 (0: tile = workgroup index) or -1 for the
+ * built-in default of that family. Process-wide; results never depend on it. */
+#define TDM_XCD_REDUCE 0      /* K1 ring-step reduce */
+#define TDM_XCD_COPY 1        /* ring copy step, pack, unit gather */
+#define TDM_XCD_FOLD 2        /* fold with the table by value (one collective) */
+#define TDM_XCD_FOLD_TABLE 3  /* K2 bucket fold over a device table */
+#define TDM_XCD_ADAMW 4       /* K3 */
+#define TDM_XCD_STEP 5        /* K2 + K3: the one-launch ZeRO-2 step */
+int tdm_set_xcd_group(int kind, int shift);
+
 /* Bytes of every stream that one record of the K2 and K2+K3 device tables covers (a build constant). */
 int tdm_table_tile_bytes(void);
 

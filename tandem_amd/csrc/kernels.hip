@@ -53,6 +53,26 @@ int compute_units() {
   return cus[dev];
 }
 
+// tile_of()'s shift per kernel family (TDM_XCD_*), settable through tdm_set_xcd_group.
+constexpr int kXcdKinds = TDM_XCD_STEP + 1;
+int g_xcd_shift[kXcdKinds] = {-1, -1, -1, -1, -1, -1};  // -1: the measured default below
+
+// Defaults, from sweeps of the shift (0..7) on MI355X at the 85.8M-parameter and 64-256 MiB
+// workloads. Launches with one or two write streams want the plain order (K1, the copy step and
+// the two-rank bucket fold lose 1-8 % with any grouping); the many-stream launches gain: the
+// one-launch ZeRO-2 step 2-3 % at 32 tiles per XCD, ZeRO-2's fold into the shards 3 % and AdamW
+// 0.5-1 % at 128, the single-launch all-reduce at world 4 2-3 % (32 beyond the Infinity Cache, 128 within).
+int xcd_shift(int kind, int world, bool cold) {
+  if (g_xcd_shift[kind] >= 0) return g_xcd_shift[kind];
+  switch (kind) {
+    case TDM_XCD_STEP: return 5;
+    case TDM_XCD_ADAMW: return 7;
+    case TDM_XCD_FOLD_TABLE: return world >= 3 ? 7 : 0;
+    case TDM_XCD_FOLD: return world >= 4 ? (cold ? 5 : 7) : 0;
+    default: return 0;
+  }
+}
+
 int grid_for(int64_t tiles) {
   const int64_t cap = static_cast<int64_t>(compute_units()) * g_blocks_per_cu;
   return static_cast<int>(std::max<int64_t>(1, std::min(tiles, cap)));
@@ -177,18 +197,20 @@ void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t st
   const dim3 grid(grid_for(tiles * FoldShape<kWorld>::kParts)), block(FoldShape<kWorld>::kT);
   const FoldSegDev* img = static_cast<const FoldSegDev*>(image);
   switch (div_kind(kWorld, average != 0)) {
-    case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, 0, stream, img, tiles, dv); break;
-    case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1, kAcc>), grid, block, 0, stream, img, tiles, dv); break;
-    default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2, kAcc>), grid, block, 0, stream, img, tiles, dv); break;
+    case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, 0, stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
+    case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1, kAcc>), grid, block, 0, stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
+    default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2, kAcc>), grid, block, 0, stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
   }
 }
 
 template <typename T, int kWorld>
-void launch_fold_small_w(const FoldSmall& tab, int average, hipStream_t stream) {
+void launch_fold_small_w(const FoldSmall& table, int average, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(kWorld);
-  const dim3 grid(grid_for(tab.tile_end[tab.nseg - 1])), block(kThreads);
+  const dim3 grid(grid_for(table.tile_end[table.nseg - 1])), block(kThreads);
   // bytes touched: every tile is read from kWorld ranks (and written back to most of them)
-  const bool cold = tab.tile_end[tab.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld > kColdFootprint;
+  const bool cold = table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld > kColdFootprint;
+  FoldSmall tab = table;
+  tab.shift = xcd_shift(TDM_XCD_FOLD, kWorld, cold);
   switch (div_kind(kWorld, average != 0) * 2 + (cold ? 1 : 0)) {
     case 0: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, 0, stream, tab, dv); break;
     case 1: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, 0, stream, tab, dv); break;
@@ -240,9 +262,9 @@ void launch_step_o(const void* image, int64_t tiles, int average, const tdm_adam
   const StepSegDev* t = static_cast<const StepSegDev*>(image);
   const dim3 grid(grid_for(tiles)), block(kThreads);
   switch (div_kind(kWorld, average != 0)) {
-    case 0: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 0, kOrder>), grid, block, 0, stream, t, tiles, dv, s); break;
-    case 1: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 1, kOrder>), grid, block, 0, stream, t, tiles, dv, s); break;
-    default: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 2, kOrder>), grid, block, 0, stream, t, tiles, dv, s); break;
+    case 0: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 0, kOrder>), grid, block, 0, stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
+    case 1: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 1, kOrder>), grid, block, 0, stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
+    default: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 2, kOrder>), grid, block, 0, stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
   }
 }
 
@@ -257,9 +279,9 @@ void launch_step_one_o(const StepSegDev& whole, int64_t tiles, int average, cons
   const Divisor<float> dv = make_divisor<float>(kWorld);
   const dim3 grid(grid_for(tiles)), block(kThreads);
   switch (div_kind(kWorld, average != 0)) {
-    case 0: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 0, kOrder>), grid, block, 0, stream, whole, tiles, dv, s); break;
-    case 1: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 1, kOrder>), grid, block, 0, stream, whole, tiles, dv, s); break;
-    default: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 2, kOrder>), grid, block, 0, stream, whole, tiles, dv, s); break;
+    case 0: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 0, kOrder>), grid, block, 0, stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
+    case 1: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 1, kOrder>), grid, block, 0, stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
+    default: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 2, kOrder>), grid, block, 0, stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
   }
 }
 
@@ -327,7 +349,8 @@ void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool s
   PairTable tab;
   const int64_t tiles = build_pairs(pairs, npairs, es, true, kK1TileVecs, &tab);
   if (tiles == 0) return;
-  tab.flags = (any_scale && scale_dst ? 1 : 0) | (any_scale && scale_src ? 2 : 0) | (any_scale && scale_src && writeback_src ? 4 : 0);
+  tab.flags = (any_scale && scale_dst ? 1 : 0) | (any_scale && scale_src ? 2 : 0) | (any_scale && scale_src && writeback_src ? 4 : 0) |
+              (xcd_shift(TDM_XCD_REDUCE, world, false) << 8);
   switch (dtype) {
     case TDM_F32: launch_reduce<float>(tab, tiles, world, any_scale, policy, stream); break;
     case TDM_F64: launch_reduce<double>(tab, tiles, world, any_scale, policy, stream); break;
@@ -360,6 +383,7 @@ void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStrea
     }
   }
   const int64_t tiles = build_pairs(kept.data(), static_cast<int>(kept.size()), es, false, kCopyTileVecs, &tab);
+  tab.flags = xcd_shift(TDM_XCD_COPY, world, false) << 8;
   if (tiles == 0) return;
   switch (dtype) {
     case TDM_F32: launch_copy<float>(tab, tiles, world, policy, stream); break;
@@ -618,6 +642,15 @@ int tdm_set_blocks_per_cu(int blocks) {
   });
 }
 
+int tdm_set_xcd_group(int kind, int shift) {
+  return guard([&] {
+    if (kind < -1 || kind >= kXcdKinds) throw Invalid("unknown kernel family");
+    if (shift < -1 || shift > 12) throw Invalid("the group shift must be in [0, 12], or -1 for the default");
+    for (int k = 0; k < kXcdKinds; ++k)
+      if (kind == -1 || kind == k) g_xcd_shift[k] = shift;
+  });
+}
+
 int tdm_k1_reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, int scale_dst, int scale_src,
                        int writeback_src, tdm_stream stream) {
   return guard([&] {
@@ -718,7 +751,7 @@ void adamw_launch(float* p, const float* g, float* m, float* v, int64_t n, const
   if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
   uintptr_t ptrs[4 + TDM_MAX_WORLD - 1] = {reinterpret_cast<uintptr_t>(p), reinterpret_cast<uintptr_t>(g),
                                            reinterpret_cast<uintptr_t>(m), reinterpret_cast<uintptr_t>(v)};
-  AdamwArgs a{p, g, m, v, n, *s, ncopies, {}};
+  AdamwArgs a{p, g, m, v, n, *s, ncopies, xcd_shift(TDM_XCD_ADAMW, 1, true), {}};
   for (int c = 0; c < ncopies; ++c) {
     if (!copies[c]) throw Invalid("NULL copy of the parameters");
     a.copy[c] = copies[c];

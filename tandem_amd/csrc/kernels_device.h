@@ -61,6 +61,20 @@ constexpr int kDefaultBlocksPerCu = 1024;
 int g_blocks_per_cu = kDefaultBlocksPerCu;
 constexpr int64_t kColdFootprint = int64_t(512) << 20;  // twice the Infinity Cache
 
+// Which tile a workgroup takes. The dispatcher hands consecutive workgroups to the 8 XCDs in
+// turn, so with tile = workgroup index every XCD touches every eighth 4 KiB of every stream.
+// With shift > 0 the tiles are taken in groups of 8 << shift and each XCD gets (1 << shift)
+// consecutive tiles of a group: the same tiles are in flight at any time, but each XCD's L2
+// and its path to memory see runs of (4 KiB << shift) per stream. Measured on MI355X with
+// streams of 336 MiB: nothing for one or two streams, +8-9 % for launches with four or more
+// write streams. The tiles past the last whole group keep their own index; shift 0 is the identity.
+__device__ __forceinline__ int64_t tile_of(int64_t idx, int64_t total, int shift) {
+  const int64_t span = int64_t(8) << shift;
+  if (idx >= (total & ~(span - 1))) return idx;
+  const int64_t in = idx & (span - 1);
+  return (idx - in) + ((in & 7) << shift) + (in >> 3);
+}
+
 typedef uint32_t vec16 __attribute__((ext_vector_type(4)));  // one dwordx4 access
 
 // ---------------------------------------------------------------- element types
@@ -204,7 +218,7 @@ __device__ __forceinline__ void store16(void* p, const vec16& v) {
 // Passed by value in the kernel arguments (scalar loads; no device table).
 struct PairTable {
   int npairs;
-  int flags;  // per launch: bit0 scale_dst, bit1 scale_src, bit2 writeback_src
+  int flags;  // per launch: bit0 scale_dst, bit1 scale_src, bit2 writeback_src; bits 8..: the shift of tile_of()
   int64_t tile_end[TDM_MAX_PAIRS];  // running tile count
   char* dst[TDM_MAX_PAIRS];
   char* src[TDM_MAX_PAIRS];
@@ -235,7 +249,9 @@ __global__ __launch_bounds__(kThreads) void k1_reduce_kernel(PairTable tab, Divi
   constexpr int64_t kTileElems = static_cast<int64_t>(kK1TileVecs) * L;
   const bool scale_dst = tab.flags & 1, scale_src = tab.flags & 2, writeback = tab.flags & 4;
   const int64_t total = tab.tile_end[tab.npairs - 1];
-  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+  const int shift = tab.flags >> 8;
+  for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
+    const int64_t tile = tile_of(at, total, shift);
     int p = 0;
     while (tile >= tab.tile_end[p]) ++p;
     const int64_t t = tile - (p ? tab.tile_end[p - 1] : 0);
@@ -317,7 +333,9 @@ __global__ __launch_bounds__(kCopyThreads) void k1_copy_kernel(PairTable tab, Di
   constexpr int L = lanes<T>();
   constexpr int64_t kTileElems = static_cast<int64_t>(kCopyTileVecs) * L;
   const int64_t total = tab.tile_end[tab.npairs - 1];
-  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+  const int shift = tab.flags >> 8;
+  for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
+    const int64_t tile = tile_of(at, total, shift);
     int p = 0;
     while (tile >= tab.tile_end[p]) ++p;
     const int64_t t = tile - (p ? tab.tile_end[p - 1] : 0);
@@ -511,9 +529,10 @@ struct FoldShape {
 
 template <typename T, int kWorld, int kDiv, bool kAcc>
 __global__ __launch_bounds__(kThreads) void k2_fold_kernel(const FoldSegDev* __restrict__ tiles, int64_t total,
-                                                           Divisor<T> dv) {
+                                                           Divisor<T> dv, int shift) {
   using S = FoldShape<kWorld>;
-  for (int64_t part = blockIdx.x; part < total * S::kParts; part += gridDim.x) {
+  for (int64_t at = blockIdx.x; at < total * S::kParts; at += gridDim.x) {
+    const int64_t part = tile_of(at, total * S::kParts, shift);
     fold_tile<T, kWorld, kDiv, kAcc, TDM_NT_MASK_K2, S::kRounds, S::kT>(tiles[part / S::kParts], part % S::kParts, dv);
   }
 }
@@ -521,6 +540,7 @@ __global__ __launch_bounds__(kThreads) void k2_fold_kernel(const FoldSegDev* __r
 // Table by value (one segment per ring chunk: a whole all-reduce in one launch).
 struct FoldSmall {
   int nseg;
+  int shift;  // of tile_of()
   int64_t tile_end[TDM_MAX_WORLD];
   FoldSegDev seg[TDM_MAX_WORLD];
 };
@@ -530,7 +550,8 @@ struct FoldSmall {
 template <typename T, int kWorld, int kDiv, bool kCold>
 __global__ __launch_bounds__(kThreads) void k2_fold_small_kernel(FoldSmall tab, Divisor<T> dv) {
   const int64_t total = tab.tile_end[tab.nseg - 1];
-  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+  for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
+    const int64_t tile = tile_of(at, total, tab.shift);
     int lo = 0;
     while (tile >= tab.tile_end[lo]) ++lo;
     fold_tile<T, kWorld, kDiv, false, kCold ? TDM_NT_MASK_K2 : TDM_NT_MASK>(tab.seg[lo], tile - (lo ? tab.tile_end[lo - 1] : 0), dv);
@@ -548,6 +569,7 @@ struct AdamwArgs {
   // Further copies of the updated parameters (the other ranks' flat buffers): the
   // update and the all-gather of the result in one pass.
   int ncopies;
+  int shift;  // of tile_of()
   float* copy[TDM_MAX_WORLD - 1];
 };
 
@@ -585,8 +607,8 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
     constexpr int kU = kAdamwUnroll;
     const int64_t nv = a.n / 4;
     const int64_t tiles = (nv + kThreads * kU - 1) / (kThreads * kU);
-    for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-      const int64_t v0 = tile * (kThreads * kU) + threadIdx.x;
+    for (int64_t at = blockIdx.x; at < tiles; at += gridDim.x) {
+      const int64_t v0 = tile_of(at, tiles, a.shift) * (kThreads * kU) + threadIdx.x;
       vec16 rp[kU], rg[kU], rm[kU], rv[kU];
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
@@ -746,9 +768,10 @@ __device__ __forceinline__ void step_tile(const StepSegDev& sg, int64_t at, int6
 
 template <int kWorld, int kDiv, int kOrder>
 __global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegDev* __restrict__ tiles, int64_t total,
-                                                                  Divisor<float> dv, tdm_adamw_scalars s) {
+                                                                  Divisor<float> dv, tdm_adamw_scalars s, int shift) {
   const bool small_w = __builtin_fabsf(s.w1) < 0.5f;
-  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+  for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
+    const int64_t tile = tile_of(at, total, shift);
     step_tile<kWorld, kDiv, kOrder>(tiles[tile], 0, tiles[tile].count, dv, s, small_w);
   }
 }
@@ -758,10 +781,11 @@ __global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegD
 // shard, out of its peers' gradient buffers and into their parameter buffers.
 template <int kWorld, int kDiv, int kOrder>
 __global__ __launch_bounds__(kThreads) void k23_zero2_step_one_kernel(StepSegDev whole, int64_t total, Divisor<float> dv,
-                                                                      tdm_adamw_scalars s) {
+                                                                      tdm_adamw_scalars s, int shift) {
   const bool small_w = __builtin_fabsf(s.w1) < 0.5f;
   constexpr int64_t kTileBytes = static_cast<int64_t>(kTileVecs) * 16;
-  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+  for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
+    const int64_t tile = tile_of(at, total, shift);
     const int64_t n = min(static_cast<int64_t>(kTileVecs) * 4, whole.count - tile * kTileVecs * 4);
     step_tile<kWorld, kDiv, kOrder>(whole, tile * kTileBytes, n, dv, s, small_w);
   }

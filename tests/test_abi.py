@@ -50,6 +50,9 @@ def test_argument_errors_need_no_gpu():
     assert L.tdm_k2_table_bytes(segs, 2, 99) == -1
     assert L.tdm_set_blocks_per_cu(5000) == 1
     assert L.tdm_set_blocks_per_cu(0) == 0
+    assert L.tdm_set_xcd_group(6, 0) == 1 and b"family" in L.tdm_last_error()
+    assert L.tdm_set_xcd_group(0, 13) == 1 and b"shift" in L.tdm_last_error()
+    assert L.tdm_set_xcd_group(3, 4) == 0 and L.tdm_set_xcd_group(-1, -1) == 0
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
