@@ -68,6 +68,9 @@ int tdm_set_blocks_per_cu(int blocks);
 #define TDM_XCD_ADAMW 4       /* K3 */
 #define TDM_XCD_STEP 5        /* K2 + K3: the one-launch ZeRO-2 step */
 int tdm_set_xcd_group(int kind, int shift);
+/* The tile that workgroup `index` of a launch over `total` tiles takes at group shift `shift` (the
+ * kernels' own function, evaluated on the host: for tests of the mapping). -1 for arguments out of range. */
+int64_t tdm_tile_of(int64_t index, int64_t total, int shift);
 
 /* Bytes of every stream that one record of the K2 and K2+K3 device tables covers (a build constant). */
 int tdm_table_tile_bytes(void);

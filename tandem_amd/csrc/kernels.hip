@@ -651,6 +651,11 @@ int tdm_set_xcd_group(int kind, int shift) {
   });
 }
 
+int64_t tdm_tile_of(int64_t index, int64_t total, int shift) {
+  if (index < 0 || index >= total || shift < 0 || shift > 12) return -1;
+  return tile_of(index, total, shift);
+}
+
 int tdm_k1_reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, int scale_dst, int scale_src,
                        int writeback_src, tdm_stream stream) {
   return guard([&] {

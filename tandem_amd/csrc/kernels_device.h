@@ -68,7 +68,7 @@ constexpr int64_t kColdFootprint = int64_t(512) << 20;  // twice the Infinity Ca
 // and its path to memory see runs of (4 KiB << shift) per stream. Measured on MI355X with
 // streams of 336 MiB: nothing for one or two streams, +8-9 % for launches with four or more
 // write streams. The tiles past the last whole group keep their own index; shift 0 is the identity.
-__device__ __forceinline__ int64_t tile_of(int64_t idx, int64_t total, int shift) {
+__host__ __device__ __forceinline__ int64_t tile_of(int64_t idx, int64_t total, int shift) {
   const int64_t span = int64_t(8) << shift;
   if (idx >= (total & ~(span - 1))) return idx;
   const int64_t in = idx & (span - 1);

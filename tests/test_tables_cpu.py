@@ -144,3 +144,27 @@ def test_empty_tables_and_refusals():
     bad = step_segs(2, [(10, 0, 0)])
     bad[0].count = -5
     refused(lambda: L.tdm_k23_table_build(bad, 1, 2, ptr), "negative count")
+
+
+def test_tile_order_is_a_permutation_that_keeps_runs_on_one_xcd():
+    """Every workgroup index takes exactly one tile and every tile is taken (a tile left out
+    would be data left unreduced); workgroups that go to the same XCD (index % 8) take
+    runs of 1 << shift consecutive tiles; the ragged end past the last whole group keeps
+    its own index; shift 0 is the plain order."""
+    from tandem_amd._lib import lib
+
+    L = lib()
+    for shift in range(0, 6):
+        span = 8 << shift
+        for total in (1, 7, 8, span - 1, span, span + 1, 3 * span + 5, 5 * span, 1000):
+            tiles = [L.tdm_tile_of(i, total, shift) for i in range(total)]
+            assert sorted(tiles) == list(range(total)), (shift, total)
+            whole = total - total % span
+            assert tiles[whole:] == list(range(whole, total))
+            if shift == 0:
+                assert tiles == list(range(total))
+            for i in range(0, whole - 8, 8):  # the same XCD's next workgroup
+                same_run = (i % span) // 8 + 1 < (1 << shift)
+                if same_run:
+                    assert tiles[i + 8] == tiles[i] + 1, (shift, total, i)
+    assert L.tdm_tile_of(5, 5, 0) == -1 and L.tdm_tile_of(-1, 5, 0) == -1 and L.tdm_tile_of(0, 5, 13) == -1
