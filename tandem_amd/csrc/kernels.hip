@@ -13,6 +13,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
@@ -55,7 +56,7 @@ int compute_units() {
 
 // tile_of()'s shift per kernel family (TDM_XCD_*), settable through tdm_set_xcd_group.
 constexpr int kXcdKinds = TDM_XCD_STEP + 1;
-int g_xcd_shift[kXcdKinds] = {-1, -1, -1, -1, -1, -1};  // -1: the measured default below
+std::atomic<int> g_xcd_shift[kXcdKinds] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}};  // -1: the measured default below (launches may come from several threads)
 
 // Defaults, from sweeps of the shift (0..7) on MI355X at the 85.8M-parameter and 64-256 MiB
 // workloads. Launches with one or two write streams want the plain order (K1, the copy step and
@@ -63,7 +64,8 @@ int g_xcd_shift[kXcdKinds] = {-1, -1, -1, -1, -1, -1};  // -1: the measured defa
 // one-launch ZeRO-2 step 2-3 % at 32 tiles per XCD, ZeRO-2's fold into the shards 3 % and AdamW
 // 0.5-1 % at 128, the single-launch all-reduce at world 4 2-3 % (32 beyond the Infinity Cache, 128 within).
 int xcd_shift(int kind, int world, bool cold) {
-  if (g_xcd_shift[kind] >= 0) return g_xcd_shift[kind];
+  const int set = g_xcd_shift[kind].load(std::memory_order_relaxed);
+  if (set >= 0) return set;
   switch (kind) {
     case TDM_XCD_STEP: return 5;
     case TDM_XCD_ADAMW: return 7;
@@ -647,7 +649,7 @@ int tdm_set_xcd_group(int kind, int shift) {
     if (kind < -1 || kind >= kXcdKinds) throw Invalid("unknown kernel family");
     if (shift < -1 || shift > 12) throw Invalid("the group shift must be in [0, 12], or -1 for the default");
     for (int k = 0; k < kXcdKinds; ++k)
-      if (kind == -1 || kind == k) g_xcd_shift[k] = shift;
+      if (kind == -1 || kind == k) g_xcd_shift[k].store(shift, std::memory_order_relaxed);
   });
 }
 

@@ -519,9 +519,12 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
 // Table in device memory, one record per tile (many segments: DDP's buckets). A record
 // describes 4 KiB of every stream; up to two ranks it is taken in two parts of 2 KiB, by one
 // workgroup each (the fewer streams a launch has, the smaller the part that serves it best).
+#ifndef TDM_K2_SPLIT_W2
+#define TDM_K2_SPLIT_W2 1  // 0 (measurement builds): one workgroup per record for every world size
+#endif
 template <int kWorld>
 struct FoldShape {
-  static constexpr bool kSmall = kWorld <= 2 && kThreads >= 128 && kTileVecs % 128 == 0;
+  static constexpr bool kSmall = TDM_K2_SPLIT_W2 && kWorld <= 2 && kThreads >= 128 && kTileVecs % 128 == 0;
   static constexpr int kT = kSmall ? 128 : kThreads;
   static constexpr int kRounds = kSmall ? 1 : kUnroll;
   static constexpr int kParts = kTileVecs / (kT * kRounds);
