@@ -53,14 +53,14 @@ int tdm_abi_version(void);
 int tdm_device_info(int device, char* name, int name_len, int* compute_units, int64_t* total_bytes);
 
 /* Launch geometry knob for measurements: workgroups per compute unit used by the
- * streaming kernels (0 restores the built-in default). Not needed for correctness. */
+ * streaming kernels (0 restores the built-in default). Not needed for correctness; the reference has no counterpart. */
 int tdm_set_blocks_per_cu(int blocks);
 
 /* Launch geometry knob for measurements: which tile a workgroup takes. Consecutive workgroups
  * go to the GPU's 8 XCDs in turn; with shift s each XCD takes (1 << s) consecutive tiles out of
  * every group of (8 << s), so its L2 sees runs of (tile << s) bytes per stream. `kind` names the
  * kernel family (TDM_XCD_*, -1: all), `shift` is 0..12 (0: tile = workgroup index) or -1 for the
- * built-in default of that family. Process-wide; results never depend on it. */
+ * built-in default of that family. Process-wide; results never depend on it. The reference has no counterpart. */
 #define TDM_XCD_REDUCE 0      /* K1 ring-step reduce */
 #define TDM_XCD_COPY 1        /* ring copy step, pack, unit gather */
 #define TDM_XCD_FOLD 2        /* fold with the table by value (one collective) */
