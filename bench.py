@@ -26,7 +26,6 @@ starts (world size 4 on one GPU). Prints ONE JSON line:
 
 import argparse
 import json
-import math
 import os
 import statistics
 import sys
@@ -439,7 +438,6 @@ def ipc_allreduce():
 def cpu_rank(g, n, reps, numels):
     """Timed on the host: (i) the ring all-reduce(avg) of the GPU's main workload,
     (ii) the ZeRO-2 step (16 bucket reduce-scatters, shard add, AdamW, all-gather)."""
-    import numpy as np
     import torch
 
     from oracle.adamw import AdamW

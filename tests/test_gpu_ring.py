@@ -2,8 +2,6 @@
 written by the reference's Python engine. Bit-exact: every comparison is on bit
 patterns. Run with -m gpu on an MI355X."""
 
-import ctypes
-
 import numpy as np
 import pytest
 import torch
