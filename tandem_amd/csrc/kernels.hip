@@ -62,7 +62,8 @@ std::atomic<int> g_xcd_shift[kXcdKinds] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}}; 
 // workloads. Launches with one or two write streams want the plain order (K1, the copy step and
 // the two-rank bucket fold lose 1-8 % with any grouping); the many-stream launches gain: the
 // one-launch ZeRO-2 step 2-3 % at 32 tiles per XCD, ZeRO-2's fold into the shards 3 % and AdamW
-// 0.5-1 % at 128, the single-launch all-reduce at world 4 2-3 % (32 beyond the Infinity Cache, 128 within).
+// 0.5-1 % at 128, the single-launch all-reduce 2-8 % at world 4 and 7-12 % at world 8 (32 beyond the Infinity
+// Cache, 128 within), 4-5 % at world 2 with 256 MiB per rank and nothing at world 3 beyond the cache.
 int xcd_shift(int kind, int world, bool cold) {
   const int set = g_xcd_shift[kind].load(std::memory_order_relaxed);
   if (set >= 0) return set;
@@ -70,7 +71,7 @@ int xcd_shift(int kind, int world, bool cold) {
     case TDM_XCD_STEP: return 5;
     case TDM_XCD_ADAMW: return 7;
     case TDM_XCD_FOLD_TABLE: return world >= 3 ? 7 : 0;
-    case TDM_XCD_FOLD: return world >= 4 ? (cold ? 5 : 7) : 0;
+    case TDM_XCD_FOLD: return cold ? (world == 3 ? 0 : 5) : (world >= 3 ? 7 : 0);
     default: return 0;
   }
 }
@@ -212,7 +213,7 @@ void launch_fold_small_w(const FoldSmall& table, int average, hipStream_t stream
   // bytes touched: every tile is read from kWorld ranks (and written back to most of them)
   const bool cold = table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld > kColdFootprint;
   FoldSmall tab = table;
-  tab.shift = xcd_shift(TDM_XCD_FOLD, kWorld, cold);
+  tab.shift = xcd_shift(TDM_XCD_FOLD, kWorld, table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld >= kColdFootprint);
   switch (div_kind(kWorld, average != 0) * 2 + (cold ? 1 : 0)) {
     case 0: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, 0, stream, tab, dv); break;
     case 1: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, 0, stream, tab, dv); break;
