@@ -1,7 +1,10 @@
 """Host-side planning (bucket packing, shard sizes, fold segments) against the
-plans the reference itself produced (tests/golden/plans.json)."""
+plans the reference itself produced (tests/golden/plans.json), and on random
+inputs against element-by-element brute force."""
 
 import math
+
+from hypothesis import given, settings, strategies as st
 
 from helpers import golden_json
 from tandem_amd.buckets import FlatLayout, fold_segments, pack, zero_buckets
@@ -69,3 +72,54 @@ def test_fold_segments_cover_the_bucket_once():
             assert lo <= pos and pos + count <= hi  # inside one ring chunk
             pos += count
         assert seen == numels and pos == sum(numels)
+
+
+# ---- properties on random inputs, checked against element-by-element brute force
+
+@settings(max_examples=150, deadline=None)
+@given(st.integers(0, 300), st.integers(1, 9))
+def test_split_sizes_are_tensor_splits(n, world):
+    import torch
+
+    want = [c.numel() for c in torch.tensor_split(torch.empty(n), world)]
+    assert split_sizes(n, world) == want
+    bounds = chunk_bounds(n, world)
+    assert [hi - lo for lo, hi in bounds] == want and (not bounds or bounds[0][0] == 0)
+
+
+@settings(max_examples=150, deadline=None)
+@given(st.lists(st.integers(0, 40), min_size=1, max_size=12), st.integers(1, 6), st.data())
+def test_bucket_sizes_count_the_elements_of_each_shard(numels, world, data):
+    lay = [FlatLayout(numels, world, r) for r in range(world)]
+    n = lay[0].numel
+    owner = [r for r in range(world) for _ in range(lay[r].hi - lay[r].lo)]
+    assert len(owner) == n and all(l.lo == sum(lay[0].sizes[:r]) for r, l in enumerate(lay))
+    a = data.draw(st.integers(0, n))
+    b = data.draw(st.integers(a, n))
+    assert lay[0].bucket_sizes(a, b) == [sum(1 for i in range(a, b) if owner[i] == r) for r in range(world)]
+
+
+@settings(max_examples=150, deadline=None)
+@given(st.lists(st.integers(0, 50), min_size=0, max_size=20), st.integers(1, 120))
+def test_packing_rule(sizes, cap):
+    groups = pack(sizes, cap)
+    assert [i for g in groups for i in g] == list(range(len(sizes)))  # order kept, nothing lost
+    for k, g in enumerate(groups):
+        assert g and (sum(sizes[i] for i in g) <= cap or len(g) == 1)  # only a lone oversize tensor exceeds the limit
+        if k + 1 < len(groups):  # greedy: the next tensor did not fit
+            assert sum(sizes[i] for i in g) + sizes[groups[k + 1][0]] > cap
+
+
+@settings(max_examples=150, deadline=None)
+@given(st.lists(st.integers(0, 30), min_size=1, max_size=10), st.integers(1, 8))
+def test_fold_segments_tag_every_element_with_its_ring_chunk(numels, world):
+    total = sum(numels)
+    chunk_of = [c for c, (lo, hi) in enumerate(chunk_bounds(total, world)) for _ in range(hi - lo)]
+    seen = []
+    starts = [sum(numels[:i]) for i in range(len(numels))]
+    for i, off, count, c in fold_segments(numels, world):
+        assert count > 0 and off + count <= numels[i]
+        for e in range(starts[i] + off, starts[i] + off + count):
+            assert chunk_of[e] == c
+            seen.append(e)
+    assert seen == list(range(total))  # flat order, each element once
