@@ -9,8 +9,10 @@ starts (world size 4 on one GPU). Prints ONE JSON line:
   value       algorithmic HBM bytes of the step (15 x message bytes) / step time
   roofline    the dominant kernel, the fused ring-step reduce (K1): 12 bytes per
               element per launch / the launch's duration, taken from HIP events
-              recorded around the three back-to-back K1 launches of every timed
-              step, against the 8 TB/s HBM peak; `traffic` is the HBM traffic per
+              recorded around the three back-to-back K1 launches of every step of
+              a repeat of the timed steps (the timed steps carry no events: a record
+              between two kernels holds the second one back), against the 8 TB/s
+              HBM peak; `traffic` is the HBM traffic per
               launch measured with rocprofv3 counters
   sweep       message sizes 64 KiB .. 256 MiB, ring and single-launch fold
   bucket_path DDP's bucket flatten+average+unflatten (K2), 85.8M params, world 2
