@@ -58,20 +58,23 @@ int compute_units() {
 constexpr int kXcdKinds = TDM_XCD_STEP + 1;
 std::atomic<int> g_xcd_shift[kXcdKinds] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}};  // -1: the measured default below (launches may come from several threads)
 
-// Defaults, from sweeps of the shift (0..7) on MI355X at the 85.8M-parameter and 64-256 MiB
-// workloads. Launches with one or two write streams want the plain order (K1, the copy step and
-// the two-rank bucket fold lose 1-8 % with any grouping); the many-stream launches gain: the
-// one-launch ZeRO-2 step 2-3 % at 32 tiles per XCD, ZeRO-2's fold into the shards 3 % and AdamW
-// 0.5-1 % at 128, the single-launch all-reduce 2-8 % at world 4 and 7-12 % at world 8 (32 beyond the Infinity
-// Cache, 128 within), 4-5 % at world 2 with 256 MiB per rank and nothing at world 3 beyond the cache.
+// Defaults, from sweeps of the shift (0..9) on MI355X at the 85.8M-parameter and 64-256 MiB
+// workloads. The unit is what one workgroup takes: 4 KiB for K1, the copy step and a fold within
+// the caches, 2 KiB for the table-driven folds, the one-launch step, AdamW and a fold beyond the
+// caches. Launches with one or two write streams want the plain order (K1, the copy step and the
+// two-rank bucket fold lose 1-8 % with any grouping); the many-stream launches gain: the one-launch
+// ZeRO-2 step 1-3 % at 64 parts per XCD, ZeRO-2's fold into the shards 3 % at 256, AdamW 0.5-1 %
+// at 128, the single-launch all-reduce 2-8 % (runs of 128 KiB per XCD beyond the Infinity Cache,
+// 1 MiB within). Differences of 1-2 % between neighbouring shifts do not repeat from one machine
+// to the next; the defaults are the choices that were never behind the plain order.
 int xcd_shift(int kind, int world, bool cold) {
   const int set = g_xcd_shift[kind].load(std::memory_order_relaxed);
   if (set >= 0) return set;
   switch (kind) {
-    case TDM_XCD_STEP: return 5;
+    case TDM_XCD_STEP: return 6;
     case TDM_XCD_ADAMW: return 7;
-    case TDM_XCD_FOLD_TABLE: return world >= 3 ? 7 : 0;
-    case TDM_XCD_FOLD: return cold ? (world == 3 ? 0 : 5) : (world >= 3 ? 7 : 0);
+    case TDM_XCD_FOLD_TABLE: return world >= 4 ? 8 : 0;
+    case TDM_XCD_FOLD: return cold ? (world == 3 ? 8 : world >= 4 ? 6 : 5) : (world >= 3 ? 8 : 0);
     default: return 0;
   }
 }
@@ -209,9 +212,9 @@ void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t st
 template <typename T, int kWorld>
 void launch_fold_small_w(const FoldSmall& table, int average, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(kWorld);
-  const dim3 grid(grid_for(table.tile_end[table.nseg - 1])), block(kThreads);
   // bytes touched: every tile is read from kWorld ranks (and written back to most of them)
   const bool cold = table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld > kColdFootprint;
+  const dim3 grid(grid_for(table.tile_end[table.nseg - 1] * (cold ? fold_small_parts<kWorld>() : 1))), block(kThreads);
   FoldSmall tab = table;
   tab.shift = xcd_shift(TDM_XCD_FOLD, kWorld, table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld >= kColdFootprint);
   switch (div_kind(kWorld, average != 0) * 2 + (cold ? 1 : 0)) {
@@ -263,7 +266,7 @@ template <int kWorld, int kOrder>
 void launch_step_o(const void* image, int64_t tiles, int average, const tdm_adamw_scalars& s, hipStream_t stream) {
   const Divisor<float> dv = make_divisor<float>(kWorld);
   const StepSegDev* t = static_cast<const StepSegDev*>(image);
-  const dim3 grid(grid_for(tiles)), block(kThreads);
+  const dim3 grid(grid_for(tiles * kStepParts)), block(kThreads);
   switch (div_kind(kWorld, average != 0)) {
     case 0: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 0, kOrder>), grid, block, 0, stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
     case 1: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 1, kOrder>), grid, block, 0, stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
@@ -280,7 +283,7 @@ void launch_step_w(const void* image, int64_t tiles, int average, const tdm_adam
 template <int kWorld, int kOrder>
 void launch_step_one_o(const StepSegDev& whole, int64_t tiles, int average, const tdm_adamw_scalars& s, hipStream_t stream) {
   const Divisor<float> dv = make_divisor<float>(kWorld);
-  const dim3 grid(grid_for(tiles)), block(kThreads);
+  const dim3 grid(grid_for(tiles * kStepParts)), block(kThreads);
   switch (div_kind(kWorld, average != 0)) {
     case 0: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 0, kOrder>), grid, block, 0, stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
     case 1: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 1, kOrder>), grid, block, 0, stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;

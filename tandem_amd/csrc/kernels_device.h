@@ -517,14 +517,16 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
 }
 
 // Table in device memory, one record per tile (many segments: DDP's buckets). A record
-// describes 4 KiB of every stream; up to two ranks it is taken in two parts of 2 KiB, by one
-// workgroup each (the fewer streams a launch has, the smaller the part that serves it best).
-#ifndef TDM_K2_SPLIT_W2
-#define TDM_K2_SPLIT_W2 1  // 0 (measurement builds): one workgroup per record for every world size
+// describes 4 KiB of every stream and is taken in two parts of 2 KiB, by one workgroup each:
+// launches that stream from HBM through many streams at once do better with the smaller part
+// (two-rank bucket fold 3-7 %, ZeRO-2's fold into the shards 2 %, against a build with one
+// workgroup per 4 KiB).
+#ifndef TDM_K2_SPLIT
+#define TDM_K2_SPLIT 1  // 0 (measurement builds): one workgroup per record
 #endif
 template <int kWorld>
 struct FoldShape {
-  static constexpr bool kSmall = TDM_K2_SPLIT_W2 && kWorld <= 2 && kThreads >= 128 && kTileVecs % 128 == 0;
+  static constexpr bool kSmall = TDM_K2_SPLIT && kThreads >= 128 && kTileVecs % 128 == 0;
   static constexpr int kT = kSmall ? 128 : kThreads;
   static constexpr int kRounds = kSmall ? 1 : kUnroll;
   static constexpr int kParts = kTileVecs / (kT * kRounds);
@@ -540,6 +542,12 @@ __global__ __launch_bounds__(kThreads) void k2_fold_kernel(const FoldSegDev* __r
   }
 }
 
+// Parts per tile of a launch with its table by value whose footprint is beyond the caches.
+template <int kWorld>
+constexpr int fold_small_parts() {
+  return FoldShape<kWorld>::kSmall && FoldShape<kWorld>::kT == kThreads ? FoldShape<kWorld>::kParts : 1;
+}
+
 // Table by value (one segment per ring chunk: a whole all-reduce in one launch).
 struct FoldSmall {
   int nseg;
@@ -550,14 +558,19 @@ struct FoldSmall {
 
 // kCold: the launch's footprint is far beyond the 256 MB Infinity Cache, so nothing it
 // writes will be read from there: the cache policy of the once-per-step bucket fold.
+// Such a launch also takes its tiles in two parts of 2 KiB, one workgroup each (256 MiB per rank at
+// world 4: 3 % faster; within the cache, 64 MiB per rank, the whole tile per workgroup is 6 % faster).
 template <typename T, int kWorld, int kDiv, bool kCold>
 __global__ __launch_bounds__(kThreads) void k2_fold_small_kernel(FoldSmall tab, Divisor<T> dv) {
-  const int64_t total = tab.tile_end[tab.nseg - 1];
+  constexpr int kParts = kCold ? fold_small_parts<kWorld>() : 1;
+  const int64_t total = tab.tile_end[tab.nseg - 1] * kParts;
   for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
-    const int64_t tile = tile_of(at, total, tab.shift);
+    const int64_t part = tile_of(at, total, tab.shift);
+    const int64_t tile = part / kParts;
     int lo = 0;
     while (tile >= tab.tile_end[lo]) ++lo;
-    fold_tile<T, kWorld, kDiv, false, kCold ? TDM_NT_MASK_K2 : TDM_NT_MASK>(tab.seg[lo], tile - (lo ? tab.tile_end[lo - 1] : 0), dv);
+    const int64_t t = (tile - (lo ? tab.tile_end[lo - 1] : 0)) * kParts + part % kParts;
+    fold_tile<T, kWorld, kDiv, false, kCold ? TDM_NT_MASK_K2 : TDM_NT_MASK, kUnroll / kParts>(tab.seg[lo], t, dv);
   }
 }
 
@@ -676,15 +689,22 @@ struct StepSegDev {
 #ifndef TDM_K23_UNROLL
 #define TDM_K23_UNROLL 2
 #endif
+// A record of the step's table (4 KiB of every stream) is taken in two parts of 2 KiB, by one
+// workgroup each: 3 % faster at the 85.8M-parameter step than one workgroup per record.
+#ifndef TDM_K23_PARTS
+#define TDM_K23_PARTS 2
+#endif
+constexpr int kStepParts = (TDM_K23_PARTS <= kUnroll && kUnroll % TDM_K23_PARTS == 0) ? TDM_K23_PARTS : 1;
 #ifndef TDM_NT_MASK_K23
 #define TDM_NT_MASK_K23 TDM_NT_MASK_K3
 #endif
 
-// One tile (at most 4 KiB of every stream) of the step.
-template <int kWorld, int kDiv, int kOrder>
+// One part (at most kRounds vectors per lane and stream) of the step.
+template <int kWorld, int kDiv, int kOrder, int kRounds>
 __device__ __forceinline__ void step_tile(const StepSegDev& sg, int64_t at, int64_t n, const Divisor<float>& dv,
                                           const tdm_adamw_scalars& s, bool small_w) {
-  constexpr int kU = kWorld <= 4 ? TDM_K23_UNROLL : 1;  // vectors per lane in flight, per stream
+  constexpr int kWant = kWorld <= 4 ? TDM_K23_UNROLL : 1;
+  constexpr int kU = kWant < kRounds ? kWant : kRounds;  // vectors per lane in flight, per stream
   constexpr int kM = TDM_NT_MASK_K23;
   {
     const int c = sg.chunk;  // `at`: the tile's offset in bytes from the record's pointers; n: its elements
@@ -708,7 +728,7 @@ __device__ __forceinline__ void step_tile(const StepSegDev& sg, int64_t at, int6
     if (sg.vec_ok) {
       const int64_t nv = n / 4;
 #pragma unroll
-      for (int u0 = 0; u0 < kUnroll; u0 += kU) {
+      for (int u0 = 0; u0 < kRounds; u0 += kU) {
         vec16 in[kWorld][kU], rp[kU], rm[kU], rv[kU];
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
@@ -773,9 +793,13 @@ template <int kWorld, int kDiv, int kOrder>
 __global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegDev* __restrict__ tiles, int64_t total,
                                                                   Divisor<float> dv, tdm_adamw_scalars s, int shift) {
   const bool small_w = __builtin_fabsf(s.w1) < 0.5f;
-  for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
-    const int64_t tile = tile_of(at, total, shift);
-    step_tile<kWorld, kDiv, kOrder>(tiles[tile], 0, tiles[tile].count, dv, s, small_w);
+  constexpr int64_t kPartElems = static_cast<int64_t>(kTileVecs / kStepParts) * 4;
+  for (int64_t at = blockIdx.x; at < total * kStepParts; at += gridDim.x) {
+    const int64_t part = tile_of(at, total * kStepParts, shift);
+    const StepSegDev& rec = tiles[part / kStepParts];
+    const int64_t first = (part % kStepParts) * kPartElems;  // the part's first element within the record
+    const int64_t n = min(kPartElems, rec.count - first);
+    if (n > 0) step_tile<kWorld, kDiv, kOrder, kUnroll / kStepParts>(rec, first * 4, n, dv, s, small_w);
   }
 }
 
@@ -786,11 +810,11 @@ template <int kWorld, int kDiv, int kOrder>
 __global__ __launch_bounds__(kThreads) void k23_zero2_step_one_kernel(StepSegDev whole, int64_t total, Divisor<float> dv,
                                                                       tdm_adamw_scalars s, int shift) {
   const bool small_w = __builtin_fabsf(s.w1) < 0.5f;
-  constexpr int64_t kTileBytes = static_cast<int64_t>(kTileVecs) * 16;
-  for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
-    const int64_t tile = tile_of(at, total, shift);
-    const int64_t n = min(static_cast<int64_t>(kTileVecs) * 4, whole.count - tile * kTileVecs * 4);
-    step_tile<kWorld, kDiv, kOrder>(whole, tile * kTileBytes, n, dv, s, small_w);
+  constexpr int64_t kPartElems = static_cast<int64_t>(kTileVecs / kStepParts) * 4;
+  for (int64_t at = blockIdx.x; at < total * kStepParts; at += gridDim.x) {
+    const int64_t part = tile_of(at, total * kStepParts, shift);
+    const int64_t n = min(kPartElems, whole.count - part * kPartElems);
+    if (n > 0) step_tile<kWorld, kDiv, kOrder, kUnroll / kStepParts>(whole, part * kPartElems * 4, n, dv, s, small_w);
   }
 }
 
