@@ -282,7 +282,7 @@ def fsdp_rank(g, steps, prefetch):
             waits.append(sum(b - a for name, a, b in g.waits if name == "gather_unit"))
     n_gathers = sum(1 for name, *_ in g.trace if name == "gather_unit")
     return {"fwd_bwd_ms": statistics.median(times) * 1e3, "host_blocked_on_gathers_ms": statistics.median(waits) * 1e3,
-            "gathers_per_step": n_gathers, "max_live": f.max_live, "live": f.live, "loss": float(loss)}
+            "gathers_per_step": n_gathers, "max_live": f.max_live, "live": f.live, "loss": float(loss.detach())}
 
 
 def fsdp_gather(steps):
