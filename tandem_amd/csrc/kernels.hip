@@ -778,8 +778,8 @@ void adamw_launch(float* p, const float* g, float* m, float* v, int64_t n, const
       const uintptr_t bytes = static_cast<uintptr_t>(n) * 4;
       if (ptrs[i] < ptrs[j] + bytes && ptrs[j] < ptrs[i] + bytes) throw Invalid("p, g, m, v and the copies must not overlap");
     }
-  const dim3 block(kThreads);
-  const int64_t tiles = vec ? (n / 4 + kThreads * kAdamwUnroll - 1) / (kThreads * kAdamwUnroll) : (n + kThreads - 1) / kThreads;
+  const dim3 block(kAdamwThreads);
+  const int64_t tiles = vec ? (n / 4 + kAdamwThreads * kAdamwUnroll - 1) / (kAdamwThreads * kAdamwUnroll) : (n + kAdamwThreads - 1) / kAdamwThreads;
   const dim3 grid(grid_for(std::max<int64_t>(tiles, 1)));
   const int which = (order == TDM_ADAMW_HOST_ORDER ? 0 : 4) + (vec ? 2 : 0) + (ncopies > 0 ? 1 : 0);
   switch (which) {

@@ -615,20 +615,24 @@ __device__ __forceinline__ void adamw_elem(float& p, float g, float& m, float& v
 #define TDM_K3_UNROLL 1
 #endif
 constexpr int kAdamwUnroll = TDM_K3_UNROLL;  // vectors per lane and stream in flight
+#ifndef TDM_K3_THREADS
+#define TDM_K3_THREADS TDM_THREADS
+#endif
+constexpr int kAdamwThreads = TDM_K3_THREADS;  // lanes per workgroup of K3
 
 template <int kOrder, bool kVec, bool kCopies>
-__global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
+__global__ __launch_bounds__(kAdamwThreads) void k3_adamw_kernel(AdamwArgs a) {
   const bool small_w = __builtin_fabsf(a.s.w1) < 0.5f;
   if constexpr (kVec) {
     constexpr int kU = kAdamwUnroll;
     const int64_t nv = a.n / 4;
-    const int64_t tiles = (nv + kThreads * kU - 1) / (kThreads * kU);
+    const int64_t tiles = (nv + kAdamwThreads * kU - 1) / (kAdamwThreads * kU);
     for (int64_t at = blockIdx.x; at < tiles; at += gridDim.x) {
-      const int64_t v0 = tile_of(at, tiles, a.shift) * (kThreads * kU) + threadIdx.x;
+      const int64_t v0 = tile_of(at, tiles, a.shift) * (kAdamwThreads * kU) + threadIdx.x;
       vec16 rp[kU], rg[kU], rm[kU], rv[kU];
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
-        const int64_t i = v0 + u * kThreads;
+        const int64_t i = v0 + u * kAdamwThreads;
         if (i < nv) {
           rp[u] = load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.p) + i * 16);
           rg[u] = load_stream<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.g) + i * 16);
@@ -638,7 +642,7 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
       }
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
-        const int64_t i = v0 + u * kThreads;
+        const int64_t i = v0 + u * kAdamwThreads;
         if (i < nv) {
           Lanes<float> P = unpack<float>(rp[u]), G = unpack<float>(rg[u]), M = unpack<float>(rm[u]),
                        V = unpack<float>(rv[u]);
@@ -660,8 +664,8 @@ __global__ __launch_bounds__(kThreads) void k3_adamw_kernel(AdamwArgs a) {
         for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
     }
   } else {
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < a.n; i += stride) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kAdamwThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kAdamwThreads + threadIdx.x; i < a.n; i += stride) {
       adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
       if constexpr (kCopies)
         for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
