@@ -160,6 +160,22 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
 int tdm_k2_bucket_fold(const void* table_dev, int64_t ntiles, int dtype, int world, int average, int accumulate,
                        tdm_stream stream);
 
+/* tdm_k2_bucket_fold for callers that cannot allocate device memory or copy a table to the
+ * device: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference. The per-tile table that tdm_k2_table_build +
+ * tdm_k2_bucket_fold keep in a buffer of the caller's is written here by a small kernel
+ * (the segments travel in its launch arguments, 16 per launch) into a fixed array inside the
+ * library, tdm_k2_static_max_tiles() records = 16,384 tiles = 64 MiB of every rank's stream
+ * per call, 2.25 MiB of device memory that every GPU the library runs on holds until the
+ * process ends; then the same fold kernel runs over it, on `stream`. Same arguments
+ * otherwise, same bits. Segments that need more records are refused (TDM_EINVAL) before
+ * anything is launched: split the call. The call allocates nothing on the device and makes no
+ * host-to-device copy. All calls on one GPU share the array: calls on one stream are ordered
+ * by it; calls that overlap on different streams (or threads) race and give wrong results. */
+int64_t tdm_k2_static_max_tiles(void);
+int tdm_k2_bucket_fold_static(const tdm_fold_seg* segs, int nseg, int world, int dtype, int average, int accumulate,
+                              tdm_stream stream);
+
 /* ---- K3: sharded AdamW --------------------------------------------------- */
 
 /* The step's constants, each already rounded to fp32 from the Python-double

@@ -74,6 +74,9 @@ _SIGNATURES = {
     "tdm_k2_table_tiles": (ctypes.c_int64, [ctypes.POINTER(FoldSeg), ctypes.c_int, ctypes.c_int]),
     "tdm_k2_bucket_fold": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                           ctypes.c_int, ctypes.c_void_p]),
+    "tdm_k2_static_max_tiles": (ctypes.c_int64, []),
+    "tdm_k2_bucket_fold_static": (ctypes.c_int, [ctypes.POINTER(FoldSeg), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                 ctypes.c_int, ctypes.c_void_p]),
     "tdm_k3_adamw": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                     ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
     "tdm_k3_adamw_gather": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,

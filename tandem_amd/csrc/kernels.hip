@@ -17,6 +17,7 @@
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <type_traits>
 #include <vector>
@@ -25,6 +26,12 @@
 #include "common.h"
 
 #include "kernels_device.h"
+
+// The table of tdm_k2_bucket_fold_static: records for up to kStaticTiles tiles, in every GPU's
+// memory for as long as the library is loaded (2.25 MiB). Host code reaches it through
+// static_table() only.
+constexpr int64_t kStaticTiles = 16384;
+static __device__ __align__(256) unsigned char scratch[kStaticTiles * sizeof(tandem_hip::FoldSegDev)];
 
 namespace tandem_hip {
 
@@ -695,6 +702,22 @@ int64_t tdm_k2_table_bytes(const tdm_fold_seg* segs, int nseg, int dtype) {
   return std::max<int64_t>(16, tiles * static_cast<int64_t>(sizeof(FoldSegDev)));
 }
 
+namespace {
+// Checks segment i of a K2 table; returns whether it may take the 16-byte path.
+bool fold_seg_check(const tdm_fold_seg& s, int i, int world, int es) {
+  if (s.count < 0) throw Invalid("segment " + std::to_string(i) + ": negative count");
+  if (s.chunk < 0 || s.chunk >= world) throw Invalid("segment " + std::to_string(i) + ": chunk outside [0, world)");
+  bool vec = true;
+  for (int r = 0; r < world; ++r) {
+    if (s.count > 0 && s.src[r] == nullptr) throw Invalid("segment " + std::to_string(i) + ": NULL source");
+    const uintptr_t a = reinterpret_cast<uintptr_t>(s.src[r]), b = reinterpret_cast<uintptr_t>(s.dst[r]);
+    if (a % es || b % es) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to the element size");
+    vec = vec && a % 16 == 0 && b % 16 == 0;
+  }
+  return vec;
+}
+}  // namespace
+
 int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype, void* image) {
   return guard([&] {
     const int es = elem_size(dtype);
@@ -707,15 +730,7 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
     int64_t tiles = 0;
     for (int i = 0; i < nseg; ++i) {
       const tdm_fold_seg& s = segs[i];
-      if (s.count < 0) throw Invalid("segment " + std::to_string(i) + ": negative count");
-      if (s.chunk < 0 || s.chunk >= world) throw Invalid("segment " + std::to_string(i) + ": chunk outside [0, world)");
-      bool vec = true;
-      for (int r = 0; r < world; ++r) {
-        if (s.count > 0 && s.src[r] == nullptr) throw Invalid("segment " + std::to_string(i) + ": NULL source");
-        const uintptr_t a = reinterpret_cast<uintptr_t>(s.src[r]), b = reinterpret_cast<uintptr_t>(s.dst[r]);
-        if (a % es || b % es) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to the element size");
-        vec = vec && a % 16 == 0 && b % 16 == 0;
-      }
+      const bool vec = fold_seg_check(s, i, world, es);
       for (int64_t at = 0; at < s.count; at += tile_elems) {  // a tile's byte offset is a multiple of 4 KiB
         FoldSegDev& rec = out[tiles++];
         for (int r = 0; r < world; ++r) {
@@ -730,25 +745,105 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
   });
 }
 
+namespace {
+void bucket_fold(const void* table_dev, int64_t ntiles, int dtype, int world, int average, int accumulate, hipStream_t st) {
+  if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
+  if (ntiles < 0) throw Invalid("ntiles is negative");
+  if (ntiles == 0) return;
+  if (table_dev == nullptr) throw Invalid("table is NULL");
+  if (average && world > 1 && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
+  switch (dtype) {
+    case TDM_F32: launch_fold<float>(table_dev, ntiles, world, average, accumulate != 0, st); break;
+    case TDM_F64: launch_fold<double>(table_dev, ntiles, world, average, accumulate != 0, st); break;
+    case TDM_F16: launch_fold<f16_t>(table_dev, ntiles, world, average, accumulate != 0, st); break;
+    case TDM_BF16: launch_fold<bf16_t>(table_dev, ntiles, world, average, accumulate != 0, st); break;
+    case TDM_I64: launch_fold<int64_t>(table_dev, ntiles, world, 0, accumulate != 0, st); break;
+    case TDM_I32: launch_fold<int32_t>(table_dev, ntiles, world, 0, accumulate != 0, st); break;
+    default: throw Invalid("unknown dtype " + std::to_string(dtype));
+  }
+  check_hip(hipGetLastError(), "k2_fold launch");
+}
+}  // namespace
+
 int tdm_k2_bucket_fold(const void* table_dev, int64_t ntiles, int dtype, int world, int average, int accumulate,
                        tdm_stream stream) {
+  return guard([&] { bucket_fold(table_dev, ntiles, dtype, world, average, accumulate, static_cast<hipStream_t>(stream)); });
+}
+
+// ---- the same fold for callers that cannot allocate: the table lives in a fixed device array
+namespace {
+// This GPU's copy of `scratch`, looked up once per device with that device current. The array's
+// name is only a host-side handle: everything below uses the address returned here.
+FoldSegDev* static_table() {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static FoldSegDev* table[kMaxDevices] = {nullptr};
+  int dev = 0;
+  check_hip(hipGetDevice(&dev), "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) throw std::runtime_error("device index beyond 63");
+  std::lock_guard<std::mutex> lock(mu);
+  if (table[dev] == nullptr) {
+    void* p = nullptr;
+    check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+    if (p == nullptr) throw std::runtime_error("hipGetSymbolAddress(scratch) returned NULL");
+    table[dev] = static_cast<FoldSegDev*>(p);
+  }
+  return table[dev];
+}
+}  // namespace
+
+int64_t tdm_k2_static_max_tiles(void) { return kStaticTiles; }
+
+int tdm_k2_bucket_fold_static(const tdm_fold_seg* segs, int nseg, int world, int dtype, int average, int accumulate,
+                              tdm_stream stream) {
   return guard([&] {
+    const int es = elem_size(dtype);
+    if (es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
     if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
-    if (ntiles < 0) throw Invalid("ntiles is negative");
-    if (ntiles == 0) return;
-    if (table_dev == nullptr) throw Invalid("table is NULL");
+    if (nseg < 0 || (nseg > 0 && segs == nullptr)) throw Invalid("bad table arguments");
     if (average && world > 1 && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    switch (dtype) {
-      case TDM_F32: launch_fold<float>(table_dev, ntiles, world, average, accumulate != 0, st); break;
-      case TDM_F64: launch_fold<double>(table_dev, ntiles, world, average, accumulate != 0, st); break;
-      case TDM_F16: launch_fold<f16_t>(table_dev, ntiles, world, average, accumulate != 0, st); break;
-      case TDM_BF16: launch_fold<bf16_t>(table_dev, ntiles, world, average, accumulate != 0, st); break;
-      case TDM_I64: launch_fold<int64_t>(table_dev, ntiles, world, 0, accumulate != 0, st); break;
-      case TDM_I32: launch_fold<int32_t>(table_dev, ntiles, world, 0, accumulate != 0, st); break;
-      default: throw Invalid("unknown dtype " + std::to_string(dtype));
+    const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
+    // every segment is checked, and the size known, before the first launch
+    int64_t tiles = 0;
+    for (int i = 0; i < nseg; ++i) {
+      fold_seg_check(segs[i], i, world, es);
+      tiles += (segs[i].count + tile_elems - 1) / tile_elems;
+      if (tiles > kStaticTiles) {
+        throw Invalid("the segments need more than " + std::to_string(kStaticTiles) + " table records (" +
+                      std::to_string(kStaticTiles * static_cast<int64_t>(kTileVecs) * 16) +
+                      " bytes of every rank's stream): beyond the fixed table of tdm_k2_bucket_fold_static; "
+                      "split the call or use tdm_k2_table_build + tdm_k2_bucket_fold");
+      }
     }
-    check_hip(hipGetLastError(), "k2_fold launch");
+    if (tiles == 0) return;
+    FoldSegDev* table = static_table();
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    FillBatch batch;
+    std::memset(&batch, 0, sizeof batch);
+    batch.world = world;
+    batch.es = es;
+    batch.tile_elems = tile_elems;
+    int64_t at = 0;  // records written by the batches before this one
+    auto flush = [&] {
+      if (batch.nseg == 0) return;
+      const int64_t n = batch.first[batch.nseg] - batch.first[0];
+      hipLaunchKernelGGL(k2_table_fill_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, batch, table);
+      check_hip(hipGetLastError(), "k2_table_fill launch");
+      batch.nseg = 0;
+    };
+    for (int i = 0; i < nseg; ++i) {
+      const tdm_fold_seg& s = segs[i];
+      if (s.count == 0) continue;
+      const int k = batch.nseg;
+      batch.first[k] = at;
+      at += (s.count + tile_elems - 1) / tile_elems;
+      batch.first[k + 1] = at;
+      batch.vec_ok[k] = fold_seg_check(s, i, world, es);
+      batch.seg[k] = s;
+      if (++batch.nseg == kFillSegs) flush();
+    }
+    flush();
+    bucket_fold(table, tiles, dtype, world, average, accumulate, st);
   });
 }
 

@@ -542,6 +542,39 @@ __global__ __launch_bounds__(kThreads) void k2_fold_kernel(const FoldSegDev* __r
   }
 }
 
+// Writes K2's table on the device: one thread per tile of up to kFillSegs segments that
+// arrive in the launch itself. For callers that may not allocate or copy from the host
+// (tdm_k2_bucket_fold_static): the records land in a fixed array inside the library.
+constexpr int kFillSegs = 16;
+struct FillBatch {
+  int nseg;
+  int world;
+  int es;               // element size in bytes
+  int64_t tile_elems;   // elements per record
+  int64_t first[kFillSegs + 1];  // first[k]: index of segment k's first record; first[nseg]: one past the batch's last
+  int32_t vec_ok[kFillSegs];
+  tdm_fold_seg seg[kFillSegs];
+};
+
+__global__ __launch_bounds__(256) void k2_table_fill_kernel(FillBatch b, FoldSegDev* __restrict__ out) {
+  const int64_t tile = b.first[0] + static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (tile >= b.first[b.nseg]) return;
+  int k = 0;
+  while (tile >= b.first[k + 1]) ++k;
+  const tdm_fold_seg& s = b.seg[k];
+  const int64_t at = (tile - b.first[k]) * b.tile_elems;
+  FoldSegDev rec;
+#pragma unroll
+  for (int r = 0; r < TDM_MAX_WORLD; ++r) {
+    rec.src[r] = r < b.world && s.src[r] ? static_cast<const char*>(s.src[r]) + at * b.es : nullptr;
+    rec.dst[r] = r < b.world && s.dst[r] ? static_cast<char*>(s.dst[r]) + at * b.es : nullptr;
+  }
+  rec.count = min(b.tile_elems, s.count - at);
+  rec.chunk = s.chunk;
+  rec.vec_ok = b.vec_ok[k];
+  out[tile] = rec;
+}
+
 // Parts per tile of a launch with its table by value whose footprint is beyond the caches.
 template <int kWorld>
 constexpr int fold_small_parts() {

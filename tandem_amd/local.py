@@ -208,6 +208,7 @@ class FoldTable:
 
     def _upload(self, segs, nseg):
         self.nseg = nseg
+        self._segs = segs
         self.elements = sum(segs[k].count for k in range(nseg))
         nbytes = lib().tdm_k2_table_bytes(segs, self.nseg, dtype_code(self.dtype))
         self.ntiles = lib().tdm_k2_table_tiles(segs, self.nseg, dtype_code(self.dtype))
@@ -220,6 +221,16 @@ class FoldTable:
     def run(self, average=True, accumulate=False):
         check(lib().tdm_k2_bucket_fold(ctypes.c_void_p(self.image.data_ptr()), self.ntiles, dtype_code(self.dtype),
                                        self.world, int(average), int(accumulate), stream_ptr(self.device)))
+
+
+    def run_static(self, average=True, accumulate=False):
+        """The same fold without the uploaded table: its records are written on the GPU
+        into a fixed array inside the library, so the call allocates nothing and copies
+        nothing from the host (for callers under HIP graph capture or in loops that must
+        not allocate). At most lib().tdm_k2_static_max_tiles() tiles per call; calls
+        that overlap on different streams of one GPU race."""
+        check(lib().tdm_k2_bucket_fold_static(self._segs, self.nseg, self.world, dtype_code(self.dtype), int(average),
+                                              int(accumulate), stream_ptr(self.device)))
 
 
 class LocalZeRO2:
