@@ -1,12 +1,15 @@
 """Builds libtandem_hip.so (the C-ABI library declared in include/tandem_hip.h)
 in-tree with hipcc for gfx950. Cross-compiles without a GPU.
 
-    python -m tandem_amd.build
+    python -m tandem_amd.build [extra hipcc flags, e.g. -DTDM_NT_MASK=7] [--out=path/to/variant.so]
+
+Every source is compiled to an object of its own, in parallel, then linked.
 """
 
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
@@ -16,26 +19,42 @@ SOURCES = ["kernels.hip", "abi.hip", "engine.hip", "engine_abi.hip"]
 # -ffp-contract=off: no multiply-add is fused unless the source says fma.
 # -fhip-fp32-correctly-rounded-divide-sqrt: IEEE division and sqrt (the default; stated).
 # -packed-fp32-ops disabled: the compiler must not form v_pk_*_f32 from scalar float code.
-FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-ffp-contract=off",
          "-fhip-fp32-correctly-rounded-divide-sqrt", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wall", "-Wextra", "-pthread"]
 
 
-def build(verbose=False, extra=()):
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    cmd = [hipcc, *FLAGS, *extra, "-o", LIB, *srcs, "-lrt"]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # hipcc's host pass does not know the device-only target feature and says so: harmless
     out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
     if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
+        raise RuntimeError(f"hipcc failed ({res.returncode}): {' '.join(cmd)}\n{out}")
     if verbose and out.strip():
         print(out)
-    return LIB
+
+
+def build(verbose=False, extra=(), out=LIB):
+    """Compiles every source (always: nothing is reused from an earlier build) and links `out`."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    objdir = os.path.join(CSRC, "_obj", os.path.splitext(os.path.basename(out))[0])
+    os.makedirs(objdir, exist_ok=True)
+    objs = [os.path.join(objdir, os.path.splitext(s)[0] + ".o") for s in srcs]
+    jobs = [[hipcc, *FLAGS, *extra, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(srcs, objs)]
+    with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1)) as pool:
+        list(pool.map(lambda cmd: _run(cmd, verbose), jobs))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-pthread", "-o", out, *objs, "-lrt"], verbose)
+    return out
 
 
 if __name__ == "__main__":
-    print(build(verbose=True, extra=sys.argv[1:]))
+    args = sys.argv[1:]
+    target = LIB
+    for a in list(args):
+        if a.startswith("--out="):
+            target = os.path.abspath(a[len("--out="):])
+            args.remove(a)
+    print(build(verbose=True, extra=args, out=target))
