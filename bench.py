@@ -39,9 +39,28 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X, published
 WORLD = 4
 # HBM bytes per K1 launch at the default workload (4 chunk pairs of 64 MiB), from
-# rocprofv3 FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads for
-# the plain copy kernel of known size in the same run: FETCH_SIZE x 1.9997 + WRITE_SIZE x 1.0.
-K1_TRAFFIC_256MIB = 805_273_000
+# rocprofv3 FETCH_SIZE / WRITE_SIZE runs: kept in a tracked file next to the profile
+# summary it comes from, together with the launch geometry of the build it was measured on.
+K1_TRAFFIC_FILE = os.path.join(ROOT, "profiles", "k1_traffic.json")
+
+
+def k1_traffic(mib, _lib):
+    """Counter-derived HBM bytes per K1 launch, or None when the record does not describe
+    this workload or this build (another tile size or workgroup size)."""
+    import ctypes
+
+    try:
+        with open(K1_TRAFFIC_FILE) as f:
+            rec = json.load(f)
+        a, b, c = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+        _lib.check(_lib.lib().tdm_build_geometry(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+        if rec["mib_per_rank"] != mib or rec["world"] != WORLD:
+            return None
+        if rec["k1_tile_bytes"] != a.value or rec["workgroup_lanes"] != b.value:
+            return None
+        return int(rec["hbm_bytes_per_launch"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def seeded_grads(world, n, dev, scale):
@@ -130,13 +149,18 @@ def sweep(lw, dev, steps):
         per, rs, ag = time_ring(lw, bufs, reps, 3)
         fold = timed(lambda: lw.all_reduce(bufs, "avg", algorithm="fold"), reps)
         b = n * 4
-        graph_ms = None
+        graph_ms = fold_graph_ms = None
         if kib <= 65536:  # sizes where the gaps between the six launches still count: the same ring pass replayed from a HIP graph
             flats = [x.reshape(-1) for x in bufs]
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 ring_pass(lw, flats)
             graph_ms = round(timed(graph.replay, reps) * 1e3, 4)
+            del graph
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                lw.all_reduce(bufs, "avg", algorithm="fold")
+            fold_graph_ms = round(timed(graph.replay, reps) * 1e3, 4)
             del graph
         rows.append({"MiB": kib / 1024, "ring_ms": round(per * 1e3, 4), "ring_GBps": round(15 * b / per / 1e9, 1),
                      "ring_algbw_GBps": round(b / per / 1e9, 1),
@@ -145,9 +169,49 @@ def sweep(lw, dev, steps):
                      "fold_algbw_GBps": round(b / fold / 1e9, 1)})
         if graph_ms is not None:
             rows[-1]["ring_hip_graph_ms"] = graph_ms
+            rows[-1]["fold_hip_graph_ms"] = fold_graph_ms
         del bufs
         torch.cuda.empty_cache()
     return rows
+
+
+# (streams read, streams written) of each kernel at its benchmark workload
+MIXES = {"k1_reduce": (2, 1), "ring_copy": (1, 1), "bucket_fold_w2": (2, 2), "zero2_fold_w4": (5, 1), "adamw": (4, 3),
+         "adamw_gather_w4": (4, 6), "fold_all_reduce_w4": (4, 4), "zero2_step_one_launch_w4": (7, 6)}
+
+
+def stream_mix(dev, reps):
+    """What the memory system gives a kernel that only streams: for every kernel's mix of
+    read and written streams, the library's probe (no table, no arithmetic, the kernels'
+    own launch geometry) over cold buffers of 85,842,432 fp32 each, best of a few launch
+    geometries. The fused kernels are reported against these figures as well as against
+    the 8 TB/s peak: a stream mix with many written streams does not reach the peak
+    whatever the kernel."""
+    import ctypes
+
+    import torch
+
+    from tandem_amd._lib import check, lib, stream_ptr
+
+    n = 85_842_432
+    whole = torch.empty(13 * n, device=dev).normal_()  # one allocation: the streams lie back to back
+    bufs = [whole[k * n:(k + 1) * n] for k in range(13)]
+    st = stream_ptr(dev)
+    out = {"workload": "tdm_probe_stream_mix, 85,842,432 fp32 per stream, all streams cold (footprint 0.7-4.5 GB), "
+                       "best of tile order shift 0/6 x occupancy pad 0/16/24 KiB, one 16-byte vector per lane and stream"}
+    for name, (r, w) in MIXES.items():
+        rd = (ctypes.c_void_p * 8)(*[b.data_ptr() for b in bufs[:r]])
+        wr = (ctypes.c_void_p * 8)(*[b.data_ptr() for b in bufs[r:r + w]])
+        best = None
+        for shift in (0, 6):
+            for pad in (0, 16384, 24576):
+                t = timed(lambda: check(lib().tdm_probe_stream_mix(rd, r, wr, w, n * 4, 1, shift, pad, st)), reps, warm=2)
+                rate = (r + w) * n * 4 / t / 1e9
+                if best is None or rate > best[0]:
+                    best = (rate, shift, pad)
+        out[name] = {"reads": r, "writes": w, "GBps": round(best[0], 1), "frac_of_hbm_peak": round(best[0] / HBM_PEAK_GBPS, 4),
+                     "xcd_shift": best[1], "occupancy_pad": best[2]}
+    return out
 
 
 def gpt_numels():
@@ -442,7 +506,7 @@ def cpu_rank(g, n, reps, numels):
     (ii) the ZeRO-2 step (16 bucket reduce-scatters, shard add, AdamW, all-gather)."""
     import torch
 
-    from oracle.adamw import AdamW
+    from oracle.cpu_engine import TorchCpuAdamW
     from tandem_amd.buckets import FlatLayout, zero_buckets
 
     x = torch.randn(n, generator=torch.Generator().manual_seed(g.rank)) * 1e-2
@@ -461,7 +525,7 @@ def cpu_rank(g, n, reps, numels):
     grads = torch.randn(lay.numel, generator=torch.Generator().manual_seed(10 + g.rank)) * 1e-3
     staging = torch.empty_like(grads)
     shard = torch.zeros(lay.hi - lay.lo)
-    opt = AdamW(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    opt = TorchCpuAdamW(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)  # torch ops, as tandem/optim.py:28-37
     ts = []
     for _ in range(3):
         staging.copy_(grads)
@@ -474,7 +538,7 @@ def cpu_rank(g, n, reps, numels):
             if mine.numel():
                 at = max(a, lay.lo) - lay.lo
                 shard[at:at + mine.numel()].add_(mine)
-        opt.update("flat", buf[lay.lo:lay.hi].numpy(), shard.numpy())
+        opt.update("flat", buf[lay.lo:lay.hi], shard)
         g.all_gather(buf, lay.sizes)
         ts.append(time.perf_counter() - t)
     out["zero2_step_s"] = statistics.median(ts)
@@ -511,8 +575,52 @@ def cpu_baseline(mib, reps):
     return {"all_reduce_4MB_2_ranks_ms": round(small * 1e3, 3), "all_reduce_4MB_2_ranks_GBps": round((4 << 20) / small / 1e9, 3),"value": round(15 * n * 4 / t / 1e9, 3), "unit": "GB/s", "cores": WORLD, "kind": "port",
             "sample": f"oracle CPU-process engine (tandem's Python-engine protocol): ring all-reduce(avg), world 4 x 1 torch thread, "
                       f"{mib} MiB fp32 per rank (the GPU workload), 2 x 4 MiB shared-memory slots per pair, median of {reps}: "
-                      f"{t * 1e3:.1f} ms per all-reduce; then 3 ZeRO-2 steps at 85,842,432 params; {total:.1f} s in all, {total * WORLD:.0f} core-seconds",
+                      f"{t * 1e3:.1f} ms per all-reduce; then 3 ZeRO-2 steps at 85,842,432 params (16 reduce-scatters, shard add, AdamW as torch ops, all-gather); {total:.1f} s in all, {total * WORLD:.0f} core-seconds",
             "algbw_GBps": round(n * 4 / t / 1e9, 3), "zero2_step_ms": round(z * 1e3, 1), "host_cores": os.cpu_count()}
+
+
+def summarize(line):
+    """The whole metric as plain numbers inside `config` and `roofline` (the sections
+    keep the detail): K1's fraction of the HBM peak and the ring pass's at 4, 16, 64 and
+    256 MiB per rank, the ZeRO-2 step in ms, the bucket path and AdamW, and each fused
+    kernel against the streaming ceiling of its own mix of streams."""
+    cfg, roof = line["config"], line["roofline"]
+    for row in line.get("sweep", ()):
+        mib = row["MiB"]
+        if mib in (4.0, 16.0, 64.0, 256.0):
+            tag = f"{int(mib)}MiB"
+            roof[f"k1_frac_{tag}"] = row["k1_frac_of_hbm"]
+            cfg[f"pass_frac_{tag}"] = round(row["ring_GBps"] / HBM_PEAK_GBPS, 4)
+            cfg[f"pass_ms_{tag}"] = row["ring_ms"]
+            cfg[f"fold_pass_ms_{tag}"] = row["fold_ms"]
+    mix = line.get("stream_mix", {})
+
+    def against(name, gbps):
+        top = mix.get(name, {}).get("GBps")
+        return round(gbps / top, 4) if top else None
+
+    if mix:
+        roof["k1_mix_ceiling_frac"] = mix["k1_reduce"]["frac_of_hbm_peak"]
+    z = line.get("zero2_step")
+    if z:
+        cfg["zero2_step_one_launch_ms"] = z["one_launch_ms"]
+        cfg["zero2_step_ms"] = z["ms"]
+        cfg["zero2_step_one_launch_frac"] = round(z["one_launch_GBps"] / HBM_PEAK_GBPS, 4)
+        cfg["adamw_frac"] = z["adamw_frac_of_hbm_peak"]
+        cfg["adamw_ms"] = z["adamw_4_shards_ms"]
+        if mix:
+            z["one_launch_frac_of_mix_ceiling"] = cfg["zero2_step_one_launch_frac_of_mix_ceiling"] = against("zero2_step_one_launch_w4", z["one_launch_GBps"])
+            z["adamw_frac_of_mix_ceiling"] = cfg["adamw_frac_of_mix_ceiling"] = against("adamw", z["adamw_GBps"])
+            z["adamw_gather_frac_of_mix_ceiling"] = against("adamw_gather_w4", z["adamw_gather_GBps"])
+            cfg["zero2_step_mix_ceiling_frac"] = mix["zero2_step_one_launch_w4"]["frac_of_hbm_peak"]
+            cfg["adamw_mix_ceiling_frac"] = mix["adamw"]["frac_of_hbm_peak"]
+    b = line.get("bucket_path")
+    if b:
+        cfg["bucket_path_ms"] = b["ms"]
+        cfg["bucket_path_frac"] = b["frac_of_hbm_peak"]
+        if mix:
+            b["frac_of_mix_ceiling"] = cfg["bucket_path_frac_of_mix_ceiling"] = against("bucket_fold_w2", b["GBps"])
+            cfg["bucket_path_mix_ceiling_frac"] = mix["bucket_fold_w2"]["frac_of_hbm_peak"]
 
 
 def device_name(_lib):
@@ -533,7 +641,14 @@ def main():
     ap.add_argument("--quick", action="store_true", help="only the main workload (for profiling runs)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-fsdp", action="store_true")
+    ap.add_argument("--only", default="", help="comma list of single-process sections to run besides the main workload "
+                                               "(sweep, bucket, zero2, mix), for short profiling runs; implies --no-cpu --no-fsdp")
     args = ap.parse_args()
+    only = {x for x in args.only.split(",") if x}
+    if only - {"sweep", "bucket", "zero2", "mix"}:
+        sys.exit("--only takes sweep, bucket, zero2 and mix")
+    if only:
+        args.no_cpu = args.no_fsdp = True
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every rank of the group is a buffer in that GPU's HBM, or a process sharing it; "
                  "run with --gpus 1")
@@ -607,7 +722,7 @@ def main():
                    "frac_of_hbm_peak": round(15 * b / per / 1e9 / HBM_PEAK_GBPS, 4)},
         "roofline": {"bound": "hbm", "kernel": "k1_reduce_kernel<float> (ring-step fused reduce)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": K1_TRAFFIC_256MIB if args.mib == 256 else None,
+                     "traffic": k1_traffic(args.mib, _lib),
                      "bytes_per_launch": k1_bytes, "launch_us": round(k1_launch_s * 1e6, 2),
                      "launch_us_from": "HIP events on the launch stream around the three back-to-back K1 launches of each step, "
                                        "over a repeat of the timed steps (the timed steps themselves carry no events)",
@@ -616,11 +731,17 @@ def main():
     del bufs
     torch.cuda.empty_cache()
     if not args.quick:
-        line["sweep"] = sweep(lw, dev, max(5, args.steps // 2))
-        line["bucket_path"] = bucket_path(dev, args.steps)
-        torch.cuda.empty_cache()
-        line["zero2_step"] = zero2_step(dev, max(5, args.steps // 2))
-        torch.cuda.empty_cache()
+        if not only or "mix" in only:
+            line["stream_mix"] = stream_mix(dev, 6)
+            torch.cuda.empty_cache()
+        if not only or "sweep" in only:
+            line["sweep"] = sweep(lw, dev, max(5, args.steps // 2))
+        if not only or "bucket" in only:
+            line["bucket_path"] = bucket_path(dev, args.steps)
+            torch.cuda.empty_cache()
+        if not only or "zero2" in only:
+            line["zero2_step"] = zero2_step(dev, max(5, args.steps // 2))
+            torch.cuda.empty_cache()
         if fsdp is not None:
             line["fsdp_gather"] = fsdp
         if ipc is not None:
@@ -634,6 +755,7 @@ def main():
             cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["one_launch_ms"], 1)
         if cpu is not None:
             line["cpu_baseline"] = cpu
+    summarize(line)
     line["device"] = device_name(_lib)
     print(json.dumps(line), flush=True)
 

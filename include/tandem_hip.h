@@ -68,12 +68,35 @@ int tdm_set_blocks_per_cu(int blocks);
 #define TDM_XCD_ADAMW 4       /* K3 */
 #define TDM_XCD_STEP 5        /* K2 + K3: the one-launch ZeRO-2 step */
 int tdm_set_xcd_group(int kind, int shift);
+/* Launch geometry knob for measurements: bytes of LDS that the launches of kernel family `kind`
+ * (TDM_XCD_*, -1: all) reserve per workgroup without using them, which caps how many workgroups
+ * share a compute unit (160 KiB of LDS each); 0: no cap, -1: the built-in default of that family
+ * (24 KiB for TDM_XCD_STEP and TDM_XCD_ADAMW, whose many streams do better with 3 waves per SIMD;
+ * 0 for the others). At most 65536. Process-wide; results never depend on it. The reference has
+ * no counterpart. */
+int tdm_set_occupancy_pad(int kind, int bytes);
 /* The tile that workgroup `index` of a launch over `total` tiles takes at group shift `shift` (the
  * kernels' own function, evaluated on the host: for tests of the mapping). -1 for arguments out of range. */
 int64_t tdm_tile_of(int64_t index, int64_t total, int shift);
 
+/* Measurement only; the reference has no counterpart. Reads `bytes` (a multiple of 16) from each of
+ * `nreads` device buffers and writes as many to each of `nwrites` others (0..8 each), in the launch
+ * geometry of the streaming kernels (workgroups of 128 lanes, `vectors_per_lane` = 1 or 2 16-byte
+ * vectors per lane and stream, one tile per workgroup, tile order tdm_tile_of(.., xcd_shift),
+ * `occupancy_pad` bytes of unused LDS per workgroup, non-temporal accesses), without a table and
+ * without arithmetic: what the memory system gives a kernel with that mix of streams. The written
+ * values are meaningless. */
+int tdm_probe_stream_mix(const void* const* reads, int nreads, void* const* writes, int nwrites, int64_t bytes,
+                         int vectors_per_lane, int xcd_shift, int occupancy_pad, tdm_stream stream);
+
 /* Bytes of every stream that one record of the K2 and K2+K3 device tables covers (a build constant). */
 int tdm_table_tile_bytes(void);
+
+/* Build constants of the launch geometry, for records that must name the build they were measured
+ * on: bytes of every stream that one workgroup of K1 and of the copy kernel takes, lanes per
+ * workgroup, bytes of every stream per table record (= tdm_table_tile_bytes()). The reference has
+ * no counterpart. */
+int tdm_build_geometry(int* k1_tile_bytes, int* workgroup_lanes, int* table_tile_bytes);
 
 /* ---- K1: one ring step -------------------------------------------------- */
 

@@ -36,6 +36,32 @@ class EngineError(RuntimeError):
     pass
 
 
+class TorchCpuAdamW:
+    """The optimizer of the CPU baseline: the update of tandem/optim.py:16-37 as the
+    same sequence of torch CPU tensor operations (one pass over the shard each), which is what tandem's CPU-process backend runs. The bit-exact checker
+    is oracle.adamw.AdamW; this class is timed, and checked against that one with
+    torch's own sqrt substituted (tests/test_oracle_adamw.py)."""
+
+    def __init__(self, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2):
+        self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
+        self.state = {}
+
+    def update(self, key, param, grad):
+        entry = self.state.setdefault(key, {"t": 0.0, "m": torch.zeros_like(param), "v": torch.zeros_like(param)})
+        entry["t"] += 1.0
+        if param.numel() == 0:
+            return
+        t, m, v = entry["t"], entry["m"], entry["v"]
+        b1, b2 = self.betas
+        if self.weight_decay != 0:
+            param.mul_(1 - self.lr * self.weight_decay)
+        m.lerp_(grad, 1 - b1)
+        v.mul_(b2).addcmul_(grad, grad, value=1 - b2)
+        root = (1 - b2 ** t) ** 0.5
+        spread = (v.sqrt() / root).add_(self.eps)  # two temporaries, as tandem/optim.py:36 makes
+        param.addcdiv_(m, spread, value=-(self.lr / (1 - b1 ** t)))
+
+
 class PendingWork:
     """Handle of a queued collective; wait() returns its result or re-raises."""
 

@@ -56,8 +56,12 @@ _SIGNATURES = {
                                        ctypes.POINTER(ctypes.c_int64)]),
     "tdm_set_blocks_per_cu": (ctypes.c_int, [ctypes.c_int]),
     "tdm_set_xcd_group": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
+    "tdm_set_occupancy_pad": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
+    "tdm_probe_stream_mix": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.POINTER(ctypes.c_void_p), ctypes.c_int,
+                                            ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "tdm_tile_of": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]),
     "tdm_table_tile_bytes": (ctypes.c_int, []),
+    "tdm_build_geometry": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),
     "tdm_engine_set_timing": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "tdm_k1_reduce_step": (ctypes.c_int, [ctypes.POINTER(Pair), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                           ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),

@@ -86,6 +86,28 @@ int xcd_shift(int kind, int world, bool cold) {
   }
 }
 
+// Occupancy cap per kernel family: bytes of LDS that a launch asks for per workgroup and never
+// touches, so that fewer workgroups fit a compute unit (160 KiB of LDS each). The many-stream
+// kernels keep far more loads in flight than the memory system needs (13 KiB per wave for the
+// one-launch step, thousands of waves), and what waits there only widens the set of DRAM rows
+// open at once. Measured on MI355X at the 85.8M-parameter step, 24 KiB per workgroup (6 workgroups
+// = 3 waves per SIMD): one-launch step 0.780 -> 0.745 ms, AdamW on four shards 0.385 -> 0.377 ms,
+// AdamW writing every rank's copy 0.587 -> 0.569 ms; 16 KiB and 32-40 KiB give less, 64 KiB
+// (one wave per SIMD) is 30 % slower. Launches with few streams lose with any cap (two-rank bucket
+// fold 0.212 -> 0.25 ms at 24 KiB, ZeRO-2's fold into the shards 0.36 -> 0.39).
+std::atomic<int> g_occupancy_pad[kXcdKinds] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
+
+unsigned occupancy_pad(int kind, bool cold = true) {
+  const int set = g_occupancy_pad[kind].load(std::memory_order_relaxed);
+  if (set >= 0) return static_cast<unsigned>(set);
+  switch (kind) {
+    case TDM_XCD_STEP: return 24576;
+    case TDM_XCD_ADAMW: return 24576;
+    case TDM_XCD_FOLD: return cold ? 24576 : 0;  // 256 MiB per rank at world 4: 0.350 -> 0.343 ms; 64 MiB: 0.078 -> 0.081
+    default: return 0;
+  }
+}
+
 int grid_for(int64_t tiles) {
   const int64_t cap = static_cast<int64_t>(compute_units()) * g_blocks_per_cu;
   return static_cast<int>(std::max<int64_t>(1, std::min(tiles, cap)));
@@ -210,9 +232,9 @@ void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t st
   const dim3 grid(grid_for(tiles * FoldShape<kWorld>::kParts)), block(FoldShape<kWorld>::kT);
   const FoldSegDev* img = static_cast<const FoldSegDev*>(image);
   switch (div_kind(kWorld, average != 0)) {
-    case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, 0, stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
-    case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1, kAcc>), grid, block, 0, stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
-    default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2, kAcc>), grid, block, 0, stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
+    case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, occupancy_pad(TDM_XCD_FOLD_TABLE), stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
+    case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1, kAcc>), grid, block, occupancy_pad(TDM_XCD_FOLD_TABLE), stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
+    default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2, kAcc>), grid, block, occupancy_pad(TDM_XCD_FOLD_TABLE), stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
   }
 }
 
@@ -225,12 +247,12 @@ void launch_fold_small_w(const FoldSmall& table, int average, hipStream_t stream
   FoldSmall tab = table;
   tab.shift = xcd_shift(TDM_XCD_FOLD, kWorld, table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld >= kColdFootprint);
   switch (div_kind(kWorld, average != 0) * 2 + (cold ? 1 : 0)) {
-    case 0: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, 0, stream, tab, dv); break;
-    case 1: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, 0, stream, tab, dv); break;
-    case 2: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, false>), grid, block, 0, stream, tab, dv); break;
-    case 3: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, true>), grid, block, 0, stream, tab, dv); break;
-    case 4: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2, false>), grid, block, 0, stream, tab, dv); break;
-    default: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2, true>), grid, block, 0, stream, tab, dv); break;
+    case 0: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+    case 1: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+    case 2: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+    case 3: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+    case 4: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+    default: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
   }
 }
 
@@ -275,9 +297,9 @@ void launch_step_o(const void* image, int64_t tiles, int average, const tdm_adam
   const StepSegDev* t = static_cast<const StepSegDev*>(image);
   const dim3 grid(grid_for(tiles * kStepParts)), block(kThreads);
   switch (div_kind(kWorld, average != 0)) {
-    case 0: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 0, kOrder>), grid, block, 0, stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
-    case 1: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 1, kOrder>), grid, block, 0, stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
-    default: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 2, kOrder>), grid, block, 0, stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
+    case 0: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 0, kOrder>), grid, block, occupancy_pad(TDM_XCD_STEP), stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
+    case 1: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 1, kOrder>), grid, block, occupancy_pad(TDM_XCD_STEP), stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
+    default: hipLaunchKernelGGL((k23_zero2_step_kernel<kWorld, 2, kOrder>), grid, block, occupancy_pad(TDM_XCD_STEP), stream, t, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
   }
 }
 
@@ -292,9 +314,9 @@ void launch_step_one_o(const StepSegDev& whole, int64_t tiles, int average, cons
   const Divisor<float> dv = make_divisor<float>(kWorld);
   const dim3 grid(grid_for(tiles * kStepParts)), block(kThreads);
   switch (div_kind(kWorld, average != 0)) {
-    case 0: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 0, kOrder>), grid, block, 0, stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
-    case 1: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 1, kOrder>), grid, block, 0, stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
-    default: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 2, kOrder>), grid, block, 0, stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
+    case 0: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 0, kOrder>), grid, block, occupancy_pad(TDM_XCD_STEP), stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
+    case 1: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 1, kOrder>), grid, block, occupancy_pad(TDM_XCD_STEP), stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
+    default: hipLaunchKernelGGL((k23_zero2_step_one_kernel<kWorld, 2, kOrder>), grid, block, occupancy_pad(TDM_XCD_STEP), stream, whole, tiles, dv, s, xcd_shift(TDM_XCD_STEP, kWorld, true)); break;
   }
 }
 
@@ -648,10 +670,28 @@ int tdm_local_all_reduce(void* const* bufs, int world, int64_t numel, int dtype,
 
 int tdm_table_tile_bytes(void) { return kTileVecs * 16; }
 
+int tdm_build_geometry(int* k1_tile_bytes, int* workgroup_lanes, int* table_tile_bytes) {
+  return guard([&] {
+    if (!k1_tile_bytes || !workgroup_lanes || !table_tile_bytes) throw Invalid("NULL argument");
+    *k1_tile_bytes = kK1TileVecs * 16;
+    *workgroup_lanes = kThreads;
+    *table_tile_bytes = kTileVecs * 16;
+  });
+}
+
 int tdm_set_blocks_per_cu(int blocks) {
   return guard([&] {
     if (blocks < 0 || blocks > 1024) throw Invalid("blocks per compute unit must be in [0, 1024]");
     g_blocks_per_cu = blocks == 0 ? kDefaultBlocksPerCu : blocks;
+  });
+}
+
+int tdm_set_occupancy_pad(int kind, int bytes) {
+  return guard([&] {
+    if (kind < -1 || kind >= kXcdKinds) throw Invalid("unknown kernel family");
+    if (bytes < -1 || bytes > 65536) throw Invalid("the pad must be in [0, 65536] bytes, or -1 for the default");
+    for (int k = 0; k < kXcdKinds; ++k)
+      if (kind == -1 || kind == k) g_occupancy_pad[k].store(bytes, std::memory_order_relaxed);
   });
 }
 
@@ -877,15 +917,16 @@ void adamw_launch(float* p, const float* g, float* m, float* v, int64_t n, const
   const int64_t tiles = vec ? (n / 4 + kAdamwThreads * kAdamwUnroll - 1) / (kAdamwThreads * kAdamwUnroll) : (n + kAdamwThreads - 1) / kAdamwThreads;
   const dim3 grid(grid_for(std::max<int64_t>(tiles, 1)));
   const int which = (order == TDM_ADAMW_HOST_ORDER ? 0 : 4) + (vec ? 2 : 0) + (ncopies > 0 ? 1 : 0);
+  const unsigned pad = occupancy_pad(TDM_XCD_ADAMW);
   switch (which) {
-    case 0: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, false, false>), grid, block, 0, st, a); break;
-    case 1: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, false, true>), grid, block, 0, st, a); break;
-    case 2: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true, false>), grid, block, 0, st, a); break;
-    case 3: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true, true>), grid, block, 0, st, a); break;
-    case 4: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, false, false>), grid, block, 0, st, a); break;
-    case 5: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, false, true>), grid, block, 0, st, a); break;
-    case 6: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true, false>), grid, block, 0, st, a); break;
-    default: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true, true>), grid, block, 0, st, a); break;
+    case 0: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, false, false>), grid, block, pad, st, a); break;
+    case 1: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, false, true>), grid, block, pad, st, a); break;
+    case 2: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true, false>), grid, block, pad, st, a); break;
+    case 3: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_HOST_ORDER, true, true>), grid, block, pad, st, a); break;
+    case 4: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, false, false>), grid, block, pad, st, a); break;
+    case 5: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, false, true>), grid, block, pad, st, a); break;
+    case 6: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true, false>), grid, block, pad, st, a); break;
+    default: hipLaunchKernelGGL((k3_adamw_kernel<TDM_ADAMW_DEVICE_ORDER, true, true>), grid, block, pad, st, a); break;
   }
   check_hip(hipGetLastError(), "k3_adamw launch");
 }

@@ -556,7 +556,7 @@ struct FillBatch {
   tdm_fold_seg seg[kFillSegs];
 };
 
-__global__ __launch_bounds__(256) void k2_table_fill_kernel(FillBatch b, FoldSegDev* __restrict__ out) {
+__global__ __launch_bounds__(256) __attribute__((unused)) void k2_table_fill_kernel(FillBatch b, FoldSegDev* __restrict__ out) {
   const int64_t tile = b.first[0] + static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (tile >= b.first[b.nseg]) return;
   int k = 0;

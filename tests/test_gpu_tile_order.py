@@ -132,3 +132,85 @@ def test_setter_refuses_nonsense(order):
     assert L.tdm_set_xcd_group(6, 0) == 1 and b"family" in L.tdm_last_error()
     assert L.tdm_set_xcd_group(0, 13) == 1 and b"shift" in L.tdm_last_error()
     assert L.tdm_set_xcd_group(-2, 0) == 1
+
+
+def test_occupancy_pad_changes_no_result():
+    """The unused LDS that caps how many workgroups share a compute unit is geometry too:
+    the one-launch step, AdamW with copies and the by-value fold give the same bits with no
+    pad, the defaults and the largest pad."""
+    from tandem_amd import LocalWorld
+    from tandem_amd._lib import lib
+    from tandem_amd.local import LocalZeRO2
+
+    L = lib()
+    dev = torch.device("cuda", 0)
+    world = 4
+    numels = [tiles_to_elems(61, 3), 11, tiles_to_elems(200, 0), 513]
+    n = sum(numels)
+    p0 = seeded(1, 0, n, 0.02)
+    grads = [seeded(20, r, n, 1e-3) for r in range(world)]
+
+    def run():
+        z = LocalZeRO2(world, numels, dev, bucket_bytes=1 << 20, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+        for b in z.bufs:
+            b.copy_(p0)
+        for r in range(world):
+            z.staging[r].copy_(grads[r])
+        z.reduce_and_step()
+        z.reduce_grads("fold")
+        z.step(fused_gather=True)
+        bufs = [g.to(dev) for g in grads]
+        LocalWorld(world).all_reduce(bufs, "avg", algorithm="fold")
+        torch.cuda.synchronize()
+        return [b.cpu() for b in z.bufs] + [t.cpu() for o in z.opts for t in o.state["flat"][1:]] + [b.cpu() for b in bufs]
+
+    try:
+        assert L.tdm_set_occupancy_pad(-1, 0) == 0
+        want = run()
+        for pad in (-1, 65536, 4096):
+            assert L.tdm_set_occupancy_pad(-1, pad) == 0
+            for a, b in zip(want, run()):
+                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), pad
+        assert L.tdm_set_occupancy_pad(0, 65537) == 1 and b"pad" in L.tdm_last_error()
+        assert L.tdm_set_occupancy_pad(6, 0) == 1 and b"family" in L.tdm_last_error()
+    finally:
+        assert L.tdm_set_occupancy_pad(-1, -1) == 0
+
+
+def test_stream_mix_probe_moves_what_it_says():
+    """The measurement kernel: every written stream receives the same function of the read
+    streams (their lane-wise 32-bit sum plus a pattern), whatever the geometry; bad arguments
+    are refused."""
+    import ctypes
+
+    from tandem_amd._lib import lib, stream_ptr
+
+    L = lib()
+    dev = torch.device("cuda", 0)
+    n = tiles_to_elems(37, 0) + 8
+    src = [torch.randint(-2**31, 2**31 - 1, (n,), dtype=torch.int32, device=dev) for _ in range(3)]
+    outs = {}
+    for per_lane, shift, pad in ((1, 0, 0), (2, 3, 16384), (1, 6, 65536)):
+        dst = [torch.zeros(n, dtype=torch.int32, device=dev) for _ in range(2)]
+        rd = (ctypes.c_void_p * 8)(*[t.data_ptr() for t in src])
+        wr = (ctypes.c_void_p * 8)(*[t.data_ptr() for t in dst])
+        assert L.tdm_probe_stream_mix(rd, 3, wr, 2, n * 4, per_lane, shift, pad, stream_ptr(dev)) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(dst[0], dst[1])
+        outs[(per_lane, shift, pad)] = dst[0].cpu()
+    first = outs[(1, 0, 0)]
+    total = (src[0].cpu().to(torch.int64) + src[1].cpu() + src[2].cpu())
+    lane = torch.arange(n) % 4
+    # lanes 1..3 of every vector carry sum + 1, 2, 3; lane 0 carries sum + the vector's index within the launch
+    want = ((total + lane) & 0xffffffff).to(torch.int64)
+    got = first.to(torch.int64) & 0xffffffff
+    assert torch.equal(got[lane != 0], want[lane != 0])
+    assert torch.equal(outs[(1, 6, 65536)][lane != 0], first[lane != 0])
+    assert torch.equal(outs[(2, 3, 16384)][lane != 0], first[lane != 0])
+    rd = (ctypes.c_void_p * 8)(src[0].data_ptr())
+    assert L.tdm_probe_stream_mix(rd, 1, None, 0, n * 4, 1, 0, 0, stream_ptr(dev)) == 0  # read-only
+    assert L.tdm_probe_stream_mix(rd, 0, None, 0, n * 4, 1, 0, 0, stream_ptr(dev)) == 1
+    assert L.tdm_probe_stream_mix(rd, 1, None, 0, n * 4 + 4, 1, 0, 0, stream_ptr(dev)) == 1
+    assert L.tdm_probe_stream_mix(rd, 1, None, 0, n * 4, 3, 0, 0, stream_ptr(dev)) == 1
+    assert L.tdm_probe_stream_mix(rd, 9, None, 0, n * 4, 1, 0, 0, stream_ptr(dev)) == 1
+    torch.cuda.synchronize()

@@ -133,3 +133,26 @@ def test_16bit_conversions_match_numpy_and_torch():
     lib().orc_f32_to_bf16(ctypes.c_void_p(f.ctypes.data), ctypes.c_void_p(got.ctypes.data), ctypes.c_int64(f.size))
     want = torch.from_numpy(f).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(got, want)
+
+
+def test_cpu_baseline_optimizer_is_the_same_update():
+    """The torch-op optimizer that bench.py times as tandem's CPU backend gives the
+    oracle's bits when the oracle uses torch's CPU sqrt: p, exp_avg, exp_avg_sq over
+    six steps, both lerp branches, with and without weight decay, empty shard."""
+    from oracle.cpu_engine import TorchCpuAdamW
+
+    for kw in (dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1), dict(lr=1e-2, betas=(0.3, 0.999), eps=1e-6, weight_decay=0.0)):
+        timed_one = TorchCpuAdamW(**kw)
+        checker = AdamW(**kw, sqrt=lambda v: torch.from_numpy(v).sqrt().numpy())
+        gen = torch.Generator().manual_seed(5)
+        p = torch.randn(10_007, generator=gen) * 0.02
+        pn = p.numpy().copy()
+        for step in range(6):
+            g = torch.randn(10_007, generator=gen) * 1e-3
+            timed_one.update("k", p, g)
+            checker.update("k", pn, g.numpy())
+            assert np.array_equal(bits(p.numpy()), bits(pn)), f"step {step}"
+        assert np.array_equal(bits(timed_one.state["k"]["m"].numpy()), bits(checker.state["k"][1]))
+        assert np.array_equal(bits(timed_one.state["k"]["v"].numpy()), bits(checker.state["k"][2]))
+        timed_one.update("empty", torch.zeros(0), torch.zeros(0))
+        assert timed_one.state["empty"]["t"] == 1.0
