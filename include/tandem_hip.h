@@ -23,6 +23,12 @@ extern "C" {
 
 typedef void* tdm_stream;
 
+/* The element types the reducing kernels know. A deliberate difference from the reference, whose
+ * engine reduces any ATen dtype by falling back to add_ (tandem/csrc/collectives.cpp:254-256): every
+ * entry point that adds (tdm_k1_reduce_step, tdm_local_*, tdm_k2_*, tdm_all_reduce, tdm_reduce_scatter,
+ * tdm_direct_*) refuses any other code with TDM_EINVAL ("unknown dtype"), so int8 / uint8 / int16 / bool
+ * sums are not offered. Entry points that only copy (tdm_all_gather, tdm_broadcast, tdm_sendrecv,
+ * tdm_unit_gather) also take TDM_BYTES, which covers every dtype. */
 enum tdm_dtype { TDM_F32 = 0, TDM_F64 = 1, TDM_F16 = 2, TDM_BF16 = 3, TDM_I64 = 4, TDM_I32 = 5 };
 
 enum { TDM_MAX_PAIRS = 16, TDM_MAX_WORLD = 8 };

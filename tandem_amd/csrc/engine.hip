@@ -1141,8 +1141,10 @@ std::shared_ptr<Work> Engine::direct(int kind, Buf t, std::vector<int64_t> sizes
     const auto cs = chunks(t, sizes);
     const char* base[TDM_MAX_PAIRS > TDM_MAX_WORLD ? TDM_MAX_PAIRS : TDM_MAX_WORLD];
     if (size_ > static_cast<int>(sizeof base / sizeof base[0])) throw Invalid("direct collective: too many ranks");
-    if (t.numel > 0) direct_bases(t, peer_offsets, base);  // an empty tensor still takes part in the fences
     barrier_now(true, fence_tag(5 + kind, t.dtype, t.numel));  // every rank's input is complete
+    // The peers' arenas are looked up behind the first fence: a rank that has reached it has shared its
+    // arena, so the first direct collective of a group needs no barrier of the caller's before it.
+    if (t.numel > 0) direct_bases(t, peer_offsets, base);  // an empty tensor still takes part in the fences
     if (kind != 2) {
       direct_fold(t, cs, base, average);
       barrier_now(true);  // every chunk is folded (or, for reduce_scatter: nobody reads our tensor any more)
@@ -1182,6 +1184,7 @@ std::shared_ptr<Work> Engine::zero2_step_direct(Buf param, Buf grad, std::vector
   return submit([this, param, grad, param_offsets, grad_offsets, exp_avg, exp_avg_sq, total, average, s, order] {
     tdm_step_seg seg;
     std::memset(&seg, 0, sizeof seg);
+    if (size_ > 1) barrier_now(true, fence_tag(9, TDM_F32, total));
     if (param.numel > 0) {  // a rank with an empty shard still takes part in the fences
       const char* base[TDM_MAX_WORLD];
       direct_bases(grad, grad_offsets, base);
@@ -1193,7 +1196,6 @@ std::shared_ptr<Work> Engine::zero2_step_direct(Buf param, Buf grad, std::vector
       seg.count = param.numel;
       seg.chunk = rank_;
     }
-    if (size_ > 1) barrier_now(true, fence_tag(9, TDM_F32, total));
     zero2_step_segment(seg, size_, average, s, order, stream_);
     if (size_ > 1) barrier_now(true);
   }, caller, true, true, true);

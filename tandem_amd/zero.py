@@ -8,23 +8,17 @@ parallelism that shards what every rank would otherwise keep a full copy of.
                  staging buffer, a rank keeps only the sums that fall in its
                  shard, the staging buffer is dropped.
   FSDP           stage 3, parameters sharded too, one unit of the model at a time
-                 (model.units()): a unit's full parameters exist only while it
-                 runs; the next unit's gather is already under way on the engine's
-                 stream while this one computes.
+                 (model.units()): see fsdp.py.
 
-Drop-ins for the reference's classes (tandem/zero.py:69-336 there): same
+Drop-ins for the reference's classes (tandem/zero.py:69-170 there): same
 constructors, same `loss = z(x, y); loss.backward(); z.step(); z.zero_grad()`
 protocol, same bucket ranges, shard boundaries and submission order, so every
 collective sees the same chunks and the results are the reference's bit for bit.
 Differences: gradients enter a bucket through one `group.pack` gather per bucket
-(per unit for FSDP) instead of one copy per parameter; FSDP's gather is
-`group.gather_unit` (shard placement + all-gather on the engine's stream); the
-optimizer is the fused ShardedAdamW kernel.
+instead of one copy per parameter; the optimizer is the fused ShardedAdamW kernel.
 
-`group` is anything with tandem's Group interface plus pack() and gather_unit().
+`group` is anything with tandem's Group interface plus pack().
 """
-
-import warnings
 
 import torch
 from torch.autograd import Variable
@@ -67,8 +61,9 @@ class ZeRO(torch.nn.Module):
         writes the new parameters into every rank's buffer: the reduce_scatters,
         `grad_shard.add_`, the update and the all_gather in one pass, same bits.
         `grad_shard` is then only filled when a second backward comes before step()
-        (accumulation): that backward first reduces the packed gradients the ordinary
-        way, and the step after it is the ordinary one."""
+        (accumulation) or after a step() without zero_grad() in between: that backward
+        first reduces the gradients still packed in the pool the ordinary way, and the
+        step after it is the ordinary one."""
         super().__init__()
         if stage not in (1, 2):
             raise ValueError("ZeRO handles stages 1 and 2; stage 3 is FSDP")
@@ -86,6 +81,7 @@ class ZeRO(torch.nn.Module):
             if not hasattr(self.opt, "begin_step"):
                 raise TypeError("fused_step needs an optimizer with begin_step() (tandem_amd.ShardedAdamW has it)")
         self._packed = False      # fused_step: a whole backward's gradients lie packed in the pool, not yet reduced
+        self._applied = False     # fused_step: the pool's gradients went into a step but never into grad_shard
         self._shard_zero = True   # nothing has been added to grad_shard since zero_grad()
         params = [p for p in module.parameters() if p.requires_grad]
         self.params = params
@@ -138,8 +134,11 @@ class ZeRO(torch.nn.Module):
                 rng.loose = []
             rng.work = self.g.all_reduce(self.grad[rng.a:rng.b], op="avg", async_op=True, **self._how)
         else:
-            if self._packed:
-                self._reduce_packed()  # accumulation: the previous backward's gradients, before they are overwritten
+            if self._packed or self._applied:
+                # the previous backward's gradients, before they are overwritten: accumulation over several
+                # backward passes, or a step() that was not followed by zero_grad() (the reference's
+                # grad_shard still holds that sum then, tandem/zero.py:150-170)
+                self._reduce_packed()
             p0 = rng.params[0]
             rng.staging = (self._pool[rng.a:rng.b] if self.direct
                            else torch.empty(rng.b - rng.a, device=p0.device, dtype=p0.dtype))
@@ -197,7 +196,7 @@ class ZeRO(torch.nn.Module):
                  for r in self.buckets]
         for rng, work in zip(self.buckets, works):
             self._add_mine(rng, work.wait())
-        self._packed = False
+        self._packed = self._applied = False
 
     @torch.no_grad()
     def step(self):
@@ -205,7 +204,7 @@ class ZeRO(torch.nn.Module):
         if self._packed:
             scalars, exp_avg, exp_avg_sq, order = self.opt.begin_step("flat", self.buf[lo:hi])
             self.g.zero2_step(self.buf, self._pool, self.flat.sizes, exp_avg, exp_avg_sq, scalars, order, op="avg")
-            self._packed = False
+            self._packed, self._applied = False, True
             return
         grad = self.grad[lo:hi] if self.stage == 1 else self.grad_shard
         self.opt.update("flat", self.buf[lo:hi], grad)
@@ -226,214 +225,10 @@ class ZeRO(torch.nn.Module):
             for p in self.params:
                 p.grad = None
         else:
-            self._packed = False  # packed gradients not yet reduced are dropped with the rest
+            self._packed = self._applied = False  # packed gradients not yet reduced are dropped with the rest
             if not self._shard_zero:
                 self.grad_shard.zero_()
             self._shard_zero = True
 
 
-def _pad(n):
-    """Shards start on 16-byte boundaries inside the arena (fp32: multiples of 4 elements)."""
-    return (n + 3) // 4 * 4
-
-
-class _Unit:
-    def __init__(self, index, module, params, world, rank, device, dtype):
-        self.index, self.module, self.params = index, module, params
-        self.flat = FlatLayout([p.numel() for p in params], world, rank)
-        self.offset = dict(zip(params, self.flat.offsets))
-        self.full = torch.empty(self.flat.numel, device=device, dtype=dtype)
-        self.nbytes = self.full.untyped_storage().nbytes()
-        self.shard = None
-        self.grad_shard = torch.zeros(self.flat.hi - self.flat.lo, device=device, dtype=dtype)
-        self.gathered = True
-        self.pending = None  # gather in flight
-        self.arrived = 0
-        self.rs = None  # reduce-scatter in flight
-        self.staging = None
-        self.peer_offsets = None
-
-
-class FSDP(torch.nn.Module):
-    """ZeRO stage 3 over model.units()."""
-
-    def __init__(self, model, group, optimizer=None, prefetch=True, direct=None):
-        super().__init__()
-        _need(group, "pack", "gather_unit")
-        self.module, self.g = model, group
-        self.opt = optimizer if optimizer is not None else ShardedAdamW()
-        self.prefetch = prefetch
-        # The first unit's input (token ids) needs no gradient; torch then fires the
-        # unit's backward pre-hook on its outputs, which is the moment wanted here.
-        warnings.filterwarnings("ignore", message="Full backward hook is firing when gradients are computed with respect to module outputs")
-        self.live = 0  # units whose full parameters exist right now
-        self.max_live = 0
-        self.units, self.unit_of = [], {}
-        claimed = set()
-        # Where the group offers it, all shards live in one arena that the other ranks
-        # map once and read directly: a gather is then copies only, with a fence()
-        # around the optimizer step instead of a handshake per gather.
-        self._direct = direct if direct is not None else hasattr(group, "shared_empty")
-        arena, arena_at, self._peer_at = None, 0, [0] * group.size
-        if self._direct:
-            from .buckets import FlatLayout as _L
-
-            mods = model.units()
-            seen, total = set(), [0] * group.size
-            for m in mods:
-                ps = [p for p in m.parameters() if p.requires_grad and id(p) not in seen]
-                seen.update(id(p) for p in ps)
-                sizes = _L([p.numel() for p in ps], group.size, 0).sizes
-                total = [t + _pad(s) for t, s in zip(total, sizes)]
-            p0 = next(model.parameters())
-            try:
-                arena = group.shared_empty(max(total), p0.dtype)
-            except Exception:
-                self._direct, arena = False, None  # too large for one IPC allocation: stage through the slots
-        for i, m in enumerate(model.units()):
-            ps = [p for p in m.parameters() if p.requires_grad and id(p) not in claimed]
-            claimed.update(id(p) for p in ps)
-            u = _Unit(i, m, ps, group.size, group.rank, ps[0].device, ps[0].dtype)
-            with torch.no_grad():
-                self.g.pack(u.full, [(u.offset[p], p.data) for p in ps])
-                self.g.broadcast(u.full, root=0)
-                for p in ps:
-                    o = u.offset[p]
-                    p.data = u.full[o:o + p.numel()].view_as(p)
-                if arena is not None:
-                    es = u.full.element_size()
-                    u.shard = arena[self._peer_at[group.rank]:self._peer_at[group.rank] + (u.flat.hi - u.flat.lo)]
-                    u.shard.copy_(u.full[u.flat.lo:u.flat.hi])
-                    u.peer_offsets = [at * es for at in self._peer_at]  # this unit's shard in every rank's arena, bytes
-                    self._peer_at = [at + _pad(s) for at, s in zip(self._peer_at, u.flat.sizes)]
-                else:
-                    u.shard = u.full[u.flat.lo:u.flat.hi].clone()
-            for p in ps:
-                self.unit_of[p] = u
-                p.register_post_accumulate_grad_hook(self._on_grad)
-            m.register_forward_pre_hook(self._before_forward(u))
-            m.register_forward_hook(self._after_forward(u))
-            m.register_full_backward_pre_hook(self._before_backward(u))
-            self.live += 1  # _Unit allocated it whole
-            self._release(u)
-            self.units.append(u)
-        if len(claimed) != sum(1 for p in model.parameters() if p.requires_grad):
-            raise ValueError("every parameter must belong to one of model.units()")
-        self._callback_queued = False
-        self.max_live = 0
-        if self._direct:
-            self.g.fence()  # every rank's shards are in place before anyone gathers
-
-    def forward(self, *args, **kwargs):
-        return self.module(*args, **kwargs)
-
-    # ---- a unit's full parameters: start gathering, wait, release
-    def _start(self, u):
-        if u.gathered or u.pending is not None:
-            return
-        u.full.untyped_storage().resize_(u.nbytes)
-        self.live += 1
-        self.max_live = max(self.max_live, self.live)
-        if self._direct:
-            u.pending = self.g.gather_unit(u.full, u.shard, u.flat.sizes, async_op=True, peer_offsets=u.peer_offsets)
-        else:
-            u.pending = self.g.gather_unit(u.full, u.shard, u.flat.sizes, async_op=True)
-
-    def _ensure(self, u):
-        self._start(u)
-        if u.pending is not None:
-            u.pending.wait()
-            u.pending = None
-            u.gathered = True
-
-    def _release(self, u):
-        if u.pending is not None:
-            u.pending.wait()
-            u.pending = None
-        if u.full.untyped_storage().nbytes():
-            self.live -= 1
-        u.full.untyped_storage().resize_(0)
-        u.gathered = False
-
-    # ---- hooks
-    def _before_forward(self, u):
-        def hook(mod, args):
-            self._ensure(u)
-            if self.prefetch and u.index + 1 < len(self.units):
-                self._start(self.units[u.index + 1])
-
-        return hook
-
-    def _after_forward(self, u):
-        def hook(mod, args, out):
-            # The last unit's backward comes first: keep it.
-            if torch.is_grad_enabled() and u.index == len(self.units) - 1:
-                return
-            self._release(u)
-
-        return hook
-
-    def _before_backward(self, u):
-        def hook(mod, grad_out):
-            if not self._callback_queued:
-                self._callback_queued = True
-                Variable._execution_engine.queue_callback(self._after_backward)
-            self._ensure(u)
-            if self.prefetch and u.index > 0:
-                self._start(self.units[u.index - 1])
-
-        return hook
-
-    def _on_grad(self, p):
-        u = self.unit_of[p]
-        u.arrived += 1
-        if u.arrived == len(u.params):
-            # The unit's backward is done: gather its gradients into one staging
-            # buffer with a single launch, drop its full parameters, and send the
-            # gradients on their way.
-            u.staging = torch.empty(u.flat.numel, device=p.device, dtype=p.dtype)
-            self.g.pack(u.staging, [(u.offset[q], q.grad) for q in u.params])
-            for q in u.params:
-                q.grad = None
-            self._release(u)
-            # only `mine` is kept of the staging buffer: the other chunks' partial sums are not needed
-            how = {"partial_sums": False} if getattr(self.g, "partial_sums_optional", False) else {}
-            u.rs = self.g.reduce_scatter(u.staging, u.flat.sizes, op="avg", async_op=True, **how)
-
-    def _after_backward(self):
-        self._callback_queued = False
-        for u in self.units:
-            if u.arrived != len(u.params):
-                raise RuntimeError("tandem FSDP: every parameter must receive a gradient")
-            mine = u.rs.wait()
-            if mine.numel():
-                u.grad_shard.add_(mine)
-            u.rs, u.staging, u.arrived = None, None, 0
-            if u.gathered:
-                self._release(u)
-
-    @torch.no_grad()
-    def step(self):
-        if self._direct:
-            self.g.fence()  # no rank still reads the shards this step rewrites
-        for u in self.units:
-            self.opt.update(u.index, u.shard, u.grad_shard)
-        if self._direct:
-            self.g.fence()  # the new shards are complete before any rank gathers them
-
-    def zero_grad(self):
-        for u in self.units:
-            u.grad_shard.zero_()
-
-    @torch.no_grad()
-    def full_parameters(self):
-        """All parameters, gathered (for checkpoints and tests)."""
-        out = []
-        for u in self.units:
-            full = torch.empty(u.flat.numel, device=u.shard.device, dtype=u.shard.dtype)
-            if self._direct:
-                self.g.gather_unit(full, u.shard, u.flat.sizes, peer_offsets=u.peer_offsets)
-            else:
-                self.g.gather_unit(full, u.shard, u.flat.sizes)
-            out.append(full)
-        return torch.cat(out)
+from .fsdp import FSDP  # noqa: E402,F401  (stage 3 has a file of its own; importable from here as in the reference)

@@ -27,7 +27,7 @@ def deterministic():
     torch.backends.cuda.matmul.allow_tf32 = False
 
 
-def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1):
+def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1, zero_every=1):
     from tandem_amd import ShardedAdamW
     from tandem_amd.data import synthetic
     from tandem_amd.ddp import DDP
@@ -71,7 +71,8 @@ def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1):
             opt.zero_grad()
         else:
             z.step()
-            z.zero_grad()
+            if (step + 1) % zero_every == 0:
+                z.zero_grad()
     if strategy.startswith("zero3"):
         w = z.full_parameters()
         extra = {"max_live": z.max_live, "live": z.live}
@@ -81,7 +82,7 @@ def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1):
     return {"losses": losses, "weights": w.cpu(), **extra}
 
 
-def one_process(world, accumulate=1):
+def one_process(world, accumulate=1, zero_every=1):
     """Both ranks' gradients computed in this process, averaged as (a/2) + (b/2),
     torch AdamW on the GPU."""
     from tandem_amd.data import synthetic
@@ -95,6 +96,7 @@ def one_process(world, accumulate=1):
     model = GPT(c).to(dev)
     opt = torch.optim.AdamW(model.parameters(), lr=LR, weight_decay=WD, foreach=False, fused=False)
     losses = [[] for _ in range(world)]
+    kept = None
     for step in range(STEPS):
         grads = []
         for r in range(world):
@@ -106,8 +108,10 @@ def one_process(world, accumulate=1):
             grads.append([p.grad.clone() for p in model.parameters()])
             opt.zero_grad()
         for i, p in enumerate(model.parameters()):
-            p.grad = grads[0][i] / world + grads[1][i] / world
+            mean = grads[0][i] / world + grads[1][i] / world
+            p.grad = mean if kept is None else kept[i] + mean  # what a gradient shard holds when it was not zeroed
         opt.step()
+        kept = None if (step + 1) % zero_every == 0 else [p.grad.clone() for p in model.parameters()]
         opt.zero_grad()
     return losses, torch.cat([p.detach().reshape(-1) for p in model.parameters()]).cpu()
 
@@ -192,3 +196,23 @@ def test_stream_ordered_wait_gives_the_same_weights(monkeypatch):
         for r in range(2):
             assert res[r]["losses"] == ref_losses[r], (s, r)
             assert torch.equal(res[r]["weights"], ref_w), (s, r)
+
+
+def test_step_without_zero_grad_keeps_the_old_gradients():
+    """tandem's ZeRO-2 zeroes its gradient shard only in zero_grad() (tandem/zero.py:165-170
+    in the reference): a step() followed by another backward steps on the SUM of both
+    gradients. The one-launch step never fills the shard, so it has to catch up here. Two
+    ranks: equal to one process that keeps the gradients; four ranks: equal to the
+    ordinary path, where the ring's order matters."""
+    from tandem_amd import launch
+
+    ref_losses, ref_w = one_process(2, zero_every=2)
+    for s in ("zero2", "zero2d", "zero2f"):
+        res = launch(train_rank, 2, s, 4 << 10, STEPS, BATCH, 1, 2, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT)
+        for r in range(2):
+            assert res[r]["losses"] == ref_losses[r], (s, r)
+            assert torch.equal(res[r]["weights"], ref_w), (s, r)
+    runs = {s: launch(train_rank, 4, s, 4 << 10, 5, 8, 1, 3, slot_bytes=1024, gpus=[0] * 4, timeout=TIMEOUT) for s in ("zero2", "zero2f")}
+    for r in range(4):
+        assert runs["zero2f"][r]["losses"] == runs["zero2"][r]["losses"], r
+        assert torch.equal(runs["zero2f"][r]["weights"], runs["zero2"][0]["weights"]), r
