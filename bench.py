@@ -137,19 +137,27 @@ def time_ring(lw, bufs, steps, warmup):
 
 
 def sweep(lw, dev, steps):
-    """Per-rank message sizes 64 KiB ... 256 MiB. Ring: algorithmic bytes 15 B per
-    pass. Fold: the same all-reduce as one launch, 8 W B = 32 B... per pass."""
+    """Per-rank message sizes 64 KiB ... 256 MiB, reduce-scatter (avg) + all-gather three ways.
+    ring_*: the ring's steps, one launch each (K1 and the copy step), 15 B algorithmic bytes per
+    pass of a per-rank message of B bytes. one_launch_*: the reduce-scatter as one launch and the
+    all-gather as one launch, 13 B (what the library picks up to 80 MiB per rank at this world
+    size; the same bits in memory). fold_*: the all-reduce as a single launch, 8 B... 2 W B."""
     import torch
+
+    from tandem_amd._lib import check, lib
 
     rows = []
     for kib in (64, 1024, 4096, 16384, 65536, 262144):
         n = kib * 1024 // 4
         bufs = seeded_grads(WORLD, n, dev, 1e-2)
         reps = steps if kib >= 65536 else max(steps, 30)
+        check(lib().tdm_set_ring_form(1))  # reduce-scatter and all-gather as one launch each
+        one, _, _ = time_ring(lw, bufs, reps, 3)
+        check(lib().tdm_set_ring_form(0))  # the ring's steps, one launch each: K1 and the copy step
         per, rs, ag = time_ring(lw, bufs, reps, 3)
         fold = timed(lambda: lw.all_reduce(bufs, "avg", algorithm="fold"), reps)
         b = n * 4
-        graph_ms = fold_graph_ms = None
+        graph_ms = fold_graph_ms = one_graph_ms = None
         if kib <= 65536:  # sizes where the gaps between the six launches still count: the same ring pass replayed from a HIP graph
             flats = [x.reshape(-1) for x in bufs]
             graph = torch.cuda.CUDAGraph()
@@ -157,6 +165,13 @@ def sweep(lw, dev, steps):
                 ring_pass(lw, flats)
             graph_ms = round(timed(graph.replay, reps) * 1e3, 4)
             del graph
+            check(lib().tdm_set_ring_form(1))
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                ring_pass(lw, flats)
+            one_graph_ms = round(timed(graph.replay, reps) * 1e3, 4)
+            del graph
+            check(lib().tdm_set_ring_form(0))
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 lw.all_reduce(bufs, "avg", algorithm="fold")
@@ -167,11 +182,19 @@ def sweep(lw, dev, steps):
                      "k1_frac_of_hbm": round(12 * n * (WORLD - 1) / (rs * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                      "fold_ms": round(fold * 1e3, 4), "fold_GBps": round(2 * WORLD * b / fold / 1e9, 1),  # every rank's b bytes read once, written once
                      "fold_algbw_GBps": round(b / fold / 1e9, 1)})
+        # one launch each: W reads + (W-1) writes per element, then W-1 copies from the owner = (4W - 3) B per pass
+        one_bytes = (4 * WORLD - 3) * b
+        default_one = kib * 1024 * WORLD <= (320 << 20)
+        rows[-1].update({"one_launch_ms": round(one * 1e3, 4), "one_launch_GBps": round(one_bytes / one / 1e9, 1),
+                         "one_launch_frac_of_hbm": round(one_bytes / one / 1e9 / HBM_PEAK_GBPS, 4),
+                         "default_form": "one_launch" if default_one else "steps"})
         if graph_ms is not None:
             rows[-1]["ring_hip_graph_ms"] = graph_ms
+            rows[-1]["one_launch_hip_graph_ms"] = one_graph_ms
             rows[-1]["fold_hip_graph_ms"] = fold_graph_ms
         del bufs
         torch.cuda.empty_cache()
+    check(lib().tdm_set_ring_form(-1))
     return rows
 
 
@@ -590,8 +613,12 @@ def summarize(line):
         if mib in (4.0, 16.0, 64.0, 256.0):
             tag = f"{int(mib)}MiB"
             roof[f"k1_frac_{tag}"] = row["k1_frac_of_hbm"]
-            cfg[f"pass_frac_{tag}"] = round(row["ring_GBps"] / HBM_PEAK_GBPS, 4)
-            cfg[f"pass_ms_{tag}"] = row["ring_ms"]
+            # the pass as the library runs it by default at this size, on that form's own byte count
+            one = row["default_form"] == "one_launch"
+            cfg[f"pass_ms_{tag}"] = row["one_launch_ms"] if one else row["ring_ms"]
+            cfg[f"pass_frac_{tag}"] = row["one_launch_frac_of_hbm"] if one else round(row["ring_GBps"] / HBM_PEAK_GBPS, 4)
+            cfg[f"pass_steps_ms_{tag}"] = row["ring_ms"]
+            cfg[f"pass_steps_frac_{tag}"] = round(row["ring_GBps"] / HBM_PEAK_GBPS, 4)
             cfg[f"fold_pass_ms_{tag}"] = row["fold_ms"]
     mix = line.get("stream_mix", {})
 
@@ -698,7 +725,9 @@ def main():
     lw = LocalWorld(WORLD)
     n = args.mib * (1 << 20) // 4
     bufs = seeded_grads(WORLD, n, dev, 1e-2)
+    _lib.check(_lib.lib().tdm_set_ring_form(0))  # the headline is the ring's steps (K1) at every --mib
     per, rs_ms, ag_ms = time_ring(lw, bufs, args.steps, args.warmup)
+    _lib.check(_lib.lib().tdm_set_ring_form(-1))
     b = n * 4
     k1_launch_s = rs_ms * 1e-3 / (WORLD - 1)
     k1_bytes = 12 * n  # one launch: 4 chunk pairs of n/4 elements; two loads and one store of 4 bytes per element

@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(CSRC, "libtandem_hip.so")
-SOURCES = ["kernels.hip", "probe.hip", "abi.hip", "engine.hip", "engine_abi.hip"]
+SOURCES = ["kernels.hip", "kernels_chain.hip", "probe.hip", "abi.hip", "engine.hip", "engine_abi.hip"]
 
 # -ffp-contract=off: no multiply-add is fused unless the source says fma.
 # -fhip-fp32-correctly-rounded-divide-sqrt: IEEE division and sqrt (the default; stated).

@@ -51,6 +51,12 @@ void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool s
                  bool writeback_src, hipStream_t stream, int policy = 2);
 void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream, int policy = 2);
 void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream);
+// kernels_chain.hip: the ring reduce-scatter of a whole group in one launch (rank q's buffer at base[q], chunk c =
+// elements [lo[c], lo[c] + len[c])); world sizes 2..kChainMaxWorld
+constexpr int kChainMaxWorld = 4;
+bool chain_handles(int world);
+void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
+                          bool keep_sent, int max_grid, hipStream_t stream);
 void zero2_step_segment(const tdm_step_seg& seg, int world, bool average, const tdm_adamw_scalars& s, int order, hipStream_t stream);
 
 }  // namespace tandem_hip

@@ -20,7 +20,6 @@
 #include <mutex>
 #include <string>
 #include <type_traits>
-#include <vector>
 
 #include "../../include/tandem_hip.h"
 #include "common.h"
@@ -49,17 +48,27 @@ int elem_size(int dtype) {
 
 bool is_floating(int dtype) { return dtype == TDM_F32 || dtype == TDM_F64 || dtype == TDM_F16 || dtype == TDM_BF16; }
 
+// Compute units of the current device: asked of the runtime once per device, and looked up once per
+// entry-point call (a collective of several launches asks hipGetDevice once, not per launch).
 int compute_units() {
-  static int cus[64] = {0};
+  static std::atomic<int> cus[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cus[dev] == 0) {
-    int n = 0;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cus[dev] = n;
+    cus[dev].store(n, std::memory_order_relaxed);
   }
-  return cus[dev];
+  return n;
 }
+
+thread_local int t_call_cus = 0;  // set while a collective of several launches runs on this thread
+
+struct CallScope {
+  bool outer;
+  CallScope() : outer(t_call_cus == 0) { if (outer) t_call_cus = compute_units(); }
+  ~CallScope() { if (outer) t_call_cus = 0; }
+};
 
 // tile_of()'s shift per kernel family (TDM_XCD_*), settable through tdm_set_xcd_group.
 constexpr int kXcdKinds = TDM_XCD_STEP + 1;
@@ -109,7 +118,7 @@ unsigned occupancy_pad(int kind, bool cold = true) {
 }
 
 int grid_for(int64_t tiles) {
-  const int64_t cap = static_cast<int64_t>(compute_units()) * g_blocks_per_cu;
+  const int64_t cap = static_cast<int64_t>(t_call_cus ? t_call_cus : compute_units()) * g_blocks_per_cu;
   return static_cast<int>(std::max<int64_t>(1, std::min(tiles, cap)));
 }
 
@@ -403,21 +412,21 @@ void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStrea
   if (world > 1 && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
   PairTable tab;
   // dst == src is allowed when scaling in place (div_ of a chunk); partial overlap never is
-  std::vector<tdm_pair> kept;
-  for (int i = 0; i < npairs && pairs != nullptr; ++i) {
-    if (pairs[i].dst == pairs[i].src && pairs[i].count > 0 && world <= 1) continue;  // copying onto itself
-    kept.push_back(pairs[i]);
-  }
   if (npairs > 0 && pairs == nullptr) throw Invalid("pairs is NULL");
   if (npairs < 0 || npairs > TDM_MAX_PAIRS) throw Invalid("npairs must be in [0, " + std::to_string(TDM_MAX_PAIRS) + "]");
-  for (const tdm_pair& p : kept) {
+  tdm_pair kept[TDM_MAX_PAIRS];
+  int nkept = 0;
+  for (int i = 0; i < npairs; ++i) {
+    const tdm_pair& p = pairs[i];
+    if (p.dst == p.src && p.count > 0 && world <= 1) continue;  // copying onto itself
     if (p.count > 0 && p.dst != p.src && p.dst != nullptr && p.src != nullptr) {
       const uintptr_t d = reinterpret_cast<uintptr_t>(p.dst), s = reinterpret_cast<uintptr_t>(p.src);
       const uintptr_t bytes = static_cast<uintptr_t>(p.count) * es;
       if (d < s + bytes && s < d + bytes) throw Invalid("copy: destination and source overlap");
     }
+    kept[nkept++] = p;
   }
-  const int64_t tiles = build_pairs(kept.data(), static_cast<int>(kept.size()), es, false, kCopyTileVecs, &tab);
+  const int64_t tiles = build_pairs(kept, nkept, es, false, kCopyTileVecs, &tab);
   tab.flags = xcd_shift(TDM_XCD_COPY, world, false) << 8;
   if (tiles == 0) return;
   switch (dtype) {
@@ -436,9 +445,10 @@ void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStrea
 namespace {
 
 struct LocalRanks {
-  std::vector<char*> base;
-  std::vector<int64_t> lo, len;  // chunk bounds, in elements
+  char* base[TDM_MAX_PAIRS];
+  int64_t lo[TDM_MAX_PAIRS], len[TDM_MAX_PAIRS];  // chunk bounds, in elements
   int world, es, dtype;
+  int64_t footprint;  // bytes of all ranks' tensors together
 };
 
 LocalRanks local_ranks(void* const* bufs, int world, int64_t numel, int dtype, const int64_t* sizes, int nsizes) {
@@ -450,9 +460,10 @@ LocalRanks local_ranks(void* const* bufs, int world, int64_t numel, int dtype, c
   if (bufs == nullptr) throw Invalid("NULL rank buffers");
   lr.world = world;
   lr.dtype = dtype;
+  lr.footprint = numel * lr.es * world;
   for (int r = 0; r < world; ++r) {
     if (numel > 0 && bufs[r] == nullptr) throw Invalid("rank " + std::to_string(r) + ": NULL buffer");
-    lr.base.push_back(static_cast<char*>(bufs[r]));
+    lr.base[r] = static_cast<char*>(bufs[r]);
   }
   for (int a = 0; a < world && numel > 0; ++a)
     for (int b = a + 1; b < world; ++b) {
@@ -460,8 +471,6 @@ LocalRanks local_ranks(void* const* bufs, int world, int64_t numel, int dtype, c
       const uintptr_t bytes = static_cast<uintptr_t>(numel) * lr.es;
       if (x < y + bytes && y < x + bytes) throw Invalid("rank buffers overlap");
     }
-  lr.lo.resize(world);
-  lr.len.resize(world);
   if (nsizes == 0) {  // as torch.tensor_split cuts
     const int64_t base = numel / world, extra = numel % world;
     int64_t at = 0;
@@ -501,7 +510,9 @@ int wrap(int a, int n) { return ((a % n) + n) % n; }
 // fits with room to spare does best with everything cached.
 int ring_policy(int world, int step, bool gather, int64_t footprint_bytes) {
   // Measurement knob: TDM_RING_POLICY="r0,r1,...,g0,g1,..." (one digit per step; reduce steps, then gather steps).
-  if (const char* env = std::getenv("TDM_RING_POLICY")) {
+  static const std::string knob = [] { const char* e = std::getenv("TDM_RING_POLICY"); return std::string(e ? e : ""); }();  // read once
+  if (!knob.empty()) {
+    const char* env = knob.c_str();
     const size_t at = static_cast<size_t>(2 * ((gather ? world - 1 : 0) + step));
 #ifdef TDM_ALL_POLICIES
     if (std::strlen(env) > at && env[at] >= '0' && env[at] <= '7') return env[at] - '0';
@@ -525,14 +536,35 @@ int ring_policy(int world, int step, bool gather, int64_t footprint_bytes) {
   }
 }
 
-int64_t footprint(const LocalRanks& lr) {  // bytes of all ranks' tensors together
-  int64_t elems = 0;
-  for (int64_t l : lr.len) elems += l;
-  return elems * lr.es * lr.world;
+int64_t footprint(const LocalRanks& lr) { return lr.footprint; }
+
+// Which form a ring collective of buffer ranks takes: its W-1 steps, one launch each, or the
+// whole reduce-scatter (all-gather) as ONE launch. -1: by footprint. The one-launch forms read
+// every rank's copy of a chunk once and write the W-1 partial sums (the W-1 copies), 4 (2W-1)
+// (4 W) bytes per element where the steps move 12 (W-1) (8 (W-1)); they are what a footprint
+// inside the caches wants, where the gaps between launches cost more than the bytes. Measured on
+// MI355X, reduce-scatter + all-gather, steps against one launch each: world 4 at 4 MiB per rank 26.9
+// against 12.3 us, 16 MiB 41.9 / 31.5, 64 MiB 145 / 115, 80 MiB 184 / 169, 96 MiB equal, 128 MiB 293 /
+// 303, 256 MiB 566 / 585; world 3 at 4 MiB 20.8 / 15.8, 64 MiB 104 / 92, 96 MiB 152 / 133, 128 MiB
+// 203 / 216. At world 2 a collective is one step anyway and the step kernels' cache policies do better
+// (64 MiB 49 / 51 us, 256 MiB 186 / 236). Beyond the caches the steps' per-step policies win and remain the form.
+std::atomic<int> g_ring_form{-1};
+constexpr int64_t kOneLaunchFootprint = int64_t(320) << 20;
+
+bool one_launch_form(const LocalRanks& lr) {
+  if (!chain_handles(lr.world)) return false;
+  const int set = g_ring_form.load(std::memory_order_relaxed);
+  return set >= 0 ? set == 1 : lr.world >= 3 && lr.footprint <= kOneLaunchFootprint;
 }
 
 void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hipStream_t stream) {
   const int n = lr.world;
+  if (one_launch_form(lr)) {
+    const int64_t cap = static_cast<int64_t>(t_call_cus ? t_call_cus : compute_units()) * g_blocks_per_cu;
+    chain_reduce_scatter(lr.base, lr.lo, lr.len, n, lr.dtype, lr.es, average, keep_sent,
+                         static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
+    return;
+  }
   for (int s = 0; s < n - 1; ++s) {
     tdm_pair pairs[TDM_MAX_PAIRS];
     int np = 0;
@@ -548,6 +580,16 @@ void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hi
 // Step s: rank r copies chunk (r-s-1) from rank r-1 (tandem/comm.py:307-311).
 void local_all_gather(const LocalRanks& lr, hipStream_t stream) {
   const int n = lr.world;
+  if (one_launch_form(lr) && n * (n - 1) <= TDM_MAX_PAIRS) {
+    // every rank copies every chunk straight from its owner: the ring's W-1 forwarding steps leave the same bytes
+    tdm_pair pairs[TDM_MAX_PAIRS];
+    int np = 0;
+    for (int c = 0; c < n; ++c)
+      for (int r = 0; r < n; ++r)
+        if (r != c && lr.len[c] > 0) pairs[np++] = tdm_pair{lr.base[r] + lr.lo[c] * lr.es, lr.base[c] + lr.lo[c] * lr.es, lr.len[c]};
+    if (np) copy_step(pairs, np, lr.dtype, 0, stream, 0);
+    return;
+  }
   for (int s = 0; s < n - 1; ++s) {
     tdm_pair pairs[TDM_MAX_PAIRS];
     int np = 0;
@@ -636,6 +678,7 @@ extern "C" {
 int tdm_local_reduce_scatter(void* const* bufs, int world, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
                              int average, int keep_sent, tdm_stream stream) {
   return guard([&] {
+    CallScope scope;
     if (average && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
     const LocalRanks lr = local_ranks(bufs, world, numel, dtype, sizes, nsizes);
     if (world > 1) local_reduce_scatter(lr, average != 0, keep_sent != 0, static_cast<hipStream_t>(stream));
@@ -645,6 +688,7 @@ int tdm_local_reduce_scatter(void* const* bufs, int world, int64_t numel, int dt
 int tdm_local_all_gather(void* const* bufs, int world, int64_t numel, int dtype, const int64_t* sizes, int nsizes,
                          tdm_stream stream) {
   return guard([&] {
+    CallScope scope;
     const LocalRanks lr = local_ranks(bufs, world, numel, dtype, sizes, nsizes);
     if (world > 1) local_all_gather(lr, static_cast<hipStream_t>(stream));
   });
@@ -653,6 +697,7 @@ int tdm_local_all_gather(void* const* bufs, int world, int64_t numel, int dtype,
 int tdm_local_all_reduce(void* const* bufs, int world, int64_t numel, int dtype, int average, int algorithm,
                          tdm_stream stream) {
   return guard([&] {
+    CallScope scope;
     if (average && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
     if (algorithm != TDM_ALLREDUCE_RING && algorithm != TDM_ALLREDUCE_FOLD) throw Invalid("unknown all-reduce algorithm");
     const LocalRanks lr = local_ranks(bufs, world, numel, dtype, nullptr, 0);
@@ -683,6 +728,13 @@ int tdm_set_blocks_per_cu(int blocks) {
   return guard([&] {
     if (blocks < 0 || blocks > 1024) throw Invalid("blocks per compute unit must be in [0, 1024]");
     g_blocks_per_cu = blocks == 0 ? kDefaultBlocksPerCu : blocks;
+  });
+}
+
+int tdm_set_ring_form(int form) {
+  return guard([&] {
+    if (form < -1 || form > 1) throw Invalid("the ring form is 0 (steps), 1 (one launch) or -1 (by footprint)");
+    g_ring_form.store(form, std::memory_order_relaxed);
   });
 }
 

@@ -1,0 +1,199 @@
+// The ring reduce-scatter of a whole group in ONE launch, for ranks that are buffers of one
+// process and a footprint that stays in the caches.
+//
+// The ring's W-1 steps (tandem/comm.py:301-305 in the reference) pass chunk c round the ring:
+// rank c+1 sends it, rank c+2 adds its own and sends the sum on, ..., rank c adds last. Every
+// element of chunk c is therefore a chain
+//     acc = y[c+1];   acc = y[c+k] + acc   (k = 2 .. W),      y_q = x_q / W when averaging,
+// and after the last step rank c+k's copy of chunk c holds the chain's value after k terms
+// (observable: tandem/comm.py:350-352). One workgroup can run the whole chain for its tile: it
+// reads the W ranks' copies once, and stores the partial sum after k terms into rank c+k's copy,
+// which leaves memory bit for bit as the W-1 launches of the step kernel do, with W reads and
+// W-1 (keep_sent: W) writes of 4 bytes per element instead of 3 (W-1) (+1) accesses.
+// The ring steps remain the form for footprints beyond the caches, where their per-step cache
+// policies win.
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstring>
+#include <string>
+
+#include "../../include/tandem_hip.h"
+#include "common.h"
+
+#include "kernels_device.h"
+
+namespace tandem_hip {
+
+namespace {
+
+// One chunk per segment: rank q's copy of the chunk at ptr[q].
+struct ChainTable {
+  int nseg;
+  int keep_sent;  // the first sender's copy is left holding y (x / W), as div_ of the whole tensor does
+  int64_t tile_end[TDM_MAX_WORLD];
+  char* ptr[TDM_MAX_WORLD][TDM_MAX_WORLD];  // [segment][rank]
+  int64_t count[TDM_MAX_WORLD];
+  int32_t chunk[TDM_MAX_WORLD];
+  int32_t vec_ok[TDM_MAX_WORLD];  // every rank's copy starts on a 16-byte boundary
+};
+
+template <typename T, int kWorld, int kDiv>
+__device__ __forceinline__ void chain_elem(const T (&in)[kWorld], T (&out)[kWorld], const Divisor<T>& dv) {
+  // in[k]: rank (c+1+k) % W's element; out[k]: what that rank holds afterwards
+  using A = typename Elem<T>::acc;
+  A acc = scaled<T, kDiv>(Elem<T>::widen(in[0]), dv.divisor, dv.reciprocal);
+  out[0] = Elem<T>::narrow(acc);
+#pragma unroll
+  for (int k = 1; k < kWorld; ++k) {
+    const A y = scaled<T, kDiv>(Elem<T>::widen(in[k]), dv.divisor, dv.reciprocal);
+    acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+    out[k] = Elem<T>::narrow(acc);
+  }
+}
+
+template <typename T, int kWorld, int kDiv>
+__global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divisor<T> dv) {
+  constexpr int L = lanes<T>();
+  constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
+  const int64_t total = tab.tile_end[tab.nseg - 1];
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    int sg = 0;
+    while (tile >= tab.tile_end[sg]) ++sg;
+    const int64_t t = tile - (sg ? tab.tile_end[sg - 1] : 0);
+    const int c = tab.chunk[sg];
+    const int64_t n = tab.count[sg];
+    char* p[kWorld];  // in ring order: p[k] is rank (c+1+k) % W's copy
+#pragma unroll
+    for (int k = 0; k < kWorld; ++k) p[k] = tab.ptr[sg][(c + 1 + k) % kWorld];
+    const bool keep = tab.keep_sent != 0;
+    if (tab.vec_ok[sg]) {
+      const int64_t nv = n / L;
+      vec16 raw[kWorld][kUnroll];
+#pragma unroll
+      for (int k = 0; k < kWorld; ++k)
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          const int64_t v = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
+          if (v < nv) raw[k][u] = load_rmw<0>(p[k] + v * 16);
+        }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int64_t v = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
+        if (v < nv) {
+          Lanes<T> res[kWorld];
+#pragma unroll
+          for (int l = 0; l < L; ++l) {
+            T in[kWorld], out[kWorld];
+#pragma unroll
+            for (int k = 0; k < kWorld; ++k) in[k] = unpack<T>(raw[k][u]).v[l];
+            chain_elem<T, kWorld, kDiv>(in, out, dv);
+#pragma unroll
+            for (int k = 0; k < kWorld; ++k) res[k].v[l] = out[k];
+          }
+          if (keep) store16<0>(p[0] + v * 16, pack<T>(res[0]));
+#pragma unroll
+          for (int k = 1; k < kWorld; ++k) store16<0>(p[k] + v * 16, pack<T>(res[k]));
+        }
+      }
+      if (t == 0 && threadIdx.x < n - nv * L) {  // the chunk's last few elements
+        const int64_t i = nv * L + threadIdx.x;
+        T in[kWorld], out[kWorld];
+#pragma unroll
+        for (int k = 0; k < kWorld; ++k) in[k] = reinterpret_cast<const T*>(p[k])[i];
+        chain_elem<T, kWorld, kDiv>(in, out, dv);
+        if (keep) reinterpret_cast<T*>(p[0])[i] = out[0];
+#pragma unroll
+        for (int k = 1; k < kWorld; ++k) reinterpret_cast<T*>(p[k])[i] = out[k];
+      }
+    } else {  // a copy off the 16-byte grid: element by element, still coalesced
+      const int64_t e0 = t * kTileElems + threadIdx.x;
+      for (int r = 0; r < kUnroll * L; ++r) {
+        const int64_t i = e0 + static_cast<int64_t>(r) * kThreads;
+        if (i < n) {
+          T in[kWorld], out[kWorld];
+#pragma unroll
+          for (int k = 0; k < kWorld; ++k) in[k] = reinterpret_cast<const T*>(p[k])[i];
+          chain_elem<T, kWorld, kDiv>(in, out, dv);
+          if (keep) reinterpret_cast<T*>(p[0])[i] = out[0];
+#pragma unroll
+          for (int k = 1; k < kWorld; ++k) reinterpret_cast<T*>(p[k])[i] = out[k];
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int kWorld>
+void launch_chain_w(const ChainTable& tab, bool average, int grid, hipStream_t stream) {
+  Divisor<T> dv;
+  using A = typename Elem<T>::acc;
+  dv.divisor = static_cast<A>(kWorld);
+  if constexpr (Elem<T>::floating) dv.reciprocal = static_cast<A>(1) / dv.divisor; else dv.reciprocal = 1;
+  const dim3 g(grid), b(kThreads);
+  if constexpr (Elem<T>::floating) {
+    if (average && (kWorld & (kWorld - 1)) == 0) {
+      hipLaunchKernelGGL((k1_chain_kernel<T, kWorld, 1>), g, b, 0, stream, tab, dv);
+      return;
+    }
+    if (average) {
+      hipLaunchKernelGGL((k1_chain_kernel<T, kWorld, 2>), g, b, 0, stream, tab, dv);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((k1_chain_kernel<T, kWorld, 0>), g, b, 0, stream, tab, dv);
+}
+
+template <typename T>
+void launch_chain(const ChainTable& tab, int world, bool average, int grid, hipStream_t stream) {
+  switch (world) {
+    case 2: launch_chain_w<T, 2>(tab, average, grid, stream); break;
+    case 3: launch_chain_w<T, 3>(tab, average, grid, stream); break;
+    default: launch_chain_w<T, 4>(tab, average, grid, stream); break;
+  }
+}
+
+}  // namespace
+
+bool chain_handles(int world) { return world >= 2 && world <= kChainMaxWorld; }
+
+void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
+                          bool keep_sent, int max_grid, hipStream_t stream) {
+  if (!chain_handles(world)) throw Invalid("the one-launch reduce-scatter handles world sizes 2..4");
+  ChainTable tab;
+  std::memset(&tab, 0, sizeof tab);
+  tab.keep_sent = keep_sent && average ? 1 : 0;  // without a division the first sender's copy is x already
+  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
+  int64_t tiles = 0;
+  int k = 0;
+  for (int c = 0; c < world; ++c) {
+    if (len[c] == 0) continue;  // an empty chunk travels nowhere (tandem/comm.py:292-294)
+    bool vec = true;
+    for (int q = 0; q < world; ++q) {
+      tab.ptr[k][q] = base[q] + lo[c] * es;
+      vec = vec && reinterpret_cast<uintptr_t>(tab.ptr[k][q]) % 16 == 0;
+    }
+    tab.count[k] = len[c];
+    tab.chunk[k] = c;
+    tab.vec_ok[k] = vec;
+    tiles += (len[c] + tile_elems - 1) / tile_elems;
+    tab.tile_end[k] = tiles;
+    ++k;
+  }
+  tab.nseg = k;
+  if (k == 0) return;
+  const int grid = static_cast<int>(tiles < max_grid ? tiles : max_grid);
+  switch (dtype) {
+    case TDM_F32: launch_chain<float>(tab, world, average, grid, stream); break;
+    case TDM_F64: launch_chain<double>(tab, world, average, grid, stream); break;
+    case TDM_F16: launch_chain<f16_t>(tab, world, average, grid, stream); break;
+    case TDM_BF16: launch_chain<bf16_t>(tab, world, average, grid, stream); break;
+    case TDM_I64: launch_chain<int64_t>(tab, world, false, grid, stream); break;
+    case TDM_I32: launch_chain<int32_t>(tab, world, false, grid, stream); break;
+    default: throw Invalid("unknown dtype " + std::to_string(dtype));
+  }
+  check_hip(hipGetLastError(), "k1_chain launch");
+}
+
+}  // namespace tandem_hip

@@ -26,6 +26,17 @@ def from_np(a, dtype, dev):
     return torch.from_numpy(np.array(a, copy=True)).to(dev)
 
 
+@pytest.fixture(params=["steps", "one_launch"], autouse=True)
+def ring_form(request):
+    """Every test here runs with the ring collectives as W-1 launches and as one launch
+    (world sizes 2..4 have the second form; the others take the steps either way)."""
+    from tandem_amd._lib import lib
+
+    assert lib().tdm_set_ring_form(0 if request.param == "steps" else 1) == 0
+    yield request.param
+    assert lib().tdm_set_ring_form(-1) == 0
+
+
 @pytest.fixture(scope="module")
 def dev():
     assert torch.cuda.is_available(), "these tests need the MI355X"
