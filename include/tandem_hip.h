@@ -169,6 +169,9 @@ int tdm_local_all_reduce(void* const* bufs, int world, int64_t numel, int dtype,
  * bucket's flat buffer, held by every rank at src[r]; the averaged value is
  * written to every non-NULL dst[r] (the rank's gradient itself, or its view in
  * the bucket). */
+/* Entries of ranks beyond the world size must be NULL. When every pointer of a segment lies at the same
+ * distance from a 16-byte boundary, the kernels peel the few elements before the boundary and run the
+ * rest on 16-byte vectors; pointers that disagree within 16 bytes cost the element-wise path. */
 typedef struct tdm_fold_seg {
   const void* src[TDM_MAX_WORLD];
   void* dst[TDM_MAX_WORLD];
@@ -261,6 +264,7 @@ int tdm_k3_adamw_gather(float* p, const float* g, float* m, float* v, int64_t n,
 /* One segment: `count` elements that lie in ring chunk `chunk` (= the rank that owns
  * them) of a ZeRO bucket. grad[r]: rank r's gradient (its staging buffer); param[r]: rank
  * r's copy of the parameters; exp_avg, exp_avg_sq: the owner's optimizer state. fp32. */
+/* Entries of ranks beyond the world size must be NULL; alignment as for tdm_fold_seg. */
 typedef struct tdm_step_seg {
   const void* grad[TDM_MAX_WORLD];
   void* param[TDM_MAX_WORLD];

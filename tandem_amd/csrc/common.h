@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
 #include <stdexcept>
 #include <string>
 
@@ -43,6 +44,31 @@ int guard(F&& body) {
     set_last_error("unknown error");
     return TDM_ERUNTIME;
   }
+}
+
+// How a segment of `count` elements whose streams start at ptrs[0..n) is walked. When every stream starts at
+// the same distance from a 16-byte boundary, the first `head` elements (fewer than a vector) are peeled off,
+// the remaining `body` elements start aligned and take the dwordx4 path (vec), in `tiles` tiles of tile_elems.
+// Otherwise (or when the segment is shorter than its head) everything goes element by element: head 0, body = count.
+struct SegPlan {
+  bool vec;
+  int head;
+  int64_t body, tiles;
+};
+
+inline SegPlan plan_segment(const uintptr_t* ptrs, int n, int64_t count, int es, int64_t tile_elems) {
+  SegPlan p{false, 0, count, count > 0 ? (count + tile_elems - 1) / tile_elems : 0};
+  if (count <= 0 || n <= 0) return p;
+  const uintptr_t phase = ptrs[0] % 16;
+  for (int i = 1; i < n; ++i)
+    if (ptrs[i] % 16 != phase) return p;
+  const int64_t head = static_cast<int64_t>((16 - phase) % 16) / es;
+  if (head >= count) return p;
+  p.vec = true;
+  p.head = static_cast<int>(head);
+  p.body = count - head;
+  p.tiles = (p.body + tile_elems - 1) / tile_elems;
+  return p;
 }
 
 // kernels.hip

@@ -46,6 +46,30 @@ int elem_size(int dtype) {
   }
 }
 
+// How the fold and step kernels walk a segment (plan_segment), over the pointers that exist: entries of
+// ranks beyond the world size are NULL by contract, so the plan does not need the world size.
+SegPlan plan_fold(const tdm_fold_seg& s, int es) {
+  uintptr_t ptrs[2 * TDM_MAX_WORLD];
+  int n = 0;
+  for (int r = 0; r < TDM_MAX_WORLD; ++r) {
+    if (s.src[r]) ptrs[n++] = reinterpret_cast<uintptr_t>(s.src[r]);
+    if (s.dst[r]) ptrs[n++] = reinterpret_cast<uintptr_t>(s.dst[r]);
+  }
+  return plan_segment(ptrs, n, s.count, es, static_cast<int64_t>(kTileVecs) * (16 / es));
+}
+
+SegPlan plan_step(const tdm_step_seg& s) {
+  uintptr_t ptrs[2 * TDM_MAX_WORLD + 2];
+  int n = 0;
+  for (int r = 0; r < TDM_MAX_WORLD; ++r) {
+    if (s.grad[r]) ptrs[n++] = reinterpret_cast<uintptr_t>(s.grad[r]);
+    if (s.param[r]) ptrs[n++] = reinterpret_cast<uintptr_t>(s.param[r]);
+  }
+  if (s.exp_avg) ptrs[n++] = reinterpret_cast<uintptr_t>(s.exp_avg);
+  if (s.exp_avg_sq) ptrs[n++] = reinterpret_cast<uintptr_t>(s.exp_avg_sq);
+  return plan_segment(ptrs, n, s.count, 4, static_cast<int64_t>(kTileVecs) * 4);
+}
+
 bool is_floating(int dtype) { return dtype == TDM_F32 || dtype == TDM_F64 || dtype == TDM_F16 || dtype == TDM_BF16; }
 
 // Compute units of the current device: asked of the runtime once per device, and looked up once per
@@ -336,9 +360,8 @@ void launch_step_one_w(const StepSegDev& whole, int64_t tiles, int average, cons
 }
 
 int64_t step_tiles(const tdm_step_seg* segs, int nseg) {
-  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * 4;
   int64_t tiles = 0;
-  for (int i = 0; i < nseg; ++i) tiles += segs[i].count > 0 ? (segs[i].count + tile_elems - 1) / tile_elems : 0;
+  for (int i = 0; i < nseg; ++i) tiles += plan_step(segs[i]).tiles;
   return tiles;
 }
 
@@ -354,22 +377,26 @@ void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const t
   if (!sg.exp_avg || !sg.exp_avg_sq) throw Invalid("NULL optimizer state");
   StepSegDev whole;
   std::memset(&whole, 0, sizeof whole);
-  bool vec = reinterpret_cast<uintptr_t>(sg.exp_avg) % 16 == 0 && reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % 16 == 0;
   if (reinterpret_cast<uintptr_t>(sg.exp_avg) % 4 || reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % 4) throw Invalid("pointer not aligned to 4 bytes");
   for (int r = 0; r < world; ++r) {
     if (!sg.grad[r] || !sg.param[r]) throw Invalid("NULL gradient or parameter");
     const uintptr_t a = reinterpret_cast<uintptr_t>(sg.grad[r]), b = reinterpret_cast<uintptr_t>(sg.param[r]);
     if (a % 4 || b % 4) throw Invalid("pointer not aligned to 4 bytes");
-    vec = vec && a % 16 == 0 && b % 16 == 0;
-    whole.g[r] = static_cast<const char*>(sg.grad[r]);
-    whole.p[r] = static_cast<char*>(sg.param[r]);
   }
-  whole.m = static_cast<char*>(sg.exp_avg);
-  whole.v = static_cast<char*>(sg.exp_avg_sq);
-  whole.count = sg.count;
+  for (int r = world; r < TDM_MAX_WORLD; ++r)
+    if (sg.grad[r] || sg.param[r]) throw Invalid("pointers of ranks beyond the world size must be NULL");
+  const SegPlan plan = plan_step(sg);
+  const int64_t skip = static_cast<int64_t>(plan.head) * 4;  // the kernel reaches back for the head
+  for (int r = 0; r < world; ++r) {
+    whole.g[r] = static_cast<const char*>(sg.grad[r]) + skip;
+    whole.p[r] = static_cast<char*>(sg.param[r]) + skip;
+  }
+  whole.m = static_cast<char*>(sg.exp_avg) + skip;
+  whole.v = static_cast<char*>(sg.exp_avg_sq) + skip;
+  whole.count = plan.body;
   whole.chunk = sg.chunk;
-  whole.vec_ok = vec;
-  const int64_t tiles = step_tiles(&sg, 1);
+  whole.vec_ok = plan.vec ? 1 + plan.head : 0;
+  const int64_t tiles = plan.tiles;
   switch (world) {
     case 1: launch_step_one_w<1>(whole, tiles, average, s, order, stream); break;
     case 2: launch_step_one_w<2>(whole, tiles, average, s, order, stream); break;
@@ -632,7 +659,6 @@ void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool av
   if (average && !is_floating(dtype)) throw Invalid("integer tensors cannot be averaged in place");
   FoldSmall tab;
   std::memset(&tab, 0, sizeof tab);
-  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
   int64_t tiles = 0;
   int k = 0;
   for (int i = 0; i < nseg; ++i) {
@@ -640,19 +666,23 @@ void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool av
     if (s.count < 0) throw Invalid("fold: negative count");
     if (s.count == 0) continue;
     if (s.chunk < 0 || s.chunk >= world) throw Invalid("fold: chunk outside [0, world)");
-    bool vec = true;
     for (int r = 0; r < world; ++r) {
       if (s.src[r] == nullptr) throw Invalid("fold: NULL source");
       const uintptr_t a = reinterpret_cast<uintptr_t>(s.src[r]), b = reinterpret_cast<uintptr_t>(s.dst[r]);
       if (a % es || b % es) throw Invalid("fold: pointer not aligned to the element size");
-      vec = vec && a % 16 == 0 && b % 16 == 0;
-      tab.seg[k].src[r] = static_cast<const char*>(s.src[r]);
-      tab.seg[k].dst[r] = static_cast<char*>(s.dst[r]);
     }
-    tab.seg[k].count = s.count;
+    for (int r = world; r < TDM_MAX_WORLD; ++r)
+      if (s.src[r] || s.dst[r]) throw Invalid("fold: pointers of ranks beyond the world size must be NULL");
+    const SegPlan plan = plan_fold(s, es);
+    const int64_t skip = static_cast<int64_t>(plan.head) * es;  // the kernel reaches back for the head
+    for (int r = 0; r < world; ++r) {
+      tab.seg[k].src[r] = static_cast<const char*>(s.src[r]) + skip;
+      tab.seg[k].dst[r] = s.dst[r] ? static_cast<char*>(s.dst[r]) + skip : nullptr;
+    }
+    tab.seg[k].count = plan.body;
     tab.seg[k].chunk = s.chunk;
-    tab.seg[k].vec_ok = vec;
-    tiles += (s.count + tile_elems - 1) / tile_elems;
+    tab.seg[k].vec_ok = plan.vec ? 1 + plan.head : 0;
+    tiles += plan.tiles;
     tab.tile_end[k] = tiles;
     ++k;
   }
@@ -775,9 +805,8 @@ int tdm_k1_copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, td
 
 namespace {
 int64_t fold_tiles(const tdm_fold_seg* segs, int nseg, int es) {
-  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
   int64_t tiles = 0;
-  for (int i = 0; i < nseg; ++i) tiles += segs[i].count > 0 ? (segs[i].count + tile_elems - 1) / tile_elems : 0;
+  for (int i = 0; i < nseg; ++i) tiles += plan_fold(segs[i], es).tiles;
   return tiles;
 }
 }  // namespace
@@ -795,18 +824,20 @@ int64_t tdm_k2_table_bytes(const tdm_fold_seg* segs, int nseg, int dtype) {
 }
 
 namespace {
-// Checks segment i of a K2 table; returns whether it may take the 16-byte path.
-bool fold_seg_check(const tdm_fold_seg& s, int i, int world, int es) {
+// Checks segment i of a K2 table and says how it is walked.
+SegPlan fold_seg_check(const tdm_fold_seg& s, int i, int world, int es) {
   if (s.count < 0) throw Invalid("segment " + std::to_string(i) + ": negative count");
   if (s.chunk < 0 || s.chunk >= world) throw Invalid("segment " + std::to_string(i) + ": chunk outside [0, world)");
-  bool vec = true;
-  for (int r = 0; r < world; ++r) {
+  for (int r = 0; r < TDM_MAX_WORLD; ++r) {
+    if (r >= world) {
+      if (s.src[r] || s.dst[r]) throw Invalid("segment " + std::to_string(i) + ": pointers of ranks beyond the world size must be NULL");
+      continue;
+    }
     if (s.count > 0 && s.src[r] == nullptr) throw Invalid("segment " + std::to_string(i) + ": NULL source");
     const uintptr_t a = reinterpret_cast<uintptr_t>(s.src[r]), b = reinterpret_cast<uintptr_t>(s.dst[r]);
     if (a % es || b % es) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to the element size");
-    vec = vec && a % 16 == 0 && b % 16 == 0;
   }
-  return vec;
+  return plan_fold(s, es);
 }
 }  // namespace
 
@@ -822,16 +853,18 @@ int tdm_k2_table_build(const tdm_fold_seg* segs, int nseg, int world, int dtype,
     int64_t tiles = 0;
     for (int i = 0; i < nseg; ++i) {
       const tdm_fold_seg& s = segs[i];
-      const bool vec = fold_seg_check(s, i, world, es);
-      for (int64_t at = 0; at < s.count; at += tile_elems) {  // a tile's byte offset is a multiple of 4 KiB
+      const SegPlan plan = fold_seg_check(s, i, world, es);
+      // records describe the body (the segment without its peeled head): a record's byte offset within it is a
+      // multiple of 4 KiB; the first record also carries the head
+      for (int64_t at = 0; at < plan.body && s.count > 0; at += tile_elems) {
         FoldSegDev& rec = out[tiles++];
         for (int r = 0; r < world; ++r) {
-          rec.src[r] = static_cast<const char*>(s.src[r]) + at * es;
-          rec.dst[r] = s.dst[r] ? static_cast<char*>(s.dst[r]) + at * es : nullptr;
+          rec.src[r] = static_cast<const char*>(s.src[r]) + (plan.head + at) * es;
+          rec.dst[r] = s.dst[r] ? static_cast<char*>(s.dst[r]) + (plan.head + at) * es : nullptr;
         }
-        rec.count = std::min<int64_t>(tile_elems, s.count - at);
+        rec.count = std::min<int64_t>(tile_elems, plan.body - at);
         rec.chunk = s.chunk;
-        rec.vec_ok = vec;
+        rec.vec_ok = plan.vec ? (at == 0 ? 1 + plan.head : 1) : 0;
       }
     }
   });
@@ -898,8 +931,7 @@ int tdm_k2_bucket_fold_static(const tdm_fold_seg* segs, int nseg, int world, int
     // every segment is checked, and the size known, before the first launch
     int64_t tiles = 0;
     for (int i = 0; i < nseg; ++i) {
-      fold_seg_check(segs[i], i, world, es);
-      tiles += (segs[i].count + tile_elems - 1) / tile_elems;
+      tiles += fold_seg_check(segs[i], i, world, es).tiles;
       if (tiles > kStaticTiles) {
         throw Invalid("the segments need more than " + std::to_string(kStaticTiles) + " table records (" +
                       std::to_string(kStaticTiles * static_cast<int64_t>(kTileVecs) * 16) +
@@ -927,11 +959,17 @@ int tdm_k2_bucket_fold_static(const tdm_fold_seg* segs, int nseg, int world, int
       const tdm_fold_seg& s = segs[i];
       if (s.count == 0) continue;
       const int k = batch.nseg;
+      const SegPlan plan = plan_fold(s, es);
       batch.first[k] = at;
-      at += (s.count + tile_elems - 1) / tile_elems;
+      at += plan.tiles;
       batch.first[k + 1] = at;
-      batch.vec_ok[k] = fold_seg_check(s, i, world, es);
-      batch.seg[k] = s;
+      batch.vec_ok[k] = plan.vec ? 1 + plan.head : 0;
+      batch.seg[k] = s;  // the fill kernel sees the body: the segment without its peeled head
+      for (int r = 0; r < world; ++r) {
+        batch.seg[k].src[r] = static_cast<const char*>(s.src[r]) + static_cast<int64_t>(plan.head) * es;
+        if (s.dst[r]) batch.seg[k].dst[r] = static_cast<char*>(s.dst[r]) + static_cast<int64_t>(plan.head) * es;
+      }
+      batch.seg[k].count = plan.body;
       if (++batch.nseg == kFillSegs) flush();
     }
     flush();
@@ -1019,27 +1057,31 @@ int tdm_k23_table_build(const tdm_step_seg* segs, int nseg, int world, void* ima
       if (sg.count == 0) continue;
       if (sg.chunk < 0 || sg.chunk >= world) throw Invalid("segment " + std::to_string(i) + ": chunk outside [0, world)");
       if (!sg.exp_avg || !sg.exp_avg_sq) throw Invalid("segment " + std::to_string(i) + ": NULL optimizer state");
-      bool vec = reinterpret_cast<uintptr_t>(sg.exp_avg) % 16 == 0 && reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % 16 == 0;
       if (reinterpret_cast<uintptr_t>(sg.exp_avg) % 4 || reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % 4) {
         throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to 4 bytes");
       }
-      for (int r = 0; r < world; ++r) {
+      for (int r = 0; r < TDM_MAX_WORLD; ++r) {
+        if (r >= world) {
+          if (sg.grad[r] || sg.param[r]) throw Invalid("segment " + std::to_string(i) + ": pointers of ranks beyond the world size must be NULL");
+          continue;
+        }
         if (!sg.grad[r] || !sg.param[r]) throw Invalid("segment " + std::to_string(i) + ": NULL gradient or parameter");
         const uintptr_t a = reinterpret_cast<uintptr_t>(sg.grad[r]), b = reinterpret_cast<uintptr_t>(sg.param[r]);
         if (a % 4 || b % 4) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to 4 bytes");
-        vec = vec && a % 16 == 0 && b % 16 == 0;
       }
-      for (int64_t at = 0; at < sg.count; at += tile_elems) {
+      const SegPlan plan = plan_step(sg);
+      for (int64_t at = 0; at < plan.body; at += tile_elems) {  // records describe the body; the first one carries the head
         StepSegDev& rec = out[tiles++];
+        const int64_t off = (plan.head + at) * 4;
         for (int r = 0; r < world; ++r) {
-          rec.g[r] = static_cast<const char*>(sg.grad[r]) + at * 4;
-          rec.p[r] = static_cast<char*>(sg.param[r]) + at * 4;
+          rec.g[r] = static_cast<const char*>(sg.grad[r]) + off;
+          rec.p[r] = static_cast<char*>(sg.param[r]) + off;
         }
-        rec.m = static_cast<char*>(sg.exp_avg) + at * 4;
-        rec.v = static_cast<char*>(sg.exp_avg_sq) + at * 4;
-        rec.count = std::min<int64_t>(tile_elems, sg.count - at);
+        rec.m = static_cast<char*>(sg.exp_avg) + off;
+        rec.v = static_cast<char*>(sg.exp_avg_sq) + off;
+        rec.count = std::min<int64_t>(tile_elems, plan.body - at);
         rec.chunk = sg.chunk;
-        rec.vec_ok = vec;
+        rec.vec_ok = plan.vec ? (at == 0 ? 1 + plan.head : 1) : 0;
       }
     }
   });

@@ -36,7 +36,7 @@ struct ChainTable {
   char* ptr[TDM_MAX_WORLD][TDM_MAX_WORLD];  // [segment][rank]
   int64_t count[TDM_MAX_WORLD];
   int32_t chunk[TDM_MAX_WORLD];
-  int32_t vec_ok[TDM_MAX_WORLD];  // every rank's copy starts on a 16-byte boundary
+  int32_t vec_ok[TDM_MAX_WORLD];  // 0: element by element; 1 + h: ptr 16-byte aligned with h more elements directly before it
 };
 
 template <typename T, int kWorld, int kDiv>
@@ -97,8 +97,10 @@ __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divi
           for (int k = 1; k < kWorld; ++k) store16<0>(p[k] + v * 16, pack<T>(res[k]));
         }
       }
-      if (t == 0 && threadIdx.x < n - nv * L) {  // the chunk's last few elements
-        const int64_t i = nv * L + threadIdx.x;
+      const int head = tab.vec_ok[sg] - 1;
+      // the chunk's last few elements (lanes 0..) and the few before its first whole vector (lanes 32..)
+      if (t == 0 && (threadIdx.x < n - nv * L || (threadIdx.x >= 32 && static_cast<int>(threadIdx.x) - 32 < head))) {
+        const int64_t i = threadIdx.x < 32 ? nv * L + threadIdx.x : -1 - (static_cast<int64_t>(threadIdx.x) - 32);
         T in[kWorld], out[kWorld];
 #pragma unroll
         for (int k = 0; k < kWorld; ++k) in[k] = reinterpret_cast<const T*>(p[k])[i];
@@ -169,15 +171,14 @@ void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* l
   int k = 0;
   for (int c = 0; c < world; ++c) {
     if (len[c] == 0) continue;  // an empty chunk travels nowhere (tandem/comm.py:292-294)
-    bool vec = true;
-    for (int q = 0; q < world; ++q) {
-      tab.ptr[k][q] = base[q] + lo[c] * es;
-      vec = vec && reinterpret_cast<uintptr_t>(tab.ptr[k][q]) % 16 == 0;
-    }
-    tab.count[k] = len[c];
+    uintptr_t at[TDM_MAX_WORLD];
+    for (int q = 0; q < world; ++q) at[q] = reinterpret_cast<uintptr_t>(base[q] + lo[c] * es);
+    const SegPlan plan = plan_segment(at, world, len[c], es, tile_elems);
+    for (int q = 0; q < world; ++q) tab.ptr[k][q] = base[q] + (lo[c] + plan.head) * es;
+    tab.count[k] = plan.body;
     tab.chunk[k] = c;
-    tab.vec_ok[k] = vec;
-    tiles += (len[c] + tile_elems - 1) / tile_elems;
+    tab.vec_ok[k] = plan.vec ? 1 + plan.head : 0;
+    tiles += plan.tiles;
     tab.tile_end[k] = tiles;
     ++k;
   }

@@ -402,7 +402,10 @@ struct FoldSegDev {
   char* dst[TDM_MAX_WORLD];
   int64_t count;
   int32_t chunk;
-  int32_t vec_ok;  // every pointer of the segment is 16-byte aligned
+  // 0: the pointers disagree within 16 bytes, element by element. Otherwise 1 + h: every pointer is
+  // 16-byte aligned and h (< 16 / element size) further elements lie directly BEFORE the pointers:
+  // the head of a segment whose pointers all started at the same distance from a 16-byte boundary.
+  int32_t vec_ok;
 };
 
 // One tile of one segment: W loads per element, the fold in ring order, W stores.
@@ -479,8 +482,10 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
         }
       }
     }
-    if (t == 0 && threadIdx.x < n - nv * L) {  // tail elements
-      const int64_t i = nv * L + threadIdx.x;
+    const int head = sg.vec_ok - 1;
+    // the few elements after the last whole vector (lanes 0..) and before the first (lanes 32..)
+    if (t == 0 && (threadIdx.x < n - nv * L || (threadIdx.x >= 32 && static_cast<int>(threadIdx.x) - 32 < head))) {
+      const int64_t i = threadIdx.x < 32 ? nv * L + threadIdx.x : -1 - (static_cast<int64_t>(threadIdx.x) - 32);
       A acc = scaled<T, kDiv>(Elem<T>::widen(reinterpret_cast<const T*>(sp[0])[i]), dv.divisor, dv.reciprocal);
 #pragma unroll
       for (int k = 1; k < kWorld; ++k) {
@@ -571,7 +576,7 @@ __global__ __launch_bounds__(256) __attribute__((unused)) void k2_table_fill_ker
   }
   rec.count = min(b.tile_elems, s.count - at);
   rec.chunk = s.chunk;
-  rec.vec_ok = b.vec_ok[k];
+  rec.vec_ok = b.vec_ok[k] == 0 ? 0 : (tile == b.first[k] ? b.vec_ok[k] : 1);  // the head belongs to the first record
   out[tile] = rec;
 }
 
@@ -720,7 +725,7 @@ struct StepSegDev {
   char* v;                       // the owner's exp_avg_sq
   int64_t count;
   int32_t chunk;                 // the owner
-  int32_t vec_ok;
+  int32_t vec_ok;                // as FoldSegDev's
 };
 
 #ifndef TDM_K23_UNROLL
@@ -738,7 +743,7 @@ constexpr int kStepParts = (TDM_K23_PARTS <= kUnroll && kUnroll % TDM_K23_PARTS 
 
 // One part (at most kRounds vectors per lane and stream) of the step.
 template <int kWorld, int kDiv, int kOrder, int kRounds>
-__device__ __forceinline__ void step_tile(const StepSegDev& sg, int64_t at, int64_t n, const Divisor<float>& dv,
+__device__ __forceinline__ void step_tile(const StepSegDev& sg, int64_t at, int64_t n, int head, const Divisor<float>& dv,
                                           const tdm_adamw_scalars& s, bool small_w) {
   constexpr int kWant = kWorld <= 4 ? TDM_K23_UNROLL : 1;
   constexpr int kU = kWant < kRounds ? kWant : kRounds;  // vectors per lane in flight, per stream
@@ -798,8 +803,9 @@ __device__ __forceinline__ void step_tile(const StepSegDev& sg, int64_t at, int6
           }
         }
       }
-      if (threadIdx.x < n - nv * 4) {  // the tile's last few elements
-        const int64_t i = nv * 4 + threadIdx.x;
+      // the tile's last few elements (lanes 0..), and the segment's head before its first vector (lanes 32..)
+      if (threadIdx.x < n - nv * 4 || (threadIdx.x >= 32 && static_cast<int>(threadIdx.x) - 32 < head)) {
+        const int64_t i = threadIdx.x < 32 ? nv * 4 + threadIdx.x : -1 - (static_cast<int64_t>(threadIdx.x) - 32);
         float gs[kWorld];
 #pragma unroll
         for (int k = 0; k < kWorld; ++k) gs[k] = reinterpret_cast<const float*>(gp[k])[i];
@@ -836,7 +842,8 @@ __global__ __launch_bounds__(kThreads) void k23_zero2_step_kernel(const StepSegD
     const StepSegDev& rec = tiles[part / kStepParts];
     const int64_t first = (part % kStepParts) * kPartElems;  // the part's first element within the record
     const int64_t n = min(kPartElems, rec.count - first);
-    if (n > 0) step_tile<kWorld, kDiv, kOrder, kUnroll / kStepParts>(rec, first * 4, n, dv, s, small_w);
+    const int head = first == 0 ? rec.vec_ok - 1 : 0;
+    if (n > 0) step_tile<kWorld, kDiv, kOrder, kUnroll / kStepParts>(rec, first * 4, n, head, dv, s, small_w);
   }
 }
 
@@ -851,7 +858,8 @@ __global__ __launch_bounds__(kThreads) void k23_zero2_step_one_kernel(StepSegDev
   for (int64_t at = blockIdx.x; at < total * kStepParts; at += gridDim.x) {
     const int64_t part = tile_of(at, total * kStepParts, shift);
     const int64_t n = min(kPartElems, whole.count - part * kPartElems);
-    if (n > 0) step_tile<kWorld, kDiv, kOrder, kUnroll / kStepParts>(whole, part * kPartElems * 4, n, dv, s, small_w);
+    const int head = part == 0 ? whole.vec_ok - 1 : 0;
+    if (n > 0) step_tile<kWorld, kDiv, kOrder, kUnroll / kStepParts>(whole, part * kPartElems * 4, n, head, dv, s, small_w);
   }
 }
 

@@ -164,21 +164,57 @@ def test_unaligned_views_and_special_values(dev):
         x[100:110] = 1e-40 * (r + 1)
         xs.append(x)
     xn = [x.numpy() for x in xs]
-    for shifts in ([1, 1, 1, 1], [0, 1, 2, 3], [3, 0, 0, 1]):
+    # every rank the same distance from a 16-byte boundary (the kernels peel a head and run on vectors), and ranks
+    # that disagree (element by element)
+    for shifts in ([1, 1, 1, 1], [2, 2, 2, 2], [3, 3, 3, 3], [0, 1, 2, 3], [3, 0, 0, 1]):
         for op in ("sum", "avg"):
-            store = [torch.zeros(n + 8, device=dev) for _ in range(world)]
-            bufs = [store[r][shifts[r]:shifts[r] + n] for r in range(world)]
+            for algorithm in ("ring", "fold"):
+                store = [torch.zeros(n + 8, device=dev) for _ in range(world)]
+                bufs = [store[r][shifts[r]:shifts[r] + n] for r in range(world)]
+                for b, x in zip(bufs, xs):
+                    b.copy_(x)
+                lw.all_reduce(bufs, op=op, algorithm=algorithm)
+                want = ring.expected_all_reduce(xn, op == "avg")
+                for r in range(world):
+                    got = to_np(bufs[r])
+                    nan = np.isnan(want)
+                    assert np.array_equal(np.isnan(got), nan)
+                    assert np.array_equal(bits(got)[~nan], bits(want)[~nan]), (shifts, op, algorithm, r)
+                    # nothing outside the view was touched
+                    assert float(store[r][:shifts[r]].abs().sum()) == 0 and float(store[r][shifts[r] + n:].abs().sum()) == 0
+
+
+@pytest.mark.parametrize("world", [2, 3])
+def test_two_byte_elements_off_the_vector_grid(dev, world):
+    """bf16 views 1..7 elements past a 16-byte boundary, the same on every rank: up to seven head elements are
+    peeled before the vectors start. Reduce-scatter with its partial sums, all-gather and both all-reduces."""
+    from oracle import ring
+    from tandem_amd import LocalWorld
+
+    lw = LocalWorld(world)
+    n = 20_011
+    xs = [seeded(7, r, n).to(torch.bfloat16) for r in range(world)]
+    xn = [to_np(x) for x in xs]
+    for shift in (1, 3, 4, 7):
+        def views():
+            store = [torch.zeros(n + 16, dtype=torch.bfloat16, device=dev) for _ in range(world)]
+            bufs = [st[shift:shift + n] for st in store]
             for b, x in zip(bufs, xs):
                 b.copy_(x)
-            lw.all_reduce(bufs, op=op, algorithm="ring" if shifts[0] else "fold")
-            want = ring.expected_all_reduce(xn, op == "avg")
+            return store, bufs
+
+        for algorithm in ("ring", "fold"):
+            store, bufs = views()
+            lw.all_reduce(bufs, op="avg", algorithm=algorithm)
+            want = ring.expected_all_reduce(xn, True, "bf16")
             for r in range(world):
-                got = to_np(bufs[r])
-                nan = np.isnan(want)
-                assert np.array_equal(np.isnan(got), nan)
-                assert np.array_equal(bits(got)[~nan], bits(want)[~nan]), (shifts, op, r)
-                # nothing outside the view was touched
-                assert float(store[r][:shifts[r]].abs().sum()) == 0 and float(store[r][shifts[r] + n:].abs().sum()) == 0
+                assert np.array_equal(bits(to_np(bufs[r])), bits(want)), (shift, algorithm, r)
+                assert float(store[r][:shift].float().abs().sum()) == 0 and float(store[r][shift + n:].float().abs().sum()) == 0
+        store, bufs = views()
+        lw.reduce_scatter(bufs, None, op="avg")
+        want = ring.expected_reduce_scatter(xn, None, True, "bf16")
+        for r in range(world):
+            assert np.array_equal(bits(to_np(bufs[r])), bits(want[r])), (shift, r)
 
 
 def test_unit_gather(dev):

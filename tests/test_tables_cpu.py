@@ -20,39 +20,59 @@ TILE_BYTES = lib().tdm_table_tile_bytes()
 
 
 def fold_segs(world, es, rows):
-    """rows: (count, chunk, byte offset added to every pointer)."""
+    """rows: (count, chunk, byte offset added to every pointer[, extra bytes on the last rank's source])."""
     segs = (_lib.FoldSeg * len(rows))()
-    for k, (count, chunk, off) in enumerate(rows):
+    for k, (count, chunk, off, *skew) in enumerate(rows):
         for r in range(world):
-            segs[k].src[r] = (1 << 32) * (r + 1) + (k << 24) + off
+            segs[k].src[r] = (1 << 32) * (r + 1) + (k << 24) + off + (skew[0] if skew and r == world - 1 else 0)
             segs[k].dst[r] = (1 << 40) * (r + 1) + (k << 24) + off if r != 1 or world == 1 else 0  # rank 1 receives nothing
         segs[k].count, segs[k].chunk = count, chunk
     return segs
+
+
+def walk(count, off, es, tile, skew=0):
+    """How a segment is walked: (vectorised, head elements peeled, body elements, tiles). Pointers that all lie
+    `off` bytes past a 16-byte boundary lose (16 - off) / es head elements and run vectorised from there; a segment
+    no longer than its head, or one whose pointers disagree within 16 bytes, goes element by element."""
+    if count == 0:
+        return False, 0, 0, 0
+    head = ((16 - off % 16) % 16) // es
+    if skew % 16 or head >= count:
+        return False, 0, count, -(-count // tile)
+    return True, head, count - head, -(-(count - head) // tile)
 
 
 @pytest.mark.parametrize("dtype,es", [(F32, 4), (F64, 8), (BF16, 2)])
 @pytest.mark.parametrize("world", [1, 2, 3, 8])
 def test_fold_table_records(world, dtype, es):
     tile = TILE_BYTES // es
-    rows = [(1, 0, 0), (tile, world - 1, 0), (tile + 1, world // 2, es), (0, 0, 0), (5 * tile - 3, 0, 16), (17, world - 1, 32 + es)]
+    # aligned; off the grid by one element on every pointer (same phase: head peeled); a whole tile + 1 that ends up
+    # exactly one tile after the peel; empty; 16 bytes in; a segment shorter than its head; pointers that disagree
+    rows = [(1, 0, 0), (tile, world - 1, 0), (tile + 1, world // 2, es), (tile + 16 // es - 1, 0, es), (0, 0, 0), (5 * tile - 3, 0, 16),
+            (17, world - 1, 32 + es), (1, 0, 16 - es), (3 * tile + 5, 0, es, es if world > 1 else 0)]
     segs = fold_segs(world, es, rows)
+    plans = [walk(c, off, es, tile, *skew) for c, _, off, *skew in rows]
+    assert any(p[0] and p[1] for p in plans) and any(not p[0] and p[2] for p in plans)
     ntiles = lib().tdm_k2_table_tiles(segs, len(rows), dtype)
-    assert ntiles == sum(-(-c // tile) for c, _, _ in rows)
+    assert ntiles == sum(p[3] for p in plans)
     nbytes = lib().tdm_k2_table_bytes(segs, len(rows), dtype)
     assert nbytes == ntiles * FOLD_REC.itemsize
     image = np.full(nbytes, 0xAB, np.uint8)
     assert lib().tdm_k2_table_build(segs, len(rows), world, dtype, ctypes.c_void_p(image.ctypes.data)) == 0
     recs = image.view(FOLD_REC)
     at = 0
-    for k, (count, chunk, off) in enumerate(rows):
+    for k, ((count, chunk, off, *skew), (vec, head, body, tiles)) in enumerate(zip(rows, plans)):
         done = 0
-        while done < count:
+        while done < body:
             rec = recs[at]
-            assert rec["count"] == min(tile, count - done) and rec["chunk"] == chunk
-            assert rec["vec_ok"] == int(off % 16 == 0)
+            assert rec["count"] == min(tile, body - done) and rec["chunk"] == chunk
+            # 0: element by element; 1: vectors; 1 + h on a segment's first record: h peeled elements lie before its pointers
+            assert rec["vec_ok"] == (0 if not vec else 1 + head if done == 0 else 1), (k, done)
             for r in range(world):
-                assert rec["src"][r] == segs[k].src[r] + done * es
-                assert rec["dst"][r] == (segs[k].dst[r] + done * es if segs[k].dst[r] else 0)
+                assert rec["src"][r] == segs[k].src[r] + (head + done) * es
+                assert rec["dst"][r] == (segs[k].dst[r] + (head + done) * es if segs[k].dst[r] else 0)
+                if vec:
+                    assert rec["src"][r] % 16 == 0 and rec["dst"][r] % 16 == 0
             assert not rec["src"][world:].any() and not rec["dst"][world:].any()  # unused ranks stay zero
             done += int(rec["count"])
             at += 1
@@ -73,24 +93,26 @@ def step_segs(world, rows):
 @pytest.mark.parametrize("world", [1, 2, 4, 7])
 def test_step_table_records(world):
     tile = TILE_BYTES // 4
-    rows = [(3, 0, 0), (2 * tile, world - 1, 0), (0, 0, 0), (tile + 9, world // 2, 4), (4 * tile - 1, 0, 48)]
+    rows = [(3, 0, 0), (2 * tile, world - 1, 0), (0, 0, 0), (tile + 9, world // 2, 4), (4 * tile - 1, 0, 48), (tile + 2, 0, 8), (1, 0, 12)]
     segs = step_segs(world, rows)
+    plans = [walk(c, off, 4, tile) for c, _, off in rows]
     ntiles = lib().tdm_k23_table_tiles(segs, len(rows))
-    assert ntiles == sum(-(-c // tile) for c, _, _ in rows)
+    assert ntiles == sum(p[3] for p in plans)
     nbytes = lib().tdm_k23_table_bytes(segs, len(rows))
     assert nbytes == ntiles * STEP_REC.itemsize
     image = np.full(nbytes, 0xCD, np.uint8)
     assert lib().tdm_k23_table_build(segs, len(rows), world, ctypes.c_void_p(image.ctypes.data)) == 0
     recs = image.view(STEP_REC)
     at = 0
-    for k, (count, chunk, off) in enumerate(rows):
+    for k, ((count, chunk, off), (vec, head, body, tiles)) in enumerate(zip(rows, plans)):
         done = 0
-        while done < count:
+        while done < body:
             rec = recs[at]
-            assert rec["count"] == min(tile, count - done) and rec["chunk"] == chunk and rec["vec_ok"] == int(off % 16 == 0)
+            assert rec["count"] == min(tile, body - done) and rec["chunk"] == chunk
+            assert rec["vec_ok"] == (0 if not vec else 1 + head if done == 0 else 1), (k, done)
             for r in range(world):
-                assert rec["g"][r] == segs[k].grad[r] + done * 4 and rec["p"][r] == segs[k].param[r] + done * 4
-            assert rec["m"] == segs[k].exp_avg + done * 4 and rec["v"] == segs[k].exp_avg_sq + done * 4
+                assert rec["g"][r] == segs[k].grad[r] + (head + done) * 4 and rec["p"][r] == segs[k].param[r] + (head + done) * 4
+            assert rec["m"] == segs[k].exp_avg + (head + done) * 4 and rec["v"] == segs[k].exp_avg_sq + (head + done) * 4
             assert not rec["g"][world:].any() and not rec["p"][world:].any()
             done += int(rec["count"])
             at += 1
