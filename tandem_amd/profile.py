@@ -13,99 +13,103 @@ then still waits for shows in the Chrome trace, where compute and communication
 rows share one clock.
 """
 
-import contextlib
 import json
 import time
 
 import torch
 
 
+class _Span:
+    """One `with timeline.span(name):` block."""
+
+    def __init__(self, timeline, name):
+        self.timeline, self.name = timeline, name
+
+    def __enter__(self):
+        self.begin = self.timeline.clock() if self.timeline.enabled else None
+        return self
+
+    def __exit__(self, *exc):
+        if self.begin is not None:
+            self.timeline.spans.append((self.name, self.begin, self.timeline.clock()))
+        return False
+
+
 class Timeline:
-    """Named spans on the calling thread; with a GPU device each end of a span
-    waits for the device first (tandem/profile.py:13-35)."""
+    """Named spans on the calling thread, (name, start, end) in time.perf_counter seconds; with a
+    GPU device each end of a span waits for the device first (tandem/profile.py:13-35)."""
 
     def __init__(self, enabled=True, device=None):
         self.enabled = enabled
         self.device = None if device is None else torch.device(device)
-        self.spans = []  # (name, start, end), perf_counter seconds
+        self.spans = []
 
-    def _now(self):
+    def clock(self):
         if self.device is not None and self.device.type == "cuda":
             torch.cuda.synchronize(self.device)
         return time.perf_counter()
 
-    @contextlib.contextmanager
     def span(self, name):
-        if not self.enabled:
-            yield
-            return
-        start = self._now()
-        try:
-            yield
-        finally:
-            self.spans.append((name, start, self._now()))
-
-
-def _covered(intervals):
-    """Sorted, disjoint intervals covering the same points as `intervals`."""
-    merged = []
-    for lo, hi in sorted((float(a), float(b)) for a, b in intervals if b > a):
-        if merged and lo <= merged[-1][1]:
-            if hi > merged[-1][1]:
-                merged[-1][1] = hi
-        else:
-            merged.append([lo, hi])
-    return merged
+        return _Span(self, name)
 
 
 def overlap_seconds(a, b):
-    """Total length of the points that lie in some interval of `a` and some
-    interval of `b`."""
-    a, b = _covered(a), _covered(b)
-    total, i, j = 0.0, 0, 0
-    while i < len(a) and j < len(b):
-        lo, hi = max(a[i][0], b[j][0]), min(a[i][1], b[j][1])
-        if hi > lo:
-            total += hi - lo
-        if a[i][1] <= b[j][1]:
-            i += 1
-        else:
-            j += 1
+    """Total length of the points that lie in some interval of `a` and in some interval of
+    `b`: one sweep over all end points, counting how many intervals of each family are open."""
+    marks = []
+    for family, intervals in enumerate((a, b)):
+        for lo, hi in intervals:
+            if hi > lo:
+                marks.append((float(lo), family, +1))
+                marks.append((float(hi), family, -1))
+    marks.sort(key=lambda m: m[0])
+    open_now, total, last = [0, 0], 0.0, None
+    for at, family, step in marks:
+        if open_now[0] and open_now[1]:
+            total += at - last
+        open_now[family] += step
+        last = at
     return total
 
 
 def summarize(compute_spans, comm_spans, waits, step_time):
-    """The reference's summary (tandem/profile.py:61-76): communication time is
-    the sum of the collectives' own spans; exposed is the part of the caller's
-    waits during which a collective was actually running; overlap is the share
-    of communication that was not exposed (None without communication)."""
-    comm = sum(end - start for _, start, end, _ in comm_spans)
-    exposed = overlap_seconds([(s, e) for _, s, e in waits], [(s, e) for _, s, e, _ in comm_spans])
-    return {
-        "step_s": step_time,
-        "compute_s": sum(end - start for _, start, end in compute_spans),
-        "comm_s": comm,
-        "exposed_comm_s": exposed,
-        "overlap": (max(0.0, 1 - exposed / comm) if comm > 0 else None),
-        "comm_bytes": sum(nbytes for _, _, _, nbytes in comm_spans),
-    }
+    """The reference's summary (tandem/profile.py:61-76): communication time is the sum of the
+    collectives' own spans; exposed is the part of the caller's waits during which a collective
+    was actually running; overlap is the share of communication that was not exposed (None
+    without communication)."""
+    busy = [(start, end) for _, start, end, _ in comm_spans]
+    blocked = [(start, end) for _, start, end in waits]
+    comm = sum(end - start for start, end in busy)
+    exposed = overlap_seconds(blocked, busy)
+    out = {"step_s": step_time, "compute_s": sum(end - start for _, start, end in compute_spans)}
+    out["comm_s"], out["exposed_comm_s"] = comm, exposed
+    out["overlap"] = None if comm <= 0 else max(0.0, 1 - exposed / comm)
+    out["comm_bytes"] = sum(span[3] for span in comm_spans)
+    return out
+
+
+def _name_row(pid, tid, label):
+    what = {"ph": "M", "pid": pid, "args": {"name": label}}
+    what.update({"name": "process_name"} if tid is None else {"name": "thread_name", "tid": tid})
+    return what
+
+
+def _slice(pid, tid, origin, name, start, end, **args):
+    event = {"ph": "X", "pid": pid, "tid": tid, "name": name, "ts": (start - origin) * 1e6, "dur": (end - start) * 1e6}
+    if args:
+        event["args"] = args
+    return event
 
 
 def chrome_trace(per_rank, path):
-    """Writes a chrome://tracing / Perfetto file: one process per rank with a
-    "compute" and a "communication" row. per_rank: [(compute_spans, comm_spans)]
-    on a shared clock (tandem/profile.py:79-93)."""
-    starts = [s for comp, comm in per_rank for _, s, _ in comp] + [s for comp, comm in per_rank for _, s, _, _ in comm]
-    origin = min(starts) if starts else 0.0
+    """Writes a chrome://tracing / Perfetto file: one process per rank with a "compute" row
+    (tid 0) and a "communication" row (tid 1). per_rank: [(compute_spans, comm_spans)] on a
+    shared clock (tandem/profile.py:79-93)."""
+    origin = min((span[1] for compute, comm in per_rank for span in list(compute) + list(comm)), default=0.0)
     events = []
-    for rank, (comp, comm) in enumerate(per_rank):
-        events.append({"ph": "M", "pid": rank, "name": "process_name", "args": {"name": f"rank {rank}"}})
-        for row, label in enumerate(("compute", "communication")):
-            events.append({"ph": "M", "pid": rank, "tid": row, "name": "thread_name", "args": {"name": label}})
-        for name, s, e in comp:
-            events.append({"ph": "X", "pid": rank, "tid": 0, "name": name, "ts": (s - origin) * 1e6, "dur": (e - s) * 1e6})
-        for name, s, e, nbytes in comm:
-            events.append({"ph": "X", "pid": rank, "tid": 1, "name": name, "ts": (s - origin) * 1e6, "dur": (e - s) * 1e6,
-                           "args": {"bytes": nbytes}})
+    for rank, (compute, comm) in enumerate(per_rank):
+        events += [_name_row(rank, None, f"rank {rank}"), _name_row(rank, 0, "compute"), _name_row(rank, 1, "communication")]
+        events += [_slice(rank, 0, origin, name, start, end) for name, start, end in compute]
+        events += [_slice(rank, 1, origin, name, start, end, bytes=nbytes) for name, start, end, nbytes in comm]
     with open(path, "w") as f:
         json.dump({"traceEvents": events}, f)
