@@ -140,8 +140,8 @@ def sweep(lw, dev, steps):
     """Per-rank message sizes 64 KiB ... 256 MiB, reduce-scatter (avg) + all-gather three ways.
     ring_*: the ring's steps, one launch each (K1 and the copy step), 15 B algorithmic bytes per
     pass of a per-rank message of B bytes. one_launch_*: the reduce-scatter as one launch and the
-    all-gather as one launch, 13 B (what the library picks up to 80 MiB per rank at this world
-    size; the same bits in memory). fold_*: the all-reduce as a single launch, 8 B... 2 W B."""
+    all-gather as one launch, 11 B (what the library picks up to 80 MiB per rank at this world
+    size; beyond, the reduce-scatter goes back to steps; the same bits in memory). fold_*: the all-reduce as a single launch, 8 B... 2 W B."""
     import torch
 
     from tandem_amd._lib import check, lib
@@ -182,11 +182,12 @@ def sweep(lw, dev, steps):
                      "k1_frac_of_hbm": round(12 * n * (WORLD - 1) / (rs * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                      "fold_ms": round(fold * 1e3, 4), "fold_GBps": round(2 * WORLD * b / fold / 1e9, 1),  # every rank's b bytes read once, written once
                      "fold_algbw_GBps": round(b / fold / 1e9, 1)})
-        # one launch each: W reads + (W-1) writes per element, then W-1 copies from the owner = (4W - 3) B per pass
-        one_bytes = (4 * WORLD - 3) * b
+        # one launch each: W reads + (W-1) writes per element, then every chunk read once and written W-1 times = (3W - 1) B per pass
+        one_bytes = (3 * WORLD - 1) * b
         default_one = kib * 1024 * WORLD <= (320 << 20)
         rows[-1].update({"one_launch_ms": round(one * 1e3, 4), "one_launch_GBps": round(one_bytes / one / 1e9, 1),
                          "one_launch_frac_of_hbm": round(one_bytes / one / 1e9 / HBM_PEAK_GBPS, 4),
+                         "one_launch_ring_equivalent_GBps": round(15 * b / one / 1e9, 1),  # the ring's 15 B over this form's time
                          "default_form": "one_launch" if default_one else "steps"})
         if graph_ms is not None:
             rows[-1]["ring_hip_graph_ms"] = graph_ms

@@ -83,6 +83,11 @@ constexpr int kChainMaxWorld = 4;
 bool chain_handles(int world);
 void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
                           bool keep_sent, int max_grid, hipStream_t stream);
+// the ring all-gather of a whole group in one launch: every chunk read once from its owner and stored into the
+// other ranks' buffers; world sizes 2..8; `cold`: the footprint is beyond the caches (non-temporal accesses)
+bool gather_handles(int world);
+void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, int world, int es, bool cold, int max_grid,
+                      hipStream_t stream);
 void zero2_step_segment(const tdm_step_seg& seg, int world, bool average, const tdm_adamw_scalars& s, int order, hipStream_t stream);
 
 }  // namespace tandem_hip

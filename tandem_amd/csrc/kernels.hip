@@ -566,10 +566,11 @@ int ring_policy(int world, int step, bool gather, int64_t footprint_bytes) {
 int64_t footprint(const LocalRanks& lr) { return lr.footprint; }
 
 // Which form a ring collective of buffer ranks takes: its W-1 steps, one launch each, or the
-// whole reduce-scatter (all-gather) as ONE launch. -1: by footprint. The one-launch forms read
-// every rank's copy of a chunk once and write the W-1 partial sums (the W-1 copies), 4 (2W-1)
-// (4 W) bytes per element where the steps move 12 (W-1) (8 (W-1)); they are what a footprint
-// inside the caches wants, where the gaps between launches cost more than the bytes. Measured on
+// whole reduce-scatter (all-gather) as ONE launch. -1: by world size and footprint. The one-launch
+// forms read every rank's copy of a chunk once and write the W-1 partial sums (read the owner's
+// chunk once and write the W-1 copies), 4 (2W-1) (4 W) bytes per element where the steps move
+// 12 (W-1) (8 (W-1)). The reduce-scatter in one launch is what a footprint inside the caches
+// wants, where the gaps between launches cost more than the bytes. Measured on
 // MI355X, reduce-scatter + all-gather, steps against one launch each: world 4 at 4 MiB per rank 26.9
 // against 12.3 us, 16 MiB 41.9 / 31.5, 64 MiB 145 / 115, 80 MiB 184 / 169, 96 MiB equal, 128 MiB 293 /
 // 303, 256 MiB 566 / 585; world 3 at 4 MiB 20.8 / 15.8, 64 MiB 104 / 92, 96 MiB 152 / 133, 128 MiB
@@ -582,6 +583,15 @@ bool one_launch_form(const LocalRanks& lr) {
   if (!chain_handles(lr.world)) return false;
   const int set = g_ring_form.load(std::memory_order_relaxed);
   return set >= 0 ? set == 1 : lr.world >= 3 && lr.footprint <= kOneLaunchFootprint;
+}
+
+// The all-gather as one launch wins at every size from world 3 on (world 4, 256 MiB per rank: 236 -> 191 us;
+// 16 MiB: 22.5 -> 13.5; world 8, 256 MiB: 556 -> 383): it moves 4 W instead of 8 (W-1) bytes per element. At
+// world 2 both forms are one launch and the step kernel's policy does better (74 against 80 us at 256 MiB).
+bool gather_in_one_launch(const LocalRanks& lr) {
+  if (!gather_handles(lr.world)) return false;
+  const int set = g_ring_form.load(std::memory_order_relaxed);
+  return set >= 0 ? set == 1 : lr.world >= 3;
 }
 
 void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hipStream_t stream) {
@@ -607,14 +617,12 @@ void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hi
 // Step s: rank r copies chunk (r-s-1) from rank r-1 (tandem/comm.py:307-311).
 void local_all_gather(const LocalRanks& lr, hipStream_t stream) {
   const int n = lr.world;
-  if (one_launch_form(lr) && n * (n - 1) <= TDM_MAX_PAIRS) {
-    // every rank copies every chunk straight from its owner: the ring's W-1 forwarding steps leave the same bytes
-    tdm_pair pairs[TDM_MAX_PAIRS];
-    int np = 0;
-    for (int c = 0; c < n; ++c)
-      for (int r = 0; r < n; ++r)
-        if (r != c && lr.len[c] > 0) pairs[np++] = tdm_pair{lr.base[r] + lr.lo[c] * lr.es, lr.base[c] + lr.lo[c] * lr.es, lr.len[c]};
-    if (np) copy_step(pairs, np, lr.dtype, 0, stream, 0);
+  if (gather_in_one_launch(lr)) {
+    // every chunk is read once from its owner and stored into the other ranks' buffers: the ring's W-1
+    // forwarding steps leave the same bytes
+    const int64_t cap = static_cast<int64_t>(t_call_cus ? t_call_cus : compute_units()) * g_blocks_per_cu;
+    gather_multicast(lr.base, lr.lo, lr.len, n, lr.es, lr.footprint > kOneLaunchFootprint,
+                     static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
     return;
   }
   for (int s = 0; s < n - 1; ++s) {

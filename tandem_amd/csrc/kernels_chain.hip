@@ -156,6 +156,99 @@ void launch_chain(const ChainTable& tab, int world, bool average, int grid, hipS
   }
 }
 
+// ---------------------------------------------------------------- the all-gather in one launch
+// The ring forwards every chunk W-1 times, one neighbour at a time: W-1 launches that each read and write a
+// chunk's worth per rank, 8 (W-1) bytes per element of the tensor. With every rank's buffer in reach, a
+// workgroup reads its tile of chunk c ONCE from the owner and stores it into the W-1 other ranks' copies:
+// 4 W bytes per element, the same bytes in memory afterwards (copies have no order to preserve).
+struct GatherTable {
+  int nseg;
+  int ndst;  // destinations per segment (W - 1)
+  int64_t tile_end[TDM_MAX_WORLD];
+  const char* src[TDM_MAX_WORLD];
+  char* dst[TDM_MAX_WORLD][TDM_MAX_WORLD - 1];
+  int64_t bytes[TDM_MAX_WORLD];
+  int32_t vec_ok[TDM_MAX_WORLD];  // as the other tables': 0 byte by byte, 1 + h with h bytes before the pointers
+};
+
+template <int kMask>
+__global__ __launch_bounds__(kThreads) void k1_gather_kernel(GatherTable tab) {
+  constexpr int64_t kTileBytes = static_cast<int64_t>(kTileVecs) * 16;
+  const int64_t total = tab.tile_end[tab.nseg - 1];
+  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    int sg = 0;
+    while (tile >= tab.tile_end[sg]) ++sg;
+    const int64_t t = tile - (sg ? tab.tile_end[sg - 1] : 0);
+    const char* __restrict__ from = tab.src[sg];
+    const int64_t n = tab.bytes[sg];
+    if (tab.vec_ok[sg]) {
+      const int64_t nv = n / 16;
+      vec16 raw[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int64_t v = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
+        if (v < nv) raw[u] = load_stream<kMask>(from + v * 16);
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int64_t v = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
+        if (v < nv)
+          for (int k = 0; k < tab.ndst; ++k) store16<kMask>(tab.dst[sg][k] + v * 16, raw[u]);
+      }
+      const int head = tab.vec_ok[sg] - 1;
+      // the bytes after the last whole vector (lanes 0..15) and before the first (lanes 32..47)
+      if (t == 0 && (threadIdx.x < n - nv * 16 || (threadIdx.x >= 32 && static_cast<int>(threadIdx.x) - 32 < head))) {
+        const int64_t i = threadIdx.x < 32 ? nv * 16 + threadIdx.x : -1 - (static_cast<int64_t>(threadIdx.x) - 32);
+        const char byte = from[i];
+        for (int k = 0; k < tab.ndst; ++k) tab.dst[sg][k][i] = byte;
+      }
+    } else {  // the copies disagree within 16 bytes: byte by byte, still coalesced
+      const int64_t b0 = t * kTileBytes + threadIdx.x;
+      for (int64_t i = b0; i < n && i < (t + 1) * kTileBytes; i += kThreads) {
+        const char byte = from[i];
+        for (int k = 0; k < tab.ndst; ++k) tab.dst[sg][k][i] = byte;
+      }
+    }
+  }
+}
+
+}  // namespace
+
+bool gather_handles(int world) { return world >= 2 && world <= TDM_MAX_WORLD; }
+
+void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, int world, int es, bool cold, int max_grid,
+                      hipStream_t stream) {
+  if (!gather_handles(world)) throw Invalid("the one-launch all-gather handles world sizes 2..8");
+  GatherTable tab;
+  std::memset(&tab, 0, sizeof tab);
+  tab.ndst = world - 1;
+  const int64_t tile_bytes = static_cast<int64_t>(kTileVecs) * 16;
+  int64_t tiles = 0;
+  int k = 0;
+  for (int c = 0; c < world; ++c) {
+    if (len[c] == 0) continue;
+    uintptr_t at[TDM_MAX_WORLD];
+    for (int q = 0; q < world; ++q) at[q] = reinterpret_cast<uintptr_t>(base[q] + lo[c] * es);
+    const SegPlan plan = plan_segment(at, world, len[c] * es, 1, tile_bytes);  // in bytes: copies have no element type
+    tab.src[k] = base[c] + lo[c] * es + plan.head;
+    int d = 0;
+    for (int q = 0; q < world; ++q)
+      if (q != c) tab.dst[k][d++] = base[q] + lo[c] * es + plan.head;
+    tab.bytes[k] = plan.body;
+    tab.vec_ok[k] = plan.vec ? 1 + plan.head : 0;
+    tiles += plan.tiles;
+    tab.tile_end[k] = tiles;
+    ++k;
+  }
+  tab.nseg = k;
+  if (k == 0) return;
+  const dim3 grid(static_cast<unsigned>(tiles < max_grid ? tiles : max_grid)), block(kThreads);
+  if (cold) hipLaunchKernelGGL((k1_gather_kernel<7>), grid, block, 0, stream, tab);
+  else hipLaunchKernelGGL((k1_gather_kernel<0>), grid, block, 0, stream, tab);
+  check_hip(hipGetLastError(), "k1_gather launch");
+}
+
+namespace {
 }  // namespace
 
 bool chain_handles(int world) { return world >= 2 && world <= kChainMaxWorld; }
