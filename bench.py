@@ -140,8 +140,8 @@ def sweep(lw, dev, steps):
     """Per-rank message sizes 64 KiB ... 256 MiB, reduce-scatter (avg) + all-gather three ways.
     ring_*: the ring's steps, one launch each (K1 and the copy step), 15 B algorithmic bytes per
     pass of a per-rank message of B bytes. one_launch_*: the reduce-scatter as one launch and the
-    all-gather as one launch, 11 B (what the library picks up to 80 MiB per rank at this world
-    size; beyond, the reduce-scatter goes back to steps; the same bits in memory). fold_*: the all-reduce as a single launch, 8 B... 2 W B."""
+    all-gather as one launch, 11 B (what the library picks at this world size; the same bits in
+    memory). fold_*: the all-reduce as a single launch, 8 B... 2 W B."""
     import torch
 
     from tandem_amd._lib import check, lib
@@ -184,7 +184,7 @@ def sweep(lw, dev, steps):
                      "fold_algbw_GBps": round(b / fold / 1e9, 1)})
         # one launch each: W reads + (W-1) writes per element, then every chunk read once and written W-1 times = (3W - 1) B per pass
         one_bytes = (3 * WORLD - 1) * b
-        default_one = kib * 1024 * WORLD <= (320 << 20)
+        default_one = True  # at world 4 the library takes the one-launch forms at every size
         rows[-1].update({"one_launch_ms": round(one * 1e3, 4), "one_launch_GBps": round(one_bytes / one / 1e9, 1),
                          "one_launch_frac_of_hbm": round(one_bytes / one / 1e9 / HBM_PEAK_GBPS, 4),
                          "one_launch_ring_equivalent_GBps": round(15 * b / one / 1e9, 1),  # the ring's 15 B over this form's time

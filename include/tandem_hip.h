@@ -151,8 +151,8 @@ int tdm_local_all_gather(void* const* bufs, int world, int64_t numel, int dtype,
  * launch (world sizes 2..4: every tile runs the ring's chain of additions for its chunk and stores each
  * partial sum where the ring would have left it) and the whole all-gather as one launch (world sizes
  * 2..8: every chunk read once from its owner and stored into the other ranks' buffers); -1 (default)
- * the one-launch all-gather from world size 3 on, the one-launch reduce-scatter at world sizes 3 and 4
- * while all ranks' tensors together are at most 320 MiB, the steps otherwise. Memory ends bit for bit the
+ * the one-launch all-gather from world size 3 on, the one-launch reduce-scatter at world sizes 3 and 4,
+ * the steps otherwise. Memory ends bit for bit the
  * same either way, partial sums included. Process-wide; for measurements and tests. The reference has no
  * counterpart. */
 int tdm_set_ring_form(int form);

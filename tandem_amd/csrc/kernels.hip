@@ -566,23 +566,23 @@ int ring_policy(int world, int step, bool gather, int64_t footprint_bytes) {
 int64_t footprint(const LocalRanks& lr) { return lr.footprint; }
 
 // Which form a ring collective of buffer ranks takes: its W-1 steps, one launch each, or the
-// whole reduce-scatter (all-gather) as ONE launch. -1: by world size and footprint. The one-launch
-// forms read every rank's copy of a chunk once and write the W-1 partial sums (read the owner's
-// chunk once and write the W-1 copies), 4 (2W-1) (4 W) bytes per element where the steps move
-// 12 (W-1) (8 (W-1)). The reduce-scatter in one launch is what a footprint inside the caches
-// wants, where the gaps between launches cost more than the bytes. Measured on
-// MI355X, reduce-scatter + all-gather, steps against one launch each: world 4 at 4 MiB per rank 26.9
-// against 12.3 us, 16 MiB 41.9 / 31.5, 64 MiB 145 / 115, 80 MiB 184 / 169, 96 MiB equal, 128 MiB 293 /
-// 303, 256 MiB 566 / 585; world 3 at 4 MiB 20.8 / 15.8, 64 MiB 104 / 92, 96 MiB 152 / 133, 128 MiB
-// 203 / 216. At world 2 a collective is one step anyway and the step kernels' cache policies do better
-// (64 MiB 49 / 51 us, 256 MiB 186 / 236). Beyond the caches the steps' per-step policies win and remain the form.
+// whole reduce-scatter (all-gather) as ONE launch. -1: by world size. The one-launch forms read
+// every rank's copy of a chunk once and write the W-1 partial sums (read the owner's chunk once
+// and write the W-1 copies), 4 (2W-1) (4 W) bytes per element where the steps move 12 (W-1)
+// (8 (W-1)), and leave no gaps between launches. Measured on MI355X, reduce-scatter, steps
+// against one launch: world 4 at 4 MiB per rank 15.3 against 10.4 us, 16 MiB 25.8 / 21.6, 64 MiB
+// 88 / 70, 96 MiB 132 / 120, 128 MiB 175 / 152, 256 MiB 336 / 326 (non-temporal accesses once the
+// ranks' tensors together exceed 320 MiB; with everything cached the one launch loses there:
+// 343); world 3 at 64 MiB 65 / 55, 96 MiB 94 / 79, 256 MiB 236 / 239 (222 with the occupancy cap).
+// At world 2 a collective is one step anyway and the step kernels' policies do better (64 MiB
+// 49 / 51 us, 256 MiB 186 / 236).
 std::atomic<int> g_ring_form{-1};
-constexpr int64_t kOneLaunchFootprint = int64_t(320) << 20;
+constexpr int64_t kOneLaunchFootprint = int64_t(320) << 20;  // beyond: nothing written is found in the caches again
 
 bool one_launch_form(const LocalRanks& lr) {
   if (!chain_handles(lr.world)) return false;
   const int set = g_ring_form.load(std::memory_order_relaxed);
-  return set >= 0 ? set == 1 : lr.world >= 3 && lr.footprint <= kOneLaunchFootprint;
+  return set >= 0 ? set == 1 : lr.world >= 3;
 }
 
 // The all-gather as one launch wins at every size from world 3 on (world 4, 256 MiB per rank: 236 -> 191 us;
@@ -598,8 +598,9 @@ void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hi
   const int n = lr.world;
   if (one_launch_form(lr)) {
     const int64_t cap = static_cast<int64_t>(t_call_cus ? t_call_cus : compute_units()) * g_blocks_per_cu;
-    chain_reduce_scatter(lr.base, lr.lo, lr.len, n, lr.dtype, lr.es, average, keep_sent,
-                         static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
+    const bool cold = lr.footprint > kOneLaunchFootprint;
+    chain_reduce_scatter(lr.base, lr.lo, lr.len, n, lr.dtype, lr.es, average, keep_sent, cold,
+                         cold ? occupancy_pad(TDM_XCD_REDUCE) : 0, static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
     return;
   }
   for (int s = 0; s < n - 1; ++s) {

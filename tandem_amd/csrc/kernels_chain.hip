@@ -53,7 +53,9 @@ __device__ __forceinline__ void chain_elem(const T (&in)[kWorld], T (&out)[kWorl
   }
 }
 
-template <typename T, int kWorld, int kDiv>
+// kMask: the cache policy (kernels_device.h): 0 everything cached, for footprints that stay in the caches; 7 non-temporal
+// loads and stores, for footprints beyond them.
+template <typename T, int kWorld, int kDiv, int kMask>
 __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divisor<T> dv) {
   constexpr int L = lanes<T>();
   constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
@@ -76,7 +78,7 @@ __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divi
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
           const int64_t v = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
-          if (v < nv) raw[k][u] = load_rmw<0>(p[k] + v * 16);
+          if (v < nv) raw[k][u] = load_rmw<kMask>(p[k] + v * 16);
         }
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
@@ -92,9 +94,9 @@ __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divi
 #pragma unroll
             for (int k = 0; k < kWorld; ++k) res[k].v[l] = out[k];
           }
-          if (keep) store16<0>(p[0] + v * 16, pack<T>(res[0]));
+          if (keep) store16<kMask>(p[0] + v * 16, pack<T>(res[0]));
 #pragma unroll
-          for (int k = 1; k < kWorld; ++k) store16<0>(p[k] + v * 16, pack<T>(res[k]));
+          for (int k = 1; k < kWorld; ++k) store16<kMask>(p[k] + v * 16, pack<T>(res[k]));
         }
       }
       const int head = tab.vec_ok[sg] - 1;
@@ -127,8 +129,8 @@ __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divi
   }
 }
 
-template <typename T, int kWorld>
-void launch_chain_w(const ChainTable& tab, bool average, int grid, hipStream_t stream) {
+template <typename T, int kWorld, int kMask>
+void launch_chain_m(const ChainTable& tab, bool average, int grid, unsigned pad, hipStream_t stream) {
   Divisor<T> dv;
   using A = typename Elem<T>::acc;
   dv.divisor = static_cast<A>(kWorld);
@@ -136,23 +138,26 @@ void launch_chain_w(const ChainTable& tab, bool average, int grid, hipStream_t s
   const dim3 g(grid), b(kThreads);
   if constexpr (Elem<T>::floating) {
     if (average && (kWorld & (kWorld - 1)) == 0) {
-      hipLaunchKernelGGL((k1_chain_kernel<T, kWorld, 1>), g, b, 0, stream, tab, dv);
+      hipLaunchKernelGGL((k1_chain_kernel<T, kWorld, 1, kMask>), g, b, pad, stream, tab, dv);
       return;
     }
     if (average) {
-      hipLaunchKernelGGL((k1_chain_kernel<T, kWorld, 2>), g, b, 0, stream, tab, dv);
+      hipLaunchKernelGGL((k1_chain_kernel<T, kWorld, 2, kMask>), g, b, pad, stream, tab, dv);
       return;
     }
   }
-  hipLaunchKernelGGL((k1_chain_kernel<T, kWorld, 0>), g, b, 0, stream, tab, dv);
+  hipLaunchKernelGGL((k1_chain_kernel<T, kWorld, 0, kMask>), g, b, pad, stream, tab, dv);
 }
 
 template <typename T>
-void launch_chain(const ChainTable& tab, int world, bool average, int grid, hipStream_t stream) {
-  switch (world) {
-    case 2: launch_chain_w<T, 2>(tab, average, grid, stream); break;
-    case 3: launch_chain_w<T, 3>(tab, average, grid, stream); break;
-    default: launch_chain_w<T, 4>(tab, average, grid, stream); break;
+void launch_chain(const ChainTable& tab, int world, bool average, int grid, bool cold, unsigned pad, hipStream_t stream) {
+  switch (world * 2 + (cold ? 1 : 0)) {
+    case 4: launch_chain_m<T, 2, 0>(tab, average, grid, pad, stream); break;
+    case 5: launch_chain_m<T, 2, 7>(tab, average, grid, pad, stream); break;
+    case 6: launch_chain_m<T, 3, 0>(tab, average, grid, pad, stream); break;
+    case 7: launch_chain_m<T, 3, 7>(tab, average, grid, pad, stream); break;
+    case 8: launch_chain_m<T, 4, 0>(tab, average, grid, pad, stream); break;
+    default: launch_chain_m<T, 4, 7>(tab, average, grid, pad, stream); break;
   }
 }
 
@@ -254,7 +259,7 @@ namespace {
 bool chain_handles(int world) { return world >= 2 && world <= kChainMaxWorld; }
 
 void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
-                          bool keep_sent, int max_grid, hipStream_t stream) {
+                          bool keep_sent, bool cold, unsigned pad, int max_grid, hipStream_t stream) {
   if (!chain_handles(world)) throw Invalid("the one-launch reduce-scatter handles world sizes 2..4");
   ChainTable tab;
   std::memset(&tab, 0, sizeof tab);
@@ -279,12 +284,12 @@ void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* l
   if (k == 0) return;
   const int grid = static_cast<int>(tiles < max_grid ? tiles : max_grid);
   switch (dtype) {
-    case TDM_F32: launch_chain<float>(tab, world, average, grid, stream); break;
-    case TDM_F64: launch_chain<double>(tab, world, average, grid, stream); break;
-    case TDM_F16: launch_chain<f16_t>(tab, world, average, grid, stream); break;
-    case TDM_BF16: launch_chain<bf16_t>(tab, world, average, grid, stream); break;
-    case TDM_I64: launch_chain<int64_t>(tab, world, false, grid, stream); break;
-    case TDM_I32: launch_chain<int32_t>(tab, world, false, grid, stream); break;
+    case TDM_F32: launch_chain<float>(tab, world, average, grid, cold, pad, stream); break;
+    case TDM_F64: launch_chain<double>(tab, world, average, grid, cold, pad, stream); break;
+    case TDM_F16: launch_chain<f16_t>(tab, world, average, grid, cold, pad, stream); break;
+    case TDM_BF16: launch_chain<bf16_t>(tab, world, average, grid, cold, pad, stream); break;
+    case TDM_I64: launch_chain<int64_t>(tab, world, false, grid, cold, pad, stream); break;
+    case TDM_I32: launch_chain<int32_t>(tab, world, false, grid, cold, pad, stream); break;
     default: throw Invalid("unknown dtype " + std::to_string(dtype));
   }
   check_hip(hipGetLastError(), "k1_chain launch");
