@@ -82,7 +82,7 @@ void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool av
 constexpr int kChainMaxWorld = 4;
 bool chain_handles(int world);
 void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
-                          bool keep_sent, bool cold, unsigned occupancy_pad, int max_grid, hipStream_t stream);
+                          bool keep_sent, bool cold, unsigned occupancy_pad, int xcd_shift, int max_grid, hipStream_t stream);
 // the ring all-gather of a whole group in one launch: every chunk read once from its owner and stored into the
 // other ranks' buffers; world sizes 2..8; `cold`: the footprint is beyond the caches (non-temporal accesses)
 bool gather_handles(int world);

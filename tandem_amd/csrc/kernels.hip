@@ -111,6 +111,7 @@ int xcd_shift(int kind, int world, bool cold) {
   const int set = g_xcd_shift[kind].load(std::memory_order_relaxed);
   if (set >= 0) return set;
   switch (kind) {
+    case TDM_XCD_REDUCE: return cold && world == 3 ? 6 : 0;  // cold: the one-launch reduce-scatter (256 MiB per rank at world 3: 233 -> 218 us; world 4: none)
     case TDM_XCD_STEP: return 6;
     case TDM_XCD_ADAMW: return 7;
     case TDM_XCD_FOLD_TABLE: return world >= 4 ? 8 : 0;
@@ -571,9 +572,10 @@ int64_t footprint(const LocalRanks& lr) { return lr.footprint; }
 // and write the W-1 copies), 4 (2W-1) (4 W) bytes per element where the steps move 12 (W-1)
 // (8 (W-1)), and leave no gaps between launches. Measured on MI355X, reduce-scatter, steps
 // against one launch: world 4 at 4 MiB per rank 15.3 against 10.4 us, 16 MiB 25.8 / 21.6, 64 MiB
-// 88 / 70, 96 MiB 132 / 120, 128 MiB 175 / 152, 256 MiB 336 / 326 (non-temporal accesses once the
-// ranks' tensors together exceed 320 MiB; with everything cached the one launch loses there:
-// 343); world 3 at 64 MiB 65 / 55, 96 MiB 94 / 79, 256 MiB 236 / 239 (222 with the occupancy cap).
+// 88 / 70, 96 MiB 132 / 120, 128 MiB 175 / 152, 256 MiB 337 / 291 (once the ranks' tensors together
+// exceed 320 MiB: non-temporal accesses and 2 KiB per workgroup and stream; with everything cached
+// and 4 KiB the one launch loses there, 343; an occupancy cap only loses); world 3 at 64 MiB 65 / 55,
+// 96 MiB 94 / 79, 256 MiB 235 / 218.
 // At world 2 a collective is one step anyway and the step kernels' policies do better (64 MiB
 // 49 / 51 us, 256 MiB 186 / 236).
 std::atomic<int> g_ring_form{-1};
@@ -600,7 +602,8 @@ void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hi
     const int64_t cap = static_cast<int64_t>(t_call_cus ? t_call_cus : compute_units()) * g_blocks_per_cu;
     const bool cold = lr.footprint > kOneLaunchFootprint;
     chain_reduce_scatter(lr.base, lr.lo, lr.len, n, lr.dtype, lr.es, average, keep_sent, cold,
-                         cold ? occupancy_pad(TDM_XCD_REDUCE) : 0, static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
+                         cold ? occupancy_pad(TDM_XCD_REDUCE) : 0, xcd_shift(TDM_XCD_REDUCE, n, cold),
+                         static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
     return;
   }
   for (int s = 0; s < n - 1; ++s) {

@@ -32,6 +32,7 @@ namespace {
 struct ChainTable {
   int nseg;
   int keep_sent;  // the first sender's copy is left holding y (x / W), as div_ of the whole tensor does
+  int shift;      // of tile_of()
   int64_t tile_end[TDM_MAX_WORLD];
   char* ptr[TDM_MAX_WORLD][TDM_MAX_WORLD];  // [segment][rank]
   int64_t count[TDM_MAX_WORLD];
@@ -55,12 +56,15 @@ __device__ __forceinline__ void chain_elem(const T (&in)[kWorld], T (&out)[kWorl
 
 // kMask: the cache policy (kernels_device.h): 0 everything cached, for footprints that stay in the caches; 7 non-temporal
 // loads and stores, for footprints beyond them.
-template <typename T, int kWorld, int kDiv, int kMask>
+// A workgroup takes kU vectors per lane and stream: 2 (4 KiB of every stream) within the caches, 1 beyond.
+template <typename T, int kWorld, int kDiv, int kMask, int kU = (kMask == 0 ? kUnroll : 1)>
 __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divisor<T> dv) {
   constexpr int L = lanes<T>();
-  constexpr int64_t kTileElems = static_cast<int64_t>(kTileVecs) * L;
+  constexpr int kVecs = kThreads * kU;  // vectors of every stream per workgroup
+  constexpr int64_t kTileElems = static_cast<int64_t>(kVecs) * L;
   const int64_t total = tab.tile_end[tab.nseg - 1];
-  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+  for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
+    const int64_t tile = tile_of(at, total, tab.shift);
     int sg = 0;
     while (tile >= tab.tile_end[sg]) ++sg;
     const int64_t t = tile - (sg ? tab.tile_end[sg - 1] : 0);
@@ -72,17 +76,17 @@ __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divi
     const bool keep = tab.keep_sent != 0;
     if (tab.vec_ok[sg]) {
       const int64_t nv = n / L;
-      vec16 raw[kWorld][kUnroll];
+      vec16 raw[kWorld][kU];
 #pragma unroll
       for (int k = 0; k < kWorld; ++k)
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-          const int64_t v = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
+        for (int u = 0; u < kU; ++u) {
+          const int64_t v = t * kVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
           if (v < nv) raw[k][u] = load_rmw<kMask>(p[k] + v * 16);
         }
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const int64_t v = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
+      for (int u = 0; u < kU; ++u) {
+        const int64_t v = t * kVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
         if (v < nv) {
           Lanes<T> res[kWorld];
 #pragma unroll
@@ -113,7 +117,7 @@ __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divi
       }
     } else {  // a copy off the 16-byte grid: element by element, still coalesced
       const int64_t e0 = t * kTileElems + threadIdx.x;
-      for (int r = 0; r < kUnroll * L; ++r) {
+      for (int r = 0; r < kU * L; ++r) {
         const int64_t i = e0 + static_cast<int64_t>(r) * kThreads;
         if (i < n) {
           T in[kWorld], out[kWorld];
@@ -259,12 +263,13 @@ namespace {
 bool chain_handles(int world) { return world >= 2 && world <= kChainMaxWorld; }
 
 void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
-                          bool keep_sent, bool cold, unsigned pad, int max_grid, hipStream_t stream) {
+                          bool keep_sent, bool cold, unsigned pad, int shift, int max_grid, hipStream_t stream) {
   if (!chain_handles(world)) throw Invalid("the one-launch reduce-scatter handles world sizes 2..4");
   ChainTable tab;
   std::memset(&tab, 0, sizeof tab);
   tab.keep_sent = keep_sent && average ? 1 : 0;  // without a division the first sender's copy is x already
-  const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
+  tab.shift = shift;
+  const int64_t tile_elems = static_cast<int64_t>(cold ? kThreads : kTileVecs) * (16 / es);  // as the kernel's kU
   int64_t tiles = 0;
   int k = 0;
   for (int c = 0; c < world; ++c) {
