@@ -86,8 +86,8 @@ void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* l
 // the ring all-gather of a whole group in one launch: every chunk read once from its owner and stored into the
 // other ranks' buffers; world sizes 2..8; `cold`: the footprint is beyond the caches (non-temporal accesses)
 bool gather_handles(int world);
-void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, int world, int es, bool cold, int max_grid,
-                      hipStream_t stream);
+void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, int world, int es, bool cold, unsigned occupancy_pad,
+                      int xcd_shift, int vectors_per_lane, int max_grid, hipStream_t stream);
 void zero2_step_segment(const tdm_step_seg& seg, int world, bool average, const tdm_adamw_scalars& s, int order, hipStream_t stream);
 
 }  // namespace tandem_hip

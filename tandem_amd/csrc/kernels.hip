@@ -137,6 +137,7 @@ unsigned occupancy_pad(int kind, bool cold = true) {
   switch (kind) {
     case TDM_XCD_STEP: return 24576;
     case TDM_XCD_ADAMW: return 24576;
+    case TDM_XCD_COPY: return cold ? 16384 : 0;  // the one-launch all-gather (the ring's copy step takes no pad)
     case TDM_XCD_FOLD: return cold ? 24576 : 0;  // 256 MiB per rank at world 4: 0.350 -> 0.343 ms; 64 MiB: 0.078 -> 0.081
     default: return 0;
   }
@@ -625,8 +626,11 @@ void local_all_gather(const LocalRanks& lr, hipStream_t stream) {
     // every chunk is read once from its owner and stored into the other ranks' buffers: the ring's W-1
     // forwarding steps leave the same bytes
     const int64_t cap = static_cast<int64_t>(t_call_cus ? t_call_cus : compute_units()) * g_blocks_per_cu;
-    gather_multicast(lr.base, lr.lo, lr.len, n, lr.es, lr.footprint > kOneLaunchFootprint,
-                     static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
+    const bool cold = lr.footprint > kOneLaunchFootprint;
+    // beyond the caches: 2 KiB per workgroup and stream and 16 KiB of occupancy pad (world 4, 256 MiB per rank: 189 us with
+    // 4 KiB and no pad, 174 with the pad, 168 with both; 32 KiB: 202-232)
+    gather_multicast(lr.base, lr.lo, lr.len, n, lr.es, cold, occupancy_pad(TDM_XCD_COPY, cold), xcd_shift(TDM_XCD_COPY, n, cold),
+                     cold ? 1 : 2, static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
     return;
   }
   for (int s = 0; s < n - 1; ++s) {

@@ -173,6 +173,8 @@ void launch_chain(const ChainTable& tab, int world, bool average, int grid, bool
 struct GatherTable {
   int nseg;
   int ndst;  // destinations per segment (W - 1)
+  int shift;  // of tile_of()
+  int pad_;
   int64_t tile_end[TDM_MAX_WORLD];
   const char* src[TDM_MAX_WORLD];
   char* dst[TDM_MAX_WORLD][TDM_MAX_WORLD - 1];
@@ -180,11 +182,13 @@ struct GatherTable {
   int32_t vec_ok[TDM_MAX_WORLD];  // as the other tables': 0 byte by byte, 1 + h with h bytes before the pointers
 };
 
-template <int kMask>
+template <int kMask, int kU>
 __global__ __launch_bounds__(kThreads) void k1_gather_kernel(GatherTable tab) {
-  constexpr int64_t kTileBytes = static_cast<int64_t>(kTileVecs) * 16;
+  constexpr int kVecs = kThreads * kU;  // vectors of every stream per workgroup
+  constexpr int64_t kTileBytes = static_cast<int64_t>(kVecs) * 16;
   const int64_t total = tab.tile_end[tab.nseg - 1];
-  for (int64_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+  for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
+    const int64_t tile = tile_of(at, total, tab.shift);
     int sg = 0;
     while (tile >= tab.tile_end[sg]) ++sg;
     const int64_t t = tile - (sg ? tab.tile_end[sg - 1] : 0);
@@ -192,15 +196,15 @@ __global__ __launch_bounds__(kThreads) void k1_gather_kernel(GatherTable tab) {
     const int64_t n = tab.bytes[sg];
     if (tab.vec_ok[sg]) {
       const int64_t nv = n / 16;
-      vec16 raw[kUnroll];
+      vec16 raw[kU];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const int64_t v = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
+      for (int u = 0; u < kU; ++u) {
+        const int64_t v = t * kVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
         if (v < nv) raw[u] = load_stream<kMask>(from + v * 16);
       }
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const int64_t v = t * kTileVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
+      for (int u = 0; u < kU; ++u) {
+        const int64_t v = t * kVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
         if (v < nv)
           for (int k = 0; k < tab.ndst; ++k) store16<kMask>(tab.dst[sg][k] + v * 16, raw[u]);
       }
@@ -225,13 +229,14 @@ __global__ __launch_bounds__(kThreads) void k1_gather_kernel(GatherTable tab) {
 
 bool gather_handles(int world) { return world >= 2 && world <= TDM_MAX_WORLD; }
 
-void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, int world, int es, bool cold, int max_grid,
-                      hipStream_t stream) {
+void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, int world, int es, bool cold, unsigned pad,
+                      int shift, int per_lane, int max_grid, hipStream_t stream) {
   if (!gather_handles(world)) throw Invalid("the one-launch all-gather handles world sizes 2..8");
   GatherTable tab;
   std::memset(&tab, 0, sizeof tab);
   tab.ndst = world - 1;
-  const int64_t tile_bytes = static_cast<int64_t>(kTileVecs) * 16;
+  tab.shift = shift;
+  const int64_t tile_bytes = static_cast<int64_t>(kThreads) * per_lane * 16;
   int64_t tiles = 0;
   int k = 0;
   for (int c = 0; c < world; ++c) {
@@ -252,8 +257,13 @@ void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, 
   tab.nseg = k;
   if (k == 0) return;
   const dim3 grid(static_cast<unsigned>(tiles < max_grid ? tiles : max_grid)), block(kThreads);
-  if (cold) hipLaunchKernelGGL((k1_gather_kernel<7>), grid, block, 0, stream, tab);
-  else hipLaunchKernelGGL((k1_gather_kernel<0>), grid, block, 0, stream, tab);
+  if (per_lane != 1 && per_lane != 2) throw Invalid("1 or 2 vectors per lane");
+  switch ((cold ? 2 : 0) + (per_lane == 2 ? 1 : 0)) {
+    case 0: hipLaunchKernelGGL((k1_gather_kernel<0, 1>), grid, block, pad, stream, tab); break;
+    case 1: hipLaunchKernelGGL((k1_gather_kernel<0, 2>), grid, block, pad, stream, tab); break;
+    case 2: hipLaunchKernelGGL((k1_gather_kernel<7, 1>), grid, block, pad, stream, tab); break;
+    default: hipLaunchKernelGGL((k1_gather_kernel<7, 2>), grid, block, pad, stream, tab); break;
+  }
   check_hip(hipGetLastError(), "k1_gather launch");
 }
 
