@@ -53,6 +53,18 @@ def test_argument_errors_need_no_gpu():
     assert L.tdm_set_xcd_group(6, 0) == 1 and b"family" in L.tdm_last_error()
     assert L.tdm_set_xcd_group(0, 13) == 1 and b"shift" in L.tdm_last_error()
     assert L.tdm_set_xcd_group(3, 4) == 0 and L.tdm_set_xcd_group(-1, -1) == 0
+    assert L.tdm_set_ring_form(2) == 1 and b"ring form" in L.tdm_last_error()
+    assert L.tdm_set_ring_form(1) == 0 and L.tdm_set_ring_form(-1) == 0
+    assert L.tdm_set_occupancy_pad(4, 65537) == 1 and L.tdm_set_occupancy_pad(4, 8192) == 0 and L.tdm_set_occupancy_pad(-1, -1) == 0
+    a, b, c = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    assert L.tdm_build_geometry(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)) == 0
+    assert (a.value, b.value, c.value) == (4096, 128, 4096) and c.value == L.tdm_table_tile_bytes()
+    assert L.tdm_build_geometry(None, ctypes.byref(b), ctypes.byref(c)) == 1
+    assert L.tdm_k2_static_max_tiles() == 16384
+    # the static bucket fold and the probe check their arguments before they touch the GPU
+    assert L.tdm_k2_bucket_fold_static(segs, 2, 2, 99, 1, 0, None) == 1 and b"dtype" in L.tdm_last_error()
+    assert L.tdm_k2_bucket_fold_static(segs, 2, 9, 0, 1, 0, None) == 1 and b"world" in L.tdm_last_error()
+    assert L.tdm_probe_stream_mix(None, 0, None, 0, 16, 1, 0, 0, None) == 1 and b"streams" in L.tdm_last_error()
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
