@@ -89,25 +89,44 @@ def timed(fn, reps, warm=3):
     return e0.elapsed_time(e1) * 1e-3 / reps
 
 
-def ring_pass(lw, flats, events=None):
+def ring_pass(lw, flats, events=None, prepared=None):
     """One step: reduce-scatter (avg) then all-gather; the two halves bracketed by
-    events on the launch stream when asked."""
+    events on the launch stream when asked. `prepared`: the arguments of ring_args(), built once."""
     import torch
 
-    from tandem_amd._lib import check, lib, stream_ptr
+    from tandem_amd._lib import check
 
-    ptrs, n, st = lw._ptrs(flats), flats[0].numel(), stream_ptr(flats[0].device)
-    none = lw._sizes(None, None)[0]
+    rs, ag, ptrs, world, n, none, st = prepared or ring_args(lw, flats)
     if events is not None:
         e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
         e[0].record()
-    check(lib().tdm_local_reduce_scatter(ptrs, lw.world, n, 0, none, 0, 1, 0, st))
+    check(rs(ptrs, world, n, 0, none, 0, 1, 0, st))
     if events is not None:
         e[1].record()
-    check(lib().tdm_local_all_gather(ptrs, lw.world, n, 0, none, 0, st))
+    check(ag(ptrs, world, n, 0, none, 0, st))
     if events is not None:
         e[2].record()
         events.append(e)
+
+
+def ring_args(lw, flats):
+    """The two C entry points and their arguments for ring_pass, on torch's current stream."""
+    from tandem_amd._lib import lib, stream_ptr
+
+    return (lib().tdm_local_reduce_scatter, lib().tdm_local_all_gather, lw._ptrs(flats), lw.world, flats[0].numel(),
+            lw._sizes(None, None)[0], stream_ptr(flats[0].device))
+
+
+def fold_call(lw, flats):
+    """The all-reduce as a single launch, as a closure over arguments prepared once: what a
+    compiled host calling the C ABI pays per call (the Python wrapper's checks and views cost
+    more than the launch at small sizes)."""
+    from tandem_amd import _lib
+
+    ptrs, n, st = lw._ptrs(flats), flats[0].numel(), _lib.stream_ptr(flats[0].device)
+    fn, world = _lib.lib().tdm_local_all_reduce, lw.world
+    _lib.check(fn(ptrs, world, n, 0, 1, _lib.ALLREDUCE_FOLD, st))
+    return lambda: fn(ptrs, world, n, 0, 1, _lib.ALLREDUCE_FOLD, st)
 
 
 def time_ring(lw, bufs, steps, warmup):
@@ -119,17 +138,18 @@ def time_ring(lw, bufs, steps, warmup):
     import torch
 
     flats = [b.reshape(-1) for b in bufs]
+    prepared = ring_args(lw, flats)
     for _ in range(warmup):
-        ring_pass(lw, flats)
+        ring_pass(lw, flats, None, prepared)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        ring_pass(lw, flats)
+        ring_pass(lw, flats, None, prepared)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     events = []
     for _ in range(steps):
-        ring_pass(lw, flats, events)
+        ring_pass(lw, flats, events, prepared)
     torch.cuda.synchronize()
     rs_ms = sum(e[0].elapsed_time(e[1]) for e in events)
     ag_ms = sum(e[1].elapsed_time(e[2]) for e in events)
@@ -155,11 +175,11 @@ def sweep(lw, dev, steps):
         one, _, _ = time_ring(lw, bufs, reps, 3)
         check(lib().tdm_set_ring_form(0))  # the ring's steps, one launch each: K1 and the copy step
         per, rs, ag = time_ring(lw, bufs, reps, 3)
-        fold = timed(lambda: lw.all_reduce(bufs, "avg", algorithm="fold"), reps)
+        flats = [x.reshape(-1) for x in bufs]
+        fold = timed(fold_call(lw, flats), reps)
         b = n * 4
         graph_ms = fold_graph_ms = one_graph_ms = None
         if kib <= 65536:  # sizes where the gaps between the six launches still count: the same ring pass replayed from a HIP graph
-            flats = [x.reshape(-1) for x in bufs]
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 ring_pass(lw, flats)

@@ -3,9 +3,9 @@
 For a tandem maintainer: copy this file to `tandem/hip_engine.py`. It has the surface of the
 pybind module the reference builds from tandem/csrc/engine.cpp:103-122 (`Engine(job, rank, size,
 slots, slot_bytes, timeout, device)`, `connect`, `close`, the collectives, and a handle with
-`wait()`, `done()`, `started`, `finished`), bound with ctypes, so tandem/comm.py needs the few
-lines of INTEGRATION.md and nothing else. tandem_amd.comm.Group does not use this file: it is
-the same binding grown into a whole Group.
+`wait()`, `done()`, `started`, `finished`), bound with ctypes, so tandem/comm.py only has to
+import it where it imports its own native module. tandem_amd.comm.Group does not use this file:
+it is the same binding grown into a whole Group.
 """
 
 import ctypes

@@ -58,18 +58,20 @@ class LocalWorld:
         lib()  # fail now, not at the first collective, if the HIP library is missing
 
     # ---- checks
-    def _flat(self, bufs, what):
+    def _ranks(self, bufs, what):
+        """The rank buffers checked (one per rank, in GPU memory, contiguous, alike) and their
+        addresses for the C ABI, with the count, dtype and device they share. No views are made:
+        at small messages the host side of a call costs more than its launch."""
         if len(bufs) != self.world:
             raise ValueError(f"{what}: expected {self.world} rank buffers, got {len(bufs)}")
-        flats = []
-        for t in bufs:
+        t0 = bufs[0]
+        require_device_tensor(t0, what)
+        n, dtype, device = t0.numel(), t0.dtype, t0.device
+        for t in bufs[1:]:
             require_device_tensor(t, what)
-            flats.append(t.reshape(-1))
-        f0 = flats[0]
-        for f in flats[1:]:
-            if f.numel() != f0.numel() or f.dtype != f0.dtype or f.device != f0.device:
+            if t.numel() != n or t.dtype != dtype or t.device != device:
                 raise ValueError(f"{what}: rank buffers differ in size, dtype or device")
-        return flats
+        return self._ptrs(bufs), n, dtype, device
 
     @staticmethod
     def _op(op):
@@ -94,21 +96,19 @@ class LocalWorld:
         One launch per ring step; the other chunks are left holding the same
         partial sums as in the reference."""
         average = self._op(op)
-        flats = self._flat(bufs, "reduce_scatter")
-        bounds = chunk_bounds(flats[0].numel(), self.world, sizes)
+        ptrs, numel, dtype, device = self._ranks(bufs, "reduce_scatter")
+        bounds = chunk_bounds(numel, self.world, sizes)
         arr, n = self._sizes(bounds, sizes)
-        check(lib().tdm_local_reduce_scatter(self._ptrs(flats), self.world, flats[0].numel(), dtype_code(flats[0].dtype),
-                                             arr, n, int(average), 1, stream_ptr(flats[0].device)))
-        return [flats[r][bounds[r][0]:bounds[r][1]] for r in range(self.world)]
+        check(lib().tdm_local_reduce_scatter(ptrs, self.world, numel, dtype_code(dtype), arr, n, int(average), 1, stream_ptr(device)))
+        return [bufs[r].reshape(-1)[bounds[r][0]:bounds[r][1]] for r in range(self.world)]
 
     def all_gather(self, bufs, sizes=None):
         """Rank r holds chunk r; afterwards every rank holds every chunk
         (tandem/comm.py:371-385). One launch per ring step."""
-        flats = self._flat(bufs, "all_gather")
-        bounds = chunk_bounds(flats[0].numel(), self.world, sizes)
+        ptrs, numel, dtype, device = self._ranks(bufs, "all_gather")
+        bounds = chunk_bounds(numel, self.world, sizes)
         arr, n = self._sizes(bounds, sizes)
-        check(lib().tdm_local_all_gather(self._ptrs(flats), self.world, flats[0].numel(), dtype_code(flats[0].dtype),
-                                         arr, n, stream_ptr(flats[0].device)))
+        check(lib().tdm_local_all_gather(ptrs, self.world, numel, dtype_code(dtype), arr, n, stream_ptr(device)))
         return bufs
 
     def all_reduce(self, bufs, op="sum", algorithm=None):
@@ -118,14 +118,13 @@ class LocalWorld:
         sums in the ring's order for the element's chunk and writes every rank;
         the same bits with about half the HBM traffic."""
         average = self._op(op)
-        flats = self._flat(bufs, "all_reduce")
+        ptrs, numel, dtype, device = self._ranks(bufs, "all_reduce")
         if algorithm is None:
             algorithm = "fold" if self.world <= _lib.TDM_MAX_WORLD else "ring"
         if algorithm not in ("ring", "fold"):
             raise ValueError(f"unknown all-reduce algorithm {algorithm}")
         code = _lib.ALLREDUCE_FOLD if algorithm == "fold" else _lib.ALLREDUCE_RING
-        check(lib().tdm_local_all_reduce(self._ptrs(flats), self.world, flats[0].numel(), dtype_code(flats[0].dtype),
-                                         int(average), code, stream_ptr(flats[0].device)))
+        check(lib().tdm_local_all_reduce(ptrs, self.world, numel, dtype_code(dtype), int(average), code, stream_ptr(device)))
         return bufs
 
     def unit_gather(self, fulls, shards, sizes):

@@ -1,4 +1,4 @@
-"""tandem_amd/hip_engine.py, the binding INTEGRATION.md gives a tandem maintainer, driven on
+"""tandem_amd/hip_engine.py, the binding offered to a tandem maintainer, driven on
 the GPU the way the reference's own Group drives its native engine (tandem/comm.py:149-170:
 create, the launcher's barrier, connect, barrier; tandem/comm.py:326-452: every collective
 returns a handle that is waited for), by two processes that share the GPU. Results against

@@ -1,5 +1,5 @@
-"""INTEGRATION.md quotes tandem_amd/hip_engine.py, the binding a tandem maintainer would copy
-into the reference tree: the quotation and the file must be the same text, and the file must
+"""The integration notes at the repository root quote tandem_amd/hip_engine.py, the binding a tandem
+maintainer would copy into the reference tree: the quotation and the file must be the same text, and the file must
 offer what the reference's Group calls on its native engine (tandem/comm.py:149-160,326-452 and
 the pybind surface tandem/csrc/engine.cpp:103-122 there)."""
 
