@@ -630,7 +630,7 @@ void local_all_gather(const LocalRanks& lr, hipStream_t stream) {
     // beyond the caches: 2 KiB per workgroup and stream and 16 KiB of occupancy pad (world 4, 256 MiB per rank: 189 us with
     // 4 KiB and no pad, 174 with the pad, 168 with both; 32 KiB: 202-232)
     gather_multicast(lr.base, lr.lo, lr.len, n, lr.es, cold, occupancy_pad(TDM_XCD_COPY, cold), xcd_shift(TDM_XCD_COPY, n, cold),
-                     cold ? 1 : 2, static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
+                     cold ? 1 : kWarmVecs, static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
     return;
   }
   for (int s = 0; s < n - 1; ++s) {

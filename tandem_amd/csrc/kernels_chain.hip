@@ -57,7 +57,7 @@ __device__ __forceinline__ void chain_elem(const T (&in)[kWorld], T (&out)[kWorl
 // kMask: the cache policy (kernels_device.h): 0 everything cached, for footprints that stay in the caches; 7 non-temporal
 // loads and stores, for footprints beyond them.
 // A workgroup takes kU vectors per lane and stream: 2 (4 KiB of every stream) within the caches, 1 beyond.
-template <typename T, int kWorld, int kDiv, int kMask, int kU = (kMask == 0 ? kUnroll : 1)>
+template <typename T, int kWorld, int kDiv, int kMask, int kU = (kMask == 0 ? kWarmVecs : 1)>
 __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divisor<T> dv) {
   constexpr int L = lanes<T>();
   constexpr int kVecs = kThreads * kU;  // vectors of every stream per workgroup
@@ -267,9 +267,6 @@ void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, 
   check_hip(hipGetLastError(), "k1_gather launch");
 }
 
-namespace {
-}  // namespace
-
 bool chain_handles(int world) { return world >= 2 && world <= kChainMaxWorld; }
 
 void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
@@ -279,7 +276,7 @@ void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* l
   std::memset(&tab, 0, sizeof tab);
   tab.keep_sent = keep_sent && average ? 1 : 0;  // without a division the first sender's copy is x already
   tab.shift = shift;
-  const int64_t tile_elems = static_cast<int64_t>(cold ? kThreads : kTileVecs) * (16 / es);  // as the kernel's kU
+  const int64_t tile_elems = static_cast<int64_t>(kThreads) * (cold ? 1 : kWarmVecs) * (16 / es);  // as the kernel's kU
   int64_t tiles = 0;
   int k = 0;
   for (int c = 0; c < world; ++c) {
