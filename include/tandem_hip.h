@@ -23,13 +23,18 @@ extern "C" {
 
 typedef void* tdm_stream;
 
-/* The element types the reducing kernels know. A deliberate difference from the reference, whose
- * engine reduces any ATen dtype by falling back to add_ (tandem/csrc/collectives.cpp:254-256): every
- * entry point that adds (tdm_k1_reduce_step, tdm_local_*, tdm_k2_*, tdm_all_reduce, tdm_reduce_scatter,
- * tdm_direct_*) refuses any other code with TDM_EINVAL ("unknown dtype"), so int8 / uint8 / int16 / bool
- * sums are not offered. Entry points that only copy (tdm_all_gather, tdm_broadcast, tdm_sendrecv,
- * tdm_unit_gather) also take TDM_BYTES, which covers every dtype. */
-enum tdm_dtype { TDM_F32 = 0, TDM_F64 = 1, TDM_F16 = 2, TDM_BF16 = 3, TDM_I64 = 4, TDM_I32 = 5 };
+/* The element types the reducing kernels know. Integer sums wrap around, as ATen's add_ does; 16-bit
+ * floats are widened to fp32, added and rounded to nearest even once per add (tandem/csrc/reduce.cu:27-36).
+ * The reference's engine reduces any further ATen dtype by falling back to add_
+ * (tandem/csrc/collectives.cpp:254-256); here every entry point that adds (tdm_k1_reduce_step, tdm_local_*,
+ * tdm_k2_*, tdm_all_reduce, tdm_reduce_scatter, tdm_direct_*) refuses any other code with TDM_EINVAL
+ * ("unknown dtype"): bool, the unsigned types wider than a byte, complex and the 8-bit floats are not
+ * summed. Entry points that only copy (tdm_all_gather, tdm_broadcast, tdm_sendrecv, tdm_unit_gather) also
+ * take TDM_BYTES (code 6, declared with them), which covers every dtype. */
+enum tdm_dtype {
+  TDM_F32 = 0, TDM_F64 = 1, TDM_F16 = 2, TDM_BF16 = 3, TDM_I64 = 4, TDM_I32 = 5,
+  TDM_I16 = 7, TDM_I8 = 8, TDM_U8 = 9
+};
 
 enum { TDM_MAX_PAIRS = 16, TDM_MAX_WORLD = 8 };
 

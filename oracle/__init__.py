@@ -13,7 +13,12 @@ Contents, and what pins each against the reference (tests/test_oracle_*.py):
                            (outputs of the reference's Python engine), by the
                            independent step-by-step simulator ring.simulate, by
                            the n=2 identity x0/2 + x1/2 and by integer-valued
-                           inputs whose sums are exact in any order.
+                           inputs whose sums are exact in any order.  The integer
+                           kinds narrower than 64 bits wrap around: pinned by the
+                           order-free modular sum (numpy in 64 bits, reduced to the
+                           element's width) on inputs that overflow, and by ATen's
+                           own add_ on CPU tensors, which is what the reference's
+                           engines call for them (tandem/comm.py:276-277).
   adamw.AdamW              tandem/optim.py:16-37.  First and second moments pinned
                            bit for bit by tests/golden/adamw.npz; the parameter
                            update is pinned bit for bit when torch's own CPU sqrt

@@ -17,7 +17,10 @@ import numpy as np
 
 from . import lib
 
-KINDS = {"f32": np.float32, "f64": np.float64, "bf16": np.uint16, "f16": np.uint16, "i64": np.int64}
+KINDS = {"f32": np.float32, "f64": np.float64, "bf16": np.uint16, "f16": np.uint16, "i64": np.int64,
+         "i32": np.int32, "i16": np.int16, "i8": np.int8, "u8": np.uint8}
+# integer sums narrower than 64 bits wrap around; the C side adds their bit patterns as unsigned numbers of the same width
+_WRAPPING = {"i32": ("u32", np.uint32), "i16": ("u16", np.uint16), "i8": ("u8", np.uint8), "u8": ("u8", np.uint8)}
 
 
 def split_sizes(n, world):
@@ -57,11 +60,16 @@ def fold(xs, c, lo, hi, average, kind="f32", upto=None):
     upto = n if upto is None else upto
     dt = KINDS[kind]
     xs = [np.ascontiguousarray(x, dtype=dt) for x in xs]
-    out = np.empty(hi - lo, dtype=dt)
+    if kind in _WRAPPING:
+        if average:
+            raise ValueError("integer tensors are not averaged")
+        kind, as_unsigned = _WRAPPING[kind]
+        xs = [x.view(as_unsigned) for x in xs]
+    out = np.empty(hi - lo, dtype=xs[0].dtype if xs else dt)
     fn = getattr(lib(), f"orc_ring_fold_{kind}")
     fn(_ptr_array(xs), ctypes.c_int(n), ctypes.c_int(c), ctypes.c_int(upto), ctypes.c_int(int(average)),
        ctypes.c_int64(lo), ctypes.c_int64(hi), ctypes.c_void_p(out.ctypes.data))
-    return out
+    return out.view(dt)
 
 
 def expected_all_reduce(xs, average, kind="f32"):

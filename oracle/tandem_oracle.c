@@ -115,6 +115,14 @@ RING_FOLD(orc_ring_fold_f64, double, double, IDENT, IDENT, double)
 RING_FOLD(orc_ring_fold_bf16, uint16_t, float, bf16_to_f32, f32_to_bf16, float)
 RING_FOLD(orc_ring_fold_f16, uint16_t, float, f16_to_f32, f32_to_f16, float)
 RING_FOLD(orc_ring_fold_i64, int64_t, int64_t, IDENT, IDENT, int64_t)
+/* The narrower integers: ATen's add_ wraps around (the reference adds whatever dtype it is given with
+ * into.add_(slot), tandem/comm.py:276-277), so the sums are taken in unsigned arithmetic of the element's
+ * own width, which is the two's-complement sum of signed elements bit for bit. Never averaged. */
+#define TO_U16(v) ((uint16_t)(v))
+#define TO_U8(v) ((uint8_t)(v))
+RING_FOLD(orc_ring_fold_u32, uint32_t, uint32_t, IDENT, IDENT, uint32_t)
+RING_FOLD(orc_ring_fold_u16, uint16_t, uint32_t, IDENT, TO_U16, uint32_t)
+RING_FOLD(orc_ring_fold_u8, uint8_t, uint32_t, IDENT, TO_U8, uint32_t)
 
 /* Conversions exported so tests can check them against numpy / torch. */
 void orc_bf16_to_f32(const uint16_t* in, float* out, int64_t n) {

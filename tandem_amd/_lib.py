@@ -16,7 +16,8 @@ TDM_MAX_PAIRS = 16
 TDM_MAX_WORLD = 8
 ABI_VERSION = 1
 
-DTYPES = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3, torch.int64: 4, torch.int32: 5}
+DTYPES = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3, torch.int64: 4, torch.int32: 5,
+          torch.int16: 7, torch.int8: 8, torch.uint8: 9}  # 6 is TDM_BYTES: any dtype, copied only
 
 ALLREDUCE_RING = 0
 ALLREDUCE_FOLD = 1

@@ -857,7 +857,7 @@ std::vector<Engine::Chunk> Engine::chunks(const Buf& t, const std::vector<int64_
 
 std::shared_ptr<Work> Engine::all_reduce(Buf t, bool average, hipStream_t caller) {
   check(t, "all_reduce", true);
-  if (average && (t.dtype == TDM_I64 || t.dtype == TDM_I32)) throw Invalid("all_reduce: integer tensors cannot be averaged in place");
+  if (average && is_integer(t.dtype)) throw Invalid("all_reduce: integer tensors cannot be averaged in place");
   return submit([this, t, average] {
     if (size_ == 1) return;
     if (staged_ && size_ <= TDM_MAX_WORLD) {
@@ -873,7 +873,7 @@ std::shared_ptr<Work> Engine::all_reduce(Buf t, bool average, hipStream_t caller
 std::shared_ptr<Work> Engine::reduce_scatter(Buf t, std::vector<int64_t> sizes, bool average, bool owner_only,
                                              hipStream_t caller) {
   check(t, "reduce_scatter", true);
-  if (average && (t.dtype == TDM_I64 || t.dtype == TDM_I32)) throw Invalid("reduce_scatter: integer tensors cannot be averaged in place");
+  if (average && is_integer(t.dtype)) throw Invalid("reduce_scatter: integer tensors cannot be averaged in place");
   chunks(t, sizes);  // validate now, in the caller's thread
   return submit([this, t, sizes, average, owner_only] {
     if (size_ == 1) return;
@@ -1130,7 +1130,7 @@ std::shared_ptr<Work> Engine::direct(int kind, Buf t, std::vector<int64_t> sizes
   const char* what = kind == 0 ? "all_reduce (direct)" : kind == 1 ? "reduce_scatter (direct)" : "all_gather (direct)";
   check(t, what, kind != 2);
   if (t.dtype == kBytesDtype) throw Invalid(std::string(what) + ": needs a typed tensor");
-  if (kind != 2 && average && (t.dtype == TDM_I64 || t.dtype == TDM_I32)) {
+  if (kind != 2 && average && is_integer(t.dtype)) {
     throw Invalid(std::string(what) + ": integer tensors cannot be averaged in place");
   }
   if (kind != 2 && size_ > TDM_MAX_WORLD) throw Invalid(std::string(what) + ": the direct fold handles world sizes up to 8");

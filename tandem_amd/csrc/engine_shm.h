@@ -38,12 +38,16 @@ constexpr uint64_t fence_tag(int kind, int dtype, int64_t numel) {
   return (static_cast<uint64_t>(kind) << 56) | (static_cast<uint64_t>(dtype) << 48) | (static_cast<uint64_t>(numel) & ((uint64_t(1) << 48) - 1));
 }
 
+inline bool is_integer(int dtype) {
+  return dtype == TDM_I64 || dtype == TDM_I32 || dtype == TDM_I16 || dtype == TDM_I8 || dtype == TDM_U8;
+}
+
 inline int elem_bytes(int dtype) {
   switch (dtype) {
     case TDM_F32: case TDM_I32: return 4;
     case TDM_F64: case TDM_I64: return 8;
-    case TDM_F16: case TDM_BF16: return 2;
-    case kBytesDtype: return 1;
+    case TDM_F16: case TDM_BF16: case TDM_I16: return 2;
+    case TDM_I8: case TDM_U8: case kBytesDtype: return 1;
     default: throw Invalid("unknown dtype " + std::to_string(dtype));
   }
 }

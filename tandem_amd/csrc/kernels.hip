@@ -41,7 +41,8 @@ int elem_size(int dtype) {
   switch (dtype) {
     case TDM_F32: case TDM_I32: return 4;
     case TDM_F64: case TDM_I64: return 8;
-    case TDM_F16: case TDM_BF16: return 2;
+    case TDM_F16: case TDM_BF16: case TDM_I16: return 2;
+    case TDM_I8: case TDM_U8: return 1;
     default: return 0;
   }
 }
@@ -203,10 +204,14 @@ template <typename T, int kMask>
 void launch_reduce_m(const PairTable& tab, int64_t tiles, int world, bool any_scale, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(world);
   const dim3 grid(grid_for(tiles)), block(kThreads);
-  switch (div_kind(world, any_scale)) {
-    case 0: hipLaunchKernelGGL((k1_reduce_kernel<T, 0, kMask>), grid, block, 0, stream, tab, dv); break;
-    case 1: hipLaunchKernelGGL((k1_reduce_kernel<T, 1, kMask>), grid, block, 0, stream, tab, dv); break;
-    default: hipLaunchKernelGGL((k1_reduce_kernel<T, 2, kMask>), grid, block, 0, stream, tab, dv); break;
+  if constexpr (!Elem<T>::floating) {  // integers are never divided: only this kernel is built for them
+    hipLaunchKernelGGL((k1_reduce_kernel<T, 0, kMask>), grid, block, 0, stream, tab, dv);
+  } else {
+    switch (div_kind(world, any_scale)) {
+      case 0: hipLaunchKernelGGL((k1_reduce_kernel<T, 0, kMask>), grid, block, 0, stream, tab, dv); break;
+      case 1: hipLaunchKernelGGL((k1_reduce_kernel<T, 1, kMask>), grid, block, 0, stream, tab, dv); break;
+      default: hipLaunchKernelGGL((k1_reduce_kernel<T, 2, kMask>), grid, block, 0, stream, tab, dv); break;
+    }
   }
 }
 
@@ -235,10 +240,14 @@ template <typename T, int kMask>
 void launch_copy_m(const PairTable& tab, int64_t tiles, int world, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(world);
   const dim3 grid(grid_for(tiles)), block(kCopyThreads);
-  switch (div_kind(world, true)) {
-    case 0: hipLaunchKernelGGL((k1_copy_kernel<T, 0, kMask>), grid, block, 0, stream, tab, dv); break;
-    case 1: hipLaunchKernelGGL((k1_copy_kernel<T, 1, kMask>), grid, block, 0, stream, tab, dv); break;
-    default: hipLaunchKernelGGL((k1_copy_kernel<T, 2, kMask>), grid, block, 0, stream, tab, dv); break;
+  if constexpr (!Elem<T>::floating) {
+    hipLaunchKernelGGL((k1_copy_kernel<T, 0, kMask>), grid, block, 0, stream, tab, dv);
+  } else {
+    switch (div_kind(world, true)) {
+      case 0: hipLaunchKernelGGL((k1_copy_kernel<T, 0, kMask>), grid, block, 0, stream, tab, dv); break;
+      case 1: hipLaunchKernelGGL((k1_copy_kernel<T, 1, kMask>), grid, block, 0, stream, tab, dv); break;
+      default: hipLaunchKernelGGL((k1_copy_kernel<T, 2, kMask>), grid, block, 0, stream, tab, dv); break;
+    }
   }
 }
 
@@ -266,10 +275,14 @@ void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t st
   const Divisor<T> dv = make_divisor<T>(kWorld);
   const dim3 grid(grid_for(tiles * FoldShape<kWorld>::kParts)), block(FoldShape<kWorld>::kT);
   const FoldSegDev* img = static_cast<const FoldSegDev*>(image);
-  switch (div_kind(kWorld, average != 0)) {
-    case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, occupancy_pad(TDM_XCD_FOLD_TABLE), stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
-    case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1, kAcc>), grid, block, occupancy_pad(TDM_XCD_FOLD_TABLE), stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
-    default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2, kAcc>), grid, block, occupancy_pad(TDM_XCD_FOLD_TABLE), stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
+  if constexpr (!Elem<T>::floating) {
+    hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, occupancy_pad(TDM_XCD_FOLD_TABLE), stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true));
+  } else {
+    switch (div_kind(kWorld, average != 0)) {
+      case 0: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 0, kAcc>), grid, block, occupancy_pad(TDM_XCD_FOLD_TABLE), stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
+      case 1: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 1, kAcc>), grid, block, occupancy_pad(TDM_XCD_FOLD_TABLE), stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
+      default: hipLaunchKernelGGL((k2_fold_kernel<T, kWorld, 2, kAcc>), grid, block, occupancy_pad(TDM_XCD_FOLD_TABLE), stream, img, tiles, dv, xcd_shift(TDM_XCD_FOLD_TABLE, kWorld, true)); break;
+    }
   }
 }
 
@@ -281,13 +294,18 @@ void launch_fold_small_w(const FoldSmall& table, int average, hipStream_t stream
   const dim3 grid(grid_for(table.tile_end[table.nseg - 1] * (cold ? fold_small_parts<kWorld>() : 1))), block(kThreads);
   FoldSmall tab = table;
   tab.shift = xcd_shift(TDM_XCD_FOLD, kWorld, table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld >= kColdFootprint);
-  switch (div_kind(kWorld, average != 0) * 2 + (cold ? 1 : 0)) {
-    case 0: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
-    case 1: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
-    case 2: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
-    case 3: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
-    case 4: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
-    default: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+  if constexpr (!Elem<T>::floating) {
+    if (cold) hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv);
+    else hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv);
+  } else {
+    switch (div_kind(kWorld, average != 0) * 2 + (cold ? 1 : 0)) {
+      case 0: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+      case 1: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+      case 2: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+      case 3: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+      case 4: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+      default: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 2, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
+    }
   }
 }
 
@@ -430,7 +448,9 @@ void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool s
     case TDM_F16: launch_reduce<f16_t>(tab, tiles, world, any_scale, policy, stream); break;
     case TDM_BF16: launch_reduce<bf16_t>(tab, tiles, world, any_scale, policy, stream); break;
     case TDM_I64: launch_reduce<int64_t>(tab, tiles, 1, false, policy, stream); break;
-    default: launch_reduce<int32_t>(tab, tiles, 1, false, policy, stream); break;
+    case TDM_I32: launch_reduce<int32_t>(tab, tiles, 1, false, policy, stream); break;
+    case TDM_I16: launch_reduce<int16_t>(tab, tiles, 1, false, policy, stream); break;
+    default: launch_reduce<int8_t>(tab, tiles, 1, false, policy, stream); break;  // TDM_I8 and TDM_U8: the same bits
   }
   check_hip(hipGetLastError(), "k1_reduce launch");
 }
@@ -464,7 +484,9 @@ void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStrea
     case TDM_F16: launch_copy<f16_t>(tab, tiles, world, policy, stream); break;
     case TDM_BF16: launch_copy<bf16_t>(tab, tiles, world, policy, stream); break;
     case TDM_I64: launch_copy<int64_t>(tab, tiles, 1, policy, stream); break;
-    default: launch_copy<int32_t>(tab, tiles, 1, policy, stream); break;
+    case TDM_I32: launch_copy<int32_t>(tab, tiles, 1, policy, stream); break;
+    case TDM_I16: launch_copy<int16_t>(tab, tiles, 1, policy, stream); break;
+    default: launch_copy<int8_t>(tab, tiles, 1, policy, stream); break;
   }
   check_hip(hipGetLastError(), "k1_copy launch");
 }
@@ -710,7 +732,9 @@ void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool av
     case TDM_F16: launch_fold_small<f16_t>(tab, world, average, stream); break;
     case TDM_BF16: launch_fold_small<bf16_t>(tab, world, average, stream); break;
     case TDM_I64: launch_fold_small<int64_t>(tab, world, 0, stream); break;
-    default: launch_fold_small<int32_t>(tab, world, 0, stream); break;
+    case TDM_I32: launch_fold_small<int32_t>(tab, world, 0, stream); break;
+    case TDM_I16: launch_fold_small<int16_t>(tab, world, 0, stream); break;
+    default: launch_fold_small<int8_t>(tab, world, 0, stream); break;
   }
   check_hip(hipGetLastError(), "k2_fold_small launch");
 }
@@ -900,6 +924,8 @@ void bucket_fold(const void* table_dev, int64_t ntiles, int dtype, int world, in
     case TDM_BF16: launch_fold<bf16_t>(table_dev, ntiles, world, average, accumulate != 0, st); break;
     case TDM_I64: launch_fold<int64_t>(table_dev, ntiles, world, 0, accumulate != 0, st); break;
     case TDM_I32: launch_fold<int32_t>(table_dev, ntiles, world, 0, accumulate != 0, st); break;
+    case TDM_I16: launch_fold<int16_t>(table_dev, ntiles, world, 0, accumulate != 0, st); break;
+    case TDM_I8: case TDM_U8: launch_fold<int8_t>(table_dev, ntiles, world, 0, accumulate != 0, st); break;
     default: throw Invalid("unknown dtype " + std::to_string(dtype));
   }
   check_hip(hipGetLastError(), "k2_fold launch");

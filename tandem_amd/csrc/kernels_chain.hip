@@ -302,6 +302,8 @@ void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* l
     case TDM_BF16: launch_chain<bf16_t>(tab, world, average, grid, cold, pad, stream); break;
     case TDM_I64: launch_chain<int64_t>(tab, world, false, grid, cold, pad, stream); break;
     case TDM_I32: launch_chain<int32_t>(tab, world, false, grid, cold, pad, stream); break;
+    case TDM_I16: launch_chain<int16_t>(tab, world, false, grid, cold, pad, stream); break;
+    case TDM_I8: case TDM_U8: launch_chain<int8_t>(tab, world, false, grid, cold, pad, stream); break;
     default: throw Invalid("unknown dtype " + std::to_string(dtype));
   }
   check_hip(hipGetLastError(), "k1_chain launch");

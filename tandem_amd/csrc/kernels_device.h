@@ -113,6 +113,20 @@ template <> struct Elem<int32_t> {
   static __device__ __forceinline__ acc widen(int32_t x) { return x; }
   static __device__ __forceinline__ int32_t narrow(acc x) { return x; }
 };
+// Narrow integers add in 32 bits and keep the low bits: the wrap-around sum of the element's own width,
+// whatever the order of the terms. uint8 shares int8's kernels: the bits of the two sums are the same.
+template <> struct Elem<int16_t> {
+  using acc = int32_t;
+  static constexpr bool floating = false;
+  static __device__ __forceinline__ acc widen(int16_t x) { return x; }
+  static __device__ __forceinline__ int16_t narrow(acc x) { return static_cast<int16_t>(static_cast<uint16_t>(x)); }
+};
+template <> struct Elem<int8_t> {
+  using acc = int32_t;
+  static constexpr bool floating = false;
+  static __device__ __forceinline__ acc widen(int8_t x) { return x; }
+  static __device__ __forceinline__ int8_t narrow(acc x) { return static_cast<int8_t>(static_cast<uint8_t>(x)); }
+};
 template <> struct Elem<f16_t> {
   using acc = float;
   static constexpr bool floating = true;

@@ -31,7 +31,8 @@ for _name in ("tdm_engine_connect", "tdm_engine_close", "tdm_engine_destroy", "t
     getattr(_L, _name).argtypes = [_VP]
 
 cuda = True  # what tandem/comm.py reads from the native module to know it can take GPU tensors
-DTYPE = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3, torch.int64: 4, torch.int32: 5}
+DTYPE = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3, torch.int64: 4, torch.int32: 5,
+         torch.int16: 7, torch.int8: 8, torch.uint8: 9}
 BYTES = 6  # tensors that are only copied (all_gather, broadcast, send/recv) may have any dtype: they travel as bytes
 ERRORS = {1: ValueError, 2: RuntimeError, 3: TimeoutError}  # as tandem/csrc/engine.cpp:54-55 translates its exceptions
 

@@ -31,7 +31,7 @@ def seeded(seed, rank, n, scale=1.0):
 def bits(a):
     """Bit pattern view for exact comparison (distinguishes -0.0 from 0.0, NaNs)."""
     a = np.ascontiguousarray(a)
-    return a.view({2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize])
+    return a.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize])
 
 
 class OracleShardedAdamW:

@@ -203,3 +203,40 @@ def test_bucket_fold_into_other_buffers_and_odd_sizes(dev):
                 assert np.array_equal(bits(outs[r][i].cpu().numpy()), bits(want[off:off + numels[i]]))
                 assert torch.equal(dgrads[r][i].cpu(), grads[r][i])  # sources untouched
             off += numels[i]
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.bfloat16, torch.float16, torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8])
+def test_bucket_fold_of_every_element_type(dev, dtype):
+    """The table-driven fold over the other element types the header names: odd tensor sizes, so most
+    segments start off the 16-byte grid; integers over their whole range, so their sums wrap around."""
+    from oracle import ring
+    from tandem_amd import LocalWorld
+
+    kind = {torch.float64: "f64", torch.bfloat16: "bf16", torch.float16: "f16", torch.int64: "i64", torch.int32: "i32",
+            torch.int16: "i16", torch.int8: "i8", torch.uint8: "u8"}[dtype]
+    world = 3
+    numels = [1, 3, 1025, 7, 4096, 10_007, 2, 33]
+    def make(r, i, n):
+        if dtype.is_floating_point:
+            return seeded(r + 11, i, n).to(dtype)
+        g = torch.Generator().manual_seed(100 * r + i)
+        if dtype == torch.int64:
+            return torch.randint(-(1 << 40), 1 << 40, (n,), generator=g)
+        info = torch.iinfo(dtype)
+        return torch.randint(info.min, info.max + 1, (n,), generator=g).to(dtype)
+    def raw(t):
+        t = t.cpu()
+        return t.view(torch.int16).numpy().view(np.uint16) if dtype in (torch.bfloat16, torch.float16) else t.numpy()
+    grads = [[make(r, i, n) for i, n in enumerate(numels)] for r in range(world)]
+    dgrads = [[t.to(dev) for t in grads[r]] for r in range(world)]
+    buckets = [[7, 6, 5], [4, 3], [2, 1, 0]]
+    average = dtype.is_floating_point
+    LocalWorld(world).bucket_table(dgrads, buckets).run(average=average)
+    for b in buckets:
+        flat = [np.concatenate([raw(grads[r][i]) for i in b]) for r in range(world)]
+        want = ring.expected_all_reduce(flat, average, kind)
+        off = 0
+        for i in b:
+            for r in range(world):
+                assert np.array_equal(bits(raw(dgrads[r][i])), bits(want[off:off + numels[i]])), (dtype, i, r)
+            off += numels[i]

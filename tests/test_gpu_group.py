@@ -13,7 +13,8 @@ from helpers import bits, golden_npz, npz_json, seeded
 
 pytestmark = pytest.mark.gpu
 
-KINDS = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16", torch.int64: "i64"}
+KINDS = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16", torch.int64: "i64",
+         torch.int32: "i32", torch.int16: "i16", torch.int8: "i8", torch.uint8: "u8"}
 TIMEOUT = 60.0
 
 
@@ -28,7 +29,10 @@ def values(rank, n, dtype):
     g = torch.Generator().manual_seed(1234 + rank)
     if dtype.is_floating_point:
         return torch.randn(n, generator=g).to(dtype)
-    return torch.randint(-1000, 1000, (n,), generator=g).to(dtype)
+    if dtype == torch.int64:
+        return torch.randint(-1000, 1000, (n,), generator=g)
+    info = torch.iinfo(dtype)  # the narrower integers over their whole range: most sums wrap around
+    return torch.randint(info.min, info.max + 1, (n,), generator=g).to(dtype)
 
 
 def collectives(g, dtype, n):
@@ -65,10 +69,10 @@ def collectives(g, dtype, n):
         got = torch.empty(n, dtype=dtype, device=dev)
         g.sendrecv(x, 1 - r, got, 1 - r)
         out["sendrecv"] = got.cpu()
-    codes = torch.zeros(n, dtype=torch.uint8, device=dev)  # a dtype the kernels do not know: gathered as bytes
-    codes[lo:lo + sizes[r]] = r + 1
+    codes = torch.zeros(n, dtype=torch.complex64, device=dev)  # a dtype the kernels do not know: gathered as bytes
+    codes[lo:lo + sizes[r]] = complex(r + 1, -r)
     g.all_gather(codes, sizes)
-    out["bytes_ag_ok"] = bool(torch.equal(codes.cpu(), torch.cat([torch.full((sizes[q],), q + 1, dtype=torch.uint8) for q in range(w)])))
+    out["bytes_ag_ok"] = bool(torch.equal(codes.cpu(), torch.cat([torch.full((sizes[q],), complex(q + 1, -q), dtype=torch.complex64) for q in range(w)])))
     flags = torch.arange(n, device=dev) % 2 == 0  # bool: copied as bytes
     if r != 0:
         flags = torch.zeros_like(flags)
@@ -149,11 +153,11 @@ def test_collectives_bit_exact(world, algo, monkeypatch):
     from oracle import ring
     from tandem_amd import launch
 
-    dtypes = [torch.float32, torch.bfloat16, torch.float16, torch.int64, torch.float64]
+    dtypes = [torch.float32, torch.bfloat16, torch.float16, torch.int64, torch.float64, torch.int32, torch.int16, torch.int8, torch.uint8]
     if world == 4:
-        dtypes = [torch.float32, torch.bfloat16, torch.int64]
+        dtypes = [torch.float32, torch.bfloat16, torch.int64, torch.int16, torch.uint8]
     elif world == 3 and algo not in ("small", "staged"):
-        dtypes = [torch.float32, torch.bfloat16]
+        dtypes = [torch.float32, torch.bfloat16, torch.int8]
     choose(monkeypatch, algo)
     n = 10_007
     res = launch(collectives_of, world, dtypes, n, slot_bytes=4096, gpus=[0] * world, timeout=TIMEOUT)
@@ -554,25 +558,25 @@ def errors(g):
                 lambda: g.all_reduce(torch.zeros(4, device=g.device), op="max"),
                 lambda: g.reduce_scatter(torch.zeros(10, device=g.device), [5, 6]),
                 lambda: g.all_reduce(torch.zeros(4, device=g.device, dtype=torch.int64), op="avg"),
-                lambda: g.all_reduce(torch.zeros(4, device=g.device, dtype=torch.uint8))):
+                lambda: g.all_reduce(torch.zeros(4, device=g.device, dtype=torch.bool))):
         try:
             bad()
             seen.append(False)
         except CommError:
             seen.append(True)
-    # Sums of dtypes outside the six the kernels know are refused by name, where the reference's engine
+    # Sums of dtypes outside the nine the kernels know are refused by name, where the reference's engine
     # falls back to add_ (tandem/csrc/collectives.cpp:254-256 there); copying them works, as bytes.
     texts = []
-    for dtype in (torch.int8, torch.uint8, torch.int16, torch.bool):
+    for dtype in (torch.bool, torch.complex64, torch.uint16):
         for call in (g.all_reduce, g.reduce_scatter):
             try:
                 call(torch.zeros(8, device=g.device, dtype=dtype))
                 texts.append("accepted")
             except CommError as e:
                 texts.append(str(e))
-        t = torch.full((8,), g.rank + 1, device=g.device).to(dtype)
+        t = torch.full((8,), g.rank + 1).to(dtype).to(g.device)
         g.broadcast(t, root=1)
-        texts.append(bool((t == torch.tensor(2).to(dtype)).all()))
+        texts.append(bool(torch.equal(t.cpu().view(torch.uint8), torch.full((8,), 2).to(dtype).view(torch.uint8))))
     g.barrier()
     return seen, texts
 
@@ -582,7 +586,7 @@ def test_errors_surface_as_commerror():
 
     for seen, texts in launch(errors, 2, gpus=[0, 0], timeout=TIMEOUT):
         assert seen == [True] * 6
-        for k, dtype in enumerate(("torch.int8", "torch.uint8", "torch.int16", "torch.bool")):
+        for k, dtype in enumerate(("torch.bool", "torch.complex64", "torch.uint16")):
             assert texts[3 * k] == texts[3 * k + 1] == f"the hip backend cannot reduce {dtype}", texts[3 * k]
             assert texts[3 * k + 2] is True
 

@@ -10,7 +10,8 @@ from helpers import bits, golden_npz, npz_json, seeded
 
 pytestmark = pytest.mark.gpu
 
-KINDS = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16", torch.int64: "i64"}
+KINDS = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16", torch.int64: "i64",
+         torch.int32: "i32", torch.int16: "i16", torch.int8: "i8", torch.uint8: "u8"}
 
 
 def to_np(t):
@@ -49,6 +50,9 @@ def inputs(world, n, dtype, seed=0):
         if dtype == torch.int64:
             g = torch.Generator().manual_seed(seed * 1000 + r)
             xs.append(torch.randint(-1000, 1000, (n,), generator=g))
+        elif not dtype.is_floating_point:  # the narrower integers over their whole range: most sums wrap around
+            g, info = torch.Generator().manual_seed(seed * 1000 + r), torch.iinfo(dtype)
+            xs.append(torch.randint(info.min, info.max + 1, (n,), generator=g).to(dtype))
         else:
             xs.append(seeded(seed, r, n).to(dtype))
     return xs
@@ -145,6 +149,53 @@ def test_against_oracle(dev, world, dtype):
         want = ring.expected_all_gather(xn, sizes)
         for r in range(world):
             assert np.array_equal(bits(to_np(bufs[r])), bits(want))
+
+
+@pytest.mark.parametrize("world", [2, 3, 4, 8])
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int16, torch.int8, torch.uint8])
+def test_integer_sums_wrap_around(dev, world, dtype):
+    """The integer types narrower than 64 bits: sums wrap around as ATen's add_ does (what the
+    reference's engines call for them: tandem/comm.py:276-277, tandem/csrc/collectives.cpp:254-256
+    there), partial sums included; averaging them is refused. Also from views that start off the
+    16-byte grid, where 1-byte elements have up to 15 head elements."""
+    from oracle import ring
+    from tandem_amd import LocalWorld
+
+    kind = KINDS[dtype]
+    lw = LocalWorld(world)
+    for n, shift in ((0, 0), (1, 0), (5, 3), (1000, 0), (4099, 1), (65_536 + 3, 0), (65_536 + 35, 13)):
+        xs = inputs(world, n, dtype, seed=3)
+        xn = [to_np(x) for x in xs]
+        def on_device():
+            if shift == 0:
+                return [x.to(dev) for x in xs]
+            backing = [torch.zeros(n + 64, dtype=dtype, device=dev) for _ in xs]
+            views = [b[shift:shift + n] for b in backing]
+            for v, x in zip(views, xs):
+                v.copy_(x)
+            return views
+        want = ring.expected_all_reduce(xn, False, kind)
+        assert np.array_equal(want, sum(x.astype(np.int64) for x in xn).astype(want.dtype) if n else want)  # the order-free modular sum
+        for algorithm in ("ring", "fold"):
+            bufs = on_device()
+            lw.all_reduce(bufs, algorithm=algorithm)
+            for r in range(world):
+                assert np.array_equal(to_np(bufs[r]), want), (world, dtype, n, shift, algorithm, r)
+        sizes = [n // world] * world
+        sizes[-1] += n - sum(sizes)
+        sizes = sizes[1:] + sizes[:1]
+        bufs = on_device()
+        lw.reduce_scatter(bufs, sizes)
+        want = ring.expected_reduce_scatter(xn, sizes, False, kind)
+        for r in range(world):
+            assert np.array_equal(to_np(bufs[r]), want[r]), (world, dtype, n, shift, r)
+        bufs = on_device()
+        lw.all_gather(bufs, sizes)
+        want = ring.expected_all_gather(xn, sizes)
+        for r in range(world):
+            assert np.array_equal(to_np(bufs[r]), want)
+    with pytest.raises(ValueError, match="cannot be averaged"):
+        lw.all_reduce([torch.zeros(8, dtype=dtype, device=dev) for _ in range(world)], op="avg")
 
 
 def test_unaligned_views_and_special_values(dev):

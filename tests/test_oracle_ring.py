@@ -115,6 +115,41 @@ def test_integer_valued_inputs_sum_exactly(world):
         assert np.array_equal(ring.expected_all_reduce(xi, False, "i64"), want.astype(np.int64))
 
 
+@pytest.mark.parametrize("kind", ["i32", "i16", "i8", "u8"])
+@pytest.mark.parametrize("world", [2, 3, 4, 8])
+def test_narrow_integer_sums_wrap_around(kind, world):
+    """Full-range inputs, so most sums overflow. Two independent statements of the result: the
+    sum in 64 bits reduced to the element's width (order-free), and ATen's add_ applied in the
+    ring's order on CPU tensors, which is what the reference's engines do for these dtypes
+    (tandem/comm.py:276-277; tandem/csrc/collectives.cpp:254-256)."""
+    import torch
+
+    dt = ring.KINDS[kind]
+    info = np.iinfo(dt)
+    rng = np.random.default_rng(world * 10 + len(kind))
+    for n in (0, 1, 5, 1000, 4099):
+        xs = [rng.integers(info.min, int(info.max) + 1, n, dtype=np.int64).astype(dt) for _ in range(world)]
+        modular = sum(x.astype(np.int64) for x in xs).astype(dt) if n else np.zeros(0, dt)  # astype keeps the low bits
+        got = ring.expected_all_reduce(xs, False, kind)
+        assert got.dtype == dt and np.array_equal(got, modular)
+        sizes = [n // world] * world
+        sizes[0] += n - sum(sizes)
+        outs = ring.expected_reduce_scatter(xs, sizes, False, kind)
+        sim = ring.simulate(xs, "reduce_scatter", sizes, False, kind, piece_elems=7)
+        lo = 0
+        for c, size in enumerate(sizes):
+            acc = torch.from_numpy(xs[(c + 1) % world][lo:lo + size].copy())
+            for k in range(2, world + 1):
+                r = (c + k) % world
+                acc = torch.from_numpy(xs[r][lo:lo + size].copy()).add_(acc)  # into.add_(slot) on rank r
+                assert np.array_equal(outs[r][lo:lo + size], acc.numpy()), (kind, world, n, c, k)
+            lo += size
+        for r in range(world):
+            assert np.array_equal(outs[r], sim[r])
+    with pytest.raises(ValueError):
+        ring.expected_all_reduce([np.zeros(4, dt)] * 2, True, kind)
+
+
 def test_power_of_two_scaling_commutes_with_the_ring():
     # scaling every input by 2^k scales every partial sum exactly (no overflow here)
     xs = [seeded(9, r, 777).numpy() for r in range(4)]
