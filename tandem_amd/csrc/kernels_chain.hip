@@ -1,5 +1,5 @@
-// The ring reduce-scatter of a whole group in ONE launch, for ranks that are buffers of one
-// process and a footprint that stays in the caches.
+// The ring reduce-scatter of a whole group in ONE launch, and its all-gather in one more, for ranks
+// that are buffers of one process.
 //
 // The ring's W-1 steps (tandem/comm.py:301-305 in the reference) pass chunk c round the ring:
 // rank c+1 sends it, rank c+2 adds its own and sends the sum on, ..., rank c adds last. Every
@@ -10,8 +10,8 @@
 // reads the W ranks' copies once, and stores the partial sum after k terms into rank c+k's copy,
 // which leaves memory bit for bit as the W-1 launches of the step kernel do, with W reads and
 // W-1 (keep_sent: W) writes of 4 bytes per element instead of 3 (W-1) (+1) accesses.
-// The ring steps remain the form for footprints beyond the caches, where their per-step cache
-// policies win.
+// Within the caches everything is loaded and stored plainly, 4 KiB of every stream per workgroup;
+// beyond them non-temporally, 2 KiB per workgroup (the caller says which).
 
 #include <hip/hip_runtime.h>
 
