@@ -117,3 +117,155 @@ def test_seeded_sweep(form):
             guards_intact(stores)
     finally:
         assert lib().tdm_set_ring_form(-1) == 0
+
+
+def bucket_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    dtypes = list(KINDS)
+    for k in range(count):
+        world = int(rng.integers(1, 9))
+        dtype = dtypes[int(rng.integers(len(dtypes)))]
+        numels = [int(rng.choice([1, 2, 3, 7, 33, 255, 1024, 4097, 9000])) + int(rng.integers(0, 2)) for _ in range(int(rng.integers(1, 13)))]
+        order = rng.permutation(len(numels)).tolist()
+        buckets, at = [], 0
+        while at < len(order):
+            take = int(rng.integers(1, 5))
+            buckets.append(order[at:at + take])
+            at += take
+        starts = [[int(rng.integers(0, GUARD)) for _ in numels] for _ in range(world)]  # every tensor of every rank at a phase of its own
+        yield k, world, dtype, numels, buckets, starts, bool(rng.random() < 0.4), bool(rng.random() < 0.5), int(rng.integers(1 << 30))
+
+
+def test_seeded_sweep_of_bucket_tables():
+    """The table-driven fold (DDP's buckets in one launch): random tensor lists cut into random buckets, world sizes
+    1..8, every element type, tensors that start anywhere in their allocations, in place or into other tensors, through
+    the table on the device and through the entry point that allocates nothing. Per bucket: the ring all-reduce of the
+    flattened bucket."""
+    from oracle import ring
+    from tandem_amd import LocalWorld
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    dev = torch.device("cuda", 0)
+    for k, world, dtype, numels, buckets, starts, elsewhere, static, seed in bucket_cases(150, 77):
+        kind = KINDS[dtype]
+        rng = np.random.default_rng(seed)
+        grads = [[draw(rng, dtype, n) for n in numels] for _ in range(world)]
+        marker = draw(rng, dtype, 1)
+
+        def place(fill):
+            stores, views = [], []
+            for r in range(world):
+                row_s, row_v = [], []
+                for i, n in enumerate(numels):
+                    st = marker.repeat(n + 2 * GUARD).to(dev)
+                    v = st[starts[r][i]:starts[r][i] + n]
+                    if fill:
+                        v.copy_(grads[r][i])
+                    row_s.append(st)
+                    row_v.append(v)
+                stores.append(row_s)
+                views.append(row_v)
+            return stores, views
+
+        stores, views = place(True)
+        out_stores, outs = place(False) if elsewhere else (stores, views)
+        table = LocalWorld(world).bucket_table(views, buckets, outs if elsewhere else None)
+        average = dtype.is_floating_point
+        (table.run_static if static else table.run)(average=average)
+        label = (k, world, str(dtype), numels, buckets, elsewhere, static)
+        for b in buckets:
+            flat = [np.concatenate([raw(grads[r][i]) for i in b]) for r in range(world)]
+            want = ring.expected_all_reduce(flat, average, kind)
+            off = 0
+            for i in b:
+                for r in range(world):
+                    assert np.array_equal(bits(raw(outs[r][i])), bits(want[off:off + numels[i]])), (label, i, r)
+                    if elsewhere:
+                        assert np.array_equal(bits(raw(views[r][i])), bits(raw(grads[r][i]))), (label, "source changed", i, r)
+                off += numels[i]
+        m = bits(raw(marker))[0]
+        for r in range(world):
+            for i, n in enumerate(numels):
+                host = bits(raw(out_stores[r][i]))
+                lo = starts[r][i]
+                assert (host[:lo] == m).all() and (host[lo + n:] == m).all(), (label, "guard", i, r)
+
+
+def test_seeded_sweep_of_adamw_shards():
+    """K3 on shards of random length whose parameter and gradient views start at phases of their own
+    (0..3 elements past a 16-byte boundary), random hyper-parameters (both lerp branches, with and
+    without decay), a few steps each: parameters and both moments bit for bit the oracle's."""
+    from oracle.adamw import AdamW as Oracle
+    from tandem_amd import ShardedAdamW
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    dev = torch.device("cuda", 0)
+    rng = np.random.default_rng(4242)
+    for k in range(80):
+        n = int(rng.choice([0, 1, 3, 4, 5, 127, 128, 129, 1000, 4097, 33_333, 70_000])) + int(rng.integers(0, 2))
+        kw = dict(lr=float(10 ** rng.uniform(-4, -1.5)), betas=(float(rng.choice([0.0, 0.3, 0.5, 0.9])), float(rng.choice([0.7, 0.95, 0.999]))),
+                  eps=float(rng.choice([1e-8, 1e-6])), weight_decay=float(rng.choice([0.0, 0.01, 0.1, 0.5])))
+        ps, gs = int(rng.integers(0, 4)), int(rng.integers(0, 4))
+        ours, ref = ShardedAdamW(**kw), Oracle(**kw)
+        p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+        pstore = torch.full((n + 8,), 7.0, device=dev)
+        p = pstore[ps:ps + n]
+        p.copy_(torch.from_numpy(p0))
+        pn = p0.copy()
+        steps = int(rng.integers(1, 5))
+        for _ in range(steps):
+            g0 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+            g0[: n // 7] = 0.0
+            gstore = torch.full((n + 8,), -3.0, device=dev)
+            g = gstore[gs:gs + n]
+            g.copy_(torch.from_numpy(g0))
+            ours.update("k", p, g)
+            ref.update("k", pn, g0)
+            assert np.array_equal(g.cpu().numpy(), g0) and float(gstore[:gs].sum()) == -3.0 * gs  # the gradient is only read
+        label = (k, n, kw, ps, gs, steps)
+        assert np.array_equal(bits(p.cpu().numpy()), bits(pn)), label
+        if n:
+            _, m, v = ours.state["k"]
+            assert np.array_equal(bits(m.cpu().numpy()), bits(ref.state["k"][1])), label
+            assert np.array_equal(bits(v.cpu().numpy()), bits(ref.state["k"][2])), label
+        host = pstore.cpu().numpy()
+        assert (host[:ps] == 7.0).all() and (host[ps + n:] == 7.0).all(), label
+
+
+def test_seeded_sweep_of_zero2_steps():
+    """ZeRO-2 for a whole group on one GPU over random parameter lists, world sizes 1..8 and bucket sizes: the three
+    ways through a step (ring steps + AdamW + ring all-gather; the fold + AdamW writing every copy; everything in one
+    launch) must leave the same bits in every rank's parameters and optimizer state, two steps running."""
+    from tandem_amd.local import LocalZeRO2
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    dev = torch.device("cuda", 0)
+    rng = np.random.default_rng(9)
+    kw = dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    for k in range(40):
+        world = int(rng.integers(1, 9))
+        numels = [int(rng.choice([1, 2, 5, 64, 257, 1024, 3001, 8192])) + int(rng.integers(0, 2)) for _ in range(int(rng.integers(1, 10)))]
+        bucket_bytes = int(rng.choice([64, 1024, 4096, 1 << 20]))
+        n = sum(numels)
+        zs = [LocalZeRO2(world, numels, dev, bucket_bytes=bucket_bytes, **kw) for _ in range(3)]
+        p0 = torch.from_numpy((rng.standard_normal(n) * 0.02).astype(np.float32)).to(dev)
+        for z in zs:
+            for b in z.bufs:
+                b.copy_(p0)
+        for step in range(2):
+            for r in range(world):
+                g = torch.from_numpy((rng.standard_normal(n) * 1e-3).astype(np.float32)).to(dev)
+                for z in zs:
+                    z.staging[r].copy_(g)
+            zs[0].reduce_grads("ring"); zs[0].step(fused_gather=False); zs[0].zero_grad()
+            zs[1].reduce_grads("fold"); zs[1].step(); zs[1].zero_grad()
+            zs[2].reduce_and_step(); zs[2].zero_grad()
+        label = (k, world, numels, bucket_bytes)
+        for other in zs[1:]:
+            for r in range(world):
+                assert torch.equal(zs[0].bufs[r].view(torch.int32), other.bufs[r].view(torch.int32)), label
+                if zs[0].grad_shards[r].numel():
+                    for i in (1, 2):
+                        assert torch.equal(zs[0].opts[r].state["flat"][i].view(torch.int32), other.opts[r].state["flat"][i].view(torch.int32)), (label, r, i)
+        for r in range(1, world):
+            assert torch.equal(zs[2].bufs[0].view(torch.int32), zs[2].bufs[r].view(torch.int32)), label
