@@ -165,3 +165,43 @@ def test_refuses_more_than_the_fixed_table_and_bad_segments():
     assert lib().tdm_k2_bucket_fold_static(segs, 1, 2, 0, 1, 0, stream_ptr(dev)) == 1
     assert "chunk outside" in lib().tdm_last_error().decode()
     assert lib().tdm_k2_bucket_fold_static(segs, 0, 2, 0, 1, 0, stream_ptr(dev)) == 0  # nothing to do
+
+
+def test_replayed_from_a_hip_graph():
+    """The reason the entry point exists: a caller under HIP graph capture cannot allocate. Captured once (after one
+    eager call, which looks the fixed table's address up), replayed three times over new gradients with eager work
+    and a host wait between the replays: every replay's bits are those of the table entry point run eagerly."""
+    from tandem_amd import LocalWorld
+
+    dev = torch.device("cuda", 0)
+    world = 4
+    numels = [70_001, 9, 2048, 4099, 33, 1, 300_000] * 3  # 21 tensors: two launches of the fill kernel, then the fold
+    buckets = [list(range(k, min(k + 4, len(numels)))) for k in range(0, len(numels), 4)]
+    gen = torch.Generator().manual_seed(5)
+    ins = [[[torch.randn(m, generator=gen) * 1e-3 for m in numels] for _ in range(world)] for _ in range(4)]
+    grads = [[torch.empty(m, device=dev) for m in numels] for _ in range(world)]
+    other = [[torch.empty(m, device=dev) for m in numels] for _ in range(world)]
+    lw = LocalWorld(world)
+    static, eager = lw.bucket_table(grads, buckets), lw.bucket_table(other, buckets)
+
+    def load(k):
+        for r in range(world):
+            for i in range(len(numels)):
+                grads[r][i].copy_(ins[k][r][i])
+                other[r][i].copy_(ins[k][r][i])
+
+    load(0)
+    static.run_static(average=True)  # outside the capture
+    torch.cuda.synchronize(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static.run_static(average=True)
+    for k in range(1, 4):
+        load(k)
+        graph.replay()
+        eager.run(average=True)  # behind the replay on the same stream
+        torch.cuda.synchronize(dev)
+        for r in range(world):
+            for i in range(len(numels)):
+                assert np.array_equal(bits(grads[r][i].cpu().numpy()), bits(other[r][i].cpu().numpy())), (k, r, i)
+        assert not torch.equal(grads[0][0].cpu(), ins[k][0][0])  # (the fold did run)
