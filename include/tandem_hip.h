@@ -64,7 +64,9 @@ int tdm_abi_version(void);
 int tdm_device_info(int device, char* name, int name_len, int* compute_units, int64_t* total_bytes);
 
 /* Launch geometry knob for measurements: workgroups per compute unit used by the
- * streaming kernels (0 restores the built-in default). Not needed for correctness; the reference has no counterpart. */
+ * streaming kernels before their grids start to stride, 1..16384 (0 restores the built-in default, 16384: one
+ * workgroup per tile up to 16 GiB per launch and stream on 256 compute units). Not needed for correctness; the
+ * reference has no counterpart. */
 int tdm_set_blocks_per_cu(int blocks);
 
 /* Launch geometry knob for measurements: which tile a workgroup takes. Consecutive workgroups

@@ -796,7 +796,7 @@ int tdm_build_geometry(int* k1_tile_bytes, int* workgroup_lanes, int* table_tile
 
 int tdm_set_blocks_per_cu(int blocks) {
   return guard([&] {
-    if (blocks < 0 || blocks > 1024) throw Invalid("blocks per compute unit must be in [0, 1024]");
+    if (blocks < 0 || blocks > kDefaultBlocksPerCu) throw Invalid("blocks per compute unit must be in [0, " + std::to_string(kDefaultBlocksPerCu) + "]");
     g_blocks_per_cu = blocks == 0 ? kDefaultBlocksPerCu : blocks;
   });
 }

@@ -60,9 +60,11 @@ constexpr int kWarmVecs = TDM_WARM_VECS;
 constexpr int kTileVecs = kThreads * kUnroll;   // 256 vectors = 4 KiB of every stream
 // Measured on MI355X: one tile per workgroup beats a persistent grid-stride
 // loop by 5-8% (the hardware dispatcher balances 8 XCDs better than a fixed stride),
-// so the grid covers the tiles one to one up to 256 Ki workgroups (1-2 GiB per stream)
-// and strides only beyond that.
-constexpr int kDefaultBlocksPerCu = 1024;
+// so the grid covers the tiles one to one up to 4 Mi workgroups (16 GiB per launch and stream)
+// and strides only beyond that. (With 256 Ki workgroups at most, four ranks of 4 GiB each lost
+// 10 % on the ring's steps, 19 % on its one-launch forms and 23 % on the single-launch all-reduce.)
+// 4 Mi workgroups of up to 256 lanes stay below HIP's limit of 2^32 lanes per launch.
+constexpr int kDefaultBlocksPerCu = 16384;
 
 int g_blocks_per_cu = kDefaultBlocksPerCu;
 constexpr int64_t kColdFootprint = int64_t(512) << 20;  // twice the Infinity Cache

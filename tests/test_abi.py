@@ -48,7 +48,7 @@ def test_argument_errors_need_no_gpu():
     segs[0].count, segs[1].count = 5, 5000
     assert L.tdm_k2_table_bytes(segs, 0, 0) > 0 and L.tdm_k2_table_bytes(segs, 2, 0) > L.tdm_k2_table_bytes(segs, 1, 0)
     assert L.tdm_k2_table_bytes(segs, 2, 99) == -1
-    assert L.tdm_set_blocks_per_cu(5000) == 1
+    assert L.tdm_set_blocks_per_cu(50_000) == 1
     assert L.tdm_set_blocks_per_cu(0) == 0
     assert L.tdm_set_xcd_group(6, 0) == 1 and b"family" in L.tdm_last_error()
     assert L.tdm_set_xcd_group(0, 13) == 1 and b"shift" in L.tdm_last_error()
