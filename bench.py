@@ -522,7 +522,7 @@ def ipc_rank(g, sizes_kib, reps, direct=False):
 def ipc_allreduce():
     from tandem_amd import launch
 
-    sizes = [64, 256, 1024, 4096, 16384, 65536]
+    sizes = [64, 256, 1024, 4096, 16384, 65536, 262144]  # KiB per rank; the reference's own sweep ends at 64 MiB
     out = {"workload": "all_reduce(sum) fp32 between 2 processes sharing the GPU through HIP IPC, barrier + all_reduce + device sync, median of 20",
            "reference_T4_cpp_engine_ms": {"64": 0.64, "256": 0.80, "1024": 0.83, "4096": 0.75, "16384": 1.72, "65536": 6.24}}
 
