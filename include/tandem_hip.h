@@ -156,11 +156,11 @@ int tdm_local_all_gather(void* const* bufs, int world, int64_t numel, int dtype,
 
 /* Which form tdm_local_reduce_scatter / tdm_local_all_gather (and tdm_local_all_reduce with
  * TDM_ALLREDUCE_RING) take: 0 the ring's W-1 steps, one launch each; 1 the whole reduce-scatter as one
- * launch (world sizes 2..4: every tile runs the ring's chain of additions for its chunk and stores each
- * partial sum where the ring would have left it) and the whole all-gather as one launch (world sizes
- * 2..8: every chunk read once from its owner and stored into the other ranks' buffers); -1 (default)
- * the one-launch all-gather from world size 3 on, the one-launch reduce-scatter at world sizes 3 and 4,
- * the steps otherwise. Memory ends bit for bit the
+ * launch (world sizes 2..8: every tile runs the ring's chain of additions for its chunk and stores each
+ * partial sum where the ring would have left it; a call whose ranks' copies of a chunk disagree within
+ * 16 bytes takes the steps all the same) and the whole all-gather as one launch (world sizes 2..8: every
+ * chunk read once from its owner and stored into the other ranks' buffers); -1 (default) both one-launch
+ * forms from world size 3 on, the steps at world size 2 and beyond 8. Memory ends bit for bit the
  * same either way, partial sums included. Process-wide; for measurements and tests. The reference has no
  * counterpart. */
 int tdm_set_ring_form(int form);

@@ -78,10 +78,12 @@ void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool s
 void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream, int policy = 2);
 void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream);
 // kernels_chain.hip: the ring reduce-scatter of a whole group in one launch (rank q's buffer at base[q], chunk c =
-// elements [lo[c], lo[c] + len[c])); world sizes 2..kChainMaxWorld
-constexpr int kChainMaxWorld = 4;
+// elements [lo[c], lo[c] + len[c])); world sizes 2..kChainMaxWorld. Returns false, with nothing launched, when the ranks'
+// copies of some chunk disagree within 16 bytes: the kernel has no element-by-element path (it would set its register
+// count), and the caller takes the ring's steps.
+constexpr int kChainMaxWorld = 8;
 bool chain_handles(int world);
-void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
+bool chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
                           bool keep_sent, bool cold, unsigned occupancy_pad, int xcd_shift, int max_grid, hipStream_t stream);
 // the ring all-gather of a whole group in one launch: every chunk read once from its owner and stored into the
 // other ranks' buffers; world sizes 2..8; `cold`: the footprint is beyond the caches (non-temporal accesses)

@@ -112,7 +112,9 @@ int xcd_shift(int kind, int world, bool cold) {
   const int set = g_xcd_shift[kind].load(std::memory_order_relaxed);
   if (set >= 0) return set;
   switch (kind) {
-    case TDM_XCD_REDUCE: return cold && world == 3 ? 6 : 0;  // cold: the one-launch reduce-scatter (256 MiB per rank at world 3: 233 -> 218 us; world 4: none)
+    // cold: the one-launch reduce-scatter beyond the caches. Runs of 256 KiB per XCD, 256 MiB / 1 GiB per rank: world 3
+    // 221 -> 211 / 922 -> 890 us, world 5 432 -> 413 / 1865 -> 1704, world 8 667 -> 678 / 3097 -> 2631; world 4 loses (287 -> 299).
+    case TDM_XCD_REDUCE: return cold && world >= 3 && world != 4 ? 6 : 0;
     case TDM_XCD_STEP: return 6;
     case TDM_XCD_ADAMW: return 7;
     case TDM_XCD_FOLD_TABLE: return world >= 4 ? 8 : 0;
@@ -132,10 +134,13 @@ int xcd_shift(int kind, int world, bool cold) {
 // fold 0.212 -> 0.25 ms at 24 KiB, ZeRO-2's fold into the shards 0.36 -> 0.39).
 std::atomic<int> g_occupancy_pad[kXcdKinds] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
 
-unsigned occupancy_pad(int kind, bool cold = true) {
+unsigned occupancy_pad(int kind, bool cold = true, int world = 0) {
   const int set = g_occupancy_pad[kind].load(std::memory_order_relaxed);
   if (set >= 0) return static_cast<unsigned>(set);
   switch (kind) {
+    // the one-launch reduce-scatter (the ring's reduce step takes no pad): 2 W - 1 streams per workgroup. Beyond the caches,
+    // 256 MiB per rank, no pad against this one: world 3 221 -> 211 us, world 4 295 -> 287, world 5 437 -> 405, world 8 697 -> 667.
+    case TDM_XCD_REDUCE: return !cold ? 0 : world <= 4 ? 16384 : world <= 6 ? 24576 : 32768;
     case TDM_XCD_STEP: return 24576;
     case TDM_XCD_ADAMW: return 24576;
     case TDM_XCD_COPY: return cold ? 16384 : 0;  // the one-launch all-gather (the ring's copy step takes no pad)
@@ -596,9 +601,10 @@ int64_t footprint(const LocalRanks& lr) { return lr.footprint; }
 // (8 (W-1)), and leave no gaps between launches. Measured on MI355X, reduce-scatter, steps
 // against one launch: world 4 at 4 MiB per rank 15.3 against 10.4 us, 16 MiB 25.8 / 21.6, 64 MiB
 // 88 / 70, 96 MiB 132 / 120, 128 MiB 175 / 152, 256 MiB 337 / 291 (once the ranks' tensors together
-// exceed 320 MiB: non-temporal accesses and 2 KiB per workgroup and stream; with everything cached
-// and 4 KiB the one launch loses there, 343; an occupancy cap only loses); world 3 at 64 MiB 65 / 55,
-// 96 MiB 94 / 79, 256 MiB 235 / 218.
+// exceed 320 MiB: non-temporal accesses, 2 KiB per workgroup and stream and an occupancy cap; with
+// everything cached and 4 KiB the one launch loses there, 343); world 3 at 64 MiB 65 / 55,
+// 96 MiB 94 / 79, 256 MiB 235 / 211; world 5 at 16 MiB 45 / 31, 256 MiB 514 / 405; world 8 at 4 MiB
+// 29.5 / 14, 16 MiB 64 / 41, 256 MiB 861 / 667, 1 GiB 3690 / 2630.
 // At world 2 a collective is one step anyway and the step kernels' policies do better (64 MiB
 // 49 / 51 us, 256 MiB 186 / 236).
 std::atomic<int> g_ring_form{-1};
@@ -624,10 +630,11 @@ void local_reduce_scatter(const LocalRanks& lr, bool average, bool keep_sent, hi
   if (one_launch_form(lr)) {
     const int64_t cap = static_cast<int64_t>(t_call_cus ? t_call_cus : compute_units()) * g_blocks_per_cu;
     const bool cold = lr.footprint > kOneLaunchFootprint;
-    chain_reduce_scatter(lr.base, lr.lo, lr.len, n, lr.dtype, lr.es, average, keep_sent, cold,
-                         cold ? occupancy_pad(TDM_XCD_REDUCE) : 0, xcd_shift(TDM_XCD_REDUCE, n, cold),
-                         static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream);
-    return;
+    if (chain_reduce_scatter(lr.base, lr.lo, lr.len, n, lr.dtype, lr.es, average, keep_sent, cold,
+                             occupancy_pad(TDM_XCD_REDUCE, cold, n), xcd_shift(TDM_XCD_REDUCE, n, cold),
+                             static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), stream)) {
+      return;
+    }
   }
   for (int s = 0; s < n - 1; ++s) {
     tdm_pair pairs[TDM_MAX_PAIRS];

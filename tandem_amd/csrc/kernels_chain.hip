@@ -37,7 +37,7 @@ struct ChainTable {
   char* ptr[TDM_MAX_WORLD][TDM_MAX_WORLD];  // [segment][rank]
   int64_t count[TDM_MAX_WORLD];
   int32_t chunk[TDM_MAX_WORLD];
-  int32_t vec_ok[TDM_MAX_WORLD];  // 0: element by element; 1 + h: ptr 16-byte aligned with h more elements directly before it
+  int32_t vec_ok[TDM_MAX_WORLD];  // 1 + h: ptr 16-byte aligned with h more elements directly before it
 };
 
 template <typename T, int kWorld, int kDiv>
@@ -56,12 +56,14 @@ __device__ __forceinline__ void chain_elem(const T (&in)[kWorld], T (&out)[kWorl
 
 // kMask: the cache policy (kernels_device.h): 0 everything cached, for footprints that stay in the caches; 7 non-temporal
 // loads and stores, for footprints beyond them.
-// A workgroup takes kU vectors per lane and stream: 2 (4 KiB of every stream) within the caches, 1 beyond.
-template <typename T, int kWorld, int kDiv, int kMask, int kU = (kMask == 0 ? kWarmVecs : 1)>
+// A workgroup takes kU vectors per lane and stream: 2 (4 KiB of every stream) within the caches, 1 beyond them
+// and from five ranks on (a lane holds kU vectors of every rank at once).
+constexpr int chain_vecs(int world, bool cold) { return !cold && world <= 4 ? kWarmVecs : 1; }
+
+template <typename T, int kWorld, int kDiv, int kMask, int kU = chain_vecs(kWorld, kMask != 0)>
 __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divisor<T> dv) {
   constexpr int L = lanes<T>();
   constexpr int kVecs = kThreads * kU;  // vectors of every stream per workgroup
-  constexpr int64_t kTileElems = static_cast<int64_t>(kVecs) * L;
   const int64_t total = tab.tile_end[tab.nseg - 1];
   for (int64_t at = blockIdx.x; at < total; at += gridDim.x) {
     const int64_t tile = tile_of(at, total, tab.shift);
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divi
 #pragma unroll
     for (int k = 0; k < kWorld; ++k) p[k] = tab.ptr[sg][(c + 1 + k) % kWorld];
     const bool keep = tab.keep_sent != 0;
-    if (tab.vec_ok[sg]) {
+    {  // every segment is vectorisable: the host sends chunks whose copies disagree within 16 bytes through the ring's steps
       const int64_t nv = n / L;
       vec16 raw[kWorld][kU];
 #pragma unroll
@@ -88,19 +90,22 @@ __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divi
       for (int u = 0; u < kU; ++u) {
         const int64_t v = t * kVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
         if (v < nv) {
-          Lanes<T> res[kWorld];
+          // the chain rank by rank over the vector's lanes (chain_elem's arithmetic): a rank's partial sums are
+          // stored as soon as they exist, so a lane holds one accumulator per element and never all W results
+          using A = typename Elem<T>::acc;
+          A acc[L];
 #pragma unroll
-          for (int l = 0; l < L; ++l) {
-            T in[kWorld], out[kWorld];
+          for (int k = 0; k < kWorld; ++k) {
+            const Lanes<T> x = unpack<T>(raw[k][u]);
+            Lanes<T> o;
 #pragma unroll
-            for (int k = 0; k < kWorld; ++k) in[k] = unpack<T>(raw[k][u]).v[l];
-            chain_elem<T, kWorld, kDiv>(in, out, dv);
-#pragma unroll
-            for (int k = 0; k < kWorld; ++k) res[k].v[l] = out[k];
+            for (int l = 0; l < L; ++l) {
+              const A y = scaled<T, kDiv>(Elem<T>::widen(x.v[l]), dv.divisor, dv.reciprocal);
+              acc[l] = k == 0 ? y : Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc[l])));
+              o.v[l] = Elem<T>::narrow(acc[l]);
+            }
+            if (k > 0 || keep) store16<kMask>(p[k] + v * 16, pack<T>(o));
           }
-          if (keep) store16<kMask>(p[0] + v * 16, pack<T>(res[0]));
-#pragma unroll
-          for (int k = 1; k < kWorld; ++k) store16<kMask>(p[k] + v * 16, pack<T>(res[k]));
         }
       }
       const int head = tab.vec_ok[sg] - 1;
@@ -114,20 +119,6 @@ __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divi
         if (keep) reinterpret_cast<T*>(p[0])[i] = out[0];
 #pragma unroll
         for (int k = 1; k < kWorld; ++k) reinterpret_cast<T*>(p[k])[i] = out[k];
-      }
-    } else {  // a copy off the 16-byte grid: element by element, still coalesced
-      const int64_t e0 = t * kTileElems + threadIdx.x;
-      for (int r = 0; r < kU * L; ++r) {
-        const int64_t i = e0 + static_cast<int64_t>(r) * kThreads;
-        if (i < n) {
-          T in[kWorld], out[kWorld];
-#pragma unroll
-          for (int k = 0; k < kWorld; ++k) in[k] = reinterpret_cast<const T*>(p[k])[i];
-          chain_elem<T, kWorld, kDiv>(in, out, dv);
-          if (keep) reinterpret_cast<T*>(p[0])[i] = out[0];
-#pragma unroll
-          for (int k = 1; k < kWorld; ++k) reinterpret_cast<T*>(p[k])[i] = out[k];
-        }
       }
     }
   }
@@ -161,7 +152,15 @@ void launch_chain(const ChainTable& tab, int world, bool average, int grid, bool
     case 6: launch_chain_m<T, 3, 0>(tab, average, grid, pad, stream); break;
     case 7: launch_chain_m<T, 3, 7>(tab, average, grid, pad, stream); break;
     case 8: launch_chain_m<T, 4, 0>(tab, average, grid, pad, stream); break;
-    default: launch_chain_m<T, 4, 7>(tab, average, grid, pad, stream); break;
+    case 9: launch_chain_m<T, 4, 7>(tab, average, grid, pad, stream); break;
+    case 10: launch_chain_m<T, 5, 0>(tab, average, grid, pad, stream); break;
+    case 11: launch_chain_m<T, 5, 7>(tab, average, grid, pad, stream); break;
+    case 12: launch_chain_m<T, 6, 0>(tab, average, grid, pad, stream); break;
+    case 13: launch_chain_m<T, 6, 7>(tab, average, grid, pad, stream); break;
+    case 14: launch_chain_m<T, 7, 0>(tab, average, grid, pad, stream); break;
+    case 15: launch_chain_m<T, 7, 7>(tab, average, grid, pad, stream); break;
+    case 16: launch_chain_m<T, 8, 0>(tab, average, grid, pad, stream); break;
+    default: launch_chain_m<T, 8, 7>(tab, average, grid, pad, stream); break;
   }
 }
 
@@ -269,14 +268,14 @@ void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, 
 
 bool chain_handles(int world) { return world >= 2 && world <= kChainMaxWorld; }
 
-void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
+bool chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* len, int world, int dtype, int es, bool average,
                           bool keep_sent, bool cold, unsigned pad, int shift, int max_grid, hipStream_t stream) {
-  if (!chain_handles(world)) throw Invalid("the one-launch reduce-scatter handles world sizes 2..4");
+  if (!chain_handles(world)) throw Invalid("the one-launch reduce-scatter handles world sizes 2..8");
   ChainTable tab;
   std::memset(&tab, 0, sizeof tab);
   tab.keep_sent = keep_sent && average ? 1 : 0;  // without a division the first sender's copy is x already
   tab.shift = shift;
-  const int64_t tile_elems = static_cast<int64_t>(kThreads) * (cold ? 1 : kWarmVecs) * (16 / es);  // as the kernel's kU
+  const int64_t tile_elems = static_cast<int64_t>(kThreads) * chain_vecs(world, cold) * (16 / es);  // as the kernel's kU
   int64_t tiles = 0;
   int k = 0;
   for (int c = 0; c < world; ++c) {
@@ -284,16 +283,17 @@ void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* l
     uintptr_t at[TDM_MAX_WORLD];
     for (int q = 0; q < world; ++q) at[q] = reinterpret_cast<uintptr_t>(base[q] + lo[c] * es);
     const SegPlan plan = plan_segment(at, world, len[c], es, tile_elems);
+    if (!plan.vec) return false;  // the ranks' copies disagree within 16 bytes: nothing launched, the caller takes the ring's steps
     for (int q = 0; q < world; ++q) tab.ptr[k][q] = base[q] + (lo[c] + plan.head) * es;
     tab.count[k] = plan.body;
     tab.chunk[k] = c;
-    tab.vec_ok[k] = plan.vec ? 1 + plan.head : 0;
+    tab.vec_ok[k] = 1 + plan.head;
     tiles += plan.tiles;
     tab.tile_end[k] = tiles;
     ++k;
   }
   tab.nseg = k;
-  if (k == 0) return;
+  if (k == 0) return true;
   const int grid = static_cast<int>(tiles < max_grid ? tiles : max_grid);
   switch (dtype) {
     case TDM_F32: launch_chain<float>(tab, world, average, grid, cold, pad, stream); break;
@@ -307,6 +307,7 @@ void chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* l
     default: throw Invalid("unknown dtype " + std::to_string(dtype));
   }
   check_hip(hipGetLastError(), "k1_chain launch");
+  return true;
 }
 
 }  // namespace tandem_hip

@@ -30,7 +30,7 @@ def from_np(a, dtype, dev):
 @pytest.fixture(params=["steps", "one_launch"], autouse=True)
 def ring_form(request):
     """Every test here runs with the ring collectives as W-1 launches and as one launch
-    (world sizes 2..4 have the second form; the others take the steps either way)."""
+    (world sizes 2..8 have the second form; views whose phases differ between the ranks take the steps either way)."""
     from tandem_amd._lib import lib
 
     assert lib().tdm_set_ring_form(0 if request.param == "steps" else 1) == 0
