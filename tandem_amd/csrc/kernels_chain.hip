@@ -92,19 +92,28 @@ __global__ __launch_bounds__(kThreads) void k1_chain_kernel(ChainTable tab, Divi
         if (v < nv) {
           // the chain rank by rank over the vector's lanes (chain_elem's arithmetic): a rank's partial sums are
           // stored as soon as they exist, so a lane holds one accumulator per element and never all W results
-          using A = typename Elem<T>::acc;
-          A acc[L];
+          if constexpr (!Elem<T>::floating) {  // integers: never divided (the first sender's copy stays), whole vectors added
+            vec16 sum = raw[0][u];
 #pragma unroll
-          for (int k = 0; k < kWorld; ++k) {
-            const Lanes<T> x = unpack<T>(raw[k][u]);
-            Lanes<T> o;
-#pragma unroll
-            for (int l = 0; l < L; ++l) {
-              const A y = scaled<T, kDiv>(Elem<T>::widen(x.v[l]), dv.divisor, dv.reciprocal);
-              acc[l] = k == 0 ? y : Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc[l])));
-              o.v[l] = Elem<T>::narrow(acc[l]);
+            for (int k = 1; k < kWorld; ++k) {
+              sum = add_vec<T>(raw[k][u], sum);
+              store16<kMask>(p[k] + v * 16, sum);
             }
-            if (k > 0 || keep) store16<kMask>(p[k] + v * 16, pack<T>(o));
+          } else {
+            using A = typename Elem<T>::acc;
+            A acc[L];
+#pragma unroll
+            for (int k = 0; k < kWorld; ++k) {
+              const Lanes<T> x = unpack<T>(raw[k][u]);
+              Lanes<T> o;
+#pragma unroll
+              for (int l = 0; l < L; ++l) {
+                const A y = scaled<T, kDiv>(Elem<T>::widen(x.v[l]), dv.divisor, dv.reciprocal);
+                acc[l] = k == 0 ? y : Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc[l])));
+                o.v[l] = Elem<T>::narrow(acc[l]);
+              }
+              if (k > 0 || keep) store16<kMask>(p[k] + v * 16, pack<T>(o));
+            }
           }
         }
       }

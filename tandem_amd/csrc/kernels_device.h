@@ -198,6 +198,32 @@ __device__ __forceinline__ vec16 pack(const Lanes<T>& in) {
   return out;
 }
 
+// The lane-wise wrap-around sum of two vectors of the INTEGER type T, on the packed words: integers are never
+// divided, so their kernels need no per-element code (unpacked, sixteen 8-bit lanes cost a kernel 100-250 registers).
+// 8- and 16-bit lanes add inside their 32-bit word without carrying into the neighbour: the low bits of every lane are
+// added with the top bit masked off, and the top bits are the exclusive or of the operands' and the carry's.
+template <typename T>
+__device__ __forceinline__ vec16 add_vec(const vec16& a, const vec16& b) {
+  static_assert(!Elem<T>::floating, "integer element types only");
+  vec16 r;
+  if constexpr (sizeof(T) == 8) {
+    unsigned long long x[2], y[2];
+    __builtin_memcpy(x, &a, 16);
+    __builtin_memcpy(y, &b, 16);
+    x[0] += y[0];
+    x[1] += y[1];
+    __builtin_memcpy(&r, x, 16);
+  } else if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = a[i] + b[i];
+  } else {
+    constexpr uint32_t top = sizeof(T) == 2 ? 0x80008000u : 0x80808080u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = ((a[i] & ~top) + (b[i] & ~top)) ^ ((a[i] ^ b[i]) & top);
+  }
+  return r;
+}
+
 // Cache policy, measured on MI355X. K1 with 4 x 64 MiB chunk pairs per launch: a
 // stream that is only read does best with non-temporal loads (it is not kept in
 // L2 / Infinity Cache), a stream that is read, modified and written back does best
@@ -294,22 +320,30 @@ __global__ __launch_bounds__(kThreads) void k1_reduce_kernel(PairTable tab, Divi
         for (int k = 0; k < kK1Unroll; ++k) b[k] = load_stream<kMask>(svp + (v0 + k * kThreads) * 16);
 #pragma unroll
         for (int k = 0; k < kK1Unroll; ++k) {
-          Lanes<T> x = unpack<T>(a[k]), y = unpack<T>(b[k]);
+          if constexpr (!Elem<T>::floating) {  // (never scaled: the source stays as it is)
+            store16<kMask>(dvp + (v0 + k * kThreads) * 16, add_vec<T>(a[k], b[k]));
+          } else {
+            Lanes<T> x = unpack<T>(a[k]), y = unpack<T>(b[k]);
 #pragma unroll
-          for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
-          store16<kMask>(dvp + (v0 + k * kThreads) * 16, pack<T>(x));
-          if (writeback) store16<kMask>(svp + (v0 + k * kThreads) * 16, pack<T>(y));
+            for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
+            store16<kMask>(dvp + (v0 + k * kThreads) * 16, pack<T>(x));
+            if (writeback) store16<kMask>(svp + (v0 + k * kThreads) * 16, pack<T>(y));
+          }
         }
       } else {
 #pragma unroll
         for (int k = 0; k < kK1Unroll; ++k) {
           const int64_t v = v0 + k * kThreads;
           if (v < nv) {
-            Lanes<T> x = unpack<T>(load_rmw<kMask>(dvp + v * 16)), y = unpack<T>(load_stream<kMask>(svp + v * 16));
+            if constexpr (!Elem<T>::floating) {
+              store16<kMask>(dvp + v * 16, add_vec<T>(load_rmw<kMask>(dvp + v * 16), load_stream<kMask>(svp + v * 16)));
+            } else {
+              Lanes<T> x = unpack<T>(load_rmw<kMask>(dvp + v * 16)), y = unpack<T>(load_stream<kMask>(svp + v * 16));
 #pragma unroll
-            for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
-            store16<kMask>(dvp + v * 16, pack<T>(x));
-            if (writeback) store16<kMask>(svp + v * 16, pack<T>(y));
+              for (int l = 0; l < L; ++l) reduce_elem<T, kDiv>(x.v[l], y.v[l], scale_dst, scale_src, dv);
+              store16<kMask>(dvp + v * 16, pack<T>(x));
+              if (writeback) store16<kMask>(svp + v * 16, pack<T>(y));
+            }
           }
         }
       }
@@ -476,22 +510,31 @@ __device__ __forceinline__ void fold_tile(const FoldSegDev& sg, int64_t t, const
       for (int u = 0; u < kU; ++u) {
         const int64_t v = vbase + u * kT;
         if (v < nv) {
-          Lanes<T> out;
+          vec16 packed;
+          [[maybe_unused]] Lanes<T> out;
+          if constexpr (!Elem<T>::floating) {
+            packed = in[0][u];
 #pragma unroll
-          for (int l = 0; l < L; ++l) {
-            A acc = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[0][u]).v[l]), dv.divisor, dv.reciprocal);
+            for (int k = 1; k < kWorld; ++k) packed = add_vec<T>(in[k][u], packed);
+          } else {
 #pragma unroll
-            for (int k = 1; k < kWorld; ++k) {
-              const A y = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[k][u]).v[l]), dv.divisor, dv.reciprocal);
-              acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+            for (int l = 0; l < L; ++l) {
+              A acc = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[0][u]).v[l]), dv.divisor, dv.reciprocal);
+#pragma unroll
+              for (int k = 1; k < kWorld; ++k) {
+                const A y = scaled<T, kDiv>(Elem<T>::widen(unpack<T>(in[k][u]).v[l]), dv.divisor, dv.reciprocal);
+                acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+              }
+              out.v[l] = Elem<T>::narrow(acc);
             }
-            out.v[l] = Elem<T>::narrow(acc);
+            packed = pack<T>(out);
           }
-          const vec16 packed = pack<T>(out);
 #pragma unroll
           for (int k = 0; k < kWorld; ++k)
             if (dp[k]) {
-              if constexpr (kAcc) {
+              if constexpr (kAcc && !Elem<T>::floating) {
+                store16<kMask>(dp[k] + v * 16, add_vec<T>(load_rmw<kMask>(dp[k] + v * 16), packed));
+              } else if constexpr (kAcc) {
                 Lanes<T> cur = unpack<T>(load_rmw<kMask>(dp[k] + v * 16));
 #pragma unroll
                 for (int l = 0; l < L; ++l)
