@@ -295,10 +295,10 @@ template <typename T, int kWorld>
 void launch_fold_small_w(const FoldSmall& table, int average, hipStream_t stream) {
   const Divisor<T> dv = make_divisor<T>(kWorld);
   // bytes touched: every tile is read from kWorld ranks (and written back to most of them)
-  const bool cold = table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld > kColdFootprint;
+  const bool cold = table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld >= cold_footprint(kWorld);
   const dim3 grid(grid_for(table.tile_end[table.nseg - 1] * (cold ? fold_small_parts<kWorld>() : 1))), block(kThreads);
   FoldSmall tab = table;
-  tab.shift = xcd_shift(TDM_XCD_FOLD, kWorld, table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld >= kColdFootprint);
+  tab.shift = xcd_shift(TDM_XCD_FOLD, kWorld, cold);
   if constexpr (!Elem<T>::floating) {
     if (cold) hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv);
     else hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv);

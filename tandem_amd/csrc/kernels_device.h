@@ -67,7 +67,11 @@ constexpr int kTileVecs = kThreads * kUnroll;   // 256 vectors = 4 KiB of every 
 constexpr int kDefaultBlocksPerCu = 16384;
 
 int g_blocks_per_cu = kDefaultBlocksPerCu;
-constexpr int64_t kColdFootprint = int64_t(512) << 20;  // twice the Infinity Cache
+// From which footprint (all ranks' tensors together) a single-launch all-reduce takes the kernel built for data that
+// is not found in the caches again (non-temporal stores, half tiles, an occupancy cap). Measured, cached against
+// uncached kernel, footprints of 256 / 320 / 384 / 448 MiB: world 4 77 / 107 / 149 / 174 against 87 / 109 / 130 / 148 us
+// (worlds 3 and 8 alike); world 2 82 / 102 / 138 / 165 against 92 / 120 / 147 / 163.
+constexpr int64_t cold_footprint(int world) { return int64_t(world == 2 ? 448 : 352) << 20; }
 
 // Which tile a workgroup takes. The dispatcher hands consecutive workgroups to the 8 XCDs in
 // turn, so with tile = workgroup index every XCD touches every eighth 4 KiB of every stream.
