@@ -608,7 +608,7 @@ int64_t footprint(const LocalRanks& lr) { return lr.footprint; }
 // At world 2 a collective is one step anyway and the step kernels' policies do better (64 MiB
 // 49 / 51 us, 256 MiB 186 / 236).
 std::atomic<int> g_ring_form{-1};
-constexpr int64_t kOneLaunchFootprint = int64_t(320) << 20;  // beyond: nothing written is found in the caches again
+constexpr int64_t kOneLaunchFootprint = int64_t(296) << 20;  // beyond: nothing written is found in the caches again (world 4, reduce-scatter at 320 MiB: 112 us with the cached kernel, 99 with the other)
 
 bool one_launch_form(const LocalRanks& lr) {
   if (!chain_handles(lr.world)) return false;
