@@ -85,8 +85,9 @@ int tdm_set_xcd_group(int kind, int shift);
  * (TDM_XCD_*, -1: all) reserve per workgroup without using them, which caps how many workgroups
  * share a compute unit (160 KiB of LDS each); 0: no cap, -1: the built-in default of that family
  * (24 KiB for TDM_XCD_STEP and TDM_XCD_ADAMW, whose many streams do better with 3 waves per SIMD;
- * beyond the caches also 24 KiB for a by-value fold (TDM_XCD_FOLD) and 16 KiB for the one-launch
- * all-gather (TDM_XCD_COPY); 0 otherwise). At most 65536. Process-wide; results never depend on it. The reference has
+ * beyond the caches also 24 KiB for a by-value fold (TDM_XCD_FOLD), 16 KiB for the one-launch
+ * all-gather (TDM_XCD_COPY) and 16 to 32 KiB, by world size, for the one-launch reduce-scatter
+ * (TDM_XCD_REDUCE); 0 otherwise). At most 65536. Process-wide; results never depend on it. The reference has
  * no counterpart. */
 int tdm_set_occupancy_pad(int kind, int bytes);
 /* The tile that workgroup `index` of a launch over `total` tiles takes at group shift `shift` (the
