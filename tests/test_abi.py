@@ -95,3 +95,18 @@ def test_cpu_tensors_are_refused():
 def test_fixtures_present():
     for f in ("ring_w2.npz", "ring_w3.npz", "ring_w4.npz", "ring_dtypes_w3.npz", "adamw.npz", "plans.json", "data.json"):
         assert os.path.exists(os.path.join(GOLDEN, f))
+
+
+def test_the_header_is_plain_c():
+    """include/tandem_hip.h is what a C, Go (cgo) or Rust (bindgen) host would bind: it must compile as C99 on its own."""
+    import shutil
+    import subprocess
+
+    import pytest
+
+    if shutil.which("gcc") is None:
+        pytest.skip("needs gcc")
+    header = os.path.join(ROOT, "include", "tandem_hip.h")
+    res = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", "c", header],
+                         stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert res.returncode == 0, res.stdout
