@@ -514,8 +514,17 @@ def launch(fn, size, *args, device="cuda", slot_bytes=DEFAULT_SLOT_BYTES, slots=
     ctx = mp.get_context("spawn")
     barrier = ctx.Barrier(size)
     with tempfile.TemporaryDirectory(prefix="tandem-") as results:
-        mp.spawn(_worker, args=(size, fn, args, barrier, device, slot_bytes, slots, backend, job, gpus, timeout, results),
-                 nprocs=size, join=True)
+        try:
+            mp.spawn(_worker, args=(size, fn, args, barrier, device, slot_bytes, slots, backend, job, gpus, timeout, results),
+                     nprocs=size, join=True)
+        finally:
+            # A rank unlinks its shared-memory region when its engine goes; ranks that were killed because another
+            # one failed never get there. The job's name is this call's own, so whatever is left is ours to remove.
+            for r in range(size):
+                try:
+                    os.unlink(f"/dev/shm/tandem-{job}-{r}-hip")
+                except OSError:
+                    pass
         out = []
         for r in range(size):
             path = os.path.join(results, f"rank{r}.pt")

@@ -600,8 +600,15 @@ def failing(g):
 def test_error_propagates_from_a_rank():
     from tandem_amd import launch
 
+    import glob
+
+    before = set(glob.glob("/dev/shm/tandem-*"))
     with pytest.raises(Exception, match="boom"):
         launch(failing, 2, gpus=[0, 0], timeout=10.0)
+    # the rank that was killed because its peer failed never unlinked its shared-memory region: launch() did
+    assert set(glob.glob("/dev/shm/tandem-*")) <= before
+    assert launch(failing, 1, gpus=[0], timeout=10.0) == [True]
+    assert set(glob.glob("/dev/shm/tandem-*")) <= before
 
 
 def out_of_step(g):
