@@ -293,6 +293,32 @@ def bucket_path(dev, reps):
             "segments": table.nseg}
 
 
+def unit_gather(dev, reps):
+    """K4 on its own: ZeRO-3's gather of one block unit of the 85.8M GPT (7,087,872 fp32) for both ranks of a
+    world of two, the ranks being buffers of this process. Twelve units are gathered in turn, as a forward
+    pass does, so no gather finds its shards in the caches. Accounted as 8 B per element and rank (what a rank's own
+    gather moves); the one launch for both ranks reads every shard once, 4 (W + 1) B per element."""
+    import torch
+
+    from tandem_amd import LocalWorld
+
+    world, unit, units = 2, 7_087_872, 12
+    sizes = [unit // world] * world
+    lw = LocalWorld(world)
+    shards = [[torch.randn(sizes[r], device=dev) for r in range(world)] for _ in range(units)]
+    fulls = [[torch.empty(unit, device=dev) for _ in range(world)] for _ in range(units)]
+
+    def forward():
+        for k in range(units):
+            lw.unit_gather(fulls[k], shards[k], sizes)
+
+    t = timed(forward, reps) / units
+    nbytes = 8 * unit * world
+    return {"workload": "ZeRO-3 unit gather, 7,087,872 fp32 per unit, 2 buffer ranks, 12 units in turn, one launch for both ranks",
+            "us_per_unit": round(t * 1e6, 2), "algorithmic_bytes": nbytes, "GBps": round(nbytes / t / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4)}
+
+
 def zero2_step(dev, reps):
     """ZeRO-2's reduce-scatter + AdamW + all-gather for the 85.8M GPT, world 4 on
     one GPU, all four shards stepped."""
@@ -669,6 +695,12 @@ def summarize(line):
         if mix:
             b["frac_of_mix_ceiling"] = cfg["bucket_path_frac_of_mix_ceiling"] = against("bucket_fold_w2", b["GBps"])
             cfg["bucket_path_mix_ceiling_frac"] = mix["bucket_fold_w2"]["frac_of_hbm_peak"]
+    u = line.get("unit_gather")
+    if u:
+        cfg["unit_gather_us"] = u["us_per_unit"]
+        cfg["unit_gather_frac"] = u["frac_of_hbm_peak"]
+        if mix:
+            u["frac_of_mix_ceiling"] = cfg["unit_gather_frac_of_mix_ceiling"] = against("ring_copy", u["GBps"])
 
 
 def device_name(_lib):
@@ -788,6 +820,8 @@ def main():
             line["sweep"] = sweep(lw, dev, max(5, args.steps // 2))
         if not only or "bucket" in only:
             line["bucket_path"] = bucket_path(dev, args.steps)
+            torch.cuda.empty_cache()
+            line["unit_gather"] = unit_gather(dev, args.steps)
             torch.cuda.empty_cache()
         if not only or "zero2" in only:
             line["zero2_step"] = zero2_step(dev, max(5, args.steps // 2))

@@ -317,6 +317,14 @@ int tdm_k23_zero2_step_segment(const tdm_step_seg* seg, int world, int average, 
 int tdm_k4_unit_gather(void* full, const void* const* shards, const int64_t* sizes, int world, int dtype,
                        tdm_stream stream);
 
+/* The same gather for EVERY rank of a group whose ranks are buffers of one process, in one launch
+ * (world sizes up to 8; one launch per rank beyond): shard q is read once and stored into elements
+ * [lo_q, lo_q + sizes[q]) of all `world` buffers fulls[0..world): 4 (W + 1) bytes per element of the
+ * unit where W calls of tdm_k4_unit_gather move 8 W. No counterpart in the reference, which has one
+ * process per rank. */
+int tdm_k4_unit_gather_all(void* const* fulls, const void* const* shards, const int64_t* sizes, int world, int dtype,
+                           tdm_stream stream);
+
 /* ---- the engine: Group(backend="hip") --------------------------------------- */
 
 /* One rank's half of a group whose ranks are processes sharing one GPU. Mirrors

@@ -95,6 +95,8 @@ _SIGNATURES = {
                                           ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
     "tdm_k23_zero2_step_segment": (ctypes.c_int, [ctypes.POINTER(StepSeg), ctypes.c_int, ctypes.c_int,
                                                   ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
+    "tdm_k4_unit_gather_all": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p),
+                                              ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "tdm_k4_unit_gather": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_int64),
                                           ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
 }

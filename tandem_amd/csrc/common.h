@@ -90,6 +90,9 @@ bool chain_reduce_scatter(char* const* base, const int64_t* lo, const int64_t* l
 bool gather_handles(int world);
 void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, int world, int es, bool cold, unsigned occupancy_pad,
                       int xcd_shift, int vectors_per_lane, int max_grid, hipStream_t stream);
+// ZeRO-3's unit gather for every rank in one launch (world sizes 1..8): shard q read once, stored into all the full buffers
+void unit_gather_multicast(char* const* fulls, const char* const* shards, const int64_t* sizes, int world, int es, bool cold,
+                           unsigned occupancy_pad, int xcd_shift, int vectors_per_lane, int max_grid, hipStream_t stream);
 void zero2_step_segment(const tdm_step_seg& seg, int world, bool average, const tdm_adamw_scalars& s, int order, hipStream_t stream);
 
 }  // namespace tandem_hip

@@ -178,14 +178,15 @@ void launch_chain(const ChainTable& tab, int world, bool average, int grid, bool
 // chunk's worth per rank, 8 (W-1) bytes per element of the tensor. With every rank's buffer in reach, a
 // workgroup reads its tile of chunk c ONCE from the owner and stores it into the W-1 other ranks' copies:
 // 4 W bytes per element, the same bytes in memory afterwards (copies have no order to preserve).
+// The same kernel gathers a ZeRO-3 unit for every rank at once: a segment is then one rank's shard, read once and stored
+// into its slice of all W ranks' full buffers.
 struct GatherTable {
   int nseg;
-  int ndst;  // destinations per segment (W - 1)
   int shift;  // of tile_of()
-  int pad_;
+  int32_t ndst[TDM_MAX_WORLD];  // destinations of every segment (W - 1 for the all-gather, up to W for a unit gather)
   int64_t tile_end[TDM_MAX_WORLD];
   const char* src[TDM_MAX_WORLD];
-  char* dst[TDM_MAX_WORLD][TDM_MAX_WORLD - 1];
+  char* dst[TDM_MAX_WORLD][TDM_MAX_WORLD];
   int64_t bytes[TDM_MAX_WORLD];
   int32_t vec_ok[TDM_MAX_WORLD];  // as the other tables': 0 byte by byte, 1 + h with h bytes before the pointers
 };
@@ -202,6 +203,7 @@ __global__ __launch_bounds__(kThreads) void k1_gather_kernel(GatherTable tab) {
     const int64_t t = tile - (sg ? tab.tile_end[sg - 1] : 0);
     const char* __restrict__ from = tab.src[sg];
     const int64_t n = tab.bytes[sg];
+    const int ndst = tab.ndst[sg];
     if (tab.vec_ok[sg]) {
       const int64_t nv = n / 16;
       vec16 raw[kU];
@@ -214,25 +216,40 @@ __global__ __launch_bounds__(kThreads) void k1_gather_kernel(GatherTable tab) {
       for (int u = 0; u < kU; ++u) {
         const int64_t v = t * kVecs + threadIdx.x + static_cast<int64_t>(u) * kThreads;
         if (v < nv)
-          for (int k = 0; k < tab.ndst; ++k) store16<kMask>(tab.dst[sg][k] + v * 16, raw[u]);
+          for (int k = 0; k < ndst; ++k) store16<kMask>(tab.dst[sg][k] + v * 16, raw[u]);
       }
       const int head = tab.vec_ok[sg] - 1;
       // the bytes after the last whole vector (lanes 0..15) and before the first (lanes 32..47)
       if (t == 0 && (threadIdx.x < n - nv * 16 || (threadIdx.x >= 32 && static_cast<int>(threadIdx.x) - 32 < head))) {
         const int64_t i = threadIdx.x < 32 ? nv * 16 + threadIdx.x : -1 - (static_cast<int64_t>(threadIdx.x) - 32);
         const char byte = from[i];
-        for (int k = 0; k < tab.ndst; ++k) tab.dst[sg][k][i] = byte;
+        for (int k = 0; k < ndst; ++k) tab.dst[sg][k][i] = byte;
       }
     } else {  // the copies disagree within 16 bytes: byte by byte, still coalesced
       const int64_t b0 = t * kTileBytes + threadIdx.x;
       for (int64_t i = b0; i < n && i < (t + 1) * kTileBytes; i += kThreads) {
         const char byte = from[i];
-        for (int k = 0; k < tab.ndst; ++k) tab.dst[sg][k][i] = byte;
+        for (int k = 0; k < ndst; ++k) tab.dst[sg][k][i] = byte;
       }
     }
   }
 }
 
+}  // namespace
+
+namespace {
+void launch_gather(const GatherTable& tab, int64_t tiles, bool cold, unsigned pad, int per_lane, int max_grid, hipStream_t stream) {
+  if (tab.nseg == 0) return;
+  if (per_lane != 1 && per_lane != 2) throw Invalid("1 or 2 vectors per lane");
+  const dim3 grid(static_cast<unsigned>(tiles < max_grid ? tiles : max_grid)), block(kThreads);
+  switch ((cold ? 2 : 0) + (per_lane == 2 ? 1 : 0)) {
+    case 0: hipLaunchKernelGGL((k1_gather_kernel<0, 1>), grid, block, pad, stream, tab); break;
+    case 1: hipLaunchKernelGGL((k1_gather_kernel<0, 2>), grid, block, pad, stream, tab); break;
+    case 2: hipLaunchKernelGGL((k1_gather_kernel<7, 1>), grid, block, pad, stream, tab); break;
+    default: hipLaunchKernelGGL((k1_gather_kernel<7, 2>), grid, block, pad, stream, tab); break;
+  }
+  check_hip(hipGetLastError(), "k1_gather launch");
+}
 }  // namespace
 
 bool gather_handles(int world) { return world >= 2 && world <= TDM_MAX_WORLD; }
@@ -242,7 +259,6 @@ void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, 
   if (!gather_handles(world)) throw Invalid("the one-launch all-gather handles world sizes 2..8");
   GatherTable tab;
   std::memset(&tab, 0, sizeof tab);
-  tab.ndst = world - 1;
   tab.shift = shift;
   const int64_t tile_bytes = static_cast<int64_t>(kThreads) * per_lane * 16;
   int64_t tiles = 0;
@@ -256,6 +272,7 @@ void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, 
     int d = 0;
     for (int q = 0; q < world; ++q)
       if (q != c) tab.dst[k][d++] = base[q] + lo[c] * es + plan.head;
+    tab.ndst[k] = d;
     tab.bytes[k] = plan.body;
     tab.vec_ok[k] = plan.vec ? 1 + plan.head : 0;
     tiles += plan.tiles;
@@ -263,16 +280,50 @@ void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, 
     ++k;
   }
   tab.nseg = k;
-  if (k == 0) return;
-  const dim3 grid(static_cast<unsigned>(tiles < max_grid ? tiles : max_grid)), block(kThreads);
-  if (per_lane != 1 && per_lane != 2) throw Invalid("1 or 2 vectors per lane");
-  switch ((cold ? 2 : 0) + (per_lane == 2 ? 1 : 0)) {
-    case 0: hipLaunchKernelGGL((k1_gather_kernel<0, 1>), grid, block, pad, stream, tab); break;
-    case 1: hipLaunchKernelGGL((k1_gather_kernel<0, 2>), grid, block, pad, stream, tab); break;
-    case 2: hipLaunchKernelGGL((k1_gather_kernel<7, 1>), grid, block, pad, stream, tab); break;
-    default: hipLaunchKernelGGL((k1_gather_kernel<7, 2>), grid, block, pad, stream, tab); break;
+  launch_gather(tab, tiles, cold, pad, per_lane, max_grid, stream);
+}
+
+// ZeRO-3's gather of one unit for EVERY rank in one launch: rank q's shard is read once and stored into elements
+// [lo_q, lo_q + sizes[q]) of all `world` full buffers (a full buffer whose slice IS the shard is skipped).
+void unit_gather_multicast(char* const* fulls, const char* const* shards, const int64_t* sizes, int world, int es, bool cold,
+                           unsigned pad, int shift, int per_lane, int max_grid, hipStream_t stream) {
+  if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("the one-launch unit gather handles world sizes 1..8");
+  GatherTable tab;
+  std::memset(&tab, 0, sizeof tab);
+  tab.shift = shift;
+  const int64_t tile_bytes = static_cast<int64_t>(kThreads) * per_lane * 16;
+  int64_t tiles = 0, lo = 0;
+  int k = 0;
+  for (int q = 0; q < world; ++q) {
+    const int64_t bytes = sizes[q] * es;
+    const int64_t at_bytes = lo * es;
+    lo += sizes[q];
+    if (bytes == 0) continue;
+    uintptr_t at[TDM_MAX_WORLD + 1];
+    int np = 0, d = 0;
+    at[np++] = reinterpret_cast<uintptr_t>(shards[q]);
+    char* dsts[TDM_MAX_WORLD];
+    for (int r = 0; r < world; ++r) {
+      char* dst = fulls[r] + at_bytes;
+      if (dst == shards[q]) continue;  // the shard already lies in this rank's full buffer
+      const uintptr_t a = reinterpret_cast<uintptr_t>(dst), b = reinterpret_cast<uintptr_t>(shards[q]);
+      if (a < b + static_cast<uintptr_t>(bytes) && b < a + static_cast<uintptr_t>(bytes)) throw Invalid("unit gather: a full buffer overlaps a shard");
+      dsts[d++] = dst;
+      at[np++] = a;
+    }
+    if (d == 0) continue;
+    const SegPlan plan = plan_segment(at, np, bytes, 1, tile_bytes);
+    tab.src[k] = shards[q] + plan.head;
+    for (int i = 0; i < d; ++i) tab.dst[k][i] = dsts[i] + plan.head;
+    tab.ndst[k] = d;
+    tab.bytes[k] = plan.body;
+    tab.vec_ok[k] = plan.vec ? 1 + plan.head : 0;
+    tiles += plan.tiles;
+    tab.tile_end[k] = tiles;
+    ++k;
   }
-  check_hip(hipGetLastError(), "k1_gather launch");
+  tab.nseg = k;
+  launch_gather(tab, tiles, cold, pad, per_lane, max_grid, stream);
 }
 
 bool chain_handles(int world) { return world >= 2 && world <= kChainMaxWorld; }

@@ -128,8 +128,8 @@ class LocalWorld:
         return bufs
 
     def unit_gather(self, fulls, shards, sizes):
-        """ZeRO-3's gather of one unit for every rank: fulls[r] receives every
-        rank's shard in one launch per rank (tandem/zero.py:238-245)."""
+        """ZeRO-3's gather of one unit for every rank (tandem/zero.py:238-245): every rank's shard
+        is read once and stored into its place in all the fulls[r], in one launch (up to 8 ranks)."""
         if len(fulls) != self.world or len(shards) != self.world:
             raise ValueError("unit_gather: one full buffer and one shard per rank")
         bounds = chunk_bounds(fulls[0].numel(), self.world, sizes)
@@ -140,10 +140,9 @@ class LocalWorld:
                 raise ValueError(f"unit_gather: shard {q} has {shards[q].numel()} elements, its chunk {hi - lo}")
         code = dtype_code(fulls[0].dtype)
         ptrs = (ctypes.c_void_p * self.world)(*[s.data_ptr() for s in shards])
+        outs = (ctypes.c_void_p * self.world)(*[f.data_ptr() for f in fulls])
         szs = (ctypes.c_int64 * self.world)(*[hi - lo for lo, hi in bounds])
-        st = stream_ptr(fulls[0].device)
-        for full in fulls:
-            check(lib().tdm_k4_unit_gather(ctypes.c_void_p(full.data_ptr()), ptrs, szs, self.world, code, st))
+        check(lib().tdm_k4_unit_gather_all(outs, ptrs, szs, self.world, code, stream_ptr(fulls[0].device)))
         return fulls
 
     def bucket_table(self, tensors_per_rank, buckets, out_per_rank=None):

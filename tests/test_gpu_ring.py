@@ -284,8 +284,44 @@ def test_unit_gather(dev):
     lw = LocalWorld(2)
     full = torch.arange(10, dtype=torch.float32, device=dev)
     other = torch.full((4,), 5.0, device=dev)
-    lw.unit_gather([full, full.clone()], [full[:6], other], [6, 4])
+    second = full.clone()
+    lw.unit_gather([full, second], [full[:6], other], [6, 4])
     assert torch.equal(full, torch.tensor([0, 1, 2, 3, 4, 5, 5, 5, 5, 5.0], device=dev))
+    assert torch.equal(second, full)
+
+
+@pytest.mark.parametrize("world", [1, 2, 3, 5, 8, 9, 12])
+def test_unit_gather_for_every_rank_at_once(dev, world):
+    """One launch fills all the ranks' full buffers (up to 8 ranks; beyond, a launch per rank): other element types,
+    shards and full buffers that start anywhere in their allocations, an empty shard, and nothing written outside."""
+    from tandem_amd import LocalWorld
+
+    lw = LocalWorld(world)
+    rng = np.random.default_rng(world)
+    for dtype in (torch.float32, torch.bfloat16, torch.int8, torch.float64):
+        for numel in (0, 5, 4099, 70_001):
+            cuts = np.sort(rng.integers(0, numel + 1, world - 1))
+            sizes = np.diff(np.concatenate([[0], cuts, [numel]])).astype(int).tolist()
+            if world > 2:
+                sizes[1] += sizes[2]
+                sizes[2] = 0
+            starts = [int(rng.integers(0, 16)) for _ in range(2 * world)]
+            data = [torch.from_numpy(rng.integers(-100, 100, m)).to(dtype) for m in sizes]
+            shard_store = [torch.full((m + 32,), 9, dtype=dtype, device=dev) for m in sizes]
+            shards = [st[starts[q]:starts[q] + sizes[q]] for q, st in enumerate(shard_store)]
+            for sh, x in zip(shards, data):
+                sh.copy_(x)
+            full_store = [torch.full((numel + 32,), 7, dtype=dtype, device=dev) for _ in range(world)]
+            fulls = [st[starts[world + r]:starts[world + r] + numel] for r, st in enumerate(full_store)]
+            lw.unit_gather(fulls, shards, sizes)
+            want = torch.cat(data) if numel else torch.zeros(0, dtype=dtype)
+            for r in range(world):
+                assert torch.equal(fulls[r].cpu(), want), (world, dtype, numel, sizes, r)
+                lo = starts[world + r]
+                host = full_store[r].cpu()
+                assert bool((host[:lo] == 7).all()) and bool((host[lo + numel:] == 7).all()), (world, dtype, numel, r)
+            for q in range(world):
+                assert torch.equal(shards[q].cpu(), data[q])
 
 
 def test_bad_arguments_raise(dev):
