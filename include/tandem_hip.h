@@ -20,6 +20,10 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* The library is built with hidden visibility; what this header declares is all it exports. */
+#if defined(__GNUC__) || defined(__clang__)
+#pragma GCC visibility push(default)
+#endif
 
 typedef void* tdm_stream;
 
@@ -462,6 +466,9 @@ int tdm_work_free(tdm_work* w);
  * summarize and chrome_trace see the GPU's span of each collective. */
 int tdm_engine_set_timing(tdm_engine* e, int on);
 
+#if defined(__GNUC__) || defined(__clang__)
+#pragma GCC visibility pop
+#endif
 #ifdef __cplusplus
 }
 #endif

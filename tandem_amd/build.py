@@ -19,7 +19,8 @@ SOURCES = ["kernels.hip", "kernels_chain.hip", "probe.hip", "abi.hip", "engine.h
 # -ffp-contract=off: no multiply-add is fused unless the source says fma.
 # -fhip-fp32-correctly-rounded-divide-sqrt: IEEE division and sqrt (the default; stated).
 # -packed-fp32-ops disabled: the compiler must not form v_pk_*_f32 from scalar float code.
-FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-ffp-contract=off",
+# -fvisibility=hidden: the library exports the entry points of include/tandem_hip.h and nothing else.
+FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-ffp-contract=off",
          "-fhip-fp32-correctly-rounded-divide-sqrt", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wall", "-Wextra", "-pthread"]
 

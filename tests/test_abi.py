@@ -110,3 +110,22 @@ def test_the_header_is_plain_c():
     res = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", "c", header],
                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert res.returncode == 0, res.stdout
+
+
+def test_the_library_exports_only_what_the_header_declares():
+    """Built with hidden visibility: apart from weak instantiations of the C++ standard library's templates, the
+    dynamic symbol table holds the header's entry points and nothing of the library's own C++."""
+    import shutil
+    import subprocess
+
+    import pytest
+
+    from tandem_amd import _lib
+
+    if shutil.which("nm") is None or not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("needs nm and the built library")
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], stdout=subprocess.PIPE, text=True, check=True).stdout
+    names = [line.split()[-1] for line in out.splitlines() if line.strip()]
+    ours = sorted(n for n in names if n.startswith("tdm_"))
+    assert ours == _lib.exported_symbols()
+    assert not [n for n in names if "tandem_hip" in n], "internal C++ symbols are exported"
