@@ -90,7 +90,6 @@ def checksums(t):
 
 
 def medium_rank(g, strategy):
-    import time
 
     from tandem_amd import ShardedAdamW
     from tandem_amd.data import synthetic
