@@ -90,7 +90,6 @@ def checksums(t):
 
 
 def medium_rank(g, strategy):
-
     from tandem_amd import ShardedAdamW
     from tandem_amd.data import synthetic
     from tandem_amd.model import GPT, Config
