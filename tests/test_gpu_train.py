@@ -78,6 +78,13 @@ def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1, zero_every
         extra = {"max_live": z.max_live, "live": z.live}
     else:
         w = torch.cat([p.detach().reshape(-1) for p in model.parameters()])
+    if not strategy.startswith("ddp"):
+        # what the reference's tests/test_zero.py:35-36,54 asks of the sharded strategies: two moments for this rank's shard
+        # only, and from stage 2 on no full gradients left behind by a backward
+        numel = sum(p.numel() for p in model.parameters())
+        extra["state_ok"] = sopt.state_bytes() <= 2 * 4 * (numel // g.size + len(list(model.parameters())))
+        if int(strategy[4]) >= 2:
+            extra["no_full_grads"] = all(p.grad is None for p in model.parameters())
     torch.cuda.synchronize()
     return {"losses": losses, "weights": w.cpu(), **extra}
 
@@ -129,6 +136,10 @@ def test_two_ranks_all_strategies_agree_bit_for_bit():
             assert torch.equal(res[r]["weights"], ref_w), (s, r)
     for s in ("zero3", "zero3s"):
         assert runs[s][0]["max_live"] <= 3 and runs[s][0]["live"] == 0
+    for s, res in runs.items():
+        if not s.startswith("ddp"):
+            assert all(x["state_ok"] for x in res), f"{s}: optimizer state beyond this rank's shard"
+            assert all(x.get("no_full_grads", True) for x in res), f"{s}: full gradients were kept"
 
 
 def test_four_ranks_stay_in_step():
