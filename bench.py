@@ -461,12 +461,13 @@ def train_rank(g, strategy, steps):
     adamw = dict(lr=3e-4, betas=(0.9, 0.95), weight_decay=0.1)
     fused = strategy.endswith("+fused")
     direct = strategy.endswith("+direct") or fused
+    hostwait = strategy.endswith("+hostwait")  # DDP whose host waits for every bucket, as the reference's does
     kind = strategy.split("+")[0]
     opt = None
     if kind == "alone":
         z, opt = model, torch.optim.AdamW(model.parameters(), foreach=False, **adamw)
     elif kind == "ddp":
-        z, opt = DDP(model, g, direct=direct), torch.optim.AdamW(model.parameters(), foreach=False, **adamw)
+        z, opt = DDP(model, g, direct=direct, stream_ordered=not hostwait), torch.optim.AdamW(model.parameters(), foreach=False, **adamw)
     elif kind in ("zero1", "zero2"):
         z = ZeRO(model, g, int(kind[-1]), ShardedAdamW(**adamw), direct=direct, fused_step=fused)
     else:
@@ -505,13 +506,14 @@ def train_rank(g, strategy, steps):
             "profile": {k: (round(v, 5) if isinstance(v, float) else v) for k, v in prof.items()}}
 
 
-def train_steps(steps, world=2, strategies=("alone", "ddp", "ddp+direct", "zero1", "zero1+direct", "zero2", "zero2+direct", "zero2+fused", "zero3")):
+def train_steps(steps, world=2, strategies=("alone", "ddp", "ddp+hostwait", "ddp+direct", "zero1", "zero1+direct", "zero2", "zero2+direct", "zero2+fused", "zero3")):
     from tandem_amd import launch
 
     out = {"workload": f"{world} processes sharing the GPU, 85.8M GPT, batch 8x512 split over the ranks, fp32, full step "
                        "(forward, backward, optimizer); 'alone' = the same rows with no communication and torch AdamW; "
                        "'+direct' = buckets / flat buffers in the shared arenas, collectives arena to arena; '+fused' = that, and ZeRO-2's "
-                       "reduce-scatters, AdamW and all-gather as one launch per rank"}
+                       "reduce-scatters, AdamW and all-gather as one launch per rank; '+hostwait' = DDP whose host waits for every bucket "
+                       "at the end of backward, as the reference's does (the default only orders the stream behind them)"}
     for s in strategies:
         res = launch(train_rank, world, s, steps, gpus=[0] * world, timeout=120.0)
         out[s] = {"step_ms": round(max(r["step_ms"] for r in res), 3), "loss": round(res[0]["loss"], 4),
@@ -758,9 +760,9 @@ def main():
             train4 = train_steps(5, 4, ("alone", "ddp", "zero2", "zero2+direct", "zero2+fused", "zero3"))
         except Exception as e:
             train4 = {"error": repr(e)[:300]}
-        os.environ["TANDEM_HIP_WAIT"] = "stream"  # wait() parks the training stream instead of blocking the host
+        os.environ["TANDEM_HIP_WAIT"] = "stream"  # every wait() parks the training stream instead of blocking the host
         try:
-            train["stream_ordered_wait"] = {k: v["step_ms"] for k, v in train_steps(5, 2, ("ddp", "ddp+direct", "zero2")).items()
+            train["stream_ordered_wait"] = {k: v["step_ms"] for k, v in train_steps(5, 2, ("ddp+direct", "zero2")).items()
                                             if k != "workload"}
         except Exception as e:
             train["stream_ordered_wait"] = {"error": repr(e)[:300]}

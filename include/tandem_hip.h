@@ -456,6 +456,13 @@ int tdm_barrier(tdm_engine* e, tdm_work** out);
  * (inputs ready, first kernel not yet begun) and finished its last kernel instead, on
  * the same clock: this form blocks the host until the GPU has finished it. */
 int tdm_work_wait(tdm_work* w, tdm_stream caller);
+/* wait for callers that only need the ORDER: if the collective has not run yet, `caller` is made to wait for
+ * the word the engine sets behind the collective's last kernel and the call returns at once, whatever
+ * TANDEM_HIP_WAIT says (where the device cannot park a stream on a value, and when the collective has already run,
+ * this is tdm_work_wait). The host can then queue work behind a collective that is still in flight; a failure of
+ * that collective is returned by the next call on the engine instead of by this one. No counterpart in the
+ * reference, whose CUDA engine orders its hand-over on the GPU and so never blocks a waiting host for it. */
+int tdm_work_wait_stream(tdm_work* w, tdm_stream caller);
 int tdm_work_done(tdm_work* w);
 int tdm_work_times(tdm_work* w, double* started, double* finished);
 int tdm_work_free(tdm_work* w);

@@ -135,6 +135,7 @@ _ENGINE_SIGNATURES = {
     "tdm_unit_gather_direct": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _VP, _PI64, ctypes.c_int, _PI64,
                                               ctypes.c_int, _VP, _PVP]),
     "tdm_work_wait": (ctypes.c_int, [_VP, _VP]),
+    "tdm_work_wait_stream": (ctypes.c_int, [_VP, _VP]),
     "tdm_work_done": (ctypes.c_int, [_VP]),
     "tdm_work_times": (ctypes.c_int, [_VP, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
     "tdm_work_free": (ctypes.c_int, [_VP]),

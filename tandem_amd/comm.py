@@ -43,13 +43,19 @@ class Work:
         self._recorded = False
         self._waited = False
 
-    def wait(self):
+    def wait(self, stream_ordered=False):
+        """Returns the collective's result once the caller's current stream is ordered behind it
+        (tandem/comm.py:92-107 in the reference). stream_ordered=True: a collective that has not run yet is not
+        waited for on the host; the stream is parked on it and the call returns at once, so the host can go on
+        queueing work (an optimizer's launches, say) behind it. A failure of such a collective is raised by the
+        next call on the group instead of by this one."""
         g = self._group
         if self._handle is None:
             return self.result
         t0 = time.perf_counter() if g.tracing and not self.is_completed() else None
         try:
-            check(lib().tdm_work_wait(self._handle, _lib.stream_ptr(g.device)))
+            wait = lib().tdm_work_wait_stream if stream_ordered else lib().tdm_work_wait
+            check(wait(self._handle, _lib.stream_ptr(g.device)))
         except Exception as e:
             raise CommError(f"{self.name} failed") from e
         if t0 is not None:
@@ -74,6 +80,8 @@ class Work:
 
 class Group:
     """One rank's view of the group."""
+
+    stream_ordered_waits = True  # Work.wait(stream_ordered=True) exists (the wrappers ask before they use it)
 
     def __init__(self, rank, size, device, sync, queues=None, slot_bytes=DEFAULT_SLOT_BYTES, slots=DEFAULT_SLOTS,
                  timeout=DEFAULT_TIMEOUT, transport=None, priority=None, backend=None, job=None):

@@ -77,8 +77,9 @@ struct Work {
   // time stamps, placed on the host clock through the engine's anchor.
   hipEvent_t start_event = nullptr;
   std::shared_ptr<Anchor> anchor;
-  // Stream-ordered waiting (TANDEM_HIP_WAIT=stream): the word the caller's stream waits for.
+  // Stream-ordered waiting (tdm_work_wait_stream; TANDEM_HIP_WAIT=stream): the word the caller's stream waits for.
   std::shared_ptr<FlagPool> flags;
+  bool defer_default = false;  // tdm_work_wait parks too
   int flag = -1;
   uint32_t flag_value = 0;  // the word reaches this value when the collective is over
 
@@ -197,8 +198,9 @@ class Engine {
   // staged collectives
   bool staged_ = true;               // TANDEM_HIP_ALGO=ring switches them off
   bool gathers_on_side_stream_ = false;  // TANDEM_HIP_GATHER=stream
-  std::shared_ptr<FlagPool> flags_;      // TANDEM_HIP_WAIT=stream
-  bool want_flags_ = false;
+  std::shared_ptr<FlagPool> flags_;      // the words that tdm_work_wait_stream parks streams on
+  bool want_flags_ = false;              // the device can make a stream wait for a value
+  bool defer_default_ = false;           // TANDEM_HIP_WAIT=stream: tdm_work_wait parks as well
   std::string sticky_error_;             // under mu_: a collective failed after its wait() had already returned
   bool ready_on_host_ = true;        // TANDEM_HIP_READY=gpu: wait for the caller's stream on the GPU instead
   // bytes per half (TANDEM_HIP_STAGING_BYTES). Two ranks, all_reduce of 256 MiB / 1 GiB: 0.52 / 1.93 ms with 64 MiB halves,

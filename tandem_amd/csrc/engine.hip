@@ -67,14 +67,19 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
     if (v < 0) throw Invalid("TANDEM_HIP_SMALL_BYTES must not be negative");
     small_bytes_ = static_cast<size_t>(v);
   }
-  if (const char* wm = std::getenv("TANDEM_HIP_WAIT")) {
-    if (std::string(wm) == "stream") {
-      int can = 0;
-      (void)hipDeviceGetAttribute(&can, hipDeviceAttributeCanUseStreamWaitValue, device);
-      if (can != 1) throw Invalid("TANDEM_HIP_WAIT=stream: this device cannot make a stream wait for a value");
-      want_flags_ = true;
-    } else if (std::string(wm) != "host") {
-      throw Invalid("TANDEM_HIP_WAIT must be \"host\" or \"stream\"");
+  {
+    // Every Work gets a word that streams can be parked on (tdm_work_wait_stream) where the device can do that;
+    // TANDEM_HIP_WAIT=stream makes the plain tdm_work_wait park too.
+    int can = 0;
+    (void)hipDeviceGetAttribute(&can, hipDeviceAttributeCanUseStreamWaitValue, device);
+    want_flags_ = can == 1;
+    if (const char* wm = std::getenv("TANDEM_HIP_WAIT")) {
+      if (std::string(wm) == "stream") {
+        if (!want_flags_) throw Invalid("TANDEM_HIP_WAIT=stream: this device cannot make a stream wait for a value");
+        defer_default_ = true;
+      } else if (std::string(wm) != "host") {
+        throw Invalid("TANDEM_HIP_WAIT must be \"host\" or \"stream\"");
+      }
     }
   }
   if (const char* gm = std::getenv("TANDEM_HIP_GATHER")) gathers_on_side_stream_ = std::string(gm) == "stream";
@@ -249,6 +254,7 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
   if (flags_ && uses_gpu) {
     work->flag = flags_->acquire(&work->flag_value);
     if (work->flag >= 0) work->flags = flags_;
+    work->defer_default = defer_default_;
   }
   hipEvent_t ready = nullptr;
   if (uses_gpu) {

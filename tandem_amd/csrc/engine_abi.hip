@@ -206,13 +206,20 @@ int tdm_barrier(tdm_engine* e, tdm_work** out) {
   });
 }
 
-int tdm_work_wait(tdm_work* w, tdm_stream caller) {
+static int wait_for(tdm_work* w, tdm_stream caller, bool may_park);
+
+int tdm_work_wait(tdm_work* w, tdm_stream caller) { return wait_for(w, caller, w && w->impl && w->impl->defer_default); }
+
+int tdm_work_wait_stream(tdm_work* w, tdm_stream caller) { return wait_for(w, caller, true); }
+
+// may_park: a collective that has not run yet is not waited for on the host; the caller's stream is parked on its word.
+static int wait_for(tdm_work* w, tdm_stream caller, bool may_park) {
   if (w == nullptr || !w->impl) {
     set_last_error("NULL work");
     return TDM_EINVAL;
   }
   Work& work = *w->impl;
-  if (work.flag >= 0 && !work.finished_hint.load(std::memory_order_acquire)) {
+  if (may_park && work.flag >= 0 && !work.finished_hint.load(std::memory_order_acquire)) {
     // The job has not run yet: park the caller's stream on its word and return. The host
     // goes on queueing work behind the collective; a failure shows at the next call.
     return guard([&] {

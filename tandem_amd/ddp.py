@@ -44,8 +44,12 @@ class Bucket:
 
 
 class DDP(torch.nn.Module):
-    def __init__(self, module, group, bucket_bytes=25 << 20, overlap=True, rebuild=True, direct=False):
-        """direct: the buckets live in the group's shared arena (one is created if the
+    def __init__(self, module, group, bucket_bytes=25 << 20, overlap=True, rebuild=True, direct=False, stream_ordered=True):
+        """stream_ordered: at the end of backward the training stream is ordered behind the buckets' all-reduces
+        without the host waiting for them (`Work.wait(stream_ordered=True)`), so the optimizer's launches are
+        queued while the last buckets are still in flight; a bucket that fails then raises from the next collective
+        instead of from this backward. False: the host waits, as the reference's DDP does (tandem/ddp.py:111-115).
+        direct: the buckets live in the group's shared arena (one is created if the
         group has none: the gradients' size plus padding, under 2 GiB) and every
         all-reduce runs arena to arena (`group.all_reduce(..., direct=True)`): same
         bits, 2.5 instead of 4.5 passes over a bucket per rank at two ranks, three
@@ -57,6 +61,7 @@ class DDP(torch.nn.Module):
             raise TypeError("DDP(direct=True) needs a group with a shared arena (tandem_amd.Group has one)")
         self.module, self.g = module, group
         self.direct, self._pools = bool(direct), {}
+        self.stream_ordered = bool(stream_ordered) and getattr(group, "stream_ordered_waits", False)
         self.bucket_bytes, self.overlap = bucket_bytes, overlap
         self._rebuild_pending = rebuild
         self.params = [p for p in module.parameters() if p.requires_grad]
@@ -160,7 +165,7 @@ class DDP(torch.nn.Module):
             unused = [tuple(p.shape) for b in short for p in b.params if p.grad is None]
             raise RuntimeError(f"tandem DDP: some parameters received no gradient ({unused[:3]}...); every parameter must be used")
         for b in self.buckets:
-            b.work.wait()
+            b.work.wait(stream_ordered=True) if self.stream_ordered else b.work.wait()
             b.arrived, b.work = 0, None
         self._cursor = 0
         if self._rebuild_pending and len(self._arrival) == len(self.params):

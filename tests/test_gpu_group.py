@@ -765,3 +765,36 @@ def test_unknown_backend_and_cpu_device_are_refused():
         launch(failing, 2, backend="python")
     with pytest.raises(CommError, match="no CPU path"):
         Group(0, 1, "cpu", None, backend="hip", job="x")
+
+
+def stream_ordered_waits(g):
+    """Work.wait(stream_ordered=True): the call may return before the collective has run; whatever the caller's
+    stream does next must still see the reduced tensor. The stream is kept busy first, so that most waits find their
+    collective still queued."""
+    dev, w = g.device, g.size
+    n = 300_001
+    busy = torch.randn(1024, 1024, device=dev)
+    ok, parked = True, 0
+    for k in range(40):
+        x = torch.full((n,), float(g.rank + 1 + k), device=dev)
+        for _ in range(3):
+            busy = (busy @ busy) * 1e-3  # the all-reduce's inputs are ready only after these
+        x += busy[0, 0] * 0  # (a dependency on the busy work)
+        work = g.all_reduce(x, async_op=True)
+        parked += 0 if work.is_completed() else 1
+        out = work.wait(stream_ordered=True)
+        y = out * 2  # queued right behind the wait
+        want = 2.0 * sum(q + 1 + k for q in range(w))
+        ok = ok and bool((y == want).all())
+    g.barrier()
+    torch.cuda.synchronize()
+    return ok, parked
+
+
+@pytest.mark.parametrize("world", [2, 3])
+def test_waits_that_only_order_the_stream(world):
+    from tandem_amd import launch
+
+    for ok, parked in launch(stream_ordered_waits, world, gpus=[0] * world, timeout=TIMEOUT):
+        assert ok
+        assert parked > 0, "every collective had run before its wait: the test did not exercise the parked path"
