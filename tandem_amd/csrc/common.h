@@ -76,7 +76,8 @@ inline SegPlan plan_segment(const uintptr_t* ptrs, int n, int64_t count, int es,
 void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool scale_dst, bool scale_src,
                  bool writeback_src, hipStream_t stream, int policy = 2);
 void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream, int policy = 2);
-void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream);
+// divide_by: what averaging divides by when that is not `world` (a partial sum of a larger ring: world = the terms folded)
+void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream, int divide_by = 0);
 // kernels_chain.hip: the ring reduce-scatter of a whole group in one launch (rank q's buffer at base[q], chunk c =
 // elements [lo[c], lo[c] + len[c])); world sizes 2..kChainMaxWorld. Returns false, with nothing launched, when the ranks'
 // copies of some chunk disagree within 16 bytes: the kernel has no element-by-element path (it would set its register

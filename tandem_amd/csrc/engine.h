@@ -148,7 +148,7 @@ class Engine {
   void staged_all_reduce(const Buf& t, bool average);
   void staged_all_reduce_small(const Buf& t, bool average);
   void staged_all_gather(const Buf& t, const std::vector<Chunk>& cs, const char* own);
-  void staged_reduce_scatter_owner(const Buf& t, const std::vector<Chunk>& cs, bool average);
+  void staged_reduce_scatter(const Buf& t, const std::vector<Chunk>& cs, bool average, bool partial_sums);
   void direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets, const char** base);
   void direct_fold(const Buf& t, const std::vector<Chunk>& cs, const char* const* base, bool average);
   void direct_copies(const Buf& t, const std::vector<Chunk>& cs, const char* const* base);

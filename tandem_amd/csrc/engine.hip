@@ -747,11 +747,14 @@ void Engine::staged_all_reduce(const Buf& t, bool average) {
   }
 }
 
-// reduce_scatter when only the owner's chunk is wanted (the ring also leaves partial
-// sums in the other chunks; ZeRO drops them). Per pass over a window of `half` bytes of
-// the tensor: copy the window's parts of the chunks I do not own into my staging, at
-// the same offsets; fence; fold my chunk's part out of my tensor and the peers' stagings.
-void Engine::staged_reduce_scatter_owner(const Buf& t, const std::vector<Chunk>& cs, bool average) {
+// reduce_scatter through the stagings. Per pass over a window of `half` bytes of the tensor: copy the
+// window's parts of the chunks I do not own into my staging, at the same offsets; fence; fold my chunk's
+// part out of my tensor and the peers' stagings. partial_sums: the ring also leaves, in chunk c of rank
+// c + k, the sum after k terms (tandem/comm.py:350-352 in the reference; ZeRO drops them and asks for
+// the owner's chunk only). Every rank then folds those too, each out of the stagings of the ranks the
+// ring would have passed before it, in the ring's order, and with the whole group's divisor: k - 1
+// staged copies and its own, written over its own. One handshake per pass instead of two per 4 MiB piece.
+void Engine::staged_reduce_scatter(const Buf& t, const std::vector<Chunk>& cs, bool average, bool partial_sums) {
   const int es = elem_bytes(t.dtype), n = size_, r = rank_;
   const int64_t cap = static_cast<int64_t>(staging_half_) / es;
   for (int64_t at = 0; at < t.numel; at += cap) {
@@ -782,6 +785,27 @@ void Engine::staged_reduce_scatter_owner(const Buf& t, const std::vector<Chunk>&
       seg.count = hi(r) - lo(r);
       seg.chunk = r;
       fold_step(&seg, 1, n, t.dtype, average, stream_);
+    }
+    if (!partial_sums) continue;
+    for (int k = 1; k < n; ++k) {  // chunk c = r - k: I am the k-th rank the ring passes with it
+      const int c = mod(r - k, n);
+      if (hi(c) <= lo(c)) continue;
+      char* own = t.ptr + lo(c) * es;
+      if (k == 1) {  // the first sender's own term, divided when averaging (the reference divides the whole tensor first)
+        if (average) {
+          tdm_pair pr{own, own, hi(c) - lo(c)};
+          copy_step(&pr, 1, t.dtype, n, stream_);
+        }
+        continue;
+      }
+      tdm_fold_seg seg;
+      std::memset(&seg, 0, sizeof seg);
+      for (int j = 0; j < k - 1; ++j) seg.src[j] = peer_staging(mod(c + 1 + j, n), half) + (lo(c) - at) * es;
+      seg.src[k - 1] = own;  // my term is added last
+      seg.dst[0] = own;
+      seg.count = hi(c) - lo(c);
+      seg.chunk = k - 1;  // a fold over k sources starts at source (chunk + 1) % k = 0
+      fold_step(&seg, 1, k, t.dtype, average, stream_, n);
     }
   }
 }
@@ -884,7 +908,7 @@ std::shared_ptr<Work> Engine::reduce_scatter(Buf t, std::vector<int64_t> sizes, 
   return submit([this, t, sizes, average, owner_only] {
     if (size_ == 1) return;
     const auto cs = chunks(t, sizes);
-    if (owner_only && staged_ && size_ <= TDM_MAX_WORLD) staged_reduce_scatter_owner(t, cs, average);
+    if (staged_ && size_ <= TDM_MAX_WORLD) staged_reduce_scatter(t, cs, average, !owner_only);
     else ring_reduce_scatter(cs, t.dtype, average, true);
   }, caller, true, ready_on_host_);
 }

@@ -292,8 +292,9 @@ void launch_fold_w(const void* image, int64_t tiles, int average, hipStream_t st
 }
 
 template <typename T, int kWorld>
-void launch_fold_small_w(const FoldSmall& table, int average, hipStream_t stream) {
-  const Divisor<T> dv = make_divisor<T>(kWorld);
+void launch_fold_small_w(const FoldSmall& table, int average, hipStream_t stream, int divide_by) {
+  const int divisor = divide_by > 0 ? divide_by : kWorld;
+  const Divisor<T> dv = make_divisor<T>(divisor);
   // bytes touched: every tile is read from kWorld ranks (and written back to most of them)
   const bool cold = table.tile_end[table.nseg - 1] * static_cast<int64_t>(kTileVecs) * 16 * kWorld >= cold_footprint(kWorld);
   const dim3 grid(grid_for(table.tile_end[table.nseg - 1] * (cold ? fold_small_parts<kWorld>() : 1))), block(kThreads);
@@ -303,7 +304,7 @@ void launch_fold_small_w(const FoldSmall& table, int average, hipStream_t stream
     if (cold) hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv);
     else hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv);
   } else {
-    switch (div_kind(kWorld, average != 0) * 2 + (cold ? 1 : 0)) {
+    switch (div_kind(divisor, average != 0) * 2 + (cold ? 1 : 0)) {
       case 0: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
       case 1: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 0, true>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
       case 2: hipLaunchKernelGGL((k2_fold_small_kernel<T, kWorld, 1, false>), grid, block, occupancy_pad(TDM_XCD_FOLD, cold), stream, tab, dv); break;
@@ -315,15 +316,15 @@ void launch_fold_small_w(const FoldSmall& table, int average, hipStream_t stream
 }
 
 template <typename T>
-void launch_fold_small(const FoldSmall& tab, int world, int average, hipStream_t stream) {
+void launch_fold_small(const FoldSmall& tab, int world, int average, hipStream_t stream, int divide_by = 0) {
   switch (world) {
-    case 2: launch_fold_small_w<T, 2>(tab, average, stream); break;
-    case 3: launch_fold_small_w<T, 3>(tab, average, stream); break;
-    case 4: launch_fold_small_w<T, 4>(tab, average, stream); break;
-    case 5: launch_fold_small_w<T, 5>(tab, average, stream); break;
-    case 6: launch_fold_small_w<T, 6>(tab, average, stream); break;
-    case 7: launch_fold_small_w<T, 7>(tab, average, stream); break;
-    case 8: launch_fold_small_w<T, 8>(tab, average, stream); break;
+    case 2: launch_fold_small_w<T, 2>(tab, average, stream, divide_by); break;
+    case 3: launch_fold_small_w<T, 3>(tab, average, stream, divide_by); break;
+    case 4: launch_fold_small_w<T, 4>(tab, average, stream, divide_by); break;
+    case 5: launch_fold_small_w<T, 5>(tab, average, stream, divide_by); break;
+    case 6: launch_fold_small_w<T, 6>(tab, average, stream, divide_by); break;
+    case 7: launch_fold_small_w<T, 7>(tab, average, stream, divide_by); break;
+    case 8: launch_fold_small_w<T, 8>(tab, average, stream, divide_by); break;
     default: throw Invalid("the direct fold handles world sizes 2..8");
   }
 }
@@ -696,7 +697,7 @@ void local_all_reduce_fold(const LocalRanks& lr, bool average, hipStream_t strea
 
 // Up to 8 segments folded in one launch, the table passed by value. Used by the
 // engine too (a rank folding its own chunk out of its peers' shared arenas).
-void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream) {
+void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream, int divide_by) {
   const int es = elem_size(dtype);
   if (es == 0) throw Invalid("unknown dtype " + std::to_string(dtype));
   if (world < 2 || world > TDM_MAX_WORLD) throw Invalid("the direct fold handles world sizes 2..8");
@@ -734,10 +735,10 @@ void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool av
   tab.nseg = k;
   if (k == 0) return;
   switch (dtype) {
-    case TDM_F32: launch_fold_small<float>(tab, world, average, stream); break;
-    case TDM_F64: launch_fold_small<double>(tab, world, average, stream); break;
-    case TDM_F16: launch_fold_small<f16_t>(tab, world, average, stream); break;
-    case TDM_BF16: launch_fold_small<bf16_t>(tab, world, average, stream); break;
+    case TDM_F32: launch_fold_small<float>(tab, world, average, stream, divide_by); break;
+    case TDM_F64: launch_fold_small<double>(tab, world, average, stream, divide_by); break;
+    case TDM_F16: launch_fold_small<f16_t>(tab, world, average, stream, divide_by); break;
+    case TDM_BF16: launch_fold_small<bf16_t>(tab, world, average, stream, divide_by); break;
     case TDM_I64: launch_fold_small<int64_t>(tab, world, 0, stream); break;
     case TDM_I32: launch_fold_small<int32_t>(tab, world, 0, stream); break;
     case TDM_I16: launch_fold_small<int16_t>(tab, world, 0, stream); break;
