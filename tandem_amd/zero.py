@@ -208,7 +208,11 @@ class ZeRO(torch.nn.Module):
             return
         grad = self.grad[lo:hi] if self.stage == 1 else self.grad_shard
         self.opt.update("flat", self.buf[lo:hi], grad)
-        self.g.all_gather(self.buf, self.flat.sizes, **self._how)
+        if getattr(self.g, "stream_ordered_waits", False):
+            # the next forward only has to come after the gather on the stream: the host does not wait for it
+            self.g.all_gather(self.buf, self.flat.sizes, async_op=True, **self._how).wait(stream_ordered=True)
+        else:
+            self.g.all_gather(self.buf, self.flat.sizes, **self._how)
 
     @property
     def _how(self):
