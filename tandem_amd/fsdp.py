@@ -28,6 +28,7 @@ import torch
 from torch.autograd import Variable
 
 from .buckets import FlatLayout
+from .comm import CommError
 from .optim import ShardedAdamW
 
 RELEASED, GATHERING, WHOLE = "released", "gathering", "whole"
@@ -230,7 +231,9 @@ class FSDP(torch.nn.Module):
             sizes = [FlatLayout([p.numel() for p in ps], group.size, 0).sizes for _, ps in owned]
             try:
                 home = ShardHome(group, sizes, owned[0][1][0].dtype)
-            except Exception:
+            except CommError:
+                if direct:  # asked for by name: say why it cannot be had
+                    raise
                 self._direct = False  # does not fit one exported allocation: gathers go through the group's own path
         self.units, self._unit_of = [], {}
         for k, (module, params) in enumerate(owned):
