@@ -52,6 +52,9 @@ struct FlagPool {
     std::lock_guard<std::mutex> lock(mu);
     free_list.push_back(i);
   }
+  bool reached(int i, uint32_t value) const {  // as hipStreamWaitValueGte compares
+    return reinterpret_cast<const volatile uint32_t*>(base)[i] >= value;
+  }
   void set(int i, uint32_t value) {
     reinterpret_cast<volatile uint32_t*>(base)[i] = value;
     std::atomic_thread_fence(std::memory_order_seq_cst);
@@ -66,7 +69,7 @@ struct Work {
   int status = TDM_OK;
   std::string error;
   double t0 = 0, t1 = 0;
-  hipEvent_t done_event = nullptr;  // recorded on the engine's stream after the job (jobs with GPU work)
+  hipEvent_t done_event = nullptr;  // recorded on the engine's stream after the job: jobs with GPU work that have no flag word, or are timed
   bool uses_gpu = false;
   bool on_callers_stream = false;  // its kernels were launched on the submitting stream itself:
   hipStream_t launched_on = nullptr;  // wait() from that stream has nothing to order
@@ -150,7 +153,7 @@ class Engine {
   void staged_all_gather(const Buf& t, const std::vector<Chunk>& cs, const char* own);
   void staged_reduce_scatter(const Buf& t, const std::vector<Chunk>& cs, bool average, bool partial_sums);
   void direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets, const char** base);
-  void direct_fold(const Buf& t, const std::vector<Chunk>& cs, const char* const* base, bool average);
+  void direct_fold(const Buf& t, const std::vector<Chunk>& cs, const char* const* base, bool average, bool to_all);
   void direct_copies(const Buf& t, const std::vector<Chunk>& cs, const char* const* base);
   void start();
   void release_device();

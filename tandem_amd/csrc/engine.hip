@@ -349,7 +349,9 @@ void Engine::loop() {
     } catch (...) {
       status = TDM_ERUNTIME; error = "unknown error";
     }
-    if (status == TDM_OK && w.uses_gpu && !(w.drained && !w.start_event)) {
+    // Its end on the GPU: the flag word where the job has one (written by the engine's stream below), an event
+    // where it has none, and for the time stamps.
+    if (status == TDM_OK && w.uses_gpu && (w.start_event || (w.flag < 0 && !w.drained))) {
       if (hipEventCreateWithFlags(&w.done_event, w.start_event ? hipEventDefault : hipEventDisableTiming) != hipSuccess ||
           hipEventRecord(w.done_event, stream_) != hipSuccess) {
         status = TDM_ERUNTIME;
@@ -1097,14 +1099,15 @@ std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, st
 // For tensors that live in the ranks' shared arenas. No slots and no per-piece
 // messages: a rank reads its peers' tensors where they lie.
 //   all_reduce      fence; fold my chunk out of all ranks' tensors, in the ring's order
-//                   for that chunk, into my tensor; fence; copy every other chunk from
-//                   its owner's tensor; fence.
-//   reduce_scatter  fence; the same fold; fence. Only the owner's chunk is produced.
-//   all_gather      fence; the same copies; fence.
-// Per rank and element of the tensor that is (W+1)/W + 2(W-1)/W accesses for an
-// all-reduce where the slot ring makes 9(W-1)/W, and three handshakes in all instead
-// of two per piece. The first fence says every rank's input is complete, the last
-// that nobody reads a tensor any more, so the caller may change it again.
+//                   for that chunk, into every rank's tensor (one kernel, W reads and W
+//                   writes per element of the chunk); fence.
+//   reduce_scatter  fence; the same fold into my tensor only; fence. Only the owner's
+//                   chunk is produced.
+//   all_gather      fence; copy every other chunk from its owner's tensor; fence.
+// Per rank and element of the tensor that is 2 accesses for an all-reduce where the
+// slot ring makes 9(W-1)/W, and two handshakes in all instead of two per piece. The
+// first fence says every rank's input is complete, the last that nobody reads or
+// writes a tensor any more, so the caller may change it again.
 void Engine::direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets, const char** base) {
   const int es = elem_bytes(t.dtype);
   const size_t bytes = static_cast<size_t>(t.numel) * es;
@@ -1128,13 +1131,18 @@ void Engine::direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets
   }
 }
 
-void Engine::direct_fold(const Buf& t, const std::vector<Chunk>& cs, const char* const* base, bool average) {
+// to_all: the folded chunk is also written into every peer's tensor (their arenas are mapped writable). Chunk r of
+// every rank's tensor is read and written by rank r's kernel alone, so the ranks' kernels need no order among them.
+void Engine::direct_fold(const Buf& t, const std::vector<Chunk>& cs, const char* const* base, bool average, bool to_all) {
   const Chunk& mine = cs[rank_];
   if (mine.numel == 0) return;
   tdm_fold_seg seg;
   std::memset(&seg, 0, sizeof seg);
   const size_t lo = static_cast<size_t>(mine.ptr - t.ptr);
   for (int q = 0; q < size_; ++q) seg.src[q] = base[q] + lo;
+  if (to_all) {
+    for (int q = 0; q < size_; ++q) seg.dst[q] = const_cast<char*>(base[q]) + lo;
+  }
   seg.dst[rank_] = mine.ptr;
   seg.count = mine.numel;
   seg.chunk = rank_;
@@ -1175,14 +1183,9 @@ std::shared_ptr<Work> Engine::direct(int kind, Buf t, std::vector<int64_t> sizes
     // The peers' arenas are looked up behind the first fence: a rank that has reached it has shared its
     // arena, so the first direct collective of a group needs no barrier of the caller's before it.
     if (t.numel > 0) direct_bases(t, peer_offsets, base);  // an empty tensor still takes part in the fences
-    if (kind != 2) {
-      direct_fold(t, cs, base, average);
-      barrier_now(true);  // every chunk is folded (or, for reduce_scatter: nobody reads our tensor any more)
-    }
-    if (kind != 1) {
-      direct_copies(t, cs, base);
-      barrier_now(true);  // nobody reads our tensor any more
-    }
+    if (kind == 2) direct_copies(t, cs, base);
+    else direct_fold(t, cs, base, average, kind == 0);  // all_reduce: every rank's copy of my chunk written by my fold
+    barrier_now(true);  // nobody reads or writes our tensor any more
   }, caller, true, true, true);
 }
 

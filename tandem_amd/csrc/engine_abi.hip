@@ -237,10 +237,19 @@ static int wait_for(tdm_work* w, tdm_stream caller, bool may_park) {
       return work.status;
     }
   }
-  if (work.done_event && !(work.on_callers_stream && work.launched_on == static_cast<hipStream_t>(caller))) {
+  if (work.on_callers_stream && work.launched_on == static_cast<hipStream_t>(caller)) return TDM_OK;
+  if (work.flag >= 0) {
+    if (work.flags->reached(work.flag, work.flag_value)) return TDM_OK;  // the GPU is past it already: nothing to order
+    return guard([&] {
+      check_hip(hipStreamWaitValue32(static_cast<hipStream_t>(caller), work.flags->base + work.flag, work.flag_value,
+                                     hipStreamWaitValueGte, 0xffffffffu),
+                "hipStreamWaitValue32 (wait)");
+    });
+  }
+  if (work.done_event) {
     return guard([&] {
       const hipError_t q = hipEventQuery(work.done_event);
-      if (q == hipSuccess) return;  // the GPU is past it already: nothing to order
+      if (q == hipSuccess) return;
       if (q == hipErrorNotReady) (void)hipGetLastError();
       check_hip(hipStreamWaitEvent(static_cast<hipStream_t>(caller), work.done_event, 0), "hipStreamWaitEvent (wait)");
     });
@@ -253,7 +262,9 @@ int tdm_work_done(tdm_work* w) {
   Work& work = *w->impl;
   std::lock_guard<std::mutex> lock(work.mu);
   if (!work.finished) return 0;
-  if (work.status == TDM_OK && work.done_event) return hipEventQuery(work.done_event) == hipSuccess ? 1 : 0;
+  if (work.status != TDM_OK) return 1;
+  if (work.flag >= 0) return work.flags->reached(work.flag, work.flag_value) ? 1 : 0;
+  if (work.done_event) return hipEventQuery(work.done_event) == hipSuccess ? 1 : 0;
   return 1;
 }
 
