@@ -798,3 +798,30 @@ def test_waits_that_only_order_the_stream(world):
     for ok, parked in launch(stream_ordered_waits, world, gpus=[0] * world, timeout=TIMEOUT):
         assert ok
         assert parked > 0, "every collective had run before its wait: the test did not exercise the parked path"
+
+
+def more_works_than_words(g):
+    """Every Work in flight owns one of the engine's 1024 done words; those beyond wait on an event as before."""
+    dev, w = g.device, g.size
+    count, n = 1100, 257
+    rows = torch.arange(count, device=dev, dtype=torch.float32).unsqueeze(1).expand(count, n)
+    x = (rows + float(g.rank)).contiguous()
+    works = [g.all_reduce(x[k], async_op=True) for k in range(count)]
+    done_before = sum(wk.is_completed() for wk in works)
+    for wk in works:
+        wk.wait()
+    y = x * 1  # on the caller's stream, behind every wait
+    ok = bool((y == rows * w + float(sum(range(w)))).all()) and all(wk.is_completed() for wk in works[:8])
+    torch.cuda.synchronize()
+    ok = ok and all(wk.is_completed() for wk in works)
+    del works
+    z = torch.ones(5, device=dev)
+    g.all_reduce(z)  # the words are free again
+    return ok and bool((z == w).all()), done_before
+
+
+def test_more_collectives_in_flight_than_done_words():
+    from tandem_amd import launch
+
+    for ok, _ in launch(more_works_than_words, 2, gpus=[0, 0], timeout=TIMEOUT):
+        assert ok
