@@ -1232,7 +1232,7 @@ int tdm_k4_unit_gather_all(void* const* fulls, const void* const* shards, const 
       s[q] = static_cast<const char*>(shards[q]);
     }
     const int64_t cap = static_cast<int64_t>(t_call_cus ? t_call_cus : compute_units()) * g_blocks_per_cu;
-        // Everything cached: what a gather writes is read by the unit's forward or backward straight away. (Twelve block units of
+    // Everything cached: what a gather writes is read by the unit's forward or backward straight away. (Twelve block units of
     // the 85.8M GPT gathered in turn at world 2: 19.4 us per unit with two vectors per lane, 18.8 with one; 17.6-18.0 with
     // non-temporal accesses, which would leave the consumer to fetch the unit from HBM.)
     unit_gather_multicast(f, s, sizes, world, es, false, occupancy_pad(TDM_XCD_COPY, false), xcd_shift(TDM_XCD_COPY, world, false), 1,
