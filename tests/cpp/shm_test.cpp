@@ -192,6 +192,45 @@ static int ring_two_processes(int slots, int count) {
   return 0;
 }
 
+// two threads, for the data-race sanitizer: the sender fills a payload slot with plain stores before it publishes, the
+// receiver reads the slot after ring_read and then releases; a slot is rewritten only once the ring has room again.
+// That is the engine's use of a ring (a message means the bytes have landed, a release that they have been read), and
+// head's and tail's release/acquire pairs are all that orders the plain accesses.
+static int ring_two_threads(int slots, int count) {
+  const std::string name = unique_name("ring3");
+  Region mine;
+  mine.create(name, 2);
+  Ring& r = mine.entry(1)->ring;
+  constexpr int kWords = 8;
+  std::vector<uint64_t> payload(static_cast<size_t>(slots) * kWords);
+  std::atomic<int> sender_failed{0};
+  std::thread sender([&] {
+    try {
+      for (uint64_t k = 0; k < static_cast<uint64_t>(count); ++k) {
+        ring_wait_for_room(r, k, slots, 10.0, "sender: no room");
+        for (int i = 0; i < kWords; ++i) payload[(k % slots) * kWords + i] = k * kWords + i;
+        ring_publish(r, slots, k * 3 + 1);
+      }
+    } catch (...) {
+      sender_failed.store(1);
+    }
+  });
+  int bad = 0;
+  try {
+    for (uint64_t k = 0; k < static_cast<uint64_t>(count); ++k) {
+      if (ring_read(r, k, slots, 10.0, "receiver: nothing arrived") != k * 3 + 1) ++bad;
+      for (int i = 0; i < kWords; ++i) bad += payload[(k % slots) * kWords + i] != k * kWords + i;
+      ring_release(r);
+    }
+  } catch (const Timeout&) {
+    ++bad;
+  }
+  sender.join();
+  CHECK(bad == 0 && sender_failed.load() == 0);
+  CHECK(r.head.load() == static_cast<uint64_t>(count) && r.tail.load() == static_cast<uint64_t>(count));
+  return 0;
+}
+
 // the waiting helpers: spin_for gives up after its limit; wait_until returns as soon as the condition holds
 static int waiting() {
   const double t0 = now_s();
@@ -216,6 +255,7 @@ int main(int argc, char** argv) {
     if (which == "region_errors") return region_errors();
     if (which == "ring_one_process") return ring_one_process();
     if (which == "ring_two_processes") return ring_two_processes(argc > 2 ? std::atoi(argv[2]) : 2, argc > 3 ? std::atoi(argv[3]) : 1000);
+    if (which == "ring_two_threads") return ring_two_threads(argc > 2 ? std::atoi(argv[2]) : 2, argc > 3 ? std::atoi(argv[3]) : 1000);
     if (which == "waiting") return waiting();
   } catch (const std::exception& e) {
     std::fprintf(stderr, "unexpected exception: %s\n", e.what());
