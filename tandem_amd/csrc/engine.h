@@ -25,6 +25,7 @@ struct FlagPool {
   uint32_t* base = nullptr;
   std::mutex mu;
   std::vector<int> free_list;
+  std::vector<int> pending;  // released by their Works, not yet written by the GPU
   std::vector<uint32_t> generation;  // a word only ever grows: a stream still parked on an earlier
                                      // generation of it is let go by every later one as well
 
@@ -42,16 +43,28 @@ struct FlagPool {
   // A word and the value its owner will wait for; -1: none left (the Work then waits on the host as usual).
   int acquire(uint32_t* value) {
     std::lock_guard<std::mutex> lock(mu);
+    for (size_t k = 0; k < pending.size();) {  // words given back before the engine's stream had written them
+      if (reached(pending[k])) {
+        free_list.push_back(pending[k]);
+        pending[k] = pending.back();
+        pending.pop_back();
+      } else {
+        ++k;
+      }
+    }
     if (free_list.empty()) return -1;
     const int i = free_list.back();
     free_list.pop_back();
     *value = ++generation[i];
     return i;
   }
+  // A word whose write is still queued on the engine's stream is not handed out again until the write has landed:
+  // the next owner's value, set early by the host after a failure, would otherwise be overwritten by the smaller one.
   void release(int i) {
     std::lock_guard<std::mutex> lock(mu);
-    free_list.push_back(i);
+    (reached(i) ? free_list : pending).push_back(i);
   }
+  bool reached(int i) const { return reached(i, generation[i]); }  // its latest generation (callers hold mu)
   bool reached(int i, uint32_t value) const {  // as hipStreamWaitValueGte compares
     return reinterpret_cast<const volatile uint32_t*>(base)[i] >= value;
   }
