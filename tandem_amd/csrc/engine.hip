@@ -362,7 +362,19 @@ void Engine::loop() {
       // Whoever waits for the word on the GPU is let go behind the job's last kernel, by the
       // engine's own stream; after a failure (or with that stream idle anyway) at once, by the host.
       uint32_t* word = w.flags->base + w.flag;
-      if (status != TDM_OK || w.drained || hipStreamWriteValue32(stream_, word, w.flag_value, 0) != hipSuccess) {
+      if (status == TDM_OK && !w.drained && hipStreamWriteValue32(stream_, word, w.flag_value, 0) != hipSuccess) {
+        // The stream cannot say so itself: the host does, once the stream has run dry.
+        (void)hipGetLastError();
+        try {
+          const hipError_t err = poll_gpu([this] { return hipStreamQuery(stream_); }, timeout_s_);
+          if (err != hipSuccess) throw std::runtime_error(hipGetErrorString(err));
+        } catch (const std::exception& e) {
+          status = TDM_ERUNTIME;
+          error = std::string("could not signal the collective's end: ") + e.what();
+        }
+        (void)hipGetLastError();
+        w.flags->set(w.flag, w.flag_value);
+      } else if (status != TDM_OK || w.drained) {
         w.flags->set(w.flag, w.flag_value);
       }
       if (status != TDM_OK) {  // its wait() may have returned long ago: the next call reports it
