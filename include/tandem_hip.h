@@ -408,11 +408,13 @@ int tdm_fence(tdm_engine* e, tdm_stream caller, tdm_work** out);
  * for bit, by reading the peers' tensors where they lie instead of passing pieces
  * through slots:
  *   all_reduce      fence; this rank folds its own ring chunk out of all W tensors in
- *                   the ring's order for that chunk (the sum order of tandem/comm.py:301-305),
- *                   in place; fence; it copies every other chunk from its owner; fence.
- *   reduce_scatter  fence; the same fold; fence. Unlike the ring (tandem/comm.py:350-352),
- *                   the chunks this rank does not own are left as they were.
- *   all_gather      fence; the same copies; fence.
+ *                   the ring's order for that chunk (the sum order of tandem/comm.py:301-305)
+ *                   and writes the result into all W tensors (the arenas are mapped
+ *                   writable; chunk r of every tensor is touched by rank r alone); fence.
+ *   reduce_scatter  fence; the same fold, written into this rank's tensor only; fence.
+ *                   Unlike the ring (tandem/comm.py:350-352), the chunks this rank does
+ *                   not own are left as they were.
+ *   all_gather      fence; this rank copies every other chunk from its owner; fence.
  * World sizes up to 8 for the two that reduce. The tensors must not change between
  * the call and the end of the Work on any rank. */
 int tdm_direct_all_reduce(tdm_engine* e, void* ptr, int64_t numel, int dtype, int average, const int64_t* peer_offsets,

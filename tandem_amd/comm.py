@@ -223,8 +223,8 @@ class Group:
     def all_reduce(self, t, op="sum", async_op=False, direct=False):
         """Ring all-reduce in place: reduce-scatter, then all-gather. With `direct`
         (tensors in the ranks' shared arenas) each rank folds its own chunk straight
-        out of its peers' tensors, in the ring's order, and copies the other chunks
-        from their owners: the same bits, without slots."""
+        out of its peers' tensors, in the ring's order, and writes the result into
+        every rank's tensor: the same bits, without slots."""
         if op not in ("sum", "avg"):
             raise CommError(f"unknown op {op}")
         flat = self._flat(t, "all_reduce")

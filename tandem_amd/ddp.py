@@ -52,7 +52,7 @@ class DDP(torch.nn.Module):
         direct: the buckets live in the group's shared arena (one is created if the
         group has none: the gradients' size plus padding, under 2 GiB) and every
         all-reduce runs arena to arena (`group.all_reduce(..., direct=True)`): same
-        bits, 2.5 instead of 4.5 passes over a bucket per rank at two ranks, three
+        bits, 2 instead of 4.5 passes over a bucket per rank at two ranks, two
         handshakes per bucket instead of two per 4 MiB piece."""
         super().__init__()
         if not hasattr(group, "pack"):
