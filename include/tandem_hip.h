@@ -388,22 +388,27 @@ int tdm_broadcast(tdm_engine* e, void* ptr, int64_t numel, int dtype, int root, 
  * FSDP._start_gather (tandem/zero.py:238-245). */
 int tdm_unit_gather(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes, int nsizes,
                     tdm_stream caller, tdm_work** out);
-/* Shared arena + direct gather (no counterpart in the reference, which stages every
- * gather through its slots): tdm_engine_share allocates `bytes` (< 2 GiB) of device
- * memory on this rank and publishes its hipIpcMemHandle_t; peers map it on first use.
+/* Shared arenas + direct gather (no counterpart in the reference, which stages every
+ * gather through its slots): tdm_engine_share allocates `bytes` (< 2 GiB: one exported
+ * allocation) of device memory on this rank and publishes its hipIpcMemHandle_t; peers
+ * map it on first use. A rank may share up to 64 arenas. A place in a rank's arenas is
+ * named by one number, its arena offset: the arena's index (0 for the first one shared)
+ * times 2^31, plus the byte offset within that arena; tdm_engine_arena_offset gives it
+ * for `bytes` bytes at `ptr` (-1 when they do not lie within one arena of this rank).
  * tdm_unit_gather_direct then fills `full` with W-1 copy kernels that read chunk q
- * straight from rank q's arena at byte offset peer_offsets[q] (own chunk: from `shard`),
+ * straight from rank q's arenas at arena offset peer_offsets[q] (own chunk: from `shard`),
  * on the engine's stream, without any message. The caller must bracket every change of
  * arena contents with tdm_fence, a barrier that is also ordered against the GPU: it
  * starts once `caller` has finished what it held, and a rank's arrival is announced
  * only when its engine stream has finished as well. */
 int tdm_engine_share(tdm_engine* e, int64_t bytes, void** ptr);
+int tdm_engine_arena_offset(tdm_engine* e, const void* ptr, int64_t bytes, int64_t* offset);
 int tdm_unit_gather_direct(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes,
                            int nsizes, const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out);
 int tdm_fence(tdm_engine* e, tdm_stream caller, tdm_work** out);
 
 /* The three collectives for tensors that lie in the ranks' shared arenas (this rank's
- * at `ptr`, rank q's at byte offset peer_offsets[q] of its arena), with the results of
+ * at `ptr`, rank q's at arena offset peer_offsets[q] of its arenas), with the results of
  * tdm_all_reduce / tdm_reduce_scatter / tdm_all_gather (tandem/comm.py:326-385) bit
  * for bit, by reading the peers' tensors where they lie instead of passing pieces
  * through slots:

@@ -132,6 +132,7 @@ _ENGINE_SIGNATURES = {
     "tdm_direct_zero2_step": (ctypes.c_int, [_VP, _VP, _PI64, _VP, _PI64, ctypes.c_int, _VP, _VP, ctypes.c_int64, ctypes.c_int64,
                                              ctypes.c_int, ctypes.POINTER(AdamwScalars), ctypes.c_int, _VP, _PVP]),
     "tdm_engine_share": (ctypes.c_int, [_VP, ctypes.c_int64, _PVP]),
+    "tdm_engine_arena_offset": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.POINTER(ctypes.c_int64)]),
     "tdm_unit_gather_direct": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _VP, _PI64, ctypes.c_int, _PI64,
                                               ctypes.c_int, _VP, _PVP]),
     "tdm_work_wait": (ctypes.c_int, [_VP, _VP]),

@@ -95,6 +95,7 @@ class Group:
         self._closed = False
         self._engine = None
         self._arena = None
+        self.arena_count = 0  # arenas shared so far
         if self.backend != "hip":
             raise CommError(f"unknown backend {self.backend} (tandem_amd provides \"hip\")")
         if self.transport != "device":
@@ -207,9 +208,9 @@ class Group:
 
     # ---- collectives
     def _direct_offsets(self, flat, direct, what):
-        """Arena byte offsets of every rank's tensor for a direct collective:
-        `direct=True` says every rank holds it at the same offset of its arena (ranks
-        that allocate the same things in the same order do), a list gives them."""
+        """Arena offsets of every rank's tensor for a direct collective: `direct=True`
+        says every rank holds it at the same place of its arenas (ranks that allocate
+        the same things in the same order do), a list gives them (arena_offset())."""
         if flat.numel() == 0:  # nothing to read, but the ranks still meet
             return (ctypes.c_int64 * self.size)()
         mine = self.arena_offset(flat)
@@ -315,13 +316,14 @@ class Group:
             ctypes.byref(scalars), order, self._stream(), out),
             params, (2 * self.size + 5) * 4 * n, async_op, keep=(p, g, exp_avg, exp_avg_sq, scalars))
 
-    # ---- shared arena: long-lived data that peers read directly
+    # ---- shared arenas: long-lived data that peers read (and the direct collectives write) in place
+    ARENA_LIMIT = (1 << 31) - 4096  # an arena is one exported allocation, and those stay under 2 GiB
+
     def share_arena(self, nbytes):
-        """Creates this rank's shared arena: `nbytes` (under 2 GiB) of device memory
-        owned by the engine (freed by close()) and exported once through HIP IPC, so
-        that the other ranks can read it directly. One arena per group."""
-        if self._arena is not None:
-            raise CommError("this group already has a shared arena")
+        """Shares an arena: `nbytes` (under 2 GiB) of device memory owned by the engine
+        (freed by close()) and exported once through HIP IPC, so that the other ranks can
+        read and write it directly. A group may share up to 64; shared_empty() carves from
+        the newest."""
         nbytes = max(16, int(nbytes))
         ptr = ctypes.c_void_p()
         try:
@@ -334,30 +336,38 @@ class Group:
 
         self._arena = torch.as_tensor(_Raw(), device=self.device)
         self._arena_used = 0
+        self.arena_count += 1
 
-    def shared_empty(self, numel, dtype=torch.float32):
-        """A tensor of `numel` elements in this rank's shared arena, for
-        gather_unit(..., peer_offsets=...) and the `direct` collectives. Without an
-        arena, one of exactly this size is created; otherwise the tensor is carved
-        from what share_arena() reserved (256-byte aligned, never given back). Every
-        change of an arena tensor that peers read on their own (gather_unit) must sit
-        between two fence() calls; the direct collectives fence by themselves."""
+    def shared_empty(self, numel, dtype=torch.float32, grow=None):
+        """A tensor of `numel` elements in this rank's newest shared arena, for
+        gather_unit(..., peer_offsets=...) and the `direct` collectives (256-byte aligned,
+        never given back). Without an arena, one of exactly this size is shared first. A
+        tensor that does not fit into what is left is refused, unless `grow` says how many
+        bytes a further arena should have (at least the tensor's): then one is shared and
+        the tensor starts it. Every change of an arena tensor that peers read on their own
+        (gather_unit) must sit between two fence() calls; the direct collectives fence by
+        themselves."""
         es = torch.empty(0, dtype=dtype).element_size()
+        need = numel * es
         if self._arena is None:
-            self.share_arena(numel * es)
+            self.share_arena(need if grow is None else max(need, min(int(grow), self.ARENA_LIMIT)))
         at = -(-self._arena_used // 256) * 256
-        if at + numel * es > self._arena.numel():
-            raise CommError(f"shared_empty: {numel * es} bytes do not fit in the arena "
-                            f"({self._arena.numel() - at} of {self._arena.numel()} left)")
-        self._arena_used = at + numel * es
-        return self._arena[at:at + numel * es].view(dtype)
+        if at + need > self._arena.numel():
+            if grow is None:
+                raise CommError(f"shared_empty: {need} bytes do not fit in the arena "
+                                f"({self._arena.numel() - at} of {self._arena.numel()} left)")
+            self.share_arena(max(need, min(int(grow), self.ARENA_LIMIT)))
+            at = 0
+        self._arena_used = at + need
+        return self._arena[at:at + need].view(dtype)
 
     def arena_offset(self, t):
-        """Byte offset of tensor `t` inside this rank's arena (None if it is not there)."""
-        if self._arena is None:
-            return None
-        off = t.data_ptr() - self._arena.data_ptr()
-        return off if 0 <= off and off + t.numel() * t.element_size() <= self._arena.numel() else None
+        """Where tensor `t` lies in this rank's arenas, as the one number the peers name the place by (the
+        arena's index times 2^31 plus the byte offset within it); None if it does not lie within one of them."""
+        off = ctypes.c_int64(-1)
+        check(lib().tdm_engine_arena_offset(self._engine, ctypes.c_void_p(t.data_ptr() if t.numel() else 0),
+                                            t.numel() * t.element_size(), ctypes.byref(off)))
+        return off.value if off.value >= 0 else None
 
     def fence(self):
         """A barrier ordered against the GPU: returns (on the caller's stream) once

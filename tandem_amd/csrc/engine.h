@@ -134,6 +134,7 @@ class Engine {
   std::shared_ptr<Work> barrier();
   std::shared_ptr<Work> fence(hipStream_t caller);
   void* share(size_t bytes);
+  int64_t own_arena_offset(const char* ptr, size_t bytes);
   std::shared_ptr<Work> unit_gather_direct(Buf full, const char* shard, std::vector<int64_t> sizes,
                                            std::vector<int64_t> peer_offsets, hipStream_t caller);
   // kind 0: all_reduce, 1: reduce_scatter (the owner's chunk only), 2: all_gather
@@ -185,7 +186,7 @@ class Engine {
   uint64_t await(int src);
   void release(int src);
   void barrier_now(bool after_gpu = false, uint64_t tag = 0);
-  const char* peer_arena(int peer, size_t need_bytes);
+  const char* peer_arena(int peer, int64_t offset, size_t bytes);
 
   std::string region_name(int rank) const { return "/tandem-" + job_ + "-" + std::to_string(rank) + "-hip"; }
 
@@ -202,10 +203,10 @@ class Engine {
   Region mine_;
   std::vector<std::unique_ptr<Region>> theirs_;
   std::vector<void*> out_mem_, peer_mem_;
-  void* arena_ = nullptr;
-  size_t arena_bytes_ = 0;
-  std::vector<void*> peer_arena_;
-  std::vector<size_t> peer_arena_bytes_;
+  std::vector<void*> arenas_;                      // in the order they were shared
+  std::vector<size_t> arena_sizes_;
+  std::vector<std::vector<void*>> peer_arena_;     // [peer][arena]: mapped at first use
+  std::vector<std::vector<size_t>> peer_arena_bytes_;
   std::vector<std::vector<hipEvent_t>> full_, free_, peer_full_, peer_free_;
   std::vector<uint64_t> sent_, got_;     // pieces, per peer: pick the slot
   std::vector<uint64_t> posted_;         // messages queued or published to each peer (flow control)

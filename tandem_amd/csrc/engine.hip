@@ -42,8 +42,8 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
     : job_(job), rank_(rank), size_(size), slots_(slots), slot_bytes_(slot_bytes), timeout_s_(timeout_s),
       device_(device), theirs_(size), out_mem_(size, nullptr), peer_mem_(size, nullptr), full_(size), free_(size),
       peer_full_(size), peer_free_(size), sent_(size, 0), got_(size, 0), posted_(size, 0), taken_(size, 0) {
-  peer_arena_.assign(size, nullptr);
-  peer_arena_bytes_.assign(size, 0);
+  peer_arena_.assign(size, std::vector<void*>(kMaxArenas, nullptr));
+  peer_arena_bytes_.assign(size, std::vector<size_t>(kMaxArenas, 0));
   if (size < 1 || rank < 0 || rank >= size) throw Invalid("rank must be in [0, size)");
   if (slots < 1 || slots > kMaxSlots) throw Invalid("slots must be in [1, " + std::to_string(kMaxSlots) + "]");
   if (slot_bytes < 16 || slot_bytes % 16) throw Invalid("slot_bytes must be a positive multiple of 16");
@@ -215,8 +215,10 @@ void Engine::release_device() {
     for (hipEvent_t e : full_[p]) (void)hipEventDestroy(e);
     for (hipEvent_t e : free_[p]) (void)hipEventDestroy(e);
     if (out_mem_[p]) (void)hipFree(out_mem_[p]);
-    if (peer_arena_[p]) (void)hipIpcCloseMemHandle(peer_arena_[p]);
-    peer_arena_[p] = nullptr;
+    for (void*& a : peer_arena_[p]) {
+      if (a) (void)hipIpcCloseMemHandle(a);
+      a = nullptr;
+    }
     if (peer_staging_[p]) (void)hipIpcCloseMemHandle(peer_staging_[p]);
     peer_staging_[p] = nullptr;
     peer_mem_[p] = out_mem_[p] = nullptr;
@@ -227,8 +229,9 @@ void Engine::release_device() {
     if (*st) (void)hipStreamDestroy(*st);
     *st = nullptr;
   }
-  if (arena_) (void)hipFree(arena_);
-  arena_ = nullptr;
+  for (void* a : arenas_) (void)hipFree(a);
+  arenas_.clear();
+  arena_sizes_.clear();
   if (staging_) (void)hipFree(staging_);
   staging_ = nullptr;
   mine_.reset();
@@ -1010,33 +1013,49 @@ std::shared_ptr<Work> Engine::sendrecv(Buf send, int dst, Buf recv, int src, hip
 // complete) -- ZeRO-3 changes its shards once per step, and gathers them 27 times.
 void* Engine::share(size_t bytes) {
   std::lock_guard<std::mutex> lock(arena_mu_);
-  if (arena_) throw std::runtime_error("share: this engine already has an arena");
-  if (bytes == 0 || bytes >= (size_t(2) << 30)) throw Invalid("share: the arena must be between 1 byte and 2 GiB (one IPC allocation)");
+  if (arenas_.size() == static_cast<size_t>(kMaxArenas)) throw std::runtime_error("share: this engine already has " + std::to_string(kMaxArenas) + " arenas");
+  if (bytes == 0 || bytes >= kArenaLimit) throw Invalid("share: an arena must be between 1 byte and 2 GiB (one IPC allocation)");
   check_hip(hipSetDevice(device_), "hipSetDevice");
-  check_hip(hipMalloc(&arena_, bytes), "hipMalloc (arena)");
+  void* arena = nullptr;
+  check_hip(hipMalloc(&arena, bytes), "hipMalloc (arena)");
   RegionHeader* h = mine_.header();
-  hipError_t err = hipIpcGetMemHandle(&h->arena_mem, arena_);
+  const size_t k = arenas_.size();
+  hipError_t err = hipIpcGetMemHandle(&h->arena_mem[k], arena);
   if (err != hipSuccess) {
-    (void)hipFree(arena_);
-    arena_ = nullptr;
+    (void)hipFree(arena);
     check_hip(err, "hipIpcGetMemHandle (arena)");
   }
-  arena_bytes_ = bytes;
-  h->arena_bytes.store(bytes, std::memory_order_release);  // the handle is visible before the size
-  return arena_;
+  arenas_.push_back(arena);
+  arena_sizes_.push_back(bytes);
+  h->arena_bytes[k].store(bytes, std::memory_order_release);  // the handle is visible before the size
+  return arena;
 }
 
-const char* Engine::peer_arena(int peer, size_t need_bytes) {
+// Where `bytes` bytes at `ptr` lie in this rank's arenas, as the one number its peers name them by; -1: not in any.
+int64_t Engine::own_arena_offset(const char* ptr, size_t bytes) {
   std::lock_guard<std::mutex> lock(arena_mu_);
-  if (!peer_arena_[peer]) {
-    RegionHeader* h = theirs_[peer]->header();
-    const uint64_t bytes = h->arena_bytes.load(std::memory_order_acquire);
-    if (bytes == 0) throw std::runtime_error("direct gather: rank " + std::to_string(peer) + " has not shared an arena");
-    check_hip(hipIpcOpenMemHandle(&peer_arena_[peer], h->arena_mem, hipIpcMemLazyEnablePeerAccess), "hipIpcOpenMemHandle (arena)");
-    peer_arena_bytes_[peer] = bytes;
+  for (size_t k = 0; k < arenas_.size(); ++k) {
+    const char* a = static_cast<const char*>(arenas_[k]);
+    if (ptr >= a && ptr + bytes <= a + arena_sizes_[k]) return static_cast<int64_t>((static_cast<uint64_t>(k) << kArenaShift) | static_cast<uint64_t>(ptr - a));
   }
-  if (need_bytes > peer_arena_bytes_[peer]) throw Invalid("direct gather: the range lies outside rank " + std::to_string(peer) + "'s arena");
-  return static_cast<const char*>(peer_arena_[peer]);
+  return -1;
+}
+
+// `bytes` bytes at `offset` of the peer's arenas (index and offset in one number), mapped at first use.
+const char* Engine::peer_arena(int peer, int64_t offset, size_t bytes) {
+  if (offset < 0) throw Invalid("direct: negative arena offset");
+  const uint64_t k = static_cast<uint64_t>(offset) >> kArenaShift, at = static_cast<uint64_t>(offset) & (kArenaLimit - 1);
+  if (k >= static_cast<uint64_t>(kMaxArenas)) throw Invalid("direct: no such arena");
+  std::lock_guard<std::mutex> lock(arena_mu_);
+  if (!peer_arena_[peer][k]) {
+    RegionHeader* h = theirs_[peer]->header();
+    const uint64_t size = h->arena_bytes[k].load(std::memory_order_acquire);
+    if (size == 0) throw std::runtime_error("direct: rank " + std::to_string(peer) + " has not shared arena " + std::to_string(k));
+    check_hip(hipIpcOpenMemHandle(&peer_arena_[peer][k], h->arena_mem[k], hipIpcMemLazyEnablePeerAccess), "hipIpcOpenMemHandle (arena)");
+    peer_arena_bytes_[peer][k] = size;
+  }
+  if (at + bytes > peer_arena_bytes_[peer][k]) throw Invalid("direct: the range lies outside rank " + std::to_string(peer) + "'s arena");
+  return static_cast<const char*>(peer_arena_[peer][k]) + at;
 }
 
 // Launched by the caller's thread: a direct gather exchanges no message with any
@@ -1069,7 +1088,7 @@ std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, st
       from = shard;
     } else {
       if (peer_offsets[q] < 0 || peer_offsets[q] % es) throw Invalid("unit_gather: bad arena offset");
-      from = peer_arena(q, static_cast<size_t>(peer_offsets[q]) + static_cast<size_t>(cs[q].numel) * es) + peer_offsets[q];
+      from = peer_arena(q, peer_offsets[q], static_cast<size_t>(cs[q].numel) * es);
     }
     if (np == TDM_MAX_PAIRS * 2) throw Invalid("unit_gather: too many ranks");
     pairs[np++] = tdm_pair{cs[q].ptr, from, cs[q].numel};
@@ -1123,23 +1142,14 @@ std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, st
 void Engine::direct_bases(const Buf& t, const std::vector<int64_t>& peer_offsets, const char** base) {
   const int es = elem_bytes(t.dtype);
   const size_t bytes = static_cast<size_t>(t.numel) * es;
-  const char* a;
-  size_t arena_bytes;
-  {
-    std::lock_guard<std::mutex> lock(arena_mu_);
-    a = static_cast<const char*>(arena_);
-    arena_bytes = arena_bytes_;
-  }
-  if (!a || t.ptr < a || t.ptr + bytes > a + arena_bytes) {
-    throw Invalid("direct collective: the tensor does not lie in this rank's shared arena");
-  }
+  if (own_arena_offset(t.ptr, bytes) < 0) throw Invalid("direct collective: the tensor does not lie in one of this rank's shared arenas");
   for (int q = 0; q < size_; ++q) {
     if (q == rank_) {
       base[q] = t.ptr;
       continue;
     }
     if (peer_offsets[q] < 0 || peer_offsets[q] % es) throw Invalid("direct collective: bad arena offset");
-    base[q] = peer_arena(q, static_cast<size_t>(peer_offsets[q]) + bytes) + peer_offsets[q];
+    base[q] = peer_arena(q, peer_offsets[q], bytes);
   }
 }
 

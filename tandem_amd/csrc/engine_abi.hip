@@ -131,6 +131,13 @@ int tdm_engine_share(tdm_engine* e, int64_t bytes, void** ptr) {
   });
 }
 
+int tdm_engine_arena_offset(tdm_engine* e, const void* ptr, int64_t bytes, int64_t* offset) {
+  return guard([&] {
+    if (offset == nullptr || bytes < 0 || (ptr == nullptr && bytes > 0)) throw Invalid("arena_offset: bad arguments");
+    *offset = engine_of(e).own_arena_offset(static_cast<const char*>(ptr), static_cast<size_t>(bytes));
+  });
+}
+
 int tdm_unit_gather_direct(tdm_engine* e, void* full, int64_t numel, int dtype, const void* shard, const int64_t* sizes,
                            int nsizes, const int64_t* peer_offsets, int noffsets, tdm_stream caller, tdm_work** out) {
   return guard([&] {

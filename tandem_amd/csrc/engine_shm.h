@@ -53,9 +53,14 @@ inline int elem_bytes(int dtype) {
 }
 
 // ---------------------------------------------------------------- shared region
-constexpr uint64_t kRegionMagic = 0x74646d4849503031ull;  // "tdmHIP01"
+constexpr uint64_t kRegionMagic = 0x74646d4849503032ull;  // "tdmHIP02"
 constexpr size_t kLine = 64;
 constexpr int kMaxSlots = 16;
+// An arena is one exported allocation and stays under 2 GiB, a rank may share several. A byte of a rank's arenas is
+// named by one number: the arena's index (in the order the rank shared them) in the bits from 31 up, the offset within it below.
+constexpr int kMaxArenas = 64;
+constexpr int kArenaShift = 31;
+constexpr uint64_t kArenaLimit = uint64_t(1) << kArenaShift;
 
 static_assert(std::atomic<uint64_t>::is_always_lock_free, "atomics shared between processes must be lock-free");
 
@@ -81,9 +86,9 @@ struct alignas(kLine) RegionHeader {
   int64_t pid;
   int32_t use_events;
   int32_t reserved;
-  // A rank's shared arena (tdm_engine_share): device memory its peers may read directly.
-  std::atomic<uint64_t> arena_bytes;  // 0 until published
-  hipIpcMemHandle_t arena_mem;
+  // A rank's shared arenas (tdm_engine_share): device memory its peers may read and write directly.
+  std::atomic<uint64_t> arena_bytes[kMaxArenas];  // 0 until published
+  hipIpcMemHandle_t arena_mem[kMaxArenas];
   // The engine's own staging memory for the staged collectives (two halves, used in turn).
   std::atomic<uint64_t> staging_bytes;  // 0 until published
   hipIpcMemHandle_t staging_mem;

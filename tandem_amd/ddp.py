@@ -49,8 +49,8 @@ class DDP(torch.nn.Module):
         without the host waiting for them (`Work.wait(stream_ordered=True)`), so the optimizer's launches are
         queued while the last buckets are still in flight; a bucket that fails then raises from the next collective
         instead of from this backward. False: the host waits, as the reference's DDP does (tandem/ddp.py:111-115).
-        direct: the buckets live in the group's shared arena (one is created if the
-        group has none: the gradients' size plus padding, under 2 GiB) and every
+        direct: the buckets live in the group's shared arenas (the gradients' size plus
+        padding, in arenas of 1 GiB where that is more) and every
         all-reduce runs arena to arena (`group.all_reduce(..., direct=True)`): same
         bits, 2 instead of 4.5 passes over a bucket per rank at two ranks, two
         handshakes per bucket instead of two per 4 MiB piece."""
@@ -83,33 +83,39 @@ class DDP(torch.nn.Module):
 
         groups = pack([p.numel() * p.element_size() for p in order], self.bucket_bytes, [p.dtype for p in order])
         self.buckets, self.bucket_of = [], {}
-        carved = {}
+        carved = {}  # per dtype: [slab, elements used of it]
         for members in groups:
             ps = [order[i] for i in members]
             flat = None
             if self.direct:
-                # Carved from one arena tensor per dtype, the same way on every rank (so
-                # a bucket has the same arena offset everywhere), 256-byte aligned.
+                # Carved from arena tensors ("slabs") per dtype, the same way on every rank (so a
+                # bucket has the same arena offset everywhere), 256-byte aligned. A rebuild carves
+                # the same slabs again.
                 dtype, numel = ps[0].dtype, sum(p.numel() for p in ps)
-                pool = self._pool(dtype)
-                at = carved.get(dtype, 0)
-                flat = pool[at:at + numel].zero_()
-                carved[dtype] = at + -(-numel // 64) * 64
+                k, at = carved.get(dtype, (0, 0))
+                if at + numel > self._slab(dtype, k, numel).numel():
+                    k, at = k + 1, 0
+                flat = self._slab(dtype, k, numel)[at:at + numel].zero_()
+                carved[dtype] = (k, at + -(-numel // 64) * 64)
             b = Bucket(ps, ps[0].device, ps[0].dtype, flat)
             self.buckets.append(b)
             for p in ps:
                 self.bucket_of[p] = b
         self._cursor = 0  # next bucket to launch: every rank launches in the same order
 
-    def _pool(self, dtype):
-        if dtype not in self._pools:
+    SLAB_BYTES = 1 << 30  # an arena is one exported allocation and stays under 2 GiB: larger models take several
+
+    def _slab(self, dtype, k, numel):
+        """Slab `k` of this dtype's buckets: room for every gradient of the dtype plus padding when that stays
+        under SLAB_BYTES, else slabs of that size (at least `numel` elements), each an arena of its own."""
+        slabs = self._pools.setdefault(dtype, [])
+        while len(slabs) <= k:
+            es = torch.empty(0, dtype=dtype).element_size()
             mine = [p for p in self.params if p.dtype == dtype]
-            # room for every gradient plus the padding of at most one bucket per parameter
-            numel = sum(p.numel() for p in mine) + 64 * len(mine)
-            if getattr(self.g, "_arena", None) is None:
-                self.g.share_arena(sum((p.numel() + 64) * p.element_size() for p in self.params) + 4096)
-            self._pools[dtype] = self.g.shared_empty(numel, dtype)
-        return self._pools[dtype]
+            whole = sum(p.numel() for p in mine) + 64 * len(mine)  # the padding of at most one bucket per parameter
+            room = max(min(whole, self.SLAB_BYTES // es), numel)
+            slabs.append(self.g.shared_empty(room, dtype, grow=room * es))
+        return slabs[k]
 
     def _gather(self, bucket):
         """Moves the bucket's loose gradients into it with one gather, and points

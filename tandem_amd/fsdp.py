@@ -51,31 +51,44 @@ class Residency:
 
 
 class ShardHome:
-    """Lays every unit's shard out in the ranks' shared arenas: unit k's shard starts
-    at the same element offset in every rank's arena only when all earlier shards had
-    equal sizes, so the offsets are kept per rank. Shards start on 16-byte boundaries."""
+    """Lays every unit's shard out in the ranks' shared arenas. Units are put into slabs: a slab is
+    one arena tensor of the same size on every rank (so it has the same arena offset everywhere),
+    large enough for the rank whose shards of the slab's units are longest; within a slab a unit's
+    shard starts at the same element offset on every rank only when all earlier shards had equal
+    sizes, so the offsets are kept per rank. Shards start on 16-byte boundaries. An arena is one
+    exported allocation and stays under 2 GiB, so a slab ends before SLAB_BYTES."""
 
     ALIGN = 4  # elements (fp32)
+    SLAB_BYTES = 1 << 30
 
     def __init__(self, group, unit_sizes, dtype):
         """unit_sizes[k][q]: elements of unit k's shard on rank q."""
         self.rank = group.rank
         world = group.size
         self.es = torch.empty(0, dtype=dtype).element_size()
-        self.at = []  # per unit: element offset of the shard in every rank's arena
-        ends = [0] * world
+        cap = max(self.SLAB_BYTES // self.es, 1)
+        self.slab_of, self.at = [], []  # per unit: its slab, and the element offset of the shard within it on every rank
+        extents, ends = [], [0] * world
         for sizes in unit_sizes:
+            padded = [-(-s // self.ALIGN) * self.ALIGN for s in sizes]
+            if max(ends) > 0 and max(e + p for e, p in zip(ends, padded)) > cap:
+                extents.append(max(ends))
+                ends = [0] * world
+            self.slab_of.append(len(extents))
             self.at.append(list(ends))
-            ends = [e + -(-s // self.ALIGN) * self.ALIGN for e, s in zip(ends, sizes)]
-        self.arena = group.shared_empty(max(max(ends), 1), dtype)
+            ends = [e + p for e, p in zip(ends, padded)]
+        extents.append(max(max(ends), 1))
+        self.slabs = [group.shared_empty(n, dtype, grow=n * self.es) for n in extents]
+        # the same on every rank: the slabs are the same allocations in the same order everywhere
+        self.base = [group.arena_offset(slab) for slab in self.slabs]
 
     def shard(self, k, numel):
         lo = self.at[k][self.rank]
-        return self.arena[lo:lo + numel]
+        return self.slabs[self.slab_of[k]][lo:lo + numel]
 
     def peer_offsets(self, k):
-        """Byte offsets of unit k's shard inside every rank's arena."""
-        return [a * self.es for a in self.at[k]]
+        """Arena offsets of unit k's shard on every rank."""
+        return [self.base[self.slab_of[k]] + a * self.es for a in self.at[k]]
 
 
 class Unit:

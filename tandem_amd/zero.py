@@ -50,8 +50,9 @@ class ZeRO(torch.nn.Module):
     def __init__(self, module, group, stage=1, optimizer=None, bucket_bytes=25 << 20, direct=False, fused_step=False):
         """direct: the flat parameter buffer and the gradient buffer (stage 2: one
         staging buffer the size of the model, kept, instead of one per bucket that is
-        dropped) live in the group's shared arena (created here if the group has none:
-        twice the model, under 2 GiB), and every collective runs arena to arena
+        dropped) live in the group's shared arenas (one of twice the model's size if the
+        group has none; an arena each once that would reach 2 GiB, the size one arena
+        stops at, so the model itself must stay under it), and every collective runs arena to arena
         (`direct=True` of tandem_amd.Group): same bits, fewer passes over memory, no
         slots.
 
@@ -89,10 +90,11 @@ class ZeRO(torch.nn.Module):
         self.flat = FlatLayout([p.numel() for p in params], group.size, group.rank)
         self.offset = dict(zip(params, self.flat.offsets))
         if self.direct:
-            if getattr(group, "_arena", None) is None:
-                group.share_arena(2 * (self.flat.numel * params[0].element_size() + 4096))
-            self.buf = group.shared_empty(self.flat.numel, dtype)
-            self._pool = group.shared_empty(self.flat.numel, dtype).zero_()  # stage 1: gradients; stage 2: staging
+            nbytes = self.flat.numel * params[0].element_size()
+            if getattr(group, "_arena", None) is None and 2 * (nbytes + 4096) < group.ARENA_LIMIT:
+                group.share_arena(2 * (nbytes + 4096))  # both in one arena while that stays one allocation
+            self.buf = group.shared_empty(self.flat.numel, dtype, grow=nbytes)
+            self._pool = group.shared_empty(self.flat.numel, dtype, grow=nbytes).zero_()  # stage 1: gradients; stage 2: staging
         else:
             self.buf = torch.empty(self.flat.numel, device=dev, dtype=dtype)
         with torch.no_grad():

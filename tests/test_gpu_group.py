@@ -825,3 +825,71 @@ def test_more_collectives_in_flight_than_done_words():
 
     for ok, _ in launch(more_works_than_words, 2, gpus=[0, 0], timeout=TIMEOUT):
         assert ok
+
+
+def several_arenas(g):
+    """Every rank shares three arenas; rank q's tensors lie in arena (q + k) % 3, so every collective reaches into
+    different arenas of different peers. Offsets are named as arena index * 2^31 + byte offset."""
+    dev, w, r = g.device, g.size, g.rank
+    arenas = []
+    for _ in range(3):
+        g.share_arena(1 << 20)
+        arenas.append(g._arena)
+    assert g.arena_count == 3
+
+    def place(q, k, n):  # (arena, byte offset) of rank q's k-th tensor of n floats: the same rule on every rank
+        return (q + k) % 3, 256 * (1 + q + 3 * k) + 4096 * k
+
+    out = {}
+    n = 10_007
+    sizes = [n // w + (1 if q < n % w else 0) for q in range(w)]
+    lo = sum(sizes[:r])
+    for k, what in enumerate(("all_reduce", "reduce_scatter", "all_gather", "gather_unit")):
+        a, off = place(r, k, n)
+        t = arenas[a][off:off + 4 * n].view(torch.float32)
+        offs = [(place(q, k, n)[0] << 31) + place(q, k, n)[1] for q in range(w)]
+        assert g.arena_offset(t) == offs[r]
+        x = values(r + 7 * k, n, torch.float32).to(dev)
+        if what == "all_reduce":
+            t.copy_(x)
+            g.all_reduce(t, op="avg", direct=offs)
+        elif what == "reduce_scatter":
+            t.copy_(x)
+            g.reduce_scatter(t, sizes, direct=offs)
+        elif what == "all_gather":
+            t.zero_()
+            t[lo:lo + sizes[r]] = x[lo:lo + sizes[r]]
+            g.all_gather(t, sizes, direct=offs)
+        else:  # the shard in the arena, the full buffer anywhere
+            shard = t[:sizes[r]]
+            shard.copy_(x[lo:lo + sizes[r]])
+            full = torch.zeros(n, device=dev)
+            g.fence()
+            g.gather_unit(full, shard, sizes, peer_offsets=offs)
+            g.fence()
+            t = full
+        out[what] = t.cpu().clone()
+    assert g.arena_offset(torch.zeros(4, device=dev)) is None
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("world", [2, 3])
+def test_tensors_in_several_arenas(world):
+    from oracle import ring
+    from tandem_amd import launch
+
+    n = 10_007
+    sizes = [n // world + (1 if q < n % world else 0) for q in range(world)]
+    res = launch(several_arenas, world, gpus=[0] * world, timeout=TIMEOUT)
+    for r, out in enumerate(res):
+        lo = sum(sizes[:r])
+        xs = [to_np(values(q, n, torch.float32)) for q in range(world)]
+        assert np.array_equal(bits(to_np(out["all_reduce"])), bits(ring.expected_all_reduce(xs, True, "f32")))
+        xs = [to_np(values(q + 7, n, torch.float32)) for q in range(world)]
+        want = xs[r].copy()
+        want[lo:lo + sizes[r]] = ring.expected_reduce_scatter(xs, sizes, False, "f32")[r][lo:lo + sizes[r]]
+        assert np.array_equal(bits(to_np(out["reduce_scatter"])), bits(want))
+        for k, what in ((2, "all_gather"), (3, "gather_unit")):
+            xs = [to_np(values(q + 7 * k, n, torch.float32)) for q in range(world)]
+            assert np.array_equal(bits(to_np(out[what])), bits(ring.expected_all_gather(xs, sizes))), what

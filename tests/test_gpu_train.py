@@ -89,6 +89,17 @@ def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1, zero_every
     return {"losses": losses, "weights": w.cpu(), **extra}
 
 
+def train_rank_small_slabs(g, strategy, bucket_bytes, steps, batch):
+    """The same run with slabs so small that the buckets (the shards) spread over several arenas."""
+    from tandem_amd.ddp import DDP
+    from tandem_amd.fsdp import ShardHome
+
+    DDP.SLAB_BYTES, ShardHome.SLAB_BYTES = 24 << 10, 8 << 10
+    out = train_rank(g, strategy, bucket_bytes, steps, batch)
+    out["arenas"] = g.arena_count
+    return out
+
+
 def one_process(world, accumulate=1, zero_every=1):
     """Both ranks' gradients computed in this process, averaged as (a/2) + (b/2),
     torch AdamW on the GPU."""
@@ -121,6 +132,19 @@ def one_process(world, accumulate=1, zero_every=1):
         kept = None if (step + 1) % zero_every == 0 else [p.grad.clone() for p in model.parameters()]
         opt.zero_grad()
     return losses, torch.cat([p.detach().reshape(-1) for p in model.parameters()]).cpu()
+
+
+def test_buckets_and_shards_spread_over_several_arenas():
+    """An arena is one exported allocation of under 2 GiB: larger models take several. Forced here with tiny slabs."""
+    from tandem_amd import launch
+
+    ref_losses, ref_w = one_process(2)
+    for s in ("ddpd", "zero3"):
+        res = launch(train_rank_small_slabs, 2, s, 4 << 10, STEPS, BATCH, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT)
+        for r in range(2):
+            assert res[r]["arenas"] >= 3, (s, res[r]["arenas"])
+            assert res[r]["losses"] == ref_losses[r], (s, r)
+            assert torch.equal(res[r]["weights"], ref_w), (s, r)
 
 
 def test_two_ranks_all_strategies_agree_bit_for_bit():
