@@ -242,10 +242,11 @@ class Engine {
   void completion_loop();
   void drain_completions();
   std::mutex cmu_;
-  std::condition_variable ccv_, cidle_;
+  std::condition_variable ccv_;
   std::deque<Completion> completions_;
-  bool cstop_ = false, cbusy_ = false;
+  bool cstop_ = false;
   std::atomic<uint64_t> cqueued_{0};  // completions ever queued
+  std::atomic<uint64_t> csettled_{0}; // completions published (or dropped after a failure): what a barrier waits for
   uint64_t cdone_ = 0;                // completions ever taken (completion thread, under cmu_)
   std::string cerror_;
   std::thread completer_;

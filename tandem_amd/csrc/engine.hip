@@ -442,21 +442,14 @@ void Engine::completion_loop() {
   (void)hipSetDevice(device_);
   for (;;) {
     Completion c;
+    spin_for([this] { return cqueued_.load(std::memory_order_acquire) != cdone_; });
     {
       std::unique_lock<std::mutex> lock(cmu_);
-      cbusy_ = false;
-      if (completions_.empty()) {
-        cidle_.notify_all();
-        lock.unlock();
-        spin_for([this] { return cqueued_.load(std::memory_order_acquire) != cdone_; });
-        lock.lock();
-      }
       ccv_.wait(lock, [this] { return cstop_ || !completions_.empty(); });
       if (completions_.empty()) return;
       c = completions_.front();
       completions_.pop_front();
       ++cdone_;
-      cbusy_ = true;
     }
     if (c.after) {
       hipError_t err;
@@ -472,22 +465,27 @@ void Engine::completion_loop() {
         if (cerror_.empty()) cerror_ = std::string("waiting for a piece's kernel: ") + hipGetErrorString(err);
       }
     }
+    bool failed;
     {
       // After a failure nothing more is published, this message or any later one:
       // the peers time out rather than read bad bytes or reuse a slot still in use.
       std::lock_guard<std::mutex> lock(cmu_);
-      if (!cerror_.empty()) continue;
+      failed = !cerror_.empty();
     }
-    if (c.is_release) release(c.peer); else signal(c.peer, c.length);
+    if (!failed) {
+      if (c.is_release) release(c.peer); else signal(c.peer, c.length);
+    }
+    csettled_.fetch_add(1, std::memory_order_release);
   }
 }
 
 void Engine::drain_completions() {
   if (use_events_) return;
-  std::unique_lock<std::mutex> lock(cmu_);
-  if (!cidle_.wait_for(lock, std::chrono::duration<double>(timeout_s_), [this] { return completions_.empty() && !cbusy_; })) {
-    throw Timeout("timed out waiting for the GPU to finish the queued pieces");
-  }
+  // Everything this thread has queued (it alone queues) has been published, or dropped after a failure.
+  const uint64_t queued = cqueued_.load(std::memory_order_acquire);
+  wait_until([&] { return csettled_.load(std::memory_order_acquire) >= queued; }, timeout_s_,
+             "timed out waiting for the GPU to finish the queued pieces");
+  std::lock_guard<std::mutex> lock(cmu_);
   if (!cerror_.empty()) throw std::runtime_error("completion thread failed: " + cerror_);
 }
 

@@ -1,0 +1,217 @@
+// The process-rank engine's host side on a machine without a GPU: W processes, each with an engine built from the very
+// sources of the library (engine.hip, engine_abi.hip, abi.hip) against a stand-in runtime (fake_hip.cpp) and stand-in
+// kernels (fake_kernels.cpp), run the collectives through the C ABI and check where every element ended up. What this
+// sees that the GPU tests do not: the engine's threads (caller, progress, completion) under the host's sanitizers
+// for data races, addresses and undefined behaviour. Numbers are integer-valued, so sums are exact in any order; the
+// order of the sums is the GPU tests' business.
+//
+// usage: engine_host_test <world> <staged|ring> [staging_bytes]
+
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/wait.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "../../include/tandem_hip.h"
+
+#define REQUIRE(cond)                                                                                     \
+  do {                                                                                                    \
+    if (!(cond)) {                                                                                        \
+      std::fprintf(stderr, "rank %d: %s:%d: %s failed (%s)\n", g_rank, __FILE__, __LINE__, #cond, tdm_last_error()); \
+      return 1;                                                                                           \
+    }                                                                                                     \
+  } while (0)
+
+static int g_rank = -1;
+
+static float value(int rank, int64_t i, int salt) { return static_cast<float>((rank + 1) * ((i + salt) % 13) - salt % 5); }
+
+static std::vector<int64_t> split(int64_t n, int w, bool uneven) {
+  std::vector<int64_t> s(w);
+  for (int q = 0; q < w; ++q) s[q] = n / w + (q < n % w ? 1 : 0);
+  if (uneven && w > 1) {  // one empty chunk, its elements given to the next rank
+    s[1 % w] += s[0];
+    s[0] = 0;
+  }
+  return s;
+}
+
+static int run_rank(int rank, int world, const std::string& job, std::atomic<int>* arrived) {
+  g_rank = rank;
+  tdm_engine* e = nullptr;
+  REQUIRE(tdm_engine_create(job.c_str(), rank, world, 2, 4096, 20.0, 0, &e) == TDM_OK);
+  arrived->fetch_add(1);  // the launcher's barrier: every rank has published its region
+  while (arrived->load() < world) std::this_thread::yield();
+  REQUIRE(tdm_engine_connect(e) == TDM_OK);
+
+  const int64_t lengths[] = {0, 1, 5, 1000, 4099, 40000};
+  int salt = 0;
+  for (int64_t n : lengths) {
+    for (int uneven = 0; uneven < 2; ++uneven) {
+      const std::vector<int64_t> sizes = split(n, world, uneven != 0);
+      int64_t lo = 0;
+      for (int q = 0; q < rank; ++q) lo += sizes[q];
+      ++salt;
+      auto total = [&](int64_t i, int s) {
+        float t = 0;
+        for (int q = 0; q < world; ++q) t += value(q, i, s);
+        return t;
+      };
+      // several collectives in flight at once, waited for in order; done() polled meanwhile
+      std::vector<float> a(n), b(n), c(n), d(n);
+      for (int64_t i = 0; i < n; ++i) {
+        a[i] = value(rank, i, salt);
+        b[i] = value(rank, i, salt + 100);
+        c[i] = i >= lo && i < lo + sizes[rank] ? value(rank, i, salt + 200) : -1.0f;
+        d[i] = rank == world - 1 ? value(rank, i, salt + 300) : -2.0f;
+      }
+      tdm_work *wa, *wb, *wb2, *wc, *wd;
+      std::vector<float> b2 = b;
+      REQUIRE(tdm_all_reduce(e, a.data(), n, TDM_F32, 0, nullptr, &wa) == TDM_OK);
+      REQUIRE(tdm_reduce_scatter(e, b.data(), n, TDM_F32, sizes.data(), world, 0, nullptr, &wb) == TDM_OK);
+      REQUIRE(tdm_reduce_scatter_owner(e, b2.data(), n, TDM_F32, uneven ? sizes.data() : nullptr, uneven ? world : 0, 0, nullptr, &wb2) == TDM_OK);
+      REQUIRE(tdm_all_gather(e, c.data(), n, TDM_F32, sizes.data(), world, nullptr, &wc) == TDM_OK);
+      REQUIRE(tdm_broadcast(e, d.data(), n, TDM_F32, world - 1, nullptr, &wd) == TDM_OK);
+      (void)tdm_work_done(wd);
+      REQUIRE(tdm_work_wait(wa, nullptr) == TDM_OK);
+      REQUIRE(tdm_work_wait_stream(wb, nullptr) == TDM_OK);
+      REQUIRE(tdm_work_wait(wb2, nullptr) == TDM_OK);
+      REQUIRE(tdm_work_wait_stream(wc, nullptr) == TDM_OK);
+      REQUIRE(tdm_work_wait(wd, nullptr) == TDM_OK);
+      REQUIRE(tdm_work_done(wa) == 1 && tdm_work_done(wd) == 1);
+      double t0 = 0, t1 = 0;
+      REQUIRE(tdm_work_times(wa, &t0, &t1) == TDM_OK && t1 >= t0);
+      for (tdm_work* w : {wa, wb, wb2, wc, wd}) REQUIRE(tdm_work_free(w) == TDM_OK);
+      const std::vector<int64_t> even = split(n, world, false);
+      const std::vector<int64_t>& owner_sizes = uneven ? sizes : even;
+      int64_t olo = 0;
+      for (int q = 0; q < rank; ++q) olo += owner_sizes[q];
+      for (int64_t i = 0; i < n; ++i) {
+        REQUIRE(a[i] == total(i, salt));
+        if (i >= lo && i < lo + sizes[rank]) REQUIRE(b[i] == total(i, salt + 100));
+        if (i >= olo && i < olo + owner_sizes[rank]) REQUIRE(b2[i] == total(i, salt + 100));
+        int owner = 0;
+        for (int64_t at = sizes[0]; i >= at; at += sizes[++owner]) {
+        }
+        REQUIRE(c[i] == value(owner, i, salt + 200));
+        REQUIRE(d[i] == value(world - 1, i, salt + 300));
+      }
+      // an average, a ring of sendrecvs, a barrier and a fence
+      std::vector<float> m(n), out(n, 0.0f), in(n, -3.0f);
+      for (int64_t i = 0; i < n; ++i) {
+        m[i] = static_cast<float>(world) * value(rank, i, salt + 400);
+        out[i] = value(rank, i, salt + 500);
+      }
+      tdm_work *wm, *ws, *wbar, *wf;
+      REQUIRE(tdm_all_reduce(e, m.data(), n, TDM_F32, 1, nullptr, &wm) == TDM_OK);
+      REQUIRE(tdm_sendrecv(e, out.data(), n, (rank + 1) % world, in.data(), n, (rank + world - 1) % world, TDM_F32, nullptr, &ws) == TDM_OK);
+      REQUIRE(tdm_barrier(e, &wbar) == TDM_OK);
+      REQUIRE(tdm_fence(e, nullptr, &wf) == TDM_OK);
+      for (tdm_work* w : {wm, ws, wbar, wf}) REQUIRE(tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
+      for (int64_t i = 0; i < n; ++i) {
+        REQUIRE(m[i] == total(i, salt + 400));
+        REQUIRE(in[i] == value((rank + world - 1) % world, i, salt + 500));
+      }
+    }
+  }
+
+  // arenas: two of them; the direct collectives and a direct unit gather reach into the peers' second one
+  void *first = nullptr, *second = nullptr;
+  REQUIRE(tdm_engine_share(e, 1 << 16, &first) == TDM_OK && tdm_engine_share(e, 1 << 20, &second) == TDM_OK);
+  const int64_t n = 30011;
+  const std::vector<int64_t> sizes = split(n, world, false);
+  int64_t lo = 0;
+  for (int q = 0; q < rank; ++q) lo += sizes[q];
+  float* t = reinterpret_cast<float*>(static_cast<char*>(second) + 256 * (rank + 1));
+  std::vector<int64_t> offs(world);
+  for (int q = 0; q < world; ++q) offs[q] = (int64_t(1) << 31) + 256 * (q + 1);
+  int64_t mine = -2;
+  REQUIRE(tdm_engine_arena_offset(e, t, n * 4, &mine) == TDM_OK && mine == offs[rank]);
+  REQUIRE(tdm_engine_arena_offset(e, &mine, 8, &mine) == TDM_OK && mine == -1);
+  for (int64_t i = 0; i < n; ++i) t[i] = value(rank, i, 900);
+  tdm_work* w = nullptr;
+  REQUIRE(tdm_direct_all_reduce(e, t, n, TDM_F32, 0, offs.data(), world, nullptr, &w) == TDM_OK);
+  REQUIRE(tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
+  for (int64_t i = 0; i < n; ++i) {
+    float want = 0;
+    for (int q = 0; q < world; ++q) want += value(q, i, 900);
+    REQUIRE(t[i] == want);
+  }
+  for (int64_t i = 0; i < n; ++i) t[i] = i >= lo && i < lo + sizes[rank] ? value(rank, i, 901) : -4.0f;
+  REQUIRE(tdm_direct_all_gather(e, t, n, TDM_F32, sizes.data(), world, offs.data(), world, nullptr, &w) == TDM_OK);
+  REQUIRE(tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
+  std::vector<float> full(n, -5.0f);
+  std::vector<int64_t> shard_offs(world);
+  int64_t at = 0;
+  for (int q = 0; q < world; ++q) {
+    shard_offs[q] = offs[q] + at * 4;  // rank q's own chunk, where the all-gather left it
+    at += sizes[q];
+  }
+  REQUIRE(tdm_unit_gather_direct(e, full.data(), n, TDM_F32, t + lo, sizes.data(), world, shard_offs.data(), world, nullptr, &w) == TDM_OK);
+  REQUIRE(tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
+  for (int64_t i = 0, owner = 0, end = sizes[0]; i < n; ++i) {
+    while (i >= end) end += sizes[++owner];
+    REQUIRE(t[i] == value(static_cast<int>(owner), i, 901) && full[i] == t[i]);
+  }
+  REQUIRE(tdm_fence(e, nullptr, &w) == TDM_OK && tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
+
+  // more collectives in flight than the engine has done words
+  const int many = 1100;
+  std::vector<float> rows(static_cast<size_t>(many) * 3);
+  std::vector<tdm_work*> works(many);
+  for (int k = 0; k < many; ++k) {
+    for (int j = 0; j < 3; ++j) rows[k * 3 + j] = static_cast<float>(k + rank);
+    REQUIRE(tdm_all_reduce(e, &rows[k * 3], 3, TDM_F32, 0, nullptr, &works[k]) == TDM_OK);
+  }
+  for (int k = 0; k < many; ++k) {
+    REQUIRE(tdm_work_wait(works[k], nullptr) == TDM_OK && tdm_work_free(works[k]) == TDM_OK);
+    REQUIRE(rows[k * 3 + 2] == static_cast<float>(world * k + world * (world - 1) / 2));
+  }
+
+  // refusals come back as codes with a message, from the calling thread
+  REQUIRE(tdm_all_reduce(e, rows.data(), 3, TDM_I32, 1, nullptr, &w) == TDM_EINVAL && std::strlen(tdm_last_error()) > 0);
+  REQUIRE(tdm_all_reduce(e, nullptr, 3, TDM_F32, 0, nullptr, &w) == TDM_EINVAL);
+  const int64_t bad[2] = {1, 1};
+  REQUIRE(tdm_all_gather(e, rows.data(), 3, TDM_F32, bad, 2, nullptr, &w) == TDM_EINVAL);
+  REQUIRE(tdm_engine_close(e) == TDM_OK);
+  REQUIRE(tdm_all_reduce(e, rows.data(), 3, TDM_F32, 0, nullptr, &w) != TDM_OK);
+  REQUIRE(tdm_engine_destroy(e) == TDM_OK);
+  return 0;
+}
+
+int main(int argc, char** argv) {
+  const int world = argc > 1 ? std::atoi(argv[1]) : 2;
+  const std::string algo = argc > 2 ? argv[2] : "staged";
+  if (world < 2 || world > 8) return 64;
+  ::setenv("TANDEM_HIP_ALGO", algo.c_str(), 1);
+  if (argc > 3) ::setenv("TANDEM_HIP_STAGING_BYTES", argv[3], 1);
+  const std::string job = "host" + std::to_string(::getpid());
+  void* shared = ::mmap(nullptr, 4096, PROT_READ | PROT_WRITE, MAP_SHARED | MAP_ANONYMOUS, -1, 0);
+  if (shared == MAP_FAILED) return 65;
+  auto* arrived = new (shared) std::atomic<int>(0);
+  std::vector<pid_t> children;
+  for (int r = 0; r < world; ++r) {  // forked before any thread exists
+    const pid_t pid = ::fork();
+    if (pid < 0) return 66;
+    if (pid == 0) {
+      std::exit(run_rank(r, world, job, arrived));  // through the exit handlers: the leak check runs there
+    }
+    children.push_back(pid);
+  }
+  int failed = 0;
+  for (pid_t pid : children) {
+    int status = 0;
+    if (::waitpid(pid, &status, 0) != pid || !WIFEXITED(status) || WEXITSTATUS(status) != 0) ++failed;
+  }
+  if (failed) std::fprintf(stderr, "%d of %d ranks failed\n", failed, world);
+  return failed ? 1 : 0;
+}

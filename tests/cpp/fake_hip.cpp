@@ -1,0 +1,189 @@
+// A stand-in for the HIP runtime, for ONE purpose: running the process-rank engine's HOST code (threads, queues, rings,
+// hand-overs, done words: tandem_amd/csrc/engine.hip, engine_abi.hip) on a machine without a GPU and under the host's
+// sanitizers, which cannot share a process with the real runtime. It is linked into tests/cpp/engine_host_test only;
+// the library the package loads is never built from it, and nothing here computes a result anybody ships.
+//
+// What it models: "device" memory is POSIX shared memory (so that an IPC memory handle can be opened by another
+// process), every stream executes at once on the calling thread (so an event is complete when recorded and a stream
+// is always idle), a stream's write of a value is a store, its wait for a value a bounded spin.
+
+#include <fcntl.h>
+#include <hip/hip_runtime_api.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <thread>
+
+namespace {
+
+struct Block {
+  std::string name;  // of the shared-memory object; empty for plain host memory
+  size_t bytes;
+};
+
+std::mutex g_mu;
+std::map<void*, Block> g_blocks;  // what this process allocated or opened
+std::atomic<uint64_t> g_serial{0};
+
+void* map_shared(const std::string& name, size_t bytes, bool create) {
+  const int fd = ::shm_open(name.c_str(), create ? (O_CREAT | O_EXCL | O_RDWR) : O_RDWR, 0600);
+  if (fd < 0) return nullptr;
+  if (create && ::ftruncate(fd, static_cast<off_t>(bytes)) != 0) {
+    ::close(fd);
+    ::shm_unlink(name.c_str());
+    return nullptr;
+  }
+  if (!create) {
+    struct stat st;
+    if (::fstat(fd, &st) != 0) {
+      ::close(fd);
+      return nullptr;
+    }
+    bytes = static_cast<size_t>(st.st_size);
+  }
+  void* p = ::mmap(nullptr, bytes, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+  ::close(fd);
+  if (p == MAP_FAILED) return nullptr;
+  std::lock_guard<std::mutex> lock(g_mu);
+  g_blocks[p] = Block{create ? name : std::string(), bytes};
+  return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+hipError_t hipSetDevice(int) { return hipSuccess; }
+hipError_t hipGetLastError(void) { return hipSuccess; }
+const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "no error" : "an error of the stand-in runtime"; }
+
+hipError_t hipDeviceGetAttribute(int* value, hipDeviceAttribute_t attr, int) {
+  *value = attr == hipDeviceAttributeCanUseStreamWaitValue ? 1 : 0;
+  return hipSuccess;
+}
+
+hipError_t hipGetDeviceProperties(hipDeviceProp_t* prop, int) {
+  std::memset(prop, 0, sizeof *prop);
+  std::snprintf(prop->name, sizeof prop->name, "stand-in");
+  prop->multiProcessorCount = 1;
+  return hipSuccess;
+}
+
+hipError_t hipMalloc(void** ptr, size_t bytes) {
+  const std::string name = "/tdmfake-" + std::to_string(::getpid()) + "-" + std::to_string(g_serial.fetch_add(1));
+  *ptr = map_shared(name, bytes ? bytes : 1, true);
+  return *ptr ? hipSuccess : hipErrorOutOfMemory;
+}
+
+hipError_t hipFree(void* ptr) {
+  if (!ptr) return hipSuccess;
+  Block b;
+  {
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_blocks.find(ptr);
+    if (it == g_blocks.end()) return hipErrorInvalidValue;
+    b = it->second;
+    g_blocks.erase(it);
+  }
+  ::munmap(ptr, b.bytes);
+  if (!b.name.empty()) ::shm_unlink(b.name.c_str());
+  return hipSuccess;
+}
+
+hipError_t hipHostMalloc(void** ptr, size_t bytes, unsigned int) {
+  *ptr = std::aligned_alloc(4096, (bytes + 4095) / 4096 * 4096);
+  return *ptr ? hipSuccess : hipErrorOutOfMemory;
+}
+
+hipError_t hipHostFree(void* ptr) {
+  std::free(ptr);
+  return hipSuccess;
+}
+
+hipError_t hipIpcGetMemHandle(hipIpcMemHandle_t* handle, void* ptr) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  auto it = g_blocks.find(ptr);
+  if (it == g_blocks.end() || it->second.name.empty() || it->second.name.size() >= sizeof handle->reserved) return hipErrorInvalidValue;
+  std::memset(handle, 0, sizeof *handle);
+  std::memcpy(handle->reserved, it->second.name.c_str(), it->second.name.size());
+  return hipSuccess;
+}
+
+hipError_t hipIpcOpenMemHandle(void** ptr, hipIpcMemHandle_t handle, unsigned int) {
+  char name[sizeof handle.reserved + 1] = {0};
+  std::memcpy(name, handle.reserved, sizeof handle.reserved);
+  *ptr = map_shared(name, 0, false);
+  return *ptr ? hipSuccess : hipErrorInvalidValue;
+}
+
+hipError_t hipIpcCloseMemHandle(void* ptr) { return hipFree(ptr); }  // opened blocks carry no name: nothing is unlinked
+
+hipError_t hipIpcGetEventHandle(hipIpcEventHandle_t*, hipEvent_t) { return hipErrorNotSupported; }
+hipError_t hipIpcOpenEventHandle(hipEvent_t*, hipIpcEventHandle_t) { return hipErrorNotSupported; }
+
+hipError_t hipStreamCreateWithFlags(hipStream_t* stream, unsigned int) {
+  *stream = reinterpret_cast<hipStream_t>(new char);
+  return hipSuccess;
+}
+hipError_t hipStreamDestroy(hipStream_t stream) {
+  delete reinterpret_cast<char*>(stream);
+  return hipSuccess;
+}
+hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+hipError_t hipStreamQuery(hipStream_t) { return hipSuccess; }
+hipError_t hipStreamWaitEvent(hipStream_t, hipEvent_t, unsigned int) { return hipSuccess; }
+
+hipError_t hipEventCreateWithFlags(hipEvent_t* event, unsigned) {
+  *event = reinterpret_cast<hipEvent_t>(new char);
+  return hipSuccess;
+}
+hipError_t hipEventCreate(hipEvent_t* event) { return hipEventCreateWithFlags(event, 0); }
+hipError_t hipEventDestroy(hipEvent_t event) {
+  delete reinterpret_cast<char*>(event);
+  return hipSuccess;
+}
+hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }
+hipError_t hipEventQuery(hipEvent_t) { return hipSuccess; }
+hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
+hipError_t hipEventElapsedTime(float* ms, hipEvent_t, hipEvent_t) {
+  *ms = 0;
+  return hipSuccess;
+}
+
+hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind, hipStream_t) {
+  std::memmove(dst, src, bytes);
+  return hipSuccess;
+}
+
+hipError_t hipStreamWriteValue32(hipStream_t, void* ptr, uint32_t value, unsigned int) {
+  reinterpret_cast<std::atomic<uint32_t>*>(ptr)->store(value, std::memory_order_release);
+  return hipSuccess;
+}
+
+// A real stream waits on the GPU and the call returns at once; here the calling thread waits (at most ten seconds).
+hipError_t hipStreamWaitValue32(hipStream_t, void* ptr, uint32_t value, unsigned int, uint32_t) {
+  const auto until = std::chrono::steady_clock::now() + std::chrono::seconds(10);
+  while (reinterpret_cast<std::atomic<uint32_t>*>(ptr)->load(std::memory_order_acquire) < value) {
+    if (std::chrono::steady_clock::now() > until) return hipErrorNotReady;
+    std::this_thread::yield();
+  }
+  return hipSuccess;
+}
+
+hipError_t hipPointerGetAttributes(hipPointerAttribute_t* attr, const void*) {
+  std::memset(attr, 0, sizeof *attr);
+  attr->type = hipMemoryTypeDevice;  // every pointer counts as memory of device 0
+  attr->device = 0;
+  return hipSuccess;
+}
+
+}  // extern "C"

@@ -1,0 +1,95 @@
+// The four launchers the engine calls (tandem_amd/csrc/common.h), as plain loops on the host: the other half of the
+// stand-in that tests/cpp/fake_hip.cpp describes, linked into tests/cpp/engine_host_test only. fp32, fp64, int32 and
+// int64; the sums are formed in the order the kernels form them, which for the integer-valued numbers the test
+// sends does not matter.
+
+#include <cstring>
+#include <string>
+
+#include "../../tandem_amd/csrc/common.h"
+
+namespace tandem_hip {
+
+namespace {
+
+int size_of(int dtype) {
+  switch (dtype) {
+    case TDM_F32: case TDM_I32: return 4;
+    case TDM_F64: case TDM_I64: return 8;
+    case TDM_F16: case TDM_BF16: case TDM_I16: return 2;
+    case TDM_I8: case TDM_U8: return 1;
+    default: throw Invalid("unknown dtype " + std::to_string(dtype));
+  }
+}
+
+template <typename F>
+void dispatch(int dtype, F&& f) {
+  switch (dtype) {
+    case TDM_F32: f(static_cast<float*>(nullptr)); break;
+    case TDM_F64: f(static_cast<double*>(nullptr)); break;
+    case TDM_I32: f(static_cast<int32_t*>(nullptr)); break;
+    case TDM_I64: f(static_cast<int64_t*>(nullptr)); break;
+    default: throw Invalid("the stand-in kernels know fp32, fp64, int32 and int64");
+  }
+}
+
+template <typename T>
+T divided(T x, int world) {
+  return world > 1 ? static_cast<T>(x / static_cast<T>(world)) : x;
+}
+
+}  // namespace
+
+void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool scale_dst, bool scale_src, bool writeback_src,
+                 hipStream_t, int) {
+  dispatch(dtype, [&](auto* tag) {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    for (int i = 0; i < npairs; ++i) {
+      T* d = static_cast<T*>(pairs[i].dst);
+      T* s = const_cast<T*>(static_cast<const T*>(pairs[i].src));
+      for (int64_t k = 0; k < pairs[i].count; ++k) {
+        const T x = scale_dst ? divided(d[k], world) : d[k], y = scale_src ? divided(s[k], world) : s[k];
+        if (scale_src && writeback_src) s[k] = y;
+        d[k] = static_cast<T>(x + y);
+      }
+    }
+  });
+}
+
+void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t, int) {
+  if (world <= 1) {
+    for (int i = 0; i < npairs; ++i) std::memmove(pairs[i].dst, pairs[i].src, static_cast<size_t>(pairs[i].count) * size_of(dtype));
+    return;
+  }
+  dispatch(dtype, [&](auto* tag) {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    for (int i = 0; i < npairs; ++i) {
+      T* d = static_cast<T*>(pairs[i].dst);
+      const T* s = static_cast<const T*>(pairs[i].src);
+      for (int64_t k = 0; k < pairs[i].count; ++k) d[k] = divided(s[k], world);
+    }
+  });
+}
+
+void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t, int divide_by) {
+  if (world < 2 || world > TDM_MAX_WORLD) throw Invalid("the direct fold handles world sizes 2..8");
+  const int by = average ? (divide_by ? divide_by : world) : 1;
+  dispatch(dtype, [&](auto* tag) {
+    using T = std::remove_pointer_t<decltype(tag)>;
+    for (int i = 0; i < nseg; ++i) {
+      const tdm_fold_seg& sg = segs[i];
+      for (int64_t k = 0; k < sg.count; ++k) {
+        T acc = divided(static_cast<const T*>(sg.src[(sg.chunk + 1) % world])[k], by);
+        for (int j = 2; j <= world; ++j) acc = static_cast<T>(divided(static_cast<const T*>(sg.src[(sg.chunk + j) % world])[k], by) + acc);
+        for (int r = 0; r < world; ++r)
+          if (sg.dst[r]) static_cast<T*>(sg.dst[r])[k] = acc;
+      }
+    }
+  });
+}
+
+void zero2_step_segment(const tdm_step_seg&, int, bool, const tdm_adamw_scalars&, int, hipStream_t) {
+  throw Invalid("the stand-in kernels have no optimizer step");
+}
+
+}  // namespace tandem_hip

@@ -1,0 +1,52 @@
+"""The process-rank engine's host side without a GPU: tests/cpp/engine_host_test.cpp builds the engine from the
+library's own sources (tandem_amd/csrc/engine.hip, engine_abi.hip, abi.hip) against a stand-in for the HIP runtime and
+for the four kernel launchers (tests/cpp/fake_hip.cpp, fake_kernels.cpp), forks one process per rank and drives every
+collective through the C ABI: many in flight, both waits, the staged and the slot-ring protocol, staging windows of
+4 KiB, arenas, more collectives in flight than done words, refusals, close. Built plainly, with the host's data-race
+sanitizer and with its address and undefined-behaviour sanitizers (which cannot share a process with the real runtime).
+The stand-ins serve this program only: the package's library is never built from them, and what the kernels compute
+is the GPU tests' business."""
+
+import os
+import shutil
+import subprocess
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+SOURCES = [os.path.join(ROOT, "tandem_amd", "csrc", f) for f in ("engine.hip", "engine_abi.hip", "abi.hip")]
+DOUBLES = [os.path.join(HERE, "cpp", f) for f in ("fake_hip.cpp", "fake_kernels.cpp", "engine_host_test.cpp")]
+CASES = [("2", "staged"), ("3", "staged"), ("4", "staged"), ("5", "staged"), ("2", "ring"), ("3", "ring"), ("4", "ring"),
+         ("3", "staged", "4096")]
+VARIANTS = {"plain": ["-O2"],
+            "race": ["-O1", "-g", "-fsanitize=thread", "-fno-omit-frame-pointer"],
+            "sanitized": ["-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
+                          "-static-libasan"]}
+
+
+@pytest.fixture(scope="module")
+def programs(tmp_path_factory):
+    if shutil.which("g++") is None or not os.path.isdir("/opt/rocm/include"):
+        pytest.skip("needs g++ and the ROCm headers")
+    out = {}
+    for name, flags in VARIANTS.items():
+        exe = str(tmp_path_factory.mktemp("engine") / f"engine_host_{name}")
+        res = subprocess.run(["g++", "-std=c++17", *flags, "-Wall", "-Wextra", "-Werror", "-pthread", "-D__HIP_PLATFORM_AMD__",
+                              "-I/opt/rocm/include", "-o", exe, "-x", "c++", *SOURCES, *DOUBLES, "-lrt"],
+                             stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        out[name] = (exe if res.returncode == 0 else None, res.stdout[-3000:])
+    assert out["plain"][0], "the test program does not build:\n" + out["plain"][1]
+    return out
+
+
+@pytest.mark.parametrize("variant", list(VARIANTS))
+@pytest.mark.parametrize("case", CASES, ids=["-".join(c) for c in CASES])
+def test_engine_host_side(programs, case, variant):
+    exe, log = programs[variant]
+    if exe is None:
+        pytest.skip("this toolchain does not build the sanitized variant: " + log[-300:])
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1",
+               TSAN_OPTIONS="halt_on_error=1:exitcode=66")
+    res = subprocess.run([exe, *case], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300, env=env)
+    assert res.returncode == 0, f"{' '.join(case)} ({variant}) exit {res.returncode}:\n{res.stdout[-4000:]}"
