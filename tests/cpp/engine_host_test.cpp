@@ -5,7 +5,10 @@
 // for data races, addresses and undefined behaviour. Numbers are integer-valued, so sums are exact in any order; the
 // order of the sums is the GPU tests' business.
 //
-// usage: engine_host_test <world> <staged|ring> [staging_bytes]
+// usage: engine_host_test <world> <staged|ring> [staging_bytes|0] [dies|out_of_step]
+//   dies:        the last rank leaves right after connecting; the others' collective must time out, later calls must fail
+//                at once, close must come back
+//   out_of_step: rank 0 brings a tensor of another length than the others; every rank must be told
 
 #include <fcntl.h>
 #include <sys/mman.h>
@@ -45,13 +48,32 @@ static std::vector<int64_t> split(int64_t n, int w, bool uneven) {
   return s;
 }
 
-static int run_rank(int rank, int world, const std::string& job, std::atomic<int>* arrived) {
+// What must happen when the group falls apart: an error with a message on every rank that is still there, no hang.
+static int run_broken(tdm_engine* e, int rank, int world, const std::string& scenario) {
+  if (scenario == "dies" && rank == world - 1) ::_exit(0);  // without closing: its peers find nobody
+  std::vector<float> x(scenario == "out_of_step" && rank == 0 ? 1000 : 1001, 1.0f);
+  tdm_work* w = nullptr;
+  REQUIRE(tdm_all_reduce(e, x.data(), static_cast<int64_t>(x.size()), TDM_F32, 0, nullptr, &w) == TDM_OK);
+  const int rc = tdm_work_wait(w, nullptr);
+  const std::string said = tdm_last_error();
+  REQUIRE(rc != TDM_OK && !said.empty());
+  if (scenario == "dies") REQUIRE(rc == TDM_ETIMEOUT);
+  REQUIRE(tdm_work_done(w) == 1 && tdm_work_free(w) == TDM_OK);
+  REQUIRE(tdm_all_reduce(e, x.data(), static_cast<int64_t>(x.size()), TDM_F32, 0, nullptr, &w) != TDM_OK);  // the engine remembers
+  REQUIRE(std::string(tdm_last_error()).find("earlier collective failed") != std::string::npos);
+  (void)tdm_engine_close(e);  // its barrier may fail as well; it must return
+  REQUIRE(tdm_engine_destroy(e) == TDM_OK);
+  return 0;
+}
+
+static int run_rank(int rank, int world, const std::string& job, std::atomic<int>* arrived, const std::string& scenario) {
   g_rank = rank;
   tdm_engine* e = nullptr;
-  REQUIRE(tdm_engine_create(job.c_str(), rank, world, 2, 4096, 20.0, 0, &e) == TDM_OK);
+  REQUIRE(tdm_engine_create(job.c_str(), rank, world, 2, 4096, scenario.empty() ? 20.0 : 1.0, 0, &e) == TDM_OK);
   arrived->fetch_add(1);  // the launcher's barrier: every rank has published its region
   while (arrived->load() < world) std::this_thread::yield();
   REQUIRE(tdm_engine_connect(e) == TDM_OK);
+  if (!scenario.empty()) return run_broken(e, rank, world, scenario);
 
   const int64_t lengths[] = {0, 1, 5, 1000, 4099, 40000};
   int salt = 0;
@@ -193,7 +215,8 @@ int main(int argc, char** argv) {
   const std::string algo = argc > 2 ? argv[2] : "staged";
   if (world < 2 || world > 8) return 64;
   ::setenv("TANDEM_HIP_ALGO", algo.c_str(), 1);
-  if (argc > 3) ::setenv("TANDEM_HIP_STAGING_BYTES", argv[3], 1);
+  if (argc > 3 && std::atoll(argv[3]) > 0) ::setenv("TANDEM_HIP_STAGING_BYTES", argv[3], 1);
+  const std::string scenario = argc > 4 ? argv[4] : "";
   const std::string job = "host" + std::to_string(::getpid());
   void* shared = ::mmap(nullptr, 4096, PROT_READ | PROT_WRITE, MAP_SHARED | MAP_ANONYMOUS, -1, 0);
   if (shared == MAP_FAILED) return 65;
@@ -203,7 +226,7 @@ int main(int argc, char** argv) {
     const pid_t pid = ::fork();
     if (pid < 0) return 66;
     if (pid == 0) {
-      std::exit(run_rank(r, world, job, arrived));  // through the exit handlers: the leak check runs there
+      std::exit(run_rank(r, world, job, arrived, scenario));  // through the exit handlers: the leak check runs there
     }
     children.push_back(pid);
   }
@@ -213,5 +236,11 @@ int main(int argc, char** argv) {
     if (::waitpid(pid, &status, 0) != pid || !WIFEXITED(status) || WEXITSTATUS(status) != 0) ++failed;
   }
   if (failed) std::fprintf(stderr, "%d of %d ranks failed\n", failed, world);
+  if (failed || !scenario.empty()) {  // what a rank that did not close left in /dev/shm
+    for (int r = 0; r < world; ++r) {
+      ::shm_unlink(("/tandem-" + job + "-" + std::to_string(r) + "-hip").c_str());
+      for (int k = 0; k < 64; ++k) ::shm_unlink(("/tdmfake-" + std::to_string(children[r]) + "-" + std::to_string(k)).c_str());
+    }
+  }
   return failed ? 1 : 0;
 }

@@ -2,7 +2,8 @@
 library's own sources (tandem_amd/csrc/engine.hip, engine_abi.hip, abi.hip) against a stand-in for the HIP runtime and
 for the four kernel launchers (tests/cpp/fake_hip.cpp, fake_kernels.cpp), forks one process per rank and drives every
 collective through the C ABI: many in flight, both waits, the staged and the slot-ring protocol, staging windows of
-4 KiB, arenas, more collectives in flight than done words, refusals, close. Built plainly, with the host's data-race
+4 KiB, arenas, more collectives in flight than done words, refusals, close, and what the ranks that remain are told
+when one leaves or brings a tensor of another length. Built plainly, with the host's data-race
 sanitizer and with its address and undefined-behaviour sanitizers (which cannot share a process with the real runtime).
 The stand-ins serve this program only: the package's library is never built from them, and what the kernels compute
 is the GPU tests' business."""
@@ -18,7 +19,9 @@ ROOT = os.path.dirname(HERE)
 SOURCES = [os.path.join(ROOT, "tandem_amd", "csrc", f) for f in ("engine.hip", "engine_abi.hip", "abi.hip")]
 DOUBLES = [os.path.join(HERE, "cpp", f) for f in ("fake_hip.cpp", "fake_kernels.cpp", "engine_host_test.cpp")]
 CASES = [("2", "staged"), ("3", "staged"), ("4", "staged"), ("5", "staged"), ("2", "ring"), ("3", "ring"), ("4", "ring"),
-         ("3", "staged", "4096")]
+         ("3", "staged", "4096"),
+         # the group falls apart: a rank that leaves without a word, ranks that bring tensors of different lengths
+         ("3", "staged", "0", "dies"), ("3", "ring", "0", "dies"), ("3", "staged", "0", "out_of_step"), ("2", "ring", "0", "out_of_step")]
 VARIANTS = {"plain": ["-O2"],
             "race": ["-O1", "-g", "-fsanitize=thread", "-fno-omit-frame-pointer"],
             "sanitized": ["-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
