@@ -65,13 +65,11 @@ struct FlagPool {
     (reached(i) ? free_list : pending).push_back(i);
   }
   bool reached(int i) const { return reached(i, generation[i]); }  // its latest generation (callers hold mu)
+  // The GPU writes these words too (hipStreamWriteValue32): the host reads and writes them as atomics.
   bool reached(int i, uint32_t value) const {  // as hipStreamWaitValueGte compares
-    return reinterpret_cast<const volatile uint32_t*>(base)[i] >= value;
+    return __atomic_load_n(base + i, __ATOMIC_ACQUIRE) >= value;
   }
-  void set(int i, uint32_t value) {
-    reinterpret_cast<volatile uint32_t*>(base)[i] = value;
-    std::atomic_thread_fence(std::memory_order_seq_cst);
-  }
+  void set(int i, uint32_t value) { __atomic_store_n(base + i, value, __ATOMIC_SEQ_CST); }
 };
 
 struct Work {

@@ -1,8 +1,10 @@
 // The process-rank engine's host side on a machine without a GPU: W processes, each with an engine built from the very
 // sources of the library (engine.hip, engine_abi.hip, abi.hip) against a stand-in runtime (fake_hip.cpp) and stand-in
 // kernels (fake_kernels.cpp), run the collectives through the C ABI and check where every element ended up. What this
-// sees that the GPU tests do not: the engine's threads (caller, progress, completion) under the host's sanitizers
-// for data races, addresses and undefined behaviour. Numbers are integer-valued, so sums are exact in any order; the
+// sees that the GPU tests do not: the engine's threads (caller, progress, completion) and the stand-in's stream threads
+// under the host's sanitizers for data races, addresses and undefined behaviour. A dependency between two streams that
+// the engine forgot (the collective on the caller's producer, the caller's consumer on the collective) is a data race
+// between those threads and is reported as one. Numbers are integer-valued, so sums are exact in any order; the
 // order of the sums is the GPU tests' business.
 //
 // usage: engine_host_test <world> <staged|ring> [staging_bytes|0] [dies|out_of_step]
@@ -25,6 +27,7 @@
 #include <vector>
 
 #include "../../include/tandem_hip.h"
+#include "fake_hip.h"
 
 #define REQUIRE(cond)                                                                                     \
   do {                                                                                                    \
@@ -75,6 +78,8 @@ static int run_rank(int rank, int world, const std::string& job, std::atomic<int
   REQUIRE(tdm_engine_connect(e) == TDM_OK);
   if (!scenario.empty()) return run_broken(e, rank, world, scenario);
 
+  hipStream_t caller = nullptr;
+  REQUIRE(hipStreamCreateWithFlags(&caller, hipStreamNonBlocking) == hipSuccess);
   const int64_t lengths[] = {0, 1, 5, 1000, 4099, 40000};
   int salt = 0;
   for (int64_t n : lengths) {
@@ -90,25 +95,50 @@ static int run_rank(int rank, int world, const std::string& job, std::atomic<int
       };
       // several collectives in flight at once, waited for in order; done() polled meanwhile
       std::vector<float> a(n), b(n), c(n), d(n);
-      for (int64_t i = 0; i < n; ++i) {
-        a[i] = value(rank, i, salt);
-        b[i] = value(rank, i, salt + 100);
-        c[i] = i >= lo && i < lo + sizes[rank] ? value(rank, i, salt + 200) : -1.0f;
-        d[i] = rank == world - 1 ? value(rank, i, salt + 300) : -2.0f;
-      }
+      // Every other round the tensors are produced and consumed on a stream of the caller's: the producer is slow,
+      // so an engine that did not wait for it would fold what was there before, and the consumer runs right behind
+      // the waits, so a wait that did not order the stream would let it read too early.
+      hipStream_t st = salt % 2 ? caller : nullptr;
+      std::vector<float> b2(n);
+      fake_enqueue(st, [&, lo] {
+        if (st) std::this_thread::sleep_for(std::chrono::microseconds(300));
+        for (int64_t i = 0; i < n; ++i) {
+          a[i] = value(rank, i, salt);
+          b[i] = b2[i] = value(rank, i, salt + 100);
+          c[i] = i >= lo && i < lo + sizes[rank] ? value(rank, i, salt + 200) : -1.0f;
+          d[i] = rank == world - 1 ? value(rank, i, salt + 300) : -2.0f;
+        }
+      });
       tdm_work *wa, *wb, *wb2, *wc, *wd;
-      std::vector<float> b2 = b;
-      REQUIRE(tdm_all_reduce(e, a.data(), n, TDM_F32, 0, nullptr, &wa) == TDM_OK);
-      REQUIRE(tdm_reduce_scatter(e, b.data(), n, TDM_F32, sizes.data(), world, 0, nullptr, &wb) == TDM_OK);
-      REQUIRE(tdm_reduce_scatter_owner(e, b2.data(), n, TDM_F32, uneven ? sizes.data() : nullptr, uneven ? world : 0, 0, nullptr, &wb2) == TDM_OK);
-      REQUIRE(tdm_all_gather(e, c.data(), n, TDM_F32, sizes.data(), world, nullptr, &wc) == TDM_OK);
-      REQUIRE(tdm_broadcast(e, d.data(), n, TDM_F32, world - 1, nullptr, &wd) == TDM_OK);
+      REQUIRE(tdm_all_reduce(e, a.data(), n, TDM_F32, 0, st, &wa) == TDM_OK);
+      REQUIRE(tdm_reduce_scatter(e, b.data(), n, TDM_F32, sizes.data(), world, 0, st, &wb) == TDM_OK);
+      REQUIRE(tdm_reduce_scatter_owner(e, b2.data(), n, TDM_F32, uneven ? sizes.data() : nullptr, uneven ? world : 0, 0, st, &wb2) == TDM_OK);
+      REQUIRE(tdm_all_gather(e, c.data(), n, TDM_F32, sizes.data(), world, st, &wc) == TDM_OK);
+      REQUIRE(tdm_broadcast(e, d.data(), n, TDM_F32, world - 1, st, &wd) == TDM_OK);
       (void)tdm_work_done(wd);
-      REQUIRE(tdm_work_wait(wa, nullptr) == TDM_OK);
-      REQUIRE(tdm_work_wait_stream(wb, nullptr) == TDM_OK);
-      REQUIRE(tdm_work_wait(wb2, nullptr) == TDM_OK);
-      REQUIRE(tdm_work_wait_stream(wc, nullptr) == TDM_OK);
-      REQUIRE(tdm_work_wait(wd, nullptr) == TDM_OK);
+      REQUIRE(tdm_work_wait(wa, st) == TDM_OK);
+      REQUIRE(tdm_work_wait_stream(wb, st) == TDM_OK);
+      REQUIRE(tdm_work_wait(wb2, st) == TDM_OK);
+      REQUIRE(tdm_work_wait_stream(wc, st) == TDM_OK);
+      REQUIRE(tdm_work_wait(wd, st) == TDM_OK);
+      std::atomic<int64_t> early{0};
+      fake_enqueue(st, [&] {  // the consumer: sums what the collectives left, behind the waits
+        double sum = 0;
+        for (int64_t i = 0; i < n; ++i) sum += a[i] + c[i] + d[i];
+        double want = 0;
+        for (int64_t i = 0; i < n; ++i) {
+          for (int q = 0; q < world; ++q) want += value(q, i, salt);
+          want += value(world - 1, i, salt + 300);
+        }
+        int owner = 0;
+        int64_t end = sizes[0];
+        for (int64_t i = 0; i < n; ++i) {
+          while (i >= end) end += sizes[++owner];
+          want += value(owner, i, salt + 200);
+        }
+        if (sum != want) early.fetch_add(1);
+      });
+      REQUIRE(hipStreamSynchronize(st) == hipSuccess && early.load() == 0);
       REQUIRE(tdm_work_done(wa) == 1 && tdm_work_done(wd) == 1);
       double t0 = 0, t1 = 0;
       REQUIRE(tdm_work_times(wa, &t0, &t1) == TDM_OK && t1 >= t0);
@@ -178,8 +208,9 @@ static int run_rank(int rank, int world, const std::string& job, std::atomic<int
     shard_offs[q] = offs[q] + at * 4;  // rank q's own chunk, where the all-gather left it
     at += sizes[q];
   }
-  REQUIRE(tdm_unit_gather_direct(e, full.data(), n, TDM_F32, t + lo, sizes.data(), world, shard_offs.data(), world, nullptr, &w) == TDM_OK);
-  REQUIRE(tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
+  REQUIRE(tdm_unit_gather_direct(e, full.data(), n, TDM_F32, t + lo, sizes.data(), world, shard_offs.data(), world, caller, &w) == TDM_OK);
+  REQUIRE(tdm_work_wait(w, caller) == TDM_OK && tdm_work_free(w) == TDM_OK);
+  REQUIRE(hipStreamSynchronize(caller) == hipSuccess);
   for (int64_t i = 0, owner = 0, end = sizes[0]; i < n; ++i) {
     while (i >= end) end += sizes[++owner];
     REQUIRE(t[i] == value(static_cast<int>(owner), i, 901) && full[i] == t[i]);
@@ -204,6 +235,7 @@ static int run_rank(int rank, int world, const std::string& job, std::atomic<int
   REQUIRE(tdm_all_reduce(e, nullptr, 3, TDM_F32, 0, nullptr, &w) == TDM_EINVAL);
   const int64_t bad[2] = {1, 1};
   REQUIRE(tdm_all_gather(e, rows.data(), 3, TDM_F32, bad, 2, nullptr, &w) == TDM_EINVAL);
+  REQUIRE(hipStreamDestroy(caller) == hipSuccess);
   REQUIRE(tdm_engine_close(e) == TDM_OK);
   REQUIRE(tdm_all_reduce(e, rows.data(), 3, TDM_F32, 0, nullptr, &w) != TDM_OK);
   REQUIRE(tdm_engine_destroy(e) == TDM_OK);

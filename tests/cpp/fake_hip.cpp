@@ -4,8 +4,11 @@
 // the library the package loads is never built from it, and nothing here computes a result anybody ships.
 //
 // What it models: "device" memory is POSIX shared memory (so that an IPC memory handle can be opened by another
-// process), every stream executes at once on the calling thread (so an event is complete when recorded and a stream
-// is always idle), a stream's write of a value is a store, its wait for a value a bounded spin.
+// process). A stream is a thread with a queue: what is launched on it runs later, in order, so work on two streams
+// overlaps unless an event or a value orders it, and the data-race sanitizer sees every pair of accesses that the
+// engine left unordered. An event is complete once the stream has passed its record; a stream's write of a value is a
+// store, its wait for a value a spin, both when the stream gets there. The null stream runs everything at once in
+// the calling thread.
 
 #include <fcntl.h>
 #include <hip/hip_runtime_api.h>
@@ -15,13 +18,19 @@
 
 #include <atomic>
 #include <chrono>
+#include <condition_variable>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <deque>
+#include <functional>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <thread>
+
+#include "fake_hip.h"
 
 namespace {
 
@@ -58,7 +67,77 @@ void* map_shared(const std::string& name, size_t bytes, bool create) {
   return p;
 }
 
+// A stream: a thread that runs what is queued, in order.
+class Stream {
+ public:
+  Stream() : worker_([this] { run(); }) {}
+  ~Stream() {
+    {
+      std::lock_guard<std::mutex> lock(mu_);
+      stop_ = true;
+    }
+    cv_.notify_all();
+    worker_.join();
+  }
+  void push(std::function<void()> work) {
+    {
+      std::lock_guard<std::mutex> lock(mu_);
+      queue_.push_back(std::move(work));
+      ++pending_;
+    }
+    cv_.notify_all();
+  }
+  bool idle() {
+    std::lock_guard<std::mutex> lock(mu_);
+    return pending_ == 0;
+  }
+  void drain() {
+    std::unique_lock<std::mutex> lock(mu_);
+    done_.wait(lock, [this] { return pending_ == 0; });
+  }
+
+ private:
+  void run() {
+    for (;;) {
+      std::function<void()> work;
+      {
+        std::unique_lock<std::mutex> lock(mu_);
+        cv_.wait(lock, [this] { return stop_ || !queue_.empty(); });
+        if (queue_.empty()) return;  // stopping, and everything queued has run
+        work = std::move(queue_.front());
+        queue_.pop_front();
+      }
+      work();
+      {
+        std::lock_guard<std::mutex> lock(mu_);
+        --pending_;
+      }
+      done_.notify_all();
+    }
+  }
+  std::mutex mu_;
+  std::condition_variable cv_, done_;
+  std::deque<std::function<void()>> queue_;
+  int pending_ = 0;  // queued or running
+  bool stop_ = false;
+  std::thread worker_;  // last: the others exist before it starts
+};
+
+struct Event {
+  std::mutex mu;
+  std::condition_variable cv;
+  uint64_t recorded = 0, completed = 0;  // records asked for, and the latest one a stream has passed
+};
+
+Stream* as_stream(hipStream_t s) { return reinterpret_cast<Stream*>(s); }
+std::shared_ptr<Event> as_event(hipEvent_t e) { return *reinterpret_cast<std::shared_ptr<Event>*>(e); }
+
 }  // namespace
+
+void fake_enqueue(hipStream_t stream, std::function<void()> work) {
+  if (stream) as_stream(stream)->push(std::move(work));
+  else work();
+}
 
 extern "C" {
 
@@ -131,51 +210,94 @@ hipError_t hipIpcGetEventHandle(hipIpcEventHandle_t*, hipEvent_t) { return hipEr
 hipError_t hipIpcOpenEventHandle(hipEvent_t*, hipIpcEventHandle_t) { return hipErrorNotSupported; }
 
 hipError_t hipStreamCreateWithFlags(hipStream_t* stream, unsigned int) {
-  *stream = reinterpret_cast<hipStream_t>(new char);
+  *stream = reinterpret_cast<hipStream_t>(new Stream);
   return hipSuccess;
 }
 hipError_t hipStreamDestroy(hipStream_t stream) {
-  delete reinterpret_cast<char*>(stream);
+  delete as_stream(stream);  // runs what is queued, then joins
   return hipSuccess;
 }
-hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
-hipError_t hipStreamQuery(hipStream_t) { return hipSuccess; }
-hipError_t hipStreamWaitEvent(hipStream_t, hipEvent_t, unsigned int) { return hipSuccess; }
+hipError_t hipStreamSynchronize(hipStream_t stream) {
+  if (stream) as_stream(stream)->drain();
+  return hipSuccess;
+}
+hipError_t hipStreamQuery(hipStream_t stream) { return !stream || as_stream(stream)->idle() ? hipSuccess : hipErrorNotReady; }
 
 hipError_t hipEventCreateWithFlags(hipEvent_t* event, unsigned) {
-  *event = reinterpret_cast<hipEvent_t>(new char);
+  *event = reinterpret_cast<hipEvent_t>(new std::shared_ptr<Event>(std::make_shared<Event>()));
   return hipSuccess;
 }
 hipError_t hipEventCreate(hipEvent_t* event) { return hipEventCreateWithFlags(event, 0); }
+// As with the real runtime, an event may be destroyed while streams still have to pass or wait for it: what is queued keeps it alive.
 hipError_t hipEventDestroy(hipEvent_t event) {
-  delete reinterpret_cast<char*>(event);
+  delete reinterpret_cast<std::shared_ptr<Event>*>(event);
   return hipSuccess;
 }
-hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }
-hipError_t hipEventQuery(hipEvent_t) { return hipSuccess; }
-hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
+hipError_t hipEventRecord(hipEvent_t event, hipStream_t stream) {
+  std::shared_ptr<Event> e = as_event(event);
+  uint64_t ticket;
+  {
+    std::lock_guard<std::mutex> lock(e->mu);
+    ticket = ++e->recorded;
+  }
+  fake_enqueue(stream, [e, ticket] {
+    std::lock_guard<std::mutex> lock(e->mu);
+    if (e->completed < ticket) e->completed = ticket;
+    e->cv.notify_all();
+  });
+  return hipSuccess;
+}
+hipError_t hipEventQuery(hipEvent_t event) {
+  std::shared_ptr<Event> e = as_event(event);
+  std::lock_guard<std::mutex> lock(e->mu);
+  return e->completed >= e->recorded ? hipSuccess : hipErrorNotReady;
+}
+hipError_t hipEventSynchronize(hipEvent_t event) {
+  std::shared_ptr<Event> e = as_event(event);
+  std::unique_lock<std::mutex> lock(e->mu);
+  const uint64_t ticket = e->recorded;
+  e->cv.wait(lock, [&] { return e->completed >= ticket; });
+  return hipSuccess;
+}
 hipError_t hipEventElapsedTime(float* ms, hipEvent_t, hipEvent_t) {
   *ms = 0;
   return hipSuccess;
 }
-
-hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind, hipStream_t) {
-  std::memmove(dst, src, bytes);
-  return hipSuccess;
-}
-
-hipError_t hipStreamWriteValue32(hipStream_t, void* ptr, uint32_t value, unsigned int) {
-  reinterpret_cast<std::atomic<uint32_t>*>(ptr)->store(value, std::memory_order_release);
-  return hipSuccess;
-}
-
-// A real stream waits on the GPU and the call returns at once; here the calling thread waits (at most ten seconds).
-hipError_t hipStreamWaitValue32(hipStream_t, void* ptr, uint32_t value, unsigned int, uint32_t) {
-  const auto until = std::chrono::steady_clock::now() + std::chrono::seconds(10);
-  while (reinterpret_cast<std::atomic<uint32_t>*>(ptr)->load(std::memory_order_acquire) < value) {
-    if (std::chrono::steady_clock::now() > until) return hipErrorNotReady;
-    std::this_thread::yield();
+// The stream waits for the record that was the event's latest when this was called (none: nothing to wait for).
+hipError_t hipStreamWaitEvent(hipStream_t stream, hipEvent_t event, unsigned int) {
+  std::shared_ptr<Event> e = as_event(event);
+  uint64_t ticket;
+  {
+    std::lock_guard<std::mutex> lock(e->mu);
+    ticket = e->recorded;
   }
+  fake_enqueue(stream, [e, ticket] {
+    std::unique_lock<std::mutex> lock(e->mu);
+    e->cv.wait(lock, [&] { return e->completed >= ticket; });
+  });
+  return hipSuccess;
+}
+
+hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind, hipStream_t stream) {
+  fake_enqueue(stream, [dst, src, bytes] { std::memmove(dst, src, bytes); });
+  return hipSuccess;
+}
+
+hipError_t hipStreamWriteValue32(hipStream_t stream, void* ptr, uint32_t value, unsigned int) {
+  fake_enqueue(stream, [ptr, value] { reinterpret_cast<std::atomic<uint32_t>*>(ptr)->store(value, std::memory_order_release); });
+  return hipSuccess;
+}
+
+// When the stream gets there it waits until the word has reached the value (at most twenty seconds: then it goes on,
+// and whoever reads behind it finds the wrong numbers).
+hipError_t hipStreamWaitValue32(hipStream_t stream, void* ptr, uint32_t value, unsigned int, uint32_t) {
+  fake_enqueue(stream, [ptr, value] {
+    const auto until = std::chrono::steady_clock::now() + std::chrono::seconds(20);
+    while (reinterpret_cast<std::atomic<uint32_t>*>(ptr)->load(std::memory_order_acquire) < value) {
+      if (std::chrono::steady_clock::now() > until) return;
+      std::this_thread::yield();
+    }
+  });
   return hipSuccess;
 }
 

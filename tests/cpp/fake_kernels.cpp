@@ -1,12 +1,15 @@
 // The four launchers the engine calls (tandem_amd/csrc/common.h), as plain loops on the host: the other half of the
 // stand-in that tests/cpp/fake_hip.cpp describes, linked into tests/cpp/engine_host_test only. fp32, fp64, int32 and
 // int64; the sums are formed in the order the kernels form them, which for the integer-valued numbers the test
-// sends does not matter.
+// sends does not matter. Like a launch, each returns at once: the loop runs when the stream gets to it.
 
 #include <cstring>
 #include <string>
 
+#include <vector>
+
 #include "../../tandem_amd/csrc/common.h"
+#include "fake_hip.h"
 
 namespace tandem_hip {
 
@@ -41,50 +44,61 @@ T divided(T x, int world) {
 }  // namespace
 
 void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool scale_dst, bool scale_src, bool writeback_src,
-                 hipStream_t, int) {
-  dispatch(dtype, [&](auto* tag) {
-    using T = std::remove_pointer_t<decltype(tag)>;
-    for (int i = 0; i < npairs; ++i) {
-      T* d = static_cast<T*>(pairs[i].dst);
-      T* s = const_cast<T*>(static_cast<const T*>(pairs[i].src));
-      for (int64_t k = 0; k < pairs[i].count; ++k) {
-        const T x = scale_dst ? divided(d[k], world) : d[k], y = scale_src ? divided(s[k], world) : s[k];
-        if (scale_src && writeback_src) s[k] = y;
-        d[k] = static_cast<T>(x + y);
+                 hipStream_t stream, int) {
+  (void)size_of(dtype);
+  const std::vector<tdm_pair> ps(pairs, pairs + npairs);
+  fake_enqueue(stream, [=] {
+    dispatch(dtype, [&](auto* tag) {
+      using T = std::remove_pointer_t<decltype(tag)>;
+      for (const tdm_pair& p : ps) {
+        T* d = static_cast<T*>(p.dst);
+        T* s = const_cast<T*>(static_cast<const T*>(p.src));
+        for (int64_t k = 0; k < p.count; ++k) {
+          const T x = scale_dst ? divided(d[k], world) : d[k], y = scale_src ? divided(s[k], world) : s[k];
+          if (scale_src && writeback_src) s[k] = y;
+          d[k] = static_cast<T>(x + y);
+        }
       }
-    }
+    });
   });
 }
 
-void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t, int) {
-  if (world <= 1) {
-    for (int i = 0; i < npairs; ++i) std::memmove(pairs[i].dst, pairs[i].src, static_cast<size_t>(pairs[i].count) * size_of(dtype));
-    return;
-  }
-  dispatch(dtype, [&](auto* tag) {
-    using T = std::remove_pointer_t<decltype(tag)>;
-    for (int i = 0; i < npairs; ++i) {
-      T* d = static_cast<T*>(pairs[i].dst);
-      const T* s = static_cast<const T*>(pairs[i].src);
-      for (int64_t k = 0; k < pairs[i].count; ++k) d[k] = divided(s[k], world);
+void copy_step(const tdm_pair* pairs, int npairs, int dtype, int world, hipStream_t stream, int) {
+  const int es = size_of(dtype);
+  const std::vector<tdm_pair> ps(pairs, pairs + npairs);
+  fake_enqueue(stream, [=] {
+    if (world <= 1) {
+      for (const tdm_pair& p : ps) std::memmove(p.dst, p.src, static_cast<size_t>(p.count) * es);
+      return;
     }
+    dispatch(dtype, [&](auto* tag) {
+      using T = std::remove_pointer_t<decltype(tag)>;
+      for (const tdm_pair& p : ps) {
+        T* d = static_cast<T*>(p.dst);
+        const T* s = static_cast<const T*>(p.src);
+        for (int64_t k = 0; k < p.count; ++k) d[k] = divided(s[k], world);
+      }
+    });
   });
 }
 
-void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t, int divide_by) {
+void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool average, hipStream_t stream, int divide_by) {
   if (world < 2 || world > TDM_MAX_WORLD) throw Invalid("the direct fold handles world sizes 2..8");
+  (void)size_of(dtype);
   const int by = average ? (divide_by ? divide_by : world) : 1;
-  dispatch(dtype, [&](auto* tag) {
-    using T = std::remove_pointer_t<decltype(tag)>;
-    for (int i = 0; i < nseg; ++i) {
-      const tdm_fold_seg& sg = segs[i];
-      for (int64_t k = 0; k < sg.count; ++k) {
-        T acc = divided(static_cast<const T*>(sg.src[(sg.chunk + 1) % world])[k], by);
-        for (int j = 2; j <= world; ++j) acc = static_cast<T>(divided(static_cast<const T*>(sg.src[(sg.chunk + j) % world])[k], by) + acc);
-        for (int r = 0; r < world; ++r)
-          if (sg.dst[r]) static_cast<T*>(sg.dst[r])[k] = acc;
+  const std::vector<tdm_fold_seg> sgs(segs, segs + nseg);
+  fake_enqueue(stream, [=] {
+    dispatch(dtype, [&](auto* tag) {
+      using T = std::remove_pointer_t<decltype(tag)>;
+      for (const tdm_fold_seg& sg : sgs) {
+        for (int64_t k = 0; k < sg.count; ++k) {
+          T acc = divided(static_cast<const T*>(sg.src[(sg.chunk + 1) % world])[k], by);
+          for (int j = 2; j <= world; ++j) acc = static_cast<T>(divided(static_cast<const T*>(sg.src[(sg.chunk + j) % world])[k], by) + acc);
+          for (int r = 0; r < world; ++r)
+            if (sg.dst[r]) static_cast<T*>(sg.dst[r])[k] = acc;
+        }
       }
-    }
+    });
   });
 }
 

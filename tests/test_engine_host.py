@@ -1,7 +1,9 @@
 """The process-rank engine's host side without a GPU: tests/cpp/engine_host_test.cpp builds the engine from the
 library's own sources (tandem_amd/csrc/engine.hip, engine_abi.hip, abi.hip) against a stand-in for the HIP runtime and
-for the four kernel launchers (tests/cpp/fake_hip.cpp, fake_kernels.cpp), forks one process per rank and drives every
-collective through the C ABI: many in flight, both waits, the staged and the slot-ring protocol, staging windows of
+for the four kernel launchers (tests/cpp/fake_hip.cpp, fake_kernels.cpp: a stream is a thread with a queue, so work on
+two streams overlaps unless the engine orders it, and the data-race sanitizer sees every pair of accesses it left
+unordered), forks one process per rank and drives every collective through the C ABI: tensors produced by a slow
+producer and consumed right behind the waits on a stream of the caller's, many in flight, both waits, the staged and the slot-ring protocol, staging windows of
 4 KiB, arenas, more collectives in flight than done words, refusals, close, and what the ranks that remain are told
 when one leaves or brings a tensor of another length. Built plainly, with the host's data-race
 sanitizer and with its address and undefined-behaviour sanitizers (which cannot share a process with the real runtime).
