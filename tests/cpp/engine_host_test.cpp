@@ -7,7 +7,8 @@
 // between those threads and is reported as one. Numbers are integer-valued, so sums are exact in any order; the
 // order of the sums is the GPU tests' business.
 //
-// usage: engine_host_test <world> <staged|ring> [staging_bytes|0] [dies|out_of_step]
+// usage: engine_host_test <world> <staged|ring> [staging_bytes|0] [-|dies|out_of_step] [NAME=VALUE,...]
+//   the last argument: environment variables the engine reads (TANDEM_HIP_GATHER=stream and the like)
 //   dies:        the last rank leaves right after connecting; the others' collective must time out, later calls must fail
 //                at once, close must come back
 //   out_of_step: rank 0 brings a tensor of another length than the others; every rank must be told
@@ -217,6 +218,28 @@ static int run_rank(int rank, int world, const std::string& job, std::atomic<int
   }
   REQUIRE(tdm_fence(e, nullptr, &w) == TDM_OK && tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
 
+  // the same gather through the engine's own path (no arenas), produced and consumed on the caller's stream, with device
+  // time stamps on
+  REQUIRE(tdm_engine_set_timing(e, 1) == TDM_OK);
+  std::vector<float> shard(sizes[rank]), whole(n, -6.0f);
+  std::atomic<int64_t> wrong{0};
+  fake_enqueue(caller, [&] {
+    std::this_thread::sleep_for(std::chrono::microseconds(300));
+    for (int64_t i = 0; i < sizes[rank]; ++i) shard[i] = value(rank, lo + i, 902);
+  });
+  REQUIRE(tdm_unit_gather(e, whole.data(), n, TDM_F32, shard.data(), sizes.data(), world, caller, &w) == TDM_OK);
+  REQUIRE(tdm_work_wait_stream(w, caller) == TDM_OK);
+  fake_enqueue(caller, [&] {
+    for (int64_t i = 0, owner = 0, end = sizes[0]; i < n; ++i) {
+      while (i >= end) end += sizes[++owner];
+      if (whole[i] != value(static_cast<int>(owner), i, 902)) wrong.fetch_add(1);
+    }
+  });
+  REQUIRE(hipStreamSynchronize(caller) == hipSuccess && wrong.load() == 0);
+  double started = 0, finished = 0;
+  REQUIRE(tdm_work_times(w, &started, &finished) == TDM_OK && finished >= started && tdm_work_free(w) == TDM_OK);
+  REQUIRE(tdm_engine_set_timing(e, 0) == TDM_OK);
+
   // more collectives in flight than the engine has done words
   const int many = 1100;
   std::vector<float> rows(static_cast<size_t>(many) * 3);
@@ -248,7 +271,13 @@ int main(int argc, char** argv) {
   if (world < 2 || world > 8) return 64;
   ::setenv("TANDEM_HIP_ALGO", algo.c_str(), 1);
   if (argc > 3 && std::atoll(argv[3]) > 0) ::setenv("TANDEM_HIP_STAGING_BYTES", argv[3], 1);
-  const std::string scenario = argc > 4 ? argv[4] : "";
+  const std::string scenario = argc > 4 && std::string(argv[4]) != "-" ? argv[4] : "";
+  for (std::string rest = argc > 5 ? argv[5] : ""; !rest.empty();) {
+    const size_t comma = rest.find(','), eq = rest.find('=');
+    if (eq == std::string::npos || eq > comma) return 64;
+    ::setenv(rest.substr(0, eq).c_str(), rest.substr(eq + 1, comma == std::string::npos ? comma : comma - eq - 1).c_str(), 1);
+    rest = comma == std::string::npos ? "" : rest.substr(comma + 1);
+  }
   const std::string job = "host" + std::to_string(::getpid());
   void* shared = ::mmap(nullptr, 4096, PROT_READ | PROT_WRITE, MAP_SHARED | MAP_ANONYMOUS, -1, 0);
   if (shared == MAP_FAILED) return 65;

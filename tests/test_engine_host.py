@@ -22,6 +22,10 @@ SOURCES = [os.path.join(ROOT, "tandem_amd", "csrc", f) for f in ("engine.hip", "
 DOUBLES = [os.path.join(HERE, "cpp", f) for f in ("fake_hip.cpp", "fake_kernels.cpp", "engine_host_test.cpp")]
 CASES = [("2", "staged"), ("3", "staged"), ("4", "staged"), ("5", "staged"), ("2", "ring"), ("3", "ring"), ("4", "ring"),
          ("3", "staged", "4096"),
+         # the engine's other ways of ordering streams: gathers on a side stream, the caller's stream waited for on the
+         # GPU instead of by polling, every wait parking the stream instead of blocking the host
+         ("3", "staged", "0", "-", "TANDEM_HIP_GATHER=stream,TANDEM_HIP_READY=gpu,TANDEM_HIP_WAIT=stream"),
+         ("2", "ring", "0", "-", "TANDEM_HIP_READY=gpu,TANDEM_HIP_WAIT=stream"),
          # the group falls apart: a rank that leaves without a word, ranks that bring tensors of different lengths
          ("3", "staged", "0", "dies"), ("3", "ring", "0", "dies"), ("3", "staged", "0", "out_of_step"), ("2", "ring", "0", "out_of_step")]
 VARIANTS = {"plain": ["-O2"],
