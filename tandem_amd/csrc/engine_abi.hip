@@ -267,10 +267,12 @@ static int wait_for(tdm_work* w, tdm_stream caller, bool may_park) {
 int tdm_work_done(tdm_work* w) {
   if (w == nullptr || !w->impl) return 0;
   Work& work = *w->impl;
+  // The word is written behind the job's last kernel (or by the host, after a failure): it may be there a moment before the
+  // progress thread has marked the job as run, and a caller whose stream was let go by it must not be told "not yet".
+  if (work.flag >= 0) return work.flags->reached(work.flag, work.flag_value) ? 1 : 0;
   std::lock_guard<std::mutex> lock(work.mu);
   if (!work.finished) return 0;
   if (work.status != TDM_OK) return 1;
-  if (work.flag >= 0) return work.flags->reached(work.flag, work.flag_value) ? 1 : 0;
   if (work.done_event) return hipEventQuery(work.done_event) == hipSuccess ? 1 : 0;
   return 1;
 }
