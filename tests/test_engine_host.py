@@ -20,7 +20,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 SOURCES = [os.path.join(ROOT, "tandem_amd", "csrc", f) for f in ("engine.hip", "engine_abi.hip", "abi.hip")]
 DOUBLES = [os.path.join(HERE, "cpp", f) for f in ("fake_hip.cpp", "fake_kernels.cpp", "engine_host_test.cpp")]
-CASES = [("2", "staged"), ("3", "staged"), ("4", "staged"), ("5", "staged"), ("2", "ring"), ("3", "ring"), ("4", "ring"),
+CASES = [("2", "staged"), ("3", "staged"), ("4", "staged"), ("5", "staged"), ("8", "staged"), ("2", "ring"), ("3", "ring"), ("4", "ring"),
          ("3", "staged", "4096"),
          # the engine's other ways of ordering streams: gathers on a side stream, the caller's stream waited for on the
          # GPU instead of by polling, every wait parking the stream instead of blocking the host
