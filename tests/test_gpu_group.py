@@ -893,3 +893,38 @@ def test_tensors_in_several_arenas(world):
         for k, what in ((2, "all_gather"), (3, "gather_unit")):
             xs = [to_np(values(q + 7 * k, n, torch.float32)) for q in range(world)]
             assert np.array_equal(bits(to_np(out[what])), bits(ring.expected_all_gather(xs, sizes))), what
+
+
+def two_groups(g):
+    """A second group of the same ranks in the same processes (its own engine, thread, streams, slots and region): collectives
+    of the two are in flight at once and waited for in the opposite order."""
+    from tandem_amd import Group
+
+    dev, w, r = g.device, g.size, g.rank
+    other = Group(r, w, dev, g._barrier, slot_bytes=g.slot_bytes, slots=g.slots, timeout=g.timeout, job="second" + str(os.getppid()))
+    ok = True
+    try:
+        for k in range(12):
+            n = (1, 1000, 70_001)[k % 3]
+            a = torch.full((n,), float(r + k), device=dev)
+            b = torch.full((n,), float(2 * r + k), device=dev)
+            wa = g.all_reduce(a, async_op=True)
+            wb = other.all_reduce(b, op="avg", async_op=True)
+            wb.wait(stream_ordered=bool(k % 2))
+            wa.wait()
+            ok = ok and bool((a == sum(q + k for q in range(w))).all()) and bool((b == sum(2 * q + k for q in range(w)) / w).all())
+        x = other.shared_empty(64)
+        x.fill_(float(r))
+        other.all_reduce(x, direct=True)
+        ok = ok and bool((x == sum(range(w))).all()) and g.arena_count == 0 and other.arena_count == 1
+        torch.cuda.synchronize()
+    finally:
+        other.close()
+    g.barrier()
+    return ok
+
+
+def test_two_groups_in_the_same_processes():
+    from tandem_amd import launch
+
+    assert launch(two_groups, 2, gpus=[0, 0], timeout=TIMEOUT) == [True, True]
