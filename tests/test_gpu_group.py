@@ -928,3 +928,36 @@ def test_two_groups_in_the_same_processes():
     from tandem_amd import launch
 
     assert launch(two_groups, 2, gpus=[0, 0], timeout=TIMEOUT) == [True, True]
+
+
+def on_a_stream_of_the_callers(g):
+    """Everything on a stream the caller made: the collective starts behind what that stream holds at the call, and both kinds
+    of wait order that stream (not the default one) behind the collective."""
+    from tandem_amd import LocalWorld
+
+    dev, w = g.device, g.size
+    s = torch.cuda.Stream()
+    busy = torch.randn(1024, 1024, device=dev)
+    torch.cuda.synchronize()
+    ok = True
+    with torch.cuda.stream(s):
+        for k in range(20):
+            for _ in range(3):
+                busy = (busy @ busy) * 1e-3
+            x = torch.full((100_003,), float(g.rank + 1 + k), device=dev) + busy[0, 0] * 0
+            work = g.all_reduce(x, async_op=True)
+            y = work.wait(stream_ordered=bool(k % 2)) * 2
+            ok = ok and bool((y == 2.0 * sum(q + 1 + k for q in range(w))).all())
+        # ranks that are buffers of this process, on the same stream
+        bufs = [torch.full((50_001,), float(q + 1), device=dev) + busy[0, 0] * 0 for q in range(3)]
+        LocalWorld(3).all_reduce(bufs)
+        ok = ok and all(bool((b == 6.0).all()) for b in bufs)
+    s.synchronize()
+    g.barrier()
+    return ok
+
+
+def test_collectives_on_a_stream_of_the_callers():
+    from tandem_amd import launch
+
+    assert launch(on_a_stream_of_the_callers, 2, gpus=[0, 0], timeout=TIMEOUT) == [True, True]
