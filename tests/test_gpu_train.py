@@ -251,3 +251,51 @@ def test_step_without_zero_grad_keeps_the_old_gradients():
     for r in range(4):
         assert runs["zero2f"][r]["losses"] == runs["zero2"][r]["losses"], r
         assert torch.equal(runs["zero2f"][r]["weights"], runs["zero2"][0]["weights"]), r
+
+
+def mixed_dtypes(g, direct):
+    """DDP over a model whose parameters are fp32 and bf16: a bucket ends where the dtype changes (tandem/ddp.py:56-68 in the
+    reference), and every gradient must come out as g0/2 + g1/2 in its own dtype."""
+    from tandem_amd.ddp import DDP
+
+    class Mixed(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = torch.nn.Linear(48, 64)
+            self.b = torch.nn.Linear(64, 64).to(torch.bfloat16)
+            self.c = torch.nn.Linear(64, 8)
+
+        def forward(self, x):
+            return self.c(self.b(self.a(x).to(torch.bfloat16)).float())
+
+    deterministic()
+    dev = g.device
+    torch.manual_seed(0)
+    model = Mixed().to(dev)
+    x = torch.randn(16, 48, device=dev, generator=torch.Generator(device=dev).manual_seed(10 + g.rank))
+    model(x).square().mean().backward()
+    local = [p.grad.clone() for p in model.parameters()]
+    want = []
+    for t in local:  # every rank's gradient, then the mean as the ring forms it at two ranks
+        both = torch.empty(2 * t.numel(), device=dev, dtype=t.dtype)
+        both[g.rank * t.numel():(g.rank + 1) * t.numel()] = t.reshape(-1)
+        g.all_gather(both)
+        want.append((both[:t.numel()] / 2 + both[t.numel():] / 2).view_as(t))
+    model.zero_grad()
+    z = DDP(model, g, bucket_bytes=8 << 10, direct=direct)
+    dtypes = [b.flat.dtype for b in z.buckets]
+    z(x).square().mean().backward()
+    torch.cuda.synchronize()
+    same = all(p.grad.dtype == w.dtype and torch.equal(p.grad.view(torch.int16 if w.dtype == torch.bfloat16 else torch.int32),
+                                                        w.view(torch.int16 if w.dtype == torch.bfloat16 else torch.int32))
+               for p, w in zip(model.parameters(), want))
+    return same, [str(d) for d in dtypes]
+
+
+@pytest.mark.parametrize("direct", [False, True])
+def test_ddp_over_parameters_of_two_dtypes(direct):
+    from tandem_amd import launch
+
+    for same, dtypes in launch(mixed_dtypes, 2, direct, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT):
+        assert same
+        assert "torch.bfloat16" in dtypes and "torch.float32" in dtypes and len(dtypes) >= 3
