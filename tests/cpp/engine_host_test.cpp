@@ -218,6 +218,34 @@ static int run_rank(int rank, int world, const std::string& job, std::atomic<int
   }
   REQUIRE(tdm_fence(e, nullptr, &w) == TDM_OK && tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
 
+  // ZeRO-2's step as one launch per rank: gradients and parameters in the second arena, every rank updates its own shard
+  // and writes it into every rank's parameters (the stand-in's "step" is parameter - averaged gradient)
+  {
+    float* grads = t;                                            // n floats at offs[q]
+    float* params = t + (n + 63) / 64 * 64;                      // behind them, on every rank at the same distance
+    std::vector<int64_t> goffs(world), poffs(world);
+    for (int q = 0; q < world; ++q) {
+      goffs[q] = offs[q] + lo * 4;
+      poffs[q] = offs[q] + ((n + 63) / 64 * 64 + lo) * 4;
+    }
+    for (int64_t i = 0; i < n; ++i) {
+      grads[i] = static_cast<float>(world) * value(rank, i, 903);
+      params[i] = value(0, i, 904);  // the same on every rank
+    }
+    std::vector<float> m(sizes[rank], 0.0f), v(sizes[rank], 0.0f);
+    tdm_adamw_scalars sc;
+    std::memset(&sc, 0, sizeof sc);
+    REQUIRE(tdm_direct_zero2_step(e, params + lo, poffs.data(), grads + lo, goffs.data(), world, m.data(), v.data(), sizes[rank], n, 1,
+                                  &sc, TDM_ADAMW_HOST_ORDER, nullptr, &w) == TDM_OK);
+    REQUIRE(tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
+    for (int64_t i = 0; i < n; ++i) {
+      float g = 0;
+      for (int q = 0; q < world; ++q) g += value(q, i, 903);
+      REQUIRE(params[i] == value(0, i, 904) - g);
+      if (i >= lo && i < lo + sizes[rank]) REQUIRE(m[i - lo] == g && v[i - lo] == g * g);
+    }
+  }
+
   // the same gather through the engine's own path (no arenas), produced and consumed on the caller's stream, with device
   // time stamps on
   REQUIRE(tdm_engine_set_timing(e, 1) == TDM_OK);

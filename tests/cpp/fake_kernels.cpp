@@ -102,8 +102,24 @@ void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool av
   });
 }
 
-void zero2_step_segment(const tdm_step_seg&, int, bool, const tdm_adamw_scalars&, int, hipStream_t) {
-  throw Invalid("the stand-in kernels have no optimizer step");
+// The data flow of ZeRO-2's step, not its arithmetic: the shard's gradients folded in the ring's order and averaged, the
+// moments bumped, and "parameter - gradient" written into every rank's parameter buffer. (AdamW itself is the kernels'
+// and the GPU tests' business.)
+void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const tdm_adamw_scalars&, int, hipStream_t stream) {
+  if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
+  const tdm_step_seg seg = sg;
+  fake_enqueue(stream, [=] {
+    float* m = static_cast<float*>(seg.exp_avg);
+    float* v = static_cast<float*>(seg.exp_avg_sq);
+    for (int64_t k = 0; k < seg.count; ++k) {
+      float g = divided(static_cast<const float*>(seg.grad[(seg.chunk + 1) % world])[k], average ? world : 1);
+      for (int j = 2; j <= world; ++j) g = divided(static_cast<const float*>(seg.grad[(seg.chunk + j) % world])[k], average ? world : 1) + g;
+      m[k] += g;
+      v[k] += g * g;
+      const float p = static_cast<const float*>(seg.param[seg.chunk])[k] - g;
+      for (int r = 0; r < world; ++r) static_cast<float*>(seg.param[r])[k] = p;
+    }
+  });
 }
 
 }  // namespace tandem_hip
