@@ -71,11 +71,18 @@ class Work:
 
     def __del__(self):
         h, self._handle = getattr(self, "_handle", None), None
-        if h is not None:
-            try:
-                lib().tdm_work_free(h)
-            except Exception:
-                pass
+        if h is None:
+            return
+        try:
+            g = self._group
+            if not self._waited and self._keep and not g._closed:
+                # Dropped without a wait: nothing orders the caller's stream behind the collective, so the tensors must
+                # outlive it here (the reference's engine holds them until the job has run, tandem/csrc/collectives.cpp:314-317).
+                g._orphans.append((h, self._keep))
+                return
+            lib().tdm_work_free(h)
+        except Exception:
+            pass
 
 
 class Group:
@@ -96,6 +103,7 @@ class Group:
         self._engine = None
         self._arena = None
         self.arena_count = 0  # arenas shared so far
+        self._orphans = []  # (handle, tensors) of collectives whose Work was dropped before anybody waited for it
         if self.backend != "hip":
             raise CommError(f"unknown backend {self.backend} (tandem_amd provides \"hip\")")
         if self.transport != "device":
@@ -158,9 +166,21 @@ class Group:
         self._trace = spans
 
     # ---- plumbing
+    def _reap(self):
+        """Lets go of the tensors of dropped collectives that have finished on the GPU."""
+        still = []
+        for h, keep in self._orphans:
+            if lib().tdm_work_done(h):
+                lib().tdm_work_free(h)
+            else:
+                still.append((h, keep))
+        self._orphans = still
+
     def _start(self, name, call, result, nbytes, async_op, keep=()):
         if self._closed:
             raise CommError("group is closed")
+        if self._orphans:
+            self._reap()
         out = ctypes.c_void_p()
         try:
             check(call(ctypes.byref(out)))
@@ -472,12 +492,15 @@ class Group:
         self.barrier()
         self._closed = True
         eng, self._engine = self._engine, None
+        orphans, self._orphans = self._orphans, []  # tdm_engine_close runs what is queued and waits for the GPU
         self._arena = None  # the engine frees it; tensors carved from it must not be used after close()
         try:
             check(lib().tdm_engine_close(eng))
         except Exception as e:
             raise CommError(f"close: {e}") from e
         finally:
+            for h, _ in orphans:
+                lib().tdm_work_free(h)
             lib().tdm_engine_destroy(eng)
 
     def abandon(self):
@@ -486,8 +509,11 @@ class Group:
         self._closed = True
         self._untimed = []
         eng, self._engine = self._engine, None
+        orphans, self._orphans = self._orphans, []
         if eng is not None:
             lib().tdm_engine_destroy(eng)
+        for h, _ in orphans:
+            lib().tdm_work_free(h)
 
 
 def _worker(rank, size, fn, args, barrier, device, slot_bytes, slots, backend, job, gpus, timeout, results):

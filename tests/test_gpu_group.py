@@ -961,3 +961,36 @@ def test_collectives_on_a_stream_of_the_callers():
     from tandem_amd import launch
 
     assert launch(on_a_stream_of_the_callers, 2, gpus=[0, 0], timeout=TIMEOUT) == [True, True]
+
+
+def dropped_without_a_wait(g):
+    """A Work that is dropped before anybody waited for it: its tensors stay alive until the collective has run (nothing
+    orders the caller's stream behind it, so the allocator must not hand their memory out again)."""
+    dev, w = g.device, g.size
+    busy = torch.randn(2048, 2048, device=dev)
+    for _ in range(10):
+        busy = (busy @ busy) * 1e-4  # the collectives' inputs are ready only behind these
+    where = []
+    for k in range(8):
+        x = torch.full((200_003,), float(g.rank + k), device=dev) + busy[0, 0] * 0
+        where.append(x.data_ptr())
+        g.all_reduce(x, async_op=True)  # the Work goes at once
+        del x
+    held = len(g._orphans)
+    fresh = [torch.zeros(200_003, device=dev) for _ in range(8)]
+    aliased = sum(f.data_ptr() in where for f in fresh)
+    y = torch.full((1000,), float(g.rank), device=dev)
+    g.all_reduce(y)  # in order behind the dropped ones
+    g.barrier()
+    torch.cuda.synchronize()
+    g._reap()
+    return held, aliased, len(g._orphans), bool((y == sum(range(w))).all())
+
+
+def test_a_work_dropped_without_a_wait_keeps_its_tensors():
+    from tandem_amd import launch
+
+    for held, aliased, left, ok in launch(dropped_without_a_wait, 2, gpus=[0, 0], timeout=TIMEOUT):
+        assert held >= 1, "every collective had finished before its Work was dropped: nothing was exercised"
+        assert aliased == 0 or held < 8
+        assert left == 0 and ok
