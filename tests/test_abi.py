@@ -129,3 +129,21 @@ def test_the_library_exports_only_what_the_header_declares():
     ours = sorted(n for n in names if n.startswith("tdm_"))
     assert ours == _lib.exported_symbols()
     assert not [n for n in names if "tandem_hip" in n], "internal C++ symbols are exported"
+
+
+def test_the_product_stays_clear_of_the_checkers():
+    """Nothing the package is made of names the oracle or the test doubles: the library is built from
+    tandem_amd/csrc alone, and no Python module of the package imports from oracle/ or tests/."""
+    import re
+
+    from tandem_amd import build
+
+    pkg = os.path.join(ROOT, "tandem_amd")
+    assert all(os.path.dirname(os.path.join(build.CSRC, s)) == build.CSRC for s in build.SOURCES)
+    for dirpath, _, names in os.walk(pkg):
+        for name in names:
+            if not name.endswith((".py", ".hip", ".h")):
+                continue
+            text = open(os.path.join(dirpath, name)).read()
+            assert not re.search(r"^\s*(from|import)\s+(oracle|tests)\b", text, re.M), name
+            assert "fake_hip" not in text and "fake_kernels" not in text and "oracle/" not in text, name
