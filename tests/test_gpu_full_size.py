@@ -205,7 +205,7 @@ def config1_rank(g, direct):
 
 @pytest.mark.parametrize("path", ["staged", "small", "ring", "direct"])
 def test_config_1_all_reduce_on_every_path(path, monkeypatch):
-    """BASELINE's first configuration as the hip backend runs it: launch(..., 2),
+    """The reference's own CPU-runnable configuration as the hip backend runs it: launch(..., 2),
     all_reduce(avg) of randn(1_048_576) seeded per rank, result x0/2 + x1/2 bit for bit on both
     ranks, through the staged passes, the one-handshake form for small tensors, the slot ring
     (two chunks of 2 MiB, one piece each) and arena to arena."""
