@@ -8,7 +8,9 @@
 // overlaps unless an event or a value orders it, and the data-race sanitizer sees every pair of accesses that the
 // engine left unordered. An event is complete once the stream has passed its record; a stream's write of a value is a
 // store, its wait for a value a spin, both when the stream gets there. The null stream runs everything at once in
-// the calling thread.
+// the calling thread. With FAKE_HIP_JITTER_US=n in the environment every piece of work on a stream starts up to n
+// microseconds late, a different amount each time: streams then lag behind the host by varying distances, and whatever
+// the engine assumed about their progress without checking shows as a wrong number or a data race.
 
 #include <fcntl.h>
 #include <hip/hip_runtime_api.h>
@@ -107,6 +109,10 @@ class Stream {
         work = std::move(queue_.front());
         queue_.pop_front();
       }
+      if (jitter_us_ > 0) {  // FAKE_HIP_JITTER_US: every piece of work starts up to that many microseconds late
+        seed_ = seed_ * 6364136223846793005ull + 1442695040888963407ull;
+        std::this_thread::sleep_for(std::chrono::microseconds((seed_ >> 33) % (static_cast<uint64_t>(jitter_us_) + 1)));
+      }
       work();
       {
         std::lock_guard<std::mutex> lock(mu_);
@@ -120,6 +126,8 @@ class Stream {
   std::deque<std::function<void()>> queue_;
   int pending_ = 0;  // queued or running
   bool stop_ = false;
+  const int jitter_us_ = std::getenv("FAKE_HIP_JITTER_US") ? std::atoi(std::getenv("FAKE_HIP_JITTER_US")) : 0;
+  uint64_t seed_ = static_cast<uint64_t>(::getpid()) * 2654435761u + reinterpret_cast<uintptr_t>(this);
   std::thread worker_;  // last: the others exist before it starts
 };
 
