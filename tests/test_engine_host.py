@@ -42,13 +42,15 @@ VARIANTS = {"plain": ["-O2"],
 def programs(tmp_path_factory):
     if shutil.which("g++") is None or not os.path.isdir("/opt/rocm/include"):
         pytest.skip("needs g++ and the ROCm headers")
-    out = {}
-    for name, flags in VARIANTS.items():
+    out, builds = {}, {}
+    for name, flags in VARIANTS.items():  # the three builds side by side
         exe = str(tmp_path_factory.mktemp("engine") / f"engine_host_{name}")
-        res = subprocess.run(["g++", "-std=c++17", *flags, "-Wall", "-Wextra", "-Werror", "-pthread", "-D__HIP_PLATFORM_AMD__",
-                              "-I/opt/rocm/include", "-o", exe, "-x", "c++", *SOURCES, *DOUBLES, "-lrt"],
-                             stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-        out[name] = (exe if res.returncode == 0 else None, res.stdout[-3000:])
+        builds[name] = (exe, subprocess.Popen(["g++", "-std=c++17", *flags, "-Wall", "-Wextra", "-Werror", "-pthread", "-D__HIP_PLATFORM_AMD__",
+                                               "-I/opt/rocm/include", "-o", exe, "-x", "c++", *SOURCES, *DOUBLES, "-lrt"],
+                                              stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
+    for name, (exe, proc) in builds.items():
+        log = proc.communicate()[0]
+        out[name] = (exe if proc.returncode == 0 else None, log[-3000:])
     assert out["plain"][0], "the test program does not build:\n" + out["plain"][1]
     return out
 
