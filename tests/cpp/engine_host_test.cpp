@@ -7,7 +7,7 @@
 // between those threads and is reported as one. Numbers are integer-valued, so sums are exact in any order; the
 // order of the sums is the GPU tests' business.
 //
-// usage: engine_host_test <world> <staged|ring> [staging_bytes|0] [-|dies|out_of_step] [NAME=VALUE,...]
+// usage: engine_host_test <world> <staged|ring> [staging_bytes|0] [-|dies|out_of_step|no_ipc_events] [NAME=VALUE,...]
 //   the last argument: environment variables the engine reads (TANDEM_HIP_GATHER=stream and the like)
 //   dies:        the last rank leaves right after connecting; the others' collective must time out, later calls must fail
 //                at once, close must come back
@@ -73,6 +73,16 @@ static int run_broken(tdm_engine* e, int rank, int world, const std::string& sce
 static int run_rank(int rank, int world, const std::string& job, std::atomic<int>* arrived, const std::string& scenario) {
   g_rank = rank;
   tdm_engine* e = nullptr;
+  if (scenario == "no_ipc_events") {  // a platform without interprocess events: the engine says so by name and leaves nothing behind
+    ::setenv("TANDEM_HIP_SYNC", "event", 1);
+    REQUIRE(tdm_engine_create(job.c_str(), rank, world, 2, 4096, 1.0, 0, &e) != TDM_OK && e == nullptr);
+    REQUIRE(std::string(tdm_last_error()).find("cannot export interprocess events") != std::string::npos);
+    REQUIRE(tdm_engine_create(job.c_str(), rank, world, 0, 4096, 1.0, 0, &e) == TDM_EINVAL);
+    REQUIRE(tdm_engine_create(job.c_str(), rank, world, 2, 100, 1.0, 0, &e) == TDM_EINVAL);
+    REQUIRE(tdm_engine_create(job.c_str(), world, world, 2, 4096, 1.0, 0, &e) == TDM_EINVAL);
+    REQUIRE(tdm_engine_create(job.c_str(), rank, world, 2, 4096, 1.0, -1, &e) == TDM_EINVAL);
+    return 0;
+  }
   REQUIRE(tdm_engine_create(job.c_str(), rank, world, 2, 4096, scenario.empty() ? 20.0 : 1.0, 0, &e) == TDM_OK);
   arrived->fetch_add(1);  // the launcher's barrier: every rank has published its region
   while (arrived->load() < world) std::this_thread::yield();

@@ -31,7 +31,9 @@ CASES = [("2", "staged"), ("3", "staged"), ("4", "staged"), ("5", "staged"), ("8
          ("3", "staged", "4096", "-", "FAKE_HIP_JITTER_US=200"), ("3", "ring", "0", "-", "FAKE_HIP_JITTER_US=200"),
          ("2", "staged", "4096", "-", "FAKE_HIP_JITTER_US=200,TANDEM_HIP_GATHER=stream,TANDEM_HIP_READY=gpu,TANDEM_HIP_WAIT=stream"),
          # the group falls apart: a rank that leaves without a word, ranks that bring tensors of different lengths
-         ("3", "staged", "0", "dies"), ("3", "ring", "0", "dies"), ("3", "staged", "0", "out_of_step"), ("2", "ring", "0", "out_of_step")]
+         ("3", "staged", "0", "dies"), ("3", "ring", "0", "dies"), ("3", "staged", "0", "out_of_step"), ("2", "ring", "0", "out_of_step"),
+         # an engine that cannot start (no interprocess events for TANDEM_HIP_SYNC=event; bad arguments) leaves nothing behind
+         ("2", "staged", "0", "no_ipc_events")]
 VARIANTS = {"plain": ["-O2"],
             "race": ["-O1", "-g", "-fsanitize=thread", "-fno-omit-frame-pointer"],
             "sanitized": ["-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer",
