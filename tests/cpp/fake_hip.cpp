@@ -131,11 +131,43 @@ class Stream {
   std::thread worker_;  // last: the others exist before it starts
 };
 
-struct Event {
-  std::mutex mu;
-  std::condition_variable cv;
-  uint64_t recorded = 0, completed = 0;  // records asked for, and the latest one a stream has passed
+// An event's state: records asked for, and the latest one a stream has passed. Two counters of atomics, so that an
+// interprocess event (FAKE_HIP_IPC_EVENTS=1; refused otherwise, as on the machines the engine was built on) can keep them in
+// shared memory, where the process that opened the handle waits for records of the process that made it.
+struct EventState {
+  std::atomic<uint64_t> recorded, completed;
 };
+
+struct Event {
+  EventState* state = nullptr;
+  std::string shared_name;  // of the shared-memory object of an interprocess event; empty: state is this process's own
+  bool owner = false;
+  ~Event() {
+    if (shared_name.empty()) {
+      delete state;
+    } else {
+      ::munmap(state, sizeof(EventState));
+      if (owner) ::shm_unlink(shared_name.c_str());
+    }
+  }
+  void wait_for(uint64_t ticket) const {
+    while (state->completed.load(std::memory_order_acquire) < ticket) std::this_thread::yield();
+  }
+};
+
+bool ipc_events() { return std::getenv("FAKE_HIP_IPC_EVENTS") != nullptr; }
+
+EventState* map_event(const std::string& name, bool create) {
+  const int fd = ::shm_open(name.c_str(), create ? (O_CREAT | O_EXCL | O_RDWR) : O_RDWR, 0600);
+  if (fd < 0) return nullptr;
+  if (create && ::ftruncate(fd, sizeof(EventState)) != 0) {
+    ::close(fd);
+    return nullptr;
+  }
+  void* p = ::mmap(nullptr, sizeof(EventState), PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+  ::close(fd);
+  return p == MAP_FAILED ? nullptr : static_cast<EventState*>(p);  // a fresh object is all zeros: both counters at 0
+}
 
 Stream* as_stream(hipStream_t s) { return reinterpret_cast<Stream*>(s); }
 std::shared_ptr<Event> as_event(hipEvent_t e) { return *reinterpret_cast<std::shared_ptr<Event>*>(e); }
@@ -214,8 +246,23 @@ hipError_t hipIpcOpenMemHandle(void** ptr, hipIpcMemHandle_t handle, unsigned in
 
 hipError_t hipIpcCloseMemHandle(void* ptr) { return hipFree(ptr); }  // opened blocks carry no name: nothing is unlinked
 
-hipError_t hipIpcGetEventHandle(hipIpcEventHandle_t*, hipEvent_t) { return hipErrorNotSupported; }
-hipError_t hipIpcOpenEventHandle(hipEvent_t*, hipIpcEventHandle_t) { return hipErrorNotSupported; }
+hipError_t hipIpcGetEventHandle(hipIpcEventHandle_t* handle, hipEvent_t event) {
+  std::shared_ptr<Event> e = as_event(event);
+  if (!ipc_events() || e->shared_name.empty() || e->shared_name.size() >= sizeof handle->reserved) return hipErrorNotSupported;
+  std::memset(handle, 0, sizeof *handle);
+  std::memcpy(handle->reserved, e->shared_name.c_str(), e->shared_name.size());
+  return hipSuccess;
+}
+hipError_t hipIpcOpenEventHandle(hipEvent_t* event, hipIpcEventHandle_t handle) {
+  char name[sizeof handle.reserved + 1] = {0};
+  std::memcpy(name, handle.reserved, sizeof handle.reserved);
+  auto e = std::make_shared<Event>();
+  e->state = map_event(name, false);
+  if (!e->state) return hipErrorInvalidValue;
+  e->shared_name = name;
+  *event = reinterpret_cast<hipEvent_t>(new std::shared_ptr<Event>(std::move(e)));
+  return hipSuccess;
+}
 
 hipError_t hipStreamCreateWithFlags(hipStream_t* stream, unsigned int) {
   *stream = reinterpret_cast<hipStream_t>(new Stream);
@@ -231,8 +278,17 @@ hipError_t hipStreamSynchronize(hipStream_t stream) {
 }
 hipError_t hipStreamQuery(hipStream_t stream) { return !stream || as_stream(stream)->idle() ? hipSuccess : hipErrorNotReady; }
 
-hipError_t hipEventCreateWithFlags(hipEvent_t* event, unsigned) {
-  *event = reinterpret_cast<hipEvent_t>(new std::shared_ptr<Event>(std::make_shared<Event>()));
+hipError_t hipEventCreateWithFlags(hipEvent_t* event, unsigned flags) {
+  auto e = std::make_shared<Event>();
+  if ((flags & hipEventInterprocess) && ipc_events()) {
+    e->shared_name = "/tdmfake-ev-" + std::to_string(::getpid()) + "-" + std::to_string(g_serial.fetch_add(1));
+    e->state = map_event(e->shared_name, true);
+    e->owner = true;
+    if (!e->state) return hipErrorOutOfMemory;
+  } else {
+    e->state = new EventState{};
+  }
+  *event = reinterpret_cast<hipEvent_t>(new std::shared_ptr<Event>(std::move(e)));
   return hipSuccess;
 }
 hipError_t hipEventCreate(hipEvent_t* event) { return hipEventCreateWithFlags(event, 0); }
@@ -243,28 +299,21 @@ hipError_t hipEventDestroy(hipEvent_t event) {
 }
 hipError_t hipEventRecord(hipEvent_t event, hipStream_t stream) {
   std::shared_ptr<Event> e = as_event(event);
-  uint64_t ticket;
-  {
-    std::lock_guard<std::mutex> lock(e->mu);
-    ticket = ++e->recorded;
-  }
+  const uint64_t ticket = e->state->recorded.fetch_add(1, std::memory_order_acq_rel) + 1;
   fake_enqueue(stream, [e, ticket] {
-    std::lock_guard<std::mutex> lock(e->mu);
-    if (e->completed < ticket) e->completed = ticket;
-    e->cv.notify_all();
+    uint64_t seen = e->state->completed.load(std::memory_order_relaxed);
+    while (seen < ticket && !e->state->completed.compare_exchange_weak(seen, ticket, std::memory_order_release)) {
+    }
   });
   return hipSuccess;
 }
 hipError_t hipEventQuery(hipEvent_t event) {
   std::shared_ptr<Event> e = as_event(event);
-  std::lock_guard<std::mutex> lock(e->mu);
-  return e->completed >= e->recorded ? hipSuccess : hipErrorNotReady;
+  return e->state->completed.load(std::memory_order_acquire) >= e->state->recorded.load(std::memory_order_acquire) ? hipSuccess : hipErrorNotReady;
 }
 hipError_t hipEventSynchronize(hipEvent_t event) {
   std::shared_ptr<Event> e = as_event(event);
-  std::unique_lock<std::mutex> lock(e->mu);
-  const uint64_t ticket = e->recorded;
-  e->cv.wait(lock, [&] { return e->completed >= ticket; });
+  e->wait_for(e->state->recorded.load(std::memory_order_acquire));
   return hipSuccess;
 }
 hipError_t hipEventElapsedTime(float* ms, hipEvent_t, hipEvent_t) {
@@ -274,15 +323,8 @@ hipError_t hipEventElapsedTime(float* ms, hipEvent_t, hipEvent_t) {
 // The stream waits for the record that was the event's latest when this was called (none: nothing to wait for).
 hipError_t hipStreamWaitEvent(hipStream_t stream, hipEvent_t event, unsigned int) {
   std::shared_ptr<Event> e = as_event(event);
-  uint64_t ticket;
-  {
-    std::lock_guard<std::mutex> lock(e->mu);
-    ticket = e->recorded;
-  }
-  fake_enqueue(stream, [e, ticket] {
-    std::unique_lock<std::mutex> lock(e->mu);
-    e->cv.wait(lock, [&] { return e->completed >= ticket; });
-  });
+  const uint64_t ticket = e->state->recorded.load(std::memory_order_acquire);
+  fake_enqueue(stream, [e, ticket] { e->wait_for(ticket); });
   return hipSuccess;
 }
 

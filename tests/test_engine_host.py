@@ -30,6 +30,10 @@ CASES = [("2", "staged"), ("3", "staged"), ("4", "staged"), ("5", "staged"), ("8
          # with staging windows of 4 KiB so that the two halves are reused many times
          ("3", "staged", "4096", "-", "FAKE_HIP_JITTER_US=200"), ("3", "ring", "0", "-", "FAKE_HIP_JITTER_US=200"),
          ("2", "staged", "4096", "-", "FAKE_HIP_JITTER_US=200,TANDEM_HIP_GATHER=stream,TANDEM_HIP_READY=gpu,TANDEM_HIP_WAIT=stream"),
+         # slot hand-over ordered by interprocess events (TANDEM_HIP_SYNC=event), which the machines this was built on
+         # refuse and the stand-in can offer: the only place that path runs
+         ("3", "ring", "0", "-", "TANDEM_HIP_SYNC=event,FAKE_HIP_IPC_EVENTS=1"),
+         ("4", "ring", "0", "-", "TANDEM_HIP_SYNC=event,FAKE_HIP_IPC_EVENTS=1,FAKE_HIP_JITTER_US=200"),
          # the group falls apart: a rank that leaves without a word, ranks that bring tensors of different lengths
          ("3", "staged", "0", "dies"), ("3", "ring", "0", "dies"), ("3", "staged", "0", "out_of_step"), ("2", "ring", "0", "out_of_step"),
          # an engine that cannot start (no interprocess events for TANDEM_HIP_SYNC=event; bad arguments) leaves nothing behind
