@@ -61,7 +61,9 @@ static int run_broken(tdm_engine* e, int rank, int world, const std::string& sce
   const int rc = tdm_work_wait(w, nullptr);
   const std::string said = tdm_last_error();
   REQUIRE(rc != TDM_OK && !said.empty());
-  if (scenario == "dies") REQUIRE(rc == TDM_ETIMEOUT);
+  // a neighbour of the rank that left times out; a rank further along the ring may instead be reached by the closing
+  // barrier of one that already has, where it expected a piece
+  if (scenario == "dies") REQUIRE(rc == TDM_ETIMEOUT || said.find("out of step") != std::string::npos);
   REQUIRE(tdm_work_done(w) == 1 && tdm_work_free(w) == TDM_OK);
   REQUIRE(tdm_all_reduce(e, x.data(), static_cast<int64_t>(x.size()), TDM_F32, 0, nullptr, &w) != TDM_OK);  // the engine remembers
   REQUIRE(std::string(tdm_last_error()).find("earlier collective failed") != std::string::npos);
