@@ -150,3 +150,72 @@ def test_wrappers_refuse_a_group_without_the_gather_helpers():
         ZeRO(GPT(CFG), Bare(), 2)
     with pytest.raises(ValueError):
         ZeRO(GPT(CFG), Bare(), 3)
+
+
+class _Arenas:
+    """What ShardHome and DDP ask of a group's arenas, on the CPU: the allocator of tandem_amd.Group.shared_empty
+    (256-byte aligned, a new arena when `grow` is given and the tensor does not fit) over plain tensors."""
+
+    ARENA_LIMIT = (1 << 31) - 4096
+
+    def __init__(self, rank, size):
+        self.rank, self.size = rank, size
+        self.arenas, self.used = [], 0
+
+    def shared_empty(self, numel, dtype=torch.float32, grow=None):
+        es = torch.empty(0, dtype=dtype).element_size()
+        need = numel * es
+        at = -(-self.used // 256) * 256
+        if not self.arenas or at + need > self.arenas[-1].numel():
+            assert grow is not None or not self.arenas
+            self.arenas.append(torch.zeros(max(need, min(int(grow or 0), self.ARENA_LIMIT)), dtype=torch.uint8))
+            at = 0
+        self.used = at + need
+        return self.arenas[-1][at:at + need].view(dtype)
+
+    def arena_offset(self, t):
+        for k, a in enumerate(self.arenas):
+            off = t.data_ptr() - a.data_ptr()
+            if 0 <= off and off + t.numel() * t.element_size() <= a.numel():
+                return (k << 31) + off
+        return None
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_shard_home_lays_units_out_in_slabs(seed, monkeypatch):
+    """Every unit's shard lies inside one slab, no two shards of a rank overlap, a slab ends before the limit unless one
+    unit alone is longer, and every rank computes the same places for every rank."""
+    import random
+
+    from tandem_amd.fsdp import ShardHome
+
+    rng = random.Random(seed)
+    world = rng.choice([2, 3, 4, 8])
+    monkeypatch.setattr(ShardHome, "SLAB_BYTES", rng.choice([4096, 16384, 1 << 20]))
+    units = []
+    for _ in range(rng.randrange(1, 20)):
+        total = rng.choice([0, 1, 7, 1000, 5000, 40_000])
+        units.append([total // world + (1 if q < total % world else 0) for q in range(world)])
+    homes = []
+    before = rng.choice([0, 0, 3, 499])  # something of the group's own before the shards: the same on every rank
+    for r in range(world):
+        g = _Arenas(r, world)
+        if before:
+            g.shared_empty(before)
+        homes.append((ShardHome(g, units, torch.float32), g))
+    cap = ShardHome.SLAB_BYTES // 4
+    for r, (home, g) in enumerate(homes):
+        spans = []
+        for k, sizes in enumerate(units):
+            shard = home.shard(k, sizes[r])
+            assert shard.numel() == sizes[r]
+            offs = home.peer_offsets(k)
+            assert offs == homes[0][0].peer_offsets(k)  # the same on every rank
+            if sizes[r]:
+                assert g.arena_offset(shard) == offs[r] and offs[r] % 16 == 0
+                spans.append((offs[r], offs[r] + 4 * sizes[r]))
+        spans.sort()
+        assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
+        for slab in home.slabs:
+            alone = any(max(-(-s // 4) * 4 for s in sizes) >= slab.numel() for sizes in units)
+            assert slab.numel() <= cap or alone
