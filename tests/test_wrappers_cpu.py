@@ -219,3 +219,41 @@ def test_shard_home_lays_units_out_in_slabs(seed, monkeypatch):
         for slab in home.slabs:
             alone = any(max(-(-s // 4) * 4 for s in sizes) >= slab.numel() for sizes in units)
             assert slab.numel() <= cap or alone
+
+
+class _ArenaGroup(_Arenas):
+    def broadcast(self, t, root=0, async_op=False):
+        return t
+
+    def pack(self, flat, pieces):
+        for at, t in pieces:
+            flat[at:at + t.numel()] = t.reshape(-1)
+
+
+@pytest.mark.parametrize("slab_bytes", [2048, 8192, 1 << 30])
+def test_ddp_carves_its_buckets_from_slabs(slab_bytes, monkeypatch):
+    """DDP(direct=True): every bucket lies inside one arena, buckets do not overlap, and a rebuild in another order
+    carves the slabs that are there again instead of asking for more."""
+    monkeypatch.setattr(DDP, "SLAB_BYTES", slab_bytes)
+    torch.manual_seed(0)
+    model = torch.nn.Sequential(*[torch.nn.Linear(17, 17) for _ in range(6)], torch.nn.Linear(17, 3))
+    g = _ArenaGroup(0, 2)
+    z = DDP(model, g, bucket_bytes=1024, direct=True)
+
+    def check():
+        spans = []
+        for b in z.buckets:
+            off = g.arena_offset(b.flat)
+            assert off is not None and off % 256 == 0
+            spans.append((off, off + 4 * b.flat.numel()))
+            assert sum(p.numel() for p in b.params) == b.flat.numel()
+        spans.sort()
+        assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
+        assert sorted(id(p) for b in z.buckets for p in b.params) == sorted(id(p) for p in z.params)
+
+    check()
+    arenas = len(g.arenas)
+    assert arenas >= (3 if slab_bytes == 2048 else 1)
+    z._build(list(z.params))  # the order in which the gradients turned out to arrive
+    check()
+    assert len(g.arenas) <= arenas + 1
