@@ -350,6 +350,17 @@ def zero2_step(dev, reps):
     out = {"workload": "85,842,432 fp32 params, world 4 on one GPU, 16 buckets of <= 25 MiB, AdamW(3e-4, (0.9, 0.95), 1e-8, 0.1) on all 4 shards"}
     shard = z.layouts[0].hi - z.layouts[0].lo
     opt = timed(lambda: [z.opts[r].update("bench", z.bufs[r][z.layouts[r].lo:z.layouts[r].hi], z.grad_shards[r]) for r in range(WORLD)], reps)
+    # the same four updates on shards that start 4 bytes off a 16-byte boundary, as tensor_split shards may (p, g, m, v at one phase)
+    from tandem_amd.optim import ShardedAdamW
+
+    off_opt = ShardedAdamW(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    off_p = [torch.zeros(shard + 4, device=dev)[1:1 + shard].normal_(0.0, 0.02, generator=gen) for _ in range(WORLD)]
+    off_g = [torch.zeros(shard + 4, device=dev)[1:1 + shard].normal_(0.0, 1e-3, generator=gen) for _ in range(WORLD)]
+    assert all(t.data_ptr() % 16 == 4 for t in off_p + off_g)
+    opt_off = timed(lambda: [off_opt.update(r, off_p[r], off_g[r]) for r in range(WORLD)], reps)
+    out["adamw_4_shards_off_grid_ms"] = round(opt_off * 1e3, 4)
+    out["adamw_off_grid_over_aligned"] = round(opt_off / opt, 4)
+    del off_p, off_g, off_opt
     # the all-gather of the flat parameter buffers in both of the library's forms, each on the bytes that form moves
     check(lib().tdm_set_ring_form(1))
     ag_one = timed(lambda: z.lw.all_gather(z.bufs, z.layouts[0].sizes), reps)

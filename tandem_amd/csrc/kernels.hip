@@ -1037,24 +1037,31 @@ void adamw_launch(float* p, const float* g, float* m, float* v, int64_t n, const
   if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
   uintptr_t ptrs[4 + TDM_MAX_WORLD - 1] = {reinterpret_cast<uintptr_t>(p), reinterpret_cast<uintptr_t>(g),
                                            reinterpret_cast<uintptr_t>(m), reinterpret_cast<uintptr_t>(v)};
-  AdamwArgs a{p, g, m, v, n, *s, ncopies, xcd_shift(TDM_XCD_ADAMW, 1, true), {}};
+  AdamwArgs a{p, g, m, v, n, *s, ncopies, xcd_shift(TDM_XCD_ADAMW, 1, true), 0, {}};
   for (int c = 0; c < ncopies; ++c) {
     if (!copies[c]) throw Invalid("NULL copy of the parameters");
     a.copy[c] = copies[c];
     ptrs[4 + c] = reinterpret_cast<uintptr_t>(copies[c]);
   }
-  bool vec = true;
-  for (int i = 0; i < 4 + ncopies; ++i) {
+  for (int i = 0; i < 4 + ncopies; ++i)
     if (ptrs[i] % 4) throw Invalid("pointer not aligned to 4 bytes");
-    vec = vec && ptrs[i] % 16 == 0;
-  }
   for (int i = 0; i < 4 + ncopies; ++i)
     for (int j = i + 1; j < 4 + ncopies; ++j) {
       const uintptr_t bytes = static_cast<uintptr_t>(n) * 4;
       if (ptrs[i] < ptrs[j] + bytes && ptrs[j] < ptrs[i] + bytes) throw Invalid("p, g, m, v and the copies must not overlap");
     }
+  // A shard cut out of a flat buffer starts anywhere (tensor_split). When all the streams start at the same distance
+  // from a 16-byte boundary, the few elements before it are peeled off and the rest runs on vectors.
+  const SegPlan plan = plan_segment(ptrs, 4 + ncopies, n, 4, static_cast<int64_t>(kAdamwThreads) * kAdamwUnroll * 4);
+  const bool vec = plan.vec;
+  if (vec && plan.head) {
+    a.p += plan.head, a.g += plan.head, a.m += plan.head, a.v += plan.head;
+    for (int c = 0; c < ncopies; ++c) a.copy[c] += plan.head;
+    a.n = plan.body;
+    a.head = plan.head;
+  }
   const dim3 block(kAdamwThreads);
-  const int64_t tiles = vec ? (n / 4 + kAdamwThreads * kAdamwUnroll - 1) / (kAdamwThreads * kAdamwUnroll) : (n + kAdamwThreads - 1) / kAdamwThreads;
+  const int64_t tiles = vec ? (a.n / 4 + kAdamwThreads * kAdamwUnroll - 1) / (kAdamwThreads * kAdamwUnroll) : (n + kAdamwThreads - 1) / kAdamwThreads;
   const dim3 grid(grid_for(std::max<int64_t>(tiles, 1)));
   const int which = (order == TDM_ADAMW_HOST_ORDER ? 0 : 4) + (vec ? 2 : 0) + (ncopies > 0 ? 1 : 0);
   const unsigned pad = occupancy_pad(TDM_XCD_ADAMW);

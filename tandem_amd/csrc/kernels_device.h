@@ -695,6 +695,7 @@ struct AdamwArgs {
   // update and the all-gather of the result in one pass.
   int ncopies;
   int shift;  // of tile_of()
+  int head;   // vector path: elements (fewer than a vector) that lie before the pointers, peeled off an unaligned shard
   float* copy[TDM_MAX_WORLD - 1];
 };
 
@@ -766,8 +767,9 @@ __global__ __launch_bounds__(kAdamwThreads) void k3_adamw_kernel(AdamwArgs a) {
         }
       }
     }
-    if (blockIdx.x == 0 && threadIdx.x < a.n - nv * 4) {
-      const int64_t i = nv * 4 + threadIdx.x;
+    // the last few elements (lanes 0..), and the head before the first vector (lanes 32..): fewer than a vector each
+    if (blockIdx.x == 0 && (threadIdx.x < a.n - nv * 4 || (threadIdx.x >= 32 && static_cast<int>(threadIdx.x) - 32 < a.head))) {
+      const int64_t i = threadIdx.x < 32 ? nv * 4 + threadIdx.x : -1 - (static_cast<int64_t>(threadIdx.x) - 32);
       adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
       if constexpr (kCopies)
         for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];

@@ -246,7 +246,7 @@ class LocalZeRO2:
 
     def __init__(self, world, numels, device, bucket_bytes=25 << 20, order="host", **adamw):
         from .buckets import FlatLayout, zero_buckets
-        from .optim import ShardedAdamW
+        from .optim import ShardedAdamW, zeros_at_phase_of
 
         self.lw = LocalWorld(world)
         self.world = world
@@ -256,7 +256,8 @@ class LocalZeRO2:
         self.buckets = zero_buckets(list(numels), 4, bucket_bytes)
         self.bufs = [torch.zeros(n, device=device) for _ in range(world)]
         self.staging = [torch.zeros(n, device=device) for _ in range(world)]
-        self.grad_shards = [torch.zeros(l.hi - l.lo, device=device) for l in self.layouts]
+        # every shard's gradient (and, below, its optimizer state) at the phase of the parameter shard it belongs to
+        self.grad_shards = [zeros_at_phase_of(self.bufs[r][l.lo:l.hi]) for r, l in enumerate(self.layouts)]
         self.opts = [ShardedAdamW(order=order, **adamw) for _ in range(world)]
         self.device = torch.device(device)
         # ring step s of every bucket: (dst, src, count) pairs, and the final adds
@@ -286,7 +287,7 @@ class LocalZeRO2:
         self._step_table = None
         if world <= _lib.TDM_MAX_WORLD:
             for r in range(world):
-                self.opts[r].state["flat"] = [0.0, torch.zeros_like(self.grad_shards[r]), torch.zeros_like(self.grad_shards[r])]
+                self.opts[r].state["flat"] = [0.0, zeros_at_phase_of(self.grad_shards[r]), zeros_at_phase_of(self.grad_shards[r])]
             segs = (_lib.StepSeg * max(1, len(rows)))()
             bb = [t.data_ptr() for t in self.bufs]
             for k, (srcs, _dsts, m, c) in enumerate(rows):

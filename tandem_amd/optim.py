@@ -34,6 +34,21 @@ def step_scalars(step, lr, betas, eps, weight_decay):
     return s
 
 
+def zeros_at_phase_of(like, numel=None):
+    """A zeroed tensor of `numel` elements (default: as many as `like`) in `like`'s memory
+    that starts at the same distance from a 16-byte boundary as `like` does. A shard cut
+    out of a flat buffer by tensor_split starts anywhere; the kernels run on 16-byte
+    vectors when all of their streams share that distance (the few elements before the
+    boundary are peeled off), so a shard's gradient and optimizer state are laid out at
+    the shard's own phase."""
+    n = like.numel() if numel is None else int(numel)
+    es = like.element_size()
+    lead = (like.data_ptr() % 16) // es
+    store = torch.zeros(n + 16 // es, device=like.device, dtype=like.dtype)
+    lead = (lead - (store.data_ptr() % 16) // es) % (16 // es)
+    return store[lead:lead + n]
+
+
 class ShardedAdamW:
     """order="host" reproduces torch's CPU addcdiv_ (p + (step*m)/d), which is
     what the reference's CPU engine computes; order="device" reproduces torch's
@@ -65,7 +80,7 @@ class ShardedAdamW:
         if param.shape != grad.shape:
             raise ValueError("param and grad differ in shape")
         if key not in self.state:
-            self.state[key] = [0.0, torch.zeros_like(param), torch.zeros_like(param)]
+            self.state[key] = [0.0, zeros_at_phase_of(param), zeros_at_phase_of(param)]
         st = self.state[key]
         st[0] += 1.0
         step, exp_avg, exp_avg_sq = st
@@ -91,7 +106,7 @@ class ShardedAdamW:
         if param.dtype != torch.float32:
             raise ValueError("ShardedAdamW handles fp32 shards")
         if key not in self.state:
-            self.state[key] = [0.0, torch.zeros_like(param), torch.zeros_like(param)]
+            self.state[key] = [0.0, zeros_at_phase_of(param), zeros_at_phase_of(param)]
         st = self.state[key]
         st[0] += 1.0
         return step_scalars(st[0], self.lr, self.betas, self.eps, self.weight_decay), st[1], st[2], self.order

@@ -24,7 +24,7 @@ import torch
 from torch.autograd import Variable
 
 from .buckets import FlatLayout, zero_buckets
-from .optim import ShardedAdamW
+from .optim import ShardedAdamW, zeros_at_phase_of
 
 
 def _need(group, *names):
@@ -106,7 +106,8 @@ class ZeRO(torch.nn.Module):
         if stage == 1:
             self.grad = self._pool if self.direct else torch.zeros_like(self.buf)
         else:
-            self.grad_shard = torch.zeros(self.flat.hi - self.flat.lo, device=dev, dtype=dtype)
+            # at the phase of this rank's parameter shard (tensor_split shards start anywhere): the update runs on vectors
+            self.grad_shard = zeros_at_phase_of(self.buf[self.flat.lo:self.flat.hi])
         # Buckets are contiguous ranges of the flat buffer taken from its end: the
         # order backward produces gradients in.
         self.buckets, self.bucket_of = [], {}

@@ -137,6 +137,84 @@ def test_adamw_writing_further_copies(dev):
         fused.update("k", q, gr, [torch.zeros(n, device=dev) for _ in range(8)])
 
 
+@pytest.mark.parametrize("order", ["host", "device"])
+def test_adamw_on_a_shard_off_the_16_byte_grid(dev, order):
+    """tensor_split shards start anywhere. With p, g, m, v (and the copies) all at the
+    same distance from a 16-byte boundary the launcher peels that head and runs vectors;
+    with streams that disagree it goes element by element. Both against the plain aligned
+    update on the same numbers, which the tests above pin to the oracle and to torch:
+    every phase 1..3, lengths that leave a head, a tail, both, fewer elements than the
+    head, with and without copies; guard elements around every stream stay untouched."""
+    import ctypes
+
+    from tandem_amd import _lib
+    from tandem_amd._lib import check, lib, stream_ptr
+    from tandem_amd.optim import step_scalars
+
+    kw = dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    code = _lib.ADAMW_HOST_ORDER if order == "host" else _lib.ADAMW_DEVICE_ORDER
+    gen = torch.Generator().manual_seed(12)
+    st = stream_ptr(dev)
+
+    def run(n, phases, ncopies):
+        """Three steps over streams laid at the given phases (elements off a 16-byte boundary) inside guarded stores."""
+        pad = 8
+        stores = [torch.full((n + 2 * pad,), -7.0, device=dev) for _ in range(4 + ncopies)]
+        views = [s_[pad + ph:pad + ph + n] for s_, ph in zip(stores, phases)]
+        for v_ in views:
+            assert v_.data_ptr() % 16 == 4 * (phases[views.index(v_)] % 4)
+        views[0].copy_(p0[:n])
+        views[2].zero_()
+        views[3].zero_()
+        for step in range(3):
+            views[1].copy_(grads[step][:n])
+            s_ = step_scalars(step + 1.0, kw["lr"], kw["betas"], kw["eps"], kw["weight_decay"])
+            ptr = [ctypes.c_void_p(v_.data_ptr()) for v_ in views]
+            if ncopies:
+                arr = (ctypes.c_void_p * ncopies)(*[v_.data_ptr() for v_ in views[4:]])
+                check(lib().tdm_k3_adamw_gather(ptr[0], ptr[1], ptr[2], ptr[3], n, ctypes.byref(s_), code, arr, ncopies, st))
+            else:
+                check(lib().tdm_k3_adamw(ptr[0], ptr[1], ptr[2], ptr[3], n, ctypes.byref(s_), code, st))
+        for s_, ph in zip(stores, phases):  # nothing outside the streams was written
+            assert float((s_[:pad + ph] + 7.0).abs().sum()) == 0 and float((s_[pad + ph + n:] + 7.0).abs().sum()) == 0
+        return [v_.clone() for v_ in views]
+
+    for n in (1, 2, 3, 5, 127, 4099, 100_003):
+        p0 = torch.randn(n, generator=gen).to(dev) * 0.02
+        grads = [(torch.randn(n, generator=gen) * 1e-3).to(dev) for _ in range(3)]
+        for ncopies in (0, 2):
+            want = run(n, [0] * (4 + ncopies), ncopies)
+            for ph in (1, 2, 3):
+                got = run(n, [ph] * (4 + ncopies), ncopies)  # one phase for all: head peeled, vectors
+                for a, b in zip(want, got):
+                    assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (n, ph, ncopies, order)
+            got = run(n, [1, 0, 3, 2, 1, 2][:4 + ncopies], ncopies)  # phases that disagree: element by element
+            for a, b in zip(want, got):
+                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (n, "mixed", ncopies, order)
+
+
+def test_optimizer_state_follows_the_shards_phase(dev):
+    """ShardedAdamW lays a shard's exp_avg and exp_avg_sq out at the shard's own distance from
+    a 16-byte boundary, and ZeRO's gradient shard likewise, so that the update of a
+    tensor_split shard that starts anywhere still runs on vectors."""
+    from tandem_amd import ShardedAdamW
+    from tandem_amd.optim import zeros_at_phase_of
+
+    flat = torch.zeros(1000, device=dev)
+    opt = ShardedAdamW()
+    for lo in (0, 1, 2, 3, 5):
+        p = flat[lo:lo + 333]
+        g = zeros_at_phase_of(p)
+        assert g.numel() == 333 and g.data_ptr() % 16 == p.data_ptr() % 16 and float(g.abs().sum()) == 0
+        opt.update(lo, p, g)
+        _, m, v = opt.state[lo]
+        assert m.data_ptr() % 16 == v.data_ptr() % 16 == p.data_ptr() % 16
+        assert m.numel() == v.numel() == 333
+    assert opt.state_bytes() == 5 * 2 * 4 * 333
+    half = torch.zeros(64, device=dev, dtype=torch.float16)[3:40]
+    assert zeros_at_phase_of(half).data_ptr() % 16 == half.data_ptr() % 16 and zeros_at_phase_of(half, 5).numel() == 5
+
+
 def test_adamw_rejects_what_it_cannot_do(dev):
     from tandem_amd import ShardedAdamW
 

@@ -77,11 +77,53 @@ def test_small_model_bit_exact_with_oracle(world, algorithm):
         assert np.array_equal(bits(z.opts[r].state["flat"][2].cpu().numpy()), bits(opts[r].state["flat"][2]))
 
 
+@pytest.mark.parametrize("algorithm", ["fold", "ring", "fused"])
+def test_shards_that_start_off_the_16_byte_grid(algorithm):
+    """World 3 over a flat buffer of odd length: tensor_split puts the second and third shard
+    1 and 2 elements past a multiple of four (tandem/zero.py:29-54 there: shards start
+    anywhere). Gradient shards and optimizer state sit at their shard's phase, so every
+    launch peels a head and runs on vectors; five steps against the oracle, bit for bit."""
+    from tandem_amd.local import LocalZeRO2
+
+    dev = torch.device("cuda", 0)
+    world, numels = 3, [4099, 10_007, 33, 5001, 1, 12_288, 782]
+    n = sum(numels)
+    z = LocalZeRO2(world, numels, dev, bucket_bytes=16 << 10, **KW)
+    assert sorted(l.lo % 4 for l in z.layouts) == [0, 1, 2], [l.lo for l in z.layouts]
+    for r, l in enumerate(z.layouts):  # the layout this test is about
+        phase = z.bufs[r][l.lo:l.hi].data_ptr() % 16
+        assert phase == 4 * (l.lo % 4)
+        assert z.grad_shards[r].data_ptr() % 16 == phase
+        assert z.opts[r].state["flat"][1].data_ptr() % 16 == z.opts[r].state["flat"][2].data_ptr() % 16 == phase
+    p0 = (seeded(2, 0, n) * 0.02).numpy()
+    steps = 5
+    grads = [[(seeded(20 + s, r, n) * 1e-3).numpy() for r in range(world)] for s in range(steps)]
+    for b in z.bufs:
+        b.copy_(torch.from_numpy(p0))
+    for s in range(steps):
+        for r in range(world):
+            z.staging[r].copy_(torch.from_numpy(grads[s][r]))
+        if algorithm == "fused":
+            assert z._step_table is not None and z._shards_zero
+            z.reduce_and_step()
+        else:
+            z.reduce_grads(algorithm)
+            z.step(fused_gather=algorithm == "fold")
+        z.zero_grad()
+    want, opts = oracle_zero2(world, numels, 16 << 10, p0, grads)
+    for r in range(world):
+        assert np.array_equal(bits(z.bufs[r].cpu().numpy()), bits(want[r])), r
+        assert np.array_equal(bits(z.opts[r].state["flat"][1].cpu().numpy()), bits(opts[r].state["flat"][1]))
+        assert np.array_equal(bits(z.opts[r].state["flat"][2].cpu().numpy()), bits(opts[r].state["flat"][2]))
+
+
 def test_full_size_step():
     """85,842,432 parameters, world 4, 25 MiB buckets, the reference's bucket_sizes
-    (plans.json). Properties: every rank ends with the same parameters; each rank's
-    shard equals a sampled oracle evaluation; the step matches torch.optim.AdamW on
-    the GPU when run in torch's GPU op order."""
+    (plans.json), one step. The ring's steps and the fold leave the same gradient
+    shards; the averaged gradient equals the oracle's ring-order fold on a sample of
+    every fifth bucket's chunks; every rank ends with the same parameters; one whole
+    shard equals the oracle's AdamW. (The twenty steps of the configuration, against
+    torch.optim.AdamW and the oracle, are test_config_4_twenty_steps below.)"""
     from oracle import ring
     from oracle.adamw import AdamW
     from tandem_amd.local import LocalZeRO2
@@ -134,6 +176,88 @@ def test_full_size_step():
     pn = p0[lay[r].lo:lay[r].hi].cpu().numpy().copy()
     AdamW(**KW).update("k", pn, shards_before[r].cpu().numpy())
     assert np.array_equal(bits(z.bufs[0][lay[r].lo:lay[r].hi].cpu().numpy()), bits(pn))
+
+
+def test_config_4_twenty_steps():
+    """The configuration as stated: the 85,842,432-parameter GPT, world 4 on one GPU,
+    16 buckets of up to 25 MiB, reduce-scatter into 21,460,608-element shards, AdamW
+    (lr 3e-4, betas 0.9/0.95, eps 1e-8, wd 0.1) for TWENTY steps with fresh seeded
+    gradients each step, all-gather; as the reference checks its ZeRO against torch's
+    AdamW end to end (tests/test_zero.py:46-66 there). Both forms of the step run side
+    by side, reduce_grads() + step() and reduce_and_step() (one launch), in both
+    operation orders. One whole shard is followed on the side, fed every step with the
+    oracle's ring-order fold of that step's four gradients (which the kernels' own
+    gradient shard must equal bit for bit):
+      order="device": torch.optim.AdamW([shard], foreach=False, fused=False) on the GPU;
+                      parameters and both moments bit for bit;
+      order="host":   the oracle's AdamW (the reference's operation order on the CPU);
+                      parameters and both moments bit for bit.
+    After step 20 every rank holds the same buffer in every run, and the one-launch form
+    equals the two-kernel form in every buffer and both moments of every rank."""
+    from oracle import ring
+    from oracle.adamw import AdamW
+    from tandem_amd.local import LocalZeRO2
+
+    dev = torch.device("cuda", 0)
+    plan = golden_json("plans.json")
+    numels = [math.prod(s) for _, s in plan["medium_params"]]
+    world, n, steps, watched = 4, sum(numels), 20, 2
+    assert n == 85_842_432
+    runs = {(order, form): LocalZeRO2(world, numels, dev, order=order, **KW)
+            for order in ("device", "host") for form in ("two_kernels", "one_launch")}
+    lay = runs["host", "two_kernels"].layouts
+    lo, hi = lay[watched].lo, lay[watched].hi
+    assert hi - lo == 21_460_608 and len(runs["host", "two_kernels"].buckets) == 16
+    p0 = torch.randn(n, device=dev, generator=torch.Generator(device=dev).manual_seed(4)) * 0.02
+    for z in runs.values():
+        for b in z.bufs:
+            b.copy_(p0)
+    torch_p = torch.nn.Parameter(p0[lo:hi].clone())
+    torch_opt = torch.optim.AdamW([torch_p], foreach=False, fused=False, **KW)
+    oracle_p = p0[lo:hi].cpu().numpy().copy()
+    oracle_opt = AdamW(**KW)
+    del p0
+    for step in range(steps):
+        shard_grads = []
+        for r in range(world):
+            g = torch.randn(n, device=dev, generator=torch.Generator(device=dev).manual_seed(1000 * step + r)) * 1e-3
+            for z in runs.values():
+                z.staging[r].copy_(g)
+            shard_grads.append(g[lo:hi].cpu().numpy())
+        del g
+        # the watched shard's gradient as the reference leaves it: the ring's order for chunk `watched`, added into a zeroed shard
+        mine = np.float32(0.0) + ring.fold(shard_grads, watched, 0, hi - lo, True)
+        for (order, form), z in runs.items():
+            if form == "one_launch":
+                assert z._step_table is not None and z._shards_zero
+                z.reduce_and_step()
+            else:
+                z.reduce_grads()
+                assert np.array_equal(bits(z.grad_shards[watched].cpu().numpy()), bits(mine)), (step, order)
+                z.step()
+            z.zero_grad()
+        torch_p.grad = torch.from_numpy(mine).to(dev)
+        torch_opt.step()
+        oracle_opt.update("k", oracle_p, mine)
+    want = {"device": (torch_p.detach().cpu().numpy(), torch_opt.state[torch_p]["exp_avg"].cpu().numpy(),
+                       torch_opt.state[torch_p]["exp_avg_sq"].cpu().numpy()),
+            "host": (oracle_p, oracle_opt.state["k"][1], oracle_opt.state["k"][2])}
+    assert not np.array_equal(bits(want["device"][0]), bits(want["host"][0]))  # the two orders do differ over twenty steps
+    for (order, form), z in runs.items():
+        what = (order, form)
+        assert z.opts[watched].state["flat"][0] == float(steps), what
+        for r in range(1, world):
+            assert torch.equal(z.bufs[0].view(torch.int32), z.bufs[r].view(torch.int32)), what + (r,)
+        p, m, v = want[order]
+        assert np.array_equal(bits(z.bufs[0][lo:hi].cpu().numpy()), bits(p)), what
+        assert np.array_equal(bits(z.opts[watched].state["flat"][1].cpu().numpy()), bits(m)), what
+        assert np.array_equal(bits(z.opts[watched].state["flat"][2].cpu().numpy()), bits(v)), what
+    for order in ("device", "host"):
+        a, b = runs[order, "two_kernels"], runs[order, "one_launch"]
+        assert torch.equal(a.bufs[0].view(torch.int32), b.bufs[0].view(torch.int32)), order
+        for r in range(world):
+            for i in (1, 2):
+                assert torch.equal(a.opts[r].state["flat"][i].view(torch.int32), b.opts[r].state["flat"][i].view(torch.int32)), (order, r, i)
 
 
 def test_full_size_step_in_one_launch():
