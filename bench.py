@@ -226,7 +226,7 @@ MIXES = {"k1_reduce": (2, 1), "ring_copy": (1, 1), "bucket_fold_w2": (2, 2), "ze
 
 def stream_mix(dev, reps):
     """What the memory system gives a kernel that only streams: for every kernel's mix of
-    read and written streams, the library's probe (no table, no arithmetic, the kernels'
+    read and written streams, the probe library's kernel (no table, no arithmetic, the kernels'
     own launch geometry) over cold buffers of 85,842,432 fp32 each, best of a few launch
     geometries. The fused kernels are reported against these figures as well as against
     the 8 TB/s peak: a stream mix with many written streams does not reach the peak
@@ -235,7 +235,8 @@ def stream_mix(dev, reps):
 
     import torch
 
-    from tandem_amd._lib import check, lib, stream_ptr
+    from tandem_amd._lib import stream_ptr
+    from tandem_amd._probe import check, lib  # libtandem_probe.so: a library of its own, not part of the plug-in
 
     n = 85_842_432
     whole = torch.empty(13 * n, device=dev).normal_()  # one allocation: the streams lie back to back

@@ -98,16 +98,6 @@ int tdm_set_occupancy_pad(int kind, int bytes);
  * kernels' own function, evaluated on the host: for tests of the mapping). -1 for arguments out of range. */
 int64_t tdm_tile_of(int64_t index, int64_t total, int shift);
 
-/* Measurement only; the reference has no counterpart. Reads `bytes` (a multiple of 16) from each of
- * `nreads` device buffers and writes as many to each of `nwrites` others (0..8 each), in the launch
- * geometry of the streaming kernels (workgroups of 128 lanes, `vectors_per_lane` = 1 or 2 16-byte
- * vectors per lane and stream, one tile per workgroup, tile order tdm_tile_of(.., xcd_shift),
- * `occupancy_pad` bytes of unused LDS per workgroup, non-temporal accesses), without a table and
- * without arithmetic: what the memory system gives a kernel with that mix of streams. The written
- * values are meaningless. */
-int tdm_probe_stream_mix(const void* const* reads, int nreads, void* const* writes, int nwrites, int64_t bytes,
-                         int vectors_per_lane, int xcd_shift, int occupancy_pad, tdm_stream stream);
-
 /* Bytes of every stream that one record of the K2 and K2+K3 device tables covers (a build constant). */
 int tdm_table_tile_bytes(void);
 

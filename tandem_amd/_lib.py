@@ -59,8 +59,6 @@ _SIGNATURES = {
     "tdm_set_xcd_group": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     "tdm_set_occupancy_pad": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     "tdm_set_ring_form": (ctypes.c_int, [ctypes.c_int]),
-    "tdm_probe_stream_mix": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.c_int, ctypes.POINTER(ctypes.c_void_p), ctypes.c_int,
-                                            ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "tdm_tile_of": (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]),
     "tdm_table_tile_bytes": (ctypes.c_int, []),
     "tdm_build_geometry": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)]),

@@ -1,5 +1,7 @@
 """Builds libtandem_hip.so (the C-ABI library declared in include/tandem_hip.h)
-in-tree with hipcc for gfx950. Cross-compiles without a GPU.
+in-tree with hipcc for gfx950, and beside it libtandem_probe.so (include/tandem_probe.h:
+the stream-mix measurement kernel that the benchmark and the GPU tests load, kept out of
+the plug-in). Cross-compiles without a GPU.
 
     python -m tandem_amd.build [extra hipcc flags, e.g. -DTDM_NT_MASK=7] [--out=path/to/variant.so]
 
@@ -14,7 +16,9 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(CSRC, "libtandem_hip.so")
-SOURCES = ["kernels.hip", "kernels_chain.hip", "probe.hip", "abi.hip", "engine.hip", "engine_abi.hip"]
+SOURCES = ["kernels.hip", "kernels_chain.hip", "abi.hip", "engine.hip", "engine_abi.hip"]
+PROBE_LIB = os.path.join(CSRC, "libtandem_probe.so")
+PROBE_SOURCES = ["probe.hip"]
 
 # -ffp-contract=off: no multiply-add is fused unless the source says fma.
 # -fhip-fp32-correctly-rounded-divide-sqrt: IEEE division and sqrt (the default; stated).
@@ -37,10 +41,10 @@ def _run(cmd, verbose):
         print(out)
 
 
-def build(verbose=False, extra=(), out=LIB):
+def build(verbose=False, extra=(), out=LIB, sources=None):
     """Compiles every source (always: nothing is reused from an earlier build) and links `out`."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    srcs = list(SOURCES if sources is None else sources)
     objdir = os.path.join(CSRC, "_obj", os.path.splitext(os.path.basename(out))[0])
     os.makedirs(objdir, exist_ok=True)
     objs = [os.path.join(objdir, os.path.splitext(s)[0] + ".o") for s in srcs]
@@ -51,6 +55,11 @@ def build(verbose=False, extra=(), out=LIB):
     return out
 
 
+def build_probe(verbose=False, extra=(), out=PROBE_LIB):
+    """The measurement library, from the same device headers and with the same flags as the plug-in."""
+    return build(verbose, extra, out, PROBE_SOURCES)
+
+
 if __name__ == "__main__":
     args = sys.argv[1:]
     target = LIB
@@ -59,3 +68,5 @@ if __name__ == "__main__":
             target = os.path.abspath(a[len("--out="):])
             args.remove(a)
     print(build(verbose=True, extra=args, out=target))
+    if target == LIB:
+        print(build_probe(verbose=True, extra=args))

@@ -1,3 +1,4 @@
+// libtandem_probe.so (include/tandem_probe.h): a library of its own, not linked into the plug-in.
 // A measurement kernel, not part of the reduction path: R streams read and W streams written in
 // the geometry the streaming kernels use (workgroups of 128 lanes, 16-byte vectors, one tile per
 // workgroup, the tile order of tile_of(), non-temporal loads and stores), with no table and no
@@ -10,12 +11,19 @@
 #include <cstdint>
 #include <string>
 
-#include "../../include/tandem_hip.h"
+#include "../../include/tandem_probe.h"
 #include "common.h"
 
 #include "kernels_device.h"
 
 namespace tandem_hip {
+
+namespace {
+thread_local std::string probe_error;
+}
+
+// common.h's guard() reports through this; the plug-in has its own in abi.hip
+void set_last_error(const std::string& message) { probe_error = message; }
 
 namespace {
 
@@ -91,8 +99,12 @@ void launch_w(const MixArgs& a, int nwrites, int per_lane, dim3 grid, unsigned p
 
 using namespace tandem_hip;
 
-extern "C" int tdm_probe_stream_mix(const void* const* reads, int nreads, void* const* writes, int nwrites, int64_t bytes,
-                                    int vectors_per_lane, int xcd_shift, int occupancy_pad, tdm_stream stream) {
+#define PROBE_EXPORT extern "C" __attribute__((visibility("default")))
+
+PROBE_EXPORT const char* tdm_probe_last_error(void) { return probe_error.c_str(); }
+
+PROBE_EXPORT int tdm_probe_stream_mix(const void* const* reads, int nreads, void* const* writes, int nwrites, int64_t bytes,
+                                      int vectors_per_lane, int xcd_shift, int occupancy_pad, void* stream) {
   return guard([&] {
     if (nreads < 0 || nreads > TDM_MAX_WORLD || nwrites < 0 || nwrites > TDM_MAX_WORLD || nreads + nwrites == 0) {
       throw Invalid("the probe takes 0..8 streams to read and 0..8 to write, at least one in all");

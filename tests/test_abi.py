@@ -61,10 +61,31 @@ def test_argument_errors_need_no_gpu():
     assert (a.value, b.value, c.value) == (4096, 128, 4096) and c.value == L.tdm_table_tile_bytes()
     assert L.tdm_build_geometry(None, ctypes.byref(b), ctypes.byref(c)) == 1
     assert L.tdm_k2_static_max_tiles() == 16384
-    # the static bucket fold and the probe check their arguments before they touch the GPU
+    # the static bucket fold checks its arguments before it touches the GPU
     assert L.tdm_k2_bucket_fold_static(segs, 2, 2, 99, 1, 0, None) == 1 and b"dtype" in L.tdm_last_error()
     assert L.tdm_k2_bucket_fold_static(segs, 2, 9, 0, 1, 0, None) == 1 and b"world" in L.tdm_last_error()
-    assert L.tdm_probe_stream_mix(None, 0, None, 0, 16, 1, 0, 0, None) == 1 and b"streams" in L.tdm_last_error()
+
+
+def test_the_measurement_probe_is_a_library_of_its_own():
+    """The stream-mix probe is not part of the plug-in: libtandem_hip.so does not export it, its header
+    does not declare it, and libtandem_probe.so exports what include/tandem_probe.h declares and
+    checks its arguments without a GPU."""
+    import subprocess
+
+    from tandem_amd import _lib, _probe
+
+    assert not hasattr(_lib.lib(), "tdm_probe_stream_mix")
+    assert not [n for n in declared_functions() if "probe" in n]
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "tandem_probe.h")).read(), flags=re.S)
+    declared = sorted(set(re.findall(r"\b(tdm_[a-z0-9_]+)\s*\(", text)))
+    assert declared == ["tdm_probe_last_error", "tdm_probe_stream_mix"]
+    P = _probe.lib()
+    assert P.tdm_probe_stream_mix(None, 0, None, 0, 16, 1, 0, 0, None) == 1 and b"streams" in P.tdm_probe_last_error()
+    out = subprocess.run(["nm", "-D", "--defined-only", _probe.PROBE_PATH], stdout=subprocess.PIPE, text=True, check=True).stdout
+    assert sorted(l.split()[-1] for l in out.splitlines() if l.split()[-1].startswith("tdm_")) == declared
+    res = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", "c",
+                          os.path.join(ROOT, "include", "tandem_probe.h")], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert res.returncode == 0, res.stdout
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
@@ -139,7 +160,8 @@ def test_the_product_stays_clear_of_the_checkers():
     from tandem_amd import build
 
     pkg = os.path.join(ROOT, "tandem_amd")
-    assert all(os.path.dirname(os.path.join(build.CSRC, s)) == build.CSRC for s in build.SOURCES)
+    assert all(os.path.dirname(os.path.join(build.CSRC, s)) == build.CSRC for s in build.SOURCES + build.PROBE_SOURCES)
+    assert "probe.hip" not in build.SOURCES
     for dirpath, _, names in os.walk(pkg):
         for name in names:
             if not name.endswith((".py", ".hip", ".h")):

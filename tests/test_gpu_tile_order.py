@@ -183,7 +183,8 @@ def test_stream_mix_probe_moves_what_it_says():
     are refused."""
     import ctypes
 
-    from tandem_amd._lib import lib, stream_ptr
+    from tandem_amd._lib import stream_ptr
+    from tandem_amd._probe import lib  # libtandem_probe.so, a library of its own beside the plug-in
 
     L = lib()
     dev = torch.device("cuda", 0)
@@ -209,7 +210,7 @@ def test_stream_mix_probe_moves_what_it_says():
     assert torch.equal(outs[(2, 3, 16384)][lane != 0], first[lane != 0])
     rd = (ctypes.c_void_p * 8)(src[0].data_ptr())
     assert L.tdm_probe_stream_mix(rd, 1, None, 0, n * 4, 1, 0, 0, stream_ptr(dev)) == 0  # read-only
-    assert L.tdm_probe_stream_mix(rd, 0, None, 0, n * 4, 1, 0, 0, stream_ptr(dev)) == 1
+    assert L.tdm_probe_stream_mix(rd, 0, None, 0, n * 4, 1, 0, 0, stream_ptr(dev)) == 1 and b"streams" in L.tdm_probe_last_error()
     assert L.tdm_probe_stream_mix(rd, 1, None, 0, n * 4 + 4, 1, 0, 0, stream_ptr(dev)) == 1
     assert L.tdm_probe_stream_mix(rd, 1, None, 0, n * 4, 3, 0, 0, stream_ptr(dev)) == 1
     assert L.tdm_probe_stream_mix(rd, 9, None, 0, n * 4, 1, 0, 0, stream_ptr(dev)) == 1
