@@ -29,6 +29,9 @@ typedef void* tdm_stream;
 
 /* The element types the reducing kernels know. Integer sums wrap around, as ATen's add_ does; 16-bit
  * floats are widened to fp32, added and rounded to nearest even once per add (tandem/csrc/reduce.cu:27-36).
+ * A NaN result of a 16-bit sum or average is the type's canonical quiet NaN (bf16 0x7fc0, f16 0x7e00): sign and
+ * payload of a NaN are not preserved, as they are not across torch builds either; elements that a collective
+ * only copies keep the bits they came with.
  * The reference's engine reduces any further ATen dtype by falling back to add_
  * (tandem/csrc/collectives.cpp:254-256); here every entry point that adds (tdm_k1_reduce_step, tdm_local_*,
  * tdm_k2_*, tdm_all_reduce, tdm_reduce_scatter, tdm_direct_*) refuses any other code with TDM_EINVAL

@@ -20,7 +20,10 @@
 #include <stdint.h>
 #include <string.h>
 
-/* ---- 16-bit floats as bit patterns: widen exactly, round to nearest even once */
+/* ---- 16-bit floats as bit patterns: widen exactly, round to nearest even once.
+ * A NaN narrows to the canonical quiet NaN of the type (bf16 0x7fc0, f16 0x7e00): sign and payload of a
+ * NaN are not kept. torch's own conversions do not agree on them from build to build (this container's CPU
+ * build narrows a float NaN to bf16 0xffff), so the reference's outputs pin no NaN bits, only where the NaNs are. */
 static float bf16_to_f32(uint16_t h) {
   uint32_t u = (uint32_t)h << 16;
   float f;
@@ -31,7 +34,7 @@ static float bf16_to_f32(uint16_t h) {
 static uint16_t f32_to_bf16(float f) {
   uint32_t u;
   memcpy(&u, &f, 4);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)0x7fc0u; /* the canonical quiet NaN */
   uint32_t lsb = (u >> 16) & 1u;
   u += 0x7fffu + lsb;
   return (uint16_t)(u >> 16);
@@ -66,7 +69,7 @@ static uint16_t f32_to_f16(float f) {
   memcpy(&u, &f, 4);
   uint32_t sign = (u >> 16) & 0x8000u;
   uint32_t a = u & 0x7fffffffu;
-  if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);
+  if (a > 0x7f800000u) return (uint16_t)0x7e00u; /* the canonical quiet NaN */
   if (a >= 0x47800000u) return (uint16_t)(sign | 0x7c00u); /* >= 65536: inf (65520 rounds up too, below) */
   if (a >= 0x38800000u) {                                  /* normal half */
     uint32_t m = a - 0x38000000u;                          /* rebias */

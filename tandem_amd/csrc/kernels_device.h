@@ -145,6 +145,7 @@ template <> struct Elem<f16_t> {
     _Float16 h = static_cast<_Float16>(x);  // round to nearest even, once
     f16_t out;
     __builtin_memcpy(&out.bits, &h, 2);
+    if (x != x) out.bits = 0x7e00u;  // a NaN narrows to the canonical quiet NaN: sign and payload are not kept
     return out;
   }
 };
@@ -156,7 +157,7 @@ template <> struct Elem<bf16_t> {
     uint32_t u = __float_as_uint(x);
     bf16_t out;
     if ((u & 0x7fffffffu) > 0x7f800000u) {
-      out.bits = 0x7fc0u;  // NaN
+      out.bits = 0x7fc0u;  // a NaN narrows to the canonical quiet NaN: sign and payload are not kept
     } else {
       u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
       out.bits = static_cast<uint16_t>(u >> 16);

@@ -235,6 +235,56 @@ def test_unaligned_views_and_special_values(dev):
                     assert float(store[r][:shifts[r]].abs().sum()) == 0 and float(store[r][shifts[r] + n:].abs().sum()) == 0
 
 
+@pytest.mark.parametrize("world", [2, 3, 4])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_nan_and_infinity_in_16_bit_collectives(dev, world, dtype):
+    """The stated policy: a NaN result of a 16-bit sum or average is the type's canonical quiet NaN
+    (bf16 0x7fc0, f16 0x7e00), whatever the sign and payload of the NaNs that went in; infinities keep
+    their sign, inf + -inf is that NaN. Inputs carry NaNs of both signs and several payloads and both
+    infinities at different places on different ranks. Every all-reduce result has passed through an
+    addition, so it is compared bit for bit with the oracle, NaNs included; a bare reduce_scatter leaves
+    chunks no arithmetic touched (their NaNs keep the bits they came with), so there the NaN positions
+    and all other bits are compared."""
+    from oracle import ring
+    from tandem_amd import LocalWorld
+
+    kind = KINDS[dtype]
+    canonical = 0x7fc0 if dtype == torch.bfloat16 else 0x7e00
+    inf = 0x7f80 if dtype == torch.bfloat16 else 0x7c00
+    nans = [canonical, canonical | 0x8000, inf | 1, inf | 0x8001, 0x7fff, 0xffff]
+    n = 3 * 2048 + 77
+    lw = LocalWorld(world)
+    xn = []
+    for r in range(world):
+        x = to_np(seeded(9, r, n).to(dtype)).copy()
+        for k, pattern in enumerate(nans):  # every NaN pattern on every rank, each at a place of its own
+            x[(7 * r + 13 * k) % n] = pattern
+            x[2048 + world * k + r] = pattern
+        x[100 + r] = inf                    # +inf on one rank only
+        x[200 + r] = inf | 0x8000           # -inf on one rank only
+        x[300] = inf if r % 2 == 0 else inf | 0x8000  # +inf and -inf meet: NaN
+        x[301] = inf                        # +inf on every rank: +inf
+        xn.append(x)
+    for op in ("sum", "avg"):
+        want = ring.expected_all_reduce(xn, op == "avg", kind)
+        is_nan = (want & 0x7fff) > inf
+        assert is_nan.sum() >= 2 * len(nans) and np.all(want[is_nan] == canonical)
+        assert is_nan[300] and want[301] == inf and not is_nan[100] and not is_nan[200]
+        for algorithm in ("ring", "fold"):
+            bufs = [from_np(x, dtype, dev) for x in xn]
+            lw.all_reduce(bufs, op=op, algorithm=algorithm)
+            for r in range(world):
+                assert np.array_equal(to_np(bufs[r]), want), (world, dtype, op, algorithm, r)
+        bufs = [from_np(x, dtype, dev) for x in xn]
+        lw.reduce_scatter(bufs, None, op=op)
+        wants = ring.expected_reduce_scatter(xn, None, op == "avg", kind)
+        for r in range(world):
+            got, w = to_np(bufs[r]), wants[r]
+            nan = (w & 0x7fff) > inf
+            assert np.array_equal((got & 0x7fff) > inf, nan), (world, dtype, op, r)
+            assert np.array_equal(got[~nan], w[~nan]), (world, dtype, op, r)
+
+
 @pytest.mark.parametrize("world", [2, 3])
 def test_two_byte_elements_off_the_vector_grid(dev, world):
     """bf16 views 1..7 elements past a 16-byte boundary, the same on every rank: up to seven head elements are

@@ -135,6 +135,25 @@ def test_16bit_conversions_match_numpy_and_torch():
     assert np.array_equal(got, want)
 
 
+def test_a_nan_narrows_to_the_canonical_quiet_nan():
+    """The stated policy for 16-bit results: every float NaN, whatever its sign and payload, narrows to
+    0x7fc0 (bf16) / 0x7e00 (f16); infinities keep their sign. torch marks the same positions as NaN but
+    its bits differ between builds, so only the positions are compared with it."""
+    import ctypes
+
+    from oracle import lib
+
+    nan_bits = np.array([0x7fc00000, 0xffc00000, 0x7f800001, 0xff800001, 0x7fffffff, 0xffffffff, 0x7fa00000, 0xffb12345], np.uint32)
+    f = np.ascontiguousarray(np.concatenate([nan_bits.view(np.float32), np.float32([np.inf, -np.inf, 1.0, -0.0])]))
+    got = np.empty(f.size, np.uint16)
+    lib().orc_f32_to_bf16(ctypes.c_void_p(f.ctypes.data), ctypes.c_void_p(got.ctypes.data), ctypes.c_int64(f.size))
+    assert list(got) == [0x7fc0] * 8 + [0x7f80, 0xff80, 0x3f80, 0x8000]
+    assert np.array_equal(torch.from_numpy(f).to(torch.bfloat16).isnan().numpy(), got == 0x7fc0)
+    lib().orc_f32_to_f16(ctypes.c_void_p(f.ctypes.data), ctypes.c_void_p(got.ctypes.data), ctypes.c_int64(f.size))
+    assert list(got) == [0x7e00] * 8 + [0x7c00, 0xfc00, 0x3c00, 0x8000]
+    assert np.array_equal(torch.from_numpy(f).to(torch.float16).isnan().numpy(), got == 0x7e00)
+
+
 def test_cpu_baseline_optimizer_is_the_same_update():
     """The torch-op optimizer that bench.py times as tandem's CPU backend gives the
     oracle's bits when the oracle uses torch's CPU sqrt: p, exp_avg, exp_avg_sq over
