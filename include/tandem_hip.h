@@ -219,8 +219,13 @@ int tdm_k2_bucket_fold(const void* table_dev, int64_t ntiles, int dtype, int wor
  * process ends; then the same fold kernel runs over it, on `stream`. Same arguments
  * otherwise, same bits. Segments that need more records are refused (TDM_EINVAL) before
  * anything is launched: split the call. The call allocates nothing on the device and makes no
- * host-to-device copy. All calls on one GPU share the array: calls on one stream are ordered
- * by it; calls that overlap on different streams (or threads) race and give wrong results. */
+ * host-to-device copy. All calls on one GPU share the array, and the library orders them: calls on
+ * one stream are ordered by the stream; a call on another stream than the one before it first makes
+ * its stream wait (on the GPU, hipStreamWaitEvent on an event created at set-up) for that call's
+ * fold; host threads take turns while they enqueue. Two such calls therefore never overlap on the
+ * GPU, whatever streams they are on. The one exception is a stream under capture, where neither the
+ * wait nor the event record is issued (they would become nodes of the caller's graph): replays of a
+ * graph that holds such a call, and any other call on the same GPU, must be ordered by the caller. */
 int64_t tdm_k2_static_max_tiles(void);
 int tdm_k2_bucket_fold_static(const tdm_fold_seg* segs, int nseg, int world, int dtype, int average, int accumulate,
                               tdm_stream stream);

@@ -948,22 +948,34 @@ int tdm_k2_bucket_fold(const void* table_dev, int64_t ntiles, int dtype, int wor
 // ---- the same fold for callers that cannot allocate: the table lives in a fixed device array
 namespace {
 // This GPU's copy of `scratch`, looked up once per device with that device current. The array's
-// name is only a host-side handle: everything below uses the address returned here.
-FoldSegDev* static_table() {
+// name is only a host-side handle: everything below uses the address kept here. With it, what orders
+// the calls that share the table: a mutex held while a call enqueues its launches, the stream of the
+// last call, and an event recorded behind that call's fold (created once, at the same set-up).
+struct StaticTable {
+  std::mutex mu;
+  FoldSegDev* table = nullptr;
+  hipEvent_t folded = nullptr;   // recorded after the last call's fold kernel
+  hipStream_t last = nullptr;    // the stream of that call
+  bool pending = false;          // `folded` has been recorded at least once
+};
+
+StaticTable* static_table() {
   constexpr int kMaxDevices = 64;
-  static std::mutex mu;
-  static FoldSegDev* table[kMaxDevices] = {nullptr};
+  static std::mutex setup;
+  static StaticTable per_device[kMaxDevices];
   int dev = 0;
   check_hip(hipGetDevice(&dev), "hipGetDevice");
   if (dev < 0 || dev >= kMaxDevices) throw std::runtime_error("device index beyond 63");
-  std::lock_guard<std::mutex> lock(mu);
-  if (table[dev] == nullptr) {
+  StaticTable& t = per_device[dev];
+  std::lock_guard<std::mutex> lock(setup);
+  if (t.table == nullptr) {
     void* p = nullptr;
     check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
     if (p == nullptr) throw std::runtime_error("hipGetSymbolAddress(scratch) returned NULL");
-    table[dev] = static_cast<FoldSegDev*>(p);
+    check_hip(hipEventCreateWithFlags(&t.folded, hipEventDisableTiming), "hipEventCreate");
+    t.table = static_cast<FoldSegDev*>(p);
   }
-  return table[dev];
+  return &t;
 }
 }  // namespace
 
@@ -990,8 +1002,17 @@ int tdm_k2_bucket_fold_static(const tdm_fold_seg* segs, int nseg, int world, int
       }
     }
     if (tiles == 0) return;
-    FoldSegDev* table = static_table();
     hipStream_t st = static_cast<hipStream_t>(stream);
+    StaticTable& shared = *static_table();
+    FoldSegDev* table = shared.table;
+    // One call at a time enqueues its launches, and a call on another stream than the last one first waits, on the
+    // GPU, for that call's fold: the records it is about to overwrite may still be in use there. A stream under
+    // capture takes no part in this (a wait or a record would become nodes of the caller's graph).
+    std::lock_guard<std::mutex> turn(shared.mu);
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    check_hip(hipStreamIsCapturing(st, &capture), "hipStreamIsCapturing");
+    const bool eager = capture == hipStreamCaptureStatusNone;
+    if (eager && shared.pending && shared.last != st) check_hip(hipStreamWaitEvent(st, shared.folded, 0), "hipStreamWaitEvent");
     FillBatch batch;
     std::memset(&batch, 0, sizeof batch);
     batch.world = world;
@@ -1024,6 +1045,11 @@ int tdm_k2_bucket_fold_static(const tdm_fold_seg* segs, int nseg, int world, int
     }
     flush();
     bucket_fold(table, tiles, dtype, world, average, accumulate, st);
+    if (eager) {
+      check_hip(hipEventRecord(shared.folded, st), "hipEventRecord");
+      shared.last = st;
+      shared.pending = true;
+    }
   });
 }
 

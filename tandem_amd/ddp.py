@@ -44,11 +44,15 @@ class Bucket:
 
 
 class DDP(torch.nn.Module):
-    def __init__(self, module, group, bucket_bytes=25 << 20, overlap=True, rebuild=True, direct=False, stream_ordered=True):
-        """stream_ordered: at the end of backward the training stream is ordered behind the buckets' all-reduces
-        without the host waiting for them (`Work.wait(stream_ordered=True)`), so the optimizer's launches are
-        queued while the last buckets are still in flight; a bucket that fails then raises from the next collective
-        instead of from this backward. False: the host waits, as the reference's DDP does (tandem/ddp.py:111-115).
+    def __init__(self, module, group, bucket_bytes=25 << 20, overlap=True, rebuild=True, direct=False, stream_ordered=False):
+        """stream_ordered=False (the default): at the end of backward the host waits for every bucket, as the
+        reference's DDP does (tandem/ddp.py:111-115), so a bucket that fails raises from this backward, before any
+        optimizer step can apply gradients that were never reduced.
+        stream_ordered=True (opt-in): the training stream is only ORDERED behind the buckets' all-reduces
+        (`Work.wait(stream_ordered=True)`) and the host goes on, so the optimizer's launches are queued while the
+        last buckets are still in flight (2-3 ms of a 30 ms step with torch's per-tensor AdamW). The price: when a
+        bucket then fails, the stream is let go, the optimizer that is already queued steps on unreduced gradients,
+        and the failure is raised by the next collective; the weights of that step must be thrown away.
         direct: the buckets live in the group's shared arenas (the gradients' size plus
         padding, in arenas of 1 GiB where that is more) and every
         all-reduce runs arena to arena (`group.all_reduce(..., direct=True)`): same

@@ -75,13 +75,16 @@ def _sizes(sizes):
 class Handle:
     """What tandem's _CppWork wraps (tandem/comm.py:84-107): wait() makes the caller's current
     stream wait for the collective, done() polls it, started / finished are its time stamps on
-    time.perf_counter's clock. Keeps the tensors alive until it is dropped: the C ABI has only
-    their addresses."""
+    time.perf_counter's clock. The C ABI has only the tensors' addresses, so the handle keeps
+    the tensors alive; one that is dropped before anybody waited for it hands them to its
+    engine, which lets go of them once the collective has run (the reference's engine holds
+    its tensor until the job has run, tandem/csrc/collectives.cpp:314-324)."""
 
-    def __init__(self, pointer, device, keep):
-        self._p, self._device, self._keep = pointer, device, keep
+    def __init__(self, pointer, device, keep, engine=None):
+        self._p, self._device, self._keep, self._engine, self._waited = pointer, device, keep, engine, False
 
     def wait(self):
+        self._waited = True  # from here on the caller's stream is ordered behind the collective
         _check(_L.tdm_work_wait(self._p, _stream(self._device)))
 
     def done(self):
@@ -97,8 +100,13 @@ class Handle:
 
     def __del__(self):
         p, self._p = getattr(self, "_p", None), None
-        if p:
-            _L.tdm_work_free(p)
+        if not p:
+            return
+        e = getattr(self, "_engine", None)
+        if e is not None and e._e and self._keep and not self._waited and not _L.tdm_work_done(p):
+            e._orphans.append((p, self._keep))  # not run yet and nobody waited: the tensors must outlive it
+            return
+        _L.tdm_work_free(p)
 
 
 class Engine:
@@ -106,6 +114,7 @@ class Engine:
 
     def __init__(self, job, rank, size, slots, slot_bytes, timeout, device):
         self._e, self._device = _VP(), torch.device("cuda", device)
+        self._orphans = []  # (work, tensors) of collectives whose handle was dropped before they had run
         _check(_L.tdm_engine_create(job.encode(), rank, size, slots, slot_bytes, float(timeout), device, ctypes.byref(self._e)))
 
     def connect(self):
@@ -113,16 +122,31 @@ class Engine:
 
     def close(self):
         e, self._e = self._e, None
+        orphans, self._orphans = self._orphans, []
         if e:
             try:
-                _check(_L.tdm_engine_close(e))
+                _check(_L.tdm_engine_close(e))  # runs what is queued and waits for the GPU
             finally:
+                for p, _ in orphans:
+                    _L.tdm_work_free(p)
                 _L.tdm_engine_destroy(e)
 
+    def _reap(self):
+        """Lets go of the tensors of dropped collectives that have finished on the GPU."""
+        still = []
+        for p, keep in self._orphans:
+            if _L.tdm_work_done(p):
+                _L.tdm_work_free(p)
+            else:
+                still.append((p, keep))
+        self._orphans = still
+
     def _start(self, call, *keep):
+        if self._orphans:
+            self._reap()
         out = _VP()
         _check(call(ctypes.byref(out)))
-        return Handle(out, self._device, keep)
+        return Handle(out, self._device, keep, self)
 
     def all_reduce(self, t, average):
         f = _flat(t)

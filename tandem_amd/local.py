@@ -225,8 +225,9 @@ class FoldTable:
         """The same fold without the uploaded table: its records are written on the GPU
         into a fixed array inside the library, so the call allocates nothing and copies
         nothing from the host (for callers under HIP graph capture or in loops that must
-        not allocate). At most lib().tdm_k2_static_max_tiles() tiles per call; calls
-        that overlap on different streams of one GPU race."""
+        not allocate). At most lib().tdm_k2_static_max_tiles() tiles per call. The calls
+        on one GPU share that array and the library orders them, across streams and host
+        threads; only graph replays holding such a call are the caller's to order."""
         check(lib().tdm_k2_bucket_fold_static(self._segs, self.nseg, self.world, dtype_code(self.dtype), int(average),
                                               int(accumulate), stream_ptr(self.device)))
 

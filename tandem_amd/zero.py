@@ -47,8 +47,14 @@ class _Range:
 class ZeRO(torch.nn.Module):
     """Stages 1 and 2."""
 
-    def __init__(self, module, group, stage=1, optimizer=None, bucket_bytes=25 << 20, direct=False, fused_step=False):
-        """direct: the flat parameter buffer and the gradient buffer (stage 2: one
+    def __init__(self, module, group, stage=1, optimizer=None, bucket_bytes=25 << 20, direct=False, fused_step=False,
+                 stream_ordered=False):
+        """stream_ordered (opt-in): step() only orders the training stream behind the all-gather of the new
+        parameters instead of making the host wait for it; should that all-gather fail, the next forward reads
+        parameters that never arrived and the failure is raised by the next collective. The default waits on the
+        host, as the reference's step() does (tandem/zero.py:157-164), and raises from step().
+
+        direct: the flat parameter buffer and the gradient buffer (stage 2: one
         staging buffer the size of the model, kept, instead of one per bucket that is
         dropped) live in the group's shared arenas (one of twice the model's size if the
         group has none; an arena each once that would reach 2 GiB, the size one arena
@@ -75,6 +81,7 @@ class ZeRO(torch.nn.Module):
         self.direct = bool(direct)
         self.opt = optimizer if optimizer is not None else ShardedAdamW()
         self.fused_step = bool(fused_step)
+        self.stream_ordered = bool(stream_ordered) and getattr(group, "stream_ordered_waits", False)
         if self.fused_step:
             if stage != 2 or not direct:
                 raise ValueError("fused_step needs stage=2 and direct=True")
@@ -211,7 +218,7 @@ class ZeRO(torch.nn.Module):
             return
         grad = self.grad[lo:hi] if self.stage == 1 else self.grad_shard
         self.opt.update("flat", self.buf[lo:hi], grad)
-        if getattr(self.g, "stream_ordered_waits", False):
+        if self.stream_ordered:
             # the next forward only has to come after the gather on the stream: the host does not wait for it
             self.g.all_gather(self.buf, self.flat.sizes, async_op=True, **self._how).wait(stream_ordered=True)
         else:

@@ -161,8 +161,8 @@ def test_adamw_on_a_shard_off_the_16_byte_grid(dev, order):
         pad = 8
         stores = [torch.full((n + 2 * pad,), -7.0, device=dev) for _ in range(4 + ncopies)]
         views = [s_[pad + ph:pad + ph + n] for s_, ph in zip(stores, phases)]
-        for v_ in views:
-            assert v_.data_ptr() % 16 == 4 * (phases[views.index(v_)] % 4)
+        for v_, ph in zip(views, phases):
+            assert v_.data_ptr() % 16 == 4 * (ph % 4)
         views[0].copy_(p0[:n])
         views[2].zero_()
         views[3].zero_()

@@ -80,6 +80,24 @@ def rank_main(rank, size, job, barrier, outdir):
             call()
         except ValueError:
             out[f"refused_{bad}"] = np.array(True)
+    # a handle dropped before anybody waited for it: its tensor must outlive the collective (the reference's engine
+    # holds it until the job has run, tandem/csrc/collectives.cpp:314-324). Rank 1 arrives late, so on rank 0 the
+    # collective has certainly not run when the handle goes; memory allocated right afterwards must not be the tensor's.
+    big = torch.full((1 << 20,), float(rank + 1), device=dev)
+    address = big.data_ptr()
+    torch.cuda.synchronize()
+    if rank == 1:
+        time.sleep(0.3)
+    handle = engine.all_reduce(big, False)
+    del handle, big
+    decoys = [torch.full((1 << 20,), -5.0, device=dev) for _ in range(3)]
+    out["dropped_parked"] = np.array(rank == 1 or len(engine._orphans) == 1)
+    out["dropped_not_reused"] = np.array(all(t.data_ptr() != address for t in decoys) or rank == 1)
+    engine.barrier().wait()
+    torch.cuda.synchronize()
+    out["decoys_intact"] = np.array(all(bool((t == -5.0).all()) for t in decoys))
+    engine.barrier().wait()  # the next call lets go of what has finished
+    out["dropped_reaped"] = np.array(len(engine._orphans) == 0)
     torch.cuda.synchronize()
     engine.barrier().wait()
     engine.close()
@@ -104,4 +122,6 @@ def test_the_documented_binding_runs_the_reference_fixtures():
         assert bool(res[r]["bool_ok"])
         for bad in ("bool", "cpu", "strided", "sizes"):
             assert bool(res[r].get(f"refused_{bad}", False)), (r, bad)
+        for what in ("dropped_parked", "dropped_not_reused", "decoys_intact", "dropped_reaped"):
+            assert bool(res[r][what]), (r, what)
     assert np.array_equal(bits(res[1]["recv_100"]), bits(d["r0_in"][:100]))

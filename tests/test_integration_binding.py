@@ -42,3 +42,63 @@ def test_the_binding_has_the_surface_the_reference_calls():
     import re
     for sym in set(re.findall(r"\btdm_[a-z0-9_]+", source)):
         assert re.search(rf"\b{sym}\s*\(", header), sym
+
+
+def test_a_handle_dropped_before_its_collective_ran_leaves_its_tensors_with_the_engine(monkeypatch):
+    """The binding's handle keeps the tensors alive (the C ABI has only addresses). Dropped without a wait while the
+    collective has not run, it parks (work, tensors) on its engine, which frees the work and lets go of the tensors
+    once the collective is done: at the next call, or in close(). A handle that was waited for, or whose collective
+    has finished, is freed at once. The reference's engine holds its tensor until the job has run
+    (tandem/csrc/collectives.cpp:314-324). The library is replaced by a recorder here; tests/test_gpu_integration.py
+    drops a handle on the GPU."""
+    from tandem_amd import hip_engine
+
+    class Recorder:
+        def __init__(self):
+            self.done, self.freed, self.closed = set(), [], []
+
+        def tdm_work_done(self, p):
+            return int(p in self.done)
+
+        def tdm_work_free(self, p):
+            self.freed.append(p)
+
+        def tdm_work_wait(self, p, stream):
+            return 0
+
+        def tdm_engine_close(self, e):
+            self.closed.append(e)
+            return 0
+
+        def tdm_engine_destroy(self, e):
+            pass
+
+        def tdm_barrier(self, e, out):
+            return 0
+
+    lib = Recorder()
+    monkeypatch.setattr(hip_engine, "_L", lib)
+    monkeypatch.setattr(hip_engine, "_stream", lambda device: None)
+    engine = hip_engine.Engine.__new__(hip_engine.Engine)
+    engine._e, engine._device, engine._orphans = "engine", None, []
+    tensor = object()
+    hip_engine.Handle("w1", None, (tensor,), engine)  # dropped at once, not run, never waited for
+    assert engine._orphans == [("w1", (tensor,))] and lib.freed == []
+    waited = hip_engine.Handle("w2", None, (tensor,), engine)
+    waited.wait()
+    del waited
+    finished = hip_engine.Handle("w3", None, (tensor,), engine)
+    lib.done.add("w3")
+    del finished
+    hip_engine.Handle("w4", None, (), engine)  # a barrier's handle keeps nothing alive
+    assert lib.freed == ["w2", "w3", "w4"] and len(engine._orphans) == 1
+    engine.barrier()  # w1 still not done: stays parked
+    assert len(engine._orphans) == 1
+    lib.done.add("w1")
+    h = engine.barrier()
+    assert engine._orphans == [] and "w1" in lib.freed
+    del h
+    hip_engine.Handle("w5", None, (tensor,), engine)
+    assert [p for p, _ in engine._orphans] == ["w5"]
+    engine.close()  # close runs what is queued, then frees what was parked
+    assert lib.closed == ["engine"] and "w5" in lib.freed and engine._orphans == []

@@ -257,3 +257,73 @@ def test_ddp_carves_its_buckets_from_slabs(slab_bytes, monkeypatch):
     z._build(list(z.params))  # the order in which the gradients turned out to arrive
     check()
     assert len(g.arenas) <= arenas + 1
+
+
+class _FailingGroup:
+    """One rank whose second all_reduce fails when waited for on the host; a wait that only orders the stream
+    (what tandem_amd.Group offers as Work.wait(stream_ordered=True)) returns without a word, as it does on the GPU
+    when the collective has not run yet."""
+
+    size, rank, stream_ordered_waits = 1, 0, True
+
+    class _Work:
+        def __init__(self, group, fails):
+            self.group, self.fails = group, fails
+
+        def wait(self, stream_ordered=False):
+            self.group.waits.append("stream" if stream_ordered else "host")
+            if self.fails and not stream_ordered:
+                raise RuntimeError("all_reduce: rank 1 did not answer in time")
+
+    def __init__(self):
+        self.calls, self.waits = 0, []
+
+    def broadcast(self, t, root=0, async_op=False):
+        return t
+
+    def pack(self, flat, pieces):
+        for off, t in pieces:
+            flat[off:off + t.numel()].copy_(t.reshape(-1))
+
+    def all_reduce(self, t, op="sum", async_op=False, **_):
+        self.calls += 1
+        return self._Work(self, fails=self.calls == 2)
+
+    def all_gather(self, t, sizes=None, async_op=False, **_):
+        work = self._Work(self, fails=False)
+        return work if async_op else work.wait()
+
+
+def test_a_failed_bucket_raises_from_backward_before_any_step():
+    """DDP's default waits for its buckets on the host at the end of backward, as the reference's does
+    (tandem/ddp.py:111-115): a bucket whose all-reduce fails raises from that backward, so no optimizer step is
+    taken on gradients that were never reduced. Ordering only the stream is opt-in, and then this backward returns."""
+    torch.manual_seed(0)
+    text = synthetic(5_000)
+    x, y = text.batch(0, 4, CFG.seq)
+    g = _FailingGroup()
+    z = DDP(GPT(CFG), g, bucket_bytes=4 << 10)
+    assert z.stream_ordered is False and len(z.buckets) > 2
+    before = [p.detach().clone() for p in z.module.parameters()]
+    with pytest.raises(RuntimeError, match="did not answer"):
+        z(x, y).backward()
+    assert set(g.waits) == {"host"}
+    assert all(torch.equal(a, b) for a, b in zip(before, z.module.parameters()))
+    g = _FailingGroup()
+    z = DDP(GPT(CFG), g, bucket_bytes=4 << 10, stream_ordered=True)
+    z(x, y).backward()  # the failure is the next collective's to raise (tests/test_gpu_group.py)
+    assert set(g.waits) == {"stream"}
+
+
+def test_zero_waits_for_its_all_gather_on_the_host_unless_asked():
+    torch.manual_seed(0)
+    text = synthetic(5_000)
+    x, y = text.batch(0, 4, CFG.seq)
+    for ordered, want in ((False, "host"), (True, "stream")):
+        g = _FailingGroup()
+        g.calls = 10  # nothing fails here
+        z = ZeRO(GPT(CFG), g, 1, OracleShardedAdamW(lr=3e-3, weight_decay=0.1), 4 << 10, stream_ordered=ordered)
+        z(x, y).backward()
+        g.waits.clear()
+        z.step()
+        assert g.waits == [want], (ordered, g.waits)

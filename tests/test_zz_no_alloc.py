@@ -1,7 +1,9 @@
 """tdm_k2_bucket_fold_static, the bucket fold that allocates nothing: through the C ABI,
 against tdm_k2_table_build + tdm_k2_bucket_fold on the same segments, bit for bit, on two
 calls in a row (the second smaller, so that it finds the first call's records in the
-shared table), then its refusal of a call beyond the fixed table."""
+shared table), then its refusal of a call beyond the fixed table, and calls that follow
+each other on different streams and from different host threads without a wait between
+them (the library orders their use of the shared table)."""
 
 import ctypes
 
@@ -205,3 +207,66 @@ def test_replayed_from_a_hip_graph():
             for i in range(len(numels)):
                 assert np.array_equal(bits(grads[r][i].cpu().numpy()), bits(other[r][i].cpu().numpy())), (k, r, i)
         assert not torch.equal(grads[0][0].cpu(), ins[k][0][0])  # (the fold did run)
+
+
+def test_calls_on_two_streams_and_from_two_threads_do_not_overlap():
+    """All calls on a GPU share one table. A large call on one stream (its fold runs for a while) is followed at
+    once, with no wait on the host, by a small call on another stream whose fill kernel overwrites the first
+    records: the library makes the second stream wait for the first call's fold. Six such pairs alternating the
+    streams, then the same from two host threads with a stream each; every call's result equals the table
+    entry point's."""
+    import threading
+
+    from tandem_amd._lib import check, dtype_code, lib
+
+    dev = torch.device("cuda", 0)
+    world, code = 4, dtype_code(torch.float32)
+    big, small = [1_048_576] * 12 + [300_001, 5, 4099], [4099, 64, 1000]
+    streams = [torch.cuda.Stream(dev), torch.cuda.Stream(dev)]
+    expected = {}
+    for name, numels, seed in (("big", big, 21), ("small", small, 22)):
+        g, o, segs, nseg = _segments(world, numels, seed, dev)
+        _with_table(segs, nseg, world, code, dev, 1, 0)
+        expected[name] = o
+
+    def fresh(name, numels, seed):
+        g, o, segs, nseg = _segments(world, numels, seed, dev)
+        return dict(name=name, grads=g, outs=o, segs=segs, nseg=nseg)
+
+    def enqueue(job, stream):
+        check(lib().tdm_k2_bucket_fold_static(job["segs"], job["nseg"], world, code, 1, 0, ctypes.c_void_p(stream.cuda_stream)))
+
+    for pair in range(6):
+        a, b = fresh("big", big, 21), fresh("small", small, 22)
+        torch.cuda.synchronize(dev)
+        print(f"static fold on two streams: pair {pair}", flush=True)
+        enqueue(a, streams[pair % 2])
+        enqueue(b, streams[1 - pair % 2])  # nothing on the host between the two
+        torch.cuda.synchronize(dev)
+        _same(expected["big"], a["outs"], f"pair {pair}, the large call")
+        _same(expected["small"], b["outs"], f"pair {pair}, the small call")
+
+    jobs = [[fresh("big", big, 21), fresh("small", small, 22), fresh("big", big, 21)],
+            [fresh("small", small, 22), fresh("big", big, 21), fresh("small", small, 22)]]
+    torch.cuda.synchronize(dev)
+    errors = []
+
+    def worker(k):
+        try:
+            torch.cuda.set_device(dev)
+            for job in jobs[k]:
+                enqueue(job, streams[k])
+        except Exception as e:  # surfaces in the main thread
+            errors.append(e)
+
+    print("static fold from two host threads", flush=True)
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize(dev)
+    assert not errors, errors
+    for k in range(2):
+        for job in jobs[k]:
+            _same(expected[job["name"]], job["outs"], f"thread {k}, a {job['name']} call")
