@@ -351,17 +351,19 @@ def zero2_step(dev, reps):
     out = {"workload": "85,842,432 fp32 params, world 4 on one GPU, 16 buckets of <= 25 MiB, AdamW(3e-4, (0.9, 0.95), 1e-8, 0.1) on all 4 shards"}
     shard = z.layouts[0].hi - z.layouts[0].lo
     opt = timed(lambda: [z.opts[r].update("bench", z.bufs[r][z.layouts[r].lo:z.layouts[r].hi], z.grad_shards[r]) for r in range(WORLD)], reps)
-    # the same four updates on shards that start 4 bytes off a 16-byte boundary, as tensor_split shards may (p, g, m, v at one phase)
+    # the same four updates on shards that start 4 bytes off a 128-byte boundary, as tensor_split shards may (p, g, m, v at one
+    # phase), and on aligned shards cut from the very same allocations, so that only the phase differs between the two
     from tandem_amd.optim import ShardedAdamW
 
-    off_opt = ShardedAdamW(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
-    off_p = [torch.zeros(shard + 4, device=dev)[1:1 + shard].normal_(0.0, 0.02, generator=gen) for _ in range(WORLD)]
-    off_g = [torch.zeros(shard + 4, device=dev)[1:1 + shard].normal_(0.0, 1e-3, generator=gen) for _ in range(WORLD)]
-    assert all(t.data_ptr() % 16 == 4 for t in off_p + off_g)
-    opt_off = timed(lambda: [off_opt.update(r, off_p[r], off_g[r]) for r in range(WORLD)], reps)
-    out["adamw_4_shards_off_grid_ms"] = round(opt_off * 1e3, 4)
-    out["adamw_off_grid_over_aligned"] = round(opt_off / opt, 4)
-    del off_p, off_g, off_opt
+    stores = [[torch.zeros(shard + 64, device=dev).normal_(0.0, scale, generator=gen) for scale in (0.02, 1e-3)] for _ in range(WORLD)]
+    for label, lead in (("on_grid", 0), ("off_grid", 1)):
+        o = ShardedAdamW(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+        ps, gs = [st[0][lead:lead + shard] for st in stores], [st[1][lead:lead + shard] for st in stores]
+        assert all(t.data_ptr() % 128 == 4 * lead for t in ps + gs)
+        out[f"adamw_4_shards_{label}_ms"] = round(timed(lambda: [o.update(r, ps[r], gs[r]) for r in range(WORLD)], reps) * 1e3, 4)
+        del o, ps, gs
+    out["adamw_off_grid_over_on_grid"] = round(out["adamw_4_shards_off_grid_ms"] / out["adamw_4_shards_on_grid_ms"], 4)
+    del stores
     # the all-gather of the flat parameter buffers in both of the library's forms, each on the bytes that form moves
     check(lib().tdm_set_ring_form(1))
     ag_one = timed(lambda: z.lw.all_gather(z.bufs, z.layouts[0].sizes), reps)
@@ -426,11 +428,12 @@ def fsdp_rank(g, steps, prefetch):
     model = GPT(cfg).to(g.device)
     f = FSDP(model, g, ShardedAdamW(lr=3e-4, betas=(0.9, 0.95), weight_decay=0.1), prefetch=prefetch)
     times, waits = [], []
-    for step in range(steps + 2):
+    for step in range(steps + 3):
+        traced = step == steps + 2  # one more step with the group's trace on, for the counts; the timed steps carry no time-stamp events
         x, y = text.batch(step, 8, cfg.seq, rank=g.rank, world=g.size, device=g.device)
         g.barrier()
         torch.cuda.synchronize()
-        g.tracing = True
+        g.tracing = traced
         g.waits.clear()
         g.trace.clear()
         t0 = time.perf_counter()
@@ -441,23 +444,28 @@ def fsdp_rank(g, steps, prefetch):
         f.step()
         f.zero_grad()
         torch.cuda.synchronize()
-        if step >= 2:
+        if 2 <= step < steps + 2:
             times.append(t1 - t0)
+        if traced:
             waits.append(sum(b - a for name, a, b in g.waits if name == "gather_unit"))
+            traced_ms = (t1 - t0) * 1e3
     n_gathers = sum(1 for name, *_ in g.trace if name == "gather_unit")
-    return {"fwd_bwd_ms": statistics.median(times) * 1e3, "host_blocked_on_gathers_ms": statistics.median(waits) * 1e3,
+    return {"fwd_bwd_ms": statistics.median(times) * 1e3, "fwd_bwd_ms_min": min(times) * 1e3, "fwd_bwd_ms_max": max(times) * 1e3,
+            "traced_step_fwd_bwd_ms": traced_ms, "traced_step_host_blocked_on_gathers_ms": statistics.median(waits) * 1e3,
             "gathers_per_step": n_gathers, "max_live": f.max_live, "live": f.live, "loss": float(loss.detach())}
 
 
 def fsdp_gather(steps):
     """ZeRO-3's unit gathers: copies launched in order on the training stream (the
-    default), or on the engine's side stream with and without prefetch."""
+    default), or on the engine's side stream, ordered against the training stream by value
+    words (one call per stream and dependency) or by events, with and without prefetch."""
     from tandem_amd import launch
 
     out = {}
     before = os.environ.get("TANDEM_HIP_GATHER")
     try:
         for label, where, prefetch in (("in_order", "caller", True), ("side_stream_prefetch", "stream", True),
+                                       ("side_stream_events_prefetch", "stream-events", True),
                                        ("side_stream_no_prefetch", "stream", False)):
             os.environ["TANDEM_HIP_GATHER"] = where
             res = launch(fsdp_rank, 2, steps, prefetch, gpus=[0, 0], timeout=120.0)
@@ -804,7 +812,7 @@ def main():
     ipc = train = train4 = None
     if not args.quick and not args.no_fsdp:
         try:
-            fsdp = fsdp_gather(3)
+            fsdp = fsdp_gather(8)
         except Exception as e:  # a secondary figure must not lose the line
             fsdp = {"error": repr(e)[:300]}
         try:

@@ -212,7 +212,8 @@ class Engine {
   bool connected_ = false, closed_ = false;
   // staged collectives
   bool staged_ = true;               // TANDEM_HIP_ALGO=ring switches them off
-  bool gathers_on_side_stream_ = false;  // TANDEM_HIP_GATHER=stream
+  bool gathers_on_side_stream_ = false;  // TANDEM_HIP_GATHER=stream (or stream-events)
+  bool gather_words_ = true;             // side-stream gathers are ordered by value words, not by events
   std::shared_ptr<FlagPool> flags_;      // the words that tdm_work_wait_stream parks streams on
   bool want_flags_ = false;              // the device can make a stream wait for a value
   bool defer_default_ = false;           // TANDEM_HIP_WAIT=stream: tdm_work_wait parks as well

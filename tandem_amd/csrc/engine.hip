@@ -82,7 +82,12 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
       }
     }
   }
-  if (const char* gm = std::getenv("TANDEM_HIP_GATHER")) gathers_on_side_stream_ = std::string(gm) == "stream";
+  if (const char* gm = std::getenv("TANDEM_HIP_GATHER")) {
+    // "stream": on the engine's side stream, ordered against the caller's by value words where the device has them;
+    // "stream-events": the same with an event per dependency (what a device without such waits falls back to)
+    gathers_on_side_stream_ = std::string(gm) == "stream" || std::string(gm) == "stream-events";
+    gather_words_ = std::string(gm) != "stream-events";
+  }
   if (const char* rd = std::getenv("TANDEM_HIP_READY")) ready_on_host_ = std::string(rd) != "gpu";
   peer_staging_.assign(size, nullptr);
 
@@ -1098,24 +1103,63 @@ std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, st
   check_hip(hipSetDevice(device_), "hipSetDevice");
   hipStream_t on = caller;
   if (gathers_on_side_stream_) {
-    // Start once the caller's stream has produced the buffer (and finished with its last use).
+    // Start once the caller's stream has produced the buffer (and finished with its last use). Where streams can write
+    // and wait for a value, that costs one call on each stream and a word of the engine's pool: the caller's stream
+    // writes the word when it gets here, the side stream waits for it. (An event for the same purpose is created,
+    // recorded, waited for and destroyed: four runtime calls of 13-31 us where these two take about 4 us each.)
     on = gather_stream_;
-    hipEvent_t ready;
-    check_hip(hipEventCreateWithFlags(&ready, hipEventDisableTiming), "hipEventCreateWithFlags (ready)");
-    hipError_t err = hipEventRecord(ready, caller);
-    if (err == hipSuccess) err = hipStreamWaitEvent(gather_stream_, ready, 0);
-    (void)hipEventDestroy(ready);
-    check_hip(err, "ordering a gather after the caller's stream");
+    bool ordered = false;
+    if (flags_ && gather_words_) {
+      uint32_t value = 0;
+      const int word = flags_->acquire(&value);
+      if (word >= 0) {
+        hipError_t err = hipStreamWriteValue32(caller, flags_->base + word, value, 0);
+        if (err == hipSuccess) {
+          err = hipStreamWaitValue32(gather_stream_, flags_->base + word, value, hipStreamWaitValueGte, 0xffffffffu);
+        } else {
+          flags_->set(word, value);  // nothing will write it: it must not be handed out as pending for ever
+        }
+        flags_->release(word);  // stays out of circulation until the caller's stream has written it
+        check_hip(err, "ordering a gather after the caller's stream (value)");
+        ordered = true;
+      }
+    }
+    if (!ordered) {
+      hipEvent_t ready;
+      check_hip(hipEventCreateWithFlags(&ready, hipEventDisableTiming), "hipEventCreateWithFlags (ready)");
+      hipError_t err = hipEventRecord(ready, caller);
+      if (err == hipSuccess) err = hipStreamWaitEvent(gather_stream_, ready, 0);
+      (void)hipEventDestroy(ready);
+      check_hip(err, "ordering a gather after the caller's stream");
+    }
   }
   stamp_start(*work, on);
   for (int at = 0; at < np; at += TDM_MAX_PAIRS) {
     copy_step(pairs + at, std::min<int>(TDM_MAX_PAIRS, np - at), full.dtype, 0, on);
   }
-  // On the caller's own stream nothing needs ordering afterwards: the done event only
-  // serves done() and the time stamps, and wait() finds it on the stream it would wait on.
-  check_hip(hipEventCreateWithFlags(&work->done_event, work->start_event ? hipEventDefault : hipEventDisableTiming),
-            "hipEventCreateWithFlags (done)");
-  check_hip(hipEventRecord(work->done_event, on), "hipEventRecord (done)");
+  // Its end. On the side stream: the Work's own word, written by that stream behind the last copy, which wait() parks
+  // the caller's stream on and done() reads (as for every collective of the progress thread). On the caller's own
+  // stream nothing needs ordering afterwards: wait() finds the Work on the stream it would wait on. An event is
+  // recorded only where there is no word, for done() on the caller's own stream, and for the time stamps.
+  if (gathers_on_side_stream_ && flags_ && gather_words_) {
+    work->flag = flags_->acquire(&work->flag_value);
+    if (work->flag >= 0) {
+      work->flags = flags_;
+      const hipError_t err = hipStreamWriteValue32(gather_stream_, flags_->base + work->flag, work->flag_value, 0);
+      if (err != hipSuccess) {  // no word after all (the Work gives it back); the event below takes its place
+        flags_->set(work->flag, work->flag_value);
+        flags_->release(work->flag);
+        work->flag = -1;
+        work->flags.reset();
+        (void)hipGetLastError();
+      }
+    }
+  }
+  if (work->flag < 0 || work->start_event) {
+    check_hip(hipEventCreateWithFlags(&work->done_event, work->start_event ? hipEventDefault : hipEventDisableTiming),
+              "hipEventCreateWithFlags (done)");
+    check_hip(hipEventRecord(work->done_event, on), "hipEventRecord (done)");
+  }
   work->on_callers_stream = !gathers_on_side_stream_;
   work->launched_on = on;
   work->t1 = now_s();

@@ -1077,14 +1077,24 @@ void adamw_launch(float* p, const float* g, float* m, float* v, int64_t n, const
       if (ptrs[i] < ptrs[j] + bytes && ptrs[j] < ptrs[i] + bytes) throw Invalid("p, g, m, v and the copies must not overlap");
     }
   // A shard cut out of a flat buffer starts anywhere (tensor_split). When all the streams start at the same distance
-  // from a 16-byte boundary, the few elements before it are peeled off and the rest runs on vectors.
+  // from a 16-byte boundary, the few elements before it are peeled off and the rest runs on vectors ...
   const SegPlan plan = plan_segment(ptrs, 4 + ncopies, n, 4, static_cast<int64_t>(kAdamwThreads) * kAdamwUnroll * 4);
   const bool vec = plan.vec;
-  if (vec && plan.head) {
-    a.p += plan.head, a.g += plan.head, a.m += plan.head, a.v += plan.head;
-    for (int c = 0; c < ncopies; ++c) a.copy[c] += plan.head;
-    a.n = plan.body;
-    a.head = plan.head;
+  if (vec) {
+    // ... and when the streams also agree on their distance from a 128-byte boundary, the head is stretched to it
+    // (up to 31 elements): every wave then writes whole cache lines, which no other wave touches.
+    int64_t head = plan.head;
+    const uintptr_t line = (ptrs[0] + head * 4) % 128;
+    bool same = true;
+    for (int i = 1; i < 4 + ncopies; ++i) same = same && (ptrs[i] + head * 4) % 128 == line;
+    const int64_t more = static_cast<int64_t>((128 - line) % 128) / 4;
+    if (same && more < plan.body) head += more;
+    if (head) {
+      a.p += head, a.g += head, a.m += head, a.v += head;
+      for (int c = 0; c < ncopies; ++c) a.copy[c] += head;
+      a.n = n - head;
+      a.head = static_cast<int>(head);
+    }
   }
   const dim3 block(kAdamwThreads);
   const int64_t tiles = vec ? (a.n / 4 + kAdamwThreads * kAdamwUnroll - 1) / (kAdamwThreads * kAdamwUnroll) : (n + kAdamwThreads - 1) / kAdamwThreads;

@@ -696,7 +696,7 @@ struct AdamwArgs {
   // update and the all-gather of the result in one pass.
   int ncopies;
   int shift;  // of tile_of()
-  int head;   // vector path: elements (fewer than a vector) that lie before the pointers, peeled off an unaligned shard
+  int head;   // vector path: elements (at most 31: up to a cache line) that lie before the pointers, peeled off an unaligned shard
   float* copy[TDM_MAX_WORLD - 1];
 };
 
@@ -768,7 +768,7 @@ __global__ __launch_bounds__(kAdamwThreads) void k3_adamw_kernel(AdamwArgs a) {
         }
       }
     }
-    // the last few elements (lanes 0..), and the head before the first vector (lanes 32..): fewer than a vector each
+    // the last few elements (lanes 0..3), and the head before the first vector (lanes 32..62)
     if (blockIdx.x == 0 && (threadIdx.x < a.n - nv * 4 || (threadIdx.x >= 32 && static_cast<int>(threadIdx.x) - 32 < a.head))) {
       const int64_t i = threadIdx.x < 32 ? nv * 4 + threadIdx.x : -1 - (static_cast<int64_t>(threadIdx.x) - 32);
       adamw_elem<kOrder>(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);

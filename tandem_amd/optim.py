@@ -34,18 +34,20 @@ def step_scalars(step, lr, betas, eps, weight_decay):
     return s
 
 
+LINE = 128  # bytes: the kernels write whole cache lines when all of a launch's streams share their distance from one
+
+
 def zeros_at_phase_of(like, numel=None):
     """A zeroed tensor of `numel` elements (default: as many as `like`) in `like`'s memory
-    that starts at the same distance from a 16-byte boundary as `like` does. A shard cut
+    that starts at the same distance from a 128-byte boundary as `like` does. A shard cut
     out of a flat buffer by tensor_split starts anywhere; the kernels run on 16-byte
-    vectors when all of their streams share that distance (the few elements before the
-    boundary are peeled off), so a shard's gradient and optimizer state are laid out at
-    the shard's own phase."""
+    vectors, and on whole cache lines, when all of their streams share that distance (the
+    few elements before the boundary are peeled off), so a shard's gradient and optimizer
+    state are laid out at the shard's own phase."""
     n = like.numel() if numel is None else int(numel)
     es = like.element_size()
-    lead = (like.data_ptr() % 16) // es
-    store = torch.zeros(n + 16 // es, device=like.device, dtype=like.dtype)
-    lead = (lead - (store.data_ptr() % 16) // es) % (16 // es)
+    store = torch.zeros(n + LINE // es, device=like.device, dtype=like.dtype)
+    lead = ((like.data_ptr() - store.data_ptr()) % LINE) // es
     return store[lead:lead + n]
 
 

@@ -140,11 +140,13 @@ def test_adamw_writing_further_copies(dev):
 @pytest.mark.parametrize("order", ["host", "device"])
 def test_adamw_on_a_shard_off_the_16_byte_grid(dev, order):
     """tensor_split shards start anywhere. With p, g, m, v (and the copies) all at the
-    same distance from a 16-byte boundary the launcher peels that head and runs vectors;
-    with streams that disagree it goes element by element. Both against the plain aligned
-    update on the same numbers, which the tests above pin to the oracle and to torch:
-    every phase 1..3, lengths that leave a head, a tail, both, fewer elements than the
-    head, with and without copies; guard elements around every stream stay untouched."""
+    same distance from a 16-byte boundary the launcher peels that head and runs vectors,
+    and when they also share their distance from a 128-byte boundary it peels up to that
+    line (as many as 31 elements); with streams that disagree within 16 bytes it goes
+    element by element. All against the plain aligned update on the same numbers, which
+    the tests above pin to the oracle and to torch: phases of 1..31 elements, streams that
+    agree only within 16 bytes, lengths that leave a head, a tail, both, fewer elements than
+    the head, with and without copies; guard elements around every stream stay untouched."""
     import ctypes
 
     from tandem_amd import _lib
@@ -158,11 +160,11 @@ def test_adamw_on_a_shard_off_the_16_byte_grid(dev, order):
 
     def run(n, phases, ncopies):
         """Three steps over streams laid at the given phases (elements off a 16-byte boundary) inside guarded stores."""
-        pad = 8
+        pad = 64  # two cache lines of guard elements either side
         stores = [torch.full((n + 2 * pad,), -7.0, device=dev) for _ in range(4 + ncopies)]
         views = [s_[pad + ph:pad + ph + n] for s_, ph in zip(stores, phases)]
         for v_, ph in zip(views, phases):
-            assert v_.data_ptr() % 16 == 4 * (ph % 4)
+            assert v_.data_ptr() % 128 == 4 * ph
         views[0].copy_(p0[:n])
         views[2].zero_()
         views[3].zero_()
@@ -179,40 +181,40 @@ def test_adamw_on_a_shard_off_the_16_byte_grid(dev, order):
             assert float((s_[:pad + ph] + 7.0).abs().sum()) == 0 and float((s_[pad + ph + n:] + 7.0).abs().sum()) == 0
         return [v_.clone() for v_ in views]
 
-    for n in (1, 2, 3, 5, 127, 4099, 100_003):
+    for n in (1, 2, 3, 5, 30, 31, 33, 127, 4099, 100_003):
         p0 = torch.randn(n, generator=gen).to(dev) * 0.02
         grads = [(torch.randn(n, generator=gen) * 1e-3).to(dev) for _ in range(3)]
         for ncopies in (0, 2):
             want = run(n, [0] * (4 + ncopies), ncopies)
-            for ph in (1, 2, 3):
-                got = run(n, [ph] * (4 + ncopies), ncopies)  # one phase for all: head peeled, vectors
+            layouts = [[ph] * 6 for ph in (1, 2, 3, 4, 5, 17, 30, 31)]  # one phase for all: peeled to the cache line, vectors
+            layouts += [[1, 5, 9, 13, 17, 29], [3, 3, 7, 3, 31, 3]]     # agreeing within 16 bytes only: peeled to the vector
+            layouts += [[1, 0, 3, 2, 1, 2]]                             # disagreeing: element by element
+            for phases in layouts:
+                got = run(n, phases[:4 + ncopies], ncopies)
                 for a, b in zip(want, got):
-                    assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (n, ph, ncopies, order)
-            got = run(n, [1, 0, 3, 2, 1, 2][:4 + ncopies], ncopies)  # phases that disagree: element by element
-            for a, b in zip(want, got):
-                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (n, "mixed", ncopies, order)
+                    assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (n, phases, ncopies, order)
 
 
 def test_optimizer_state_follows_the_shards_phase(dev):
     """ShardedAdamW lays a shard's exp_avg and exp_avg_sq out at the shard's own distance from
-    a 16-byte boundary, and ZeRO's gradient shard likewise, so that the update of a
+    a 128-byte boundary, and ZeRO's gradient shard likewise, so that the update of a
     tensor_split shard that starts anywhere still runs on vectors."""
     from tandem_amd import ShardedAdamW
     from tandem_amd.optim import zeros_at_phase_of
 
     flat = torch.zeros(1000, device=dev)
     opt = ShardedAdamW()
-    for lo in (0, 1, 2, 3, 5):
+    for lo in (0, 1, 2, 3, 29):
         p = flat[lo:lo + 333]
         g = zeros_at_phase_of(p)
-        assert g.numel() == 333 and g.data_ptr() % 16 == p.data_ptr() % 16 and float(g.abs().sum()) == 0
+        assert g.numel() == 333 and g.data_ptr() % 128 == p.data_ptr() % 128 and float(g.abs().sum()) == 0
         opt.update(lo, p, g)
         _, m, v = opt.state[lo]
-        assert m.data_ptr() % 16 == v.data_ptr() % 16 == p.data_ptr() % 16
+        assert m.data_ptr() % 128 == v.data_ptr() % 128 == p.data_ptr() % 128
         assert m.numel() == v.numel() == 333
     assert opt.state_bytes() == 5 * 2 * 4 * 333
     half = torch.zeros(64, device=dev, dtype=torch.float16)[3:40]
-    assert zeros_at_phase_of(half).data_ptr() % 16 == half.data_ptr() % 16 and zeros_at_phase_of(half, 5).numel() == 5
+    assert zeros_at_phase_of(half).data_ptr() % 128 == half.data_ptr() % 128 and zeros_at_phase_of(half, 5).numel() == 5
 
 
 def test_adamw_rejects_what_it_cannot_do(dev):

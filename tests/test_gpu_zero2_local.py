@@ -91,10 +91,10 @@ def test_shards_that_start_off_the_16_byte_grid(algorithm):
     z = LocalZeRO2(world, numels, dev, bucket_bytes=16 << 10, **KW)
     assert sorted(l.lo % 4 for l in z.layouts) == [0, 1, 2], [l.lo for l in z.layouts]
     for r, l in enumerate(z.layouts):  # the layout this test is about
-        phase = z.bufs[r][l.lo:l.hi].data_ptr() % 16
-        assert phase == 4 * (l.lo % 4)
-        assert z.grad_shards[r].data_ptr() % 16 == phase
-        assert z.opts[r].state["flat"][1].data_ptr() % 16 == z.opts[r].state["flat"][2].data_ptr() % 16 == phase
+        phase = z.bufs[r][l.lo:l.hi].data_ptr() % 128
+        assert phase == 4 * (l.lo % 32)
+        assert z.grad_shards[r].data_ptr() % 128 == phase
+        assert z.opts[r].state["flat"][1].data_ptr() % 128 == z.opts[r].state["flat"][2].data_ptr() % 128 == phase
     p0 = (seeded(2, 0, n) * 0.02).numpy()
     steps = 5
     grads = [[(seeded(20 + s, r, n) * 1e-3).numpy() for r in range(world)] for s in range(steps)]
