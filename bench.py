@@ -383,6 +383,19 @@ def zero2_step(dev, reps):
     out.update({"one_launch_ms": round(one * 1e3, 4), "one_launch_algorithmic_bytes": one_bytes,
                 "one_launch_GBps": round(one_bytes / one / 1e9, 1),
                 "one_launch_roofline_floor_ms": round(one_bytes / (HBM_PEAK_GBPS * 1e9) * 1e3, 4)})
+    # the same one-launch step with all 20 buffers carved out of ONE allocation instead of an allocation each
+    z1 = LocalZeRO2(WORLD, numels, dev, one_allocation=True, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    for b in z1.bufs:
+        b.copy_(p0)
+
+    def refill_grads_1():
+        for r in range(WORLD):
+            z1.staging[r].copy_(grads[r])
+
+    t1 = timed(refill_grads_1, reps)
+    out["one_launch_one_allocation_ms"] = round((timed(lambda: (refill_grads_1(), z1.reduce_and_step()), reps) - t1) * 1e3, 4)
+    del z1
+    torch.cuda.empty_cache()
     for algorithm, rs_bytes in (("fold", (WORLD + 2) * 4 * n), ("ring", 12 * (WORLD - 1) * n + 12 * n)):
         # default: fold + the update that also writes the other ranks' copies; ring: three ring steps, update, and the
         # all-gather pinned to the ring's three copy steps (left alone the library takes its one-launch form at this world size)
@@ -455,17 +468,61 @@ def fsdp_rank(g, steps, prefetch):
             "gathers_per_step": n_gathers, "max_live": f.max_live, "live": f.live, "loss": float(loss.detach())}
 
 
+class FileBarrier:
+    """What Group asks of the launcher's barrier, for ranks that were started as separate commands (each under a
+    profiler of its own): every rank leaves a file and waits until all of them are there."""
+
+    def __init__(self, job, rank, size):
+        self.paths = [f"/dev/shm/tandem-bench-{job}-{r}.ready" for r in range(size)]
+        self.mine = self.paths[rank]
+
+    def wait(self, timeout=None):
+        open(self.mine, "w").close()
+        end = time.monotonic() + (timeout or 60.0)
+        while not all(os.path.exists(p) for p in self.paths):
+            if time.monotonic() > end:
+                raise TimeoutError("the other ranks did not start")
+            time.sleep(0.01)
+
+    def abort(self):
+        pass
+
+
+def fsdp_rank_alone(rank, world, job, steps):
+    """One rank of fsdp_gather's workload as a process of its own: `bench.py --fsdp-rank R --fsdp-job NAME`, started
+    once per rank (by hand, each under `rocprofv3 --kernel-trace`, say); TANDEM_HIP_GATHER picks where the gathers run."""
+    import torch
+
+    from tandem_amd import Group
+
+    torch.cuda.set_device(0)
+    barrier = FileBarrier(job, rank, world)
+    g = Group(rank, world, torch.device("cuda", 0), barrier, None, timeout=120.0, backend="hip", job=job)
+    try:
+        out = fsdp_rank(g, steps, True)
+        torch.cuda.synchronize()
+        g.close()
+    finally:
+        try:
+            os.unlink(barrier.mine)
+        except OSError:
+            pass
+    out["gather"] = os.environ.get("TANDEM_HIP_GATHER", "caller")
+    print(json.dumps({k: (round(v, 3) if isinstance(v, float) else v) for k, v in out.items()}), flush=True)
+
+
 def fsdp_gather(steps):
     """ZeRO-3's unit gathers: copies launched in order on the training stream (the
-    default), or on the engine's side stream, ordered against the training stream by value
-    words (one call per stream and dependency) or by events, with and without prefetch."""
+    default), or on the engine's side stream: started behind an event from a ring and ended by
+    a value word ("stream"), value words for both, or a fresh event for each; with and without prefetch."""
     from tandem_amd import launch
 
     out = {}
     before = os.environ.get("TANDEM_HIP_GATHER")
     try:
         for label, where, prefetch in (("in_order", "caller", True), ("side_stream_prefetch", "stream", True),
-                                       ("side_stream_events_prefetch", "stream-events", True),
+                                       ("side_stream_words_prefetch", "stream-words", True),
+                                       ("side_stream_fresh_events_prefetch", "stream-events", True),
                                        ("side_stream_no_prefetch", "stream", False)):
             os.environ["TANDEM_HIP_GATHER"] = where
             res = launch(fsdp_rank, 2, steps, prefetch, gpus=[0, 0], timeout=120.0)
@@ -791,11 +848,21 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-fsdp", action="store_true")
     ap.add_argument("--only", default="", help="comma list of single-process sections to run besides the main workload "
-                                               "(sweep, bucket, gather, zero2, mix), for short profiling runs; implies --no-cpu --no-fsdp")
+                                               "(sweep, bucket, gather, zero2, mix; fsdp: the two-process ZeRO-3 gather modes), for short profiling runs; "
+                                               "implies --no-cpu and none of the other two-process sections")
+    ap.add_argument("--fsdp-rank", type=int, default=-1, help="run ONE rank of the ZeRO-3 gather workload as this process "
+                                                              "(with --fsdp-job; start every rank yourself, e.g. each under a profiler)")
+    ap.add_argument("--fsdp-job", default="", help="a name the ranks started with --fsdp-rank share")
+    ap.add_argument("--fsdp-world", type=int, default=2)
     args = ap.parse_args()
+    if args.fsdp_rank >= 0:
+        if not args.fsdp_job or args.fsdp_rank >= args.fsdp_world:
+            sys.exit("--fsdp-rank needs --fsdp-job NAME and a rank below --fsdp-world")
+        fsdp_rank_alone(args.fsdp_rank, args.fsdp_world, args.fsdp_job, args.steps)
+        return
     only = {x for x in args.only.split(",") if x}
-    if only - {"sweep", "bucket", "gather", "zero2", "mix"}:
-        sys.exit("--only takes sweep, bucket, gather, zero2 and mix")
+    if only - {"sweep", "bucket", "gather", "zero2", "mix", "fsdp"}:
+        sys.exit("--only takes sweep, bucket, gather, zero2, mix and fsdp")
     if only:
         args.no_cpu = args.no_fsdp = True
     if args.gpus != 1:
@@ -810,6 +877,8 @@ def main():
         except Exception as e:  # reported, not measured by: the GPU figures must still come out
             cpu = {"error": repr(e)[:300]}
     ipc = train = train4 = None
+    if "fsdp" in only:
+        fsdp = fsdp_gather(8)
     if not args.quick and not args.no_fsdp:
         try:
             fsdp = fsdp_gather(8)

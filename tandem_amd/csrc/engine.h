@@ -212,8 +212,12 @@ class Engine {
   bool connected_ = false, closed_ = false;
   // staged collectives
   bool staged_ = true;               // TANDEM_HIP_ALGO=ring switches them off
-  bool gathers_on_side_stream_ = false;  // TANDEM_HIP_GATHER=stream (or stream-events)
-  bool gather_words_ = true;             // side-stream gathers are ordered by value words, not by events
+  bool gathers_on_side_stream_ = false;  // TANDEM_HIP_GATHER=stream (or stream-words, stream-events)
+  enum class GatherReady { kRingEvent, kWord, kFreshEvent };
+  GatherReady gather_ready_ = GatherReady::kRingEvent;  // what a side-stream gather waits for before its copies
+  bool gather_done_word_ = true;         // its end is a value word of the pool (else an event)
+  std::vector<hipEvent_t> ready_events_; // kRingEvent: made at start, used in turn by the callers' threads
+  std::atomic<uint64_t> ready_next_{0};
   std::shared_ptr<FlagPool> flags_;      // the words that tdm_work_wait_stream parks streams on
   bool want_flags_ = false;              // the device can make a stream wait for a value
   bool defer_default_ = false;           // TANDEM_HIP_WAIT=stream: tdm_work_wait parks as well

@@ -83,10 +83,13 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
     }
   }
   if (const char* gm = std::getenv("TANDEM_HIP_GATHER")) {
-    // "stream": on the engine's side stream, ordered against the caller's by value words where the device has them;
-    // "stream-events": the same with an event per dependency (what a device without such waits falls back to)
-    gathers_on_side_stream_ = std::string(gm) == "stream" || std::string(gm) == "stream-events";
-    gather_words_ = std::string(gm) != "stream-events";
+    // "stream": on the engine's side stream; it starts behind an event of the caller's stream (from a ring of events)
+    // and ends with a value word that wait() parks the caller's stream on. "stream-words": value words for both;
+    // "stream-events": a fresh event for each, created and destroyed per gather (what the path first did).
+    const std::string mode(gm);
+    gathers_on_side_stream_ = mode == "stream" || mode == "stream-words" || mode == "stream-events";
+    gather_ready_ = mode == "stream-words" ? GatherReady::kWord : mode == "stream-events" ? GatherReady::kFreshEvent : GatherReady::kRingEvent;
+    gather_done_word_ = mode != "stream-events";
   }
   if (const char* rd = std::getenv("TANDEM_HIP_READY")) ready_on_host_ = std::string(rd) != "gpu";
   peer_staging_.assign(size, nullptr);
@@ -104,6 +107,10 @@ void Engine::start() {
   check_hip(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags");  // default priority, all three
   if (want_flags_) flags_ = FlagPool::make();
   check_hip(hipStreamCreateWithFlags(&gather_stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags (gathers)");
+  if (gathers_on_side_stream_ && gather_ready_ == GatherReady::kRingEvent) {
+    ready_events_.assign(64, nullptr);
+    for (hipEvent_t& ev : ready_events_) check_hip(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "hipEventCreateWithFlags (ready ring)");
+  }
   check_hip(hipStreamCreateWithFlags(&anchor_stream_, hipStreamNonBlocking), "hipStreamCreateWithFlags (anchors)");
 
   mine_.create(region_name(rank_), size_);
@@ -234,6 +241,9 @@ void Engine::release_device() {
     if (*st) (void)hipStreamDestroy(*st);
     *st = nullptr;
   }
+  for (hipEvent_t ev : ready_events_)
+    if (ev) (void)hipEventDestroy(ev);
+  ready_events_.clear();
   for (void* a : arenas_) (void)hipFree(a);
   arenas_.clear();
   arena_sizes_.clear();
@@ -1103,13 +1113,16 @@ std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, st
   check_hip(hipSetDevice(device_), "hipSetDevice");
   hipStream_t on = caller;
   if (gathers_on_side_stream_) {
-    // Start once the caller's stream has produced the buffer (and finished with its last use). Where streams can write
-    // and wait for a value, that costs one call on each stream and a word of the engine's pool: the caller's stream
-    // writes the word when it gets here, the side stream waits for it. (An event for the same purpose is created,
-    // recorded, waited for and destroyed: four runtime calls of 13-31 us where these two take about 4 us each.)
+    // Start once the caller's stream has produced the buffer (and finished with its last use): the side stream waits
+    // for an event recorded on the caller's stream, taken from a ring made at start-up (no create and destroy per
+    // gather). A value word would do too (TANDEM_HIP_GATHER=stream-words: the caller's stream writes it, the side
+    // stream waits for it), but on this runtime a stream waits for a value with a kernel that spins, and with prefetch
+    // the side stream waits for most of a block's compute: twelve milliseconds of spinning per step, during which the
+    // matrix kernels beside it ran 11 % slower. The END of a gather is a value word either way (below): by the time the
+    // caller needs the unit the word is usually there and no wait is queued at all.
     on = gather_stream_;
     bool ordered = false;
-    if (flags_ && gather_words_) {
+    if (flags_ && gather_ready_ == GatherReady::kWord) {
       uint32_t value = 0;
       const int word = flags_->acquire(&value);
       if (word >= 0) {
@@ -1123,6 +1136,16 @@ std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, st
         check_hip(err, "ordering a gather after the caller's stream (value)");
         ordered = true;
       }
+    }
+    if (!ordered && gather_ready_ != GatherReady::kFreshEvent && !ready_events_.empty()) {
+      // An event out of a ring made at start-up: a wait takes the event's latest record at the time of the call, so
+      // recording it again for a later gather does not disturb a wait still queued (and the ring is far longer than
+      // the two or three gathers that are ever in flight).
+      hipEvent_t ready = ready_events_[ready_next_.fetch_add(1, std::memory_order_relaxed) % ready_events_.size()];
+      hipError_t err = hipEventRecord(ready, caller);
+      if (err == hipSuccess) err = hipStreamWaitEvent(gather_stream_, ready, 0);
+      check_hip(err, "ordering a gather after the caller's stream (event)");
+      ordered = true;
     }
     if (!ordered) {
       hipEvent_t ready;
@@ -1141,7 +1164,7 @@ std::shared_ptr<Work> Engine::unit_gather_direct(Buf full, const char* shard, st
   // the caller's stream on and done() reads (as for every collective of the progress thread). On the caller's own
   // stream nothing needs ordering afterwards: wait() finds the Work on the stream it would wait on. An event is
   // recorded only where there is no word, for done() on the caller's own stream, and for the time stamps.
-  if (gathers_on_side_stream_ && flags_ && gather_words_) {
+  if (gathers_on_side_stream_ && flags_ && gather_done_word_) {
     work->flag = flags_->acquire(&work->flag_value);
     if (work->flag >= 0) {
       work->flags = flags_;

@@ -27,6 +27,7 @@ CASES = [("2", "staged"), ("3", "staged"), ("4", "staged"), ("5", "staged"), ("8
          ("3", "staged", "0", "-", "TANDEM_HIP_GATHER=stream,TANDEM_HIP_READY=gpu,TANDEM_HIP_WAIT=stream"),
          ("2", "ring", "0", "-", "TANDEM_HIP_READY=gpu,TANDEM_HIP_WAIT=stream"),
          ("3", "staged", "0", "-", "TANDEM_HIP_GATHER=stream-events"), ("2", "staged", "0", "-", "TANDEM_HIP_GATHER=stream,FAKE_HIP_JITTER_US=200"),
+         ("3", "staged", "0", "-", "TANDEM_HIP_GATHER=stream-words,FAKE_HIP_JITTER_US=200"),
          # streams that lag behind the host by varying amounts (every piece of work on a stream starts up to 200 us late),
          # with staging windows of 4 KiB so that the two halves are reused many times
          ("3", "staged", "4096", "-", "FAKE_HIP_JITTER_US=200"), ("3", "ring", "0", "-", "FAKE_HIP_JITTER_US=200"),

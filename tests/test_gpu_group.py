@@ -287,11 +287,11 @@ def direct_gather(g, numel):
     return out
 
 
-@pytest.mark.parametrize("where", ["caller", "stream", "stream-events"])
+@pytest.mark.parametrize("where", ["caller", "stream", "stream-words", "stream-events"])
 @pytest.mark.parametrize("world", [2, 3])
 def test_direct_gather_from_shared_arenas(world, where, monkeypatch):
     """The copies run on the caller's own stream (default) or on a side stream of the engine, ordered against the
-    caller's stream by value words or by events."""
+    caller's stream by an event from a ring and a value word, by value words alone, or by fresh events."""
     from tandem_amd import launch
 
     monkeypatch.setenv("TANDEM_HIP_GATHER", where)

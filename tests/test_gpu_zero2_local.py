@@ -77,8 +77,9 @@ def test_small_model_bit_exact_with_oracle(world, algorithm):
         assert np.array_equal(bits(z.opts[r].state["flat"][2].cpu().numpy()), bits(opts[r].state["flat"][2]))
 
 
+@pytest.mark.parametrize("one_allocation", [False, True])
 @pytest.mark.parametrize("algorithm", ["fold", "ring", "fused"])
-def test_shards_that_start_off_the_16_byte_grid(algorithm):
+def test_shards_that_start_off_the_16_byte_grid(algorithm, one_allocation):
     """World 3 over a flat buffer of odd length: tensor_split puts the second and third shard
     1 and 2 elements past a multiple of four (tandem/zero.py:29-54 there: shards start
     anywhere). Gradient shards and optimizer state sit at their shard's phase, so every
@@ -88,8 +89,13 @@ def test_shards_that_start_off_the_16_byte_grid(algorithm):
     dev = torch.device("cuda", 0)
     world, numels = 3, [4099, 10_007, 33, 5001, 1, 12_288, 782]
     n = sum(numels)
-    z = LocalZeRO2(world, numels, dev, bucket_bytes=16 << 10, **KW)
+    z = LocalZeRO2(world, numels, dev, bucket_bytes=16 << 10, one_allocation=one_allocation, **KW)
     assert sorted(l.lo % 4 for l in z.layouts) == [0, 1, 2], [l.lo for l in z.layouts]
+    if one_allocation:  # every buffer inside the one pool, none overlapping
+        lo, hi = z._pool.data_ptr(), z._pool.data_ptr() + 4 * z._pool.numel()
+        parts = z.bufs + z.staging + z.grad_shards + [t for o in z.opts for t in o.state["flat"][1:]]
+        spans = sorted((t.data_ptr(), t.data_ptr() + 4 * t.numel()) for t in parts)
+        assert spans[0][0] >= lo and spans[-1][1] <= hi and all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
     for r, l in enumerate(z.layouts):  # the layout this test is about
         phase = z.bufs[r][l.lo:l.hi].data_ptr() % 128
         assert phase == 4 * (l.lo % 32)
