@@ -317,11 +317,36 @@ def unit_gather(dev, reps):
 
     t = timed(forward, reps) / units
     nbytes = 4 * (world + 1) * unit
-    return {"workload": "ZeRO-3 unit gather, 7,087,872 fp32 per unit, 2 buffer ranks, 12 units in turn, one launch for both ranks",
-            "us_per_unit": round(t * 1e6, 2), "algorithmic_bytes": nbytes, "GBps": round(nbytes / t / 1e9, 1),
-            "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4),
-            "roofline_floor_us": round(nbytes / (HBM_PEAK_GBPS * 1e9) * 1e6, 2),
-            "two_separate_gathers_equivalent_GBps": round(8 * unit * world / t / 1e9, 1)}
+    out = {"workload": "ZeRO-3 unit gather, 7,087,872 fp32 per unit, 2 buffer ranks, 12 units in turn, one launch for both ranks",
+           "us_per_unit": round(t * 1e6, 2), "algorithmic_bytes": nbytes, "GBps": round(nbytes / t / 1e9, 1),
+           "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4),
+           "roofline_floor_us": round(nbytes / (HBM_PEAK_GBPS * 1e9) * 1e6, 2),
+           "two_separate_gathers_equivalent_GBps": round(8 * unit * world / t / 1e9, 1)}
+    # What a launch this SHORT can reach at all: the stream-mix probe (no table, no arithmetic) reading one stream of the unit's
+    # size and writing two, over the same twelve sets of buffers in turn. A launch of 85 MB lasts about as long as it takes the
+    # grid to fill the machine and drain again, so the yardstick for it is this and not the rate of a long stream.
+    try:
+        import ctypes
+
+        from tandem_amd._lib import stream_ptr
+        from tandem_amd._probe import check, lib
+
+        sources = [torch.randn(unit, device=dev) for _ in range(units)]
+        st = stream_ptr(dev)
+        best = None
+        for shift in (0, 3):
+            def probes():
+                for k in range(units):
+                    rd = (ctypes.c_void_p * 8)(sources[k].data_ptr())
+                    wr = (ctypes.c_void_p * 8)(fulls[k][0].data_ptr(), fulls[k][1].data_ptr())
+                    check(lib().tdm_probe_stream_mix(rd, 1, wr, 2, unit * 4, 1, shift, 0, st))
+            tp = timed(probes, reps) / units
+            best = tp if best is None or tp < best else best
+        out["same_size_probe_1r_2w_us"] = round(best * 1e6, 2)
+        out["frac_of_mix_ceiling_at_this_size"] = round(best / t, 4)
+    except Exception as e:  # the probe library is optional
+        out["same_size_probe_error"] = repr(e)[:200]
+    return out
 
 
 def zero2_step(dev, reps):

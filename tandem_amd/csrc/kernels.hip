@@ -1278,7 +1278,10 @@ int tdm_k4_unit_gather_all(void* const* fulls, const void* const* shards, const 
     // Everything cached: what a gather writes is read by the unit's forward or backward straight away. (Twelve block units of
     // the 85.8M GPT gathered in turn at world 2: 19.4 us per unit with two vectors per lane, 18.8 with one; 17.6-18.0 with
     // non-temporal accesses, which would leave the consumer to fetch the unit from HBM.)
-    unit_gather_multicast(f, s, sizes, world, es, false, occupancy_pad(TDM_XCD_COPY, false), xcd_shift(TDM_XCD_COPY, world, false), 1,
+    // Tile order: runs of 8 tiles (16 KiB) per XCD unless the family's shift is set by hand. In the same sweep of 0..6 the plain
+    // order gave 18.8 us per block unit, every grouping from 4 tiles up 18.0-18.2.
+    const int set = g_xcd_shift[TDM_XCD_COPY].load(std::memory_order_relaxed);
+    unit_gather_multicast(f, s, sizes, world, es, false, occupancy_pad(TDM_XCD_COPY, false), set >= 0 ? set : 3, 1,
                           static_cast<int>(std::min<int64_t>(cap, int64_t(1) << 30)), st);
   });
 }
