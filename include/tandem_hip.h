@@ -272,6 +272,30 @@ int tdm_k3_adamw(float* p, const float* g, float* m, float* v, int64_t n, const 
 int tdm_k3_adamw_gather(float* p, const float* g, float* m, float* v, int64_t n, const tdm_adamw_scalars* s, int order,
                         float* const* copies, int ncopies, tdm_stream stream);
 
+/* The step's constants as the Python doubles of tandem/optim.py:28-37, unrounded: what an entry point that takes the
+ * shard's element type needs, since a Python double is applied to a tensor in the tensor's own arithmetic. */
+typedef struct tdm_adamw_hyper {
+  int32_t use_decay; /* weight_decay != 0 */
+  int32_t reserved;
+  double decay;      /* 1 - lr * weight_decay */
+  double w1;         /* 1 - beta1 */
+  double beta2;
+  double one_m_b2;   /* 1 - beta2 */
+  double bc2_sqrt;   /* (1 - beta2**t) ** 0.5 */
+  double eps;
+  double neg_step;   /* -(lr / (1 - beta1**t)) */
+} tdm_adamw_hyper;
+
+/* tdm_k3_adamw / tdm_k3_adamw_gather for shards of fp32 (TDM_F32), float64 (TDM_F64) or bfloat16 (TDM_BF16): the
+ * reference's update is seven torch operations that take any floating dtype (tandem/optim.py:28-37). `copies`
+ * may be NULL with ncopies 0. fp32: the constants are rounded to fp32 once and the call is tdm_k3_adamw(_gather),
+ * in either order. float64: the same operations on doubles, the constants unrounded. bfloat16: every one of the
+ * seven operations computes in fp32 and rounds its result to bf16 (nearest even), as ATen's kernels for bf16
+ * tensors do; eps is added rounded to bf16, the other constants act as fp32. float64 and bfloat16 follow torch's
+ * CPU kernels (TDM_ADAMW_HOST_ORDER); TDM_ADAMW_DEVICE_ORDER is refused for them. */
+int tdm_k3_adamw_typed(void* p, const void* g, void* m, void* v, int64_t n, int dtype, const tdm_adamw_hyper* h, int order,
+                       void* const* copies, int ncopies, tdm_stream stream);
+
 /* ---- K2 + K3: ZeRO-2's reduce-scatter, gradient add, AdamW and all-gather in one launch ---- */
 
 /* One segment: `count` elements that lie in ring chunk `chunk` (= the rank that owns

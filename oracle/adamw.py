@@ -1,9 +1,12 @@
-"""AdamW on a flat fp32 shard, on the CPU (TEST INFRASTRUCTURE ONLY).
+"""AdamW on a flat shard, on the CPU (TEST INFRASTRUCTURE ONLY).
 
 Follows tandem/optim.py:16-37: the scalars are computed in Python doubles
 exactly as written there and rounded to fp32 once when applied to the tensor,
 the way torch applies a Python scalar to a float tensor; the per-element
-arithmetic is oracle/tandem_oracle.c.
+arithmetic is oracle/tandem_oracle.c. fp32 shards are numpy float32 arrays;
+float64 shards numpy float64 arrays (the scalars stay doubles); bfloat16 shards
+are their bit patterns in numpy uint16 arrays with kind="bf16" (fp32 arithmetic,
+rounded to bf16 after each of the reference's torch operations).
 """
 
 import ctypes
@@ -37,9 +40,18 @@ def scalars(step, lr, betas, eps, weight_decay):
     }
 
 
-def _p(a):
-    assert a.dtype == np.float32 and a.flags.c_contiguous
+def _p(a, dtype=np.float32):
+    assert a.dtype == dtype and a.flags.c_contiguous
     return ctypes.c_void_p(a.ctypes.data)
+
+
+def scalars_f64(step, lr, betas, eps, weight_decay):
+    """The same constants for float64 shards: a Python double applied to a double tensor is not rounded."""
+    beta1, beta2 = betas
+    bias_correction1 = 1 - beta1 ** step
+    bias_correction2 = 1 - beta2 ** step
+    return {"use_decay": int(weight_decay != 0), "decay": 1 - lr * weight_decay, "w1": 1 - beta1, "beta2": beta2,
+            "one_m_b2": 1 - beta2, "bc2_sqrt": bias_correction2 ** 0.5, "eps": eps, "neg_step": -(lr / bias_correction1)}
 
 
 class AdamW:
@@ -50,10 +62,12 @@ class AdamW:
     (tests substitute torch's CPU sqrt to compare bit for bit with fixtures
     produced by torch)."""
 
-    def __init__(self, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, sqrt=None):
+    def __init__(self, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, sqrt=None, kind=None):
+        """kind: None (taken from the array: float32 or float64) or "bf16" for uint16 arrays of bfloat16 bit patterns."""
         self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
         self.state = {}
         self.sqrt = sqrt
+        self.kind = kind
 
     def update(self, key, param, grad):
         if key not in self.state:
@@ -64,6 +78,8 @@ class AdamW:
         n = param.size
         if n == 0:
             return
+        if self.kind == "bf16" or param.dtype == np.float64:
+            return self._update_other(param, grad, m, v, step, n)
         s = scalars(step, self.lr, self.betas, self.eps, self.weight_decay)
         f = ctypes.c_float
         L = lib()
@@ -77,6 +93,22 @@ class AdamW:
         root = np.ascontiguousarray(self.sqrt(v), dtype=np.float32)
         L.orc_adamw_apply_f32(_p(param), _p(m), _p(root), ctypes.c_int64(n), f(s["bc2_sqrt"]), f(s["eps"]),
                               f(s["neg_step"]))
+
+    def _update_other(self, param, grad, m, v, step, n):
+        L = lib()
+        if self.kind == "bf16":
+            s, f, dt, tag = scalars(step, self.lr, self.betas, self.eps, self.weight_decay), ctypes.c_float, np.uint16, "bf16"
+        else:
+            s, f, dt, tag = scalars_f64(step, self.lr, self.betas, self.eps, self.weight_decay), ctypes.c_double, np.float64, "f64"
+        head = (_p(param, dt), _p(grad, dt), _p(m, dt), _p(v, dt), ctypes.c_int64(n), ctypes.c_int(s["use_decay"]),
+                f(s["decay"]), f(s["w1"]), f(s["beta2"]), f(s["one_m_b2"]))
+        tail = (f(s["bc2_sqrt"]), f(s["eps"]), f(s["neg_step"]))
+        if self.sqrt is None:
+            getattr(L, f"orc_adamw_{tag}")(*head, *tail)
+            return
+        getattr(L, f"orc_adamw_moments_{tag}")(*head)
+        root = np.ascontiguousarray(self.sqrt(v), dtype=dt)
+        getattr(L, f"orc_adamw_apply_{tag}")(_p(param, dt), _p(m, dt), _p(root, dt), ctypes.c_int64(n), *tail)
 
     def state_bytes(self):
         return sum(a.nbytes + b.nbytes for _, a, b in self.state.values())

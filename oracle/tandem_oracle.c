@@ -183,3 +183,77 @@ void orc_adamw_f32(float* p, const float* g, float* m, float* v, int64_t n, int 
     p[i] = p[i] + (neg_step * m[i]) / d;
   }
 }
+
+/* ---- AdamW on float64 shards: the same operations on doubles (tandem/optim.py:28-37 takes any floating dtype).
+ * A Python double applied to a double tensor is used as it is, so the scalars arrive unrounded. lerp_ and
+ * addcmul_ fuse their last multiply-add on doubles as on floats, tensor / scalar is a true division,
+ * addcdiv_ is (value*m)/d then the add: checked operation by operation against torch's CPU kernels. */
+void orc_adamw_moments_f64(double* p, const double* g, double* m, double* v, int64_t n, int use_decay, double decay,
+                           double w1, double beta2, double one_m_b2) {
+  for (int64_t i = 0; i < n; ++i) {
+    if (use_decay) p[i] = p[i] * decay;
+    const double diff = g[i] - m[i];
+    m[i] = fabs(w1) < 0.5 ? fma(w1, diff, m[i]) : fma(w1 - 1.0, diff, g[i]);
+    const double vs = v[i] * beta2;
+    v[i] = fma(one_m_b2 * g[i], g[i], vs);
+  }
+}
+
+void orc_adamw_apply_f64(double* p, const double* m, const double* sqrt_v, int64_t n, double bc2_sqrt, double eps,
+                         double neg_step) {
+  for (int64_t i = 0; i < n; ++i) {
+    const double d = sqrt_v[i] / bc2_sqrt + eps;
+    p[i] = p[i] + (neg_step * m[i]) / d;
+  }
+}
+
+void orc_adamw_f64(double* p, const double* g, double* m, double* v, int64_t n, int use_decay, double decay, double w1,
+                   double beta2, double one_m_b2, double bc2_sqrt, double eps, double neg_step) {
+  orc_adamw_moments_f64(p, g, m, v, n, use_decay, decay, w1, beta2, one_m_b2);
+  for (int64_t i = 0; i < n; ++i) {
+    const double d = sqrt(v[i]) / bc2_sqrt + eps;
+    p[i] = p[i] + (neg_step * m[i]) / d;
+  }
+}
+
+/* ---- AdamW on bfloat16 shards (bit patterns). Every one of the torch operations of tandem/optim.py:28-37 reads
+ * bf16 tensors, computes in fp32 (ATen's opmath; the Python scalars rounded to fp32, not to bf16) and writes a bf16
+ * tensor, so the result is rounded to nearest even after EACH operation: p*decay; the lerp; v*beta2; the addcmul;
+ * the sqrt; the division; + eps; the addcdiv. One scalar is narrower than the others: add_(eps) adds eps ROUNDED TO
+ * BF16 (ATen wraps the scalar of an add in the tensor's dtype), where mul_, lerp_, addcmul_, the division and addcdiv_
+ * take theirs as fp32 (checked operation by operation against torch's CPU kernels on values where the two differ).
+ * Inside an operation the fp32 arithmetic is that of the fp32 kernels
+ * above. As for fp32 the step comes in two phases, so that a test can put torch's own bf16 square roots between them. */
+#define RB(x) bf16_to_f32(f32_to_bf16(x))
+void orc_adamw_moments_bf16(uint16_t* p, const uint16_t* g, uint16_t* m, uint16_t* v, int64_t n, int use_decay,
+                            float decay, float w1, float beta2, float one_m_b2) {
+  for (int64_t i = 0; i < n; ++i) {
+    const float G = bf16_to_f32(g[i]);
+    float M = bf16_to_f32(m[i]), V = bf16_to_f32(v[i]);
+    if (use_decay) p[i] = f32_to_bf16(bf16_to_f32(p[i]) * decay);
+    const float diff = G - M; /* inside lerp_: not rounded to bf16 */
+    m[i] = f32_to_bf16(fabsf(w1) < 0.5f ? fmaf(w1, diff, M) : fmaf(w1 - 1.0f, diff, G));
+    V = RB(V * beta2);
+    v[i] = f32_to_bf16(fmaf(one_m_b2 * G, G, V));
+  }
+}
+
+void orc_adamw_apply_bf16(uint16_t* p, const uint16_t* m, const uint16_t* sqrt_v, int64_t n, float bc2_sqrt, float eps,
+                          float neg_step) {
+  for (int64_t i = 0; i < n; ++i) {
+    float D = RB(bf16_to_f32(sqrt_v[i]) / bc2_sqrt);
+    D = RB(D + RB(eps));
+    p[i] = f32_to_bf16(bf16_to_f32(p[i]) + (neg_step * bf16_to_f32(m[i])) / D);
+  }
+}
+
+void orc_adamw_bf16(uint16_t* p, const uint16_t* g, uint16_t* m, uint16_t* v, int64_t n, int use_decay, float decay,
+                    float w1, float beta2, float one_m_b2, float bc2_sqrt, float eps, float neg_step) {
+  orc_adamw_moments_bf16(p, g, m, v, n, use_decay, decay, w1, beta2, one_m_b2);
+  for (int64_t i = 0; i < n; ++i) {
+    float D = RB(sqrtf(bf16_to_f32(v[i])));
+    D = RB(D / bc2_sqrt);
+    D = RB(D + RB(eps));
+    p[i] = f32_to_bf16(bf16_to_f32(p[i]) + (neg_step * bf16_to_f32(m[i])) / D);
+  }
+}

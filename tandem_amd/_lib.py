@@ -50,6 +50,12 @@ class AdamwScalars(ctypes.Structure):
                 ("eps", ctypes.c_float), ("neg_step", ctypes.c_float), ("inv_bc2_sqrt", ctypes.c_float)]
 
 
+class AdamwHyper(ctypes.Structure):
+    _fields_ = [("use_decay", ctypes.c_int32), ("reserved", ctypes.c_int32), ("decay", ctypes.c_double), ("w1", ctypes.c_double),
+                ("beta2", ctypes.c_double), ("one_m_b2", ctypes.c_double), ("bc2_sqrt", ctypes.c_double),
+                ("eps", ctypes.c_double), ("neg_step", ctypes.c_double)]
+
+
 _SIGNATURES = {
     "tdm_last_error": (ctypes.c_char_p, []),
     "tdm_abi_version": (ctypes.c_int, []),
@@ -86,6 +92,9 @@ _SIGNATURES = {
     "tdm_k3_adamw_gather": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                            ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.POINTER(ctypes.c_void_p),
                                            ctypes.c_int, ctypes.c_void_p]),
+    "tdm_k3_adamw_typed": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+                                          ctypes.c_int, ctypes.POINTER(AdamwHyper), ctypes.c_int, ctypes.POINTER(ctypes.c_void_p),
+                                          ctypes.c_int, ctypes.c_void_p]),
     "tdm_k23_table_tiles": (ctypes.c_int64, [ctypes.POINTER(StepSeg), ctypes.c_int]),
     "tdm_k23_table_bytes": (ctypes.c_int64, [ctypes.POINTER(StepSeg), ctypes.c_int]),
     "tdm_k23_table_build": (ctypes.c_int, [ctypes.POINTER(StepSeg), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),

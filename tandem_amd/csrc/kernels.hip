@@ -1125,6 +1125,97 @@ int tdm_k3_adamw_gather(float* p, const float* g, float* m, float* v, int64_t n,
   return guard([&] { adamw_launch(p, g, m, v, n, s, order, copies, ncopies, static_cast<hipStream_t>(stream)); });
 }
 
+extern "C++" {
+namespace {
+template <typename T>
+void adamw_typed_launch(void* p_, const void* g_, void* m_, void* v_, int64_t n, const tdm_adamw_hyper& h, void* const* copies,
+                        int ncopies, hipStream_t st) {
+  using S = typename AdamwMath<T>::S;
+  constexpr int es = static_cast<int>(sizeof(T));
+  uintptr_t ptrs[4 + TDM_MAX_WORLD - 1] = {reinterpret_cast<uintptr_t>(p_), reinterpret_cast<uintptr_t>(g_),
+                                           reinterpret_cast<uintptr_t>(m_), reinterpret_cast<uintptr_t>(v_)};
+  AdamwArgsT<T> a{};
+  a.p = static_cast<T*>(p_), a.g = static_cast<const T*>(g_), a.m = static_cast<T*>(m_), a.v = static_cast<T*>(v_);
+  a.n = n;
+  a.s.use_decay = h.use_decay;
+  a.s.decay = static_cast<S>(h.decay), a.s.w1 = static_cast<S>(h.w1), a.s.beta2 = static_cast<S>(h.beta2);
+  a.s.one_m_b2 = static_cast<S>(h.one_m_b2), a.s.bc2_sqrt = static_cast<S>(h.bc2_sqrt), a.s.neg_step = static_cast<S>(h.neg_step);
+  a.s.eps = static_cast<S>(h.eps);
+  if constexpr (std::is_same_v<T, bf16_t>) {  // add_(eps) on a bf16 tensor adds eps rounded to bf16 (nearest even)
+    uint32_t u;
+    const float e = static_cast<float>(h.eps);
+    std::memcpy(&u, &e, 4);
+    u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+    float rounded;
+    std::memcpy(&rounded, &u, 4);
+    a.s.eps = rounded;
+  }
+  a.ncopies = ncopies;
+  a.shift = xcd_shift(TDM_XCD_ADAMW, 1, true);
+  for (int c = 0; c < ncopies; ++c) {
+    if (!copies[c]) throw Invalid("NULL copy of the parameters");
+    a.copy[c] = static_cast<T*>(copies[c]);
+    ptrs[4 + c] = reinterpret_cast<uintptr_t>(copies[c]);
+  }
+  for (int i = 0; i < 4 + ncopies; ++i)
+    if (ptrs[i] % es) throw Invalid("pointer not aligned to the element size");
+  for (int i = 0; i < 4 + ncopies; ++i)
+    for (int j = i + 1; j < 4 + ncopies; ++j) {
+      const uintptr_t bytes = static_cast<uintptr_t>(n) * es;
+      if (ptrs[i] < ptrs[j] + bytes && ptrs[j] < ptrs[i] + bytes) throw Invalid("p, g, m, v and the copies must not overlap");
+    }
+  const SegPlan plan = plan_segment(ptrs, 4 + ncopies, n, es, static_cast<int64_t>(kAdamwThreads) * (16 / es));
+  const bool vec = plan.vec;
+  if (vec) {  // as for fp32: the head is stretched to the cache line when every stream agrees on it
+    int64_t head = plan.head;
+    const uintptr_t line = (ptrs[0] + head * es) % 128;
+    bool same = true;
+    for (int i = 1; i < 4 + ncopies; ++i) same = same && (ptrs[i] + head * es) % 128 == line;
+    const int64_t more = static_cast<int64_t>((128 - line) % 128) / es;
+    if (same && more < plan.body) head += more;
+    a.p += head, a.g += head, a.m += head, a.v += head;
+    for (int c = 0; c < ncopies; ++c) a.copy[c] += head;
+    a.n = n - head;
+    a.head = static_cast<int>(head);
+  }
+  const int64_t per = vec ? static_cast<int64_t>(kAdamwThreads) * (16 / es) : kAdamwThreads;
+  const dim3 grid(grid_for(std::max<int64_t>((a.n + per - 1) / per, 1))), block(kAdamwThreads);
+  const unsigned pad = occupancy_pad(TDM_XCD_ADAMW);
+  switch ((vec ? 2 : 0) + (ncopies > 0 ? 1 : 0)) {
+    case 0: hipLaunchKernelGGL((k3_adamw_typed_kernel<T, false, false>), grid, block, pad, st, a); break;
+    case 1: hipLaunchKernelGGL((k3_adamw_typed_kernel<T, false, true>), grid, block, pad, st, a); break;
+    case 2: hipLaunchKernelGGL((k3_adamw_typed_kernel<T, true, false>), grid, block, pad, st, a); break;
+    default: hipLaunchKernelGGL((k3_adamw_typed_kernel<T, true, true>), grid, block, pad, st, a); break;
+  }
+  check_hip(hipGetLastError(), "k3_adamw (typed) launch");
+}
+}  // namespace
+}  // extern "C++"
+
+int tdm_k3_adamw_typed(void* p, const void* g, void* m, void* v, int64_t n, int dtype, const tdm_adamw_hyper* h, int order,
+                       void* const* copies, int ncopies, tdm_stream stream) {
+  return guard([&] {
+    if (n < 0) throw Invalid("n is negative");
+    if (ncopies < 0 || ncopies > TDM_MAX_WORLD - 1) throw Invalid("at most 7 further copies of the parameters");
+    if (dtype != TDM_F32 && dtype != TDM_F64 && dtype != TDM_BF16) throw Invalid("AdamW handles fp32, fp64 and bf16 shards (dtype " + std::to_string(dtype) + ")");
+    if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
+    if (n == 0) return;
+    if (!p || !g || !m || !v || !h || (ncopies > 0 && !copies)) throw Invalid("NULL argument");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == TDM_F32) {  // a Python double applied to a float tensor is rounded to fp32 once
+      tdm_adamw_scalars s{h->use_decay, static_cast<float>(h->decay), static_cast<float>(h->w1), static_cast<float>(h->beta2),
+                          static_cast<float>(h->one_m_b2), static_cast<float>(h->bc2_sqrt), static_cast<float>(h->eps),
+                          static_cast<float>(h->neg_step), static_cast<float>(1.0 / h->bc2_sqrt)};
+      adamw_launch(static_cast<float*>(p), static_cast<const float*>(g), static_cast<float*>(m), static_cast<float*>(v), n, &s, order,
+                   reinterpret_cast<float* const*>(copies), ncopies, st);
+      return;
+    }
+    if (order != TDM_ADAMW_HOST_ORDER) throw Invalid("the device order is defined for fp32 shards only");
+    if (dtype == TDM_F64) adamw_typed_launch<double>(p, g, m, v, n, *h, copies, ncopies, st);
+    else adamw_typed_launch<bf16_t>(p, g, m, v, n, *h, copies, ncopies, st);
+  });
+}
+
 int64_t tdm_k23_table_tiles(const tdm_step_seg* segs, int nseg) {
   if (nseg < 0 || (nseg > 0 && segs == nullptr)) return -1;
   return step_tiles(segs, nseg);

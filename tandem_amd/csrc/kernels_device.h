@@ -785,6 +785,110 @@ __global__ __launch_bounds__(kAdamwThreads) void k3_adamw_kernel(AdamwArgs a) {
   }
 }
 
+// ---------------------------------------------------------------- K3 on other element types
+// The reference's update is seven torch operations that take any floating dtype (tandem/optim.py:28-37).
+// float64: the same arithmetic on doubles, the step's scalars unrounded. bfloat16: every operation reads
+// bf16, computes in fp32 and writes bf16, so the value is rounded to nearest even after EACH operation;
+// add_(eps) adds eps rounded to bf16 (ATen wraps that scalar in the tensor's dtype), the other scalars act
+// as fp32. Host order only: these follow torch's CPU kernels, which is what the reference's engine runs.
+template <typename S>
+struct AdamwHyper {
+  int use_decay;
+  S decay, w1, beta2, one_m_b2, bc2_sqrt, eps, neg_step;
+};
+
+template <typename T> struct AdamwMath;
+
+template <> struct AdamwMath<double> {
+  using S = double;
+  static __device__ __forceinline__ void step(double& p, double g, double& m, double& v, const AdamwHyper<double>& s, bool small_w) {
+    if (s.use_decay) p = p * s.decay;
+    const double diff = g - m;
+    m = small_w ? __builtin_fma(s.w1, diff, m) : __builtin_fma(s.w1 - 1.0, diff, g);
+    const double vs = v * s.beta2;
+    v = __builtin_fma(s.one_m_b2 * g, g, vs);
+    const double d = __builtin_sqrt(v) / s.bc2_sqrt + s.eps;
+    p = p + (s.neg_step * m) / d;
+  }
+};
+
+template <> struct AdamwMath<bf16_t> {
+  using S = float;
+  static __device__ __forceinline__ float rb(float x) { return Elem<bf16_t>::widen(Elem<bf16_t>::narrow(x)); }
+  static __device__ __forceinline__ void step(bf16_t& p, bf16_t g, bf16_t& m, bf16_t& v, const AdamwHyper<float>& s, bool small_w) {
+    float P = Elem<bf16_t>::widen(p), M = Elem<bf16_t>::widen(m), V = Elem<bf16_t>::widen(v);
+    const float G = Elem<bf16_t>::widen(g);
+    if (s.use_decay) P = rb(P * s.decay);
+    const float diff = G - M;  // inside lerp_: not rounded
+    M = rb(small_w ? __builtin_fmaf(s.w1, diff, M) : __builtin_fmaf(s.w1 - 1.0f, diff, G));
+    V = rb(V * s.beta2);
+    V = rb(__builtin_fmaf(s.one_m_b2 * G, G, V));
+    float D = rb(__builtin_sqrtf(V));
+    D = rb(D / s.bc2_sqrt);
+    D = rb(D + s.eps);  // s.eps arrives rounded to bf16
+    P = rb(P + (s.neg_step * M) / D);
+    p = Elem<bf16_t>::narrow(P);
+    m = Elem<bf16_t>::narrow(M);
+    v = Elem<bf16_t>::narrow(V);
+  }
+};
+
+template <typename T>
+struct AdamwArgsT {
+  T* p;
+  const T* g;
+  T* m;
+  T* v;
+  int64_t n;
+  AdamwHyper<typename AdamwMath<T>::S> s;
+  int ncopies;
+  int shift;  // of tile_of()
+  int head;   // vector path: elements before the pointers (up to a cache line), peeled off an unaligned shard
+  T* copy[TDM_MAX_WORLD - 1];
+};
+
+template <typename T, bool kVec, bool kCopies>
+__global__ __launch_bounds__(kAdamwThreads) void k3_adamw_typed_kernel(AdamwArgsT<T> a) {
+  using S = typename AdamwMath<T>::S;
+  const bool small_w = (a.s.w1 < S(0) ? -a.s.w1 : a.s.w1) < S(0.5);
+  constexpr int kL = lanes<T>();
+  if constexpr (kVec) {
+    const int64_t nv = a.n / kL;
+    const int64_t tiles = (nv + kAdamwThreads - 1) / kAdamwThreads;
+    for (int64_t at = blockIdx.x; at < tiles; at += gridDim.x) {
+      const int64_t i = tile_of(at, tiles, a.shift) * kAdamwThreads + threadIdx.x;
+      if (i < nv) {
+        Lanes<T> P = unpack<T>(load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.p) + i * 16));
+        const Lanes<T> G = unpack<T>(load_stream<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.g) + i * 16));
+        Lanes<T> M = unpack<T>(load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.m) + i * 16));
+        Lanes<T> V = unpack<T>(load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.v) + i * 16));
+#pragma unroll
+        for (int l = 0; l < kL; ++l) AdamwMath<T>::step(P.v[l], G.v[l], M.v[l], V.v[l], a.s, small_w);
+        const vec16 packed = pack<T>(P);
+        store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.p) + i * 16, packed);
+        if constexpr (kCopies)
+          for (int c = 0; c < a.ncopies; ++c) store16<TDM_NT_MASK_K3C>(reinterpret_cast<char*>(a.copy[c]) + i * 16, packed);
+        store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.m) + i * 16, pack<T>(M));
+        store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.v) + i * 16, pack<T>(V));
+      }
+    }
+    // the last few elements (lanes 0..7), and the head before the first vector (lanes 32..): up to a cache line
+    if (blockIdx.x == 0 && (threadIdx.x < a.n - nv * kL || (threadIdx.x >= 32 && static_cast<int>(threadIdx.x) - 32 < a.head))) {
+      const int64_t i = threadIdx.x < 32 ? nv * kL + threadIdx.x : -1 - (static_cast<int64_t>(threadIdx.x) - 32);
+      AdamwMath<T>::step(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
+      if constexpr (kCopies)
+        for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
+    }
+  } else {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kAdamwThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kAdamwThreads + threadIdx.x; i < a.n; i += stride) {
+      AdamwMath<T>::step(a.p[i], a.g[i], a.m[i], a.v[i], a.s, small_w);
+      if constexpr (kCopies)
+        for (int c = 0; c < a.ncopies; ++c) a.copy[c][i] = a.p[i];
+    }
+  }
+}
+
 // ---------------------------------------------------------------- K2 + K3: ZeRO-2's whole step
 // For every element of every bucket segment, in one launch: the gradients of all ranks
 // are folded in the ring's order for the segment's chunk (K2), the sum is added to a zero

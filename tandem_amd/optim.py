@@ -1,17 +1,22 @@
-"""AdamW on flat fp32 shards of the parameters, for the ZeRO stages: one fused
-HIP kernel per shard instead of seven elementwise passes.
+"""AdamW on flat shards of the parameters, for the ZeRO stages: one fused HIP
+kernel per shard instead of seven elementwise passes.
 
 Same interface as tandem's ShardedAdamW (tandem/optim.py:11-40 there) and the
 same arithmetic, operation for operation: the step's scalars are computed in
-Python doubles by the same expressions and rounded to fp32 once, as torch does
-when it applies a Python scalar to a float tensor; the per-element work is
-tdm_k3_adamw."""
+Python doubles by the same expressions and applied in the shard's own
+arithmetic, as torch does with a Python scalar. fp32 shards: the scalars are
+rounded to fp32 once (tdm_k3_adamw). float64: doubles throughout. bfloat16:
+each of the seven operations computes in fp32 and rounds to bf16
+(tdm_k3_adamw_typed)."""
 
 import ctypes
 
 import torch
 
-from ._lib import ADAMW_DEVICE_ORDER, ADAMW_HOST_ORDER, AdamwScalars, check, lib, require_device_tensor, stream_ptr
+from ._lib import (ADAMW_DEVICE_ORDER, ADAMW_HOST_ORDER, AdamwHyper, AdamwScalars, check, dtype_code, lib, require_device_tensor,
+                   stream_ptr)
+
+SHARD_DTYPES = (torch.float32, torch.float64, torch.bfloat16)
 
 
 def step_scalars(step, lr, betas, eps, weight_decay):
@@ -51,6 +56,23 @@ def zeros_at_phase_of(like, numel=None):
     return store[lead:lead + n]
 
 
+def step_hyper(step, lr, betas, eps, weight_decay):
+    """The same constants as Python doubles, unrounded, for the entry point that takes the shard's element type."""
+    beta1, beta2 = betas
+    bias_correction1 = 1 - beta1 ** step
+    bias_correction2 = 1 - beta2 ** step
+    h = AdamwHyper()
+    h.use_decay = int(weight_decay != 0)
+    h.decay = 1 - lr * weight_decay
+    h.w1 = 1 - beta1
+    h.beta2 = beta2
+    h.one_m_b2 = 1 - beta2
+    h.bc2_sqrt = bias_correction2 ** 0.5
+    h.eps = eps
+    h.neg_step = -(lr / bias_correction1)
+    return h
+
+
 class ShardedAdamW:
     """order="host" reproduces torch's CPU addcdiv_ (p + (step*m)/d), which is
     what the reference's CPU engine computes; order="device" reproduces torch's
@@ -66,8 +88,9 @@ class ShardedAdamW:
         lib()
 
     def update(self, key, param, grad, copies=()):
-        """One step for one shard: `param` and `grad` are same-shaped fp32
-        tensors in GPU memory; `key` names the shard's optimizer state. `copies`:
+        """One step for one shard: `param` and `grad` are same-shaped tensors in GPU
+        memory, fp32, float64 or bfloat16 (the last two in host order only);
+        `key` names the shard's optimizer state. `copies`:
         further tensors of the same shape (the other ranks' copies of this shard, when
         the ranks are buffers in one memory) that receive the updated parameters in the
         same pass, which makes the all-gather after the step unnecessary."""
@@ -75,10 +98,12 @@ class ShardedAdamW:
         require_device_tensor(grad, "ShardedAdamW.update(grad)")
         for c in copies:
             require_device_tensor(c, "ShardedAdamW.update(copies)")
-            if c.dtype != torch.float32 or c.shape != param.shape:
+            if c.dtype != param.dtype or c.shape != param.shape:
                 raise ValueError("a copy differs from param in dtype or shape")
-        if param.dtype != torch.float32 or grad.dtype != torch.float32:
-            raise ValueError("ShardedAdamW handles fp32 shards")
+        if param.dtype not in SHARD_DTYPES or grad.dtype != param.dtype:
+            raise ValueError(f"ShardedAdamW handles fp32, float64 and bfloat16 shards whose gradient has the same dtype (got {param.dtype}, {grad.dtype})")
+        if param.dtype != torch.float32 and self.order != ADAMW_HOST_ORDER:
+            raise ValueError("order=\"device\" is defined for fp32 shards only")
         if param.shape != grad.shape:
             raise ValueError("param and grad differ in shape")
         if key not in self.state:
@@ -87,6 +112,14 @@ class ShardedAdamW:
         st[0] += 1.0
         step, exp_avg, exp_avg_sq = st
         if param.numel() == 0:
+            return
+        if param.dtype != torch.float32:
+            h = step_hyper(step, self.lr, self.betas, self.eps, self.weight_decay)
+            arr = (ctypes.c_void_p * max(1, len(copies)))(*[c.data_ptr() for c in copies])
+            check(lib().tdm_k3_adamw_typed(ctypes.c_void_p(param.data_ptr()), ctypes.c_void_p(grad.data_ptr()),
+                                           ctypes.c_void_p(exp_avg.data_ptr()), ctypes.c_void_p(exp_avg_sq.data_ptr()),
+                                           param.numel(), dtype_code(param.dtype), ctypes.byref(h), self.order, arr, len(copies),
+                                           stream_ptr(param.device)))
             return
         s = step_scalars(step, self.lr, self.betas, self.eps, self.weight_decay)
         if copies:
@@ -106,7 +139,7 @@ class ShardedAdamW:
         returns (scalars, exp_avg, exp_avg_sq, order) for it."""
         require_device_tensor(param, "ShardedAdamW.begin_step(param)")
         if param.dtype != torch.float32:
-            raise ValueError("ShardedAdamW handles fp32 shards")
+            raise ValueError("the fused ZeRO-2 step handles fp32 shards (update() also takes float64 and bfloat16)")
         if key not in self.state:
             self.state[key] = [0.0, zeros_at_phase_of(param), zeros_at_phase_of(param)]
         st = self.state[key]

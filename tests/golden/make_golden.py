@@ -3,7 +3,7 @@ implementation (tandem's Python engine, CPU processes) on small seeded inputs.
 
 Run once, in the build container only, where the reference is mounted:
 
-    python tests/golden/make_golden.py [/root/reference]
+    python tests/golden/make_golden.py [/root/reference] [only: ring adamw adamw_dtypes plans data train]
 
 The fixtures are data only (inputs, expected outputs, digests). They pin the
 parts of the path that no test of the reference pins by itself:
@@ -14,6 +14,8 @@ parts of the path that no test of the reference pins by itself:
                       the partial sums left in the other chunks; all_gather).
   ring_dtypes_w3.npz  fp64 / fp16 / bf16 all_reduce at world 3.
   adamw.npz           ShardedAdamW.update, 20 steps, the benchmark's hyper-parameters.
+  adamw_dtypes.npz    the same update on bfloat16 and float64 shards (the reference's seven
+                      torch operations take any floating dtype), both lerp branches.
   plans.json          DDP / ZeRO bucket packing, shard sizes, bucket_sizes and the
                       GPT's parameter registration order and unit sizes.
   data.json           digests of synthetic() and Text.batch().
@@ -164,6 +166,42 @@ def write_adamw():
     np.savez_compressed(os.path.join(HERE, "adamw.npz"), **out)
 
 
+def write_adamw_dtypes():
+    """ShardedAdamW.update on bf16 and f64 tensors: 20 steps with the benchmark's hyper-parameters, and 3 steps
+    of the other branches (beta1 < 0.5, no weight decay). 16-bit tensors are stored as bit patterns."""
+    n, steps = 773, 20
+    torch.set_num_threads(1)
+    out = {}
+
+    def raw(t):
+        return (t.view(torch.int16) if t.element_size() == 2 else t).numpy().copy()
+
+    hyper = {"main": {"lr": 3e-4, "betas": [0.9, 0.95], "eps": 1e-8, "weight_decay": 0.1, "steps": steps},
+             "other": {"lr": 1e-2, "betas": [0.3, 0.7], "eps": 1e-6, "weight_decay": 0.0, "steps": 3}}
+    for name, dt in (("bf16", torch.bfloat16), ("f64", torch.float64)):
+        g = torch.Generator().manual_seed(21)
+        p0 = (torch.randn(n, generator=g, dtype=torch.float64) * 0.02).to(dt)
+        p0[:4] = torch.tensor([0.0, -0.0, 1e-30, -3e-39], dtype=torch.float64).to(dt)
+        grads = []
+        for s in range(steps):
+            gr = (torch.randn(n, generator=torch.Generator().manual_seed(200 + s), dtype=torch.float64) * 1e-3).to(dt)
+            gr[:2] = 0.0
+            grads.append(gr)
+        out[f"{name}_p0"] = raw(p0)
+        out[f"{name}_grads"] = np.stack([raw(gr) for gr in grads])
+        for case, h in hyper.items():
+            p = p0.clone()
+            opt = ShardedAdamW(lr=h["lr"], betas=tuple(h["betas"]), eps=h["eps"], weight_decay=h["weight_decay"])
+            for s in range(h["steps"]):
+                opt.update("k", p, grads[s])
+                if s in (0, h["steps"] - 1):
+                    _, m, v = opt.state["k"]
+                    assert m.dtype == dt and v.dtype == dt
+                    out[f"{name}_{case}_p{s + 1}"], out[f"{name}_{case}_m{s + 1}"], out[f"{name}_{case}_v{s + 1}"] = raw(p), raw(m), raw(v)
+    out["hyper_json"] = np.frombuffer(json.dumps(hyper).encode(), dtype=np.uint8)
+    np.savez_compressed(os.path.join(HERE, "adamw_dtypes.npz"), **out)
+
+
 def names_of(model):
     return {p: n for n, p in model.named_parameters()}
 
@@ -287,9 +325,9 @@ def write_train():
 
 
 if __name__ == "__main__":
-    write_ring()
-    write_adamw()
-    write_plans()
-    write_data()
-    write_train()
-    print("golden fixtures written to", HERE)
+    writers = {"ring": write_ring, "adamw": write_adamw, "adamw_dtypes": write_adamw_dtypes, "plans": write_plans,
+               "data": write_data, "train": write_train}
+    only = sys.argv[2:] or list(writers)
+    for name in only:
+        writers[name]()
+    print("golden fixtures", only, "written to", HERE)

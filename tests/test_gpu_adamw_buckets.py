@@ -217,6 +217,92 @@ def test_optimizer_state_follows_the_shards_phase(dev):
     assert zeros_at_phase_of(half).data_ptr() % 128 == half.data_ptr() % 128 and zeros_at_phase_of(half, 5).numel() == 5
 
 
+def _raw(t):
+    t = t.detach().cpu()
+    return t.view(torch.int16).numpy().view(np.uint16).copy() if t.element_size() == 2 else t.numpy().copy()
+
+
+@pytest.mark.parametrize("case", ["main", "other"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float64])
+def test_adamw_bf16_and_f64_against_the_reference_fixture(dev, dtype, case):
+    """tests/golden/adamw_dtypes.npz: the reference's ShardedAdamW on bfloat16 and float64 shards, 20 steps of
+    the benchmark's hyper-parameters and 3 steps of the other branches. Against the fixture: bfloat16 bit for
+    bit in p, m, v; float64 bit for bit in the moments and within 1 ulp of each step's update term in p (the
+    reference ran torch's vectorised CPU sqrt, which is not correctly rounded). Against the oracle (pinned by
+    the same fixture with torch's sqrt substituted): bit for bit in everything."""
+    from oracle.adamw import AdamW as Oracle
+    from tandem_amd import ShardedAdamW
+
+    name = "bf16" if dtype == torch.bfloat16 else "f64"
+    d = golden_npz("adamw_dtypes.npz")
+    h = npz_json(d, "hyper_json")[case]
+    kw = dict(lr=h["lr"], betas=tuple(h["betas"]), eps=h["eps"], weight_decay=h["weight_decay"])
+    last = h["steps"]
+
+    def dev_tensor(a):
+        t = torch.from_numpy(np.ascontiguousarray(a).copy())
+        return (t.view(torch.bfloat16) if name == "bf16" else t).to(dev)
+
+    ours, ref = ShardedAdamW(**kw), Oracle(**kw, kind="bf16" if name == "bf16" else None)
+    p = dev_tensor(d[f"{name}_p0"])
+    pn = (d[f"{name}_p0"].view(np.uint16) if name == "bf16" else d[f"{name}_p0"]).copy()
+    for s in range(last):
+        g = d[f"{name}_grads"][s]
+        ours.update("k", p, dev_tensor(g))
+        ref.update("k", pn, np.ascontiguousarray(g.view(np.uint16) if name == "bf16" else g))
+    _, m, v = ours.state["k"]
+    assert m.dtype == dtype and v.dtype == dtype
+    assert np.array_equal(bits(_raw(m)), bits(ref.state["k"][1])) and np.array_equal(bits(_raw(v)), bits(ref.state["k"][2]))
+    assert np.array_equal(bits(_raw(p)), bits(pn))
+    assert np.array_equal(bits(_raw(m)), bits(d[f"{name}_{case}_m{last}"]))
+    assert np.array_equal(bits(_raw(v)), bits(d[f"{name}_{case}_v{last}"]))
+    want = d[f"{name}_{case}_p{last}"]
+    if name == "bf16":
+        assert np.array_equal(bits(_raw(p)), bits(want))
+    else:
+        assert np.abs(_raw(p) - want).max() <= last * 2 * np.spacing(h["lr"])
+        assert (bits(_raw(p)) != bits(want)).mean() < 0.05
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float64])
+def test_adamw_bf16_and_f64_on_odd_shards_with_copies(dev, dtype):
+    """The typed kernel's vector path (8 bf16 or 2 doubles per 16 bytes), its peeled head (up to a cache line),
+    its tail, the element-by-element path for streams that disagree, and the copies written in the same pass:
+    three steps against the oracle, guard elements untouched."""
+    from oracle.adamw import AdamW as Oracle
+    from tandem_amd import ShardedAdamW
+
+    kw = dict(lr=1e-3, betas=(0.9, 0.95), eps=1e-6, weight_decay=0.1)
+    gen = torch.Generator().manual_seed(31)
+    per_line = 128 // torch.empty(0, dtype=dtype).element_size()
+    for n in (1, 7, 9, 63, 65, 4099, 50_001):
+        p0 = (torch.randn(n, generator=gen, dtype=torch.float64) * 0.02).to(dtype)
+        grads = [(torch.randn(n, generator=gen, dtype=torch.float64) * 1e-3).to(dtype) for _ in range(3)]
+        ref = Oracle(**kw, kind="bf16" if dtype == torch.bfloat16 else None)
+        pn = _raw(p0)
+        for g in grads:
+            ref.update("k", pn, _raw(g))
+        for phases, ncopies in (([0, 0, 0, 0], 0), ([1, 1, 1, 1, 1, 1], 2), ([per_line - 1] * 5, 1), ([3, 3 + 8, 3, 3 + 16], 0), ([1, 0, 2, 1], 0)):
+            pad = 2 * per_line
+            stores = [torch.full((n + 2 * pad,), -7.0, dtype=dtype, device=dev) for _ in range(4 + ncopies)]
+            views = [s_[pad + ph:pad + ph + n] for s_, ph in zip(stores, phases)]
+            p, g, copies = views[0], views[1], views[4:]
+            p.copy_(p0)
+            ours = ShardedAdamW(**kw)
+            ours.state["k"] = [0.0, views[2].zero_(), views[3].zero_()]
+            for gr in grads:
+                g.copy_(gr)
+                ours.update("k", p, g, copies)
+            what = (dtype, n, phases)
+            assert np.array_equal(bits(_raw(p)), bits(pn)), what
+            assert np.array_equal(bits(_raw(views[2])), bits(ref.state["k"][1])), what
+            assert np.array_equal(bits(_raw(views[3])), bits(ref.state["k"][2])), what
+            for c in copies:
+                assert np.array_equal(bits(_raw(c)), bits(pn)), what
+            for s_, ph in zip(stores, phases):
+                assert float((s_[:pad + ph].double() + 7.0).abs().sum()) == 0 and float((s_[pad + ph + n:].double() + 7.0).abs().sum()) == 0, what
+
+
 def test_adamw_rejects_what_it_cannot_do(dev):
     from tandem_amd import ShardedAdamW
 
@@ -225,6 +311,10 @@ def test_adamw_rejects_what_it_cannot_do(dev):
         opt.update("cpu", torch.zeros(4), torch.zeros(4))
     with pytest.raises(ValueError):
         opt.update("half", torch.zeros(4, device=dev, dtype=torch.float16), torch.zeros(4, device=dev, dtype=torch.float16))
+    with pytest.raises(ValueError, match="same dtype"):
+        opt.update("mixed", torch.zeros(4, device=dev, dtype=torch.bfloat16), torch.zeros(4, device=dev))
+    with pytest.raises(ValueError, match="fp32 shards only"):
+        ShardedAdamW(order="device").update("d", torch.zeros(4, device=dev, dtype=torch.float64), torch.ones(4, device=dev, dtype=torch.float64))
     opt.update("empty", torch.zeros(0, device=dev), torch.zeros(0, device=dev))
     assert opt.state["empty"][0] == 1.0
     p = torch.zeros(8, device=dev)

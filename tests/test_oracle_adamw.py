@@ -3,6 +3,7 @@ against torch.optim.AdamW(foreach=False) (what the reference itself is tested
 against), and against a float64 evaluation of the textbook formulas."""
 
 import numpy as np
+import pytest
 import torch
 
 from oracle.adamw import AdamW, scalars
@@ -175,3 +176,77 @@ def test_cpu_baseline_optimizer_is_the_same_update():
         assert np.array_equal(bits(timed_one.state["k"]["v"].numpy()), bits(checker.state["k"][2]))
         timed_one.update("empty", torch.zeros(0), torch.zeros(0))
         assert timed_one.state["empty"]["t"] == 1.0
+
+
+def _raw16(t):
+    return t.view(torch.int16).numpy().view(np.uint16).copy()
+
+
+@pytest.mark.parametrize("case", ["main", "other"])
+def test_bf16_and_f64_match_the_reference_fixture(case):
+    """tests/golden/adamw_dtypes.npz: the reference's ShardedAdamW on bfloat16 and float64 shards (its seven torch
+    operations take any floating dtype, tandem/optim.py:28-37), 20 steps with the benchmark's hyper-parameters and
+    3 steps of the other branches (beta1 < 0.5, no decay). bfloat16: parameters and both moments bit for bit (fp32
+    arithmetic, rounded to bf16 after each operation; torch's fp32 sqrt being 1 ulp off changes a bf16 result about
+    once in five million elements). float64: both moments bit for bit; the parameters bit for bit with torch's own
+    CPU sqrt substituted, and within 1 ulp of each step's update term with the correctly rounded one (torch's
+    vectorised double sqrt is off by one ulp on about 0.7 % of inputs, as its float sqrt is)."""
+    from helpers import golden_npz, npz_json
+
+    d = golden_npz("adamw_dtypes.npz")
+    h = npz_json(d, "hyper_json")[case]
+    kw = dict(lr=h["lr"], betas=tuple(h["betas"]), eps=h["eps"], weight_decay=h["weight_decay"])
+    last = h["steps"]
+    # bfloat16
+    o = AdamW(**kw, kind="bf16")
+    p = d["bf16_p0"].view(np.uint16).copy()
+    for s in range(last):
+        o.update("k", p, np.ascontiguousarray(d["bf16_grads"][s].view(np.uint16)))
+        if s == 0:
+            for got, key in ((p, "p1"), (o.state["k"][1], "m1"), (o.state["k"][2], "v1")):
+                assert np.array_equal(got, d[f"bf16_{case}_{key}"].view(np.uint16)), key
+    for got, key in ((p, f"p{last}"), (o.state["k"][1], f"m{last}"), (o.state["k"][2], f"v{last}")):
+        assert np.array_equal(got, d[f"bf16_{case}_{key}"].view(np.uint16)), key
+    # float64
+    for sqrt in (lambda v: torch.from_numpy(v).sqrt().numpy(), None):
+        o = AdamW(**kw, sqrt=sqrt)
+        p = d["f64_p0"].copy()
+        for s in range(last):
+            o.update("k", p, np.ascontiguousarray(d["f64_grads"][s]))
+        assert np.array_equal(o.state["k"][1].view(np.uint64), d[f"f64_{case}_m{last}"].view(np.uint64))
+        assert np.array_equal(o.state["k"][2].view(np.uint64), d[f"f64_{case}_v{last}"].view(np.uint64))
+        want = d[f"f64_{case}_p{last}"]
+        if sqrt is not None:
+            assert np.array_equal(p.view(np.uint64), want.view(np.uint64))
+        else:
+            assert np.abs(p - want).max() <= last * 2 * np.spacing(h["lr"])
+            assert (p.view(np.uint64) != want.view(np.uint64)).mean() < 0.05
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float64])
+def test_bf16_and_f64_match_torch_adamw_on_the_cpu(dtype):
+    """torch.optim.AdamW(foreach=False) is what the reference says it reproduces operation for operation
+    (tandem/optim.py:1-6) and what its own tests compare with (tests/test_zero.py:46-54): 20 steps on a shard of
+    20,001 elements, parameters and moments bit for bit (float64 with torch's sqrt substituted)."""
+    kw = dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    n = 20_001
+    g = torch.Generator().manual_seed(3)
+    p0 = (torch.randn(n, generator=g, dtype=torch.float64) * 0.02).to(dtype)
+    pt = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.AdamW([pt], foreach=False, **kw)
+    if dtype == torch.bfloat16:
+        raw = _raw16
+        o = AdamW(**kw, kind="bf16")
+    else:
+        raw = lambda t: t.detach().numpy().copy()
+        o = AdamW(**kw, sqrt=lambda v: torch.from_numpy(v).sqrt().numpy())
+    pn = raw(p0)
+    for s in range(20):
+        gr = (torch.randn(n, generator=g, dtype=torch.float64) * 1e-3).to(dtype)
+        pt.grad = gr.clone()
+        opt.step()
+        o.update("k", pn, raw(gr))
+    st = opt.state[pt]
+    assert np.array_equal(bits(pn), bits(raw(pt.detach())))
+    assert np.array_equal(bits(o.state["k"][1]), bits(raw(st["exp_avg"])))
+    assert np.array_equal(bits(o.state["k"][2]), bits(raw(st["exp_avg_sq"])))
