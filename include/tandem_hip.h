@@ -300,7 +300,9 @@ int tdm_k3_adamw_typed(void* p, const void* g, void* m, void* v, int64_t n, int 
 
 /* One segment: `count` elements that lie in ring chunk `chunk` (= the rank that owns
  * them) of a ZeRO bucket. grad[r]: rank r's gradient (its staging buffer); param[r]: rank
- * r's copy of the parameters; exp_avg, exp_avg_sq: the owner's optimizer state. fp32. */
+ * r's copy of the parameters; exp_avg, exp_avg_sq: the owner's optimizer state. `dtype` is the element type of all
+ * of them: TDM_F32 (0: what a caller that zeroes the struct and knows nothing of the field leaves there), TDM_F64 or
+ * TDM_BF16; the segments of one table share one dtype. */
 /* Entries of ranks beyond the world size must be NULL; alignment as for tdm_fold_seg. */
 typedef struct tdm_step_seg {
   const void* grad[TDM_MAX_WORLD];
@@ -309,7 +311,7 @@ typedef struct tdm_step_seg {
   void* exp_avg_sq;
   int64_t count;
   int32_t chunk;
-  int32_t reserved;
+  int32_t dtype;
 } tdm_step_seg;
 
 /* The device table, as for K2: tiles and bytes it needs (-1: bad arguments), its image
@@ -329,7 +331,14 @@ int tdm_k23_table_build(const tdm_step_seg* segs, int nseg, int world, void* ima
 int tdm_k23_zero2_step(const void* table_dev, int64_t ntiles, int world, int average, const tdm_adamw_scalars* s, int order,
                        tdm_stream stream);
 
-/* The same step for ONE segment, passed in the launch itself (no table in device memory):
+/* The same launch for a table of fp32, float64 or bfloat16 segments, with the step's constants as Python doubles (as
+ * tdm_k3_adamw_typed takes them): fp32 is tdm_k23_zero2_step; float64 folds and steps in doubles; bfloat16 folds as
+ * tdm_k2_bucket_fold does for bf16 (every addition rounded to bf16) and steps as tdm_k3_adamw_typed does. float64 and
+ * bfloat16 in TDM_ADAMW_HOST_ORDER only. `dtype` must be the one the table was built for. */
+int tdm_k23_zero2_step_typed(const void* table_dev, int64_t ntiles, int world, int average, int dtype, const tdm_adamw_hyper* h,
+                             int order, tdm_stream stream);
+
+/* The same step for ONE segment of fp32, passed in the launch itself (no table in device memory):
  * what a rank that is a process of its own runs over its shard, chunk = its rank. */
 int tdm_k23_zero2_step_segment(const tdm_step_seg* seg, int world, int average, const tdm_adamw_scalars* s, int order,
                                tdm_stream stream);

@@ -41,7 +41,7 @@ class FoldSeg(ctypes.Structure):
 class StepSeg(ctypes.Structure):
     _fields_ = [("grad", ctypes.c_void_p * TDM_MAX_WORLD), ("param", ctypes.c_void_p * TDM_MAX_WORLD),
                 ("exp_avg", ctypes.c_void_p), ("exp_avg_sq", ctypes.c_void_p), ("count", ctypes.c_int64),
-                ("chunk", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+                ("chunk", ctypes.c_int32), ("dtype", ctypes.c_int32)]
 
 
 class AdamwScalars(ctypes.Structure):
@@ -100,6 +100,8 @@ _SIGNATURES = {
     "tdm_k23_table_build": (ctypes.c_int, [ctypes.POINTER(StepSeg), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "tdm_k23_zero2_step": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                           ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
+    "tdm_k23_zero2_step_typed": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                ctypes.POINTER(AdamwHyper), ctypes.c_int, ctypes.c_void_p]),
     "tdm_k23_zero2_step_segment": (ctypes.c_int, [ctypes.POINTER(StepSeg), ctypes.c_int, ctypes.c_int,
                                                   ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
     "tdm_k4_unit_gather_all": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p),

@@ -59,6 +59,12 @@ SegPlan plan_fold(const tdm_fold_seg& s, int es) {
   return plan_segment(ptrs, n, s.count, es, static_cast<int64_t>(kTileVecs) * (16 / es));
 }
 
+// The element size of a step segment: its dtype field names TDM_F32 (0, what a caller that knows nothing of the field
+// leaves there), TDM_F64 or TDM_BF16; 0 for anything else.
+int step_elem_size(const tdm_step_seg& s) {
+  return s.dtype == TDM_F32 ? 4 : s.dtype == TDM_F64 ? 8 : s.dtype == TDM_BF16 ? 2 : 0;
+}
+
 SegPlan plan_step(const tdm_step_seg& s) {
   uintptr_t ptrs[2 * TDM_MAX_WORLD + 2];
   int n = 0;
@@ -68,7 +74,9 @@ SegPlan plan_step(const tdm_step_seg& s) {
   }
   if (s.exp_avg) ptrs[n++] = reinterpret_cast<uintptr_t>(s.exp_avg);
   if (s.exp_avg_sq) ptrs[n++] = reinterpret_cast<uintptr_t>(s.exp_avg_sq);
-  return plan_segment(ptrs, n, s.count, 4, static_cast<int64_t>(kTileVecs) * 4);
+  const int es = step_elem_size(s);
+  if (es == 0) throw Invalid("a step segment's dtype must be TDM_F32, TDM_F64 or TDM_BF16");
+  return plan_segment(ptrs, n, s.count, es, static_cast<int64_t>(kTileVecs) * (16 / es));
 }
 
 bool is_floating(int dtype) { return dtype == TDM_F32 || dtype == TDM_F64 || dtype == TDM_F16 || dtype == TDM_BF16; }
@@ -399,6 +407,7 @@ void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const t
   if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
   if (sg.count < 0) throw Invalid("negative count");
   if (sg.count == 0) return;
+  if (sg.dtype != TDM_F32) throw Invalid("the step over one segment handles fp32 shards (dtype " + std::to_string(sg.dtype) + ")");
   if (sg.chunk < 0 || sg.chunk >= world) throw Invalid("chunk outside [0, world)");
   if (!sg.exp_avg || !sg.exp_avg_sq) throw Invalid("NULL optimizer state");
   StepSegDev whole;
@@ -1218,6 +1227,8 @@ int tdm_k3_adamw_typed(void* p, const void* g, void* m, void* v, int64_t n, int 
 
 int64_t tdm_k23_table_tiles(const tdm_step_seg* segs, int nseg) {
   if (nseg < 0 || (nseg > 0 && segs == nullptr)) return -1;
+  for (int i = 0; i < nseg; ++i)
+    if (step_elem_size(segs[i]) == 0) return -1;
   return step_tiles(segs, nseg);
 }
 
@@ -1233,16 +1244,19 @@ int tdm_k23_table_build(const tdm_step_seg* segs, int nseg, int world, void* ima
     if (nseg < 0 || (nseg > 0 && segs == nullptr) || image == nullptr) throw Invalid("bad table arguments");
     std::memset(image, 0, static_cast<size_t>(tdm_k23_table_bytes(segs, nseg)));
     StepSegDev* out = static_cast<StepSegDev*>(image);
-    const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * 4;
+    const int es = nseg > 0 ? step_elem_size(segs[0]) : 4;
+    if (es == 0) throw Invalid("a step segment's dtype must be TDM_F32, TDM_F64 or TDM_BF16");
+    const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
     int64_t tiles = 0;
     for (int i = 0; i < nseg; ++i) {
       const tdm_step_seg& sg = segs[i];
+      if (sg.dtype != segs[0].dtype) throw Invalid("segment " + std::to_string(i) + ": the segments of one table share one dtype");
       if (sg.count < 0) throw Invalid("segment " + std::to_string(i) + ": negative count");
       if (sg.count == 0) continue;
       if (sg.chunk < 0 || sg.chunk >= world) throw Invalid("segment " + std::to_string(i) + ": chunk outside [0, world)");
       if (!sg.exp_avg || !sg.exp_avg_sq) throw Invalid("segment " + std::to_string(i) + ": NULL optimizer state");
-      if (reinterpret_cast<uintptr_t>(sg.exp_avg) % 4 || reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % 4) {
-        throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to 4 bytes");
+      if (reinterpret_cast<uintptr_t>(sg.exp_avg) % es || reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % es) {
+        throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to the element size");
       }
       for (int r = 0; r < TDM_MAX_WORLD; ++r) {
         if (r >= world) {
@@ -1251,12 +1265,12 @@ int tdm_k23_table_build(const tdm_step_seg* segs, int nseg, int world, void* ima
         }
         if (!sg.grad[r] || !sg.param[r]) throw Invalid("segment " + std::to_string(i) + ": NULL gradient or parameter");
         const uintptr_t a = reinterpret_cast<uintptr_t>(sg.grad[r]), b = reinterpret_cast<uintptr_t>(sg.param[r]);
-        if (a % 4 || b % 4) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to 4 bytes");
+        if (a % es || b % es) throw Invalid("segment " + std::to_string(i) + ": pointer not aligned to the element size");
       }
       const SegPlan plan = plan_step(sg);
       for (int64_t at = 0; at < plan.body; at += tile_elems) {  // records describe the body; the first one carries the head
         StepSegDev& rec = out[tiles++];
-        const int64_t off = (plan.head + at) * 4;
+        const int64_t off = (plan.head + at) * es;
         for (int r = 0; r < world; ++r) {
           rec.g[r] = static_cast<const char*>(sg.grad[r]) + off;
           rec.p[r] = static_cast<char*>(sg.param[r]) + off;
@@ -1291,6 +1305,73 @@ int tdm_k23_zero2_step(const void* table_dev, int64_t ntiles, int world, int ave
       default: throw Invalid("world must be in [1, 8]");
     }
     check_hip(hipGetLastError(), "k23_zero2_step launch");
+  });
+}
+
+extern "C++" {
+namespace {
+template <typename T, int kWorld>
+void launch_step_typed_w(const void* image, int64_t tiles, int average, const tdm_adamw_hyper& h, hipStream_t stream) {
+  using S = typename AdamwMath<T>::S;
+  AdamwHyper<S> s{h.use_decay, static_cast<S>(h.decay), static_cast<S>(h.w1), static_cast<S>(h.beta2), static_cast<S>(h.one_m_b2),
+                  static_cast<S>(h.bc2_sqrt), static_cast<S>(h.eps), static_cast<S>(h.neg_step)};
+  if constexpr (std::is_same_v<T, bf16_t>) {  // add_(eps) on a bf16 tensor adds eps rounded to bf16 (nearest even)
+    uint32_t u;
+    std::memcpy(&u, &s.eps, 4);
+    u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+    std::memcpy(&s.eps, &u, 4);
+  }
+  const Divisor<T> dv = make_divisor<T>(kWorld);
+  const StepSegDev* t = static_cast<const StepSegDev*>(image);
+  const dim3 grid(grid_for(tiles * kStepParts)), block(kThreads);
+  const unsigned pad = occupancy_pad(TDM_XCD_STEP);
+  const int shift = xcd_shift(TDM_XCD_STEP, kWorld, true);
+  switch (div_kind(kWorld, average != 0)) {
+    case 0: hipLaunchKernelGGL((k23_zero2_step_typed_kernel<T, kWorld, 0>), grid, block, pad, stream, t, tiles, dv, s, shift); break;
+    case 1: hipLaunchKernelGGL((k23_zero2_step_typed_kernel<T, kWorld, 1>), grid, block, pad, stream, t, tiles, dv, s, shift); break;
+    default: hipLaunchKernelGGL((k23_zero2_step_typed_kernel<T, kWorld, 2>), grid, block, pad, stream, t, tiles, dv, s, shift); break;
+  }
+}
+
+template <typename T>
+void launch_step_typed(const void* image, int64_t tiles, int world, int average, const tdm_adamw_hyper& h, hipStream_t stream) {
+  switch (world) {
+    case 1: launch_step_typed_w<T, 1>(image, tiles, average, h, stream); break;
+    case 2: launch_step_typed_w<T, 2>(image, tiles, average, h, stream); break;
+    case 3: launch_step_typed_w<T, 3>(image, tiles, average, h, stream); break;
+    case 4: launch_step_typed_w<T, 4>(image, tiles, average, h, stream); break;
+    case 5: launch_step_typed_w<T, 5>(image, tiles, average, h, stream); break;
+    case 6: launch_step_typed_w<T, 6>(image, tiles, average, h, stream); break;
+    case 7: launch_step_typed_w<T, 7>(image, tiles, average, h, stream); break;
+    case 8: launch_step_typed_w<T, 8>(image, tiles, average, h, stream); break;
+    default: throw Invalid("world must be in [1, 8]");
+  }
+}
+}  // namespace
+}  // extern "C++"
+
+int tdm_k23_zero2_step_typed(const void* table_dev, int64_t ntiles, int world, int average, int dtype, const tdm_adamw_hyper* h,
+                             int order, tdm_stream stream) {
+  return guard([&] {
+    if (ntiles < 0) throw Invalid("ntiles is negative");
+    if (dtype != TDM_F32 && dtype != TDM_F64 && dtype != TDM_BF16) throw Invalid("the step handles fp32, fp64 and bf16 shards (dtype " + std::to_string(dtype) + ")");
+    if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
+    if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
+    if (ntiles == 0) return;
+    if (table_dev == nullptr || h == nullptr) throw Invalid("NULL argument");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == TDM_F32) {  // a Python double applied to a float tensor is rounded to fp32 once
+      const tdm_adamw_scalars s{h->use_decay, static_cast<float>(h->decay), static_cast<float>(h->w1), static_cast<float>(h->beta2),
+                                static_cast<float>(h->one_m_b2), static_cast<float>(h->bc2_sqrt), static_cast<float>(h->eps),
+                                static_cast<float>(h->neg_step), static_cast<float>(1.0 / h->bc2_sqrt)};
+      const int status = tdm_k23_zero2_step(table_dev, ntiles, world, average, &s, order, stream);
+      if (status != TDM_OK) throw std::runtime_error(tdm_last_error());
+      return;
+    }
+    if (order != TDM_ADAMW_HOST_ORDER) throw Invalid("the device order is defined for fp32 shards only");
+    if (dtype == TDM_F64) launch_step_typed<double>(table_dev, ntiles, world, average, *h, st);
+    else launch_step_typed<bf16_t>(table_dev, ntiles, world, average, *h, st);
+    check_hip(hipGetLastError(), "k23_zero2_step (typed) launch");
   });
 }
 

@@ -1041,6 +1041,99 @@ __global__ __launch_bounds__(kThreads) void k23_zero2_step_one_kernel(StepSegDev
   }
 }
 
+// ---------------------------------------------------------------- K2 + K3 on float64 and bfloat16
+// The one-launch step on the other shard types of K3: the gradients folded in the ring's order with the
+// element type's own rounding (as K2 folds them: every addition rounded to the type), 0 + mine as
+// grad_shard.add_(mine) leaves it, the typed AdamW step of AdamwMath<T>, the new parameter stored into every
+// rank's buffer. Host order. One vector per lane and stream in flight (a vector is 2 doubles or 8 bf16).
+template <typename T, int kWorld, int kDiv, int kRounds>
+__device__ __forceinline__ void step_tile_typed(const StepSegDev& sg, int64_t at, int64_t n, int head, const Divisor<T>& dv,
+                                                const AdamwHyper<typename AdamwMath<T>::S>& s, bool small_w) {
+  using A = typename Elem<T>::acc;
+  constexpr int L = lanes<T>();
+  constexpr int kM = TDM_NT_MASK_K23;
+  const int c = sg.chunk;  // `at`: the tile's offset in bytes from the record's pointers; n: its elements
+  const char* gp[kWorld];
+  char* pp[kWorld];
+#pragma unroll
+  for (int k = 0; k < kWorld; ++k) {
+    gp[k] = sg.g[(c + 1 + k) % kWorld] + at;  // the fold ends with the owner's own term
+    pp[k] = sg.p[k] + at;
+  }
+  char* own = sg.p[c] + at;
+  char* const mm = sg.m + at;
+  char* const vv = sg.v + at;
+  auto one = [&](const T (&gs)[kWorld], T& P, T& M, T& V) {
+    A acc = scaled<T, kDiv>(Elem<T>::widen(gs[0]), dv.divisor, dv.reciprocal);
+#pragma unroll
+    for (int k = 1; k < kWorld; ++k) {
+      const A y = scaled<T, kDiv>(Elem<T>::widen(gs[k]), dv.divisor, dv.reciprocal);
+      acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
+    }
+    const T g = Elem<T>::narrow(static_cast<A>(A(0) + acc));  // grad_shard (zero) += mine
+    AdamwMath<T>::step(P, g, M, V, s, small_w);
+  };
+  auto scalar_at = [&](int64_t i) {
+    T gs[kWorld];
+#pragma unroll
+    for (int k = 0; k < kWorld; ++k) gs[k] = reinterpret_cast<const T*>(gp[k])[i];
+    T P = reinterpret_cast<T*>(own)[i], M = reinterpret_cast<T*>(mm)[i], V = reinterpret_cast<T*>(vv)[i];
+    one(gs, P, M, V);
+#pragma unroll
+    for (int q = 0; q < kWorld; ++q) reinterpret_cast<T*>(pp[q])[i] = P;
+    reinterpret_cast<T*>(mm)[i] = M;
+    reinterpret_cast<T*>(vv)[i] = V;
+  };
+  if (sg.vec_ok) {
+    const int64_t nv = n / L;
+#pragma unroll
+    for (int u = 0; u < kRounds; ++u) {
+      const int64_t v = threadIdx.x + static_cast<int64_t>(u) * kThreads;
+      if (v < nv) {
+        vec16 in[kWorld];
+#pragma unroll
+        for (int k = 0; k < kWorld; ++k) in[k] = load_stream<kM>(gp[k] + v * 16);
+        Lanes<T> P = unpack<T>(load_rmw<kM>(own + v * 16)), M = unpack<T>(load_rmw<kM>(mm + v * 16)),
+                 V = unpack<T>(load_rmw<kM>(vv + v * 16));
+#pragma unroll
+        for (int l = 0; l < L; ++l) {
+          T gs[kWorld];
+#pragma unroll
+          for (int k = 0; k < kWorld; ++k) gs[k] = unpack<T>(in[k]).v[l];
+          one(gs, P.v[l], M.v[l], V.v[l]);
+        }
+        const vec16 packed = pack<T>(P);
+#pragma unroll
+        for (int q = 0; q < kWorld; ++q) store16<kM>(pp[q] + v * 16, packed);
+        store16<kM>(mm + v * 16, pack<T>(M));
+        store16<kM>(vv + v * 16, pack<T>(V));
+      }
+    }
+    // the tile's last few elements (lanes 0..), and the segment's head before its first vector (lanes 32..)
+    if (threadIdx.x < n - nv * L || (threadIdx.x >= 32 && static_cast<int>(threadIdx.x) - 32 < head)) {
+      scalar_at(threadIdx.x < 32 ? nv * L + threadIdx.x : -1 - (static_cast<int64_t>(threadIdx.x) - 32));
+    }
+  } else {
+    for (int64_t i = threadIdx.x; i < n; i += kThreads) scalar_at(i);
+  }
+}
+
+template <typename T, int kWorld, int kDiv>
+__global__ __launch_bounds__(kThreads) void k23_zero2_step_typed_kernel(const StepSegDev* __restrict__ tiles, int64_t total, Divisor<T> dv,
+                                                                        AdamwHyper<typename AdamwMath<T>::S> s, int shift) {
+  using S = typename AdamwMath<T>::S;
+  const bool small_w = (s.w1 < S(0) ? -s.w1 : s.w1) < S(0.5);
+  constexpr int64_t kPartElems = static_cast<int64_t>(kTileVecs / kStepParts) * lanes<T>();
+  for (int64_t at = blockIdx.x; at < total * kStepParts; at += gridDim.x) {
+    const int64_t part = tile_of(at, total * kStepParts, shift);
+    const StepSegDev& rec = tiles[part / kStepParts];
+    const int64_t first = (part % kStepParts) * kPartElems;  // the part's first element within the record
+    const int64_t n = min(kPartElems, rec.count - first);
+    const int head = first == 0 ? rec.vec_ok - 1 : 0;
+    if (n > 0) step_tile_typed<T, kWorld, kDiv, kUnroll / kStepParts>(rec, first * static_cast<int64_t>(sizeof(T)), n, head, dv, s, small_w);
+  }
+}
+
 }  // namespace
 
 }  // namespace tandem_hip

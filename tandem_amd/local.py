@@ -245,21 +245,32 @@ class LocalZeRO2:
     step() is ZeRO.step (tandem/zero.py:158-163): sharded AdamW on every rank's
     shard, then the all-gather of the flat parameter buffer."""
 
-    def __init__(self, world, numels, device, bucket_bytes=25 << 20, order="host", one_allocation=False, **adamw):
-        """one_allocation: every buffer (the ranks' parameters and gradients, the gradient shards, the optimizer
+    def __init__(self, world, numels, device, bucket_bytes=25 << 20, order="host", one_allocation=False, dtype=torch.float32,
+                 **adamw):
+        """dtype: the element type of parameters, gradients and optimizer state: fp32, float64 or bfloat16 (the last two in
+        host order; their gradients are reduced by the fold, which rounds every addition to the type as the ring does).
+        one_allocation: every buffer (the ranks' parameters and gradients, the gradient shards, the optimizer
         state) is carved out of a single allocation, back to back at 128-byte boundaries, instead of being an
         allocation of its own. Where the streams of a launch lie relative to each other is worth a few per cent
         either way on this memory system; the default is what measured faster for the one-launch step."""
         from .buckets import FlatLayout, zero_buckets
         from .optim import LINE, ShardedAdamW, zeros_at_phase_of
 
+        from .optim import SHARD_DTYPES
+
+        if dtype not in SHARD_DTYPES:
+            raise ValueError(f"LocalZeRO2 handles fp32, float64 and bfloat16 (got {dtype})")
+        es = torch.empty(0, dtype=dtype).element_size()
+        self.dtype = dtype
         self.lw = LocalWorld(world)
         self.world = world
         self.layouts = [FlatLayout(numels, world, r) for r in range(world)]
         n = self.layouts[0].numel
         self.numel = n
-        self.buckets = zero_buckets(list(numels), 4, bucket_bytes)
+        self.buckets = zero_buckets(list(numels), es, bucket_bytes)
         if one_allocation:
+            if dtype != torch.float32:
+                raise ValueError("one_allocation lays out fp32 buffers")
             per = LINE // 4
             room = lambda m: -(-m // per) * per + per  # a line of slack for the phase
             shard_room = sum(room(l.hi - l.lo) for l in self.layouts)
@@ -278,14 +289,13 @@ class LocalZeRO2:
             self.staging = [zeros_like_phase(self.bufs[0], n) for _ in range(world)]
         else:
             zeros_like_phase = zeros_at_phase_of
-            self.bufs = [torch.zeros(n, device=device) for _ in range(world)]
-            self.staging = [torch.zeros(n, device=device) for _ in range(world)]
+            self.bufs = [torch.zeros(n, device=device, dtype=dtype) for _ in range(world)]
+            self.staging = [torch.zeros(n, device=device, dtype=dtype) for _ in range(world)]
         # every shard's gradient (and, below, its optimizer state) at the phase of the parameter shard it belongs to
         self.grad_shards = [zeros_like_phase(self.bufs[r][l.lo:l.hi]) for r, l in enumerate(self.layouts)]
         self.opts = [ShardedAdamW(order=order, **adamw) for _ in range(world)]
         self.device = torch.device(device)
         # ring step s of every bucket: (dst, src, count) pairs, and the final adds
-        es = 4
         self._steps = [[] for _ in range(world - 1)]
         self._adds = []
         rows = []
@@ -304,7 +314,7 @@ class LocalZeRO2:
                     dsts[c] = self.grad_shards[c].data_ptr() + shard_at * es
                     rows.append(([p + lo * es for p in sb], dsts, m, c))
                 lo += m
-        self._fold = (FoldTable.from_segments(world, torch.float32, device, rows, keep=(self.staging, self.grad_shards))
+        self._fold = (FoldTable.from_segments(world, dtype, device, rows, keep=(self.staging, self.grad_shards))
                       if world <= _lib.TDM_MAX_WORLD else None)
         # The whole step as one launch (reduce_and_step): the optimizer state must exist, at fixed addresses.
         self._shards_zero = True
@@ -323,7 +333,7 @@ class LocalZeRO2:
                     segs[k].param[r] = bb[r] + lo * es
                 segs[k].exp_avg = exp_avg.data_ptr() + at * es
                 segs[k].exp_avg_sq = exp_avg_sq.data_ptr() + at * es
-                segs[k].count, segs[k].chunk = m, c
+                segs[k].count, segs[k].chunk, segs[k].dtype = m, c, dtype_code(dtype)
             ntiles = lib().tdm_k23_table_tiles(segs, len(rows))
             image = torch.empty(max(16, lib().tdm_k23_table_bytes(segs, len(rows))), dtype=torch.uint8)
             check(lib().tdm_k23_table_build(segs, len(rows), world, ctypes.c_void_p(image.data_ptr())))
@@ -333,7 +343,7 @@ class LocalZeRO2:
         st = stream_ptr(self.device)
         for k in range(0, len(items), _lib.TDM_MAX_PAIRS):
             part = items[k:k + _lib.TDM_MAX_PAIRS]
-            check(lib().tdm_k1_reduce_step(_pairs(part), len(part), 0, self.world if scale_dst else 1,
+            check(lib().tdm_k1_reduce_step(_pairs(part), len(part), dtype_code(self.dtype), self.world if scale_dst else 1,
                                            int(scale_dst), int(scale_src), int(writeback), st))
 
     def reduce_grads(self, algorithm="fold"):
@@ -359,7 +369,7 @@ class LocalZeRO2:
         with 8W + 20 instead of 12W + 28 bytes of HBM traffic per element. Needs the
         gradient shards at zero (no accumulation since zero_grad()) and at most 8 ranks;
         the shards stay zero."""
-        from .optim import step_scalars
+        from .optim import step_hyper, step_scalars
 
         if self._step_table is None or not self._shards_zero:
             self.reduce_grads()
@@ -368,8 +378,13 @@ class LocalZeRO2:
         for opt in self.opts:
             opt.state["flat"][0] += 1.0
         o = self.opts[0]
-        scalars = step_scalars(o.state["flat"][0], o.lr, o.betas, o.eps, o.weight_decay)
         image, ntiles = self._step_table
+        if self.dtype != torch.float32:
+            hyper = step_hyper(o.state["flat"][0], o.lr, o.betas, o.eps, o.weight_decay)
+            check(lib().tdm_k23_zero2_step_typed(ctypes.c_void_p(image.data_ptr()), ntiles, self.world, 1, dtype_code(self.dtype),
+                                                 ctypes.byref(hyper), o.order, stream_ptr(self.device)))
+            return
+        scalars = step_scalars(o.state["flat"][0], o.lr, o.betas, o.eps, o.weight_decay)
         check(lib().tdm_k23_zero2_step(ctypes.c_void_p(image.data_ptr()), ntiles, self.world, 1, ctypes.byref(scalars),
                                        o.order, stream_ptr(self.device)))
 

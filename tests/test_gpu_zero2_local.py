@@ -123,6 +123,80 @@ def test_shards_that_start_off_the_16_byte_grid(algorithm, one_allocation):
         assert np.array_equal(bits(z.opts[r].state["flat"][2].cpu().numpy()), bits(opts[r].state["flat"][2]))
 
 
+def _raw(t):
+    t = t.detach().cpu()
+    return t.view(torch.int16).numpy().view(np.uint16).copy() if t.element_size() == 2 else t.numpy().copy()
+
+
+@pytest.mark.parametrize("algorithm", ["fold", "ring", "fused"])
+@pytest.mark.parametrize("world", [2, 4, 3])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float64])
+def test_other_shard_dtypes_bit_exact_with_oracle(dtype, world, algorithm):
+    """The ZeRO-2 step over bfloat16 and float64 models (the reference's classes and its seven-operation AdamW take
+    any floating dtype, tandem/zero.py:69-170, tandem/optim.py:28-37): per-bucket ring reduce-scatter in the type's own
+    rounding, the add into the zeroed gradient shard, the typed AdamW, the all-gather; by ring steps, by the fold and as
+    ONE launch (tdm_k23_zero2_step_typed). Four steps against the oracle, bit for bit in every rank's parameters and in
+    both moments; world 3 puts the shards off the 16-byte grid."""
+    from oracle import ring
+    from oracle.adamw import AdamW
+    from tandem_amd.buckets import FlatLayout, zero_buckets
+    from tandem_amd.local import LocalZeRO2
+
+    dev = torch.device("cuda", 0)
+    kind = "bf16" if dtype == torch.bfloat16 else "f64"
+    es = 2 if kind == "bf16" else 8
+    numels = [4099, 10_007, 33, 5001, 1, 12_288, 782]
+    n = sum(numels)
+    steps = 4
+    kw = dict(lr=1e-3, betas=(0.9, 0.95), eps=1e-6, weight_decay=0.1)
+    p0 = (seeded(3, 0, n).double() * 0.02).to(dtype)
+    grads = [[(seeded(30 + s, r, n).double() * 1e-3).to(dtype) for r in range(world)] for s in range(steps)]
+    for g in grads[0]:
+        g[:4] = torch.tensor([0.0, -0.0, 1e-30, -1e-30], dtype=torch.float64).to(dtype)
+    z = LocalZeRO2(world, numels, dev, bucket_bytes=16 << 10, dtype=dtype, **kw)
+    assert z.bufs[0].dtype == dtype and z.opts[0].state["flat"][1].dtype == dtype
+    for b in z.bufs:
+        b.copy_(p0)
+    for s in range(steps):
+        for r in range(world):
+            z.staging[r].copy_(grads[s][r])
+        if algorithm == "fused":
+            assert z._step_table is not None and z._shards_zero
+            z.reduce_and_step()
+        else:
+            z.reduce_grads(algorithm)
+            z.step(fused_gather=algorithm == "fold")
+        z.zero_grad()
+    # the same step written with the oracle only
+    lay = [FlatLayout(numels, world, r) for r in range(world)]
+    bufs = [_raw(p0) for _ in range(world)]
+    opts = [AdamW(**kw, kind="bf16" if kind == "bf16" else None) for _ in range(world)]
+    for s in range(steps):
+        gs = [_raw(g) for g in grads[s]]
+        shards = [np.zeros(l.hi - l.lo, bufs[0].dtype) for l in lay]
+        for a, b, _ in zero_buckets(numels, es, 16 << 10):
+            sizes = lay[0].bucket_sizes(a, b)
+            outs = ring.expected_reduce_scatter([g[a:b] for g in gs], sizes, True, kind)
+            lo = a
+            for c, m in enumerate(sizes):
+                if m:
+                    mine = outs[c][lo - a:lo - a + m].copy()
+                    if kind == "bf16":
+                        mine[mine == 0x8000] = 0  # 0 + (-0) = +0, as grad_shard.add_(mine) leaves it; nothing else changes
+                    else:
+                        mine = 0.0 + mine
+                    shards[c][lo - lay[c].lo:lo - lay[c].lo + m] = mine
+                lo += m
+        for r in range(world):
+            opts[r].update("flat", bufs[r][lay[r].lo:lay[r].hi], shards[r])
+        full = ring.expected_all_gather(bufs, lay[0].sizes)
+        bufs = [full.copy() for _ in range(world)]
+    for r in range(world):
+        assert np.array_equal(bits(_raw(z.bufs[r])), bits(bufs[r])), (dtype, world, algorithm, r)
+        assert np.array_equal(bits(_raw(z.opts[r].state["flat"][1])), bits(opts[r].state["flat"][1])), (dtype, world, algorithm, r)
+        assert np.array_equal(bits(_raw(z.opts[r].state["flat"][2])), bits(opts[r].state["flat"][2])), (dtype, world, algorithm, r)
+
+
 def test_full_size_step():
     """85,842,432 parameters, world 4, 25 MiB buckets, the reference's bucket_sizes
     (plans.json), one step. The ring's steps and the fold leave the same gradient
