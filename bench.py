@@ -434,6 +434,34 @@ def zero2_step(dev, reps):
         out.update({f"{key}ms": round(step * 1e3, 4), f"{key}reduce_scatter_ms": round(rs * 1e3, 4),
                     f"{key}algorithmic_bytes": nbytes, f"{key}GBps": round(nbytes / step / 1e9, 1),
                     f"{key}roofline_floor_ms": round(nbytes / (HBM_PEAK_GBPS * 1e9) * 1e3, 4)})
+    # the same two kernels on the other shard types: AdamW over four shards (7 x the element size per element), and the whole
+    # step as one launch ((2 W + 5) x the element size per element), in bfloat16 and float64
+    for dtype, tag in ((torch.bfloat16, "bf16"), (torch.float64, "f64")):
+        es = torch.empty(0, dtype=dtype).element_size()
+        zt = LocalZeRO2(WORLD, numels, dev, dtype=dtype, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+        for b in zt.bufs:
+            b.copy_(p0)
+        gt = [g.to(dtype) for g in grads]
+        for r in range(WORLD):
+            zt.grad_shards[r].copy_(gt[r][zt.layouts[r].lo:zt.layouts[r].hi])
+        t_opt = timed(lambda: [zt.opts[r].update("bench", zt.bufs[r][zt.layouts[r].lo:zt.layouts[r].hi], zt.grad_shards[r])
+                               for r in range(WORLD)], reps)
+        zt.zero_grad()
+        zt._shards_zero = True
+
+        def refill_t():
+            for r in range(WORLD):
+                zt.staging[r].copy_(gt[r])
+
+        t_fill = timed(refill_t, reps)
+        t_one = timed(lambda: (refill_t(), zt.reduce_and_step()), reps) - t_fill
+        k3_bytes, one_b = 7 * es * shard * WORLD, (2 * WORLD + 5) * es * n
+        out.update({f"adamw_{tag}_4_shards_ms": round(t_opt * 1e3, 4), f"adamw_{tag}_GBps": round(k3_bytes / t_opt / 1e9, 1),
+                    f"adamw_{tag}_frac_of_hbm_peak": round(k3_bytes / t_opt / 1e9 / HBM_PEAK_GBPS, 4),
+                    f"one_launch_{tag}_ms": round(t_one * 1e3, 4), f"one_launch_{tag}_GBps": round(one_b / t_one / 1e9, 1),
+                    f"one_launch_{tag}_frac_of_hbm_peak": round(one_b / t_one / 1e9 / HBM_PEAK_GBPS, 4)})
+        del zt, gt
+        torch.cuda.empty_cache()
     ag_one_bytes, ag_steps_bytes = 4 * WORLD * n, 8 * (WORLD - 1) * n
     out.update({"adamw_4_shards_ms": round(opt * 1e3, 4), "adamw_GBps": round(28 * shard * WORLD / opt / 1e9, 1),
                 "adamw_frac_of_hbm_peak": round(28 * shard * WORLD / opt / 1e9 / HBM_PEAK_GBPS, 4),

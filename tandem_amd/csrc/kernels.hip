@@ -1189,7 +1189,11 @@ void adamw_typed_launch(void* p_, const void* g_, void* m_, void* v_, int64_t n,
   }
   const int64_t per = vec ? static_cast<int64_t>(kAdamwThreads) * (16 / es) : kAdamwThreads;
   const dim3 grid(grid_for(std::max<int64_t>((a.n + per - 1) / per, 1))), block(kAdamwThreads);
-  const unsigned pad = occupancy_pad(TDM_XCD_ADAMW);
+  // bf16 rounds eight times per element and is bound by its arithmetic (0.52 of the HBM peak), where the cap of three waves per
+  // SIMD that suits the memory-bound fp32 and fp64 kernels costs it 5 %: four 21.46M-element shards take 0.243 ms with 8 KiB,
+  // 0.255 with none, 0.257 with 24 KiB.
+  const int set = g_occupancy_pad[TDM_XCD_ADAMW].load(std::memory_order_relaxed);
+  const unsigned pad = set >= 0 ? static_cast<unsigned>(set) : std::is_same_v<T, bf16_t> ? 8192u : occupancy_pad(TDM_XCD_ADAMW);
   switch ((vec ? 2 : 0) + (ncopies > 0 ? 1 : 0)) {
     case 0: hipLaunchKernelGGL((k3_adamw_typed_kernel<T, false, false>), grid, block, pad, st, a); break;
     case 1: hipLaunchKernelGGL((k3_adamw_typed_kernel<T, false, true>), grid, block, pad, st, a); break;

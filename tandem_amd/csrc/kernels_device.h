@@ -814,7 +814,13 @@ template <> struct AdamwMath<double> {
 
 template <> struct AdamwMath<bf16_t> {
   using S = float;
-  static __device__ __forceinline__ float rb(float x) { return Elem<bf16_t>::widen(Elem<bf16_t>::narrow(x)); }
+  // x rounded to bf16 (nearest even) and back, by the conversion instruction (v_cvt_pk_bf16_f32) instead of the seven integer
+  // operations of Elem<bf16_t>::narrow: this kernel rounds eight times per element and is bound by its arithmetic, not by
+  // memory. A NaN stays a NaN here; what is stored goes through narrow(), which makes it the canonical one.
+  static __device__ __forceinline__ float rb(float x) {
+    const __bf16 h = static_cast<__bf16>(x);
+    return static_cast<float>(h);
+  }
   static __device__ __forceinline__ void step(bf16_t& p, bf16_t g, bf16_t& m, bf16_t& v, const AdamwHyper<float>& s, bool small_w) {
     float P = Elem<bf16_t>::widen(p), M = Elem<bf16_t>::widen(m), V = Elem<bf16_t>::widen(v);
     const float G = Elem<bf16_t>::widen(g);
@@ -827,9 +833,15 @@ template <> struct AdamwMath<bf16_t> {
     D = rb(D / s.bc2_sqrt);
     D = rb(D + s.eps);  // s.eps arrives rounded to bf16
     P = rb(P + (s.neg_step * M) / D);
-    p = Elem<bf16_t>::narrow(P);
-    m = Elem<bf16_t>::narrow(M);
-    v = Elem<bf16_t>::narrow(V);
+    p = exact(P);
+    m = exact(M);
+    v = exact(V);
+  }
+  // The bits of a float that rb() has already rounded: its upper half; a NaN becomes the canonical one, as narrow() makes it.
+  static __device__ __forceinline__ bf16_t exact(float x) {
+    bf16_t out;
+    out.bits = x != x ? static_cast<uint16_t>(0x7fc0u) : static_cast<uint16_t>(__float_as_uint(x) >> 16);
+    return out;
   }
 };
 
