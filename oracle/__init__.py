@@ -25,6 +25,14 @@ Contents, and what pins each against the reference (tests/test_oracle_*.py):
                            is substituted, and to 1 ulp of the update term with
                            the correctly rounded sqrtf (torch's vectorised CPU
                            sqrt is not correctly rounded on ~0.7% of inputs).
+                           float64 and bfloat16 shards (the reference's seven torch
+                           operations take any floating dtype): pinned by
+                           tests/golden/adamw_dtypes.npz, the reference's ShardedAdamW on
+                           such shards (bf16 bit for bit in p, m, v; f64 like fp32), by
+                           torch.optim.AdamW(foreach=False) on the CPU, and operation by
+                           operation against torch's CPU kernels on inputs where the
+                           candidate formulas differ (which scalar is rounded to bf16,
+                           what is fused).
   cpu_engine               from-scratch CPU-process engine speaking the Python
                            engine's protocol (tandem/comm.py:172-311); pinned by
                            the same ring fixtures and by tests/golden/train_w*.json.

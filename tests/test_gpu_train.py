@@ -166,6 +166,70 @@ def test_two_ranks_all_strategies_agree_bit_for_bit():
             assert all(x.get("no_full_grads", True) for x in res), f"{s}: full gradients were kept"
 
 
+def train_rank_typed(g, strategy, dtype_name, steps, batch):
+    """The small GPT in bfloat16 or float64 under every strategy, stepped by ShardedAdamW in the reference's operation
+    order (the reference's wrappers and its optimizer take any floating dtype). DDP has no sharded optimizer of its own:
+    it applies the same per-element update to every parameter after its buckets are reduced, which is what the sharded
+    strategies compute shard by shard."""
+    from tandem_amd import ShardedAdamW
+    from tandem_amd.data import synthetic
+    from tandem_amd.ddp import DDP
+    from tandem_amd.model import GPT
+    from tandem_amd.zero import FSDP, ZeRO
+
+    deterministic()
+    dtype = getattr(torch, dtype_name)
+    c = cfg()
+    torch.manual_seed(0)
+    text = synthetic(20_000)
+    model = GPT(c).to(g.device).to(dtype)
+    sopt = ShardedAdamW(lr=LR, weight_decay=WD)
+    if strategy.startswith("ddp"):
+        z = DDP(model, g, bucket_bytes=4 << 10, direct=strategy.endswith("d"))
+    elif strategy.startswith("zero3"):
+        z = FSDP(model, g, sopt, direct=not strategy.endswith("s"))
+    else:
+        z = ZeRO(model, g, int(strategy[4]), sopt, 4 << 10, direct=strategy.endswith("d"))
+    losses = []
+    for step in range(steps):
+        x, y = text.batch(step, batch, c.seq, rank=g.rank, world=g.size, device=g.device)
+        loss = z(x, y)
+        loss.backward()
+        losses.append(loss.item())
+        if strategy.startswith("ddp"):
+            with torch.no_grad():
+                for i, p in enumerate(model.parameters()):
+                    sopt.update(i, p.data.view(-1), p.grad.reshape(-1).contiguous())
+            for p in model.parameters():
+                p.grad = None
+        else:
+            z.step()
+            z.zero_grad()
+    w = z.full_parameters() if strategy.startswith("zero3") else torch.cat([p.detach().reshape(-1) for p in model.parameters()])
+    torch.cuda.synchronize()
+    assert w.dtype == dtype and all(m.dtype == dtype for _, m, _ in sopt.state.values())
+    return {"losses": losses, "weights": w.cpu()}
+
+
+@pytest.mark.parametrize("dtype_name", ["bfloat16", "float64"])
+def test_bf16_and_f64_models_all_strategies_agree(dtype_name):
+    """Two ranks, a bfloat16 and a float64 model: DDP, ZeRO-1, ZeRO-2 and FSDP, through the slots and arena to arena, must
+    end with the same weights bit for bit and see the same losses (at two ranks the average is (a/2) + (b/2) in any order,
+    and the update is per element), and the model must learn. What the kernels compute for these types is pinned against
+    the oracle elsewhere; this is the wrappers carrying the dtype through buckets, shards, optimizer state and gathers."""
+    from tandem_amd import launch
+
+    runs = {s: launch(train_rank_typed, 2, s, dtype_name, STEPS, BATCH, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT)
+            for s in ("ddp", "ddpd", "zero1", "zero1d", "zero2", "zero2d", "zero3", "zero3s")}
+    ref = runs["ddp"]
+    assert ref[0]["losses"][-1] < ref[0]["losses"][0]
+    for s, res in runs.items():
+        assert torch.equal(res[0]["weights"].view(torch.uint8), res[1]["weights"].view(torch.uint8)), f"{s}: the ranks drifted apart"
+        for r in range(2):
+            assert res[r]["losses"] == ref[r]["losses"], (s, r, dtype_name)
+            assert torch.equal(res[r]["weights"].view(torch.uint8), ref[0]["weights"].view(torch.uint8)), (s, r, dtype_name)
+
+
 def test_four_ranks_stay_in_step():
     """World 4: the ring's order now matters and is pinned elsewhere (kernels against
     the oracle, host logic against the reference's runs on the CPU); here the ranks
