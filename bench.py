@@ -435,8 +435,8 @@ def zero2_step(dev, reps):
                     f"{key}algorithmic_bytes": nbytes, f"{key}GBps": round(nbytes / step / 1e9, 1),
                     f"{key}roofline_floor_ms": round(nbytes / (HBM_PEAK_GBPS * 1e9) * 1e3, 4)})
     # the same two kernels on the other shard types: AdamW over four shards (7 x the element size per element), and the whole
-    # step as one launch ((2 W + 5) x the element size per element), in bfloat16 and float64
-    for dtype, tag in ((torch.bfloat16, "bf16"), (torch.float64, "f64")):
+    # step as one launch ((2 W + 5) x the element size per element), in bfloat16, float16 and float64
+    for dtype, tag in ((torch.bfloat16, "bf16"), (torch.float16, "f16"), (torch.float64, "f64")):
         es = torch.empty(0, dtype=dtype).element_size()
         zt = LocalZeRO2(WORLD, numels, dev, dtype=dtype, lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
         for b in zt.bufs:

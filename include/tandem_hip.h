@@ -286,13 +286,14 @@ typedef struct tdm_adamw_hyper {
   double neg_step;   /* -(lr / (1 - beta1**t)) */
 } tdm_adamw_hyper;
 
-/* tdm_k3_adamw / tdm_k3_adamw_gather for shards of fp32 (TDM_F32), float64 (TDM_F64) or bfloat16 (TDM_BF16): the
- * reference's update is seven torch operations that take any floating dtype (tandem/optim.py:28-37). `copies`
- * may be NULL with ncopies 0. fp32: the constants are rounded to fp32 once and the call is tdm_k3_adamw(_gather),
- * in either order. float64: the same operations on doubles, the constants unrounded. bfloat16: every one of the
- * seven operations computes in fp32 and rounds its result to bf16 (nearest even), as ATen's kernels for bf16
- * tensors do; eps is added rounded to bf16, the other constants act as fp32. float64 and bfloat16 follow torch's
- * CPU kernels (TDM_ADAMW_HOST_ORDER); TDM_ADAMW_DEVICE_ORDER is refused for them. */
+/* tdm_k3_adamw / tdm_k3_adamw_gather for shards of fp32 (TDM_F32), float64 (TDM_F64), bfloat16 (TDM_BF16) or float16
+ * (TDM_F16): the reference's update is seven torch operations that take any floating dtype (tandem/optim.py:28-37).
+ * `copies` may be NULL with ncopies 0. fp32: the constants are rounded to fp32 once and the call is
+ * tdm_k3_adamw(_gather), in either order. float64: the same operations on doubles, the constants unrounded. The
+ * 16-bit types: every one of the seven operations computes in fp32 and rounds its result to the type (nearest even),
+ * as ATen's kernels for such tensors do; eps is added rounded to the type (float16 turns 1e-8 into 0, as it does for
+ * the reference), the other constants act as fp32; a NaN is stored as the type's canonical quiet NaN. Everything but
+ * fp32 follows torch's CPU kernels (TDM_ADAMW_HOST_ORDER); TDM_ADAMW_DEVICE_ORDER is refused for it. */
 int tdm_k3_adamw_typed(void* p, const void* g, void* m, void* v, int64_t n, int dtype, const tdm_adamw_hyper* h, int order,
                        void* const* copies, int ncopies, tdm_stream stream);
 
@@ -301,8 +302,8 @@ int tdm_k3_adamw_typed(void* p, const void* g, void* m, void* v, int64_t n, int 
 /* One segment: `count` elements that lie in ring chunk `chunk` (= the rank that owns
  * them) of a ZeRO bucket. grad[r]: rank r's gradient (its staging buffer); param[r]: rank
  * r's copy of the parameters; exp_avg, exp_avg_sq: the owner's optimizer state. `dtype` is the element type of all
- * of them: TDM_F32 (0: what a caller that zeroes the struct and knows nothing of the field leaves there), TDM_F64 or
- * TDM_BF16; the segments of one table share one dtype. */
+ * of them: TDM_F32 (0: what a caller that zeroes the struct and knows nothing of the field leaves there), TDM_F64,
+ * TDM_BF16 or TDM_F16; the segments of one table share one dtype. */
 /* Entries of ranks beyond the world size must be NULL; alignment as for tdm_fold_seg. */
 typedef struct tdm_step_seg {
   const void* grad[TDM_MAX_WORLD];
@@ -331,10 +332,11 @@ int tdm_k23_table_build(const tdm_step_seg* segs, int nseg, int world, void* ima
 int tdm_k23_zero2_step(const void* table_dev, int64_t ntiles, int world, int average, const tdm_adamw_scalars* s, int order,
                        tdm_stream stream);
 
-/* The same launch for a table of fp32, float64 or bfloat16 segments, with the step's constants as Python doubles (as
- * tdm_k3_adamw_typed takes them): fp32 is tdm_k23_zero2_step; float64 folds and steps in doubles; bfloat16 folds as
- * tdm_k2_bucket_fold does for bf16 (every addition rounded to bf16) and steps as tdm_k3_adamw_typed does. float64 and
- * bfloat16 in TDM_ADAMW_HOST_ORDER only. `dtype` must be the one the table was built for. */
+/* The same launch for a table of fp32, float64, bfloat16 or float16 segments, with the step's constants as Python
+ * doubles (as tdm_k3_adamw_typed takes them): fp32 is tdm_k23_zero2_step; float64 folds and steps in doubles; the
+ * 16-bit types fold as tdm_k2_bucket_fold does for them (every addition rounded to the type) and step as
+ * tdm_k3_adamw_typed does. Everything but fp32 in TDM_ADAMW_HOST_ORDER only. `dtype` must be the one the table was
+ * built for. */
 int tdm_k23_zero2_step_typed(const void* table_dev, int64_t ntiles, int world, int average, int dtype, const tdm_adamw_hyper* h,
                              int order, tdm_stream stream);
 

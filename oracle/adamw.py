@@ -4,9 +4,10 @@ Follows tandem/optim.py:16-37: the scalars are computed in Python doubles
 exactly as written there and rounded to fp32 once when applied to the tensor,
 the way torch applies a Python scalar to a float tensor; the per-element
 arithmetic is oracle/tandem_oracle.c. fp32 shards are numpy float32 arrays;
-float64 shards numpy float64 arrays (the scalars stay doubles); bfloat16 shards
-are their bit patterns in numpy uint16 arrays with kind="bf16" (fp32 arithmetic,
-rounded to bf16 after each of the reference's torch operations).
+float64 shards numpy float64 arrays (the scalars stay doubles); bfloat16 and
+float16 shards are their bit patterns in numpy uint16 arrays with kind="bf16" /
+"f16" (fp32 arithmetic, rounded to the 16-bit type after each of the
+reference's torch operations).
 """
 
 import ctypes
@@ -63,7 +64,7 @@ class AdamW:
     produced by torch)."""
 
     def __init__(self, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, sqrt=None, kind=None):
-        """kind: None (taken from the array: float32 or float64) or "bf16" for uint16 arrays of bfloat16 bit patterns."""
+        """kind: None (taken from the array: float32 or float64), or "bf16" / "f16" for uint16 arrays of bit patterns."""
         self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
         self.state = {}
         self.sqrt = sqrt
@@ -78,7 +79,7 @@ class AdamW:
         n = param.size
         if n == 0:
             return
-        if self.kind == "bf16" or param.dtype == np.float64:
+        if self.kind in ("bf16", "f16") or param.dtype == np.float64:
             return self._update_other(param, grad, m, v, step, n)
         s = scalars(step, self.lr, self.betas, self.eps, self.weight_decay)
         f = ctypes.c_float
@@ -96,8 +97,8 @@ class AdamW:
 
     def _update_other(self, param, grad, m, v, step, n):
         L = lib()
-        if self.kind == "bf16":
-            s, f, dt, tag = scalars(step, self.lr, self.betas, self.eps, self.weight_decay), ctypes.c_float, np.uint16, "bf16"
+        if self.kind in ("bf16", "f16"):
+            s, f, dt, tag = scalars(step, self.lr, self.betas, self.eps, self.weight_decay), ctypes.c_float, np.uint16, self.kind
         else:
             s, f, dt, tag = scalars_f64(step, self.lr, self.betas, self.eps, self.weight_decay), ctypes.c_double, np.float64, "f64"
         head = (_p(param, dt), _p(grad, dt), _p(m, dt), _p(v, dt), ctypes.c_int64(n), ctypes.c_int(s["use_decay"]),

@@ -216,44 +216,46 @@ void orc_adamw_f64(double* p, const double* g, double* m, double* v, int64_t n, 
   }
 }
 
-/* ---- AdamW on bfloat16 shards (bit patterns). Every one of the torch operations of tandem/optim.py:28-37 reads
- * bf16 tensors, computes in fp32 (ATen's opmath; the Python scalars rounded to fp32, not to bf16) and writes a bf16
- * tensor, so the result is rounded to nearest even after EACH operation: p*decay; the lerp; v*beta2; the addcmul;
+/* ---- AdamW on bfloat16 and float16 shards (bit patterns). Every one of the torch operations of tandem/optim.py:28-37 reads
+ * 16-bit tensors, computes in fp32 (ATen's opmath; the Python scalars rounded to fp32, not to the 16-bit type) and writes a
+ * 16-bit tensor, so the result is rounded to nearest even after EACH operation: p*decay; the lerp; v*beta2; the addcmul;
  * the sqrt; the division; + eps; the addcdiv. One scalar is narrower than the others: add_(eps) adds eps ROUNDED TO
- * BF16 (ATen wraps the scalar of an add in the tensor's dtype), where mul_, lerp_, addcmul_, the division and addcdiv_
+ * THE 16-BIT TYPE (float16 turns the usual 1e-8 into 0, and an element whose gradients were all zero into 0/0) (ATen wraps the scalar of an add in the tensor's dtype), where mul_, lerp_, addcmul_, the division and addcdiv_
  * take theirs as fp32 (checked operation by operation against torch's CPU kernels on values where the two differ).
  * Inside an operation the fp32 arithmetic is that of the fp32 kernels
  * above. As for fp32 the step comes in two phases, so that a test can put torch's own bf16 square roots between them. */
-#define RB(x) bf16_to_f32(f32_to_bf16(x))
-void orc_adamw_moments_bf16(uint16_t* p, const uint16_t* g, uint16_t* m, uint16_t* v, int64_t n, int use_decay,
-                            float decay, float w1, float beta2, float one_m_b2) {
-  for (int64_t i = 0; i < n; ++i) {
-    const float G = bf16_to_f32(g[i]);
-    float M = bf16_to_f32(m[i]), V = bf16_to_f32(v[i]);
-    if (use_decay) p[i] = f32_to_bf16(bf16_to_f32(p[i]) * decay);
-    const float diff = G - M; /* inside lerp_: not rounded to bf16 */
-    m[i] = f32_to_bf16(fabsf(w1) < 0.5f ? fmaf(w1, diff, M) : fmaf(w1 - 1.0f, diff, G));
-    V = RB(V * beta2);
-    v[i] = f32_to_bf16(fmaf(one_m_b2 * G, G, V));
+/* The three functions for one 16-bit type: NAME = bf16 or f16, W widens its bit pattern to fp32, N narrows (nearest even). */
+#define ADAMW_16(NAME, W, N)                                                                                              \
+  void orc_adamw_moments_##NAME(uint16_t* p, const uint16_t* g, uint16_t* m, uint16_t* v, int64_t n, int use_decay,       \
+                                float decay, float w1, float beta2, float one_m_b2) {                                     \
+    for (int64_t i = 0; i < n; ++i) {                                                                                     \
+      const float G = W(g[i]);                                                                                            \
+      float M = W(m[i]), V = W(v[i]);                                                                                     \
+      if (use_decay) p[i] = N(W(p[i]) * decay);                                                                           \
+      const float diff = G - M; /* inside lerp_: not rounded to the 16-bit type */                                        \
+      m[i] = N(fabsf(w1) < 0.5f ? fmaf(w1, diff, M) : fmaf(w1 - 1.0f, diff, G));                                          \
+      V = W(N(V * beta2));                                                                                                \
+      v[i] = N(fmaf(one_m_b2 * G, G, V));                                                                                 \
+    }                                                                                                                     \
+  }                                                                                                                       \
+  void orc_adamw_apply_##NAME(uint16_t* p, const uint16_t* m, const uint16_t* sqrt_v, int64_t n, float bc2_sqrt,          \
+                              float eps, float neg_step) {                                                                \
+    for (int64_t i = 0; i < n; ++i) {                                                                                     \
+      float D = W(N(W(sqrt_v[i]) / bc2_sqrt));                                                                            \
+      D = W(N(D + W(N(eps))));                                                                                            \
+      p[i] = N(W(p[i]) + (neg_step * W(m[i])) / D);                                                                       \
+    }                                                                                                                     \
+  }                                                                                                                       \
+  void orc_adamw_##NAME(uint16_t* p, const uint16_t* g, uint16_t* m, uint16_t* v, int64_t n, int use_decay, float decay,  \
+                        float w1, float beta2, float one_m_b2, float bc2_sqrt, float eps, float neg_step) {               \
+    orc_adamw_moments_##NAME(p, g, m, v, n, use_decay, decay, w1, beta2, one_m_b2);                                       \
+    for (int64_t i = 0; i < n; ++i) {                                                                                     \
+      float D = W(N(sqrtf(W(v[i]))));                                                                                     \
+      D = W(N(D / bc2_sqrt));                                                                                             \
+      D = W(N(D + W(N(eps))));                                                                                            \
+      p[i] = N(W(p[i]) + (neg_step * W(m[i])) / D);                                                                       \
+    }                                                                                                                     \
   }
-}
 
-void orc_adamw_apply_bf16(uint16_t* p, const uint16_t* m, const uint16_t* sqrt_v, int64_t n, float bc2_sqrt, float eps,
-                          float neg_step) {
-  for (int64_t i = 0; i < n; ++i) {
-    float D = RB(bf16_to_f32(sqrt_v[i]) / bc2_sqrt);
-    D = RB(D + RB(eps));
-    p[i] = f32_to_bf16(bf16_to_f32(p[i]) + (neg_step * bf16_to_f32(m[i])) / D);
-  }
-}
-
-void orc_adamw_bf16(uint16_t* p, const uint16_t* g, uint16_t* m, uint16_t* v, int64_t n, int use_decay, float decay,
-                    float w1, float beta2, float one_m_b2, float bc2_sqrt, float eps, float neg_step) {
-  orc_adamw_moments_bf16(p, g, m, v, n, use_decay, decay, w1, beta2, one_m_b2);
-  for (int64_t i = 0; i < n; ++i) {
-    float D = RB(sqrtf(bf16_to_f32(v[i])));
-    D = RB(D / bc2_sqrt);
-    D = RB(D + RB(eps));
-    p[i] = f32_to_bf16(bf16_to_f32(p[i]) + (neg_step * bf16_to_f32(m[i])) / D);
-  }
-}
+ADAMW_16(bf16, bf16_to_f32, f32_to_bf16)
+ADAMW_16(f16, f16_to_f32, f32_to_f16)

@@ -60,9 +60,9 @@ SegPlan plan_fold(const tdm_fold_seg& s, int es) {
 }
 
 // The element size of a step segment: its dtype field names TDM_F32 (0, what a caller that knows nothing of the field
-// leaves there), TDM_F64 or TDM_BF16; 0 for anything else.
+// leaves there), TDM_F64, TDM_BF16 or TDM_F16; 0 for anything else.
 int step_elem_size(const tdm_step_seg& s) {
-  return s.dtype == TDM_F32 ? 4 : s.dtype == TDM_F64 ? 8 : s.dtype == TDM_BF16 ? 2 : 0;
+  return s.dtype == TDM_F32 ? 4 : s.dtype == TDM_F64 ? 8 : (s.dtype == TDM_BF16 || s.dtype == TDM_F16) ? 2 : 0;
 }
 
 SegPlan plan_step(const tdm_step_seg& s) {
@@ -75,7 +75,7 @@ SegPlan plan_step(const tdm_step_seg& s) {
   if (s.exp_avg) ptrs[n++] = reinterpret_cast<uintptr_t>(s.exp_avg);
   if (s.exp_avg_sq) ptrs[n++] = reinterpret_cast<uintptr_t>(s.exp_avg_sq);
   const int es = step_elem_size(s);
-  if (es == 0) throw Invalid("a step segment's dtype must be TDM_F32, TDM_F64 or TDM_BF16");
+  if (es == 0) throw Invalid("a step segment's dtype must be TDM_F32, TDM_F64, TDM_BF16 or TDM_F16");
   return plan_segment(ptrs, n, s.count, es, static_cast<int64_t>(kTileVecs) * (16 / es));
 }
 
@@ -1136,6 +1136,24 @@ int tdm_k3_adamw_gather(float* p, const float* g, float* m, float* v, int64_t n,
 
 extern "C++" {
 namespace {
+// eps as add_(eps) applies it to a 16-bit tensor: rounded to the tensor's type (nearest even), as a float again.
+template <typename T>
+float eps_as_applied(double eps) {
+  const float e = static_cast<float>(eps);
+  if constexpr (std::is_same_v<T, bf16_t>) {
+    uint32_t u;
+    std::memcpy(&u, &e, 4);
+    u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+    float rounded;
+    std::memcpy(&rounded, &u, 4);
+    return rounded;
+  } else if constexpr (std::is_same_v<T, f16_t>) {
+    return static_cast<float>(static_cast<_Float16>(e));
+  } else {
+    return e;
+  }
+}
+
 template <typename T>
 void adamw_typed_launch(void* p_, const void* g_, void* m_, void* v_, int64_t n, const tdm_adamw_hyper& h, void* const* copies,
                         int ncopies, hipStream_t st) {
@@ -1150,15 +1168,7 @@ void adamw_typed_launch(void* p_, const void* g_, void* m_, void* v_, int64_t n,
   a.s.decay = static_cast<S>(h.decay), a.s.w1 = static_cast<S>(h.w1), a.s.beta2 = static_cast<S>(h.beta2);
   a.s.one_m_b2 = static_cast<S>(h.one_m_b2), a.s.bc2_sqrt = static_cast<S>(h.bc2_sqrt), a.s.neg_step = static_cast<S>(h.neg_step);
   a.s.eps = static_cast<S>(h.eps);
-  if constexpr (std::is_same_v<T, bf16_t>) {  // add_(eps) on a bf16 tensor adds eps rounded to bf16 (nearest even)
-    uint32_t u;
-    const float e = static_cast<float>(h.eps);
-    std::memcpy(&u, &e, 4);
-    u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
-    float rounded;
-    std::memcpy(&rounded, &u, 4);
-    a.s.eps = rounded;
-  }
+  if constexpr (sizeof(T) == 2) a.s.eps = eps_as_applied<T>(h.eps);
   a.ncopies = ncopies;
   a.shift = xcd_shift(TDM_XCD_ADAMW, 1, true);
   for (int c = 0; c < ncopies; ++c) {
@@ -1193,7 +1203,7 @@ void adamw_typed_launch(void* p_, const void* g_, void* m_, void* v_, int64_t n,
   // SIMD that suits the memory-bound fp32 and fp64 kernels costs it 5 %: four 21.46M-element shards take 0.243 ms with 8 KiB,
   // 0.255 with none, 0.257 with 24 KiB.
   const int set = g_occupancy_pad[TDM_XCD_ADAMW].load(std::memory_order_relaxed);
-  const unsigned pad = set >= 0 ? static_cast<unsigned>(set) : std::is_same_v<T, bf16_t> ? 8192u : occupancy_pad(TDM_XCD_ADAMW);
+  const unsigned pad = set >= 0 ? static_cast<unsigned>(set) : sizeof(T) == 2 ? 8192u : occupancy_pad(TDM_XCD_ADAMW);
   switch ((vec ? 2 : 0) + (ncopies > 0 ? 1 : 0)) {
     case 0: hipLaunchKernelGGL((k3_adamw_typed_kernel<T, false, false>), grid, block, pad, st, a); break;
     case 1: hipLaunchKernelGGL((k3_adamw_typed_kernel<T, false, true>), grid, block, pad, st, a); break;
@@ -1210,7 +1220,7 @@ int tdm_k3_adamw_typed(void* p, const void* g, void* m, void* v, int64_t n, int 
   return guard([&] {
     if (n < 0) throw Invalid("n is negative");
     if (ncopies < 0 || ncopies > TDM_MAX_WORLD - 1) throw Invalid("at most 7 further copies of the parameters");
-    if (dtype != TDM_F32 && dtype != TDM_F64 && dtype != TDM_BF16) throw Invalid("AdamW handles fp32, fp64 and bf16 shards (dtype " + std::to_string(dtype) + ")");
+    if (dtype != TDM_F32 && dtype != TDM_F64 && dtype != TDM_BF16 && dtype != TDM_F16) throw Invalid("AdamW handles fp32, fp64, bf16 and fp16 shards (dtype " + std::to_string(dtype) + ")");
     if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
     if (n == 0) return;
     if (!p || !g || !m || !v || !h || (ncopies > 0 && !copies)) throw Invalid("NULL argument");
@@ -1225,7 +1235,8 @@ int tdm_k3_adamw_typed(void* p, const void* g, void* m, void* v, int64_t n, int 
     }
     if (order != TDM_ADAMW_HOST_ORDER) throw Invalid("the device order is defined for fp32 shards only");
     if (dtype == TDM_F64) adamw_typed_launch<double>(p, g, m, v, n, *h, copies, ncopies, st);
-    else adamw_typed_launch<bf16_t>(p, g, m, v, n, *h, copies, ncopies, st);
+    else if (dtype == TDM_BF16) adamw_typed_launch<bf16_t>(p, g, m, v, n, *h, copies, ncopies, st);
+    else adamw_typed_launch<f16_t>(p, g, m, v, n, *h, copies, ncopies, st);
   });
 }
 
@@ -1249,7 +1260,7 @@ int tdm_k23_table_build(const tdm_step_seg* segs, int nseg, int world, void* ima
     std::memset(image, 0, static_cast<size_t>(tdm_k23_table_bytes(segs, nseg)));
     StepSegDev* out = static_cast<StepSegDev*>(image);
     const int es = nseg > 0 ? step_elem_size(segs[0]) : 4;
-    if (es == 0) throw Invalid("a step segment's dtype must be TDM_F32, TDM_F64 or TDM_BF16");
+    if (es == 0) throw Invalid("a step segment's dtype must be TDM_F32, TDM_F64, TDM_BF16 or TDM_F16");
     const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
     int64_t tiles = 0;
     for (int i = 0; i < nseg; ++i) {
@@ -1319,19 +1330,14 @@ void launch_step_typed_w(const void* image, int64_t tiles, int average, const td
   using S = typename AdamwMath<T>::S;
   AdamwHyper<S> s{h.use_decay, static_cast<S>(h.decay), static_cast<S>(h.w1), static_cast<S>(h.beta2), static_cast<S>(h.one_m_b2),
                   static_cast<S>(h.bc2_sqrt), static_cast<S>(h.eps), static_cast<S>(h.neg_step)};
-  if constexpr (std::is_same_v<T, bf16_t>) {  // add_(eps) on a bf16 tensor adds eps rounded to bf16 (nearest even)
-    uint32_t u;
-    std::memcpy(&u, &s.eps, 4);
-    u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
-    std::memcpy(&s.eps, &u, 4);
-  }
+  if constexpr (sizeof(T) == 2) s.eps = eps_as_applied<T>(h.eps);
   const Divisor<T> dv = make_divisor<T>(kWorld);
   const StepSegDev* t = static_cast<const StepSegDev*>(image);
   const dim3 grid(grid_for(tiles * kStepParts)), block(kThreads);
   // bf16 carries more arithmetic per byte and does better with more waves than the fp32 and fp64 steps: the 85.8M-parameter
   // step at world 4 takes 0.357-0.360 ms with a pad of 0-16 KiB and 0.399 with the family's 24 KiB.
   const int set = g_occupancy_pad[TDM_XCD_STEP].load(std::memory_order_relaxed);
-  const unsigned pad = set >= 0 ? static_cast<unsigned>(set) : std::is_same_v<T, bf16_t> ? 16384u : occupancy_pad(TDM_XCD_STEP);
+  const unsigned pad = set >= 0 ? static_cast<unsigned>(set) : sizeof(T) == 2 ? 16384u : occupancy_pad(TDM_XCD_STEP);
   const int shift = xcd_shift(TDM_XCD_STEP, kWorld, true);
   switch (div_kind(kWorld, average != 0)) {
     case 0: hipLaunchKernelGGL((k23_zero2_step_typed_kernel<T, kWorld, 0>), grid, block, pad, stream, t, tiles, dv, s, shift); break;
@@ -1361,7 +1367,7 @@ int tdm_k23_zero2_step_typed(const void* table_dev, int64_t ntiles, int world, i
                              int order, tdm_stream stream) {
   return guard([&] {
     if (ntiles < 0) throw Invalid("ntiles is negative");
-    if (dtype != TDM_F32 && dtype != TDM_F64 && dtype != TDM_BF16) throw Invalid("the step handles fp32, fp64 and bf16 shards (dtype " + std::to_string(dtype) + ")");
+    if (dtype != TDM_F32 && dtype != TDM_F64 && dtype != TDM_BF16 && dtype != TDM_F16) throw Invalid("the step handles fp32, fp64, bf16 and fp16 shards (dtype " + std::to_string(dtype) + ")");
     if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
     if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
     if (ntiles == 0) return;
@@ -1377,7 +1383,8 @@ int tdm_k23_zero2_step_typed(const void* table_dev, int64_t ntiles, int world, i
     }
     if (order != TDM_ADAMW_HOST_ORDER) throw Invalid("the device order is defined for fp32 shards only");
     if (dtype == TDM_F64) launch_step_typed<double>(table_dev, ntiles, world, average, *h, st);
-    else launch_step_typed<bf16_t>(table_dev, ntiles, world, average, *h, st);
+    else if (dtype == TDM_BF16) launch_step_typed<bf16_t>(table_dev, ntiles, world, average, *h, st);
+    else launch_step_typed<f16_t>(table_dev, ntiles, world, average, *h, st);
     check_hip(hipGetLastError(), "k23_zero2_step (typed) launch");
   });
 }

@@ -787,10 +787,10 @@ __global__ __launch_bounds__(kAdamwThreads) void k3_adamw_kernel(AdamwArgs a) {
 
 // ---------------------------------------------------------------- K3 on other element types
 // The reference's update is seven torch operations that take any floating dtype (tandem/optim.py:28-37).
-// float64: the same arithmetic on doubles, the step's scalars unrounded. bfloat16: every operation reads
-// bf16, computes in fp32 and writes bf16, so the value is rounded to nearest even after EACH operation;
-// add_(eps) adds eps rounded to bf16 (ATen wraps that scalar in the tensor's dtype), the other scalars act
-// as fp32. Host order only: these follow torch's CPU kernels, which is what the reference's engine runs.
+// float64: the same arithmetic on doubles, the step's scalars unrounded. bfloat16 and float16: every operation
+// reads the 16-bit type, computes in fp32 and writes the 16-bit type, so the value is rounded to nearest even
+// after EACH operation; add_(eps) adds eps rounded to the type (ATen wraps that scalar in the tensor's dtype),
+// the other scalars act as fp32. Host order only: these follow torch's CPU kernels, which is what the reference's engine runs.
 template <typename S>
 struct AdamwHyper {
   int use_decay;
@@ -812,38 +812,69 @@ template <> struct AdamwMath<double> {
   }
 };
 
-template <> struct AdamwMath<bf16_t> {
-  using S = float;
-  // x rounded to bf16 (nearest even) and back, by the conversion instruction (v_cvt_pk_bf16_f32) instead of the seven integer
-  // operations of Elem<bf16_t>::narrow: this kernel rounds eight times per element and is bound by its arithmetic, not by
-  // memory. A NaN stays a NaN here; what is stored goes through narrow(), which makes it the canonical one.
+// The two 16-bit types share the step; they differ in how a float is rounded to the type and back (a conversion
+// instruction either way: v_cvt_pk_bf16_f32, v_cvt_f16_f32) and in the canonical NaN that is stored.
+template <typename T> struct Round16;
+template <> struct Round16<bf16_t> {
   static __device__ __forceinline__ float rb(float x) {
     const __bf16 h = static_cast<__bf16>(x);
     return static_cast<float>(h);
   }
-  static __device__ __forceinline__ void step(bf16_t& p, bf16_t g, bf16_t& m, bf16_t& v, const AdamwHyper<float>& s, bool small_w) {
-    float P = Elem<bf16_t>::widen(p), M = Elem<bf16_t>::widen(m), V = Elem<bf16_t>::widen(v);
-    const float G = Elem<bf16_t>::widen(g);
-    if (s.use_decay) P = rb(P * s.decay);
+  // the bits of a float that rb() has already rounded: its upper half
+  static __device__ __forceinline__ uint16_t bits(float x) { return static_cast<uint16_t>(__float_as_uint(x) >> 16); }
+  static constexpr uint16_t kNan = 0x7fc0u;
+};
+template <> struct Round16<f16_t> {
+  // The float must exist as a float before it is narrowed: left to itself the compiler folds the multiplication or
+  // fused multiply-add that produced it into a mixed-precision instruction that rounds the exact result to f16 ONCE,
+  // where torch rounds to fp32 and then to f16. With operands that are not all f16 values (beta2, the step's other
+  // constants) the two differ on ties: 10 ulps x f32(0.95) is 9.49999988 exactly, 9.5 as a float, and rounds to 9 the
+  // one way and to 10 the other. The empty asm is the barrier; it emits nothing.
+  static __device__ __forceinline__ float rb(float x) {
+    asm volatile("" : "+v"(x));
+    const _Float16 h = static_cast<_Float16>(x);
+    return static_cast<float>(h);
+  }
+  static __device__ __forceinline__ uint16_t bits(float x) {  // exact: x is representable
+    const _Float16 h = static_cast<_Float16>(x);
+    uint16_t b;
+    __builtin_memcpy(&b, &h, 2);
+    return b;
+  }
+  static constexpr uint16_t kNan = 0x7e00u;
+};
+
+// x is rounded to the 16-bit type and back by the conversion instruction instead of the integer operations of
+// Elem<T>::narrow: this kernel rounds eight times per element and is bound by its arithmetic, not by memory. A NaN
+// stays a NaN through the roundings; what is stored is the canonical one, as narrow() makes it.
+template <typename T>
+struct AdamwMath16 {
+  using S = float;
+  using R = Round16<T>;
+  static __device__ __forceinline__ void step(T& p, T g, T& m, T& v, const AdamwHyper<float>& s, bool small_w) {
+    float P = Elem<T>::widen(p), M = Elem<T>::widen(m), V = Elem<T>::widen(v);
+    const float G = Elem<T>::widen(g);
+    if (s.use_decay) P = R::rb(P * s.decay);
     const float diff = G - M;  // inside lerp_: not rounded
-    M = rb(small_w ? __builtin_fmaf(s.w1, diff, M) : __builtin_fmaf(s.w1 - 1.0f, diff, G));
-    V = rb(V * s.beta2);
-    V = rb(__builtin_fmaf(s.one_m_b2 * G, G, V));
-    float D = rb(__builtin_sqrtf(V));
-    D = rb(D / s.bc2_sqrt);
-    D = rb(D + s.eps);  // s.eps arrives rounded to bf16
-    P = rb(P + (s.neg_step * M) / D);
+    M = R::rb(small_w ? __builtin_fmaf(s.w1, diff, M) : __builtin_fmaf(s.w1 - 1.0f, diff, G));
+    V = R::rb(V * s.beta2);
+    V = R::rb(__builtin_fmaf(s.one_m_b2 * G, G, V));
+    float D = R::rb(__builtin_sqrtf(V));
+    D = R::rb(D / s.bc2_sqrt);
+    D = R::rb(D + s.eps);  // s.eps arrives rounded to the 16-bit type
+    P = R::rb(P + (s.neg_step * M) / D);
     p = exact(P);
     m = exact(M);
     v = exact(V);
   }
-  // The bits of a float that rb() has already rounded: its upper half; a NaN becomes the canonical one, as narrow() makes it.
-  static __device__ __forceinline__ bf16_t exact(float x) {
-    bf16_t out;
-    out.bits = x != x ? static_cast<uint16_t>(0x7fc0u) : static_cast<uint16_t>(__float_as_uint(x) >> 16);
+  static __device__ __forceinline__ T exact(float x) {
+    T out;
+    out.bits = x != x ? R::kNan : R::bits(x);
     return out;
   }
 };
+template <> struct AdamwMath<bf16_t> : AdamwMath16<bf16_t> {};
+template <> struct AdamwMath<f16_t> : AdamwMath16<f16_t> {};
 
 template <typename T>
 struct AdamwArgsT {

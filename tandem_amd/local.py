@@ -247,7 +247,7 @@ class LocalZeRO2:
 
     def __init__(self, world, numels, device, bucket_bytes=25 << 20, order="host", one_allocation=False, dtype=torch.float32,
                  **adamw):
-        """dtype: the element type of parameters, gradients and optimizer state: fp32, float64 or bfloat16 (the last two in
+        """dtype: the element type of parameters, gradients and optimizer state: fp32, float64, bfloat16 or float16 (all but fp32 in
         host order; their gradients are reduced by the fold, which rounds every addition to the type as the ring does).
         one_allocation: every buffer (the ranks' parameters and gradients, the gradient shards, the optimizer
         state) is carved out of a single allocation, back to back at 128-byte boundaries, instead of being an
@@ -259,7 +259,7 @@ class LocalZeRO2:
         from .optim import SHARD_DTYPES
 
         if dtype not in SHARD_DTYPES:
-            raise ValueError(f"LocalZeRO2 handles fp32, float64 and bfloat16 (got {dtype})")
+            raise ValueError(f"LocalZeRO2 handles fp32, float64, bfloat16 and float16 (got {dtype})")
         es = torch.empty(0, dtype=dtype).element_size()
         self.dtype = dtype
         self.lw = LocalWorld(world)

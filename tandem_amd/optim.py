@@ -5,8 +5,8 @@ Same interface as tandem's ShardedAdamW (tandem/optim.py:11-40 there) and the
 same arithmetic, operation for operation: the step's scalars are computed in
 Python doubles by the same expressions and applied in the shard's own
 arithmetic, as torch does with a Python scalar. fp32 shards: the scalars are
-rounded to fp32 once (tdm_k3_adamw). float64: doubles throughout. bfloat16:
-each of the seven operations computes in fp32 and rounds to bf16
+rounded to fp32 once (tdm_k3_adamw). float64: doubles throughout. bfloat16 and
+float16: each of the seven operations computes in fp32 and rounds to the type
 (tdm_k3_adamw_typed)."""
 
 import ctypes
@@ -16,7 +16,7 @@ import torch
 from ._lib import (ADAMW_DEVICE_ORDER, ADAMW_HOST_ORDER, AdamwHyper, AdamwScalars, check, dtype_code, lib, require_device_tensor,
                    stream_ptr)
 
-SHARD_DTYPES = (torch.float32, torch.float64, torch.bfloat16)
+SHARD_DTYPES = (torch.float32, torch.float64, torch.bfloat16, torch.float16)
 
 
 def step_scalars(step, lr, betas, eps, weight_decay):
@@ -89,7 +89,7 @@ class ShardedAdamW:
 
     def update(self, key, param, grad, copies=()):
         """One step for one shard: `param` and `grad` are same-shaped tensors in GPU
-        memory, fp32, float64 or bfloat16 (the last two in host order only);
+        memory, fp32, float64, bfloat16 or float16 (all but fp32 in host order only);
         `key` names the shard's optimizer state. `copies`:
         further tensors of the same shape (the other ranks' copies of this shard, when
         the ranks are buffers in one memory) that receive the updated parameters in the
@@ -101,7 +101,7 @@ class ShardedAdamW:
             if c.dtype != param.dtype or c.shape != param.shape:
                 raise ValueError("a copy differs from param in dtype or shape")
         if param.dtype not in SHARD_DTYPES or grad.dtype != param.dtype:
-            raise ValueError(f"ShardedAdamW handles fp32, float64 and bfloat16 shards whose gradient has the same dtype (got {param.dtype}, {grad.dtype})")
+            raise ValueError(f"ShardedAdamW handles fp32, float64, bfloat16 and float16 shards whose gradient has the same dtype (got {param.dtype}, {grad.dtype})")
         if param.dtype != torch.float32 and self.order != ADAMW_HOST_ORDER:
             raise ValueError("order=\"device\" is defined for fp32 shards only")
         if param.shape != grad.shape:

@@ -14,8 +14,8 @@ parts of the path that no test of the reference pins by itself:
                       the partial sums left in the other chunks; all_gather).
   ring_dtypes_w3.npz  fp64 / fp16 / bf16 all_reduce at world 3.
   adamw.npz           ShardedAdamW.update, 20 steps, the benchmark's hyper-parameters.
-  adamw_dtypes.npz    the same update on bfloat16 and float64 shards (the reference's seven
-                      torch operations take any floating dtype), both lerp branches.
+  adamw_dtypes.npz    the same update on bfloat16, float16 and float64 shards (the reference's
+                      seven torch operations take any floating dtype), both lerp branches.
   plans.json          DDP / ZeRO bucket packing, shard sizes, bucket_sizes and the
                       GPT's parameter registration order and unit sizes.
   data.json           digests of synthetic() and Text.batch().
@@ -167,7 +167,7 @@ def write_adamw():
 
 
 def write_adamw_dtypes():
-    """ShardedAdamW.update on bf16 and f64 tensors: 20 steps with the benchmark's hyper-parameters, and 3 steps
+    """ShardedAdamW.update on bf16, f16 and f64 tensors: 20 steps with the benchmark's hyper-parameters, and 3 steps
     of the other branches (beta1 < 0.5, no weight decay). 16-bit tensors are stored as bit patterns."""
     n, steps = 773, 20
     torch.set_num_threads(1)
@@ -178,7 +178,7 @@ def write_adamw_dtypes():
 
     hyper = {"main": {"lr": 3e-4, "betas": [0.9, 0.95], "eps": 1e-8, "weight_decay": 0.1, "steps": steps},
              "other": {"lr": 1e-2, "betas": [0.3, 0.7], "eps": 1e-6, "weight_decay": 0.0, "steps": 3}}
-    for name, dt in (("bf16", torch.bfloat16), ("f64", torch.float64)):
+    for name, dt in (("bf16", torch.bfloat16), ("f16", torch.float16), ("f64", torch.float64)):
         g = torch.Generator().manual_seed(21)
         p0 = (torch.randn(n, generator=g, dtype=torch.float64) * 0.02).to(dt)
         p0[:4] = torch.tensor([0.0, -0.0, 1e-30, -3e-39], dtype=torch.float64).to(dt)

@@ -130,7 +130,7 @@ def _raw(t):
 
 @pytest.mark.parametrize("algorithm", ["fold", "ring", "fused"])
 @pytest.mark.parametrize("world", [2, 4, 3])
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float64])
 def test_other_shard_dtypes_bit_exact_with_oracle(dtype, world, algorithm):
     """The ZeRO-2 step over bfloat16 and float64 models (the reference's classes and its seven-operation AdamW take
     any floating dtype, tandem/zero.py:69-170, tandem/optim.py:28-37): per-bucket ring reduce-scatter in the type's own
@@ -143,14 +143,15 @@ def test_other_shard_dtypes_bit_exact_with_oracle(dtype, world, algorithm):
     from tandem_amd.local import LocalZeRO2
 
     dev = torch.device("cuda", 0)
-    kind = "bf16" if dtype == torch.bfloat16 else "f64"
-    es = 2 if kind == "bf16" else 8
+    kind = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float64: "f64"}[dtype]
+    es = 8 if kind == "f64" else 2
     numels = [4099, 10_007, 33, 5001, 1, 12_288, 782]
     n = sum(numels)
     steps = 4
     kw = dict(lr=1e-3, betas=(0.9, 0.95), eps=1e-6, weight_decay=0.1)
     p0 = (seeded(3, 0, n).double() * 0.02).to(dtype)
-    grads = [[(seeded(30 + s, r, n).double() * 1e-3).to(dtype) for r in range(world)] for s in range(steps)]
+    scale = 1e-3 if kind != "f16" else 2e-2  # float16 holds the squares of these; smaller ones only as subnormals or zero
+    grads = [[(seeded(30 + s, r, n).double() * scale).to(dtype) for r in range(world)] for s in range(steps)]
     for g in grads[0]:
         g[:4] = torch.tensor([0.0, -0.0, 1e-30, -1e-30], dtype=torch.float64).to(dtype)
     z = LocalZeRO2(world, numels, dev, bucket_bytes=16 << 10, dtype=dtype, **kw)
@@ -170,7 +171,7 @@ def test_other_shard_dtypes_bit_exact_with_oracle(dtype, world, algorithm):
     # the same step written with the oracle only
     lay = [FlatLayout(numels, world, r) for r in range(world)]
     bufs = [_raw(p0) for _ in range(world)]
-    opts = [AdamW(**kw, kind="bf16" if kind == "bf16" else None) for _ in range(world)]
+    opts = [AdamW(**kw, kind=kind if kind != "f64" else None) for _ in range(world)]
     for s in range(steps):
         gs = [_raw(g) for g in grads[s]]
         shards = [np.zeros(l.hi - l.lo, bufs[0].dtype) for l in lay]
@@ -181,7 +182,7 @@ def test_other_shard_dtypes_bit_exact_with_oracle(dtype, world, algorithm):
             for c, m in enumerate(sizes):
                 if m:
                     mine = outs[c][lo - a:lo - a + m].copy()
-                    if kind == "bf16":
+                    if kind != "f64":
                         mine[mine == 0x8000] = 0  # 0 + (-0) = +0, as grad_shard.add_(mine) leaves it; nothing else changes
                     else:
                         mine = 0.0 + mine
