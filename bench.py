@@ -1005,7 +1005,10 @@ def main():
     torch.cuda.empty_cache()
     if not args.quick:
         if not only or "mix" in only:
-            line["stream_mix"] = stream_mix(dev, 6)
+            try:  # the probe is a library of its own; without it the line simply lacks the mix ceilings
+                line["stream_mix"] = stream_mix(dev, 6)
+            except Exception as e:
+                line["stream_mix_error"] = repr(e)[:300]
             torch.cuda.empty_cache()
         if not only or "sweep" in only:
             line["sweep"] = sweep(lw, dev, max(5, args.steps // 2))
