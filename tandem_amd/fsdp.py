@@ -55,10 +55,10 @@ class ShardHome:
     one arena tensor of the same size on every rank (so it has the same arena offset everywhere),
     large enough for the rank whose shards of the slab's units are longest; within a slab a unit's
     shard starts at the same element offset on every rank only when all earlier shards had equal
-    sizes, so the offsets are kept per rank. Shards start on 16-byte boundaries. An arena is one
+    sizes, so the offsets are kept per rank. Shards start on 128-byte boundaries (cache lines). An arena is one
     exported allocation and stays under 2 GiB, so a slab ends before SLAB_BYTES."""
 
-    ALIGN = 4  # elements (fp32)
+    ALIGN_BYTES = 128  # every shard starts on a cache line: the gather and the update then move whole lines
     SLAB_BYTES = 1 << 30
 
     def __init__(self, group, unit_sizes, dtype):
@@ -70,7 +70,8 @@ class ShardHome:
         self.slab_of, self.at = [], []  # per unit: its slab, and the element offset of the shard within it on every rank
         extents, ends = [], [0] * world
         for sizes in unit_sizes:
-            padded = [-(-s // self.ALIGN) * self.ALIGN for s in sizes]
+            per = max(self.ALIGN_BYTES // self.es, 1)
+            padded = [-(-s // per) * per for s in sizes]
             if max(ends) > 0 and max(e + p for e, p in zip(ends, padded)) > cap:
                 extents.append(max(ends))
                 ends = [0] * world

@@ -212,12 +212,12 @@ def test_shard_home_lays_units_out_in_slabs(seed, monkeypatch):
             offs = home.peer_offsets(k)
             assert offs == homes[0][0].peer_offsets(k)  # the same on every rank
             if sizes[r]:
-                assert g.arena_offset(shard) == offs[r] and offs[r] % 16 == 0
+                assert g.arena_offset(shard) == offs[r] and offs[r] % 128 == 0
                 spans.append((offs[r], offs[r] + 4 * sizes[r]))
         spans.sort()
         assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
         for slab in home.slabs:
-            alone = any(max(-(-s // 4) * 4 for s in sizes) >= slab.numel() for sizes in units)
+            alone = any(max(-(-s // 32) * 32 for s in sizes) >= slab.numel() for sizes in units)
             assert slab.numel() <= cap or alone
 
 
