@@ -128,6 +128,16 @@ class Group:
             raise CommError(f"could not start the hip engine: {e}") from e
         self.barrier()
 
+    @staticmethod
+    def make_sync(ctx, size, slots):
+        """What a launcher creates once and every rank inherits, with the reference's signature and shape
+        (tandem/comm.py:175-181 there): (full, free, barrier). The hip engine hands pieces over through its own
+        shared-memory rings, so only the barrier is used; the two semaphore lists are there so that code written
+        for the reference's launcher runs unchanged."""
+        full = [ctx.Semaphore(0) for _ in range(size * size)]
+        free = [ctx.Semaphore(slots) for _ in range(size * size)]
+        return full, free, ctx.Barrier(size)
+
     # ---- tracing (tandem/comm.py:132-134 there: trace, waits, tracing)
     @property
     def tracing(self):

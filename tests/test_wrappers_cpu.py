@@ -327,3 +327,16 @@ def test_zero_waits_for_its_all_gather_on_the_host_unless_asked():
         g.waits.clear()
         z.step()
         assert g.waits == [want], (ordered, g.waits)
+
+
+def test_make_sync_has_the_references_shape():
+    """Group.make_sync(ctx, size, slots) -> (full, free, barrier), as the reference's launcher calls it
+    (tandem/comm.py:175-181,537 there); the Group takes the tuple or the barrier alone."""
+    import multiprocessing as mp
+
+    from tandem_amd import Group
+
+    full, free, barrier = Group.make_sync(mp.get_context("spawn"), 3, 2)
+    assert len(full) == len(free) == 9 and barrier.parties == 3
+    assert not full[0].acquire(block=False) and free[0].acquire(block=False) and free[0].acquire(block=False)
+    assert not free[0].acquire(block=False)
