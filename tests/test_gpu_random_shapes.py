@@ -269,3 +269,95 @@ def test_seeded_sweep_of_zero2_steps():
                         assert torch.equal(zs[0].opts[r].state["flat"][i].view(torch.int32), other.opts[r].state["flat"][i].view(torch.int32)), (label, r, i)
         for r in range(1, world):
             assert torch.equal(zs[2].bufs[0].view(torch.int32), zs[2].bufs[r].view(torch.int32)), label
+
+
+def _raw_any(t):
+    t = t.detach().cpu()
+    return t.view(torch.int16).numpy().view(np.uint16).copy() if t.element_size() == 2 else t.numpy().copy()
+
+
+def test_seeded_sweep_of_adamw_shards_of_other_dtypes():
+    """The same sweep over float64, bfloat16 and float16 shards (tdm_k3_adamw_typed): random lengths, parameter,
+    gradient and state views at phases of their own (so that some launches peel to the cache line, some to the vector,
+    some go element by element), random hyper-parameters with an eps and gradients that the 16-bit types can hold, now
+    and then with copies written in the same pass: parameters, both moments and every copy bit for bit the oracle's."""
+    from oracle.adamw import AdamW as Oracle
+    from tandem_amd import ShardedAdamW
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    dev = torch.device("cuda", 0)
+    rng = np.random.default_rng(777)
+    kinds = {torch.float64: None, torch.bfloat16: "bf16", torch.float16: "f16"}
+    for k in range(90):
+        dtype = [torch.float64, torch.bfloat16, torch.float16][k % 3]
+        per_line = 128 // torch.empty(0, dtype=dtype).element_size()
+        n = int(rng.choice([1, 3, 7, 8, 9, 63, 64, 65, 127, 1000, 4097, 33_333])) + int(rng.integers(0, 2))
+        kw = dict(lr=float(10 ** rng.uniform(-4, -2)), betas=(float(rng.choice([0.0, 0.3, 0.5, 0.9])), float(rng.choice([0.7, 0.95, 0.999]))),
+                  eps=float(rng.choice([1e-4, 1e-3])), weight_decay=float(rng.choice([0.0, 0.01, 0.1])))
+        ncopies = int(rng.choice([0, 0, 1, 3]))
+        same = bool(rng.integers(0, 2))  # every stream at one phase, or phases of their own
+        phases = [int(rng.integers(0, per_line))] * (4 + ncopies) if same else [int(rng.integers(0, per_line)) for _ in range(4 + ncopies)]
+        pad = 2 * per_line
+        stores = [torch.full((n + 2 * pad,), -7.0, dtype=dtype, device=dev) for _ in range(4 + ncopies)]
+        views = [s_[pad + ph:pad + ph + n] for s_, ph in zip(stores, phases)]
+        p0 = torch.from_numpy(rng.standard_normal(n) * 0.05).to(dtype)
+        views[0].copy_(p0)
+        ours, ref = ShardedAdamW(**kw), Oracle(**kw, kind=kinds[dtype])
+        ours.state["k"] = [0.0, views[2].zero_(), views[3].zero_()]
+        pn = _raw_any(p0)
+        steps = int(rng.integers(1, 4))
+        for _ in range(steps):
+            g0 = torch.from_numpy(rng.standard_normal(n) * 3e-2).to(dtype)
+            g0[: n // 7] = 0.0
+            views[1].copy_(g0)
+            ours.update("k", views[0], views[1], views[4:])
+            ref.update("k", pn, _raw_any(g0))
+        label = (k, str(dtype), n, kw, phases, ncopies, steps)
+        assert np.array_equal(bits(_raw_any(views[0])), bits(pn)), label
+        assert np.array_equal(bits(_raw_any(views[2])), bits(ref.state["k"][1])), label
+        assert np.array_equal(bits(_raw_any(views[3])), bits(ref.state["k"][2])), label
+        for c in views[4:]:
+            assert np.array_equal(bits(_raw_any(c)), bits(pn)), label
+        for s_, ph in zip(stores, phases):
+            assert float((s_[:pad + ph].double() + 7.0).abs().sum()) == 0 and float((s_[pad + ph + n:].double() + 7.0).abs().sum()) == 0, label
+
+
+def test_seeded_sweep_of_zero2_steps_of_other_dtypes():
+    """The three ways through a ZeRO-2 step over float64, bfloat16 and float16 models, random parameter lists, world
+    sizes 1..8 and bucket sizes: ring steps + AdamW + all-gather, the fold + AdamW writing every copy, and everything in
+    one launch (tdm_k23_zero2_step_typed) must leave the same bits in every rank's parameters and optimizer state."""
+    from tandem_amd.local import LocalZeRO2
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    dev = torch.device("cuda", 0)
+    rng = np.random.default_rng(31)
+    kw = dict(lr=1e-3, betas=(0.9, 0.95), eps=1e-4, weight_decay=0.1)
+    for k in range(36):
+        dtype = [torch.float64, torch.bfloat16, torch.float16][k % 3]
+        world = int(rng.integers(1, 9))
+        numels = [int(rng.choice([1, 2, 5, 64, 257, 1024, 3001, 8192])) + int(rng.integers(0, 2)) for _ in range(int(rng.integers(1, 10)))]
+        bucket_bytes = int(rng.choice([64, 1024, 4096, 1 << 20]))
+        n = sum(numels)
+        zs = [LocalZeRO2(world, numels, dev, bucket_bytes=bucket_bytes, dtype=dtype, **kw) for _ in range(3)]
+        p0 = torch.from_numpy(rng.standard_normal(n) * 0.05).to(dtype).to(dev)
+        for z in zs:
+            for b in z.bufs:
+                b.copy_(p0)
+        for step in range(2):
+            for r in range(world):
+                g = torch.from_numpy(rng.standard_normal(n) * 3e-2).to(dtype).to(dev)
+                for z in zs:
+                    z.staging[r].copy_(g)
+            zs[0].reduce_grads("ring"); zs[0].step(fused_gather=False); zs[0].zero_grad()
+            zs[1].reduce_grads("fold"); zs[1].step(); zs[1].zero_grad()
+            zs[2].reduce_and_step(); zs[2].zero_grad()
+        label = (k, str(dtype), world, numels, bucket_bytes)
+        for other in zs[1:]:
+            for r in range(world):
+                assert np.array_equal(bits(_raw_any(zs[0].bufs[r])), bits(_raw_any(other.bufs[r]))), label
+                if zs[0].grad_shards[r].numel():
+                    for i in (1, 2):
+                        assert np.array_equal(bits(_raw_any(zs[0].opts[r].state["flat"][i])), bits(_raw_any(other.opts[r].state["flat"][i]))), (label, r, i)
+        for r in range(1, world):
+            assert np.array_equal(bits(_raw_any(zs[2].bufs[0])), bits(_raw_any(zs[2].bufs[r]))), label
+        assert np.isfinite(zs[2].bufs[0].double().cpu().numpy()).all(), label
