@@ -102,11 +102,14 @@ class Handle:
         p, self._p = getattr(self, "_p", None), None
         if not p:
             return
-        e = getattr(self, "_engine", None)
-        if e is not None and e._e and self._keep and not self._waited and not _L.tdm_work_done(p):
-            e._orphans.append((p, self._keep))  # not run yet and nobody waited: the tensors must outlive it
-            return
-        _L.tdm_work_free(p)
+        try:
+            e = getattr(self, "_engine", None)
+            if e is not None and e._e and self._keep and not self._waited and not _L.tdm_work_done(p):
+                e._orphans.append((p, self._keep))  # not run yet and nobody waited: the tensors must outlive it
+                return
+            _L.tdm_work_free(p)
+        except Exception:  # the interpreter is going down and has taken the library first
+            pass
 
 
 class Engine:
