@@ -1257,15 +1257,17 @@ int tdm_k23_table_build(const tdm_step_seg* segs, int nseg, int world, void* ima
   return guard([&] {
     if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
     if (nseg < 0 || (nseg > 0 && segs == nullptr) || image == nullptr) throw Invalid("bad table arguments");
+    const int es = nseg > 0 ? step_elem_size(segs[0]) : 4;
+    for (int i = 0; i < nseg; ++i) {  // before anything is sized by them
+      if (step_elem_size(segs[i]) == 0) throw Invalid("segment " + std::to_string(i) + ": a step segment's dtype must be TDM_F32, TDM_F64, TDM_BF16 or TDM_F16");
+      if (segs[i].dtype != segs[0].dtype) throw Invalid("segment " + std::to_string(i) + ": the segments of one table share one dtype");
+    }
     std::memset(image, 0, static_cast<size_t>(tdm_k23_table_bytes(segs, nseg)));
     StepSegDev* out = static_cast<StepSegDev*>(image);
-    const int es = nseg > 0 ? step_elem_size(segs[0]) : 4;
-    if (es == 0) throw Invalid("a step segment's dtype must be TDM_F32, TDM_F64, TDM_BF16 or TDM_F16");
     const int64_t tile_elems = static_cast<int64_t>(kTileVecs) * (16 / es);
     int64_t tiles = 0;
     for (int i = 0; i < nseg; ++i) {
       const tdm_step_seg& sg = segs[i];
-      if (sg.dtype != segs[0].dtype) throw Invalid("segment " + std::to_string(i) + ": the segments of one table share one dtype");
       if (sg.count < 0) throw Invalid("segment " + std::to_string(i) + ": negative count");
       if (sg.count == 0) continue;
       if (sg.chunk < 0 || sg.chunk >= world) throw Invalid("segment " + std::to_string(i) + ": chunk outside [0, world)");

@@ -12,7 +12,7 @@ from tandem_amd import _lib
 from tandem_amd._lib import lib
 
 W = _lib.TDM_MAX_WORLD
-F32, F64, BF16, EINVAL = 0, 1, 3, 1  # enum tdm_dtype and TDM_EINVAL of include/tandem_hip.h
+F32, F64, F16, BF16, EINVAL = 0, 1, 2, 3, 1  # enum tdm_dtype and TDM_EINVAL of include/tandem_hip.h
 FOLD_REC = np.dtype([("src", np.uint64, W), ("dst", np.uint64, W), ("count", np.int64), ("chunk", np.int32), ("vec_ok", np.int32)])
 STEP_REC = np.dtype([("g", np.uint64, W), ("p", np.uint64, W), ("m", np.uint64), ("v", np.uint64), ("count", np.int64),
                      ("chunk", np.int32), ("vec_ok", np.int32)])
@@ -79,9 +79,10 @@ def test_fold_table_records(world, dtype, es):
     assert at == ntiles
 
 
-def step_segs(world, rows):
+def step_segs(world, rows, dtype=F32):
     segs = (_lib.StepSeg * len(rows))()
     for k, (count, chunk, off) in enumerate(rows):
+        segs[k].dtype = dtype
         for r in range(world):
             segs[k].grad[r] = (1 << 32) * (r + 1) + (k << 24) + off
             segs[k].param[r] = (1 << 40) * (r + 1) + (k << 24) + off
@@ -90,12 +91,16 @@ def step_segs(world, rows):
     return segs
 
 
+@pytest.mark.parametrize("dtype,es", [(F32, 4), (F64, 8), (BF16, 2), (F16, 2)])
 @pytest.mark.parametrize("world", [1, 2, 4, 7])
-def test_step_table_records(world):
-    tile = TILE_BYTES // 4
-    rows = [(3, 0, 0), (2 * tile, world - 1, 0), (0, 0, 0), (tile + 9, world // 2, 4), (4 * tile - 1, 0, 48), (tile + 2, 0, 8), (1, 0, 12)]
-    segs = step_segs(world, rows)
-    plans = [walk(c, off, 4, tile) for c, _, off in rows]
+def test_step_table_records(world, dtype, es):
+    """A step segment names its element type (0 = fp32, what a caller that knows nothing of the field leaves there): a record
+    covers tdm_table_tile_bytes() of every stream whatever the type, heads are peeled in elements of that type."""
+    tile = TILE_BYTES // es
+    rows = [(3, 0, 0), (2 * tile, world - 1, 0), (0, 0, 0), (tile + 9, world // 2, es), (4 * tile - 1, 0, 48), (tile + 2, 0, 8), (1, 0, 16 - es)]
+    segs = step_segs(world, rows, dtype)
+    plans = [walk(c, off, es, tile) for c, _, off in rows]
+    assert any(p[0] and p[1] for p in plans)
     ntiles = lib().tdm_k23_table_tiles(segs, len(rows))
     assert ntiles == sum(p[3] for p in plans)
     nbytes = lib().tdm_k23_table_bytes(segs, len(rows))
@@ -111,12 +116,75 @@ def test_step_table_records(world):
             assert rec["count"] == min(tile, body - done) and rec["chunk"] == chunk
             assert rec["vec_ok"] == (0 if not vec else 1 + head if done == 0 else 1), (k, done)
             for r in range(world):
-                assert rec["g"][r] == segs[k].grad[r] + (head + done) * 4 and rec["p"][r] == segs[k].param[r] + (head + done) * 4
-            assert rec["m"] == segs[k].exp_avg + (head + done) * 4 and rec["v"] == segs[k].exp_avg_sq + (head + done) * 4
+                assert rec["g"][r] == segs[k].grad[r] + (head + done) * es and rec["p"][r] == segs[k].param[r] + (head + done) * es
+            assert rec["m"] == segs[k].exp_avg + (head + done) * es and rec["v"] == segs[k].exp_avg_sq + (head + done) * es
             assert not rec["g"][world:].any() and not rec["p"][world:].any()
             done += int(rec["count"])
             at += 1
     assert at == ntiles
+
+
+def test_step_tables_refuse_mixed_and_unknown_dtypes():
+    L = lib()
+    image = np.zeros(1 << 16, np.uint8)
+    ptr = ctypes.c_void_p(image.ctypes.data)
+    segs = step_segs(2, [(100, 0, 0), (100, 1, 0)], BF16)
+    assert L.tdm_k23_table_build(segs, 2, 2, ptr) == 0
+    segs[1].dtype = F64
+    assert L.tdm_k23_table_build(segs, 2, 2, ptr) == EINVAL and "share one dtype" in L.tdm_last_error().decode()
+    segs[0].dtype = segs[1].dtype = 5  # TDM_I32: not a shard type
+    assert L.tdm_k23_table_tiles(segs, 2) == -1
+    assert L.tdm_k23_table_build(segs, 2, 2, ptr) == EINVAL and "dtype" in L.tdm_last_error().decode()
+    segs[0].dtype = segs[1].dtype = F64
+    segs[0].grad[0] += 4  # a double 4 bytes off its grid
+    assert L.tdm_k23_table_build(segs, 2, 2, ptr) == EINVAL and "element size" in L.tdm_last_error().decode()
+    # the typed launch and the typed update check their arguments before they touch the GPU
+    hyper = _lib.AdamwHyper()
+    assert L.tdm_k23_zero2_step_typed(ptr, 1, 2, 1, 5, ctypes.byref(hyper), 0, None) == EINVAL and "dtype" in L.tdm_last_error().decode()
+    assert L.tdm_k23_zero2_step_typed(ptr, 1, 2, 1, F64, ctypes.byref(hyper), 1, None) == EINVAL and "fp32 shards only" in L.tdm_last_error().decode()
+    assert L.tdm_k23_zero2_step_typed(ptr, 1, 9, 1, F64, ctypes.byref(hyper), 0, None) == EINVAL and "world" in L.tdm_last_error().decode()
+    assert L.tdm_k3_adamw_typed(ptr, ptr, ptr, ptr, 4, 5, ctypes.byref(hyper), 0, None, 0, None) == EINVAL and "dtype" in L.tdm_last_error().decode()
+    assert L.tdm_k3_adamw_typed(ptr, ptr, ptr, ptr, 4, BF16, ctypes.byref(hyper), 1, None, 0, None) == EINVAL and "fp32 shards only" in L.tdm_last_error().decode()
+    assert L.tdm_k3_adamw_typed(ptr, ptr, ptr, ptr, 0, BF16, ctypes.byref(hyper), 0, None, 0, None) == 0  # nothing to do
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "float64", "bfloat16", "float16"])
+def test_state_and_gradient_shards_follow_the_parameter_shards_phase(dtype_name):
+    """optim.zeros_at_phase_of and the layout LocalZeRO2 makes with it (on CPU tensors: nothing is launched): world 3
+    over a flat buffer of odd length puts the shards at three different distances from a cache line, and every shard's
+    gradient and both moments start at the same distance; with one_allocation every buffer lies inside the one pool
+    and none overlap; the step table counts the tiles of the element type."""
+    import torch
+
+    from tandem_amd.local import LocalZeRO2
+    from tandem_amd.optim import zeros_at_phase_of
+
+    dtype = getattr(torch, dtype_name)
+    es = torch.empty(0, dtype=dtype).element_size()
+    flat = torch.zeros(4096, dtype=dtype)
+    for lo in (0, 1, 3, 128 // es - 1, 128 // es + 5):
+        like = flat[lo:lo + 100]
+        z = zeros_at_phase_of(like)
+        assert z.numel() == 100 and z.dtype == dtype and z.data_ptr() % 128 == like.data_ptr() % 128 and not z.any()
+        assert zeros_at_phase_of(like, 7).numel() == 7
+    numels = [4099, 10_007, 33, 5001, 1, 12_288, 782]
+    for one in ([False, True] if dtype == torch.float32 else [False]):
+        z = LocalZeRO2(3, numels, "cpu", bucket_bytes=16 << 10, dtype=dtype, one_allocation=one)
+        phases = set()
+        for r, l in enumerate(z.layouts):
+            phase = z.bufs[r][l.lo:l.hi].data_ptr() % 128
+            phases.add(phase)
+            assert z.grad_shards[r].data_ptr() % 128 == phase
+            assert z.opts[r].state["flat"][1].data_ptr() % 128 == z.opts[r].state["flat"][2].data_ptr() % 128 == phase
+            assert z.grad_shards[r].dtype == z.opts[r].state["flat"][1].dtype == dtype
+        assert len(phases) == 3
+        parts = z.bufs + z.staging + z.grad_shards + [t for o in z.opts for t in o.state["flat"][1:]]
+        spans = sorted((t.data_ptr(), t.data_ptr() + es * t.numel()) for t in parts)
+        assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
+        if one:
+            assert spans[0][0] >= z._pool.data_ptr() and spans[-1][1] <= z._pool.data_ptr() + 4 * z._pool.numel()
+        image, ntiles = z._step_table
+        assert ntiles >= sum(numels) * es // TILE_BYTES and image.numel() == ntiles * STEP_REC.itemsize
 
 
 def test_empty_tables_and_refusals():
