@@ -1,12 +1,13 @@
 /* A host written in C that uses the library through include/tandem_hip.h and nothing else of this
  * repository: no Python, no torch. Four rank buffers from hipMalloc, integer-valued fp32 data (so that
  * every sum and every division by four is exact and the expected bits need no oracle), then the ring
- * collectives of buffer ranks in both of their forms, the single-launch all-reduce, one AdamW step
- * with zero gradients and no decay (which must leave the parameters alone), and the refusals that a
- * C caller sees as status codes. Exit status 0 and "abi_host: ok" when everything matched.
+ * collectives of buffer ranks in both of their forms, the single-launch all-reduce, three AdamW steps
+ * on a float64 shard through tdm_k3_adamw_typed (checked bit for bit against the same seven operations
+ * written out in C doubles below), and the refusals that a C caller sees as status codes. Exit status 0 and "abi_host: ok" when everything matched.
  * Built by __graft_entry__.build() with gcc; run on the GPU by tests/test_gpu_c_host.py. */
 
 #include <hip/hip_runtime_api.h>
+#include <math.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -63,6 +64,68 @@ static int all_equal_the_mean(const char* what) {
   return 0;
 }
 
+/* tandem/optim.py:28-37 on doubles, operation for operation (lerp_ and addcmul_ fuse their last multiply-add). */
+#define SHARD 4099
+static double sp[SHARD], sg[SHARD], sm[SHARD], sv[SHARD], got_p[SHARD], got_m[SHARD], got_v[SHARD];
+
+static int adamw_in_doubles(hipStream_t stream) {
+  const double lr = 3e-4, beta1 = 0.9, beta2 = 0.95, eps = 1e-8, wd = 0.1;
+  void *dp, *dg, *dm, *dv;
+  HIP_OK(hipMalloc(&dp, sizeof sp));
+  HIP_OK(hipMalloc(&dg, sizeof sg));
+  HIP_OK(hipMalloc(&dm, sizeof sm));
+  HIP_OK(hipMalloc(&dv, sizeof sv));
+  for (int i = 0; i < SHARD; ++i) {
+    sp[i] = 0.02 * sin(0.37 * i + 1.0);
+    sm[i] = sv[i] = 0.0;
+  }
+  HIP_OK(hipMemcpy(dp, sp, sizeof sp, hipMemcpyHostToDevice));
+  HIP_OK(hipMemset(dm, 0, sizeof sm));
+  HIP_OK(hipMemset(dv, 0, sizeof sv));
+  for (int step = 1; step <= 3; ++step) {
+    for (int i = 0; i < SHARD; ++i) sg[i] = 1e-3 * cos(0.11 * i + step);
+    HIP_OK(hipMemcpy(dg, sg, sizeof sg, hipMemcpyHostToDevice));
+    tdm_adamw_hyper h;
+    memset(&h, 0, sizeof h);
+    h.use_decay = 1;
+    h.decay = 1 - lr * wd;
+    h.w1 = 1 - beta1;
+    h.beta2 = beta2;
+    h.one_m_b2 = 1 - beta2;
+    h.bc2_sqrt = sqrt(1 - pow(beta2, step));
+    h.eps = eps;
+    h.neg_step = -(lr / (1 - pow(beta1, step)));
+    TDM_OK_(tdm_k3_adamw_typed(dp, dg, dm, dv, SHARD, TDM_F64, &h, TDM_ADAMW_HOST_ORDER, NULL, 0, stream));
+    for (int i = 0; i < SHARD; ++i) {
+      sp[i] = sp[i] * h.decay;
+      sm[i] = fma(h.w1, sg[i] - sm[i], sm[i]);
+      sv[i] = fma(h.one_m_b2 * sg[i], sg[i], sv[i] * h.beta2);
+      const double d = sqrt(sv[i]) / h.bc2_sqrt + h.eps;
+      sp[i] = sp[i] + (h.neg_step * sm[i]) / d;
+    }
+  }
+  HIP_OK(hipStreamSynchronize(stream));
+  HIP_OK(hipMemcpy(got_p, dp, sizeof sp, hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(got_m, dm, sizeof sm, hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(got_v, dv, sizeof sv, hipMemcpyDeviceToHost));
+  if (memcmp(got_p, sp, sizeof sp) || memcmp(got_m, sm, sizeof sm) || memcmp(got_v, sv, sizeof sv)) {
+    fprintf(stderr, "AdamW on doubles: the GPU's bits differ from the same operations in C\n");
+    return 1;
+  }
+  tdm_adamw_hyper h;
+  memset(&h, 0, sizeof h);
+  if (tdm_k3_adamw_typed(dp, dg, dm, dv, SHARD, TDM_I32, &h, TDM_ADAMW_HOST_ORDER, NULL, 0, stream) != TDM_EINVAL ||
+      tdm_k3_adamw_typed(dp, dg, dm, dv, SHARD, TDM_F64, &h, TDM_ADAMW_DEVICE_ORDER, NULL, 0, stream) != TDM_EINVAL) {
+    fprintf(stderr, "AdamW: an integer shard or the device order on doubles was not refused\n");
+    return 1;
+  }
+  HIP_OK(hipFree(dp));
+  HIP_OK(hipFree(dg));
+  HIP_OK(hipFree(dm));
+  HIP_OK(hipFree(dv));
+  return 0;
+}
+
 int main(void) {
   int count = 0;
   HIP_OK(hipGetDeviceCount(&count));
@@ -110,6 +173,10 @@ int main(void) {
   if (tdm_local_all_reduce(aliased, WORLD, N, TDM_F32, 0, TDM_ALLREDUCE_RING, stream) != TDM_EINVAL) {
     fprintf(stderr, "two ranks sharing a buffer were not refused\n");
     return 1;
+  }
+  {
+    const int status = adamw_in_doubles(stream);
+    if (status) return status;
   }
   char name[128];
   int cus = 0;

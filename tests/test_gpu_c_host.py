@@ -1,5 +1,6 @@
 """The library driven by a host written in C (tests/cpp/abi_host.c): four hipMalloc'ed rank buffers, the ring
-collectives in both forms, the single-launch all-reduce and the refusals, through include/tandem_hip.h alone.
+collectives in both forms, the single-launch all-reduce, AdamW on a float64 shard (against the same operations in C
+doubles) and the refusals, through include/tandem_hip.h alone.
 The program is built beforehand (__graft_entry__.build(), or `make -C tests/cpp`); only if it is missing
 is it built here. Run with -m gpu."""
 
