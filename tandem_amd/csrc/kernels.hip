@@ -1154,21 +1154,38 @@ float eps_as_applied(double eps) {
   }
 }
 
+// The step's constants as the kernels for T take them.
+template <typename T>
+AdamwHyper<typename AdamwMath<T>::S> typed_hyper(const tdm_adamw_hyper& h) {
+  using S = typename AdamwMath<T>::S;
+  AdamwHyper<S> s{};
+  s.use_decay = h.use_decay;
+  s.decay = static_cast<S>(h.decay), s.w1 = static_cast<S>(h.w1), s.beta2 = static_cast<S>(h.beta2);
+  s.one_m_b2 = static_cast<S>(h.one_m_b2), s.bc2_sqrt = static_cast<S>(h.bc2_sqrt), s.neg_step = static_cast<S>(h.neg_step);
+  s.eps = static_cast<S>(h.eps);
+  if constexpr (sizeof(T) == 2) s.eps = eps_as_applied<T>(h.eps);
+  // bfloat16's way round the division by bc2_sqrt: a product with the reciprocal, redone as a division where the low
+  // 16 bits of the product come within 6 of a rounding tie (0x8000); the product is within 2.5 ulps of the quotient
+  // as long as neither leaves the normal floats, which a divisor within [2^-30, 2^30] guarantees for every square
+  // root of a bfloat16. Any other divisor: every element by division.
+  s.inv_bc2 = static_cast<S>(1.0 / static_cast<double>(s.bc2_sqrt));
+  constexpr uint32_t kWindow = 6;
+  const bool usual = s.bc2_sqrt >= S(0x1p-30) && s.bc2_sqrt <= S(0x1p30);
+  s.tie_bias = usual ? (kWindow - 0x8000u) & 0xffffu : 0u;
+  s.tie_span = usual ? 2 * kWindow : 0xffffu;
+  return s;
+}
+
 template <typename T>
 void adamw_typed_launch(void* p_, const void* g_, void* m_, void* v_, int64_t n, const tdm_adamw_hyper& h, void* const* copies,
                         int ncopies, hipStream_t st) {
-  using S = typename AdamwMath<T>::S;
   constexpr int es = static_cast<int>(sizeof(T));
   uintptr_t ptrs[4 + TDM_MAX_WORLD - 1] = {reinterpret_cast<uintptr_t>(p_), reinterpret_cast<uintptr_t>(g_),
                                            reinterpret_cast<uintptr_t>(m_), reinterpret_cast<uintptr_t>(v_)};
   AdamwArgsT<T> a{};
   a.p = static_cast<T*>(p_), a.g = static_cast<const T*>(g_), a.m = static_cast<T*>(m_), a.v = static_cast<T*>(v_);
   a.n = n;
-  a.s.use_decay = h.use_decay;
-  a.s.decay = static_cast<S>(h.decay), a.s.w1 = static_cast<S>(h.w1), a.s.beta2 = static_cast<S>(h.beta2);
-  a.s.one_m_b2 = static_cast<S>(h.one_m_b2), a.s.bc2_sqrt = static_cast<S>(h.bc2_sqrt), a.s.neg_step = static_cast<S>(h.neg_step);
-  a.s.eps = static_cast<S>(h.eps);
-  if constexpr (sizeof(T) == 2) a.s.eps = eps_as_applied<T>(h.eps);
+  a.s = typed_hyper<T>(h);
   a.ncopies = ncopies;
   a.shift = xcd_shift(TDM_XCD_ADAMW, 1, true);
   for (int c = 0; c < ncopies; ++c) {
@@ -1199,9 +1216,8 @@ void adamw_typed_launch(void* p_, const void* g_, void* m_, void* v_, int64_t n,
   }
   const int64_t per = vec ? static_cast<int64_t>(kAdamwThreads) * (16 / es) : kAdamwThreads;
   const dim3 grid(grid_for(std::max<int64_t>((a.n + per - 1) / per, 1))), block(kAdamwThreads);
-  // bf16 rounds eight times per element and is bound by its arithmetic (0.52 of the HBM peak), where the cap of three waves per
-  // SIMD that suits the memory-bound fp32 and fp64 kernels costs it 5 %: four 21.46M-element shards take 0.243 ms with 8 KiB,
-  // 0.255 with none, 0.257 with 24 KiB.
+  // The 16-bit types round eight times per element and carry far more arithmetic per byte than fp32 and fp64, whose cap of three
+  // waves per SIMD costs them 5-10 %: four 21.46M-element shards take 0.200-0.212 ms with 8 KiB, 0.22 with 16 or 24 KiB.
   const int set = g_occupancy_pad[TDM_XCD_ADAMW].load(std::memory_order_relaxed);
   const unsigned pad = set >= 0 ? static_cast<unsigned>(set) : sizeof(T) == 2 ? 8192u : occupancy_pad(TDM_XCD_ADAMW);
   switch ((vec ? 2 : 0) + (ncopies > 0 ? 1 : 0)) {
@@ -1329,10 +1345,7 @@ extern "C++" {
 namespace {
 template <typename T, int kWorld>
 void launch_step_typed_w(const void* image, int64_t tiles, int average, const tdm_adamw_hyper& h, hipStream_t stream) {
-  using S = typename AdamwMath<T>::S;
-  AdamwHyper<S> s{h.use_decay, static_cast<S>(h.decay), static_cast<S>(h.w1), static_cast<S>(h.beta2), static_cast<S>(h.one_m_b2),
-                  static_cast<S>(h.bc2_sqrt), static_cast<S>(h.eps), static_cast<S>(h.neg_step)};
-  if constexpr (sizeof(T) == 2) s.eps = eps_as_applied<T>(h.eps);
+  const AdamwHyper<typename AdamwMath<T>::S> s = typed_hyper<T>(h);
   const Divisor<T> dv = make_divisor<T>(kWorld);
   const StepSegDev* t = static_cast<const StepSegDev*>(image);
   const dim3 grid(grid_for(tiles * kStepParts)), block(kThreads);

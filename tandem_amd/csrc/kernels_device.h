@@ -795,12 +795,23 @@ template <typename S>
 struct AdamwHyper {
   int use_decay;
   S decay, w1, beta2, one_m_b2, bc2_sqrt, eps, neg_step;
+  // bfloat16 only (see AdamwMath16::root_over): 1 / bc2_sqrt rounded to fp32, and the window around a rounding tie inside
+  // which the quotient is recomputed by a true division: low 16 bits + tie_bias (mod 2^16) <= tie_span.
+  // tie_span = 0xffff sends every element the exact way.
+  S inv_bc2;
+  uint32_t tie_bias, tie_span;
 };
 
 template <typename T> struct AdamwMath;
 
 template <> struct AdamwMath<double> {
   using S = double;
+  static constexpr int kGroup = 1;
+  template <int N>
+  static __device__ __forceinline__ void step_n(double* p, const double* g, double* m, double* v, const AdamwHyper<double>& s, bool small_w) {
+    static_assert(N == 1, "doubles are stepped one at a time");
+    step(*p, *g, *m, *v, s, small_w);
+  }
   static __device__ __forceinline__ void step(double& p, double g, double& m, double& v, const AdamwHyper<double>& s, bool small_w) {
     if (s.use_decay) p = p * s.decay;
     const double diff = g - m;
@@ -819,6 +830,17 @@ template <> struct Round16<bf16_t> {
   static __device__ __forceinline__ float rb(float x) {
     const __bf16 h = static_cast<__bf16>(x);
     return static_cast<float>(h);
+  }
+  // two floats through one conversion instruction (v_cvt_pk_bf16_f32 takes a pair)
+  static __device__ __forceinline__ void rb2(float& x, float& y) {
+    typedef float float_pair __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16_pair __attribute__((ext_vector_type(2)));
+    const float_pair in = {x, y};
+    const bf16_pair h = __builtin_convertvector(in, bf16_pair);
+    uint32_t u;
+    __builtin_memcpy(&u, &h, 4);
+    x = __uint_as_float(u << 16);
+    y = __uint_as_float(u & 0xffff0000u);
   }
   // the bits of a float that rb() has already rounded: its upper half
   static __device__ __forceinline__ uint16_t bits(float x) { return static_cast<uint16_t>(__float_as_uint(x) >> 16); }
@@ -845,27 +867,106 @@ template <> struct Round16<f16_t> {
 };
 
 // x is rounded to the 16-bit type and back by the conversion instruction instead of the integer operations of
-// Elem<T>::narrow: this kernel rounds eight times per element and is bound by its arithmetic, not by memory. A NaN
-// stays a NaN through the roundings; what is stored is the canonical one, as narrow() makes it.
+// Elem<T>::narrow: this kernel rounds eight times per element, and on bfloat16 its arithmetic showed in the time
+// until the root and the division by bc2_sqrt were shortened (root_over below; TDM_BF16_SHORT_ROOT=0 builds the
+// version that does them to the letter, for comparison). A NaN stays a NaN through the roundings; what is stored is
+// the canonical one, as narrow() makes it.
+#ifndef TDM_BF16_SHORT_ROOT
+#define TDM_BF16_SHORT_ROOT 1
+#endif
 template <typename T>
 struct AdamwMath16 {
   using S = float;
   using R = Round16<T>;
+  static constexpr bool kBf16 = std::is_same<T, bf16_t>::value;
+  // Elements are stepped in groups: bfloat16 rounds two floats with one conversion instruction.
+  static constexpr int kGroup = kBf16 ? 2 : 1;
+
+  template <int N>
+  static __device__ __forceinline__ void round_all(float (&x)[N]) {
+    if constexpr (N == 2 && kBf16) {
+      R::rb2(x[0], x[1]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < N; ++i) x[i] = R::rb(x[i]);
+    }
+  }
+
+  // d = rb(rb(sqrt(v)) / bc2_sqrt), the two operations that cost the most arithmetic when done to the letter (a
+  // correctly rounded fp32 square root and a true division are a dozen instructions each).
+  //
+  // bfloat16 takes a shorter way to the same bits. (1) The hardware's square root (within 1 ulp of fp32) instead of the
+  // correctly rounded one: v has 8 significant bits, so sqrt(v) cannot come close to a value half way between two
+  // bfloat16 neighbours (such a T has an odd 9-bit significand, T*T an odd significand of 17 or 18 bits, v's has at
+  // most 8, so |v - T*T| is at least one unit of T*T's last place and sqrt(v) stays more than 30 fp32 ulps away from
+  // T): every float within a few ulps of sqrt(v) rounds to the same bfloat16. The instruction does not take denormal
+  // floats: a nonzero v below 2^-96 goes the exact way. (2) A multiplication by 1 / bc2_sqrt instead of the division:
+  // the product lies within 2.5 fp32 ulps of the correctly rounded quotient, so both round to the same bfloat16 unless
+  // a tie (low 16 bits 0x8000) lies within a few ulps; then the pair goes the exact way (about 3 % of a wave's pairs).
+  // The host sets the window, and sets it to everything when bc2_sqrt is outside [2^-30, 2^30].
+  template <int N>
+  static __device__ __forceinline__ void root_over(const float (&v)[N], float (&d)[N], const AdamwHyper<float>& s) {
+    if constexpr (kBf16 && TDM_BF16_SHORT_ROOT) {
+      float q[N];
+      bool exact_way = false;
+#pragma unroll
+      for (int i = 0; i < N; ++i) d[i] = __builtin_amdgcn_sqrtf(v[i]);
+      round_all(d);
+#pragma unroll
+      for (int i = 0; i < N; ++i) {
+        q[i] = d[i] * s.inv_bc2;
+        exact_way |= ((__float_as_uint(q[i]) + s.tie_bias) & 0xffffu) <= s.tie_span;
+        exact_way |= !(v[i] >= 0x1p-96f) && v[i] != 0.0f;  // denormal floats, negative numbers, NaN
+      }
+      if (__builtin_expect(exact_way, 0)) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) q[i] = R::rb(__builtin_sqrtf(v[i])) / s.bc2_sqrt;
+      }
+#pragma unroll
+      for (int i = 0; i < N; ++i) d[i] = q[i];
+      round_all(d);
+    } else {
+#pragma unroll
+      for (int i = 0; i < N; ++i) d[i] = R::rb(__builtin_sqrtf(v[i]));
+#pragma unroll
+      for (int i = 0; i < N; ++i) d[i] = R::rb(d[i] / s.bc2_sqrt);
+    }
+  }
+
+  template <int N>
+  static __device__ __forceinline__ void step_n(T* p, const T* g, T* m, T* v, const AdamwHyper<float>& s, bool small_w) {
+    float P[N], G[N], M[N], V[N], D[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) P[i] = Elem<T>::widen(p[i]), G[i] = Elem<T>::widen(g[i]), M[i] = Elem<T>::widen(m[i]), V[i] = Elem<T>::widen(v[i]);
+    if (s.use_decay) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) P[i] = P[i] * s.decay;
+      round_all(P);
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const float diff = G[i] - M[i];  // inside lerp_: not rounded
+      M[i] = small_w ? __builtin_fmaf(s.w1, diff, M[i]) : __builtin_fmaf(s.w1 - 1.0f, diff, G[i]);
+    }
+    round_all(M);
+#pragma unroll
+    for (int i = 0; i < N; ++i) V[i] = V[i] * s.beta2;
+    round_all(V);
+#pragma unroll
+    for (int i = 0; i < N; ++i) V[i] = __builtin_fmaf(s.one_m_b2 * G[i], G[i], V[i]);
+    round_all(V);
+    root_over(V, D, s);
+#pragma unroll
+    for (int i = 0; i < N; ++i) D[i] = D[i] + s.eps;  // s.eps arrives rounded to the 16-bit type
+    round_all(D);
+#pragma unroll
+    for (int i = 0; i < N; ++i) P[i] = P[i] + (s.neg_step * M[i]) / D[i];
+    round_all(P);
+#pragma unroll
+    for (int i = 0; i < N; ++i) p[i] = exact(P[i]), m[i] = exact(M[i]), v[i] = exact(V[i]);
+  }
   static __device__ __forceinline__ void step(T& p, T g, T& m, T& v, const AdamwHyper<float>& s, bool small_w) {
-    float P = Elem<T>::widen(p), M = Elem<T>::widen(m), V = Elem<T>::widen(v);
-    const float G = Elem<T>::widen(g);
-    if (s.use_decay) P = R::rb(P * s.decay);
-    const float diff = G - M;  // inside lerp_: not rounded
-    M = R::rb(small_w ? __builtin_fmaf(s.w1, diff, M) : __builtin_fmaf(s.w1 - 1.0f, diff, G));
-    V = R::rb(V * s.beta2);
-    V = R::rb(__builtin_fmaf(s.one_m_b2 * G, G, V));
-    float D = R::rb(__builtin_sqrtf(V));
-    D = R::rb(D / s.bc2_sqrt);
-    D = R::rb(D + s.eps);  // s.eps arrives rounded to the 16-bit type
-    P = R::rb(P + (s.neg_step * M) / D);
-    p = exact(P);
-    m = exact(M);
-    v = exact(V);
+    step_n<1>(&p, &g, &m, &v, s, small_w);
   }
   static __device__ __forceinline__ T exact(float x) {
     T out;
@@ -894,7 +995,8 @@ template <typename T, bool kVec, bool kCopies>
 __global__ __launch_bounds__(kAdamwThreads) void k3_adamw_typed_kernel(AdamwArgsT<T> a) {
   using S = typename AdamwMath<T>::S;
   const bool small_w = (a.s.w1 < S(0) ? -a.s.w1 : a.s.w1) < S(0.5);
-  constexpr int kL = lanes<T>();
+  constexpr int kL = lanes<T>(), kG = AdamwMath<T>::kGroup;
+  static_assert(kL % kG == 0, "a vector holds whole groups");
   if constexpr (kVec) {
     const int64_t nv = a.n / kL;
     const int64_t tiles = (nv + kAdamwThreads - 1) / kAdamwThreads;
@@ -906,7 +1008,7 @@ __global__ __launch_bounds__(kAdamwThreads) void k3_adamw_typed_kernel(AdamwArgs
         Lanes<T> M = unpack<T>(load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.m) + i * 16));
         Lanes<T> V = unpack<T>(load_rmw<TDM_NT_MASK_K3>(reinterpret_cast<const char*>(a.v) + i * 16));
 #pragma unroll
-        for (int l = 0; l < kL; ++l) AdamwMath<T>::step(P.v[l], G.v[l], M.v[l], V.v[l], a.s, small_w);
+        for (int l = 0; l < kL; l += kG) AdamwMath<T>::template step_n<kG>(&P.v[l], &G.v[l], &M.v[l], &V.v[l], a.s, small_w);
         const vec16 packed = pack<T>(P);
         store16<TDM_NT_MASK_K3>(reinterpret_cast<char*>(a.p) + i * 16, packed);
         if constexpr (kCopies)
@@ -1093,7 +1195,7 @@ template <typename T, int kWorld, int kDiv, int kRounds>
 __device__ __forceinline__ void step_tile_typed(const StepSegDev& sg, int64_t at, int64_t n, int head, const Divisor<T>& dv,
                                                 const AdamwHyper<typename AdamwMath<T>::S>& s, bool small_w) {
   using A = typename Elem<T>::acc;
-  constexpr int L = lanes<T>();
+  constexpr int L = lanes<T>(), kG = AdamwMath<T>::kGroup;
   constexpr int kM = TDM_NT_MASK_K23;
   const int c = sg.chunk;  // `at`: the tile's offset in bytes from the record's pointers; n: its elements
   const char* gp[kWorld];
@@ -1106,16 +1208,16 @@ __device__ __forceinline__ void step_tile_typed(const StepSegDev& sg, int64_t at
   char* own = sg.p[c] + at;
   char* const mm = sg.m + at;
   char* const vv = sg.v + at;
-  auto one = [&](const T (&gs)[kWorld], T& P, T& M, T& V) {
+  auto folded = [&](const T (&gs)[kWorld]) {
     A acc = scaled<T, kDiv>(Elem<T>::widen(gs[0]), dv.divisor, dv.reciprocal);
 #pragma unroll
     for (int k = 1; k < kWorld; ++k) {
       const A y = scaled<T, kDiv>(Elem<T>::widen(gs[k]), dv.divisor, dv.reciprocal);
       acc = Elem<T>::widen(Elem<T>::narrow(static_cast<A>(y + acc)));
     }
-    const T g = Elem<T>::narrow(static_cast<A>(A(0) + acc));  // grad_shard (zero) += mine
-    AdamwMath<T>::step(P, g, M, V, s, small_w);
+    return Elem<T>::narrow(static_cast<A>(A(0) + acc));  // grad_shard (zero) += mine
   };
+  auto one = [&](const T (&gs)[kWorld], T& P, T& M, T& V) { AdamwMath<T>::step(P, folded(gs), M, V, s, small_w); };
   auto scalar_at = [&](int64_t i) {
     T gs[kWorld];
 #pragma unroll
@@ -1139,11 +1241,16 @@ __device__ __forceinline__ void step_tile_typed(const StepSegDev& sg, int64_t at
         Lanes<T> P = unpack<T>(load_rmw<kM>(own + v * 16)), M = unpack<T>(load_rmw<kM>(mm + v * 16)),
                  V = unpack<T>(load_rmw<kM>(vv + v * 16));
 #pragma unroll
-        for (int l = 0; l < L; ++l) {
-          T gs[kWorld];
+        for (int l = 0; l < L; l += kG) {
+          T g[kG];
 #pragma unroll
-          for (int k = 0; k < kWorld; ++k) gs[k] = unpack<T>(in[k]).v[l];
-          one(gs, P.v[l], M.v[l], V.v[l]);
+          for (int j = 0; j < kG; ++j) {
+            T gs[kWorld];
+#pragma unroll
+            for (int k = 0; k < kWorld; ++k) gs[k] = unpack<T>(in[k]).v[l + j];
+            g[j] = folded(gs);
+          }
+          AdamwMath<T>::template step_n<kG>(&P.v[l], g, &M.v[l], &V.v[l], s, small_w);
         }
         const vec16 packed = pack<T>(P);
 #pragma unroll

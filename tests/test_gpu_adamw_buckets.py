@@ -310,6 +310,43 @@ def test_adamw_bf16_and_f64_on_odd_shards_with_copies(dev, dtype):
                 assert float((s_[:pad + ph].double() + 7.0).abs().sum()) == 0 and float((s_[pad + ph + n:].double() + 7.0).abs().sum()) == 0, what
 
 
+def test_bf16_square_roots_and_divisors_over_every_second_moment(dev):
+    """The bfloat16 kernel takes the hardware's square root and a product with 1/bc2_sqrt where the oracle takes the
+    correctly rounded root and a true division, and goes the oracle's way only near a rounding tie, for floats the
+    root instruction does not take, and for divisors outside [2^-30, 2^30]. Every one of the 65,536 bit patterns as
+    the second moment (zeros, denormals, negative numbers, infinities, NaNs among them; beta2 = 1 and a zero gradient
+    leave it as it is), sixteen first moments each so that a denominator one step off shows in the parameter, against
+    divisors from the steps of three beta2, the window's two ends, values beyond them, 0, infinity, NaN and a negative
+    number: bit for bit with the oracle."""
+    import ctypes
+
+    from oracle import lib as oracle_lib
+    from tandem_amd import _lib
+
+    L, O = _lib.lib(), oracle_lib()
+    moments = (np.arange(16, dtype=np.uint16) << 3) + 0x3f80  # 1, 1.0625 ... 1.9375 as bf16 patterns
+    moments[8:] |= 0x8000
+    v0 = np.repeat(np.arange(65536, dtype=np.uint32).astype(np.uint16), moments.size)
+    m0 = np.tile(moments, 65536)
+    n = v0.size
+    divisors = [math.sqrt(1 - b ** t) for b in (0.95, 0.999, 0.98) for t in (1, 2, 3, 7, 20, 100, 1000)]
+    divisors += [1.0, 2.0 ** -30, 2.0 ** 30, 2.0 ** -31, 2.0 ** 31, 1e-38, 3.0, 0.0, math.inf, math.nan, -0.5]
+    f = ctypes.c_float
+    for k, c in enumerate(divisors):
+        c = float(np.float32(c))
+        eps = (1e-8, 0.0, 1e-3)[k % 3]
+        h = _lib.AdamwHyper(use_decay=0, decay=1.0, w1=0.0, beta2=1.0, one_m_b2=0.0, bc2_sqrt=c, eps=eps, neg_step=-1.0)
+        t = [torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16).to(dev) for a in (np.zeros(n, np.uint16), np.zeros(n, np.uint16), m0, v0)]
+        _lib.check(L.tdm_k3_adamw_typed(*(x.data_ptr() for x in t), n, _lib.DTYPES[torch.bfloat16], ctypes.byref(h), _lib.ADAMW_HOST_ORDER, None, 0, _lib.stream_ptr(dev)))
+        want = [np.zeros(n, np.uint16), np.zeros(n, np.uint16), m0.copy(), v0.copy()]
+        O.orc_adamw_bf16(*(ctypes.c_void_p(a.ctypes.data) for a in want), ctypes.c_int64(n), ctypes.c_int(0), f(1.0), f(0.0), f(1.0), f(0.0),
+                         f(c), f(eps), f(-1.0))
+        for name, got, w in zip("pgmv", t, want):
+            got = _raw(got)
+            bad = np.flatnonzero(got != w)
+            assert bad.size == 0, (c, name, bad.size, [(hex(v0[i]), hex(m0[i]), hex(got[i]), hex(w[i])) for i in bad[:5]])
+
+
 def test_adamw_rejects_what_it_cannot_do(dev):
     from tandem_amd import ShardedAdamW
 

@@ -266,3 +266,47 @@ def test_bf16_and_f64_match_torch_adamw_on_the_cpu(dtype):
     assert np.array_equal(bits(pn), bits(raw(pt.detach())))
     assert np.array_equal(bits(o.state["k"][1]), bits(raw(st["exp_avg"])))
     assert np.array_equal(bits(o.state["k"][2]), bits(raw(st["exp_avg_sq"])))
+
+
+def _to_bf16_bits(x):
+    """float32 array -> bfloat16 bit patterns, nearest even (finite inputs)."""
+    u = x.view(np.uint32).astype(np.uint64)
+    return ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def test_sqrt_of_a_bfloat16_stays_clear_of_rounding_ties():
+    """What lets the bfloat16 kernel (tandem_amd/csrc/kernels_device.h, AdamwMath16::root_over) take a square root that is
+    only within 1 ulp of fp32: for every positive bfloat16 in the range of normal floats the exact root lies tens of fp32
+    ulps away from every value half way between two bfloat16 neighbours, so any float within a few ulps of it rounds
+    to the same bfloat16 as the correctly rounded one."""
+    v = (np.arange(0x0080, 0x7f80, dtype=np.uint32) << 16).view(np.float32).astype(np.float64)
+    root = np.sqrt(v)  # within 2^-53 of exact
+    f = root.astype(np.float32)
+    ulp = np.spacing(np.abs(f)).astype(np.float64)
+    below = ((f.view(np.uint32) & 0xffff0000) | 0x8000).view(np.float32).astype(np.float64)  # the tie inside this bf16 step
+    steps = np.abs(root - below) / ulp
+    assert steps.min() > 30
+    for shift in (-3, -2, -1, 1, 2, 3):
+        near = (f.view(np.uint32).astype(np.int64) + shift).astype(np.uint32).view(np.float32)
+        assert np.array_equal(_to_bf16_bits(near), _to_bf16_bits(f))
+
+
+def test_product_with_the_reciprocal_rounds_like_the_division_away_from_ties():
+    """The other half of that shortcut: d * fl(1 / c) lies within two fp32 steps of fl(d / c) for every bfloat16 d that
+    a square root can be and c in [2^-30, 2^30], so the two round to different bfloat16 only when the product's low 16
+    bits are within a few steps of 0x8000: where the kernel's window (6 on either side) sends the element to the division."""
+    d = (np.arange(0x1f80, 0x5f81, dtype=np.uint32) << 16).view(np.float32)  # 2^-64 .. 2^64: the roots of all normal bf16
+    rng = np.random.default_rng(12)
+    cs = [np.sqrt(1 - b ** t) for b in (0.95, 0.999, 0.98, 0.9) for t in range(1, 60)]
+    cs += list(np.exp2(rng.uniform(-30, 30, 300))) + [2.0 ** -30, 2.0 ** 30, 1.0, 1 - 2.0 ** -24, 1 + 2.0 ** -23]
+    worst = 0
+    for c in cs:
+        c = np.float32(c)
+        inv = np.float32(1.0 / np.float64(c))
+        q, r = d * inv, d / c
+        away = np.abs(q.view(np.uint32).astype(np.int64) - r.view(np.uint32).astype(np.int64))
+        worst = max(worst, int(away.max()))
+        differ = _to_bf16_bits(q) != _to_bf16_bits(r)
+        low = (q.view(np.uint32) & 0xffff).astype(np.int64)
+        assert np.all(np.abs(low[differ] - 0x8000) <= 2), float(c)
+    assert worst <= 2
