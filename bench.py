@@ -1010,17 +1010,23 @@ def main():
             except Exception as e:
                 line["stream_mix_error"] = repr(e)[:300]
             torch.cuda.empty_cache()
+        def section(name, measure):
+            """A section that fails is named in the line (and on stderr); the headline and the other sections still come out."""
+            try:
+                line[name] = measure()
+            except Exception as e:
+                line[name + "_error"] = repr(e)[:300]
+                print(f"bench.py: section {name} failed: {e!r}", file=sys.stderr)
+            torch.cuda.empty_cache()
+
         if not only or "sweep" in only:
-            line["sweep"] = sweep(lw, dev, max(5, args.steps // 2))
+            section("sweep", lambda: sweep(lw, dev, max(5, args.steps // 2)))
         if not only or "bucket" in only:
-            line["bucket_path"] = bucket_path(dev, args.steps)
-            torch.cuda.empty_cache()
+            section("bucket_path", lambda: bucket_path(dev, args.steps))
         if not only or "gather" in only:
-            line["unit_gather"] = unit_gather(dev, args.steps)
-            torch.cuda.empty_cache()
+            section("unit_gather", lambda: unit_gather(dev, args.steps))
         if not only or "zero2" in only:
-            line["zero2_step"] = zero2_step(dev, max(5, args.steps // 2))
-            torch.cuda.empty_cache()
+            section("zero2_step", lambda: zero2_step(dev, max(5, args.steps // 2)))
         if fsdp is not None:
             line["fsdp_gather"] = fsdp
         if ipc is not None:
@@ -1031,7 +1037,8 @@ def main():
             line["train_step_4_processes"] = train4
         if cpu is not None and "error" not in cpu:
             cpu["gpu_over_cpu"] = round(line["value"] / cpu["value"], 1)
-            cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["one_launch_ms"], 1)
+            if "zero2_step" in line:
+                cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["one_launch_ms"], 1)
         if cpu is not None:
             line["cpu_baseline"] = cpu
     summarize(line)
