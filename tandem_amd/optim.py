@@ -139,7 +139,7 @@ class ShardedAdamW:
         returns (scalars, exp_avg, exp_avg_sq, order) for it."""
         require_device_tensor(param, "ShardedAdamW.begin_step(param)")
         if param.dtype != torch.float32:
-            raise ValueError("the fused ZeRO-2 step handles fp32 shards (update() also takes float64 and bfloat16)")
+            raise ValueError("the fused ZeRO-2 step between process ranks handles fp32 shards (update() also takes float64, bfloat16 and float16)")
         if key not in self.state:
             self.state[key] = [0.0, zeros_at_phase_of(param), zeros_at_phase_of(param)]
         st = self.state[key]
