@@ -610,12 +610,13 @@ def train_rank(g, strategy, steps):
     fused = "+fused" in strategy
     direct = "+direct" in strategy or fused
     streamwait = strategy.endswith("+streamwait")  # DDP/ZeRO that only order the training stream behind their collectives (opt-in)
+    overlap = "+nooverlap" not in strategy  # DDP(overlap=False): every bucket's all-reduce starts when backward has ended
     kind = strategy.split("+")[0]
     opt = None
     if kind == "alone":
         z, opt = model, torch.optim.AdamW(model.parameters(), foreach=False, **adamw)
     elif kind == "ddp":
-        z, opt = DDP(model, g, direct=direct, stream_ordered=streamwait), torch.optim.AdamW(model.parameters(), foreach=False, **adamw)
+        z, opt = DDP(model, g, overlap=overlap, direct=direct, stream_ordered=streamwait), torch.optim.AdamW(model.parameters(), foreach=False, **adamw)
     elif kind in ("zero1", "zero2"):
         z = ZeRO(model, g, int(kind[-1]), ShardedAdamW(**adamw), direct=direct, fused_step=fused, stream_ordered=streamwait)
     else:
@@ -654,14 +655,15 @@ def train_rank(g, strategy, steps):
             "profile": {k: (round(v, 5) if isinstance(v, float) else v) for k, v in prof.items()}}
 
 
-def train_steps(steps, world=2, strategies=("alone", "ddp", "ddp+streamwait", "ddp+direct", "ddp+direct+streamwait", "zero1", "zero1+direct", "zero2", "zero2+streamwait", "zero2+direct", "zero2+fused", "zero3")):
+def train_steps(steps, world=2, strategies=("alone", "ddp", "ddp+nooverlap", "ddp+streamwait", "ddp+direct", "ddp+direct+streamwait", "zero1", "zero1+direct", "zero2", "zero2+streamwait", "zero2+direct", "zero2+fused", "zero3")):
     from tandem_amd import launch
 
     out = {"workload": f"{world} processes sharing the GPU, 85.8M GPT, batch 8x512 split over the ranks, fp32, full step "
                        "(forward, backward, optimizer); 'alone' = the same rows with no communication and torch AdamW; "
                        "'+direct' = buckets / flat buffers in the shared arenas, collectives arena to arena; '+fused' = that, and ZeRO-2's "
                        "reduce-scatters, AdamW and all-gather as one launch per rank; '+streamwait' = the training stream is only ordered "
-                       "behind the collectives (stream_ordered=True, opt-in) where by default the host waits for them, as the reference's does"}
+                       "behind the collectives (stream_ordered=True, opt-in) where by default the host waits for them, as the reference's does; "
+                       "'+nooverlap' = DDP(overlap=False), every all-reduce started after backward"}
     for s in strategies:
         res = launch(train_rank, world, s, steps, gpus=[0] * world, timeout=120.0)
         out[s] = {"step_ms": round(max(r["step_ms"] for r in res), 3), "loss": round(res[0]["loss"], 4),
