@@ -344,6 +344,9 @@ int tdm_k23_zero2_step_typed(const void* table_dev, int64_t ntiles, int world, i
  * what a rank that is a process of its own runs over its shard, chunk = its rank. */
 int tdm_k23_zero2_step_segment(const tdm_step_seg* seg, int world, int average, const tdm_adamw_scalars* s, int order,
                                tdm_stream stream);
+/* The same for one segment of any of K3's shard types (seg->dtype), the step's constants as Python doubles. */
+int tdm_k23_zero2_step_segment_typed(const tdm_step_seg* seg, int world, int average, const tdm_adamw_hyper* h, int order,
+                                     tdm_stream stream);
 
 /* ---- K4: ZeRO-3 unit gather ---------------------------------------------- */
 
@@ -477,6 +480,11 @@ int tdm_direct_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, co
 int tdm_direct_zero2_step(tdm_engine* e, void* param, const int64_t* param_offsets, const void* grad, const int64_t* grad_offsets,
                           int noffsets, void* exp_avg, void* exp_avg_sq, int64_t count, int64_t total, int average,
                           const tdm_adamw_scalars* s, int order, tdm_stream caller, tdm_work** out);
+/* The same for buffers and optimizer state of `dtype` (TDM_F32, TDM_F64, TDM_BF16, TDM_F16; `count` elements of it),
+ * the step's constants as Python doubles: tdm_k23_zero2_step_segment_typed between the two fences. */
+int tdm_direct_zero2_step_typed(tdm_engine* e, void* param, const int64_t* param_offsets, const void* grad, const int64_t* grad_offsets,
+                                int noffsets, void* exp_avg, void* exp_avg_sq, int64_t count, int64_t total, int average, int dtype,
+                                const tdm_adamw_hyper* h, int order, tdm_stream caller, tdm_work** out);
 int tdm_sendrecv(tdm_engine* e, const void* send, int64_t send_numel, int dst, void* recv, int64_t recv_numel, int src,
                  int dtype, tdm_stream caller, tdm_work** out);
 int tdm_barrier(tdm_engine* e, tdm_work** out);

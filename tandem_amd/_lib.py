@@ -104,6 +104,8 @@ _SIGNATURES = {
                                                 ctypes.POINTER(AdamwHyper), ctypes.c_int, ctypes.c_void_p]),
     "tdm_k23_zero2_step_segment": (ctypes.c_int, [ctypes.POINTER(StepSeg), ctypes.c_int, ctypes.c_int,
                                                   ctypes.POINTER(AdamwScalars), ctypes.c_int, ctypes.c_void_p]),
+    "tdm_k23_zero2_step_segment_typed": (ctypes.c_int, [ctypes.POINTER(StepSeg), ctypes.c_int, ctypes.c_int,
+                                                        ctypes.POINTER(AdamwHyper), ctypes.c_int, ctypes.c_void_p]),
     "tdm_k4_unit_gather_all": (ctypes.c_int, [ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p),
                                               ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "tdm_k4_unit_gather": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_int64),
@@ -140,6 +142,8 @@ _ENGINE_SIGNATURES = {
                                              _VP, _PVP]),
     "tdm_direct_zero2_step": (ctypes.c_int, [_VP, _VP, _PI64, _VP, _PI64, ctypes.c_int, _VP, _VP, ctypes.c_int64, ctypes.c_int64,
                                              ctypes.c_int, ctypes.POINTER(AdamwScalars), ctypes.c_int, _VP, _PVP]),
+    "tdm_direct_zero2_step_typed": (ctypes.c_int, [_VP, _VP, _PI64, _VP, _PI64, ctypes.c_int, _VP, _VP, ctypes.c_int64, ctypes.c_int64,
+                                                   ctypes.c_int, ctypes.c_int, ctypes.POINTER(AdamwHyper), ctypes.c_int, _VP, _PVP]),
     "tdm_engine_share": (ctypes.c_int, [_VP, ctypes.c_int64, _PVP]),
     "tdm_engine_arena_offset": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.POINTER(ctypes.c_int64)]),
     "tdm_unit_gather_direct": (ctypes.c_int, [_VP, _VP, ctypes.c_int64, ctypes.c_int, _VP, _PI64, ctypes.c_int, _PI64,

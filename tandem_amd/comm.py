@@ -22,7 +22,7 @@ import torch
 import torch.multiprocessing as mp
 
 from . import _lib
-from ._lib import check, lib
+from ._lib import AdamwHyper, check, dtype_code, lib
 
 DEFAULT_SLOT_BYTES = 4 << 20
 DEFAULT_SLOTS = 2
@@ -321,30 +321,36 @@ class Group:
         all_gather of it). `params` and `grads` are the flat parameter and gradient
         buffers, from shared_empty() at the same arena offsets on every rank; `sizes`
         the shard sizes; `exp_avg`/`exp_avg_sq` this rank's state for its shard;
-        `scalars` from optim.step_scalars. The same bits as the separate calls when the
-        gradient shard was zero before."""
+        `scalars` from optim.step_scalars (fp32 buffers) or optim.step_hyper (fp32, fp64,
+        bf16 or fp16 buffers). The same bits as the separate calls when the gradient shard
+        was zero before."""
         if op not in ("sum", "avg"):
             raise CommError(f"unknown op {op}")
         p, g = self._flat(params, "zero2_step"), self._flat(grads, "zero2_step")
-        if p.dtype != torch.float32 or g.dtype != torch.float32 or p.numel() != g.numel():
-            raise CommError("zero2_step: two fp32 buffers of one length")
+        typed = isinstance(scalars, AdamwHyper)  # doubles: any of the shard types; fp32 constants: fp32 buffers
+        kinds = (torch.float32, torch.float64, torch.bfloat16, torch.float16) if typed else (torch.float32,)
+        if p.dtype not in kinds or g.dtype != p.dtype or p.numel() != g.numel():
+            raise CommError("zero2_step: two buffers of one length and dtype (fp32; with constants from optim.step_hyper also fp64, bf16, fp16)")
+        es = p.element_size()
         sizes, _, _ = self._sizes(p, sizes if sizes is not None else [c.numel() for c in torch.tensor_split(p, self.size)])
         lo, n = sum(sizes[:self.rank]), sizes[self.rank]
         for name, t in (("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq)):
-            if t.device != self.device or t.dtype != torch.float32 or t.numel() != n or not t.is_contiguous():
-                raise CommError(f"zero2_step: {name} must be this rank's shard ({n} fp32 elements on {self.device})")
+            if t.device != self.device or t.dtype != p.dtype or t.numel() != n or not t.is_contiguous():
+                raise CommError(f"zero2_step: {name} must be this rank's shard ({n} {p.dtype} elements on {self.device})")
         bases = []
         for t in (p, g):
             off = self.arena_offset(t) if t.numel() else 0  # empty buffers: nothing to read, but the ranks still meet
             if off is None:
                 raise CommError("zero2_step: the buffers must come from shared_empty()")
-            bases.append((ctypes.c_int64 * self.size)(*[off + lo * 4] * self.size))
+            bases.append((ctypes.c_int64 * self.size)(*[off + lo * es] * self.size))
         mine_p, mine_g = p[lo:lo + n], g[lo:lo + n]
-        return self._start("zero2_step", lambda out: lib().tdm_direct_zero2_step(
-            self._engine, ctypes.c_void_p(mine_p.data_ptr()), bases[0], ctypes.c_void_p(mine_g.data_ptr()), bases[1], self.size,
-            ctypes.c_void_p(exp_avg.data_ptr()), ctypes.c_void_p(exp_avg_sq.data_ptr()), n, p.numel(), int(op == "avg"),
-            ctypes.byref(scalars), order, self._stream(), out),
-            params, (2 * self.size + 5) * 4 * n, async_op, keep=(p, g, exp_avg, exp_avg_sq, scalars))
+        head = lambda: (self._engine, ctypes.c_void_p(mine_p.data_ptr()), bases[0], ctypes.c_void_p(mine_g.data_ptr()), bases[1], self.size,
+                        ctypes.c_void_p(exp_avg.data_ptr()), ctypes.c_void_p(exp_avg_sq.data_ptr()), n, p.numel(), int(op == "avg"))
+        if typed:
+            call = lambda out: lib().tdm_direct_zero2_step_typed(*head(), dtype_code(p.dtype), ctypes.byref(scalars), order, self._stream(), out)
+        else:
+            call = lambda out: lib().tdm_direct_zero2_step(*head(), ctypes.byref(scalars), order, self._stream(), out)
+        return self._start("zero2_step", call, params, (2 * self.size + 5) * es * n, async_op, keep=(p, g, exp_avg, exp_avg_sq, scalars))
 
     # ---- shared arenas: long-lived data that peers read (and the direct collectives write) in place
     ARENA_LIMIT = (1 << 31) - 4096  # an arena is one exported allocation, and those stay under 2 GiB

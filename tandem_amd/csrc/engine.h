@@ -139,9 +139,10 @@ class Engine {
   std::shared_ptr<Work> direct(int kind, Buf t, std::vector<int64_t> sizes, bool average, std::vector<int64_t> peer_offsets,
                                hipStream_t caller);
 
+  // The step's constants come as fp32 (`s`, for fp32 buffers) or as doubles (`h`, any of K3's shard types): exactly one is set.
   std::shared_ptr<Work> zero2_step_direct(Buf param, Buf grad, std::vector<int64_t> param_offsets, std::vector<int64_t> grad_offsets,
-                                          char* exp_avg, char* exp_avg_sq, int64_t total, bool average, tdm_adamw_scalars s,
-                                          int order, hipStream_t caller);
+                                          char* exp_avg, char* exp_avg_sq, int64_t total, bool average, const tdm_adamw_scalars* s,
+                                          const tdm_adamw_hyper* h, int order, hipStream_t caller);
 
   int device() const { return device_; }
   hipStream_t stream() const { return stream_; }

@@ -1285,26 +1285,38 @@ std::shared_ptr<Work> Engine::direct(int kind, Buf t, std::vector<int64_t> sizes
 // all_gather (tandem/zero.py:141-163) with (8W + 20) bytes per element of the shard.
 std::shared_ptr<Work> Engine::zero2_step_direct(Buf param, Buf grad, std::vector<int64_t> param_offsets,
                                                 std::vector<int64_t> grad_offsets, char* exp_avg, char* exp_avg_sq,
-                                                int64_t total, bool average, tdm_adamw_scalars s, int order, hipStream_t caller) {
+                                                int64_t total, bool average, const tdm_adamw_scalars* s_in,
+                                                const tdm_adamw_hyper* h_in, int order, hipStream_t caller) {
   const char* what = "zero2_step (direct)";
   check(param, what, true);
   check(grad, what, true);
-  if (param.dtype != TDM_F32 || grad.dtype != TDM_F32) throw Invalid(std::string(what) + ": fp32 only");
+  if ((s_in == nullptr) == (h_in == nullptr)) throw Invalid(std::string(what) + ": the step's constants as fp32 or as doubles, one of the two");
+  const int dtype = param.dtype;
+  if (dtype != grad.dtype) throw Invalid(std::string(what) + ": parameters and gradients differ in dtype");
+  if (s_in != nullptr && dtype != TDM_F32) throw Invalid(std::string(what) + ": fp32 constants go with fp32 buffers");
+  if (dtype != TDM_F32 && dtype != TDM_F64 && dtype != TDM_BF16 && dtype != TDM_F16) {
+    throw Invalid(std::string(what) + ": fp32, fp64, bf16 or fp16 buffers");
+  }
   if (param.numel != grad.numel) throw Invalid(std::string(what) + ": parameters and gradients differ in length");
   if (size_ > TDM_MAX_WORLD) throw Invalid(std::string(what) + ": world sizes up to 8");
   if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid(std::string(what) + ": unknown update order");
+  if (dtype != TDM_F32 && order != TDM_ADAMW_HOST_ORDER) throw Invalid(std::string(what) + ": the device order is defined for fp32 shards only");
   if (static_cast<int>(param_offsets.size()) != size_ || static_cast<int>(grad_offsets.size()) != size_) {
     throw Invalid(std::string(what) + ": one arena offset per rank");
   }
   if (param.numel > 0) {
     if (!exp_avg || !exp_avg_sq) throw Invalid(std::string(what) + ": NULL optimizer state");
-    check(Buf{exp_avg, param.numel, TDM_F32}, what, false);
-    check(Buf{exp_avg_sq, param.numel, TDM_F32}, what, false);
+    check(Buf{exp_avg, param.numel, dtype}, what, false);
+    check(Buf{exp_avg_sq, param.numel, dtype}, what, false);
   }
-  return submit([this, param, grad, param_offsets, grad_offsets, exp_avg, exp_avg_sq, total, average, s, order] {
+  const bool typed = h_in != nullptr;
+  const tdm_adamw_scalars s = typed ? tdm_adamw_scalars{} : *s_in;
+  const tdm_adamw_hyper h = typed ? *h_in : tdm_adamw_hyper{};
+  return submit([this, param, grad, param_offsets, grad_offsets, exp_avg, exp_avg_sq, total, average, s, h, typed, dtype, order] {
     tdm_step_seg seg;
     std::memset(&seg, 0, sizeof seg);
-    if (size_ > 1) barrier_now(true, fence_tag(9, TDM_F32, total));
+    seg.dtype = dtype;
+    if (size_ > 1) barrier_now(true, fence_tag(9, dtype, total));
     if (param.numel > 0) {  // a rank with an empty shard still takes part in the fences
       const char* base[TDM_MAX_WORLD];
       direct_bases(grad, grad_offsets, base);
@@ -1316,7 +1328,8 @@ std::shared_ptr<Work> Engine::zero2_step_direct(Buf param, Buf grad, std::vector
       seg.count = param.numel;
       seg.chunk = rank_;
     }
-    zero2_step_segment(seg, size_, average, s, order, stream_);
+    if (typed) zero2_step_segment_typed(seg, size_, average, h, order, stream_);
+    else zero2_step_segment(seg, size_, average, s, order, stream_);
     if (size_ > 1) barrier_now(true);
   }, caller, true, true, true);
 }

@@ -182,21 +182,39 @@ int tdm_direct_all_gather(tdm_engine* e, void* ptr, int64_t numel, int dtype, co
   return direct_call(e, 2, ptr, numel, dtype, sizes, nsizes, 0, peer_offsets, noffsets, caller, out);
 }
 
-int tdm_direct_zero2_step(tdm_engine* e, void* param, const int64_t* param_offsets, const void* grad, const int64_t* grad_offsets,
-                          int noffsets, void* exp_avg, void* exp_avg_sq, int64_t count, int64_t total, int average,
-                          const tdm_adamw_scalars* s, int order, tdm_stream caller, tdm_work** out) {
+namespace {
+int direct_zero2_step(tdm_engine* e, void* param, const int64_t* param_offsets, const void* grad, const int64_t* grad_offsets,
+                      int noffsets, void* exp_avg, void* exp_avg_sq, int64_t count, int64_t total, int average, int dtype,
+                      const tdm_adamw_scalars* s, const tdm_adamw_hyper* h, int order, tdm_stream caller, tdm_work** out) {
   return guard([&] {
     if (out == nullptr) throw Invalid("NULL work pointer");
-    if (s == nullptr) throw Invalid("NULL scalars");
+    if (s == nullptr && h == nullptr) throw Invalid("NULL constants");
     if (noffsets < 0 || (noffsets > 0 && (param_offsets == nullptr || grad_offsets == nullptr))) throw Invalid("bad offsets argument");
     std::vector<int64_t> po(param_offsets, param_offsets + noffsets), go(grad_offsets, grad_offsets + noffsets);
-    finish_submit(engine_of(e).zero2_step_direct(Engine::Buf{static_cast<char*>(param), count, TDM_F32},
-                                                 Engine::Buf{static_cast<char*>(const_cast<void*>(grad)), count, TDM_F32},
+    finish_submit(engine_of(e).zero2_step_direct(Engine::Buf{static_cast<char*>(param), count, dtype},
+                                                 Engine::Buf{static_cast<char*>(const_cast<void*>(grad)), count, dtype},
                                                  std::move(po), std::move(go), static_cast<char*>(exp_avg),
-                                                 static_cast<char*>(exp_avg_sq), total, average != 0, *s, order,
+                                                 static_cast<char*>(exp_avg_sq), total, average != 0, s, h, order,
                                                  static_cast<hipStream_t>(caller)),
                   out);
   });
+}
+}  // namespace
+
+int tdm_direct_zero2_step(tdm_engine* e, void* param, const int64_t* param_offsets, const void* grad, const int64_t* grad_offsets,
+                          int noffsets, void* exp_avg, void* exp_avg_sq, int64_t count, int64_t total, int average,
+                          const tdm_adamw_scalars* s, int order, tdm_stream caller, tdm_work** out) {
+  if (s == nullptr) return guard([] { throw Invalid("NULL scalars"); });
+  return direct_zero2_step(e, param, param_offsets, grad, grad_offsets, noffsets, exp_avg, exp_avg_sq, count, total, average, TDM_F32, s,
+                           nullptr, order, caller, out);
+}
+
+int tdm_direct_zero2_step_typed(tdm_engine* e, void* param, const int64_t* param_offsets, const void* grad, const int64_t* grad_offsets,
+                                int noffsets, void* exp_avg, void* exp_avg_sq, int64_t count, int64_t total, int average, int dtype,
+                                const tdm_adamw_hyper* h, int order, tdm_stream caller, tdm_work** out) {
+  if (h == nullptr) return guard([] { throw Invalid("NULL constants"); });
+  return direct_zero2_step(e, param, param_offsets, grad, grad_offsets, noffsets, exp_avg, exp_avg_sq, count, total, average, dtype,
+                           nullptr, h, order, caller, out);
 }
 
 int tdm_fence(tdm_engine* e, tdm_stream caller, tdm_work** out) {

@@ -401,27 +401,25 @@ int64_t step_tiles(const tdm_step_seg* segs, int nseg) {
 
 }  // namespace
 
-// Used by the engine too: ZeRO-2's step over one segment (a rank's shard), see tdm_k23_zero2_step_segment.
-void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const tdm_adamw_scalars& s, int order, hipStream_t stream) {
-  if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
-  if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
-  if (sg.count < 0) throw Invalid("negative count");
-  if (sg.count == 0) return;
-  if (sg.dtype != TDM_F32) throw Invalid("the step over one segment handles fp32 shards (dtype " + std::to_string(sg.dtype) + ")");
+namespace {
+// One segment as the record the one-segment kernels take in their arguments; *tiles: how many tiles it spans.
+StepSegDev whole_segment(const tdm_step_seg& sg, int world, int64_t* tiles) {
   if (sg.chunk < 0 || sg.chunk >= world) throw Invalid("chunk outside [0, world)");
   if (!sg.exp_avg || !sg.exp_avg_sq) throw Invalid("NULL optimizer state");
+  const int es = step_elem_size(sg);
+  if (es == 0) throw Invalid("a step segment's dtype must be TDM_F32, TDM_F64, TDM_BF16 or TDM_F16");
   StepSegDev whole;
   std::memset(&whole, 0, sizeof whole);
-  if (reinterpret_cast<uintptr_t>(sg.exp_avg) % 4 || reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % 4) throw Invalid("pointer not aligned to 4 bytes");
+  if (reinterpret_cast<uintptr_t>(sg.exp_avg) % es || reinterpret_cast<uintptr_t>(sg.exp_avg_sq) % es) throw Invalid("pointer not aligned to the element size");
   for (int r = 0; r < world; ++r) {
     if (!sg.grad[r] || !sg.param[r]) throw Invalid("NULL gradient or parameter");
     const uintptr_t a = reinterpret_cast<uintptr_t>(sg.grad[r]), b = reinterpret_cast<uintptr_t>(sg.param[r]);
-    if (a % 4 || b % 4) throw Invalid("pointer not aligned to 4 bytes");
+    if (a % es || b % es) throw Invalid("pointer not aligned to the element size");
   }
   for (int r = world; r < TDM_MAX_WORLD; ++r)
     if (sg.grad[r] || sg.param[r]) throw Invalid("pointers of ranks beyond the world size must be NULL");
   const SegPlan plan = plan_step(sg);
-  const int64_t skip = static_cast<int64_t>(plan.head) * 4;  // the kernel reaches back for the head
+  const int64_t skip = static_cast<int64_t>(plan.head) * es;  // the kernel reaches back for the head
   for (int r = 0; r < world; ++r) {
     whole.g[r] = static_cast<const char*>(sg.grad[r]) + skip;
     whole.p[r] = static_cast<char*>(sg.param[r]) + skip;
@@ -431,7 +429,20 @@ void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const t
   whole.count = plan.body;
   whole.chunk = sg.chunk;
   whole.vec_ok = plan.vec ? 1 + plan.head : 0;
-  const int64_t tiles = plan.tiles;
+  *tiles = plan.tiles;
+  return whole;
+}
+}  // namespace
+
+// Used by the engine too: ZeRO-2's step over one segment (a rank's shard), see tdm_k23_zero2_step_segment.
+void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const tdm_adamw_scalars& s, int order, hipStream_t stream) {
+  if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
+  if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
+  if (sg.count < 0) throw Invalid("negative count");
+  if (sg.count == 0) return;
+  if (sg.dtype != TDM_F32) throw Invalid("the step with fp32 constants handles fp32 shards (dtype " + std::to_string(sg.dtype) + "): tdm_k23_zero2_step_segment_typed takes the others");
+  int64_t tiles = 0;
+  const StepSegDev whole = whole_segment(sg, world, &tiles);
   switch (world) {
     case 1: launch_step_one_w<1>(whole, tiles, average, s, order, stream); break;
     case 2: launch_step_one_w<2>(whole, tiles, average, s, order, stream); break;
@@ -1344,7 +1355,7 @@ int tdm_k23_zero2_step(const void* table_dev, int64_t ntiles, int world, int ave
 extern "C++" {
 namespace {
 template <typename T, int kWorld>
-void launch_step_typed_w(const void* image, int64_t tiles, int average, const tdm_adamw_hyper& h, hipStream_t stream) {
+void launch_step_typed_w(const void* image, const StepSegDev* whole, int64_t tiles, int average, const tdm_adamw_hyper& h, hipStream_t stream) {
   const AdamwHyper<typename AdamwMath<T>::S> s = typed_hyper<T>(h);
   const Divisor<T> dv = make_divisor<T>(kWorld);
   const StepSegDev* t = static_cast<const StepSegDev*>(image);
@@ -1354,6 +1365,14 @@ void launch_step_typed_w(const void* image, int64_t tiles, int average, const td
   const int set = g_occupancy_pad[TDM_XCD_STEP].load(std::memory_order_relaxed);
   const unsigned pad = set >= 0 ? static_cast<unsigned>(set) : sizeof(T) == 2 ? 16384u : occupancy_pad(TDM_XCD_STEP);
   const int shift = xcd_shift(TDM_XCD_STEP, kWorld, true);
+  if (whole != nullptr) {  // one segment, described in the kernel's arguments
+    switch (div_kind(kWorld, average != 0)) {
+      case 0: hipLaunchKernelGGL((k23_zero2_step_one_typed_kernel<T, kWorld, 0>), grid, block, pad, stream, *whole, tiles, dv, s, shift); break;
+      case 1: hipLaunchKernelGGL((k23_zero2_step_one_typed_kernel<T, kWorld, 1>), grid, block, pad, stream, *whole, tiles, dv, s, shift); break;
+      default: hipLaunchKernelGGL((k23_zero2_step_one_typed_kernel<T, kWorld, 2>), grid, block, pad, stream, *whole, tiles, dv, s, shift); break;
+    }
+    return;
+  }
   switch (div_kind(kWorld, average != 0)) {
     case 0: hipLaunchKernelGGL((k23_zero2_step_typed_kernel<T, kWorld, 0>), grid, block, pad, stream, t, tiles, dv, s, shift); break;
     case 1: hipLaunchKernelGGL((k23_zero2_step_typed_kernel<T, kWorld, 1>), grid, block, pad, stream, t, tiles, dv, s, shift); break;
@@ -1362,16 +1381,16 @@ void launch_step_typed_w(const void* image, int64_t tiles, int average, const td
 }
 
 template <typename T>
-void launch_step_typed(const void* image, int64_t tiles, int world, int average, const tdm_adamw_hyper& h, hipStream_t stream) {
+void launch_step_typed(const void* image, const StepSegDev* whole, int64_t tiles, int world, int average, const tdm_adamw_hyper& h, hipStream_t stream) {
   switch (world) {
-    case 1: launch_step_typed_w<T, 1>(image, tiles, average, h, stream); break;
-    case 2: launch_step_typed_w<T, 2>(image, tiles, average, h, stream); break;
-    case 3: launch_step_typed_w<T, 3>(image, tiles, average, h, stream); break;
-    case 4: launch_step_typed_w<T, 4>(image, tiles, average, h, stream); break;
-    case 5: launch_step_typed_w<T, 5>(image, tiles, average, h, stream); break;
-    case 6: launch_step_typed_w<T, 6>(image, tiles, average, h, stream); break;
-    case 7: launch_step_typed_w<T, 7>(image, tiles, average, h, stream); break;
-    case 8: launch_step_typed_w<T, 8>(image, tiles, average, h, stream); break;
+    case 1: launch_step_typed_w<T, 1>(image, whole, tiles, average, h, stream); break;
+    case 2: launch_step_typed_w<T, 2>(image, whole, tiles, average, h, stream); break;
+    case 3: launch_step_typed_w<T, 3>(image, whole, tiles, average, h, stream); break;
+    case 4: launch_step_typed_w<T, 4>(image, whole, tiles, average, h, stream); break;
+    case 5: launch_step_typed_w<T, 5>(image, whole, tiles, average, h, stream); break;
+    case 6: launch_step_typed_w<T, 6>(image, whole, tiles, average, h, stream); break;
+    case 7: launch_step_typed_w<T, 7>(image, whole, tiles, average, h, stream); break;
+    case 8: launch_step_typed_w<T, 8>(image, whole, tiles, average, h, stream); break;
     default: throw Invalid("world must be in [1, 8]");
   }
 }
@@ -1397,10 +1416,45 @@ int tdm_k23_zero2_step_typed(const void* table_dev, int64_t ntiles, int world, i
       return;
     }
     if (order != TDM_ADAMW_HOST_ORDER) throw Invalid("the device order is defined for fp32 shards only");
-    if (dtype == TDM_F64) launch_step_typed<double>(table_dev, ntiles, world, average, *h, st);
-    else if (dtype == TDM_BF16) launch_step_typed<bf16_t>(table_dev, ntiles, world, average, *h, st);
-    else launch_step_typed<f16_t>(table_dev, ntiles, world, average, *h, st);
+    if (dtype == TDM_F64) launch_step_typed<double>(table_dev, nullptr, ntiles, world, average, *h, st);
+    else if (dtype == TDM_BF16) launch_step_typed<bf16_t>(table_dev, nullptr, ntiles, world, average, *h, st);
+    else launch_step_typed<f16_t>(table_dev, nullptr, ntiles, world, average, *h, st);
     check_hip(hipGetLastError(), "k23_zero2_step (typed) launch");
+  });
+}
+
+extern "C++" {
+namespace tandem_hip {
+// Used by the engine too: the same over a segment of any of K3's shard types (seg.dtype), constants as Python doubles.
+void zero2_step_segment_typed(const tdm_step_seg& sg, int world, bool average, const tdm_adamw_hyper& h, int order, hipStream_t stream) {
+  if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
+  if (order != TDM_ADAMW_HOST_ORDER && order != TDM_ADAMW_DEVICE_ORDER) throw Invalid("unknown update order");
+  if (sg.count < 0) throw Invalid("negative count");
+  if (step_elem_size(sg) == 0) throw Invalid("a step segment's dtype must be TDM_F32, TDM_F64, TDM_BF16 or TDM_F16");
+  if (sg.dtype == TDM_F32) {  // a Python double applied to a float tensor is rounded to fp32 once
+    const tdm_adamw_scalars s{h.use_decay, static_cast<float>(h.decay), static_cast<float>(h.w1), static_cast<float>(h.beta2),
+                              static_cast<float>(h.one_m_b2), static_cast<float>(h.bc2_sqrt), static_cast<float>(h.eps),
+                              static_cast<float>(h.neg_step), static_cast<float>(1.0 / h.bc2_sqrt)};
+    zero2_step_segment(sg, world, average, s, order, stream);
+    return;
+  }
+  if (order != TDM_ADAMW_HOST_ORDER) throw Invalid("the device order is defined for fp32 shards only");
+  if (sg.count == 0) return;
+  int64_t tiles = 0;
+  const StepSegDev whole = whole_segment(sg, world, &tiles);
+  if (sg.dtype == TDM_F64) launch_step_typed<double>(nullptr, &whole, tiles, world, average, h, stream);
+  else if (sg.dtype == TDM_BF16) launch_step_typed<bf16_t>(nullptr, &whole, tiles, world, average, h, stream);
+  else launch_step_typed<f16_t>(nullptr, &whole, tiles, world, average, h, stream);
+  check_hip(hipGetLastError(), "k23_zero2_step_one (typed) launch");
+}
+}  // namespace tandem_hip
+}  // extern "C++"
+
+int tdm_k23_zero2_step_segment_typed(const tdm_step_seg* seg, int world, int average, const tdm_adamw_hyper* h, int order,
+                                     tdm_stream stream) {
+  return guard([&] {
+    if (seg == nullptr || h == nullptr) throw Invalid("NULL argument");
+    zero2_step_segment_typed(*seg, world, average != 0, *h, order, static_cast<hipStream_t>(stream));
   });
 }
 

@@ -1284,6 +1284,21 @@ __global__ __launch_bounds__(kThreads) void k23_zero2_step_typed_kernel(const St
   }
 }
 
+// The typed step for ONE segment described in the kernel's arguments (as k23_zero2_step_one_kernel is for fp32).
+template <typename T, int kWorld, int kDiv>
+__global__ __launch_bounds__(kThreads) void k23_zero2_step_one_typed_kernel(StepSegDev whole, int64_t total, Divisor<T> dv,
+                                                                            AdamwHyper<typename AdamwMath<T>::S> s, int shift) {
+  using S = typename AdamwMath<T>::S;
+  const bool small_w = (s.w1 < S(0) ? -s.w1 : s.w1) < S(0.5);
+  constexpr int64_t kPartElems = static_cast<int64_t>(kTileVecs / kStepParts) * lanes<T>();
+  for (int64_t at = blockIdx.x; at < total * kStepParts; at += gridDim.x) {
+    const int64_t part = tile_of(at, total * kStepParts, shift);
+    const int64_t n = min(kPartElems, whole.count - part * kPartElems);
+    const int head = part == 0 ? whole.vec_ok - 1 : 0;
+    if (n > 0) step_tile_typed<T, kWorld, kDiv, kUnroll / kStepParts>(whole, part * kPartElems * static_cast<int64_t>(sizeof(T)), n, head, dv, s, small_w);
+  }
+}
+
 }  // namespace
 
 }  // namespace tandem_hip

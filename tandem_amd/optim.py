@@ -136,15 +136,19 @@ class ShardedAdamW:
     def begin_step(self, key, param):
         """For a caller that runs the update inside a fused launch of its own
         (Group.zero2_step): creates the shard's state if need be, counts the step, and
-        returns (scalars, exp_avg, exp_avg_sq, order) for it."""
+        returns (constants, exp_avg, exp_avg_sq, order) for it: the constants rounded to fp32
+        for an fp32 shard (AdamwScalars), as doubles for the other shard types (AdamwHyper)."""
         require_device_tensor(param, "ShardedAdamW.begin_step(param)")
-        if param.dtype != torch.float32:
-            raise ValueError("the fused ZeRO-2 step between process ranks handles fp32 shards (update() also takes float64, bfloat16 and float16)")
+        if param.dtype not in SHARD_DTYPES:
+            raise ValueError(f"ShardedAdamW handles float32, float64, bfloat16 and float16 shards, not {param.dtype}")
+        if param.dtype != torch.float32 and self.order != ADAMW_HOST_ORDER:
+            raise ValueError("order='device' is defined for fp32 shards only")
         if key not in self.state:
             self.state[key] = [0.0, zeros_at_phase_of(param), zeros_at_phase_of(param)]
         st = self.state[key]
         st[0] += 1.0
-        return step_scalars(st[0], self.lr, self.betas, self.eps, self.weight_decay), st[1], st[2], self.order
+        constants = step_scalars if param.dtype == torch.float32 else step_hyper  # fp32 constants for fp32 shards, doubles otherwise
+        return constants(st[0], self.lr, self.betas, self.eps, self.weight_decay), st[1], st[2], self.order
 
     def state_bytes(self):
         return sum(t.numel() * t.element_size() for _, a, b in self.state.values() for t in (a, b))

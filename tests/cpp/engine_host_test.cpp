@@ -258,6 +258,39 @@ static int run_rank(int rank, int world, const std::string& job, std::atomic<int
     }
   }
 
+  // the same step over float64 buffers, its constants as doubles: the typed entry point, the element size in the arena offsets
+  {
+    double* grads = reinterpret_cast<double*>(t);
+    double* params = grads + (n + 63) / 64 * 64;
+    std::vector<int64_t> goffs(world), poffs(world);
+    for (int q = 0; q < world; ++q) {
+      goffs[q] = offs[q] + lo * 8;
+      poffs[q] = offs[q] + ((n + 63) / 64 * 64 + lo) * 8;
+    }
+    for (int64_t i = 0; i < n; ++i) {
+      grads[i] = static_cast<double>(world) * value(rank, i, 905);
+      params[i] = value(0, i, 906);
+    }
+    std::vector<double> m(sizes[rank], 0.0), v(sizes[rank], 0.0);
+    tdm_adamw_hyper hy;
+    std::memset(&hy, 0, sizeof hy);
+    REQUIRE(tdm_direct_zero2_step_typed(e, params + lo, poffs.data(), grads + lo, goffs.data(), world, m.data(), v.data(), sizes[rank], n, 1,
+                                        TDM_F64, &hy, TDM_ADAMW_DEVICE_ORDER, nullptr, &w) == TDM_EINVAL);  // fp32 only
+    REQUIRE(tdm_direct_zero2_step_typed(e, params + lo, poffs.data(), grads + lo, goffs.data(), world, m.data(), v.data(), sizes[rank], n, 1,
+                                        TDM_I32, &hy, TDM_ADAMW_HOST_ORDER, nullptr, &w) == TDM_EINVAL);
+    REQUIRE(tdm_direct_zero2_step_typed(e, params + lo, poffs.data(), grads + lo, goffs.data(), world, m.data(), v.data(), sizes[rank], n, 1,
+                                        TDM_F64, nullptr, TDM_ADAMW_HOST_ORDER, nullptr, &w) == TDM_EINVAL);
+    REQUIRE(tdm_direct_zero2_step_typed(e, params + lo, poffs.data(), grads + lo, goffs.data(), world, m.data(), v.data(), sizes[rank], n, 1,
+                                        TDM_F64, &hy, TDM_ADAMW_HOST_ORDER, nullptr, &w) == TDM_OK);
+    REQUIRE(tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
+    for (int64_t i = 0; i < n; ++i) {
+      double g = 0;
+      for (int q = 0; q < world; ++q) g += value(q, i, 905);
+      REQUIRE(params[i] == value(0, i, 906) - g);
+      if (i >= lo && i < lo + sizes[rank]) REQUIRE(m[i - lo] == g && v[i - lo] == g * g);
+    }
+  }
+
   // the same gather through the engine's own path (no arenas), produced and consumed on the caller's stream, with device
   // time stamps on
   REQUIRE(tdm_engine_set_timing(e, 1) == TDM_OK);

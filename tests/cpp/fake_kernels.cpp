@@ -105,21 +105,36 @@ void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool av
 // The data flow of ZeRO-2's step, not its arithmetic: the shard's gradients folded in the ring's order and averaged, the
 // moments bumped, and "parameter - gradient" written into every rank's parameter buffer. (AdamW itself is the kernels'
 // and the GPU tests' business.)
-void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const tdm_adamw_scalars&, int, hipStream_t stream) {
+namespace {
+template <typename T>
+void step_data_flow(const tdm_step_seg& sg, int world, bool average, hipStream_t stream) {
   if (world < 1 || world > TDM_MAX_WORLD) throw Invalid("world must be in [1, 8]");
   const tdm_step_seg seg = sg;
   fake_enqueue(stream, [=] {
-    float* m = static_cast<float*>(seg.exp_avg);
-    float* v = static_cast<float*>(seg.exp_avg_sq);
+    T* m = static_cast<T*>(seg.exp_avg);
+    T* v = static_cast<T*>(seg.exp_avg_sq);
     for (int64_t k = 0; k < seg.count; ++k) {
-      float g = divided(static_cast<const float*>(seg.grad[(seg.chunk + 1) % world])[k], average ? world : 1);
-      for (int j = 2; j <= world; ++j) g = divided(static_cast<const float*>(seg.grad[(seg.chunk + j) % world])[k], average ? world : 1) + g;
+      T g = divided(static_cast<const T*>(seg.grad[(seg.chunk + 1) % world])[k], average ? world : 1);
+      for (int j = 2; j <= world; ++j) g = divided(static_cast<const T*>(seg.grad[(seg.chunk + j) % world])[k], average ? world : 1) + g;
       m[k] += g;
       v[k] += g * g;
-      const float p = static_cast<const float*>(seg.param[seg.chunk])[k] - g;
-      for (int r = 0; r < world; ++r) static_cast<float*>(seg.param[r])[k] = p;
+      const T p = static_cast<const T*>(seg.param[seg.chunk])[k] - g;
+      for (int r = 0; r < world; ++r) static_cast<T*>(seg.param[r])[k] = p;
     }
   });
+}
+}  // namespace
+
+void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const tdm_adamw_scalars&, int, hipStream_t stream) {
+  if (sg.dtype != TDM_F32) throw Invalid("fp32 constants go with fp32 shards");
+  step_data_flow<float>(sg, world, average, stream);
+}
+
+// The same for the shard types that take their constants as doubles; the stand-in knows fp32 and float64.
+void zero2_step_segment_typed(const tdm_step_seg& sg, int world, bool average, const tdm_adamw_hyper&, int, hipStream_t stream) {
+  if (sg.dtype == TDM_F32) step_data_flow<float>(sg, world, average, stream);
+  else if (sg.dtype == TDM_F64) step_data_flow<double>(sg, world, average, stream);
+  else throw Invalid("the stand-in steps fp32 and float64 shards");
 }
 
 }  // namespace tandem_hip

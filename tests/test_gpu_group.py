@@ -462,6 +462,80 @@ def test_zero2_step_in_one_launch_per_rank(world):
     assert all(out["refused"] == 5 for out in res)
 
 
+def zero2_steps_typed(g, name, ns, steps):
+    """zero2_steps over buffers of another shard type: begin_step hands out the constants as doubles."""
+    from tandem_amd import CommError, ShardedAdamW
+    from tandem_amd._lib import AdamwHyper
+    from tandem_amd.optim import step_scalars
+
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f64": torch.float64}[name]
+    w, r = g.size, g.rank
+    g.share_arena(8 << 20)
+    out = {}
+    for n in ns:
+        sizes = [n // w + (1 if q < n % w else 0) for q in range(w)]
+        lo = sum(sizes[:r])
+        params, grads = g.shared_empty(n, dtype), g.shared_empty(n, dtype)
+        params.copy_((seeded(3, 0, n).double() * 0.02).to(dtype))
+        opt = ShardedAdamW(lr=1e-3, betas=(0.9, 0.95), eps=1e-6, weight_decay=0.1)
+        for step in range(steps):
+            grads.copy_((seeded(100 + step, r, n).double() * (2e-2 if name == "f16" else 1e-3)).to(dtype))
+            constants, m, v, order = opt.begin_step("flat", params[lo:lo + sizes[r]])
+            assert isinstance(constants, AdamwHyper) and m.dtype == dtype
+            assert g.zero2_step(params, grads, sizes, m, v, constants, order) is params
+        view = (lambda t: t.cpu().view(torch.int16).numpy().view(np.uint16).copy()) if name != "f64" else (lambda t: t.cpu().numpy().copy())
+        out[n] = (view(params), view(m), view(v))
+    refused = 0
+    n = 1000
+    sizes = [n // w + (1 if q < n % w else 0) for q in range(w)]
+    arena, state = g.shared_empty(n, dtype), torch.zeros(sizes[r], device=g.device, dtype=dtype)
+    for constants, order in ((step_scalars(1.0, 3e-4, (0.9, 0.95), 1e-8, 0.1), 0), (opt.begin_step("other", arena[:sizes[r]])[0], 1)):
+        try:  # fp32 constants with another dtype; the device order on another dtype
+            g.zero2_step(arena, g.shared_empty(n, dtype), sizes, state, state.clone(), constants, order)
+        except (CommError, ValueError):
+            refused += 1
+    out["refused"] = refused
+    return out
+
+
+@pytest.mark.parametrize("name", ["bf16", "f16", "f64"])
+@pytest.mark.parametrize("world", [2, 3])
+def test_zero2_step_in_one_launch_per_rank_on_other_shard_types(world, name):
+    """The same fused step between process ranks over bfloat16, float16 and float64 buffers
+    (tdm_direct_zero2_step_typed): the ring's fold in the type's own rounding, 0 + mine, the typed AdamW,
+    the new parameters in every rank's buffer; bit for bit with the oracle, state included."""
+    from oracle import ring
+    from oracle.adamw import AdamW
+    from tandem_amd import launch
+
+    ns, steps = (0, 5, 1001, 40_007), 3
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f64": torch.float64}[name]
+    raw = (lambda t: t.view(torch.int16).numpy().view(np.uint16).copy()) if name != "f64" else (lambda t: t.numpy().copy())
+    res = launch(zero2_steps_typed, world, name, ns, steps, gpus=[0] * world, timeout=TIMEOUT)
+    for n in ns:
+        sizes = [n // world + (1 if q < n % world else 0) for q in range(world)]
+        want = raw((seeded(3, 0, n).double() * 0.02).to(dtype))
+        opts = [AdamW(lr=1e-3, betas=(0.9, 0.95), eps=1e-6, weight_decay=0.1, kind=name if name != "f64" else None) for _ in range(world)]
+        for step in range(steps):
+            xs = [raw((seeded(100 + step, q, n).double() * (2e-2 if name == "f16" else 1e-3)).to(dtype)) for q in range(world)]
+            outs = ring.expected_reduce_scatter(xs, sizes, True, name)
+            for q in range(world):
+                lo = sum(sizes[:q])
+                mine = outs[q][lo:lo + sizes[q]].copy()
+                if name != "f64":
+                    mine[mine == 0x8000] = 0  # 0 + (-0) = +0
+                else:
+                    mine = 0.0 + mine
+                opts[q].update("flat", want[lo:lo + sizes[q]], mine)
+        for r, out in enumerate(res):
+            p, m, v = out[n]
+            assert np.array_equal(bits(p), bits(want)), (world, n, r)
+            if sizes[r]:
+                assert np.array_equal(bits(m), bits(opts[r].state["flat"][1])), (world, n, r)
+                assert np.array_equal(bits(v), bits(opts[r].state["flat"][2])), (world, n, r)
+    assert all(out["refused"] == 2 for out in res)
+
+
 def async_order(g):
     # several collectives in flight complete in submission order with the right values
     xs = [torch.full((3000 + k,), float(g.rank + k), device=g.device) for k in range(5)]

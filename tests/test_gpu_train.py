@@ -189,7 +189,8 @@ def train_rank_typed(g, strategy, dtype_name, steps, batch):
     elif strategy.startswith("zero3"):
         z = FSDP(model, g, sopt, direct=not strategy.endswith("s"))
     else:
-        z = ZeRO(model, g, int(strategy[4]), sopt, 4 << 10, direct=strategy.endswith("d"))
+        fused = strategy.endswith("f")  # reduce-scatters, AdamW and all-gather as one launch per rank
+        z = ZeRO(model, g, int(strategy[4]), sopt, 4 << 10, direct=strategy.endswith("d") or fused, fused_step=fused)
     losses = []
     for step in range(steps):
         x, y = text.batch(step, batch, c.seq, rank=g.rank, world=g.size, device=g.device)
@@ -213,14 +214,14 @@ def train_rank_typed(g, strategy, dtype_name, steps, batch):
 
 @pytest.mark.parametrize("dtype_name", ["bfloat16", "float64"])
 def test_bf16_and_f64_models_all_strategies_agree(dtype_name):
-    """Two ranks, a bfloat16 and a float64 model: DDP, ZeRO-1, ZeRO-2 and FSDP, through the slots and arena to arena, must
+    """Two ranks, a bfloat16 and a float64 model: DDP, ZeRO-1, ZeRO-2 (also with its step as one launch per rank) and FSDP, through the slots and arena to arena, must
     end with the same weights bit for bit and see the same losses (at two ranks the average is (a/2) + (b/2) in any order,
     and the update is per element), and the model must learn. What the kernels compute for these types is pinned against
     the oracle elsewhere; this is the wrappers carrying the dtype through buckets, shards, optimizer state and gathers."""
     from tandem_amd import launch
 
     runs = {s: launch(train_rank_typed, 2, s, dtype_name, STEPS, BATCH, slot_bytes=4096, gpus=[0, 0], timeout=TIMEOUT)
-            for s in ("ddp", "ddpd", "zero1", "zero1d", "zero2", "zero2d", "zero3", "zero3s")}
+            for s in ("ddp", "ddpd", "zero1", "zero1d", "zero2", "zero2d", "zero2f", "zero3", "zero3s")}
     ref = runs["ddp"]
     assert ref[0]["losses"][-1] < ref[0]["losses"][0]
     for s, res in runs.items():
