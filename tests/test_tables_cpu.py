@@ -146,6 +146,20 @@ def test_step_tables_refuse_mixed_and_unknown_dtypes():
     assert L.tdm_k3_adamw_typed(ptr, ptr, ptr, ptr, 4, 5, ctypes.byref(hyper), 0, None, 0, None) == EINVAL and "dtype" in L.tdm_last_error().decode()
     assert L.tdm_k3_adamw_typed(ptr, ptr, ptr, ptr, 4, BF16, ctypes.byref(hyper), 1, None, 0, None) == EINVAL and "fp32 shards only" in L.tdm_last_error().decode()
     assert L.tdm_k3_adamw_typed(ptr, ptr, ptr, ptr, 0, BF16, ctypes.byref(hyper), 0, None, 0, None) == 0  # nothing to do
+    # so does the step over one segment passed in the launch
+    one = step_segs(2, [(100, 1, 0)], F64)
+    scalars = _lib.AdamwScalars()
+    assert L.tdm_k23_zero2_step_segment(one, 2, 1, ctypes.byref(scalars), 0, None) == EINVAL and "fp32 shards" in L.tdm_last_error().decode()
+    assert L.tdm_k23_zero2_step_segment_typed(one, 2, 1, ctypes.byref(hyper), 1, None) == EINVAL and "fp32 shards only" in L.tdm_last_error().decode()
+    assert L.tdm_k23_zero2_step_segment_typed(one, 9, 1, ctypes.byref(hyper), 0, None) == EINVAL and "world" in L.tdm_last_error().decode()
+    assert L.tdm_k23_zero2_step_segment_typed(one, 1, 1, ctypes.byref(hyper), 0, None) == EINVAL and "chunk" in L.tdm_last_error().decode()
+    assert L.tdm_k23_zero2_step_segment_typed(one, 2, 1, None, 0, None) == EINVAL and L.tdm_k23_zero2_step_segment_typed(None, 2, 1, ctypes.byref(hyper), 0, None) == EINVAL
+    one[0].grad[1] += 4
+    assert L.tdm_k23_zero2_step_segment_typed(one, 2, 1, ctypes.byref(hyper), 0, None) == EINVAL and "element size" in L.tdm_last_error().decode()
+    one[0].dtype = 7  # TDM_I16
+    assert L.tdm_k23_zero2_step_segment_typed(one, 2, 1, ctypes.byref(hyper), 0, None) == EINVAL and "dtype" in L.tdm_last_error().decode()
+    one[0].dtype, one[0].count = BF16, 0
+    assert L.tdm_k23_zero2_step_segment_typed(one, 2, 1, ctypes.byref(hyper), 0, None) == 0  # nothing to do
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "float64", "bfloat16", "float16"])
