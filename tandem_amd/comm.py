@@ -344,12 +344,12 @@ class Group:
                 raise CommError("zero2_step: the buffers must come from shared_empty()")
             bases.append((ctypes.c_int64 * self.size)(*[off + lo * es] * self.size))
         mine_p, mine_g = p[lo:lo + n], g[lo:lo + n]
-        head = lambda: (self._engine, ctypes.c_void_p(mine_p.data_ptr()), bases[0], ctypes.c_void_p(mine_g.data_ptr()), bases[1], self.size,
-                        ctypes.c_void_p(exp_avg.data_ptr()), ctypes.c_void_p(exp_avg_sq.data_ptr()), n, p.numel(), int(op == "avg"))
+        head = (self._engine, ctypes.c_void_p(mine_p.data_ptr()), bases[0], ctypes.c_void_p(mine_g.data_ptr()), bases[1], self.size,
+                ctypes.c_void_p(exp_avg.data_ptr()), ctypes.c_void_p(exp_avg_sq.data_ptr()), n, p.numel(), int(op == "avg"))
         if typed:
-            call = lambda out: lib().tdm_direct_zero2_step_typed(*head(), dtype_code(p.dtype), ctypes.byref(scalars), order, self._stream(), out)
+            call = lambda out: lib().tdm_direct_zero2_step_typed(*head, dtype_code(p.dtype), ctypes.byref(scalars), order, self._stream(), out)
         else:
-            call = lambda out: lib().tdm_direct_zero2_step(*head(), ctypes.byref(scalars), order, self._stream(), out)
+            call = lambda out: lib().tdm_direct_zero2_step(*head, ctypes.byref(scalars), order, self._stream(), out)
         return self._start("zero2_step", call, params, (2 * self.size + 5) * es * n, async_op, keep=(p, g, exp_avg, exp_avg_sq, scalars))
 
     # ---- shared arenas: long-lived data that peers read (and the direct collectives write) in place
