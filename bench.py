@@ -784,6 +784,54 @@ def cpu_config1_rank(g, reps):
     return statistics.median(ts)
 
 
+def cpu_two_rank_paths(g, numels):
+    """The two-rank paths on the host. DDP's bucket path (tandem/ddp.py:89-119): 149 gradients copied into 16
+    buckets of up to 25 MiB in reverse registration order, one all_reduce(avg) per bucket, copied back. ZeRO-3's
+    unit gather (tandem/zero.py:238-252): the all_gather of one block unit of 7,087,872 fp32, twelve units in turn."""
+    import torch
+
+    from tandem_amd.buckets import pack
+
+    gen = torch.Generator().manual_seed(100 + g.rank)
+    grads = [torch.randn(m, generator=gen) * 1e-3 for m in numels]
+    order = list(range(len(numels)))[::-1]
+    buckets = [[order[k] for k in b] for b in pack([numels[i] * 4 for i in order], 25 << 20)]
+    flats = [torch.empty(sum(numels[i] for i in b)) for b in buckets]
+    ts = []
+    for _ in range(3):
+        g.barrier()
+        t = time.perf_counter()
+        works = []
+        for b, flat in zip(buckets, flats):
+            at = 0
+            for i in b:
+                flat[at:at + numels[i]].copy_(grads[i])
+                at += numels[i]
+            works.append(g.all_reduce(flat, op="avg", async_op=True))
+        for b, flat, w in zip(buckets, flats, works):
+            w.wait()
+            at = 0
+            for i in b:
+                grads[i].copy_(flat[at:at + numels[i]])
+                at += numels[i]
+        ts.append(time.perf_counter() - t)
+    out = {"bucket_path_s": statistics.median(ts)}
+    del grads, flats
+    unit, units = 7_087_872, 12
+    sizes = [unit // g.size] * g.size
+    lo = sum(sizes[:g.rank])
+    fulls = [torch.zeros(unit) for _ in range(units)]
+    for k, full in enumerate(fulls):
+        full[lo:lo + sizes[g.rank]] = torch.randn(sizes[g.rank], generator=torch.Generator().manual_seed(7 * k + g.rank))
+    g.all_gather(fulls[0], sizes)
+    g.barrier()
+    t = time.perf_counter()
+    for full in fulls:
+        g.all_gather(full, sizes)
+    out["unit_gather_s"] = (time.perf_counter() - t) / units
+    return out
+
+
 def cpu_baseline(mib, reps):
     from oracle.cpu_engine import cpu_launch
 
@@ -791,6 +839,7 @@ def cpu_baseline(mib, reps):
     t0 = time.perf_counter()
     res = cpu_launch(cpu_rank, WORLD, n, reps, gpt_numels())
     small = max(cpu_launch(cpu_config1_rank, 2, 20))
+    two = cpu_launch(cpu_two_rank_paths, 2, gpt_numels())
     total = time.perf_counter() - t0
     t = max(r["all_reduce_s"] for r in res)
     z = max(r["zero2_step_s"] for r in res)
@@ -798,7 +847,12 @@ def cpu_baseline(mib, reps):
             "sample": f"oracle CPU-process engine (tandem's Python-engine protocol): ring all-reduce(avg), world 4 x 1 torch thread, "
                       f"{mib} MiB fp32 per rank (the GPU workload), 2 x 4 MiB shared-memory slots per pair, median of {reps}: "
                       f"{t * 1e3:.1f} ms per all-reduce; then 3 ZeRO-2 steps at 85,842,432 params (16 reduce-scatters, shard add, AdamW as torch ops, all-gather); {total:.1f} s in all, {total * WORLD:.0f} core-seconds",
-            "algbw_GBps": round(n * 4 / t / 1e9, 3), "zero2_step_ms": round(z * 1e3, 1), "host_cores": os.cpu_count()}
+            "algbw_GBps": round(n * 4 / t / 1e9, 3), "zero2_step_ms": round(z * 1e3, 1),
+            "bucket_path_2_ranks_ms": round(max(r["bucket_path_s"] for r in two) * 1e3, 1),
+            "unit_gather_2_ranks_ms": round(max(r["unit_gather_s"] for r in two) * 1e3, 2),
+            "two_rank_sample": "2 ranks x 1 torch thread: DDP's bucket path for the 85.8M GPT (149 gradients into 16 buckets, all_reduce(avg) each, "
+                               "copied back), median of 3; ZeRO-3's all_gather of a 7,087,872-element unit, mean of 12 units in turn",
+            "host_cores": os.cpu_count()}
 
 
 CONFIG_KEYS_KEPT = 24  # a record that keeps only the first keys of `config` must still hold the whole metric
@@ -1041,6 +1095,10 @@ def main():
             cpu["gpu_over_cpu"] = round(line["value"] / cpu["value"], 1)
             if "zero2_step" in line:
                 cpu["zero2_step_gpu_over_cpu"] = round(cpu["zero2_step_ms"] / line["zero2_step"]["one_launch_ms"], 1)
+            if "bucket_path" in line:
+                cpu["bucket_path_gpu_over_cpu"] = round(cpu["bucket_path_2_ranks_ms"] / line["bucket_path"]["ms"], 1)
+            if "unit_gather" in line:
+                cpu["unit_gather_gpu_over_cpu"] = round(cpu["unit_gather_2_ranks_ms"] * 1e3 / line["unit_gather"]["us_per_unit"], 1)
         if cpu is not None:
             line["cpu_baseline"] = cpu
     summarize(line)
