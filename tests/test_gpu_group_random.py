@@ -4,6 +4,8 @@ on every rank), the operation and its variant drawn at random, many in a row on 
 staging halves and slots are reused in every combination. Every rank checks its own result bit
 for bit against the oracle and the guard elements around its view. Run with -m gpu."""
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -11,6 +13,7 @@ import torch
 from helpers import bits
 
 pytestmark = pytest.mark.gpu
+SHIFT = int(os.environ.get("TANDEM_SWEEP_SEED", "0"))  # added to the sweep's seed: other cases of the same kinds
 
 KINDS = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16", torch.int64: "i64",
          torch.int32: "i32", torch.int16: "i16", torch.int8: "i8", torch.uint8: "u8"}
@@ -103,5 +106,5 @@ def test_seeded_sweep_between_processes(world, algo, monkeypatch):
 
     monkeypatch.setenv("TANDEM_HIP_ALGO", algo)
     monkeypatch.setenv("TANDEM_HIP_STAGING_BYTES", "65536")  # a 40,000-element fp64 tensor takes several passes
-    for wrong in launch(sweep, world, 31 + world, 120, slot_bytes=16384, gpus=[0] * world, timeout=TIMEOUT):
+    for wrong in launch(sweep, world, 31 + world + SHIFT, 120, slot_bytes=16384, gpus=[0] * world, timeout=TIMEOUT):
         assert wrong == []

@@ -4,6 +4,8 @@ inside their allocation (every rank at the same distance from a 16-byte boundary
 forms of the ring and the single-launch all-reduce. Every result bit for bit against the
 oracle, and the guard elements around every view untouched. Run with -m gpu."""
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -11,6 +13,7 @@ import torch
 from helpers import bits
 
 pytestmark = pytest.mark.gpu
+SHIFT = int(os.environ.get("TANDEM_SWEEP_SEED", "0"))  # added to every sweep's seed: other cases of the same kinds
 
 KINDS = {torch.float32: "f32", torch.float64: "f64", torch.float16: "f16", torch.bfloat16: "bf16", torch.int64: "i64",
          torch.int32: "i32", torch.int16: "i16", torch.int8: "i8", torch.uint8: "u8"}
@@ -63,7 +66,7 @@ def test_seeded_sweep(form):
     dev = torch.device("cuda", 0)
     assert lib().tdm_set_ring_form(0 if form == "steps" else 1) == 0
     try:
-        for k, world, dtype, n, sizes, starts, seed in cases(600, 20260):
+        for k, world, dtype, n, sizes, starts, seed in cases(600, 20260 + SHIFT):
             kind = KINDS[dtype]
             rng = np.random.default_rng(seed)
             xs = [draw(rng, dtype, n) for _ in range(world)]
@@ -146,7 +149,7 @@ def test_seeded_sweep_of_bucket_tables():
 
     assert torch.cuda.is_available(), "these tests need the MI355X"
     dev = torch.device("cuda", 0)
-    for k, world, dtype, numels, buckets, starts, elsewhere, static, seed in bucket_cases(150, 77):
+    for k, world, dtype, numels, buckets, starts, elsewhere, static, seed in bucket_cases(150, 77 + SHIFT):
         kind = KINDS[dtype]
         rng = np.random.default_rng(seed)
         grads = [[draw(rng, dtype, n) for n in numels] for _ in range(world)]
@@ -200,7 +203,7 @@ def test_seeded_sweep_of_adamw_shards():
 
     assert torch.cuda.is_available(), "these tests need the MI355X"
     dev = torch.device("cuda", 0)
-    rng = np.random.default_rng(4242)
+    rng = np.random.default_rng(4242 + SHIFT)
     for k in range(80):
         n = int(rng.choice([0, 1, 3, 4, 5, 127, 128, 129, 1000, 4097, 33_333, 70_000])) + int(rng.integers(0, 2))
         kw = dict(lr=float(10 ** rng.uniform(-4, -1.5)), betas=(float(rng.choice([0.0, 0.3, 0.5, 0.9])), float(rng.choice([0.7, 0.95, 0.999]))),
@@ -240,7 +243,7 @@ def test_seeded_sweep_of_zero2_steps():
 
     assert torch.cuda.is_available(), "these tests need the MI355X"
     dev = torch.device("cuda", 0)
-    rng = np.random.default_rng(9)
+    rng = np.random.default_rng(9 + SHIFT)
     kw = dict(lr=3e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
     for k in range(40):
         world = int(rng.integers(1, 9))
@@ -286,7 +289,7 @@ def test_seeded_sweep_of_adamw_shards_of_other_dtypes():
 
     assert torch.cuda.is_available(), "these tests need the MI355X"
     dev = torch.device("cuda", 0)
-    rng = np.random.default_rng(777)
+    rng = np.random.default_rng(777 + SHIFT)
     kinds = {torch.float64: None, torch.bfloat16: "bf16", torch.float16: "f16"}
     for k in range(90):
         dtype = [torch.float64, torch.bfloat16, torch.float16][k % 3]
@@ -330,7 +333,7 @@ def test_seeded_sweep_of_zero2_steps_of_other_dtypes():
 
     assert torch.cuda.is_available(), "these tests need the MI355X"
     dev = torch.device("cuda", 0)
-    rng = np.random.default_rng(31)
+    rng = np.random.default_rng(31 + SHIFT)
     kw = dict(lr=1e-3, betas=(0.9, 0.95), eps=1e-4, weight_decay=0.1)
     for k in range(36):
         dtype = [torch.float64, torch.bfloat16, torch.float16][k % 3]
