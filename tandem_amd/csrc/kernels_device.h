@@ -997,6 +997,7 @@ __global__ __launch_bounds__(kAdamwThreads) void k3_adamw_typed_kernel(AdamwArgs
   const bool small_w = (a.s.w1 < S(0) ? -a.s.w1 : a.s.w1) < S(0.5);
   constexpr int kL = lanes<T>(), kG = AdamwMath<T>::kGroup;
   static_assert(kL % kG == 0, "a vector holds whole groups");
+  static_assert(kL <= 32 && 32 + 128 / static_cast<int>(sizeof(T)) <= kAdamwThreads, "lanes 0.. take the tail, lanes 32.. a head of up to a cache line");
   if constexpr (kVec) {
     const int64_t nv = a.n / kL;
     const int64_t tiles = (nv + kAdamwThreads - 1) / kAdamwThreads;
