@@ -303,10 +303,38 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
       inner();
     };
   }
+  hipEvent_t mark = nullptr;
+  if (uses_gpu && gathers_on_side_stream_) {
+    // What a fence inside this job waits for on the gather stream: the gathers launched (by callers' threads) BEFORE
+    // this call. A later gather may itself wait, through the caller's stream, for this job's end (a wait() that parks
+    // the stream, then the next unit's gather): a fence that waited for everything on that stream would wait for itself.
+    hipError_t err = hipEventCreateWithFlags(&mark, hipEventDisableTiming);
+    if (err == hipSuccess && (err = hipEventRecord(mark, gather_stream_)) != hipSuccess) {
+      (void)hipEventDestroy(mark);
+      mark = nullptr;
+    }
+    if (err != hipSuccess) {
+      if (ready) (void)hipEventDestroy(ready);
+      check_hip(err, "marking the gather stream");
+    }
+    job = [this, mark, inner = std::move(job)] {
+      struct Scope {  // the progress thread's alone; the event goes when the job has run or failed
+        Engine* self;
+        hipEvent_t mark;
+        ~Scope() {
+          self->gather_mark_ = nullptr;
+          (void)hipEventDestroy(mark);
+        }
+      } scope{this, mark};
+      gather_mark_ = mark;
+      inner();
+    };
+  }
   {
     std::lock_guard<std::mutex> lock(mu_);
     if (stopping_ || !sticky_error_.empty()) {
       if (ready) (void)hipEventDestroy(ready);  // the job that would have released it never runs
+      if (mark) (void)hipEventDestroy(mark);
       throw std::runtime_error(stopping_ ? "the engine is closed" : "an earlier collective failed: " + sticky_error_);
     }
     jobs_.emplace_back(std::move(job), work);
@@ -516,11 +544,15 @@ void Engine::barrier_now(bool after_gpu, uint64_t tag) {
   // peers anyway, and handing over to the completion thread would cost two wake-ups.
   drain_completions();
   if (after_gpu) {
-    for (hipStream_t st : {stream_, gather_stream_}) {
-      const hipError_t err = poll_gpu([st] { return hipStreamQuery(st); }, timeout_s_);
-      (void)hipGetLastError();
-      check_hip(err, "hipStreamQuery (fence)");
-    }
+    hipError_t err = poll_gpu([this] { return hipStreamQuery(stream_); }, timeout_s_);
+    (void)hipGetLastError();
+    check_hip(err, "hipStreamQuery (fence)");
+    // the gather stream: up to where it stood when this job was submitted (gather_mark_), or all of it
+    hipEvent_t mark = gather_mark_;
+    err = mark ? poll_gpu([mark] { return hipEventQuery(mark); }, timeout_s_)
+               : poll_gpu([this] { return hipStreamQuery(gather_stream_); }, timeout_s_);
+    (void)hipGetLastError();
+    check_hip(err, "waiting for the gather stream (fence)");
   }
   // An empty message to every peer, then one from each. Rings are first in,
   // first out, so this also orders the barrier after every piece queued before.

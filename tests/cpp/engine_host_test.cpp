@@ -230,6 +230,27 @@ static int run_rank(int rank, int world, const std::string& job, std::atomic<int
   }
   REQUIRE(tdm_fence(e, nullptr, &w) == TDM_OK && tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
 
+  // A fence whose wait only parks the caller's stream, and behind it a gather that is launched (by this thread, on the
+  // side stream when gathers run there) before the progress thread has got to the fence: the fence is held back by a slow
+  // producer on the caller's stream. The gather waits for the caller's stream, which waits for the fence's end, so a
+  // fence that waited for EVERYTHING on the side stream would wait for itself. It waits for what was launched before it.
+  {
+    std::fill(full.begin(), full.end(), -5.0f);
+    tdm_work *wf, *wg;
+    const auto began = std::chrono::steady_clock::now();
+    fake_enqueue(caller, [] { std::this_thread::sleep_for(std::chrono::microseconds(400)); });
+    REQUIRE(tdm_fence(e, caller, &wf) == TDM_OK);
+    REQUIRE(tdm_work_wait_stream(wf, caller) == TDM_OK);
+    REQUIRE(tdm_unit_gather_direct(e, full.data(), n, TDM_F32, t + lo, sizes.data(), world, shard_offs.data(), world, caller, &wg) == TDM_OK);
+    REQUIRE(tdm_work_wait(wg, caller) == TDM_OK && tdm_work_free(wg) == TDM_OK);
+    REQUIRE(tdm_work_wait(wf, caller) == TDM_OK && tdm_work_free(wf) == TDM_OK);
+    REQUIRE(hipStreamSynchronize(caller) == hipSuccess);
+    for (int64_t i = 0; i < n; ++i) REQUIRE(full[i] == t[i]);
+    // (the stand-in's parked stream gives up after twenty seconds, so the cycle would show as a stall, not as a hang)
+    REQUIRE(std::chrono::steady_clock::now() - began < std::chrono::seconds(5));
+    REQUIRE(tdm_fence(e, nullptr, &w) == TDM_OK && tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
+  }
+
   // ZeRO-2's step as one launch per rank: gradients and parameters in the second arena, every rank updates its own shard
   // and writes it into every rank's parameters (the stand-in's "step" is parameter - averaged gradient)
   {

@@ -797,9 +797,10 @@ def disagree(g, what):
 
 
 @pytest.mark.parametrize("what", ["size", "kind"])
-def test_ranks_that_disagree_are_found_out(what):
+def test_ranks_that_disagree_are_found_out(what, monkeypatch):
     from tandem_amd import launch
 
+    monkeypatch.delenv("TANDEM_HIP_WAIT", raising=False)  # with waits that only park the stream the NEXT call reports it (tested below)
     assert launch(disagree, 2, what, gpus=[0, 0], timeout=TIMEOUT) == [True, True]
 
 
