@@ -197,6 +197,7 @@ class Engine {
   bool use_events_;
   hipStream_t stream_ = nullptr;
   hipStream_t gather_stream_ = nullptr;  // direct unit gathers, launched by the caller's thread
+  uint64_t put_tag_ = 0, take_tag_ = 0;  // progress thread only: piece_tag() of the slot-ring collective that is running
   hipEvent_t gather_mark_ = nullptr;     // progress thread only: where gather_stream_ stood when the job it runs was submitted
   hipStream_t anchor_stream_ = nullptr;  // carries nothing but the timing anchors: always idle
   std::mutex anchor_mu_, arena_mu_;      // both threads time their work and map peers' arenas

@@ -603,19 +603,21 @@ void Engine::put(int dst, const char* src, int64_t numel, int dtype, int scale_w
   sent_[dst] = k + 1;
   if (use_events_) {
     check_hip(hipEventRecord(full_[dst][j], stream_), "hipEventRecord (full)");
-    signal(dst, nbytes);
+    signal(dst, nbytes | put_tag_);
   } else {
-    complete_later(false, dst, nbytes, true);  // published once the copy has landed
+    complete_later(false, dst, nbytes | put_tag_, true);  // published once the copy has landed
   }
 }
 
 void Engine::take(int src, char* into, int64_t numel, int dtype, bool reduce, int scale_world) {
   const size_t nbytes = static_cast<size_t>(numel) * elem_bytes(dtype);
-  const uint64_t length = await(src);
-  if (length != nbytes) {
-    throw std::runtime_error((length & kNoPiece) ? "collectives out of step: expected a piece, got a barrier"
-                                                    : "a piece arrived with the wrong length");
+  const uint64_t message = await(src);
+  if (message & kNoPiece) throw std::runtime_error("collectives out of step: expected a piece, got a barrier");
+  if ((message & ~kPieceLengthMask) != take_tag_) {
+    throw std::runtime_error("collectives out of step: rank " + std::to_string(src) + " is in another collective, or in the same "
+                             "one with a tensor of another size or type");
   }
+  if ((message & kPieceLengthMask) != nbytes) throw std::runtime_error("a piece arrived with the wrong length");
   const int j = static_cast<int>(got_[src] % slots_);
   if (use_events_) check_hip(hipStreamWaitEvent(stream_, peer_full_[src][j], 0), "hipStreamWaitEvent (full)");
   const char* slot = static_cast<const char*>(peer_mem_[src]) + static_cast<size_t>(j) * slot_bytes_;
@@ -957,6 +959,7 @@ std::shared_ptr<Work> Engine::all_reduce(Buf t, bool average, hipStream_t caller
       return;
     }
     auto c = chunks(t, {});
+    put_tag_ = take_tag_ = piece_tag(1, t.dtype, t.numel);
     ring_reduce_scatter(c, t.dtype, average, false);
     ring_all_gather(c, t.dtype);
   }, caller, true, ready_on_host_);
@@ -970,8 +973,12 @@ std::shared_ptr<Work> Engine::reduce_scatter(Buf t, std::vector<int64_t> sizes, 
   return submit([this, t, sizes, average, owner_only] {
     if (size_ == 1) return;
     const auto cs = chunks(t, sizes);
-    if (staged_ && size_ <= TDM_MAX_WORLD) staged_reduce_scatter(t, cs, average, !owner_only);
-    else ring_reduce_scatter(cs, t.dtype, average, true);
+    if (staged_ && size_ <= TDM_MAX_WORLD) {
+      staged_reduce_scatter(t, cs, average, !owner_only);
+    } else {
+      put_tag_ = take_tag_ = piece_tag(2, t.dtype, t.numel);
+      ring_reduce_scatter(cs, t.dtype, average, true);
+    }
   }, caller, true, ready_on_host_);
 }
 
@@ -981,8 +988,12 @@ std::shared_ptr<Work> Engine::all_gather(Buf t, std::vector<int64_t> sizes, hipS
   return submit([this, t, sizes] {
     if (size_ == 1) return;
     const auto cs = chunks(t, sizes);
-    if (staged_ && size_ < TDM_MAX_PAIRS) staged_all_gather(t, cs, cs[rank_].ptr);
-    else ring_all_gather(cs, t.dtype);
+    if (staged_ && size_ < TDM_MAX_PAIRS) {
+      staged_all_gather(t, cs, cs[rank_].ptr);
+    } else {
+      put_tag_ = take_tag_ = piece_tag(3, t.dtype, t.numel);
+      ring_all_gather(cs, t.dtype);
+    }
   }, caller, true, ready_on_host_);
 }
 
@@ -1013,6 +1024,7 @@ std::shared_ptr<Work> Engine::unit_gather(Buf full, const char* shard, std::vect
         copy_step(&pr, 1, full.dtype, 0, stream_);
       }
     }
+    put_tag_ = take_tag_ = piece_tag(4, full.dtype, full.numel);
     if (size_ > 1) ring_all_gather(cs, full.dtype);
   }, caller, true, ready_on_host_);
 }
@@ -1027,6 +1039,7 @@ std::shared_ptr<Work> Engine::broadcast(Buf t, int root, hipStream_t caller) {
     const int nxt = mod(rank_ + 1, n), prv = mod(rank_ - 1, n);
     const int64_t pe = piece_elems(t.dtype);
     const int es = elem_bytes(t.dtype);
+    put_tag_ = take_tag_ = piece_tag(5, t.dtype, t.numel ^ (static_cast<int64_t>(root) << 40));
     for (int64_t k = 0; k * pe < t.numel; ++k) {
       char* piece = t.ptr + k * pe * es;
       const int64_t m = std::min(pe, t.numel - k * pe);
@@ -1045,6 +1058,8 @@ std::shared_ptr<Work> Engine::sendrecv(Buf send, int dst, Buf recv, int src, hip
   if (has_send && has_recv && send.dtype != recv.dtype) throw Invalid("sendrecv: the two tensors differ in dtype");
   return submit([this, send, dst, recv, src, has_send, has_recv] {
     Chunk s{send.ptr, send.numel}, r{recv.ptr, recv.numel};
+    if (has_send) put_tag_ = piece_tag(6, send.dtype, send.numel);  // what the receiver on the other side is told to expect
+    if (has_recv) take_tag_ = piece_tag(6, recv.dtype, recv.numel);
     exchange(has_send ? &s : nullptr, dst, has_recv ? &r : nullptr, src, has_send ? send.dtype : recv.dtype, false, 0, 0);
   }, caller, true, ready_on_host_);
 }

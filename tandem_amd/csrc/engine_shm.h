@@ -37,6 +37,16 @@ constexpr uint64_t kNoPiece = uint64_t(1) << 63;
 constexpr uint64_t fence_tag(int kind, int dtype, int64_t numel) {
   return (static_cast<uint64_t>(kind) << 56) | (static_cast<uint64_t>(dtype) << 48) | (static_cast<uint64_t>(numel) & ((uint64_t(1) << 48) - 1));
 }
+// A piece's message carries, above its length (bits 0-39), what the sender is doing: the kind of collective, the element type
+// and the tensor's length folded to 15 bits (bits 40-62). The reference's protocol has nothing of the kind: a rank that is
+// in another collective, or in the same one with a tensor of another size, reads the pieces as if they were its own.
+constexpr int kPieceTagShift = 40;
+constexpr uint64_t kPieceLengthMask = (uint64_t(1) << kPieceTagShift) - 1;
+constexpr uint64_t piece_tag(int kind, int dtype, int64_t numel) {
+  const uint64_t n = static_cast<uint64_t>(numel);
+  return ((static_cast<uint64_t>(kind & 15) << 19) | (static_cast<uint64_t>(dtype & 15) << 15) | ((n ^ (n >> 15) ^ (n >> 30) ^ (n >> 45)) & 0x7fff))
+         << kPieceTagShift;
+}
 
 inline bool is_integer(int dtype) {
   return dtype == TDM_I64 || dtype == TDM_I32 || dtype == TDM_I16 || dtype == TDM_I8 || dtype == TDM_U8;

@@ -796,11 +796,15 @@ def disagree(g, what):
     return False
 
 
+@pytest.mark.parametrize("algo", ["staged", "ring"])
 @pytest.mark.parametrize("what", ["size", "kind"])
-def test_ranks_that_disagree_are_found_out(what, monkeypatch):
+def test_ranks_that_disagree_are_found_out(what, algo, monkeypatch):
+    """Staged: the fence's tag. Slot ring: every piece's message says what its sender is doing (the reference's
+    protocol says nothing: there the all_gather of one rank takes the other's reduce-scatter pieces for its own)."""
     from tandem_amd import launch
 
     monkeypatch.delenv("TANDEM_HIP_WAIT", raising=False)  # with waits that only park the stream the NEXT call reports it (tested below)
+    monkeypatch.setenv("TANDEM_HIP_ALGO", algo)
     assert launch(disagree, 2, what, gpus=[0, 0], timeout=TIMEOUT) == [True, True]
 
 
