@@ -94,6 +94,7 @@ struct Work {
   // Stream-ordered waiting (tdm_work_wait_stream; TANDEM_HIP_WAIT=stream): the word the caller's stream waits for.
   std::shared_ptr<FlagPool> flags;
   bool defer_default = false;  // tdm_work_wait parks too
+  bool may_park = true;        // false: tdm_work_wait_stream waits on the host as well (a process with one hardware queue)
   int flag = -1;
   uint32_t flag_value = 0;  // the word reaches this value when the collective is over
 
@@ -224,6 +225,7 @@ class Engine {
   std::shared_ptr<FlagPool> flags_;      // the words that tdm_work_wait_stream parks streams on
   bool want_flags_ = false;              // the device can make a stream wait for a value
   bool defer_default_ = false;           // TANDEM_HIP_WAIT=stream: tdm_work_wait parks as well
+  bool may_park_ = true;                 // false with GPU_MAX_HW_QUEUES=1: no stream is parked on a collective that has not run
   std::string sticky_error_;             // under mu_: a collective failed after its wait() had already returned
   bool ready_on_host_ = true;        // TANDEM_HIP_READY=gpu: wait for the caller's stream on the GPU instead
   // bytes per half (TANDEM_HIP_STAGING_BYTES). Two ranks, all_reduce of 256 MiB / 1 GiB: 0.52 / 1.93 ms with 64 MiB halves,

@@ -81,6 +81,13 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
         throw Invalid("TANDEM_HIP_WAIT must be \"host\" or \"stream\"");
       }
     }
+    // Parking a stream on a collective that has not run yet queues the wait BEFORE the write that ends it. The two must
+    // not share a hardware queue: the runtime's wait is a kernel that spins at the head of its queue, and a write queued
+    // behind it never runs. A process told to use a single hardware queue (GPU_MAX_HW_QUEUES=1) has nowhere else to put
+    // the engine's stream: there every wait is taken on the host, whatever was asked for.
+    if (const char* hq = std::getenv("GPU_MAX_HW_QUEUES")) {
+      if (std::atoi(hq) == 1) may_park_ = false;
+    }
   }
   if (const char* gm = std::getenv("TANDEM_HIP_GATHER")) {
     // "stream": on the engine's side stream; it starts behind an event of the caller's stream (from a ring of events)
@@ -272,7 +279,8 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
   if (flags_ && uses_gpu) {
     work->flag = flags_->acquire(&work->flag_value);
     if (work->flag >= 0) work->flags = flags_;
-    work->defer_default = defer_default_;
+    work->defer_default = defer_default_ && may_park_;
+    work->may_park = may_park_;
   }
   hipEvent_t ready = nullptr;
   if (uses_gpu) {

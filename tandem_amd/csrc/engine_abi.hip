@@ -244,7 +244,7 @@ static int wait_for(tdm_work* w, tdm_stream caller, bool may_park) {
     return TDM_EINVAL;
   }
   Work& work = *w->impl;
-  if (may_park && work.flag >= 0 && !work.finished_hint.load(std::memory_order_acquire)) {
+  if (may_park && work.may_park && work.flag >= 0 && !work.finished_hint.load(std::memory_order_acquire)) {
     // The job has not run yet: park the caller's stream on its word and return. The host
     // goes on queueing work behind the collective; a failure shows at the next call.
     return guard([&] {

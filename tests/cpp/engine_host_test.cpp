@@ -251,6 +251,23 @@ static int run_rank(int rank, int world, const std::string& job, std::atomic<int
     REQUIRE(tdm_fence(e, nullptr, &w) == TDM_OK && tdm_work_wait(w, nullptr) == TDM_OK && tdm_work_free(w) == TDM_OK);
   }
 
+  // A process with a single hardware queue (GPU_MAX_HW_QUEUES=1): no stream is parked on a collective that has not run,
+  // tdm_work_wait_stream waits on the host like tdm_work_wait. Parked (any other setting), it returns at once: the
+  // collective cannot start before the slow producer on the caller's stream has finished.
+  {
+    const char* hq = std::getenv("GPU_MAX_HW_QUEUES");
+    const bool single = hq && std::atoi(hq) == 1;
+    std::vector<float> x(1000, static_cast<float>(rank + 1));
+    const auto began = std::chrono::steady_clock::now();
+    fake_enqueue(caller, [] { std::this_thread::sleep_for(std::chrono::milliseconds(40)); });
+    REQUIRE(tdm_all_reduce(e, x.data(), 1000, TDM_F32, 0, caller, &w) == TDM_OK);
+    REQUIRE(tdm_work_wait_stream(w, caller) == TDM_OK);
+    const auto took = std::chrono::steady_clock::now() - began;
+    REQUIRE(single ? took >= std::chrono::milliseconds(35) : took < std::chrono::milliseconds(25));
+    REQUIRE(hipStreamSynchronize(caller) == hipSuccess && tdm_work_free(w) == TDM_OK);
+    REQUIRE(x[0] == static_cast<float>(world * (world + 1) / 2));
+  }
+
   // ZeRO-2's step as one launch per rank: gradients and parameters in the second arena, every rank updates its own shard
   // and writes it into every rank's parameters (the stand-in's "step" is parameter - averaged gradient)
   {

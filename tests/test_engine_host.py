@@ -26,6 +26,8 @@ CASES = [("2", "staged"), ("3", "staged"), ("4", "staged"), ("5", "staged"), ("8
          # GPU instead of by polling, every wait parking the stream instead of blocking the host
          ("3", "staged", "0", "-", "TANDEM_HIP_GATHER=stream,TANDEM_HIP_READY=gpu,TANDEM_HIP_WAIT=stream"),
          ("2", "ring", "0", "-", "TANDEM_HIP_READY=gpu,TANDEM_HIP_WAIT=stream"),
+         # a single hardware queue: parked waits are taken on the host instead
+         ("3", "staged", "0", "-", "GPU_MAX_HW_QUEUES=1,TANDEM_HIP_WAIT=stream,TANDEM_HIP_GATHER=stream"),
          ("3", "staged", "0", "-", "TANDEM_HIP_GATHER=stream-events"), ("2", "staged", "0", "-", "TANDEM_HIP_GATHER=stream,FAKE_HIP_JITTER_US=200"),
          ("3", "staged", "0", "-", "TANDEM_HIP_GATHER=stream-words,FAKE_HIP_JITTER_US=200"),
          # streams that lag behind the host by varying amounts (every piece of work on a stream starts up to 200 us late),
