@@ -499,11 +499,11 @@ def zero2_steps_typed(g, name, ns, steps):
 
 
 @pytest.mark.parametrize("name", ["bf16", "f16", "f64"])
-@pytest.mark.parametrize("world", [2, 3])
+@pytest.mark.parametrize("world", [2, 3, 4])
 def test_zero2_step_in_one_launch_per_rank_on_other_shard_types(world, name):
     """The same fused step between process ranks over bfloat16, float16 and float64 buffers
     (tdm_direct_zero2_step_typed): the ring's fold in the type's own rounding, 0 + mine, the typed AdamW,
-    the new parameters in every rank's buffer; bit for bit with the oracle, state included."""
+    the new parameters in every rank's buffer; bit for bit with the oracle, state included, at worlds 2 to 4."""
     from oracle import ring
     from oracle.adamw import AdamW
     from tandem_amd import launch
