@@ -510,8 +510,8 @@ int tdm_work_wait(tdm_work* w, tdm_stream caller);
  * this is tdm_work_wait). The host can then queue work behind a collective that is still in flight; a failure of
  * that collective is returned by the next call on the engine instead of by this one. The wait is queued BEFORE
  * the write that ends it, so `caller` and the engine's stream must not share a hardware queue (the runtime's wait
- * spins at the head of its queue): in a process limited to one (GPU_MAX_HW_QUEUES=1) nothing is parked and this
- * is tdm_work_wait too. No counterpart in the
+ * spins at the head of its queue): in a process limited to fewer than four (GPU_MAX_HW_QUEUES=1..3; HIP's default is 4)
+ * nothing is parked and this is tdm_work_wait too. No counterpart in the
  * reference, whose CUDA engine orders its hand-over on the GPU and so never blocks a waiting host for it. */
 int tdm_work_wait_stream(tdm_work* w, tdm_stream caller);
 int tdm_work_done(tdm_work* w);

@@ -84,9 +84,12 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
     // Parking a stream on a collective that has not run yet queues the wait BEFORE the write that ends it. The two must
     // not share a hardware queue: the runtime's wait is a kernel that spins at the head of its queue, and a write queued
     // behind it never runs. A process told to use a single hardware queue (GPU_MAX_HW_QUEUES=1) has nowhere else to put
-    // the engine's stream: there every wait is taken on the host, whatever was asked for.
+    // the engine's stream (seen: every parked wait timed out), and with fewer queues than the four streams such a
+    // process has at least (the caller's, and the engine's three) two of them share one: there every wait is taken on
+    // the host, whatever was asked for. HIP's default is four.
     if (const char* hq = std::getenv("GPU_MAX_HW_QUEUES")) {
-      if (std::atoi(hq) == 1) may_park_ = false;
+      const int queues = std::atoi(hq);
+      if (queues >= 1 && queues < 4) may_park_ = false;
     }
   }
   if (const char* gm = std::getenv("TANDEM_HIP_GATHER")) {
