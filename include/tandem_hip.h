@@ -508,7 +508,9 @@ int tdm_work_wait(tdm_work* w, tdm_stream caller);
  * the word the engine sets behind the collective's last kernel and the call returns at once, whatever
  * TANDEM_HIP_WAIT says (where the device cannot park a stream on a value, and when the collective has already run,
  * this is tdm_work_wait). The host can then queue work behind a collective that is still in flight; a failure of
- * that collective is returned by the next call on the engine instead of by this one. The wait is queued BEFORE
+ * that collective is returned by the next call on the engine instead of by this one. The wait is a kernel of the
+ * library's own with a time limit (the engine's time limit and ten seconds, or TANDEM_HIP_PARK_LIMIT_S): a stream
+ * that gives up goes on, and the next call on the engine fails and says so. The wait is queued BEFORE
  * the write that ends it, so `caller` and the engine's stream must not share a hardware queue (the runtime's wait
  * spins at the head of its queue): in a process limited to fewer than four (GPU_MAX_HW_QUEUES=1..3; HIP's default is 4)
  * nothing is parked and this is tdm_work_wait too. No counterpart in the

@@ -95,6 +95,7 @@ void gather_multicast(char* const* base, const int64_t* lo, const int64_t* len, 
 void unit_gather_multicast(char* const* fulls, const char* const* shards, const int64_t* sizes, int world, int es, bool cold,
                            unsigned occupancy_pad, int xcd_shift, int vectors_per_lane, int max_grid, hipStream_t stream);
 void zero2_step_segment(const tdm_step_seg& seg, int world, bool average, const tdm_adamw_scalars& s, int order, hipStream_t stream);
+void park_stream(hipStream_t stream, const uint32_t* word, uint32_t value, double limit_s, uint32_t* gave_up);
 void zero2_step_segment_typed(const tdm_step_seg& seg, int world, bool average, const tdm_adamw_hyper& h, int order, hipStream_t stream);
 
 }  // namespace tandem_hip

@@ -31,8 +31,8 @@ struct FlagPool {
 
   static std::shared_ptr<FlagPool> make() {
     auto p = std::make_shared<FlagPool>();
-    check_hip(hipHostMalloc(reinterpret_cast<void**>(&p->base), kFlags * sizeof(uint32_t), hipHostMallocDefault), "hipHostMalloc (flags)");
-    std::memset(p->base, 0, kFlags * sizeof(uint32_t));
+    check_hip(hipHostMalloc(reinterpret_cast<void**>(&p->base), (kFlags + 1) * sizeof(uint32_t), hipHostMallocDefault), "hipHostMalloc (flags)");
+    std::memset(p->base, 0, (kFlags + 1) * sizeof(uint32_t));
     p->generation.assign(kFlags, 0);
     for (int i = kFlags - 1; i >= 0; --i) p->free_list.push_back(i);
     return p;
@@ -70,6 +70,9 @@ struct FlagPool {
     return __atomic_load_n(base + i, __ATOMIC_ACQUIRE) >= value;
   }
   void set(int i, uint32_t value) { __atomic_store_n(base + i, value, __ATOMIC_SEQ_CST); }
+  // One more word behind the pool: a parked stream that gave up waiting (park_kernel) leaves 1 there.
+  uint32_t* gave_up_word() const { return base + kFlags; }
+  bool gave_up() const { return __atomic_load_n(base + kFlags, __ATOMIC_ACQUIRE) != 0; }
 };
 
 struct Work {
@@ -95,6 +98,7 @@ struct Work {
   std::shared_ptr<FlagPool> flags;
   bool defer_default = false;  // tdm_work_wait parks too
   bool may_park = true;        // false: tdm_work_wait_stream waits on the host as well (a process with one hardware queue)
+  double park_limit_s = 0;     // how long a stream parked on this Work waits at most before it gives up
   int flag = -1;
   uint32_t flag_value = 0;  // the word reaches this value when the collective is over
 
@@ -225,6 +229,7 @@ class Engine {
   std::shared_ptr<FlagPool> flags_;      // the words that tdm_work_wait_stream parks streams on
   bool want_flags_ = false;              // the device can make a stream wait for a value
   bool defer_default_ = false;           // TANDEM_HIP_WAIT=stream: tdm_work_wait parks as well
+  double park_limit_s_ = 0;              // the engine's time limit and a margin, or TANDEM_HIP_PARK_LIMIT_S
   bool may_park_ = true;                 // false with GPU_MAX_HW_QUEUES=1: no stream is parked on a collective that has not run
   std::string sticky_error_;             // under mu_: a collective failed after its wait() had already returned
   bool ready_on_host_ = true;        // TANDEM_HIP_READY=gpu: wait for the caller's stream on the GPU instead

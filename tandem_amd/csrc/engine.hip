@@ -91,6 +91,14 @@ Engine::Engine(const std::string& job, int rank, int size, int slots, size_t slo
       const int queues = std::atoi(hq);
       if (queues >= 1 && queues < 4) may_park_ = false;
     }
+    // A parked stream gives up by itself after the engine's own time limit and a margin (by then the host has declared
+    // the collective failed and set the word, unless the write cannot get past the wait): no wait on the GPU is without end.
+    park_limit_s_ = timeout_s_ + 10.0;
+    if (const char* pl = std::getenv("TANDEM_HIP_PARK_LIMIT_S")) {
+      const double v = std::atof(pl);
+      if (!(v > 0)) throw Invalid("TANDEM_HIP_PARK_LIMIT_S must be a positive number of seconds");
+      park_limit_s_ = v;
+    }
   }
   if (const char* gm = std::getenv("TANDEM_HIP_GATHER")) {
     // "stream": on the engine's side stream; it starts behind an event of the caller's stream (from a ring of events)
@@ -284,6 +292,7 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
     if (work->flag >= 0) work->flags = flags_;
     work->defer_default = defer_default_ && may_park_;
     work->may_park = may_park_;
+    work->park_limit_s = park_limit_s_;
   }
   hipEvent_t ready = nullptr;
   if (uses_gpu) {
@@ -343,6 +352,9 @@ std::shared_ptr<Work> Engine::submit(std::function<void()> job, hipStream_t call
   }
   {
     std::lock_guard<std::mutex> lock(mu_);
+    if (sticky_error_.empty() && flags_ && flags_->gave_up()) {
+      sticky_error_ = "a stream parked on a collective gave up waiting for its end (do the waiting stream and the engine's share a hardware queue?)";
+    }
     if (stopping_ || !sticky_error_.empty()) {
       if (ready) (void)hipEventDestroy(ready);  // the job that would have released it never runs
       if (mark) (void)hipEventDestroy(mark);

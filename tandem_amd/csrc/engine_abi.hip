@@ -244,13 +244,18 @@ static int wait_for(tdm_work* w, tdm_stream caller, bool may_park) {
     return TDM_EINVAL;
   }
   Work& work = *w->impl;
+  if (work.flags && work.flags->gave_up()) {
+    set_last_error("a stream parked on a collective gave up waiting for its end: what that stream computed since is not to be trusted");
+    return TDM_ERUNTIME;
+  }
   if (may_park && work.may_park && work.flag >= 0 && !work.finished_hint.load(std::memory_order_acquire)) {
     // The job has not run yet: park the caller's stream on its word and return. The host
     // goes on queueing work behind the collective; a failure shows at the next call.
+    // The wait is a kernel of the library's own with a time limit: it is queued before the write that ends it, and
+    // should that write never run the stream goes on by itself and the next call on the engine says so.
     return guard([&] {
-      check_hip(hipStreamWaitValue32(static_cast<hipStream_t>(caller), work.flags->base + work.flag, work.flag_value,
-                                     hipStreamWaitValueGte, 0xffffffffu),
-                "hipStreamWaitValue32 (wait)");
+      park_stream(static_cast<hipStream_t>(caller), work.flags->base + work.flag, work.flag_value, work.park_limit_s,
+                  work.flags->gave_up_word());
     });
   }
   spin_for([&] { return work.finished_hint.load(std::memory_order_acquire); });

@@ -456,6 +456,18 @@ void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const t
   check_hip(hipGetLastError(), "k23_zero2_step_one launch");
 }
 
+// Used by the engine: `stream` waits until *word >= value, for at most limit_s seconds (then *gave_up becomes 1).
+void park_stream(hipStream_t stream, const uint32_t* word, uint32_t value, double limit_s, uint32_t* gave_up) {
+  if (word == nullptr || gave_up == nullptr) throw Invalid("park_stream: NULL word");
+  int device = 0, khz = 0;
+  check_hip(hipGetDevice(&device), "hipGetDevice");
+  check_hip(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, device), "hipDeviceGetAttribute (wall clock rate)");
+  if (khz <= 0) throw std::runtime_error("the device reports no wall clock rate");
+  const double ticks = std::min(std::max(limit_s, 0.0), 86400.0) * 1e3 * khz;
+  hipLaunchKernelGGL(park_kernel, dim3(1), dim3(1), 0, stream, word, value, static_cast<long long>(ticks), gave_up);
+  check_hip(hipGetLastError(), "park_kernel launch");
+}
+
 // Used by the engine too.
 void reduce_step(const tdm_pair* pairs, int npairs, int dtype, int world, bool scale_dst, bool scale_src,
                  bool writeback_src, hipStream_t stream, int policy) {

@@ -72,6 +72,36 @@ static int run_broken(tdm_engine* e, int rank, int world, const std::string& sce
   return 0;
 }
 
+// A stream parked on a collective whose end does not come in time gives up by itself (TANDEM_HIP_PARK_LIMIT_S, here a
+// twentieth of a second; the peers come 300 ms late), and the next call on the engine says so. The collective itself
+// still runs when the peers arrive: they are not to be left waiting for this rank.
+static int run_park_gives_up(tdm_engine* e, int rank, int world) {
+  hipStream_t caller = nullptr;
+  REQUIRE(hipStreamCreateWithFlags(&caller, hipStreamNonBlocking) == hipSuccess);
+  std::vector<float> x(1000, static_cast<float>(rank + 1));
+  tdm_work* w = nullptr;
+  if (rank != 0) std::this_thread::sleep_for(std::chrono::milliseconds(300));
+  REQUIRE(tdm_all_reduce(e, x.data(), 1000, TDM_F32, 0, caller, &w) == TDM_OK);
+  if (rank == 0) {
+    const auto began = std::chrono::steady_clock::now();
+    REQUIRE(tdm_work_wait_stream(w, caller) == TDM_OK);  // parked: the collective cannot have run
+    REQUIRE(hipStreamSynchronize(caller) == hipSuccess);
+    const auto took = std::chrono::steady_clock::now() - began;
+    REQUIRE(took >= std::chrono::milliseconds(40) && took < std::chrono::milliseconds(250));  // let go by its own limit, not by the peers
+    tdm_work* again = nullptr;
+    REQUIRE(tdm_all_reduce(e, x.data(), 1000, TDM_F32, 0, caller, &again) != TDM_OK);
+    REQUIRE(std::string(tdm_last_error()).find("gave up") != std::string::npos);
+    REQUIRE(tdm_work_wait(w, caller) != TDM_OK && std::string(tdm_last_error()).find("gave up") != std::string::npos);
+  } else {
+    REQUIRE(tdm_work_wait(w, caller) == TDM_OK && hipStreamSynchronize(caller) == hipSuccess);
+    REQUIRE(x[0] == static_cast<float>(world * (world + 1) / 2));
+  }
+  REQUIRE(tdm_work_free(w) == TDM_OK);
+  (void)tdm_engine_close(e);
+  REQUIRE(tdm_engine_destroy(e) == TDM_OK);
+  return 0;
+}
+
 static int run_rank(int rank, int world, const std::string& job, std::atomic<int>* arrived, const std::string& scenario) {
   g_rank = rank;
   tdm_engine* e = nullptr;
@@ -89,6 +119,7 @@ static int run_rank(int rank, int world, const std::string& job, std::atomic<int
   arrived->fetch_add(1);  // the launcher's barrier: every rank has published its region
   while (arrived->load() < world) std::this_thread::yield();
   REQUIRE(tdm_engine_connect(e) == TDM_OK);
+  if (scenario == "park_gives_up") return run_park_gives_up(e, rank, world);
   if (!scenario.empty()) return run_broken(e, rank, world, scenario);
 
   hipStream_t caller = nullptr;

@@ -3,8 +3,10 @@
 // int64; the sums are formed in the order the kernels form them, which for the integer-valued numbers the test
 // sends does not matter. Like a launch, each returns at once: the loop runs when the stream gets to it.
 
+#include <chrono>
 #include <cstring>
 #include <string>
+#include <thread>
 
 #include <vector>
 
@@ -105,6 +107,20 @@ void fold_step(const tdm_fold_seg* segs, int nseg, int world, int dtype, bool av
 // The data flow of ZeRO-2's step, not its arithmetic: the shard's gradients folded in the ring's order and averaged, the
 // moments bumped, and "parameter - gradient" written into every rank's parameter buffer. (AdamW itself is the kernels'
 // and the GPU tests' business.)
+// A stream parked on a word, as park_kernel parks it: until the word has reached the value, or the time is up.
+void park_stream(hipStream_t stream, const uint32_t* word, uint32_t value, double limit_s, uint32_t* gave_up) {
+  fake_enqueue(stream, [=] {
+    const auto until = std::chrono::steady_clock::now() + std::chrono::duration<double>(limit_s);
+    while (__atomic_load_n(word, __ATOMIC_ACQUIRE) < value) {
+      if (std::chrono::steady_clock::now() > until) {
+        __atomic_store_n(gave_up, 1u, __ATOMIC_RELEASE);
+        return;
+      }
+      std::this_thread::yield();
+    }
+  });
+}
+
 namespace {
 template <typename T>
 void step_data_flow(const tdm_step_seg& sg, int world, bool average, hipStream_t stream) {

@@ -40,6 +40,8 @@ CASES = [("2", "staged"), ("3", "staged"), ("4", "staged"), ("5", "staged"), ("8
          ("4", "ring", "0", "-", "TANDEM_HIP_SYNC=event,FAKE_HIP_IPC_EVENTS=1,FAKE_HIP_JITTER_US=200"),
          # the group falls apart: a rank that leaves without a word, ranks that bring tensors of different lengths
          ("3", "staged", "0", "dies"), ("3", "ring", "0", "dies"), ("3", "staged", "0", "out_of_step"), ("2", "ring", "0", "out_of_step"),
+         # a parked stream whose collective does not end in time lets itself go, and the engine says so
+         ("2", "staged", "0", "park_gives_up", "TANDEM_HIP_PARK_LIMIT_S=0.05"), ("3", "ring", "0", "park_gives_up", "TANDEM_HIP_PARK_LIMIT_S=0.05"),
          # an engine that cannot start (no interprocess events for TANDEM_HIP_SYNC=event; bad arguments) leaves nothing behind
          ("2", "staged", "0", "no_ipc_events")]
 VARIANTS = {"plain": ["-O2"],

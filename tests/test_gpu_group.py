@@ -839,6 +839,43 @@ def test_stream_ordered_wait_reports_a_failure_at_the_next_call(monkeypatch):
     assert launch(late_failure, 2, gpus=[0, 0], timeout=2.0) == [True, True]
 
 
+def parked_too_long(g):
+    """A stream parked on a collective whose end does not come within the park limit lets itself go (the wait is a
+    kernel of the library's own with a time limit), and the next call on the group says so. The collective itself still
+    runs when the late peer arrives, which must not be left waiting for this rank."""
+    import time
+
+    from tandem_amd import CommError
+
+    x = torch.full((1000,), float(g.rank + 1), device=g.device)
+    if g.rank == 1:
+        time.sleep(1.5)
+        g.all_reduce(x)
+        torch.cuda.synchronize()
+        ok = float(x[0]) == 3.0
+        g.abandon()
+        return ok
+    t0 = time.perf_counter()
+    g.all_reduce(x, async_op=True).wait(stream_ordered=True)  # returns at once: the peer has not even called yet
+    torch.cuda.synchronize()  # ... and the stream is let go by its own limit, long before the peer comes
+    took = time.perf_counter() - t0
+    try:
+        g.all_reduce(x)
+    except CommError as e:
+        time.sleep(2.0)  # the first collective still runs when the peer arrives
+        g.abandon()
+        return 0.15 < took < 1.2 and "gave up" in str(e)
+    return False
+
+
+def test_a_parked_stream_gives_up_by_itself(monkeypatch):
+    from tandem_amd import launch
+
+    monkeypatch.setenv("TANDEM_HIP_PARK_LIMIT_S", "0.2")
+    monkeypatch.delenv("GPU_MAX_HW_QUEUES", raising=False)
+    assert launch(parked_too_long, 2, gpus=[0, 0], timeout=5.0) == [True, True]
+
+
 def test_unknown_backend_and_cpu_device_are_refused():
     from tandem_amd import CommError, Group, launch
 
