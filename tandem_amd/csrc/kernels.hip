@@ -456,6 +456,24 @@ void zero2_step_segment(const tdm_step_seg& sg, int world, bool average, const t
   check_hip(hipGetLastError(), "k23_zero2_step_one launch");
 }
 
+namespace {
+// A stream parked on a word until a collective that has not run yet has ended: one lane polls the word (pinned host
+// memory, written by the engine's stream or, after a failure, by the host) until it has reached `value`, and gives up
+// after `limit_ticks` of the device's wall clock, leaving 1 in *gave_up for the host to find: whatever goes wrong with
+// the write that should end the wait, the kernel ends.
+__global__ void park_kernel(const uint32_t* word, uint32_t value, long long limit_ticks, uint32_t* gave_up) {
+  const long long began = wall_clock64();
+  for (;;) {
+    if (__hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM) >= value) return;
+    if (wall_clock64() - began > limit_ticks) {
+      __hip_atomic_store(gave_up, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+      return;
+    }
+    __builtin_amdgcn_s_sleep(16);
+  }
+}
+}  // namespace
+
 // Used by the engine: `stream` waits until *word >= value, for at most limit_s seconds (then *gave_up becomes 1).
 void park_stream(hipStream_t stream, const uint32_t* word, uint32_t value, double limit_s, uint32_t* gave_up) {
   if (word == nullptr || gave_up == nullptr) throw Invalid("park_stream: NULL word");
