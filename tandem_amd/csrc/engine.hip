@@ -1062,7 +1062,8 @@ std::shared_ptr<Work> Engine::broadcast(Buf t, int root, hipStream_t caller) {
     const int nxt = mod(rank_ + 1, n), prv = mod(rank_ - 1, n);
     const int64_t pe = piece_elems(t.dtype);
     const int es = elem_bytes(t.dtype);
-    put_tag_ = take_tag_ = piece_tag(5, t.dtype, t.numel ^ (static_cast<int64_t>(root) << 40));
+    // copies carry bytes: their tags say how many, not of what type (the reference copies a float32 tensor into a uint8 one)
+    put_tag_ = take_tag_ = piece_tag(5, 0, (t.numel * es) ^ (static_cast<int64_t>(root) << 40));
     for (int64_t k = 0; k * pe < t.numel; ++k) {
       char* piece = t.ptr + k * pe * es;
       const int64_t m = std::min(pe, t.numel - k * pe);
@@ -1081,8 +1082,8 @@ std::shared_ptr<Work> Engine::sendrecv(Buf send, int dst, Buf recv, int src, hip
   if (has_send && has_recv && send.dtype != recv.dtype) throw Invalid("sendrecv: the two tensors differ in dtype");
   return submit([this, send, dst, recv, src, has_send, has_recv] {
     Chunk s{send.ptr, send.numel}, r{recv.ptr, recv.numel};
-    if (has_send) put_tag_ = piece_tag(6, send.dtype, send.numel);  // what the receiver on the other side is told to expect
-    if (has_recv) take_tag_ = piece_tag(6, recv.dtype, recv.numel);
+    if (has_send) put_tag_ = piece_tag(6, 0, send.numel * elem_bytes(send.dtype));  // bytes, as for broadcast
+    if (has_recv) take_tag_ = piece_tag(6, 0, recv.numel * elem_bytes(recv.dtype));
     exchange(has_send ? &s : nullptr, dst, has_recv ? &r : nullptr, src, has_send ? send.dtype : recv.dtype, false, 0, 0);
   }, caller, true, ready_on_host_);
 }
