@@ -48,7 +48,10 @@ class Work:
         (tandem/comm.py:92-107 in the reference). stream_ordered=True: a collective that has not run yet is not
         waited for on the host; the stream is parked on it and the call returns at once, so the host can go on
         queueing work (an optimizer's launches, say) behind it. A failure of such a collective is raised by the
-        next call on the group instead of by this one."""
+        next call on the group instead of by this one. The parked stream waits in a kernel with a time limit
+        (the group's timeout and ten seconds; TANDEM_HIP_PARK_LIMIT_S): should the collective's end never reach
+        it, the stream goes on and the next call on the group fails with "gave up". In a process limited to
+        fewer than four hardware queues (GPU_MAX_HW_QUEUES) nothing is parked and this is the plain wait."""
         g = self._group
         if self._handle is None:
             return self.result
