@@ -254,8 +254,17 @@ static int wait_for(tdm_work* w, tdm_stream caller, bool may_park) {
     // The wait is a kernel of the library's own with a time limit: it is queued before the write that ends it, and
     // should that write never run the stream goes on by itself and the next call on the engine says so.
     return guard([&] {
-      park_stream(static_cast<hipStream_t>(caller), work.flags->base + work.flag, work.flag_value, work.park_limit_s,
-                  work.flags->gave_up_word());
+      int current = -1;  // a kernel launch wants the stream's device current; the caller's choice is put back
+      check_hip(hipGetDevice(&current), "hipGetDevice");
+      if (current != work.device) check_hip(hipSetDevice(work.device), "hipSetDevice");
+      try {
+        park_stream(static_cast<hipStream_t>(caller), work.flags->base + work.flag, work.flag_value, work.park_limit_s,
+                    work.flags->gave_up_word());
+      } catch (...) {
+        if (current != work.device) (void)hipSetDevice(current);
+        throw;
+      }
+      if (current != work.device) check_hip(hipSetDevice(current), "hipSetDevice");
     });
   }
   spin_for([&] { return work.finished_hint.load(std::memory_order_acquire); });

@@ -182,6 +182,10 @@ void fake_enqueue(hipStream_t stream, std::function<void()> work) {
 extern "C" {
 
 hipError_t hipSetDevice(int) { return hipSuccess; }
+hipError_t hipGetDevice(int* device) {
+  *device = 0;
+  return hipSuccess;
+}
 hipError_t hipGetLastError(void) { return hipSuccess; }
 const char* hipGetErrorString(hipError_t e) { return e == hipSuccess ? "no error" : "an error of the stand-in runtime"; }
 
