@@ -14,6 +14,12 @@
  *                        torch's single-tensor AdamW on CPU (lerp_ and addcmul_
  *                        fuse their last multiply-add, addcdiv_ does not).
  *
+ * What pins them (tests/test_oracle_ring.py, test_oracle_adamw.py, test_oracle_cpu_engine.py): outputs of the
+ * reference's own engine and optimizer kept as fixtures in tests/golden (ring_w2/3/4.npz and ring_dtypes_w3.npz:
+ * whole buffers, partial sums included; adamw.npz; adamw_dtypes.npz for float64, bfloat16 and float16 shards), a
+ * message-by-message simulator of the ring written independently of the closed form, torch's single-tensor AdamW,
+ * float64 recurrences and all 65,536 half-precision bit patterns. No function here is without such a check.
+ *
  * Built with -ffp-contract=off: every fused multiply-add below is explicit.
  */
 #include <math.h>
