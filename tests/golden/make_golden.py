@@ -3,7 +3,7 @@ implementation (tandem's Python engine, CPU processes) on small seeded inputs.
 
 Run once, in the build container only, where the reference is mounted:
 
-    python tests/golden/make_golden.py [/root/reference] [only: ring adamw adamw_dtypes plans data train]
+    python tests/golden/make_golden.py [/root/reference] [only: ring adamw adamw_dtypes plans data train train_dtypes]
 
 The fixtures are data only (inputs, expected outputs, digests). They pin the
 parts of the path that no test of the reference pins by itself:
@@ -21,6 +21,7 @@ parts of the path that no test of the reference pins by itself:
   data.json           digests of synthetic() and Text.batch().
   train_*.json        losses and weight digests of DDP / ZeRO-1/2/3 training
                       runs (CPU, tiny GPT) at world sizes 2, 3 and 4.
+  train_dtypes.json   the same runs with the model in bfloat16 and in float64, world sizes 2 and 3.
 
 Nothing here is loaded by the library; tests read the fixtures only.
 """
@@ -324,9 +325,50 @@ def write_train():
             json.dump(out, f, indent=0)
 
 
+def train_rank_typed(g, strategy, bucket_bytes, dtype_name):
+    """The same run with the model in another floating type: the reference's wrappers, engine and optimizer take any."""
+    torch.manual_seed(0)
+    text = synthetic(20_000)
+    model = GPT(CFG).to(getattr(torch, dtype_name))
+    losses = []
+    if strategy == "ddp":
+        z = DDP(model, g, bucket_bytes=bucket_bytes)
+        opt = torch.optim.AdamW(model.parameters(), lr=3e-3, weight_decay=0.1, foreach=False)
+    else:
+        sopt = ShardedAdamW(lr=3e-3, weight_decay=0.1)
+        stage = int(strategy[-1])
+        z = ZeRO(model, g, stage, sopt, bucket_bytes) if stage < 3 else FSDP(model, g, sopt)
+    for step in range(4):
+        x, y = text.batch(step, BATCH, CFG.seq, rank=g.rank, world=g.size)
+        loss = z(x, y)
+        loss.backward()
+        losses.append(loss.item())
+        if strategy == "ddp":
+            opt.step()
+            opt.zero_grad()
+        else:
+            z.step()
+            z.zero_grad()
+    w = z.full_parameters() if strategy == "zero3" else torch.cat([p.detach().reshape(-1) for p in model.parameters()])
+    raw = w.view(torch.int16) if w.element_size() == 2 else w
+    return {"losses": losses, "sha256": sha(raw), "first8": w[:8].double().tolist(), "last8": w[-8:].double().tolist()}
+
+
+def write_train_dtypes():
+    out = {"cfg": {"seq": 32, "layers": 2, "heads": 2, "dim": 32}, "steps": 4, "batch": BATCH, "lr": 3e-3, "weight_decay": 0.1,
+           "bucket_bytes": 4 << 10, "torch": torch.__version__}
+    for dtype_name in ("bfloat16", "float64"):
+        out[dtype_name] = {}
+        for world in (2, 3):
+            out[dtype_name][str(world)] = {strategy: launch(train_rank_typed, world, strategy, 4 << 10, dtype_name, slot_bytes=1024)
+                                           for strategy in ("ddp", "zero1", "zero2", "zero3")}
+    with open(os.path.join(HERE, "train_dtypes.json"), "w") as f:
+        json.dump(out, f, indent=0)
+
+
 if __name__ == "__main__":
     writers = {"ring": write_ring, "adamw": write_adamw, "adamw_dtypes": write_adamw_dtypes, "plans": write_plans,
-               "data": write_data, "train": write_train}
+               "data": write_data, "train": write_train, "train_dtypes": write_train_dtypes}
     only = sys.argv[2:] or list(writers)
     for name in only:
         writers[name]()

@@ -42,14 +42,27 @@ class OracleShardedAdamW:
     that used torch's CPU kernels."""
 
     def __init__(self, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, torch_sqrt=True):
+        self.hyper, self.torch_sqrt, self.inner = (lr, betas, eps, weight_decay), torch_sqrt, None
+
+    def _make(self, dtype):
         from oracle.adamw import AdamW
 
-        root = (lambda v: torch.from_numpy(v).sqrt().numpy()) if torch_sqrt else None
-        self.inner = AdamW(lr, betas, eps, weight_decay, sqrt=root)
+        # fp32 and float64: torch's vectorised CPU sqrt is not correctly rounded. bfloat16: its root is rounded to 8 bits
+        # and comes out the same either way (the exact root never lies near a bfloat16 rounding tie).
+        root = (lambda v: torch.from_numpy(v).sqrt().numpy()) if self.torch_sqrt and dtype in (torch.float32, torch.float64) else None
+        kind = {torch.bfloat16: "bf16", torch.float16: "f16"}.get(dtype)
+        return AdamW(*self.hyper, sqrt=root, kind=kind)
+
+    @staticmethod
+    def _array(t):
+        t = t.detach()
+        return t.view(torch.int16).numpy().view(np.uint16) if t.element_size() == 2 else t.numpy()
 
     def update(self, key, param, grad):
-        assert param.device.type == "cpu" and param.is_contiguous() and grad.is_contiguous()
-        self.inner.update(key, param.detach().numpy(), grad.detach().numpy())
+        assert param.device.type == "cpu" and param.is_contiguous() and grad.is_contiguous() and param.dtype == grad.dtype
+        if self.inner is None:
+            self.inner = self._make(param.dtype)
+        self.inner.update(key, self._array(param), self._array(grad))
 
     def state_bytes(self):
         return self.inner.state_bytes()

@@ -85,6 +85,52 @@ def test_reproduces_the_reference_training_runs(world, strategy):
             assert got[r]["state_bytes"] <= 2 * 4 * (got[r]["numel"] // world + 1)
 
 
+def train_rank_typed(g, strategy, bucket_bytes, steps, batch, dtype_name):
+    torch.manual_seed(0)
+    text = synthetic(20_000)
+    model = GPT(CFG).to(getattr(torch, dtype_name))
+    losses = []
+    if strategy == "ddp":
+        z = DDP(model, g, bucket_bytes=bucket_bytes)
+        opt = torch.optim.AdamW(model.parameters(), lr=3e-3, weight_decay=0.1, foreach=False)
+    else:
+        sopt = OracleShardedAdamW(lr=3e-3, weight_decay=0.1)
+        stage = int(strategy[-1])
+        z = ZeRO(model, g, stage, sopt, bucket_bytes) if stage < 3 else FSDP(model, g, sopt)
+    for step in range(steps):
+        x, y = text.batch(step, batch, CFG.seq, rank=g.rank, world=g.size)
+        loss = z(x, y)
+        loss.backward()
+        losses.append(loss.item())
+        if strategy == "ddp":
+            opt.step()
+            opt.zero_grad()
+        else:
+            z.step()
+            z.zero_grad()
+    w = z.full_parameters() if strategy == "zero3" else torch.cat([p.detach().reshape(-1) for p in model.parameters()])
+    assert w.dtype == getattr(torch, dtype_name)
+    return {"losses": losses, "sha256": sha(w.view(torch.int16) if w.element_size() == 2 else w), "first8": w[:8].double().tolist(),
+            "last8": w[-8:].double().tolist()}
+
+
+@pytest.mark.parametrize("world", [2, 3])
+@pytest.mark.parametrize("dtype_name", ["bfloat16", "float64"])
+def test_reproduces_the_reference_runs_on_bfloat16_and_float64_models(dtype_name, world):
+    """tests/golden/train_dtypes.json: the reference's DDP, ZeRO-1/2 and FSDP over its own engine with the model in
+    bfloat16 and in float64 (its wrappers, collectives and ShardedAdamW take any floating type). The product's wrappers
+    over the oracle's group and the oracle's typed AdamW must give the same losses and the same weights, bit for bit:
+    the composition of the typed ring (every addition rounded to the type) and the typed update, end to end."""
+    want = golden_json("train_dtypes.json")
+    for strategy in ("ddp", "zero1", "zero2", "zero3"):
+        got = cpu_launch(train_rank_typed, world, strategy, want["bucket_bytes"], want["steps"], want["batch"], dtype_name, slot_bytes=1024)
+        for r in range(world):
+            ref = want[dtype_name][str(world)][strategy][r]
+            assert got[r]["losses"] == ref["losses"], (dtype_name, world, strategy, r)
+            assert got[r]["first8"] == ref["first8"] and got[r]["last8"] == ref["last8"], (dtype_name, world, strategy, r)
+            assert got[r]["sha256"] == ref["sha256"], (dtype_name, world, strategy, r)
+
+
 def torch_rank(rank, world, init, out, accumulate):
     import torch.distributed as dist
     from torch.nn.parallel import DistributedDataParallel
