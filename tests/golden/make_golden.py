@@ -3,7 +3,7 @@ implementation (tandem's Python engine, CPU processes) on small seeded inputs.
 
 Run once, in the build container only, where the reference is mounted:
 
-    python tests/golden/make_golden.py [/root/reference] [only: ring adamw adamw_dtypes plans data train train_dtypes]
+    python tests/golden/make_golden.py [/root/reference] [only: ring adamw adamw_dtypes plans data train train_dtypes train_accumulating]
 
 The fixtures are data only (inputs, expected outputs, digests). They pin the
 parts of the path that no test of the reference pins by itself:
@@ -22,6 +22,7 @@ parts of the path that no test of the reference pins by itself:
   train_*.json        losses and weight digests of DDP / ZeRO-1/2/3 training
                       runs (CPU, tiny GPT) at world sizes 2, 3 and 4.
   train_dtypes.json   the same runs with the model in bfloat16 and in float64, world sizes 2 and 3.
+  train_accumulating.json   the same runs with two backward passes before every step, world sizes 2 and 3.
 
 Nothing here is loaded by the library; tests read the fixtures only.
 """
@@ -354,6 +355,50 @@ def train_rank_typed(g, strategy, bucket_bytes, dtype_name):
     return {"losses": losses, "sha256": sha(raw), "first8": w[:8].double().tolist(), "last8": w[-8:].double().tolist()}
 
 
+def train_rank_accumulating(g, strategy, bucket_bytes, micro_batches):
+    """Several backward passes before each step: the reference's ZeRO and FSDP keep adding into their gradient
+    (shard) until zero_grad() (tandem/zero.py:139-153,165-170,306-317), its DDP skips the all-reduce under no_sync()."""
+    torch.manual_seed(0)
+    text = synthetic(20_000)
+    model = GPT(CFG)
+    losses = []
+    if strategy == "ddp":
+        z = DDP(model, g, bucket_bytes=bucket_bytes)
+        opt = torch.optim.AdamW(model.parameters(), lr=3e-3, weight_decay=0.1, foreach=False)
+    else:
+        sopt = ShardedAdamW(lr=3e-3, weight_decay=0.1)
+        stage = int(strategy[-1])
+        z = ZeRO(model, g, stage, sopt, bucket_bytes) if stage < 3 else FSDP(model, g, sopt)
+    for step in range(3):
+        for micro in range(micro_batches):
+            x, y = text.batch(step * micro_batches + micro, BATCH, CFG.seq, rank=g.rank, world=g.size)
+            if strategy == "ddp" and micro < micro_batches - 1:
+                with z.no_sync():
+                    loss = z(x, y)
+                    (loss / micro_batches).backward()
+            else:
+                loss = z(x, y)
+                (loss / micro_batches).backward()
+            losses.append(loss.item())
+        if strategy == "ddp":
+            opt.step()
+            opt.zero_grad()
+        else:
+            z.step()
+            z.zero_grad()
+    w = z.full_parameters() if strategy == "zero3" else torch.cat([p.detach().reshape(-1) for p in model.parameters()])
+    return {"losses": losses, "sha256": sha(w), "first8": w[:8].tolist(), "last8": w[-8:].tolist()}
+
+
+def write_train_accumulating():
+    out = {"steps": 3, "batch": BATCH, "micro_batches": 2, "bucket_bytes": 4 << 10, "torch": torch.__version__}
+    for world in (2, 3):
+        out[str(world)] = {strategy: launch(train_rank_accumulating, world, strategy, 4 << 10, 2, slot_bytes=1024)
+                           for strategy in ("ddp", "zero1", "zero2", "zero3")}
+    with open(os.path.join(HERE, "train_accumulating.json"), "w") as f:
+        json.dump(out, f, indent=0)
+
+
 def write_train_dtypes():
     out = {"cfg": {"seq": 32, "layers": 2, "heads": 2, "dim": 32}, "steps": 4, "batch": BATCH, "lr": 3e-3, "weight_decay": 0.1,
            "bucket_bytes": 4 << 10, "torch": torch.__version__}
@@ -368,7 +413,8 @@ def write_train_dtypes():
 
 if __name__ == "__main__":
     writers = {"ring": write_ring, "adamw": write_adamw, "adamw_dtypes": write_adamw_dtypes, "plans": write_plans,
-               "data": write_data, "train": write_train, "train_dtypes": write_train_dtypes}
+               "data": write_data, "train": write_train, "train_dtypes": write_train_dtypes,
+               "train_accumulating": write_train_accumulating}
     only = sys.argv[2:] or list(writers)
     for name in only:
         writers[name]()

@@ -85,6 +85,21 @@ def test_reproduces_the_reference_training_runs(world, strategy):
             assert got[r]["state_bytes"] <= 2 * 4 * (got[r]["numel"] // world + 1)
 
 
+@pytest.mark.parametrize("world", [2, 3])
+def test_reproduces_the_reference_runs_with_two_backward_passes_a_step(world):
+    """tests/golden/train_accumulating.json: the reference's own runs with two micro-batches before every step. Its ZeRO
+    and FSDP add every backward pass into their gradient (shard) until zero_grad() (tandem/zero.py:139-153,165-170,
+    306-317), its DDP skips the all-reduce under no_sync() (tandem/ddp.py:79-87): same losses, same weights, bit for bit."""
+    want = golden_json("train_accumulating.json")
+    for strategy in ("ddp", "zero1", "zero2", "zero3"):
+        got = cpu_launch(train_rank, world, strategy, want["bucket_bytes"], want["steps"], want["batch"], want["micro_batches"], slot_bytes=1024)
+        for r in range(world):
+            ref = want[str(world)][strategy][r]
+            assert got[r]["losses"] == ref["losses"], (world, strategy, r)
+            assert got[r]["first8"] == ref["first8"] and got[r]["last8"] == ref["last8"], (world, strategy, r)
+            assert got[r]["sha256"] == ref["sha256"], (world, strategy, r)
+
+
 def train_rank_typed(g, strategy, bucket_bytes, steps, batch, dtype_name):
     torch.manual_seed(0)
     text = synthetic(20_000)
