@@ -355,7 +355,7 @@ def train_rank_typed(g, strategy, bucket_bytes, dtype_name):
     return {"losses": losses, "sha256": sha(raw), "first8": w[:8].double().tolist(), "last8": w[-8:].double().tolist()}
 
 
-def train_rank_accumulating(g, strategy, bucket_bytes, micro_batches):
+def train_rank_accumulating(g, strategy, bucket_bytes, micro_batches, zero_every=1):
     """Several backward passes before each step: the reference's ZeRO and FSDP keep adding into their gradient
     (shard) until zero_grad() (tandem/zero.py:139-153,165-170,306-317), its DDP skips the all-reduce under no_sync()."""
     torch.manual_seed(0)
@@ -380,12 +380,15 @@ def train_rank_accumulating(g, strategy, bucket_bytes, micro_batches):
                 loss = z(x, y)
                 (loss / micro_batches).backward()
             losses.append(loss.item())
+        last = (step + 1) % zero_every == 0  # zero_every=2: every other step keeps its gradients for the next one
         if strategy == "ddp":
             opt.step()
-            opt.zero_grad()
+            if last:
+                opt.zero_grad()
         else:
             z.step()
-            z.zero_grad()
+            if last:
+                z.zero_grad()
     w = z.full_parameters() if strategy == "zero3" else torch.cat([p.detach().reshape(-1) for p in model.parameters()])
     return {"losses": losses, "sha256": sha(w), "first8": w[:8].tolist(), "last8": w[-8:].tolist()}
 
@@ -395,6 +398,9 @@ def write_train_accumulating():
     for world in (2, 3):
         out[str(world)] = {strategy: launch(train_rank_accumulating, world, strategy, 4 << 10, 2, slot_bytes=1024)
                            for strategy in ("ddp", "zero1", "zero2", "zero3")}
+    # a step that is not followed by zero_grad(): the next backward adds to what is there (zero_grad after every second step)
+    out["zero_grad_every_second_step"] = {str(world): {strategy: launch(train_rank_accumulating, world, strategy, 4 << 10, 1, 2, slot_bytes=1024)
+                                                       for strategy in ("ddp", "zero1", "zero2", "zero3")} for world in (2, 3)}
     with open(os.path.join(HERE, "train_accumulating.json"), "w") as f:
         json.dump(out, f, indent=0)
 

@@ -26,7 +26,7 @@ def sha(t):
     return hashlib.sha256(t.detach().contiguous().numpy().tobytes()).hexdigest()
 
 
-def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1):
+def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1, zero_every=1):
     torch.manual_seed(0)
     text = synthetic(20_000)
     model = GPT(CFG)
@@ -49,12 +49,15 @@ def train_rank(g, strategy, bucket_bytes, steps, batch, accumulate=1):
                 loss = z(x, y)
                 (loss / accumulate).backward()
             losses.append(loss.item())
+        last = (step + 1) % zero_every == 0
         if strategy == "ddp":
             opt.step()
-            opt.zero_grad()
+            if last:
+                opt.zero_grad()
         else:
             z.step()
-            z.zero_grad()
+            if last:
+                z.zero_grad()
     if strategy == "zero3":
         w = z.full_parameters()
         extra = {"max_live": z.max_live, "live": z.live}
@@ -89,7 +92,8 @@ def test_reproduces_the_reference_training_runs(world, strategy):
 def test_reproduces_the_reference_runs_with_two_backward_passes_a_step(world):
     """tests/golden/train_accumulating.json: the reference's own runs with two micro-batches before every step. Its ZeRO
     and FSDP add every backward pass into their gradient (shard) until zero_grad() (tandem/zero.py:139-153,165-170,
-    306-317), its DDP skips the all-reduce under no_sync() (tandem/ddp.py:79-87): same losses, same weights, bit for bit."""
+    306-317), its DDP skips the all-reduce under no_sync() (tandem/ddp.py:79-87): same losses, same weights, bit for bit.
+    The fixture's second half: one backward pass a step, but zero_grad() only after every second step."""
     want = golden_json("train_accumulating.json")
     for strategy in ("ddp", "zero1", "zero2", "zero3"):
         got = cpu_launch(train_rank, world, strategy, want["bucket_bytes"], want["steps"], want["batch"], want["micro_batches"], slot_bytes=1024)
@@ -98,6 +102,12 @@ def test_reproduces_the_reference_runs_with_two_backward_passes_a_step(world):
             assert got[r]["losses"] == ref["losses"], (world, strategy, r)
             assert got[r]["first8"] == ref["first8"] and got[r]["last8"] == ref["last8"], (world, strategy, r)
             assert got[r]["sha256"] == ref["sha256"], (world, strategy, r)
+        # and a step() that is not followed by zero_grad(): the next backward adds to what is there
+        got = cpu_launch(train_rank, world, strategy, want["bucket_bytes"], want["steps"], want["batch"], 1, 2, slot_bytes=1024)
+        for r in range(world):
+            ref = want["zero_grad_every_second_step"][str(world)][strategy][r]
+            assert got[r]["losses"] == ref["losses"], (world, strategy, r, "zero_grad every second step")
+            assert got[r]["sha256"] == ref["sha256"], (world, strategy, r, "zero_grad every second step")
 
 
 def train_rank_typed(g, strategy, bucket_bytes, steps, batch, dtype_name):
