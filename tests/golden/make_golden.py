@@ -393,6 +393,21 @@ def train_rank_accumulating(g, strategy, bucket_bytes, micro_batches, zero_every
     return {"losses": losses, "sha256": sha(w), "first8": w[:8].tolist(), "last8": w[-8:].tolist()}
 
 
+def fsdp_rank_without_prefetch(g):
+    torch.manual_seed(0)
+    text = synthetic(20_000)
+    z = FSDP(GPT(CFG), g, ShardedAdamW(lr=3e-3, weight_decay=0.1), prefetch=False)
+    losses = []
+    for step in range(3):
+        x, y = text.batch(step, BATCH, CFG.seq, rank=g.rank, world=g.size)
+        loss = z(x, y)
+        loss.backward()
+        losses.append(loss.item())
+        z.step()
+        z.zero_grad()
+    return {"losses": losses, "sha256": sha(z.full_parameters()), "max_live": z.max_live, "live": z.live}
+
+
 def write_train_accumulating():
     out = {"steps": 3, "batch": BATCH, "micro_batches": 2, "bucket_bytes": 4 << 10, "torch": torch.__version__}
     for world in (2, 3):
@@ -401,6 +416,7 @@ def write_train_accumulating():
     # a step that is not followed by zero_grad(): the next backward adds to what is there (zero_grad after every second step)
     out["zero_grad_every_second_step"] = {str(world): {strategy: launch(train_rank_accumulating, world, strategy, 4 << 10, 1, 2, slot_bytes=1024)
                                                        for strategy in ("ddp", "zero1", "zero2", "zero3")} for world in (2, 3)}
+    out["fsdp_without_prefetch"] = {str(world): launch(fsdp_rank_without_prefetch, world, slot_bytes=1024) for world in (2, 3)}
     with open(os.path.join(HERE, "train_accumulating.json"), "w") as f:
         json.dump(out, f, indent=0)
 

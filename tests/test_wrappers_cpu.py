@@ -110,6 +110,32 @@ def test_reproduces_the_reference_runs_with_two_backward_passes_a_step(world):
             assert got[r]["sha256"] == ref["sha256"], (world, strategy, r, "zero_grad every second step")
 
 
+def fsdp_rank_without_prefetch(g, batch):
+    torch.manual_seed(0)
+    text = synthetic(20_000)
+    z = FSDP(GPT(CFG), g, OracleShardedAdamW(lr=3e-3, weight_decay=0.1), prefetch=False)
+    losses = []
+    for step in range(3):
+        x, y = text.batch(step, batch, CFG.seq, rank=g.rank, world=g.size)
+        loss = z(x, y)
+        loss.backward()
+        losses.append(loss.item())
+        z.step()
+        z.zero_grad()
+    return {"losses": losses, "sha256": sha(z.full_parameters()), "max_live": z.max_live, "live": z.live}
+
+
+@pytest.mark.parametrize("world", [2, 3])
+def test_fsdp_without_prefetch_as_the_reference_runs_it(world):
+    """FSDP(prefetch=False) in the reference: the same weights, and no more units whole at once than it has."""
+    want = golden_json("train_accumulating.json")
+    got = cpu_launch(fsdp_rank_without_prefetch, world, want["batch"], slot_bytes=1024)
+    for r in range(world):
+        ref = want["fsdp_without_prefetch"][str(world)][r]
+        assert got[r]["losses"] == ref["losses"] and got[r]["sha256"] == ref["sha256"], (world, r)
+        assert got[r]["max_live"] == ref["max_live"] and got[r]["live"] == ref["live"] == 0, (world, r, got[r]["max_live"], ref["max_live"])
+
+
 def train_rank_typed(g, strategy, bucket_bytes, steps, batch, dtype_name):
     torch.manual_seed(0)
     text = synthetic(20_000)
